@@ -1,0 +1,132 @@
+"""CPU fp32 oracle for the floating-point kernels of the PTv3 forward path
+(TEST INFRASTRUCTURE — only tests, the smoke check and the CPU-baseline leg of the
+benchmark may import this).
+
+Stock torch CPU operators stand in for the third-party CUDA packages the reference calls:
+
+* patch attention   -> the non-flash arithmetic of model.py:458-474 (== what
+  flash_attn_varlen_qkvpacked_func computes at model.py:476-482 with dropout 0),
+  looped per sequence so the (P,H,K,K) score tensor is never materialised
+* submanifold conv  -> gather + GEMM over the neighbour map (spconv.SubMConv3d call
+  sites model.py:546-552, :767-774)
+* segment reductions-> torch_scatter.segment_csr call sites model.py:684-689
+* unpooling add     -> model.py:746
+"""
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+
+def patch_attention(qkv, cu_seqlens, num_heads, scale=None):
+    """qkv: (Npad, 3*C) fp32 rows already in padded serialized order, channel layout
+    [3][H][D] (model.py:461,477). Returns (Npad, C)."""
+    qkv = torch.as_tensor(qkv, dtype=torch.float32)
+    npad, c3 = qkv.shape
+    C = c3 // 3
+    D = C // num_heads
+    scale = D ** -0.5 if scale is None else scale
+    cu = [int(v) for v in cu_seqlens]
+    out = torch.empty(npad, C, dtype=torch.float32)
+    for s, e in zip(cu[:-1], cu[1:]):
+        blk = qkv[s:e].reshape(e - s, 3, num_heads, D).permute(1, 2, 0, 3)  # (3,H,L,D)
+        q, k, v = blk[0], blk[1], blk[2]
+        attn = torch.softmax((q * scale) @ k.transpose(-2, -1), dim=-1)
+        out[s:e] = (attn @ v).transpose(0, 1).reshape(e - s, C)
+    return out
+
+
+def patch_attention_bruteforce(qkv, cu_seqlens, num_heads, scale=None):
+    """Triple loop in float64 numpy; toy sizes only."""
+    qkv = np.asarray(qkv, dtype=np.float64)
+    npad, c3 = qkv.shape
+    C = c3 // 3
+    D = C // num_heads
+    scale = D ** -0.5 if scale is None else scale
+    out = np.zeros((npad, C))
+    cu = [int(v) for v in cu_seqlens]
+    for s, e in zip(cu[:-1], cu[1:]):
+        for h in range(num_heads):
+            q = qkv[s:e, h * D:(h + 1) * D]
+            k = qkv[s:e, C + h * D:C + (h + 1) * D]
+            v = qkv[s:e, 2 * C + h * D:2 * C + (h + 1) * D]
+            for i in range(e - s):
+                sc = (k @ q[i]) * scale
+                w = np.exp(sc - sc.max())
+                out[s + i, h * D:(h + 1) * D] = (w / w.sum()) @ v
+    return out
+
+
+def serialized_attention_core(feat_qkv, order, inverse, pad, unpad, cu_seqlens, num_heads,
+                              scale=None):
+    """model.py:452-484: gather rows into padded serialized order, attend inside each
+    patch, keep each point's primary slot. feat_qkv: (N, 3C). Returns (N, C)."""
+    feat_qkv = torch.as_tensor(feat_qkv, dtype=torch.float32)
+    gidx = torch.as_tensor(np.asarray(order)[np.asarray(pad)])
+    back = torch.as_tensor(np.asarray(unpad)[np.asarray(inverse)])
+    out = patch_attention(feat_qkv[gidx], cu_seqlens, num_heads, scale)
+    return out[back]
+
+
+def subm_conv(feat, nbr, weight, bias=None):
+    """out[i] = sum_k W[:,k,:] @ feat[nbr[i,k]] (+ bias); rows with nbr == -1 contribute 0.
+
+    feat (N,Cin); nbr (N,V) int; weight (Cout, ks,ks,ks, Cin) — the layout spconv 2.x
+    gives SubMConv3d.weight (an assumption: spconv is not in the reference checkout);
+    cross-correlation, offset index k = (kx*ks+ky)*ks+kz."""
+    feat = torch.as_tensor(feat, dtype=torch.float32)
+    weight = torch.as_tensor(weight, dtype=torch.float32)
+    nbr = torch.as_tensor(np.asarray(nbr), dtype=torch.int64)
+    cout, cin = weight.shape[0], weight.shape[-1]
+    V = nbr.shape[1]
+    w = weight.reshape(cout, V, cin)
+    out = torch.zeros(feat.shape[0], cout, dtype=torch.float32)
+    for k in range(V):
+        col = nbr[:, k]
+        hit = (col >= 0).nonzero(as_tuple=True)[0]
+        if hit.numel() == 0:
+            continue
+        out.index_add_(0, hit, feat[col[hit]] @ w[:, k, :].t())
+    if bias is not None:
+        out += torch.as_tensor(bias, dtype=torch.float32)
+    return out
+
+
+def subm_conv_dense(feat, indices, weight, bias=None):
+    """The same convolution through torch's dense conv3d on a densified grid; tiny grids
+    only. Pins offset enumeration, weight layout and cross-correlation of subm_conv."""
+    feat = torch.as_tensor(feat, dtype=torch.float32)
+    weight = torch.as_tensor(weight, dtype=torch.float32)
+    idx = torch.as_tensor(np.asarray(indices), dtype=torch.int64)
+    cout, ks, cin = weight.shape[0], weight.shape[1], weight.shape[-1]
+    B = int(idx[:, 0].max()) + 1
+    X, Y, Z = (int(idx[:, a].max()) + 1 for a in (1, 2, 3))
+    dense = torch.zeros(B, cin, X, Y, Z)
+    dense[idx[:, 0], :, idx[:, 1], idx[:, 2], idx[:, 3]] = feat
+    w = weight.permute(0, 4, 1, 2, 3).contiguous()  # (Cout,Cin,kx,ky,kz)
+    y = F.conv3d(dense, w, None if bias is None else torch.as_tensor(bias, dtype=torch.float32),
+                 padding=ks // 2)
+    return y[idx[:, 0], :, idx[:, 1], idx[:, 2], idx[:, 3]]
+
+
+def segment_csr(src, indices, idx_ptr, reduce="max"):
+    """reduce(src[indices[idx_ptr[m]:idx_ptr[m+1]]]) per segment m (model.py:684-689).
+    Segments are never empty on this path."""
+    src = np.asarray(torch.as_tensor(src, dtype=torch.float32))[np.asarray(indices)]
+    starts = np.asarray(idx_ptr[:-1], dtype=np.int64)
+    if reduce == "max":
+        out = np.maximum.reduceat(src, starts, axis=0)
+    elif reduce == "min":
+        out = np.minimum.reduceat(src, starts, axis=0)
+    else:
+        out = np.add.reduceat(src.astype(np.float64), starts, axis=0)
+        if reduce == "mean":
+            out = out / np.diff(np.asarray(idx_ptr, dtype=np.int64))[:, None]
+        out = out.astype(np.float32)
+    return torch.from_numpy(np.ascontiguousarray(out))
+
+
+def unpool_add(parent_feat, child_feat, cluster):
+    """model.py:746."""
+    parent_feat = torch.as_tensor(parent_feat, dtype=torch.float32)
+    child_feat = torch.as_tensor(child_feat, dtype=torch.float32)
+    return parent_feat + child_feat[torch.as_tensor(np.asarray(cluster), dtype=torch.int64)]
