@@ -1,0 +1,131 @@
+/* C ABI of libptv3_hip.so — hand-written gfx950 kernels for the Point Transformer V3
+ * forward path.
+ *
+ * Conventions
+ *   - every pointer named *_dev / without suffix is DEVICE memory unless the comment says
+ *     "host"; sizes are element counts unless they end in _bytes
+ *   - `stream` is a hipStream_t passed as void*; all work is enqueued asynchronously on it
+ *   - no entry point allocates or frees device memory or synchronises the device:
+ *     outputs and workspaces are the caller's (query the size with *_workspace_bytes)
+ *   - return value: 0 ok; < 0 argument error (PTV3_E*); > 0 a hipError_t from a launch
+ *   - dtype codes: 0 = float32, 1 = float16, 2 = bfloat16
+ *
+ * The reference has no native interface; each entry point names the Python lines whose
+ * device work it replaces (paths relative to the reference checkout).
+ */
+#ifndef PTV3_HIP_H
+#define PTV3_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PTV3_OK 0
+#define PTV3_EINVAL (-1)    /* null pointer, negative size, unknown enum */
+#define PTV3_EDEPTH (-2)    /* depth outside 1..16 or code wider than 63 bits (model.py:103,108) */
+#define PTV3_EWORKSPACE (-3) /* workspace smaller than *_workspace_bytes says */
+#define PTV3_ESHAPE (-4)    /* channel / head / patch shape the kernels do not cover */
+
+#define PTV3_F32 0
+#define PTV3_F16 1
+#define PTV3_BF16 2
+
+#define PTV3_ORDER_Z 0
+#define PTV3_ORDER_Z_TRANS 1
+#define PTV3_ORDER_HILBERT 2
+#define PTV3_ORDER_HILBERT_TRANS 3
+
+int ptv3_version(void);
+const char *ptv3_strerror(int rc);
+
+/* serialization/default.py:8-24 -> z_order.py:66-101, hilbert.py:91-198.
+ * grid_coord (n,3) int32; batch (n,) int64 or NULL; order_ids: HOST array of k PTV3_ORDER_*;
+ * code (k,n) int64, row r holds order_ids[r]. All k orders are produced in one pass. */
+int ptv3_encode(const int32_t *grid_coord, const int64_t *batch, int64_t n, int depth,
+                const int32_t *order_ids_host, int k, int64_t *code, void *stream);
+
+/* model.py:119-126 and :667-674: per-row ascending argsort of (k,n) int64 codes plus the
+ * inverse permutation. Only the low `key_bits` bits are sorted on (the rest must be equal
+ * across a row, e.g. zero); ties keep their input order. */
+size_t ptv3_argsort_workspace_bytes(int64_t n, int k);
+int ptv3_argsort(const int64_t *code, int64_t n, int k, int key_bits, int64_t *order,
+                 int64_t *inverse, void *workspace, size_t workspace_bytes, void *stream);
+
+/* model.py:392-437. ptv3_pad_sizes is host-only arithmetic on a HOST copy of `offset`
+ * (nb cumulative scene ends): total padded length and number of sequences.
+ * ptv3_pad_index fills pad (n_pad,), unpad (n,), cu_seqlens (n_seq+1,) int32 from the
+ * DEVICE offset; workspace >= ptv3_pad_index_workspace_bytes(nb). */
+int ptv3_pad_sizes(const int64_t *offset_host, int nb, int64_t patch, int64_t *n_pad,
+                   int64_t *n_seq);
+size_t ptv3_pad_index_workspace_bytes(int nb);
+int ptv3_pad_index(const int64_t *offset, int nb, int64_t patch, int64_t n, int64_t n_pad,
+                   int64_t n_seq, int64_t *pad, int64_t *unpad, int32_t *cu_seqlens,
+                   void *workspace, size_t workspace_bytes, void *stream);
+
+/* model.py:452-453,456,484 folded into two int32 tables for one serialization order:
+ * slot_src[i] = order[pad[i]] (row to read for padded slot i) and
+ * slot_dst[i] = that row again when i is the row's own slot (unpad[inverse[row]] == i),
+ * else -1 (filler slots only lend keys/values, model.py:412-423). */
+int ptv3_attn_slots(const int64_t *order_row, const int64_t *inverse_row, const int64_t *pad,
+                    const int64_t *unpad, int64_t n_pad, int32_t *slot_src, int32_t *slot_dst,
+                    void *stream);
+
+/* model.py:456-484 (flash_attn_varlen_qkvpacked_func call at :476-482 and the torch
+ * fallback :460-474): non-causal softmax(q k^T * scale) v inside each sequence, per head.
+ * qkv (n_rows, 3*C) with channel layout [3][H][D], D = C/H = 16; rows are fetched through
+ * slot_src and results written to out[slot_dst[i]] (n_rows, C) when slot_dst[i] >= 0.
+ * cu_seqlens (n_seq+1,) int32 in padded-slot units; no sequence is longer than max_seqlen. */
+int ptv3_patch_attn_fwd(const void *qkv, int dtype, int64_t n_rows, int channels, int heads,
+                        const int32_t *slot_src, const int32_t *slot_dst,
+                        const int32_t *cu_seqlens, int64_t n_seq, int64_t max_seqlen,
+                        float scale, void *out, void *stream);
+
+/* spconv.SubMConv3d's index generation (call sites model.py:546-552, :767-774, tensor built
+ * at :165-172). indices (n,4) int32 [batch,x,y,z], coordinates in [0, 65535];
+ * nbr (n, ks^3) int32: nbr[i][(kx*ks+ky)*ks+kz] = row of the voxel at
+ * (b, x+kx-ks/2, y+ky-ks/2, z+kz-ks/2) or -1. ks is 3 or 5. */
+size_t ptv3_kmap_workspace_bytes(int64_t n);
+int ptv3_kmap_build(const int32_t *indices, int64_t n, int ks, int32_t *nbr, void *workspace,
+                    size_t workspace_bytes, void *stream);
+
+/* spconv.SubMConv3d forward (same call sites): out[i] = bias + sum_k W[:,k,:] feat[nbr[i][k]].
+ * feat (n,cin), weight (cout, V, cin) (spconv 2.x KRSC layout flattened over the taps),
+ * bias (cout,) or NULL, out (n,cout); all of `dtype`, accumulation in fp32. */
+int ptv3_subm_conv_fwd(const void *feat, int dtype, int64_t n, int cin, const int32_t *nbr,
+                       int taps, const void *weight, const void *bias, int cout, void *out,
+                       void *stream);
+
+/* model.py:652-664,690-695: clusters of code0 >> shift walked in sorted order (order0 sorts
+ * code0, so no further sort is needed). Outputs: cluster (n,) int64 [pooling_inverse],
+ * indices (n,) int64 (= order0: points grouped by cluster), idx_ptr (n+1 allocated, m+1 used),
+ * head (n allocated, m used), n_clusters (1,) int64 on the device. */
+size_t ptv3_pool_clusters_workspace_bytes(int64_t n);
+int ptv3_pool_clusters(const int64_t *code0, const int64_t *order0, int64_t n, int shift,
+                       int64_t *cluster, int64_t *idx_ptr, int64_t *head, int64_t *n_clusters,
+                       void *workspace, size_t workspace_bytes, void *stream);
+
+/* model.py:666-674,690,695 once the cluster count m is known on the host: pooled codes
+ * (k,m) = code[:, head] >> shift, pooled grid_coord (m,3) = grid_coord[head] >> pool_depth,
+ * pooled batch (m,) = batch[head]. */
+int ptv3_pool_gather(const int64_t *code, int64_t n, int k, int shift, const int32_t *grid_coord,
+                     int pool_depth, const int64_t *batch, const int64_t *head, int64_t m,
+                     int64_t *code_out, int32_t *grid_coord_out, int64_t *batch_out,
+                     void *stream);
+
+/* torch_scatter.segment_csr call sites model.py:684-689: reduce src[indices[j]] over
+ * j in [idx_ptr[s], idx_ptr[s+1]). op 0 = max, 1 = mean, 2 = sum, 3 = min.
+ * src (n,c) of dtype, out (m,c) of dtype. */
+int ptv3_segment_reduce(const void *src, int dtype, int64_t n, int c, const int64_t *indices,
+                        const int64_t *idx_ptr, int64_t m, int op, void *out, void *stream);
+
+/* model.py:746: out[i] = parent[i] + child[cluster[i]]; parent,out (n,c), child (m,c). */
+int ptv3_unpool_add(const void *parent, const void *child, int dtype, int64_t n, int c,
+                    const int64_t *cluster, int64_t m, void *out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PTV3_HIP_H */

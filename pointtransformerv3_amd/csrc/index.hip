@@ -1,0 +1,116 @@
+// Patch padding tables and the per-order gather/scatter tables of serialized attention.
+//
+// Replaces model.py:392-437 (a Python loop over scenes with one device->host sync per
+// scene in the reference) and the index arithmetic of model.py:452-453 by two launches
+// that never leave the device.
+#include "common.h"
+
+namespace {
+
+// Single thread: exclusive prefix of padded scene lengths and of sequence counts.
+__global__ void pad_prefix_kernel(const int64_t* __restrict__ offset, int nb, int64_t patch,
+                                  int64_t* __restrict__ pad_start, int64_t* __restrict__ seq_start) {
+    if (blockIdx.x != 0 || threadIdx.x != 0) return;
+    int64_t prev = 0, op = 0, sq = 0;
+    for (int s = 0; s < nb; ++s) {
+        const int64_t cnt = offset[s] - prev;
+        prev = offset[s];
+        const int64_t padded = cnt > patch ? ((cnt + patch - 1) / patch) * patch : cnt;
+        pad_start[s] = op;
+        seq_start[s] = sq;
+        op += padded;
+        sq += (padded + patch - 1) / patch;
+    }
+    pad_start[nb] = op;
+    seq_start[nb] = sq;
+}
+
+__global__ __launch_bounds__(256) void pad_index_kernel(
+    const int64_t* __restrict__ offset, int nb, int64_t patch, int64_t n_pad, int64_t n_seq,
+    const int64_t* __restrict__ pad_start, const int64_t* __restrict__ seq_start,
+    int64_t* __restrict__ pad, int64_t* __restrict__ unpad, int32_t* __restrict__ cu_seqlens) {
+    const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j == 0) cu_seqlens[n_seq] = (int32_t)n_pad;
+    if (j >= n_pad) return;
+    // scene s: last s with pad_start[s] <= j (empty scenes share a start and are skipped)
+    int lo = 0, hi = nb;  // invariant: pad_start[lo] <= j < pad_start[hi]
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (pad_start[mid] <= j) lo = mid; else hi = mid;
+    }
+    const int s = lo;
+    const int64_t first = s ? offset[s - 1] : 0;
+    const int64_t cnt = offset[s] - first;
+    const int64_t local = j - pad_start[s];
+    // filler slots of the last patch reuse the points one patch earlier (model.py:412-423)
+    pad[j] = first + (local < cnt ? local : local - patch);
+    if (local < cnt) unpad[first + local] = j;
+    if (local % patch == 0) cu_seqlens[seq_start[s] + local / patch] = (int32_t)j;
+}
+
+__global__ __launch_bounds__(256) void attn_slots_kernel(
+    const int64_t* __restrict__ order_row, const int64_t* __restrict__ inverse_row,
+    const int64_t* __restrict__ pad, const int64_t* __restrict__ unpad, int64_t n_pad,
+    int32_t* __restrict__ slot_src, int32_t* __restrict__ slot_dst) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_pad) return;
+    const int64_t row = order_row[pad[i]];
+    slot_src[i] = (int32_t)row;
+    slot_dst[i] = (unpad[inverse_row[row]] == i) ? (int32_t)row : -1;
+}
+
+}  // namespace
+
+extern "C" int ptv3_pad_sizes(const int64_t* offset_host, int nb, int64_t patch, int64_t* n_pad,
+                              int64_t* n_seq) {
+    if (!offset_host || nb < 0 || patch < 1 || !n_pad || !n_seq) return PTV3_EINVAL;
+    int64_t prev = 0, op = 0, sq = 0;
+    for (int s = 0; s < nb; ++s) {
+        const int64_t cnt = offset_host[s] - prev;
+        if (cnt < 0) return PTV3_EINVAL;
+        prev = offset_host[s];
+        const int64_t padded = cnt > patch ? ((cnt + patch - 1) / patch) * patch : cnt;
+        op += padded;
+        sq += (padded + patch - 1) / patch;
+    }
+    *n_pad = op;
+    *n_seq = sq;
+    return PTV3_OK;
+}
+
+extern "C" size_t ptv3_pad_index_workspace_bytes(int nb) {
+    return nb < 0 ? 0 : ptv3_align256(2 * (size_t)(nb + 1) * sizeof(int64_t));
+}
+
+extern "C" int ptv3_pad_index(const int64_t* offset, int nb, int64_t patch, int64_t n,
+                              int64_t n_pad, int64_t n_seq, int64_t* pad, int64_t* unpad,
+                              int32_t* cu_seqlens, void* workspace, size_t workspace_bytes,
+                              void* stream_) {
+    if (nb < 1 || patch < 1 || n < 0 || n_pad < n || n_seq < 0 || n_pad >= (1ll << 31))
+        return PTV3_EINVAL;
+    if (!offset || !cu_seqlens || !workspace) return PTV3_EINVAL;
+    if (n_pad > 0 && (!pad || !unpad)) return PTV3_EINVAL;
+    if (workspace_bytes < ptv3_pad_index_workspace_bytes(nb)) return PTV3_EWORKSPACE;
+    hipStream_t stream = (hipStream_t)stream_;
+    int64_t* pad_start = (int64_t*)workspace;
+    int64_t* seq_start = pad_start + (nb + 1);
+    hipLaunchKernelGGL(pad_prefix_kernel, dim3(1), dim3(1), 0, stream, offset, nb, patch, pad_start,
+                       seq_start);
+    const int64_t blocks = ptv3_ceil_div(n_pad > 0 ? n_pad : 1, 256);
+    hipLaunchKernelGGL(pad_index_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, offset, nb,
+                       patch, n_pad, n_seq, (const int64_t*)pad_start, (const int64_t*)seq_start,
+                       pad, unpad, cu_seqlens);
+    PTV3_RETURN_LAUNCH();
+}
+
+extern "C" int ptv3_attn_slots(const int64_t* order_row, const int64_t* inverse_row,
+                               const int64_t* pad, const int64_t* unpad, int64_t n_pad,
+                               int32_t* slot_src, int32_t* slot_dst, void* stream) {
+    if (n_pad < 0 || n_pad >= (1ll << 31)) return PTV3_EINVAL;
+    if (n_pad == 0) return PTV3_OK;
+    if (!order_row || !inverse_row || !pad || !unpad || !slot_src || !slot_dst) return PTV3_EINVAL;
+    const int64_t blocks = ptv3_ceil_div(n_pad, 256);
+    hipLaunchKernelGGL(attn_slots_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       order_row, inverse_row, pad, unpad, n_pad, slot_src, slot_dst);
+    PTV3_RETURN_LAUNCH();
+}

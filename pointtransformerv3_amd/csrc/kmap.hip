@@ -1,0 +1,120 @@
+// Submanifold neighbour map ("kmap") through an open-addressing voxel hash.
+//
+// Replaces the index generation spconv performs for SubMConv3d (reference call sites
+// model.py:546-552 and :767-774 on the tensor built at :165-172). Canonical output:
+// nbr[i][(kx*ks+ky)*ks+kz] = row of the voxel at coord_i + (kx,ky,kz) - ks/2, or -1.
+//
+//   fill    : table keys <- EMPTY
+//   insert  : one thread per voxel, 64-bit CAS, linear probing (load factor <= 0.5)
+//   lookup  : one thread per (voxel, tap) so the int32 map is written fully coalesced;
+//             the 16 B voxel record is shared by the ks^3 threads of a voxel through L1
+#include "common.h"
+
+namespace {
+
+constexpr uint64_t EMPTY_KEY = ~0ull;
+
+__device__ __forceinline__ uint64_t voxel_key(int b, int x, int y, int z) {
+    // 17 bits per axis after a +4 shift: neighbours of coordinate 0 stay distinct and
+    // nothing wraps for coordinates up to 65535 and kernel sizes up to 9.
+    return ((uint64_t)(uint32_t)b << 51) | ((uint64_t)(uint32_t)(x + 4) << 34) |
+           ((uint64_t)(uint32_t)(y + 4) << 17) | (uint64_t)(uint32_t)(z + 4);
+}
+
+__device__ __forceinline__ uint32_t hash_slot(uint64_t k, uint32_t mask) {
+    k ^= k >> 33;
+    k *= 0xff51afd7ed558ccdull;
+    k ^= k >> 33;
+    k *= 0xc4ceb9fe1a85ec53ull;
+    k ^= k >> 33;
+    return (uint32_t)k & mask;
+}
+
+__global__ __launch_bounds__(256) void kmap_fill_kernel(uint64_t* __restrict__ keys, int64_t cap) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < cap) keys[i] = EMPTY_KEY;
+}
+
+__global__ __launch_bounds__(256) void kmap_insert_kernel(const int32_t* __restrict__ indices,
+                                                          int64_t n, uint64_t* __restrict__ keys,
+                                                          int32_t* __restrict__ vals, uint32_t mask) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int4 v = ((const int4*)indices)[i];
+    const uint64_t key = voxel_key(v.x, v.y, v.z, v.w);
+    uint32_t slot = hash_slot(key, mask);
+    for (uint32_t probe = 0; probe <= mask; ++probe) {
+        const uint64_t prev = atomicCAS((unsigned long long*)&keys[slot], (unsigned long long)EMPTY_KEY,
+                                        (unsigned long long)key);
+        if (prev == EMPTY_KEY || prev == key) {
+            vals[slot] = (int32_t)i;
+            return;
+        }
+        slot = (slot + 1) & mask;
+    }
+}
+
+__global__ __launch_bounds__(256) void kmap_lookup_kernel(const int32_t* __restrict__ indices,
+                                                          int64_t n, int ks, int taps,
+                                                          const uint64_t* __restrict__ keys,
+                                                          const int32_t* __restrict__ vals,
+                                                          uint32_t mask, int32_t* __restrict__ nbr) {
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n * taps) return;
+    const int64_t i = e / taps;
+    const int t = (int)(e - i * taps);
+    const int r = ks >> 1;
+    const int kz = t % ks, ky = (t / ks) % ks, kx = t / (ks * ks);
+    const int4 v = ((const int4*)indices)[i];
+    int32_t found = -1;
+    if (t == taps / 2) {
+        found = (int32_t)i;   // centre tap
+    } else {
+        const uint64_t key = voxel_key(v.x, v.y + kx - r, v.z + ky - r, v.w + kz - r);
+        uint32_t slot = hash_slot(key, mask);
+        for (uint32_t probe = 0; probe <= mask; ++probe) {
+            const uint64_t cur = keys[slot];
+            if (cur == key) { found = vals[slot]; break; }
+            if (cur == EMPTY_KEY) break;
+            slot = (slot + 1) & mask;
+        }
+    }
+    nbr[e] = found;
+}
+
+int64_t table_capacity(int64_t n) {
+    int64_t cap = 1024;
+    while (cap < 2 * n) cap <<= 1;
+    return cap;
+}
+
+}  // namespace
+
+extern "C" size_t ptv3_kmap_workspace_bytes(int64_t n) {
+    if (n < 0) return 0;
+    const int64_t cap = table_capacity(n);
+    return ptv3_align256((size_t)cap * sizeof(uint64_t)) + ptv3_align256((size_t)cap * sizeof(int32_t));
+}
+
+extern "C" int ptv3_kmap_build(const int32_t* indices, int64_t n, int ks, int32_t* nbr,
+                               void* workspace, size_t workspace_bytes, void* stream_) {
+    if (n < 0 || n >= (1ll << 30)) return PTV3_EINVAL;
+    if (ks != 3 && ks != 5) return PTV3_ESHAPE;
+    if (n == 0) return PTV3_OK;
+    if (!indices || !nbr || !workspace) return PTV3_EINVAL;
+    if (workspace_bytes < ptv3_kmap_workspace_bytes(n)) return PTV3_EWORKSPACE;
+    hipStream_t stream = (hipStream_t)stream_;
+    const int64_t cap = table_capacity(n);
+    uint64_t* keys = (uint64_t*)workspace;
+    int32_t* vals = (int32_t*)((char*)workspace + ptv3_align256((size_t)cap * sizeof(uint64_t)));
+    const uint32_t mask = (uint32_t)(cap - 1);
+    const int taps = ks * ks * ks;
+    hipLaunchKernelGGL(kmap_fill_kernel, dim3((unsigned)ptv3_ceil_div(cap, 256)), dim3(256), 0, stream,
+                       keys, cap);
+    hipLaunchKernelGGL(kmap_insert_kernel, dim3((unsigned)ptv3_ceil_div(n, 256)), dim3(256), 0, stream,
+                       indices, n, keys, vals, mask);
+    hipLaunchKernelGGL(kmap_lookup_kernel, dim3((unsigned)ptv3_ceil_div(n * taps, 256)), dim3(256), 0,
+                       stream, indices, n, ks, taps, (const uint64_t*)keys, (const int32_t*)vals, mask,
+                       nbr);
+    PTV3_RETURN_LAUNCH();
+}

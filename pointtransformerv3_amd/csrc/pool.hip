@@ -1,0 +1,222 @@
+// Grid pooling / unpooling as segment operations over the serialized order.
+//
+// Replaces model.py:652-664 (torch.unique + torch.sort + cumsum), :666,:690,:695 (head
+// gathers), :684-689 (torch_scatter.segment_csr) and :746 (gather-add) of the reference.
+// The points are already sorted by row-0 code, so clusters of `code0 >> shift` are runs in
+// that order: boundary flags + an exclusive scan number them; no sort, no hash.
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+
+#include "common.h"
+
+namespace {
+
+constexpr int PB = 256;   // threads per block in the scan kernels
+
+__device__ __forceinline__ bool run_start(const int64_t* __restrict__ code0,
+                                          const int64_t* __restrict__ order0, int64_t i, int shift) {
+    if (i == 0) return true;
+    return (code0[order0[i]] >> shift) != (code0[order0[i - 1]] >> shift);
+}
+
+// inclusive scan of one value per thread across a 256-thread block; returns the inclusive
+// prefix and leaves the block total in *total.
+__device__ __forceinline__ uint32_t block_inclusive_scan(uint32_t v, uint32_t* total) {
+    __shared__ uint32_t wsum[PB / PTV3_WAVE];
+    const int lane = threadIdx.x % PTV3_WAVE, wave = threadIdx.x / PTV3_WAVE;
+    uint32_t x = v;
+#pragma unroll
+    for (int off = 1; off < PTV3_WAVE; off <<= 1) {
+        const uint32_t y = __shfl_up(x, off, PTV3_WAVE);
+        if (lane >= off) x += y;
+    }
+    if (lane == PTV3_WAVE - 1) wsum[wave] = x;
+    __syncthreads();
+    uint32_t base = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < PB / PTV3_WAVE; ++w) {
+        const uint32_t c = wsum[w];
+        if (w < wave) base += c;
+        tot += c;
+    }
+    *total = tot;
+    __syncthreads();
+    return x + base;
+}
+
+__global__ __launch_bounds__(PB) void cluster_count_kernel(const int64_t* __restrict__ code0,
+                                                           const int64_t* __restrict__ order0,
+                                                           int64_t n, int shift,
+                                                           uint32_t* __restrict__ block_cnt) {
+    const int64_t i = (int64_t)blockIdx.x * PB + threadIdx.x;
+    const uint32_t f = (i < n && run_start(code0, order0, i, shift)) ? 1u : 0u;
+    uint32_t total;
+    block_inclusive_scan(f, &total);
+    if (threadIdx.x == 0) block_cnt[blockIdx.x] = total;
+}
+
+// single block: exclusive scan of block_cnt in place, grand total to n_clusters
+__global__ __launch_bounds__(PB) void cluster_scan_kernel(uint32_t* __restrict__ block_cnt,
+                                                          int64_t blocks,
+                                                          int64_t* __restrict__ n_clusters) {
+    uint32_t carry = 0;
+    for (int64_t b0 = 0; b0 < blocks; b0 += PB) {
+        const int64_t b = b0 + threadIdx.x;
+        const uint32_t v = b < blocks ? block_cnt[b] : 0u;
+        uint32_t total;
+        const uint32_t inc = block_inclusive_scan(v, &total);
+        if (b < blocks) block_cnt[b] = carry + inc - v;
+        carry += total;
+    }
+    if (threadIdx.x == 0) *n_clusters = (int64_t)carry;
+}
+
+__global__ __launch_bounds__(PB) void cluster_assign_kernel(
+    const int64_t* __restrict__ code0, const int64_t* __restrict__ order0, int64_t n, int shift,
+    const uint32_t* __restrict__ block_base, int64_t* __restrict__ cluster,
+    int64_t* __restrict__ idx_ptr, int64_t* __restrict__ head) {
+    const int64_t i = (int64_t)blockIdx.x * PB + threadIdx.x;
+    const bool f = i < n && run_start(code0, order0, i, shift);
+    uint32_t total;
+    const uint32_t inc = block_inclusive_scan(f ? 1u : 0u, &total);
+    if (i >= n) return;
+    const int64_t cid = (int64_t)block_base[blockIdx.x] + inc - 1;
+    const int64_t pt = order0[i];
+    cluster[pt] = cid;
+    if (f) {
+        idx_ptr[cid] = i;
+        head[cid] = pt;
+    }
+    if (i == n - 1) idx_ptr[cid + 1] = n;
+}
+
+__global__ __launch_bounds__(256) void pool_gather_kernel(
+    const int64_t* __restrict__ code, int64_t n, int k, int shift,
+    const int32_t* __restrict__ grid_coord, int pool_depth, const int64_t* __restrict__ batch,
+    const int64_t* __restrict__ head, int64_t m, int64_t* __restrict__ code_out,
+    int32_t* __restrict__ grid_coord_out, int64_t* __restrict__ batch_out) {
+    const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= m) return;
+    const int64_t h = head[j];
+    for (int r = 0; r < k; ++r) code_out[(int64_t)r * m + j] = code[(int64_t)r * n + h] >> shift;
+    if (grid_coord_out) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) grid_coord_out[3 * j + a] = grid_coord[3 * h + a] >> pool_depth;
+    }
+    if (batch_out) batch_out[j] = batch[h];
+}
+
+template <typename T> __device__ __forceinline__ float ld(const T* p) { return (float)*p; }
+template <typename T> __device__ __forceinline__ void st(T* p, float v) { *p = (T)v; }
+
+template <typename T>
+__global__ __launch_bounds__(256) void segment_reduce_kernel(
+    const T* __restrict__ src, int c, const int64_t* __restrict__ indices,
+    const int64_t* __restrict__ idx_ptr, int64_t m, int op, T* __restrict__ out) {
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= m * c) return;
+    const int64_t s = e / c;
+    const int ch = (int)(e - s * c);
+    const int64_t b = idx_ptr[s], t = idx_ptr[s + 1];
+    float acc = (op == 0) ? -INFINITY : (op == 3 ? INFINITY : 0.f);
+    for (int64_t j = b; j < t; ++j) {
+        const float v = ld(src + indices[j] * c + ch);
+        acc = (op == 0) ? fmaxf(acc, v) : (op == 3 ? fminf(acc, v) : acc + v);
+    }
+    if (op == 1 && t > b) acc /= (float)(t - b);
+    if (t == b) acc = 0.f;
+    st(out + e, acc);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void unpool_add_kernel(const T* __restrict__ parent,
+                                                         const T* __restrict__ child, int64_t n,
+                                                         int c, const int64_t* __restrict__ cluster,
+                                                         T* __restrict__ out) {
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n * c) return;
+    const int64_t i = e / c;
+    const int ch = (int)(e - i * c);
+    st(out + e, ld(parent + e) + ld(child + cluster[i] * c + ch));
+}
+
+}  // namespace
+
+extern "C" size_t ptv3_pool_clusters_workspace_bytes(int64_t n) {
+    if (n < 0) return 0;
+    return ptv3_align256((size_t)(ptv3_ceil_div(n > 0 ? n : 1, PB)) * sizeof(uint32_t));
+}
+
+extern "C" int ptv3_pool_clusters(const int64_t* code0, const int64_t* order0, int64_t n, int shift,
+                                  int64_t* cluster, int64_t* idx_ptr, int64_t* head,
+                                  int64_t* n_clusters, void* workspace, size_t workspace_bytes,
+                                  void* stream_) {
+    if (n < 1 || n >= (1ll << 31) || shift < 0 || shift > 62) return PTV3_EINVAL;
+    if (!code0 || !order0 || !cluster || !idx_ptr || !head || !n_clusters || !workspace) return PTV3_EINVAL;
+    if (workspace_bytes < ptv3_pool_clusters_workspace_bytes(n)) return PTV3_EWORKSPACE;
+    hipStream_t stream = (hipStream_t)stream_;
+    const int64_t blocks = ptv3_ceil_div(n, PB);
+    uint32_t* block_cnt = (uint32_t*)workspace;
+    hipLaunchKernelGGL(cluster_count_kernel, dim3((unsigned)blocks), dim3(PB), 0, stream, code0, order0, n,
+                       shift, block_cnt);
+    hipLaunchKernelGGL(cluster_scan_kernel, dim3(1), dim3(PB), 0, stream, block_cnt, blocks, n_clusters);
+    hipLaunchKernelGGL(cluster_assign_kernel, dim3((unsigned)blocks), dim3(PB), 0, stream, code0, order0, n,
+                       shift, (const uint32_t*)block_cnt, cluster, idx_ptr, head);
+    PTV3_RETURN_LAUNCH();
+}
+
+extern "C" int ptv3_pool_gather(const int64_t* code, int64_t n, int k, int shift,
+                                const int32_t* grid_coord, int pool_depth, const int64_t* batch,
+                                const int64_t* head, int64_t m, int64_t* code_out,
+                                int32_t* grid_coord_out, int64_t* batch_out, void* stream) {
+    if (n < 0 || m < 0 || m > n || k < 1 || shift < 0 || shift > 62 || pool_depth < 0 || pool_depth > 31)
+        return PTV3_EINVAL;
+    if (m == 0) return PTV3_OK;
+    if (!code || !head || !code_out) return PTV3_EINVAL;
+    if ((grid_coord_out && !grid_coord) || (batch_out && !batch)) return PTV3_EINVAL;
+    hipLaunchKernelGGL(pool_gather_kernel, dim3((unsigned)ptv3_ceil_div(m, 256)), dim3(256), 0,
+                       (hipStream_t)stream, code, n, k, shift, grid_coord, pool_depth, batch, head, m,
+                       code_out, grid_coord_out, batch_out);
+    PTV3_RETURN_LAUNCH();
+}
+
+extern "C" int ptv3_segment_reduce(const void* src, int dtype, int64_t n, int c,
+                                   const int64_t* indices, const int64_t* idx_ptr, int64_t m, int op,
+                                   void* out, void* stream_) {
+    if (n < 0 || m < 0 || c < 1 || op < 0 || op > 3) return PTV3_EINVAL;
+    if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
+    if (m == 0) return PTV3_OK;
+    if (!src || !indices || !idx_ptr || !out) return PTV3_EINVAL;
+    hipStream_t stream = (hipStream_t)stream_;
+    const dim3 grid((unsigned)ptv3_ceil_div(m * c, 256)), block(256);
+    if (dtype == PTV3_F32)
+        hipLaunchKernelGGL(segment_reduce_kernel<float>, grid, block, 0, stream, (const float*)src, c,
+                           indices, idx_ptr, m, op, (float*)out);
+    else if (dtype == PTV3_F16)
+        hipLaunchKernelGGL(segment_reduce_kernel<_Float16>, grid, block, 0, stream, (const _Float16*)src,
+                           c, indices, idx_ptr, m, op, (_Float16*)out);
+    else
+        hipLaunchKernelGGL(segment_reduce_kernel<__bf16>, grid, block, 0, stream, (const __bf16*)src, c,
+                           indices, idx_ptr, m, op, (__bf16*)out);
+    PTV3_RETURN_LAUNCH();
+}
+
+extern "C" int ptv3_unpool_add(const void* parent, const void* child, int dtype, int64_t n, int c,
+                               const int64_t* cluster, int64_t m, void* out, void* stream_) {
+    if (n < 0 || m < 0 || c < 1) return PTV3_EINVAL;
+    if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
+    if (n == 0) return PTV3_OK;
+    if (!parent || !child || !cluster || !out) return PTV3_EINVAL;
+    hipStream_t stream = (hipStream_t)stream_;
+    const dim3 grid((unsigned)ptv3_ceil_div(n * c, 256)), block(256);
+    if (dtype == PTV3_F32)
+        hipLaunchKernelGGL(unpool_add_kernel<float>, grid, block, 0, stream, (const float*)parent,
+                           (const float*)child, n, c, cluster, (float*)out);
+    else if (dtype == PTV3_F16)
+        hipLaunchKernelGGL(unpool_add_kernel<_Float16>, grid, block, 0, stream, (const _Float16*)parent,
+                           (const _Float16*)child, n, c, cluster, (_Float16*)out);
+    else
+        hipLaunchKernelGGL(unpool_add_kernel<__bf16>, grid, block, 0, stream, (const __bf16*)parent,
+                           (const __bf16*)child, n, c, cluster, (__bf16*)out);
+    PTV3_RETURN_LAUNCH();
+}

@@ -1,0 +1,203 @@
+// Batched LSD radix argsort of (k, n) int64 curve codes, with the inverse permutation
+// produced by the last pass.
+//
+// Replaces torch.argsort + scatter_ at model.py:119-126 and :667-674 of the reference.
+// Only the significant low bits are sorted (3*depth + batch bits, e.g. 29 instead of 64),
+// 8 bits per pass; all k rows share every launch (blockIdx.y = row). A pass is
+//   tile_hist  : per-tile digit histogram (LDS atomics)
+//   tile_scan  : per row, exclusive scan over (digit, tile) -> global start of every
+//                (tile, digit) run
+//   scatter    : stable rank inside the tile by wave-level digit matching, then one write
+// The payload between passes is a 32-bit point index; int64 order/inverse appear only in
+// the last pass.
+#include "common.h"
+
+namespace {
+
+constexpr int RADIX = 256;
+constexpr int SORT_THREADS = 256;
+constexpr int SORT_WAVES = SORT_THREADS / PTV3_WAVE;
+constexpr int SORT_ITEMS = 8;
+constexpr int SORT_TILE = SORT_THREADS * SORT_ITEMS;
+
+__global__ __launch_bounds__(SORT_THREADS) void tile_hist_kernel(
+    const int64_t* __restrict__ keys, int64_t n, int shift, uint32_t* __restrict__ tile_hist,
+    int tiles) {
+    __shared__ uint32_t hist[RADIX];
+    const int row = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
+    hist[tid] = 0;
+    __syncthreads();
+    const int64_t base = (int64_t)tile * SORT_TILE;
+    const int64_t* src = keys + (int64_t)row * n;
+#pragma unroll
+    for (int j = 0; j < SORT_ITEMS; ++j) {
+        const int64_t i = base + j * SORT_THREADS + tid;
+        if (i < n) atomicAdd(&hist[(uint32_t)((uint64_t)src[i] >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    tile_hist[((int64_t)row * tiles + tile) * RADIX + tid] = hist[tid];
+}
+
+// One block per row. Thread d owns digit d: serial exclusive scan over the tiles, then a
+// block-wide exclusive scan over the digit totals; the digit base is folded back in.
+__global__ __launch_bounds__(RADIX) void tile_scan_kernel(uint32_t* __restrict__ tile_hist,
+                                                          int tiles) {
+    __shared__ uint32_t total[RADIX];
+    const int row = blockIdx.x, d = threadIdx.x;
+    uint32_t* h = tile_hist + (int64_t)row * tiles * RADIX;
+    uint32_t run = 0;
+    for (int t = 0; t < tiles; ++t) {
+        const uint32_t c = h[(int64_t)t * RADIX + d];
+        h[(int64_t)t * RADIX + d] = run;
+        run += c;
+    }
+    total[d] = run;
+    __syncthreads();
+    // Hillis-Steele inclusive scan over 256 digit totals
+    for (int off = 1; off < RADIX; off <<= 1) {
+        const uint32_t v = (d >= off) ? total[d - off] : 0u;
+        __syncthreads();
+        total[d] += v;
+        __syncthreads();
+    }
+    const uint32_t dbase = total[d] - run;
+    if (dbase != 0)
+        for (int t = 0; t < tiles; ++t) h[(int64_t)t * RADIX + d] += dbase;
+}
+
+template <bool FIRST, bool LAST>
+__global__ __launch_bounds__(SORT_THREADS) void scatter_kernel(
+    const int64_t* __restrict__ keys_in, const int32_t* __restrict__ idx_in, int64_t n, int shift,
+    const uint32_t* __restrict__ tile_off, int tiles, int64_t* __restrict__ keys_out,
+    int32_t* __restrict__ idx_out, int64_t* __restrict__ order, int64_t* __restrict__ inverse) {
+    __shared__ uint32_t whist[SORT_WAVES][RADIX];
+    const int row = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
+    const int wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
+    for (int w = 0; w < SORT_WAVES; ++w) whist[w][tid] = 0;
+    __syncthreads();
+
+    const int64_t rbase = (int64_t)row * n;
+    const int64_t wbase = (int64_t)tile * SORT_TILE + (int64_t)wave * (PTV3_WAVE * SORT_ITEMS);
+    int64_t key[SORT_ITEMS];
+    int32_t idx[SORT_ITEMS];
+    uint32_t rank[SORT_ITEMS];
+    const uint64_t below = (1ull << lane) - 1ull;
+
+#pragma unroll
+    for (int j = 0; j < SORT_ITEMS; ++j) {
+        const int64_t i = wbase + j * PTV3_WAVE + lane;
+        const bool valid = i < n;
+        key[j] = valid ? keys_in[rbase + i] : 0;
+        idx[j] = FIRST ? (int32_t)i : (valid ? idx_in[rbase + i] : 0);
+        const uint32_t digit = (uint32_t)((uint64_t)key[j] >> shift) & 255u;
+        uint64_t peers = __ballot(valid);
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const bool bit = (digit >> b) & 1u;
+            const uint64_t bal = __ballot(bit);
+            peers &= bit ? bal : ~bal;
+        }
+        // peers: valid lanes of this wave whose digit equals mine (meaningless if !valid)
+        const int leader = __ffsll((unsigned long long)peers) - 1;
+        uint32_t pre = 0;
+        if (valid && lane == leader) pre = atomicAdd(&whist[wave][digit], (uint32_t)__popcll(peers));
+        pre = __shfl(pre, leader < 0 ? 0 : leader, PTV3_WAVE);
+        rank[j] = pre + (uint32_t)__popcll(peers & below);
+    }
+    __syncthreads();
+    {
+        // digit `tid`: turn per-wave counts into global starts of each wave's run
+        uint32_t run = tile_off[((int64_t)row * tiles + tile) * RADIX + tid];
+        for (int w = 0; w < SORT_WAVES; ++w) {
+            const uint32_t c = whist[w][tid];
+            whist[w][tid] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < SORT_ITEMS; ++j) {
+        const int64_t i = wbase + j * PTV3_WAVE + lane;
+        if (i < n) {
+            const uint32_t digit = (uint32_t)((uint64_t)key[j] >> shift) & 255u;
+            const int64_t pos = (int64_t)whist[wave][digit] + rank[j];
+            if (LAST) {
+                order[rbase + pos] = idx[j];
+                inverse[rbase + idx[j]] = pos;
+            } else {
+                keys_out[rbase + pos] = key[j];
+                idx_out[rbase + pos] = idx[j];
+            }
+        }
+    }
+}
+
+struct SortWs {
+    int64_t* keys[2];
+    int32_t* idx[2];
+    uint32_t* tile_hist;
+    size_t bytes;
+};
+
+SortWs carve(void* base, int64_t n, int k) {
+    SortWs w;
+    const int64_t tiles = ptv3_ceil_div(n > 0 ? n : 1, SORT_TILE);
+    size_t off = 0;
+    char* p = (char*)base;
+    for (int i = 0; i < 2; ++i) {
+        w.keys[i] = (int64_t*)(p + off);
+        off += ptv3_align256((size_t)k * n * sizeof(int64_t));
+    }
+    for (int i = 0; i < 2; ++i) {
+        w.idx[i] = (int32_t*)(p + off);
+        off += ptv3_align256((size_t)k * n * sizeof(int32_t));
+    }
+    w.tile_hist = (uint32_t*)(p + off);
+    off += ptv3_align256((size_t)k * tiles * RADIX * sizeof(uint32_t));
+    w.bytes = off;
+    return w;
+}
+
+}  // namespace
+
+extern "C" size_t ptv3_argsort_workspace_bytes(int64_t n, int k) {
+    if (n < 0 || k < 1) return 0;
+    return carve(nullptr, n, k).bytes;
+}
+
+extern "C" int ptv3_argsort(const int64_t* code, int64_t n, int k, int key_bits, int64_t* order,
+                            int64_t* inverse, void* workspace, size_t workspace_bytes,
+                            void* stream_) {
+    if (n < 0 || k < 1 || k > 65535 || n >= (1ll << 31)) return PTV3_EINVAL;
+    if (key_bits < 1 || key_bits > 63) return PTV3_EDEPTH;
+    if (n == 0) return PTV3_OK;
+    if (!code || !order || !inverse || !workspace) return PTV3_EINVAL;
+    SortWs w = carve(workspace, n, k);
+    if (workspace_bytes < w.bytes) return PTV3_EWORKSPACE;
+    hipStream_t stream = (hipStream_t)stream_;
+    const int tiles = (int)ptv3_ceil_div(n, SORT_TILE);
+    const int passes = (key_bits + 7) / 8;
+    const dim3 grid((unsigned)tiles, (unsigned)k), block(SORT_THREADS);
+
+    const int64_t* kin = code;
+    const int32_t* iin = nullptr;
+    for (int p = 0; p < passes; ++p) {
+        const int shift = 8 * p;
+        const bool first = (p == 0), last = (p == passes - 1);
+        int64_t* kout = w.keys[p & 1];
+        int32_t* iout = w.idx[p & 1];
+        hipLaunchKernelGGL(tile_hist_kernel, grid, block, 0, stream, kin, n, shift, w.tile_hist, tiles);
+        hipLaunchKernelGGL(tile_scan_kernel, dim3((unsigned)k), dim3(RADIX), 0, stream, w.tile_hist, tiles);
+#define PTV3_SCATTER(F, L)                                                                    \
+    hipLaunchKernelGGL((scatter_kernel<F, L>), grid, block, 0, stream, kin, iin, n, shift,    \
+                       (const uint32_t*)w.tile_hist, tiles, kout, iout, order, inverse)
+        if (first && last) PTV3_SCATTER(true, true);
+        else if (first) PTV3_SCATTER(true, false);
+        else if (last) PTV3_SCATTER(false, true);
+        else PTV3_SCATTER(false, false);
+#undef PTV3_SCATTER
+        kin = kout;
+        iin = iout;
+    }
+    PTV3_RETURN_LAUNCH();
+}

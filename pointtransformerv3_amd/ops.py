@@ -1,0 +1,225 @@
+"""torch-tensor wrappers over the C ABI of libptv3_hip.so.
+
+torch is used for device memory and the current stream only; every computation happens in
+the HIP kernels. All tensors must live on the GPU; CPU tensors are rejected.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+ORDER_IDS = {"z": 0, "z-trans": 1, "hilbert": 2, "hilbert-trans": 3}
+_DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+REDUCE_OPS = {"max": 0, "mean": 1, "sum": 2, "min": 3}
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise _lib.Ptv3Error("ptv3 ops run on the GPU only; got a CPU tensor (there is no CPU fallback)")
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _ws(nbytes, device):
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
+def _dtype_code(t):
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise _lib.Ptv3Error(f"unsupported dtype {t.dtype}") from None
+
+
+def encode_orders(grid_coord, batch, depth, orders):
+    """All requested curve codes in one pass: returns (k, N) int64."""
+    _dev(grid_coord, batch)
+    lib = _lib.load()
+    g = grid_coord.to(torch.int32).contiguous()
+    b = None if batch is None else batch.to(torch.int64).contiguous()
+    n, k = g.shape[0], len(orders)
+    ids = (ctypes.c_int32 * k)(*[ORDER_IDS[o] for o in orders])
+    code = torch.empty((k, n), dtype=torch.int64, device=g.device)
+    _lib.check(lib.ptv3_encode(_ptr(g), _ptr(b), n, int(depth), ids, k, _ptr(code), _stream()),
+               "ptv3_encode")
+    return code
+
+
+def argsort_rows(code, key_bits):
+    """Row-wise ascending argsort of (k,N) int64 codes + inverse permutation."""
+    _dev(code)
+    lib = _lib.load()
+    code = code.contiguous()
+    k, n = code.shape
+    order = torch.empty_like(code)
+    inverse = torch.empty_like(code)
+    nbytes = lib.ptv3_argsort_workspace_bytes(n, k)
+    ws = _ws(nbytes, code.device)
+    _lib.check(lib.ptv3_argsort(_ptr(code), n, k, int(key_bits), _ptr(order), _ptr(inverse), _ptr(ws),
+                                nbytes, _stream()), "ptv3_argsort")
+    return order, inverse
+
+
+def pad_sizes(offset_host, patch):
+    """(n_pad, n_seq) from a host list of cumulative scene ends."""
+    lib = _lib.load()
+    nb = len(offset_host)
+    arr = (ctypes.c_int64 * nb)(*[int(v) for v in offset_host])
+    n_pad, n_seq = ctypes.c_int64(0), ctypes.c_int64(0)
+    _lib.check(lib.ptv3_pad_sizes(arr, nb, int(patch), ctypes.byref(n_pad), ctypes.byref(n_seq)),
+               "ptv3_pad_sizes")
+    return n_pad.value, n_seq.value
+
+
+def pad_index(offset, offset_host, patch):
+    """pad (Npad,), unpad (N,), cu_seqlens (P+1,) int32 for the scenes in `offset`."""
+    _dev(offset)
+    lib = _lib.load()
+    offset = offset.to(torch.int64).contiguous()
+    nb = len(offset_host)
+    n = int(offset_host[-1])
+    n_pad, n_seq = pad_sizes(offset_host, patch)
+    dev = offset.device
+    pad = torch.empty(n_pad, dtype=torch.int64, device=dev)
+    unpad = torch.empty(n, dtype=torch.int64, device=dev)
+    cu = torch.empty(n_seq + 1, dtype=torch.int32, device=dev)
+    nbytes = lib.ptv3_pad_index_workspace_bytes(nb)
+    ws = _ws(nbytes, dev)
+    _lib.check(lib.ptv3_pad_index(_ptr(offset), nb, int(patch), n, n_pad, n_seq, _ptr(pad), _ptr(unpad),
+                                  _ptr(cu), _ptr(ws), nbytes, _stream()), "ptv3_pad_index")
+    return pad, unpad, cu
+
+
+def attn_slots(order_row, inverse_row, pad, unpad):
+    """int32 gather (slot_src) and scatter (slot_dst, -1 for filler slots) tables."""
+    _dev(order_row, inverse_row, pad, unpad)
+    lib = _lib.load()
+    n_pad = pad.shape[0]
+    src = torch.empty(n_pad, dtype=torch.int32, device=pad.device)
+    dst = torch.empty(n_pad, dtype=torch.int32, device=pad.device)
+    _lib.check(lib.ptv3_attn_slots(_ptr(order_row.contiguous()), _ptr(inverse_row.contiguous()),
+                                   _ptr(pad), _ptr(unpad), n_pad, _ptr(src), _ptr(dst), _stream()),
+               "ptv3_attn_slots")
+    return src, dst
+
+
+def patch_attention(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale):
+    """softmax(q k^T * scale) v inside each sequence; qkv (N, 3C) in point order, result (N, C)
+    in point order (gather and scatter fused into the kernel)."""
+    _dev(qkv, slot_src, slot_dst, cu_seqlens)
+    lib = _lib.load()
+    qkv = qkv.contiguous()
+    n, c3 = qkv.shape
+    c = c3 // 3
+    out = torch.empty((n, c), dtype=qkv.dtype, device=qkv.device)
+    n_seq = cu_seqlens.shape[0] - 1
+    _lib.check(lib.ptv3_patch_attn_fwd(_ptr(qkv), _dtype_code(qkv), n, c, int(num_heads), _ptr(slot_src),
+                                       _ptr(slot_dst), _ptr(cu_seqlens), n_seq, int(max_seqlen),
+                                       float(scale), _ptr(out), _stream()), "ptv3_patch_attn_fwd")
+    return out
+
+
+def kmap_build(indices, ks):
+    """(N, ks^3) int32 neighbour map of (N,4) int32 [batch,x,y,z] voxels."""
+    _dev(indices)
+    lib = _lib.load()
+    idx = indices.to(torch.int32).contiguous()
+    n = idx.shape[0]
+    nbr = torch.empty((n, ks ** 3), dtype=torch.int32, device=idx.device)
+    nbytes = lib.ptv3_kmap_workspace_bytes(n)
+    ws = _ws(nbytes, idx.device)
+    _lib.check(lib.ptv3_kmap_build(_ptr(idx), n, int(ks), _ptr(nbr), _ptr(ws), nbytes, _stream()),
+               "ptv3_kmap_build")
+    return nbr
+
+
+def subm_conv(feat, nbr, weight, bias=None):
+    """feat (N,Cin), nbr (N,V) int32, weight (Cout,V,Cin) or (Cout,k,k,k,Cin), bias (Cout,)."""
+    _dev(feat, nbr, weight, bias)
+    lib = _lib.load()
+    feat = feat.contiguous()
+    n, cin = feat.shape
+    cout = weight.shape[0]
+    taps = nbr.shape[1]
+    w = weight.reshape(cout, taps, cin).to(feat.dtype).contiguous()
+    b = None if bias is None else bias.to(feat.dtype).contiguous()
+    out = torch.empty((n, cout), dtype=feat.dtype, device=feat.device)
+    _lib.check(lib.ptv3_subm_conv_fwd(_ptr(feat), _dtype_code(feat), n, cin, _ptr(nbr), taps, _ptr(w),
+                                      _ptr(b), cout, _ptr(out), _stream()), "ptv3_subm_conv_fwd")
+    return out
+
+
+def pool_clusters(code0, order0, shift):
+    """Clusters of code0 >> shift in sorted order. One host sync (the cluster count).
+
+    Returns cluster (N,), idx_ptr (M+1,), head (M,), M."""
+    _dev(code0, order0)
+    lib = _lib.load()
+    n = code0.shape[0]
+    dev = code0.device
+    cluster = torch.empty(n, dtype=torch.int64, device=dev)
+    idx_ptr = torch.empty(n + 1, dtype=torch.int64, device=dev)
+    head = torch.empty(n, dtype=torch.int64, device=dev)
+    count = torch.empty(1, dtype=torch.int64, device=dev)
+    nbytes = lib.ptv3_pool_clusters_workspace_bytes(n)
+    ws = _ws(nbytes, dev)
+    _lib.check(lib.ptv3_pool_clusters(_ptr(code0.contiguous()), _ptr(order0.contiguous()), n, int(shift),
+                                      _ptr(cluster), _ptr(idx_ptr), _ptr(head), _ptr(count), _ptr(ws),
+                                      nbytes, _stream()), "ptv3_pool_clusters")
+    m = int(count.item())
+    return cluster, idx_ptr[: m + 1], head[:m], m
+
+
+def pool_gather(code, shift, grid_coord, pool_depth, batch, head):
+    """Pooled code (k,M), grid_coord (M,3) int32, batch (M,) at the cluster heads."""
+    _dev(code, grid_coord, batch, head)
+    lib = _lib.load()
+    code = code.contiguous()
+    k, n = code.shape
+    m = head.shape[0]
+    dev = code.device
+    code_out = torch.empty((k, m), dtype=torch.int64, device=dev)
+    gc = grid_coord.to(torch.int32).contiguous()
+    gc_out = torch.empty((m, 3), dtype=torch.int32, device=dev)
+    b = batch.to(torch.int64).contiguous()
+    b_out = torch.empty(m, dtype=torch.int64, device=dev)
+    _lib.check(lib.ptv3_pool_gather(_ptr(code), n, k, int(shift), _ptr(gc), int(pool_depth), _ptr(b),
+                                    _ptr(head.contiguous()), m, _ptr(code_out), _ptr(gc_out), _ptr(b_out),
+                                    _stream()), "ptv3_pool_gather")
+    return code_out, gc_out, b_out
+
+
+def segment_reduce(src, indices, idx_ptr, reduce="max"):
+    """reduce(src[indices[idx_ptr[s]:idx_ptr[s+1]]]) per segment."""
+    _dev(src, indices, idx_ptr)
+    lib = _lib.load()
+    src = src.contiguous()
+    n, c = src.shape
+    m = idx_ptr.shape[0] - 1
+    out = torch.empty((m, c), dtype=src.dtype, device=src.device)
+    _lib.check(lib.ptv3_segment_reduce(_ptr(src), _dtype_code(src), n, c, _ptr(indices.contiguous()),
+                                       _ptr(idx_ptr.contiguous()), m, REDUCE_OPS[reduce], _ptr(out),
+                                       _stream()), "ptv3_segment_reduce")
+    return out
+
+
+def unpool_add(parent, child, cluster):
+    """parent + child[cluster]."""
+    _dev(parent, child, cluster)
+    lib = _lib.load()
+    parent = parent.contiguous()
+    child = child.to(parent.dtype).contiguous()
+    n, c = parent.shape
+    out = torch.empty_like(parent)
+    _lib.check(lib.ptv3_unpool_add(_ptr(parent), _ptr(child), _dtype_code(parent), n, c,
+                                   _ptr(cluster.contiguous()), child.shape[0], _ptr(out), _stream()),
+               "ptv3_unpool_add")
+    return out

@@ -1,0 +1,115 @@
+"""HIP encode / argsort / padding tables vs the CPU oracle: bit-exact."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import indexing as OI
+from oracle import serialization as OS
+from gpu_util import DEV, to_dev, unique_voxels
+
+pytestmark = pytest.mark.gpu
+
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "hilbert_golden.npz"))
+
+
+def ops():
+    from pointtransformerv3_amd import ops as _ops
+    return _ops
+
+
+@pytest.mark.parametrize("name", sorted(k[:-3] for k in GOLD.files if k.endswith("_in")))
+def test_hilbert_kernel_matches_reference_golden(name):
+    depth = int(name.split("_d")[1])
+    got = ops().encode_orders(to_dev(GOLD[name + "_in"]), None, depth, ["hilbert"])[0]
+    assert np.array_equal(got.cpu().numpy(), GOLD[name + "_out"])
+
+
+@pytest.mark.parametrize("depth", [1, 4, 8, 9, 12, 16])
+@pytest.mark.parametrize("n", [1, 63, 100_003])
+def test_encode_all_orders(depth, n):
+    rng = np.random.default_rng(depth * 1000 + n)
+    g = rng.integers(0, 1 << 16, size=(n, 3)).astype(np.int32)   # wider than depth: low bits are kept
+    b = rng.integers(0, 4, size=n).astype(np.int64)
+    got = ops().encode_orders(to_dev(g), to_dev(b), depth, list(OS.ORDERS)).cpu().numpy()
+    for r, name in enumerate(OS.ORDERS):
+        assert np.array_equal(got[r], OS.encode(g, b, depth, name)), name
+    got1 = ops().encode_orders(to_dev(g), None, depth, ["hilbert-trans", "z"]).cpu().numpy()
+    assert np.array_equal(got1[0], OS.encode(g, None, depth, "hilbert-trans"))
+    assert np.array_equal(got1[1], OS.encode(g, None, depth, "z"))
+
+
+def test_encode_mirror_of_reference_signature():
+    from pointtransformerv3_amd.serialization import encode
+    g = np.array([[1, 0, 0], [3, 0, 0], [256, 0, 0]], np.int32)
+    assert encode(to_dev(g), None, 16, "z").tolist() == [4, 36, 1 << 26]
+    b = to_dev(np.array([3, 3, 3], np.int64))
+    assert encode(to_dev(g), b, 16, "z").tolist() == [(3 << 48) | 4, (3 << 48) | 36, (3 << 48) | (1 << 26)]
+
+
+def test_encode_rejects_bad_depth_and_cpu_tensors():
+    from pointtransformerv3_amd._lib import Ptv3Error
+    g = to_dev(np.zeros((4, 3), np.int32))
+    with pytest.raises(Ptv3Error):
+        ops().encode_orders(g, None, 17, ["z"])
+    with pytest.raises(Ptv3Error):
+        ops().encode_orders(g.cpu(), None, 8, ["z"])
+
+
+@pytest.mark.parametrize("n,extent,nb", [(1, 4, 1), (2047, 32, 1), (2049, 32, 2), (50_000, 64, 3)])
+def test_argsort_unique_codes_bit_exact(n, extent, nb):
+    rng = np.random.default_rng(n)
+    g, batch, _ = unique_voxels(rng, n, extent, nb)
+    depth, code, order, inverse = OS.serialize(g, batch)
+    key_bits = 3 * depth + max(1, (nb - 1).bit_length())
+    o, inv = ops().argsort_rows(to_dev(code), key_bits)
+    assert np.array_equal(o.cpu().numpy(), order)
+    assert np.array_equal(inv.cpu().numpy(), inverse)
+
+
+def test_argsort_full_size_properties():
+    # 4 x 100k-point scenes worth of codes at depth 16: sortedness + permutation validity
+    rng = np.random.default_rng(5)
+    n = 400_000
+    g, batch, _ = unique_voxels(rng, n // 4, 200, 4)
+    code = np.stack([OS.encode(g, batch, 16, o) for o in OS.ORDERS])
+    o, inv = ops().argsort_rows(to_dev(code), 3 * 16 + 2)
+    o, inv = o.cpu().numpy(), inv.cpu().numpy()
+    for r in range(4):
+        assert np.all(np.diff(code[r][o[r]]) > 0)
+        assert np.array_equal(inv[r][o[r]], np.arange(n))
+    assert np.array_equal(o, np.argsort(code, axis=1, kind="stable"))
+
+
+def test_argsort_ties_are_stable():
+    rng = np.random.default_rng(8)
+    code = rng.integers(0, 50, size=(2, 10_000)).astype(np.int64)
+    o, inv = ops().argsort_rows(to_dev(code), 6)
+    assert np.array_equal(o.cpu().numpy(), np.argsort(code, axis=1, kind="stable"))
+
+
+@pytest.mark.parametrize("counts,patch", [([2500], 1024), ([1500], 1024), ([1024], 1024), ([700], 1024),
+                                          ([1300, 700, 2049], 512), ([5, 0, 40], 16), ([100_000], 1024)])
+def test_pad_index(counts, patch):
+    offset = np.cumsum(counts).astype(np.int64)
+    pad, unpad, cu = OI.padding_tables(offset, patch)
+    gp, gu, gc = ops().pad_index(to_dev(offset), offset.tolist(), patch)
+    assert np.array_equal(gp.cpu().numpy(), pad)
+    assert np.array_equal(gu.cpu().numpy(), unpad)
+    assert gc.dtype == torch.int32 and np.array_equal(gc.cpu().numpy(), cu)
+
+
+def test_attn_slots():
+    rng = np.random.default_rng(1)
+    n, patch = 2500, 1024
+    order = rng.permutation(n).astype(np.int64)
+    inverse = np.empty(n, np.int64)
+    inverse[order] = np.arange(n)
+    pad, unpad, _ = OI.padding_tables([n], patch)
+    src, dst = ops().attn_slots(to_dev(order), to_dev(inverse), to_dev(pad), to_dev(unpad))
+    want_src = order[pad]
+    primary = unpad[inverse[want_src]] == np.arange(len(pad))
+    assert np.array_equal(src.cpu().numpy(), want_src)
+    assert np.array_equal(dst.cpu().numpy(), np.where(primary, want_src, -1))
+    assert primary.sum() == n

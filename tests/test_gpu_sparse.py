@@ -1,0 +1,101 @@
+"""HIP kmap / submanifold conv / pooling kernels vs the CPU oracle.
+Integer outputs bit-exact; conv within 1e-4 (fp32) / 2e-2 (fp16, bf16) max-abs relative."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import functional as OF
+from oracle import indexing as OI
+from oracle import serialization as OS
+from gpu_util import DEV, rel_err, to_dev, unique_voxels
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-4, torch.float16: 2e-2, torch.bfloat16: 2e-2}
+
+
+def ops():
+    from pointtransformerv3_amd import ops as _ops
+    return _ops
+
+
+def _indices(rng, n, extent, nb):
+    g, batch, offset = unique_voxels(rng, n, extent, nb)
+    return np.concatenate([batch[:, None].astype(np.int32), g], 1), g, batch, offset
+
+
+@pytest.mark.parametrize("ks", [3, 5])
+@pytest.mark.parametrize("n,extent,nb", [(1, 4, 1), (500, 10, 2), (30_000, 48, 2)])
+def test_kmap_bit_exact(ks, n, extent, nb):
+    rng = np.random.default_rng(n + ks)
+    idx, *_ = _indices(rng, n, extent, nb)
+    got = ops().kmap_build(to_dev(idx), ks).cpu().numpy()
+    assert np.array_equal(got, OI.subm_kmap(idx, ks))
+
+
+def test_kmap_room_200k_properties():
+    from pointtransformerv3_amd import synthetic
+    g = synthetic.room_voxels(200_000, 3000)["grid_coord"]
+    idx = np.concatenate([np.zeros((len(g), 1), np.int32), g], 1)
+    got = ops().kmap_build(to_dev(idx), 3).cpu().numpy()
+    assert np.array_equal(got[:, 13], np.arange(len(g)))
+    i, k = np.nonzero(got >= 0)
+    assert np.array_equal(got[got[i, k], 26 - k], i)
+    assert np.array_equal(got, OI.subm_kmap(idx, 3))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("ks,cin,cout,n", [(3, 32, 32, 3000), (3, 64, 64, 5000), (3, 128, 128, 700),
+                                           (5, 16, 32, 2000), (3, 64, 64, 70_000)])
+def test_subm_conv_parity(dtype, ks, cin, cout, n):
+    rng = np.random.default_rng(cin + n)
+    g = torch.Generator().manual_seed(cin + n)
+    idx, *_ = _indices(rng, n // 2, 40 if n > 10_000 else 14, 2)
+    nbr = OI.subm_kmap(idx, ks)
+    feat = torch.randn(len(idx), cin, generator=g).to(dtype)
+    bound = 1.0 / np.sqrt(ks ** 3 * cin)
+    w = ((torch.rand(cout, ks, ks, ks, cin, generator=g) * 2 - 1) * bound).to(dtype)
+    b = ((torch.rand(cout, generator=g) * 2 - 1) * bound).to(dtype) if ks == 3 else None
+    want = OF.subm_conv(feat.float(), nbr, w.float(), None if b is None else b.float())
+    got = ops().subm_conv(feat.to(DEV), to_dev(nbr), w.to(DEV), None if b is None else b.to(DEV))
+    assert got.dtype == dtype
+    assert rel_err(got, want) < TOL[dtype]
+
+
+def test_pool_clusters_and_gather_bit_exact():
+    rng = np.random.default_rng(4)
+    idx, g, batch, offset = _indices(rng, 20_000, 40, 3)
+    depth, code, order, inverse = OS.serialize(g, batch)
+    want = OI.pool_clusters(code, g, batch, 1)
+    o = ops()
+    cluster, idx_ptr, head, m = o.pool_clusters(to_dev(code[0]), to_dev(order[0]), 3)
+    assert m == len(want["counts"])
+    assert np.array_equal(cluster.cpu().numpy(), want["cluster"])
+    assert np.array_equal(idx_ptr.cpu().numpy(), want["idx_ptr"])
+    # any member may stand for its cluster; ours is the first in sorted order like the oracle's
+    assert np.array_equal(head.cpu().numpy(), want["head"])
+    pc, pg, pb = o.pool_gather(to_dev(code), 3, to_dev(g), 1, to_dev(batch), head)
+    assert np.array_equal(pc.cpu().numpy(), want["code"])
+    assert np.array_equal(pg.cpu().numpy(), want["grid_coord"])
+    assert np.array_equal(pb.cpu().numpy(), want["batch"])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_segment_reduce_and_unpool(dtype):
+    rng = np.random.default_rng(6)
+    g0 = torch.Generator().manual_seed(6)
+    idx, g, batch, offset = _indices(rng, 6000, 24, 2)
+    depth, code, order, inverse = OS.serialize(g, batch)
+    pc = OI.pool_clusters(code, g, batch, 1)
+    feat = torch.randn(len(g), 48, generator=g0).to(dtype)
+    o = ops()
+    got = o.segment_reduce(feat.to(DEV), to_dev(pc["indices"]), to_dev(pc["idx_ptr"]), "max")
+    want = OF.segment_csr(feat.float(), pc["indices"], pc["idx_ptr"], "max")
+    assert torch.equal(got.float().cpu(), want)   # max picks an input value: exact
+    coord = torch.rand(len(g), 3, generator=g0)
+    gotm = o.segment_reduce(coord.to(DEV), to_dev(pc["indices"]), to_dev(pc["idx_ptr"]), "mean")
+    assert rel_err(gotm, OF.segment_csr(coord, pc["indices"], pc["idx_ptr"], "mean")) < 1e-6
+    child = torch.randn(len(pc["counts"]), 48, generator=g0).to(dtype)
+    gotu = o.unpool_add(feat.to(DEV), child.to(DEV), to_dev(pc["cluster"]))
+    wantu = OF.unpool_add(feat.float(), child.float(), pc["cluster"])
+    assert rel_err(gotu, wantu) < (1e-6 if dtype == torch.float32 else 1e-2)
