@@ -72,8 +72,9 @@ def test_pool_clusters_and_gather_bit_exact():
     assert m == len(want["counts"])
     assert np.array_equal(cluster.cpu().numpy(), want["cluster"])
     assert np.array_equal(idx_ptr.cpu().numpy(), want["idx_ptr"])
-    # any member may stand for its cluster; ours is the first in sorted order like the oracle's
-    assert np.array_equal(head.cpu().numpy(), want["head"])
+    # the reference takes whichever member an unstable sort puts first (model.py:660-664);
+    # only values shared by all members are read through it, so membership is the contract
+    assert np.array_equal(want["cluster"][head.cpu().numpy()], np.arange(m))
     pc, pg, pb = o.pool_gather(to_dev(code), 3, to_dev(g), 1, to_dev(batch), head)
     assert np.array_equal(pc.cpu().numpy(), want["code"])
     assert np.array_equal(pg.cpu().numpy(), want["grid_coord"])
