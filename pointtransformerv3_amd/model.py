@@ -1,0 +1,120 @@
+"""PointTransformerV3 with the constructor and forward contract of model.py:786-982 of the
+reference, running on the gfx950 HIP kernels of this package."""
+from functools import partial
+
+import torch
+import torch.nn as nn
+
+from .modules import (MLP, Block, DropPath, Embedding, PDNorm, PointModule, PointSequential,  # noqa: F401
+                      SerializedAttention, SerializedPooling, SerializedUnpooling)
+from .point import Point, batch2offset, offset2batch, offset2bincount  # noqa: F401
+from .sparse import SparseConvTensor, SubMConv3d  # noqa: F401
+
+
+class PointTransformerV3(PointModule):
+    def __init__(
+        self,
+        in_channels=6,
+        order=("z", "z-trans", "hilbert", "hilbert-trans"),
+        stride=(2, 2, 2, 2),
+        enc_depths=(2, 2, 2, 6, 2),
+        enc_channels=(32, 64, 128, 256, 512),
+        enc_num_head=(2, 4, 8, 16, 32),
+        enc_patch_size=(1024, 1024, 1024, 1024, 1024),
+        dec_depths=(2, 2, 2, 2),
+        dec_channels=(64, 64, 128, 256),
+        dec_num_head=(4, 4, 8, 16),
+        dec_patch_size=(1024, 1024, 1024, 1024),
+        mlp_ratio=4,
+        qkv_bias=True,
+        qk_scale=None,
+        attn_drop=0.0,
+        proj_drop=0.0,
+        drop_path=0.3,
+        pre_norm=True,
+        shuffle_orders=True,
+        enable_rpe=False,
+        enable_flash=True,
+        upcast_attention=False,
+        upcast_softmax=False,
+        cls_mode=False,
+        pdnorm_bn=False,
+        pdnorm_ln=False,
+        pdnorm_decouple=True,
+        pdnorm_adaptive=False,
+        pdnorm_affine=True,
+        pdnorm_conditions=("ScanNet", "S3DIS", "Structured3D"),
+    ):
+        super().__init__()
+        self.num_stages = len(enc_depths)
+        self.order = [order] if isinstance(order, str) else order
+        self.cls_mode = cls_mode
+        self.shuffle_orders = shuffle_orders
+        n = self.num_stages
+        assert n == len(stride) + 1 == len(enc_channels) == len(enc_num_head) == len(enc_patch_size)
+        assert cls_mode or n == len(dec_depths) + 1 == len(dec_channels) + 1
+        assert cls_mode or n == len(dec_num_head) + 1 == len(dec_patch_size) + 1
+
+        pd = dict(conditions=pdnorm_conditions, decouple=pdnorm_decouple, adaptive=pdnorm_adaptive)
+        bn = partial(nn.BatchNorm1d, eps=1e-3, momentum=0.01)
+        if pdnorm_bn:
+            bn = partial(PDNorm, norm_layer=partial(nn.BatchNorm1d, eps=1e-3, momentum=0.01,
+                                                    affine=pdnorm_affine), **pd)
+        ln = nn.LayerNorm
+        if pdnorm_ln:
+            ln = partial(PDNorm, norm_layer=partial(nn.LayerNorm, elementwise_affine=pdnorm_affine), **pd)
+        act = nn.GELU
+
+        def make_block(channels, heads, patch, rate, i, stage):
+            return Block(channels=channels, num_heads=heads, patch_size=patch, mlp_ratio=mlp_ratio,
+                         qkv_bias=qkv_bias, qk_scale=qk_scale, attn_drop=attn_drop, proj_drop=proj_drop,
+                         drop_path=rate, norm_layer=ln, act_layer=act, pre_norm=pre_norm,
+                         order_index=i % len(self.order), cpe_indice_key=f"stage{stage}",
+                         enable_rpe=enable_rpe, enable_flash=enable_flash,
+                         upcast_attention=upcast_attention, upcast_softmax=upcast_softmax)
+
+        self.embedding = Embedding(in_channels=in_channels, embed_channels=enc_channels[0],
+                                   norm_layer=bn, act_layer=act)
+
+        # encoder: stochastic-depth rate grows linearly over all encoder blocks
+        rates = [r.item() for r in torch.linspace(0, drop_path, sum(enc_depths))]
+        self.enc = PointSequential()
+        for s in range(n):
+            stage = PointSequential()
+            if s > 0:
+                stage.add(SerializedPooling(in_channels=enc_channels[s - 1], out_channels=enc_channels[s],
+                                            stride=stride[s - 1], norm_layer=bn, act_layer=act), name="down")
+            first = sum(enc_depths[:s])
+            for i in range(enc_depths[s]):
+                stage.add(make_block(enc_channels[s], enc_num_head[s], enc_patch_size[s], rates[first + i], i, s),
+                          name=f"block{i}")
+            if len(stage) != 0:
+                self.enc.add(module=stage, name=f"enc{s}")
+
+        # decoder: walks the stages back up; rates are laid out per stage and reversed inside
+        if not cls_mode:
+            rates = [r.item() for r in torch.linspace(0, drop_path, sum(dec_depths))]
+            widths = list(dec_channels) + [enc_channels[-1]]
+            self.dec = PointSequential()
+            for s in reversed(range(n - 1)):
+                first = sum(dec_depths[:s])
+                stage_rates = rates[first:first + dec_depths[s]][::-1]
+                stage = PointSequential()
+                stage.add(SerializedUnpooling(in_channels=widths[s + 1], skip_channels=enc_channels[s],
+                                              out_channels=widths[s], norm_layer=bn, act_layer=act), name="up")
+                for i in range(dec_depths[s]):
+                    stage.add(make_block(widths[s], dec_num_head[s], dec_patch_size[s], stage_rates[i], i, s),
+                              name=f"block{i}")
+                self.dec.add(module=stage, name=f"dec{s}")
+
+    def forward(self, data_dict):
+        """data_dict: feat, grid_coord (or coord + grid_size), offset or batch. Returns the Point
+        whose feat is (N, dec_channels[0]) in the original point order."""
+        point = Point(data_dict)
+        point.serialization(order=self.order, shuffle_orders=self.shuffle_orders)
+        point.sparsify()
+        point = self.embedding(point)
+        point = self.enc(point)
+        if not self.cls_mode:
+            point = self.dec(point)
+        return point

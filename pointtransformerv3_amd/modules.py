@@ -1,0 +1,378 @@
+"""The building blocks of PTv3 as thin host glue over the HIP kernels.
+
+Module and parameter names follow model.py:177-783 of the reference, so its state_dicts load
+unchanged. Dense layers (Linear / LayerNorm / BatchNorm / GELU) are torch's; serialization,
+attention, sparse convolution and pooling run in libptv3_hip.so.
+"""
+import math
+from collections import OrderedDict
+
+import torch
+import torch.nn as nn
+
+from . import ops
+from .point import AttrDict, Point, offset2bincount
+from .sparse import SparseConvTensor, SubMConv3d, is_spconv_module
+
+
+class DropPath(nn.Module):
+    """Stochastic depth per sample row (stands in for timm's DropPath, model.py:17,583)."""
+
+    def __init__(self, drop_prob=0.0, scale_by_keep=True):
+        super().__init__()
+        self.drop_prob, self.scale_by_keep = drop_prob, scale_by_keep
+
+    def forward(self, x):
+        if self.drop_prob == 0.0 or not self.training:
+            return x
+        keep = 1.0 - self.drop_prob
+        mask = x.new_empty((x.shape[0],) + (1,) * (x.ndim - 1)).bernoulli_(keep)
+        if keep > 0.0 and self.scale_by_keep:
+            mask.div_(keep)
+        return x * mask
+
+
+class PointModule(nn.Module):
+    """Marker base class: PointSequential hands the whole Point to subclasses (model.py:177-183)."""
+
+
+class PointSequential(PointModule):
+    """Sequential container that knows three kinds of children (model.py:186-252):
+    PointModules get the Point, sparse convolutions get point.sparse_conv_feat, anything
+    else gets point.feat."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__()
+        if len(args) == 1 and isinstance(args[0], OrderedDict):
+            for name, module in args[0].items():
+                self.add_module(name, module)
+        else:
+            for i, module in enumerate(args):
+                self.add_module(str(i), module)
+        for name, module in kwargs.items():
+            if name in self._modules:
+                raise ValueError("name exists.")
+            self.add_module(name, module)
+
+    def __getitem__(self, idx):
+        if not (-len(self) <= idx < len(self)):
+            raise IndexError("index {} is out of range".format(idx))
+        return list(self._modules.values())[idx]
+
+    def __len__(self):
+        return len(self._modules)
+
+    def add(self, module, name=None):
+        if name is None:
+            name = str(len(self._modules))
+            if name in self._modules:
+                raise KeyError("name exists")
+        self.add_module(name, module)
+
+    def forward(self, input):
+        for module in self._modules.values():
+            if isinstance(module, PointModule):
+                input = module(input)
+            elif is_spconv_module(module):
+                if isinstance(input, Point):
+                    input.sparse_conv_feat = module(input.sparse_conv_feat)
+                    input.feat = input.sparse_conv_feat.features
+                else:
+                    input = module(input)
+            elif isinstance(input, Point):
+                input.feat = module(input.feat)
+                if "sparse_conv_feat" in input:
+                    input.sparse_conv_feat = input.sparse_conv_feat.replace_feature(input.feat)
+            elif isinstance(input, SparseConvTensor):
+                if input.indices.shape[0] != 0:
+                    input = input.replace_feature(module(input.features))
+            else:
+                input = module(input)
+        return input
+
+
+class PDNorm(PointModule):
+    """Per-dataset (de)coupled normalisation of PPT training (model.py:255-294); plain torch."""
+
+    def __init__(self, num_features, norm_layer, context_channels=256,
+                 conditions=("ScanNet", "S3DIS", "Structured3D"), decouple=True, adaptive=False):
+        super().__init__()
+        self.conditions, self.decouple, self.adaptive = conditions, decouple, adaptive
+        if decouple:
+            self.norm = nn.ModuleList([norm_layer(num_features) for _ in conditions])
+        else:
+            self.norm = norm_layer
+        if adaptive:
+            self.modulation = nn.Sequential(nn.SiLU(), nn.Linear(context_channels, 2 * num_features, bias=True))
+
+    def forward(self, point):
+        assert {"feat", "condition"}.issubset(point.keys())
+        condition = point.condition if isinstance(point.condition, str) else point.condition[0]
+        if self.decouple:
+            assert condition in self.conditions
+            norm = self.norm[self.conditions.index(condition)]
+        else:
+            norm = self.norm
+        point.feat = norm(point.feat)
+        if self.adaptive:
+            assert "context" in point.keys()
+            shift, scale = self.modulation(point.context).chunk(2, dim=1)
+            point.feat = point.feat * (1.0 + scale) + shift
+        return point
+
+
+class SerializedAttention(PointModule):
+    """Attention inside patches of the serialized point sequence (model.py:319-490).
+
+    The qkv projection and the output projection are torch Linears; everything between them —
+    gathering rows into padded serialized order, softmax(q k^T) v per patch and head,
+    scattering rows back — is one HIP kernel launch reading through int32 slot tables that
+    are built once per (Point, order) and cached on the Point."""
+
+    def __init__(self, channels, num_heads, patch_size, qkv_bias=True, qk_scale=None, attn_drop=0.0,
+                 proj_drop=0.0, order_index=0, enable_rpe=False, enable_flash=True,
+                 upcast_attention=True, upcast_softmax=True):
+        super().__init__()
+        assert channels % num_heads == 0
+        self.channels, self.num_heads = channels, num_heads
+        self.scale = qk_scale or (channels // num_heads) ** -0.5
+        self.order_index = order_index
+        self.upcast_attention, self.upcast_softmax = upcast_attention, upcast_softmax
+        self.enable_rpe, self.enable_flash = enable_rpe, enable_flash
+        if enable_rpe:
+            raise NotImplementedError(
+                "relative position bias is not covered by the HIP attention kernel; it is "
+                "mutually exclusive with the flash path every released PTv3 config uses")
+        if enable_flash:
+            assert upcast_attention is False, "Set upcast_attention to False when enable Flash Attention"
+            assert upcast_softmax is False, "Set upcast_softmax to False when enable Flash Attention"
+            self.patch_size = patch_size
+        else:
+            # without the fused path the reference shrinks the patch to the smallest scene so
+            # that no padding is ever needed (model.py:359-363, :441-444)
+            self.patch_size_max = patch_size
+            self.patch_size = 0
+        assert attn_drop == 0.0, "attention dropout is a training feature outside this forward path"
+        self.attn_drop = attn_drop
+        self.qkv = nn.Linear(channels, channels * 3, bias=qkv_bias)
+        self.proj = nn.Linear(channels, channels)
+        self.proj_drop = nn.Dropout(proj_drop)
+
+    @torch.no_grad()
+    def get_padding_and_inverse(self, point):
+        """pad / unpad / cu_seqlens, cached on the Point under the reference's keys
+        (model.py:382-438)."""
+        if not {"pad", "unpad", "cu_seqlens_key"}.issubset(point.keys()):
+            pad, unpad, cu = ops.pad_index(point.offset, point.offset_host(), self.patch_size)
+            point["pad"], point["unpad"], point["cu_seqlens_key"] = pad, unpad, cu
+        return point["pad"], point["unpad"], point["cu_seqlens_key"]
+
+    @torch.no_grad()
+    def _slots(self, point):
+        key = f"_attn_slots_{self.order_index}"
+        if key not in point:
+            pad, unpad, _ = self.get_padding_and_inverse(point)
+            point[key] = ops.attn_slots(point.serialized_order[self.order_index],
+                                        point.serialized_inverse[self.order_index], pad, unpad)
+        return point[key]
+
+    def forward(self, point):
+        if not self.enable_flash:
+            sizes = offset2bincount(torch.as_tensor(point.offset_host()))
+            self.patch_size = min(int(sizes.min()), self.patch_size_max)
+        _, _, cu_seqlens = self.get_padding_and_inverse(point)
+        slot_src, slot_dst = self._slots(point)
+
+        qkv = self.qkv(point.feat)
+        if self.enable_flash and qkv.dtype == torch.float32:
+            # the fused path of the reference always computes in half precision (model.py:477,483)
+            feat = ops.patch_attention(qkv.half(), self.num_heads, slot_src, slot_dst, cu_seqlens,
+                                       self.patch_size, self.scale).to(qkv.dtype)
+        else:
+            feat = ops.patch_attention(qkv, self.num_heads, slot_src, slot_dst, cu_seqlens,
+                                       self.patch_size, self.scale)
+        feat = self.proj(feat)
+        feat = self.proj_drop(feat)
+        point.feat = feat
+        return point
+
+
+class MLP(nn.Module):
+    """fc1 -> act -> drop -> fc2 -> drop (model.py:493-516)."""
+
+    def __init__(self, in_channels, hidden_channels=None, out_channels=None, act_layer=nn.GELU, drop=0.0):
+        super().__init__()
+        out_channels = out_channels or in_channels
+        hidden_channels = hidden_channels or in_channels
+        self.fc1 = nn.Linear(in_channels, hidden_channels)
+        self.act = act_layer()
+        self.fc2 = nn.Linear(hidden_channels, out_channels)
+        self.drop = nn.Dropout(drop)
+
+    def forward(self, x):
+        return self.drop(self.fc2(self.drop(self.act(self.fc1(x)))))
+
+
+class Block(PointModule):
+    """xCPE conv + attention + MLP, each with a residual (model.py:519-606)."""
+
+    def __init__(self, channels, num_heads, patch_size=48, mlp_ratio=4.0, qkv_bias=True, qk_scale=None,
+                 attn_drop=0.0, proj_drop=0.0, drop_path=0.0, norm_layer=nn.LayerNorm, act_layer=nn.GELU,
+                 pre_norm=True, order_index=0, cpe_indice_key=None, enable_rpe=False, enable_flash=True,
+                 upcast_attention=True, upcast_softmax=True):
+        super().__init__()
+        self.channels, self.pre_norm = channels, pre_norm
+        self.cpe = PointSequential(
+            SubMConv3d(channels, channels, kernel_size=3, bias=True, indice_key=cpe_indice_key),
+            nn.Linear(channels, channels),
+            norm_layer(channels),
+        )
+        self.norm1 = PointSequential(norm_layer(channels))
+        self.attn = SerializedAttention(
+            channels=channels, patch_size=patch_size, num_heads=num_heads, qkv_bias=qkv_bias,
+            qk_scale=qk_scale, attn_drop=attn_drop, proj_drop=proj_drop, order_index=order_index,
+            enable_rpe=enable_rpe, enable_flash=enable_flash, upcast_attention=upcast_attention,
+            upcast_softmax=upcast_softmax)
+        self.norm2 = PointSequential(norm_layer(channels))
+        self.mlp = PointSequential(MLP(in_channels=channels, hidden_channels=int(channels * mlp_ratio),
+                                       out_channels=channels, act_layer=act_layer, drop=proj_drop))
+        self.drop_path = PointSequential(DropPath(drop_path) if drop_path > 0.0 else nn.Identity())
+
+    def forward(self, point):
+        skip = point.feat
+        point = self.cpe(point)
+        point.feat = skip + point.feat
+
+        skip = point.feat
+        if self.pre_norm:
+            point = self.norm1(point)
+        point = self.drop_path(self.attn(point))
+        point.feat = skip + point.feat
+        if not self.pre_norm:
+            point = self.norm1(point)
+
+        skip = point.feat
+        if self.pre_norm:
+            point = self.norm2(point)
+        point = self.drop_path(self.mlp(point))
+        point.feat = skip + point.feat
+        if not self.pre_norm:
+            point = self.norm2(point)
+        # the sparse view is refreshed only here (model.py:605); within the block the conv of
+        # the NEXT block therefore sees exactly this tensor
+        point.sparse_conv_feat = point.sparse_conv_feat.replace_feature(point.feat)
+        return point
+
+
+class SerializedPooling(PointModule):
+    """Grid pooling along the serialized order (model.py:609-712).
+
+    Points whose row-0 code agrees after dropping 3*log2(stride) bits form a cluster. Because
+    serialized_order[0] already sorts those codes, clusters are runs: one flag+scan kernel
+    numbers them (no unique, no sort), a gather kernel produces the pooled codes, coordinates
+    and scene ids, and a segment kernel reduces the projected features."""
+
+    def __init__(self, in_channels, out_channels, stride=2, norm_layer=None, act_layer=None,
+                 reduce="max", shuffle_orders=True, traceable=True):
+        super().__init__()
+        self.in_channels, self.out_channels = in_channels, out_channels
+        assert stride == 2 ** (math.ceil(stride) - 1).bit_length()   # 2, 4, 8
+        self.stride = stride
+        assert reduce in ["sum", "mean", "min", "max"]
+        self.reduce, self.shuffle_orders, self.traceable = reduce, shuffle_orders, traceable
+        self.proj = nn.Linear(in_channels, out_channels)
+        self.norm = PointSequential(norm_layer(out_channels)) if norm_layer is not None else None
+        self.act = PointSequential(act_layer()) if act_layer is not None else None
+
+    def forward(self, point):
+        pooling_depth = (math.ceil(self.stride) - 1).bit_length()
+        if pooling_depth > point.serialized_depth:
+            pooling_depth = 0
+        assert {"serialized_code", "serialized_order", "serialized_inverse", "serialized_depth"}.issubset(
+            point.keys()), "Run point.serialization() point cloud before SerializedPooling"
+        shift = 3 * pooling_depth
+        depth = point.serialized_depth - pooling_depth
+
+        # clusters in ascending order of the (shifted) row-0 code
+        indices = point.serialized_order[0]
+        cluster, idx_ptr, head, m = ops.pool_clusters(point.serialized_code[0], indices, shift)
+        code, grid_coord, batch = ops.pool_gather(point.serialized_code, shift, point.grid_coord,
+                                                  pooling_depth, point.batch, head)
+        n_scenes = len(point.offset_host())
+        order, inverse = ops.argsort_rows(code, 3 * depth + max(1, (n_scenes - 1).bit_length()))
+        if self.shuffle_orders:
+            perm = torch.randperm(code.shape[0]).to(code.device)   # CPU generator (model.py:677)
+            code, order, inverse = code[perm], order[perm], inverse[perm]
+
+        fields = AttrDict(
+            feat=ops.segment_reduce(self.proj(point.feat), indices, idx_ptr, self.reduce),
+            grid_coord=grid_coord,
+            serialized_code=code,
+            serialized_order=order,
+            serialized_inverse=inverse,
+            serialized_depth=depth,
+            batch=batch,
+        )
+        if "coord" in point:
+            fields["coord"] = ops.segment_reduce(point.coord.float(), indices, idx_ptr, "mean")
+        for key in ("condition", "context"):
+            if key in point:
+                fields[key] = point[key]
+        if self.traceable:
+            fields["pooling_inverse"] = cluster
+            fields["pooling_parent"] = point
+        pooled = Point(fields)
+        if self.norm is not None:
+            pooled = self.norm(pooled)
+        if self.act is not None:
+            pooled = self.act(pooled)
+        pooled.sparsify()
+        return pooled
+
+
+class SerializedUnpooling(PointModule):
+    """Project child and parent, then parent += child[cluster] (model.py:715-750)."""
+
+    def __init__(self, in_channels, skip_channels, out_channels, norm_layer=None, act_layer=None,
+                 traceable=False):
+        super().__init__()
+        self.proj = PointSequential(nn.Linear(in_channels, out_channels))
+        self.proj_skip = PointSequential(nn.Linear(skip_channels, out_channels))
+        if norm_layer is not None:
+            self.proj.add(norm_layer(out_channels))
+            self.proj_skip.add(norm_layer(out_channels))
+        if act_layer is not None:
+            self.proj.add(act_layer())
+            self.proj_skip.add(act_layer())
+        self.traceable = traceable
+
+    def forward(self, point):
+        assert "pooling_parent" in point.keys()
+        assert "pooling_inverse" in point.keys()
+        parent = point.pop("pooling_parent")
+        inverse = point.pop("pooling_inverse")
+        point = self.proj(point)
+        parent = self.proj_skip(parent)
+        # only .feat is updated; parent.sparse_conv_feat keeps the skip projection, which is
+        # what the first decoder block's conv reads in the reference as well (model.py:746)
+        parent.feat = ops.unpool_add(parent.feat, point.feat, inverse)
+        if self.traceable:
+            parent["unpooling_parent"] = point
+        return parent
+
+
+class Embedding(PointModule):
+    """Stem: 5x5x5 submanifold conv -> norm -> act (model.py:753-783)."""
+
+    def __init__(self, in_channels, embed_channels, norm_layer=None, act_layer=None):
+        super().__init__()
+        self.in_channels, self.embed_channels = in_channels, embed_channels
+        self.stem = PointSequential(conv=SubMConv3d(in_channels, embed_channels, kernel_size=5, padding=1,
+                                                    bias=False, indice_key="stem"))
+        if norm_layer is not None:
+            self.stem.add(norm_layer(embed_channels), name="norm")
+        if act_layer is not None:
+            self.stem.add(act_layer(), name="act")
+
+    def forward(self, point):
+        return self.stem(point)

@@ -14,6 +14,16 @@ _DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 REDUCE_OPS = {"max": 0, "mean": 1, "sum": 2, "min": 3}
 
 
+_LAUNCH_TIMER = None
+
+
+def set_launch_timer(timer):
+    """Install (or clear, with None) an object whose launch(name, work, fn) brackets selected
+    kernel launches with device events; used by the benchmark, off by default."""
+    global _LAUNCH_TIMER
+    _LAUNCH_TIMER = timer
+
+
 def _stream():
     return torch.cuda.current_stream().cuda_stream
 
@@ -121,9 +131,16 @@ def patch_attention(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, 
     c = c3 // 3
     out = torch.empty((n, c), dtype=qkv.dtype, device=qkv.device)
     n_seq = cu_seqlens.shape[0] - 1
-    _lib.check(lib.ptv3_patch_attn_fwd(_ptr(qkv), _dtype_code(qkv), n, c, int(num_heads), _ptr(slot_src),
-                                       _ptr(slot_dst), _ptr(cu_seqlens), n_seq, int(max_seqlen),
-                                       float(scale), _ptr(out), _stream()), "ptv3_patch_attn_fwd")
+
+    def call():
+        _lib.check(lib.ptv3_patch_attn_fwd(_ptr(qkv), _dtype_code(qkv), n, c, int(num_heads), _ptr(slot_src),
+                                           _ptr(slot_dst), _ptr(cu_seqlens), n_seq, int(max_seqlen),
+                                           float(scale), _ptr(out), _stream()), "ptv3_patch_attn_fwd")
+
+    if _LAUNCH_TIMER is not None:
+        _LAUNCH_TIMER.launch("patch_attn", (cu_seqlens, c), call)
+    else:
+        call()
     return out
 
 

@@ -1,0 +1,134 @@
+"""The Point dictionary of PTv3 and its two preparation steps, serialization and
+sparsification, on top of the HIP kernels.
+
+Interface (keys, method names, arguments) follows model.py:28-174 of the reference so user
+code that builds a data_dict keeps working. What differs is where the work happens: all k
+curve codes come from one fused kernel, the k argsorts and inverse permutations from one
+batched radix sort, and the host learns the three things it needs (grid extent, hence depth
+and sparse shape, and scene sizes) from a single device->host copy that is cached on the
+Point.
+"""
+import torch
+
+from . import ops
+
+
+@torch.inference_mode()
+def offset2bincount(offset):
+    """Scene sizes from cumulative scene ends (model.py:28-32)."""
+    return torch.diff(offset, prepend=offset.new_zeros(1))
+
+
+@torch.inference_mode()
+def offset2batch(offset):
+    """Scene id per point from cumulative scene ends (model.py:35-40)."""
+    sizes = offset2bincount(offset)
+    ids = torch.arange(sizes.numel(), device=offset.device, dtype=torch.long)
+    return ids.repeat_interleave(sizes)
+
+
+@torch.inference_mode()
+def batch2offset(batch):
+    """Cumulative scene ends from sorted scene ids (model.py:43-45)."""
+    return batch.bincount().cumsum(0).long()
+
+
+class AttrDict(dict):
+    """dict whose items are also attributes (stands in for addict.Dict, model.py:11,48)."""
+
+    def __getattr__(self, name):
+        try:
+            return self[name]
+        except KeyError:
+            raise AttributeError(name) from None
+
+    def __setattr__(self, name, value):
+        self[name] = value
+
+    def __delattr__(self, name):
+        try:
+            del self[name]
+        except KeyError:
+            raise AttributeError(name) from None
+
+
+class Point(AttrDict):
+    """Batched point cloud as a dictionary (model.py:48-79).
+
+    Recognised keys: coord, grid_coord, grid_size, feat, offset, batch, and — written by the
+    methods below — serialized_depth/code/order/inverse, sparse_shape, sparse_conv_feat.
+    Keys starting with an underscore are host-side caches of this implementation."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        if "batch" not in self and "offset" in self:
+            self["batch"] = offset2batch(self["offset"])
+        elif "offset" not in self and "batch" in self:
+            self["offset"] = batch2offset(self["batch"])
+
+    # ---- host-side facts, one device->host copy each, cached -------------------------
+    def offset_host(self):
+        """Cumulative scene ends as a Python list."""
+        if "_offset_host" not in self:
+            self["_offset_host"] = [int(v) for v in self["offset"].tolist()]
+        return self["_offset_host"]
+
+    def grid_max_host(self):
+        """Per-axis maximum of grid_coord as a Python list of 3 ints."""
+        if "_grid_max_host" not in self:
+            self._ensure_grid_coord()
+            self["_grid_max_host"] = [int(v) for v in self["grid_coord"].max(0).values.tolist()]
+        return self["_grid_max_host"]
+
+    def _ensure_grid_coord(self):
+        if "grid_coord" not in self:
+            # fallback voxelisation of the reference (model.py:88-96)
+            assert {"grid_size", "coord"}.issubset(self.keys())
+            shifted = self["coord"] - self["coord"].min(0)[0]
+            self["grid_coord"] = torch.div(shifted, self["grid_size"], rounding_mode="trunc").int()
+
+    # ---- serialization ---------------------------------------------------------------
+    def serialization(self, order="z", depth=None, shuffle_orders=False):
+        """Curve codes, sort order and inverse for every requested order (model.py:81-136).
+
+        Writes serialized_depth (int) and serialized_code / serialized_order /
+        serialized_inverse, each (k, N) int64."""
+        assert "batch" in self
+        self._ensure_grid_coord()
+        orders = [order] if isinstance(order, str) else list(order)
+        if depth is None:
+            depth = max(self.grid_max_host()).bit_length()   # model.py:98-101
+        self["serialized_depth"] = depth
+        n_scenes = len(self.offset_host())
+        assert depth * 3 + n_scenes.bit_length() <= 63       # model.py:103
+        assert depth <= 16                                    # model.py:108
+
+        code = ops.encode_orders(self["grid_coord"], self["batch"], depth, orders)
+        key_bits = 3 * depth + max(1, (n_scenes - 1).bit_length())
+        sort_order, inverse = ops.argsort_rows(code, key_bits)
+
+        if shuffle_orders:
+            perm = torch.randperm(code.shape[0])              # CPU generator, as model.py:129
+            perm = perm.to(code.device)
+            code, sort_order, inverse = code[perm], sort_order[perm], inverse[perm]
+
+        self["serialized_code"] = code
+        self["serialized_order"] = sort_order
+        self["serialized_inverse"] = inverse
+
+    # ---- sparsify --------------------------------------------------------------------
+    def sparsify(self, pad=96):
+        """Attach the sparse-conv view of the features (model.py:138-174)."""
+        from .sparse import SparseConvTensor
+
+        assert {"feat", "batch"}.issubset(self.keys())
+        self._ensure_grid_coord()
+        if "sparse_shape" in self:
+            sparse_shape = self["sparse_shape"]
+        else:
+            sparse_shape = [v + pad for v in self.grid_max_host()]
+        indices = torch.cat([self["batch"].unsqueeze(-1).int(), self["grid_coord"].int()], dim=1).contiguous()
+        self["sparse_shape"] = sparse_shape
+        self["sparse_conv_feat"] = SparseConvTensor(
+            features=self["feat"], indices=indices, spatial_shape=sparse_shape,
+            batch_size=len(self.offset_host()))

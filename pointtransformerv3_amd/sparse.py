@@ -1,0 +1,79 @@
+"""Sparse-convolution tensor and submanifold convolution on the HIP kmap / implicit-GEMM
+kernels. Stands in for the two spconv types the reference touches (model.py:165-172,
+:233-236, :546-552, :767-774): same constructor arguments and attribute names."""
+import math
+
+import torch
+import torch.nn as nn
+
+from . import ops
+
+
+class SparseConvTensor:
+    """features (N,C), indices (N,4) int32 [batch,x,y,z], spatial_shape, batch_size.
+    Neighbour maps are cached per indice_key in `indice_dict` and shared by every tensor
+    derived through replace_feature, like spconv's."""
+
+    def __init__(self, features, indices, spatial_shape, batch_size, indice_dict=None):
+        self.features = features
+        self.indices = indices
+        self.spatial_shape = list(spatial_shape)
+        self.batch_size = batch_size
+        self.indice_dict = {} if indice_dict is None else indice_dict
+
+    def replace_feature(self, features):
+        return SparseConvTensor(features, self.indices, self.spatial_shape, self.batch_size,
+                                self.indice_dict)
+
+    def neighbour_map(self, kernel_size, indice_key=None):
+        key = (indice_key, kernel_size) if indice_key is not None else None
+        if key is not None and key in self.indice_dict:
+            return self.indice_dict[key]
+        nbr = ops.kmap_build(self.indices, kernel_size)
+        if key is not None:
+            self.indice_dict[key] = nbr
+        return nbr
+
+
+class SubMConv3d(nn.Module):
+    """Submanifold 3-D convolution: output sites = input sites. weight has spconv 2.x's
+    (out, k, k, k, in) layout so checkpoints keep loading; `padding` is accepted and unused,
+    as submanifold convolutions are centred by construction."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
+                 groups=1, bias=True, indice_key=None):
+        super().__init__()
+        assert stride == 1 and dilation == 1 and groups == 1
+        assert kernel_size in (3, 5), "the kmap kernel covers 3x3x3 and 5x5x5"
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.kernel_size, self.indice_key = kernel_size, indice_key
+        k = kernel_size
+        self.weight = nn.Parameter(torch.empty(out_channels, k, k, k, in_channels))
+        self.bias = nn.Parameter(torch.empty(out_channels)) if bias else None
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        fan_in = self.kernel_size ** 3 * self.in_channels
+        bound = 1.0 / math.sqrt(fan_in)   # kaiming_uniform(a=sqrt(5)) on fan_in
+        nn.init.uniform_(self.weight, -bound, bound)
+        if self.bias is not None:
+            nn.init.uniform_(self.bias, -bound, bound)
+
+    def forward(self, x):
+        feat = x.features
+        if torch.is_autocast_enabled():
+            feat = feat.to(torch.get_autocast_gpu_dtype())
+        nbr = x.neighbour_map(self.kernel_size, self.indice_key)
+        weight = self.weight.reshape(self.out_channels, -1, self.in_channels)
+        cin = self.in_channels
+        if feat.dtype != torch.float32 and cin % 16 != 0:
+            # the MFMA kernel consumes input channels 16 at a time: zero-pad the thin stem input
+            pad = 16 - cin % 16
+            feat = nn.functional.pad(feat, (0, pad))
+            weight = nn.functional.pad(weight, (0, pad))
+        out = ops.subm_conv(feat, nbr, weight.to(feat.dtype), self.bias)
+        return x.replace_feature(out)
+
+
+def is_spconv_module(module):
+    return isinstance(module, SubMConv3d)

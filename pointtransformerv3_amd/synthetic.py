@@ -110,11 +110,12 @@ def collate(scenes):
 
 
 def room_features(coord, seed):
-    """6-dim input: xyz, RGB U[0,1], unit normals."""
+    """6-dim input as in Pointcept's indoor configs: RGB U[0,1] and unit normals (the xyz of a
+    point enters the model through coord / grid_coord)."""
     rng = np.random.default_rng(seed)
     nrm = rng.normal(size=(len(coord), 3))
     nrm /= np.linalg.norm(nrm, axis=1, keepdims=True)
-    return np.concatenate([coord, rng.random((len(coord), 3)), nrm], 1).astype(np.float32)
+    return np.concatenate([rng.random((len(coord), 3)), nrm], 1).astype(np.float32)
 
 
 def lidar_features(coord, seed):
