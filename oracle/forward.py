@@ -99,11 +99,13 @@ def _unpool(sd, name, child):
     return parent
 
 
-def ptv3_forward(state_dict, grid_coord, feat, offset, perms=None, **config):
+def ptv3_forward(state_dict, grid_coord, feat, offset, perms=None, trace=None, **config):
     """Returns the (N, dec_channels[0]) output features in original point order (fp32 torch).
 
     perms: None (no shuffling) or a list of row permutations, one for the initial
-    serialization followed by one per pooling stage."""
+    serialization followed by one per pooling stage.
+    trace: optional dict; receives the feature tensor after the stem and after every
+    pooling / unpooling / block, keyed by the module's state_dict prefix."""
     cfg = dict(DEFAULTS)
     cfg.update(config)
     sd = {k: torch.as_tensor(v).float() for k, v in state_dict.items()}
@@ -125,17 +127,27 @@ def ptv3_forward(state_dict, grid_coord, feat, offset, perms=None, **config):
     y = OF.subm_conv(x, _kmap(level, 5), sd["embedding.stem.conv.weight"], None)
     y = F.gelu(_bn(sd, "embedding.stem.norm", y))
     level["feat"] = level["sparse_feat"] = y
+    def note(name, lv):
+        if trace is not None:
+            trace[name] = lv["feat"]
+            trace[name + "#level"] = lv   # integer structures of the level, for debugging
+
+    note("embedding", level)
 
     assert all(st == 2 for st in cfg["stride"]), "the oracle pools by 2 per stage"
     n_stage = len(cfg["enc_depths"])
     for s in range(n_stage):
         if s > 0:
             level = _pool(sd, f"enc.enc{s}.down", level, perms[s])
+            note(f"enc.enc{s}.down", level)
         for i in range(cfg["enc_depths"][s]):
             _block(sd, f"enc.enc{s}.block{i}", level, cfg["enc_num_head"][s], cfg["enc_patch_size"][s], i % k)
+            note(f"enc.enc{s}.block{i}", level)
     if not cfg["cls_mode"]:
         for s in reversed(range(n_stage - 1)):
             level = _unpool(sd, f"dec.dec{s}.up", level)
+            note(f"dec.dec{s}.up", level)
             for i in range(cfg["dec_depths"][s]):
                 _block(sd, f"dec.dec{s}.block{i}", level, cfg["dec_num_head"][s], cfg["dec_patch_size"][s], i % k)
+                note(f"dec.dec{s}.block{i}", level)
     return level["feat"]

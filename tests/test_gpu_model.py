@@ -23,6 +23,18 @@ def _data(n_per_scene, n_scenes, grid=0.05, seed=10, lidar=False):
     return d, feat
 
 
+def _draw_perms(seed, shuffle_first, n_pool=4, k=4):
+    """The row permutations a forward will draw from torch's CPU generator after
+    torch.manual_seed(seed): one in Point.serialization when the model shuffles, then one per
+    pooling stage — SerializedPooling is built without shuffle_orders (model.py:881-887), so it
+    always shuffles. Re-seeds so the forward that follows draws the same sequence."""
+    torch.manual_seed(seed)
+    perms = [torch.randperm(k).numpy() if shuffle_first else None]
+    perms += [torch.randperm(k).numpy() for _ in range(n_pool)]
+    torch.manual_seed(seed)
+    return perms
+
+
 def _run(model, d, feat, dtype):
     data = dict(feat=torch.from_numpy(feat).to(DEV, dtype), grid_coord=torch.from_numpy(d["grid_coord"]).to(DEV),
                 coord=torch.from_numpy(d["coord"]).to(DEV), offset=torch.from_numpy(d["offset"]).to(DEV))
@@ -36,7 +48,8 @@ def test_forward_fp32_no_flash_small_patches():
     torch.manual_seed(0)
     model = PointTransformerV3(shuffle_orders=False, enable_flash=False, **kw).eval()
     d, feat = _data(3000, 2)
-    want = ptv3_forward(model.state_dict(), d["grid_coord"], feat, d["offset"], enable_flash=False, **kw)
+    perms = _draw_perms(5, False)
+    want = ptv3_forward(model.state_dict(), d["grid_coord"], feat, d["offset"], enable_flash=False, perms=perms, **kw)
     point = _run(model.to(DEV), d, feat, torch.float32)
     assert point.feat.shape == want.shape
     assert rel_err(point.feat, want) < 1e-4
@@ -48,11 +61,7 @@ def test_forward_fp16_default_model(shuffle):
     torch.manual_seed(1)
     model = PointTransformerV3(shuffle_orders=shuffle).eval().half()
     d, feat = _data(20000, 2, grid=0.02)
-    perms = None
-    if shuffle:
-        torch.manual_seed(77)
-        perms = [torch.randperm(4).numpy() for _ in range(5)]   # serialization + 4 poolings
-        torch.manual_seed(77)
+    perms = _draw_perms(77, shuffle)
     sd = {k: v.float() for k, v in model.state_dict().items()}   # the fp16-rounded weights, in fp32
     point = _run(model.to(DEV), d, feat.astype(np.float16).astype(np.float32), torch.float16)
     want = ptv3_forward(sd, d["grid_coord"], feat.astype(np.float16).astype(np.float32), d["offset"], perms=perms)
@@ -74,8 +83,9 @@ def test_forward_lidar_4dim_fp16():
     d, feat = _data(0, 1, grid=0.05, seed=5000, lidar=True)
     feat = feat.astype(np.float16).astype(np.float32)
     sd = {k: v.float() for k, v in model.state_dict().items()}
+    perms = _draw_perms(3, False)
     point = _run(model.to(DEV), d, feat, torch.float16)
-    want = ptv3_forward(sd, d["grid_coord"], feat, d["offset"], **kw)
+    want = ptv3_forward(sd, d["grid_coord"], feat, d["offset"], perms=perms, **kw)
     assert point.serialized_depth == 12
     assert rel_err(point.feat, want) < 2e-2
 
