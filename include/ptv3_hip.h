@@ -125,6 +125,16 @@ int ptv3_segment_reduce(const void *src, int dtype, int64_t n, int c, const int6
 int ptv3_unpool_add(const void *parent, const void *child, int dtype, int64_t n, int c,
                     const int64_t *cluster, int64_t m, void *out, void *stream);
 
+/* nn.LayerNorm calls model.py:554,557,572 fused with the residual adds :589,:594,:602.
+ * x,res,out0,out1 (n,c); gamma,beta (c,); all of dtype, statistics in fp32.
+ * mode 0: out0 = LN(x).  mode 1: out0 = res + LN(x).
+ * mode 2: out0 = x + res, out1 = LN(out0).
+ * mode 3: out0 = res + LN(x), out1 = LN(out0) with the second affine pair gamma2,beta2.
+ * Intermediates are rounded to dtype where separate kernels would have stored them. */
+int ptv3_layer_norm(const void *x, const void *res, const void *gamma, const void *beta,
+                    const void *gamma2, const void *beta2, int dtype, int64_t n, int c, float eps,
+                    int mode, void *out0, void *out1, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,205 @@
+// Row-wise LayerNorm fused with the residual additions that surround it in a PTv3 block.
+//
+// Replaces the nn.LayerNorm calls of model.py:554,557,572 together with the residual adds
+// of :589,:594,:602. HBM-bound: every row is read once and written once (or twice when
+// both the sum and its normalisation are needed). A row of C channels is spread over
+// C/8 lanes (8 channels = one 16-byte load per lane in half precision), so a 64-lane wave
+// normalises 64/(C/8) rows at a time and reductions are a few cross-lane steps.
+//
+//   mode 0: out0 = LN(x)
+//   mode 1: out0 = res + LN(x)                      (cpe: shortcut + LN(Linear(conv)))
+//   mode 2: out0 = x + res; out1 = LN(out0)         (shortcut + branch, then pre-norm)
+//   mode 3: out0 = res + LN(x); out1 = LN2(out0)    (cpe residual, then the attention pre-norm)
+// Intermediate results are rounded to the storage type exactly where separate kernels would
+// have stored them, so fusing changes no value.
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+
+#include "common.h"
+
+namespace {
+
+template <typename T> struct Vec8 { T v[8]; };
+
+template <typename T>
+__device__ __forceinline__ void load8(const T* p, float (&f)[8]) {
+    const Vec8<T> r = *(const Vec8<T>*)p;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = (float)r.v[i];
+}
+template <typename T>
+__device__ __forceinline__ void store8(T* p, const float (&f)[8]) {
+    Vec8<T> r;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r.v[i] = (T)f[i];
+    *(Vec8<T>*)p = r;
+}
+
+template <typename T> __device__ __forceinline__ float round_to(float v) { return (float)(T)v; }
+
+// statistics of 8 values per lane over the LPR lanes of a row
+template <int LPR>
+__device__ __forceinline__ void row_stats(const float (&v)[8], float eps, float& mean, float& rstd) {
+    constexpr int C = 8 * LPR;
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += v[i];
+#pragma unroll
+    for (int o = 1; o < LPR; o <<= 1) s += __shfl_xor(s, o, PTV3_WAVE);
+    mean = s * (1.f / C);
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) q += (v[i] - mean) * (v[i] - mean);
+#pragma unroll
+    for (int o = 1; o < LPR; o <<= 1) q += __shfl_xor(q, o, PTV3_WAVE);
+    rstd = rsqrtf(q * (1.f / C) + eps);
+}
+
+// LPR lanes per row, C = 8 * LPR channels.
+template <typename T, int LPR, int MODE>
+__global__ __launch_bounds__(256) void layer_norm_kernel(
+    const T* __restrict__ x, const T* __restrict__ res, const T* __restrict__ gamma,
+    const T* __restrict__ beta, const T* __restrict__ gamma2, const T* __restrict__ beta2, int64_t n,
+    float eps, T* __restrict__ out0, T* __restrict__ out1) {
+    constexpr int C = 8 * LPR;
+    constexpr int ROWS_PER_BLOCK = 256 / LPR;
+    const int sub = threadIdx.x % LPR;
+    const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / LPR;
+    const bool live = row < n;   // dead lanes still take part in the cross-lane sums
+    const int64_t off = row * C + sub * 8;
+    float v[8], r[8], g[8], b[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { v[i] = 0.f; r[i] = 0.f; }
+    load8(gamma + sub * 8, g);
+    load8(beta + sub * 8, b);
+    if (live) {
+        load8(x + off, v);
+        if (MODE != 0) load8(res + off, r);
+    }
+    if (MODE == 2) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = round_to<T>(v[i] + r[i]);
+        if (live) store8(out0 + off, v);
+    }
+    float mean, rstd;
+    row_stats<LPR>(v, eps, mean, rstd);
+    float y[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = (v[i] - mean) * rstd * g[i] + b[i];
+    if (MODE == 1 || MODE == 3) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = round_to<T>(round_to<T>(y[i]) + r[i]);
+    }
+    if (MODE == 3) {
+        if (live) store8(out0 + off, y);
+        load8(gamma2 + sub * 8, g);
+        load8(beta2 + sub * 8, b);
+        row_stats<LPR>(y, eps, mean, rstd);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = (y[i] - mean) * rstd * g[i] + b[i];
+    }
+    if (live) store8((MODE >= 2) ? out1 + off : out0 + off, y);
+}
+
+// Any C: one wave per row, strided scalar accesses.
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void layer_norm_generic_kernel(
+    const T* __restrict__ x, const T* __restrict__ res, const T* __restrict__ gamma,
+    const T* __restrict__ beta, int64_t n, int c, float eps, T* __restrict__ out0,
+    T* __restrict__ out1) {
+    const int lane = threadIdx.x % PTV3_WAVE;
+    const int64_t row = (int64_t)blockIdx.x * (256 / PTV3_WAVE) + threadIdx.x / PTV3_WAVE;
+    if (row >= n) return;   // whole wave leaves together
+    const T* xr = x + row * c;
+    const T* rr = res ? res + row * c : nullptr;
+    float s = 0.f;
+    for (int i = lane; i < c; i += PTV3_WAVE) {
+        float v = (float)xr[i];
+        if (MODE == 2) {
+            const T t = (T)(v + (float)rr[i]);
+            out0[row * c + i] = t;
+            v = (float)t;
+        }
+        s += v;
+    }
+#pragma unroll
+    for (int o = 1; o < PTV3_WAVE; o <<= 1) s += __shfl_xor(s, o, PTV3_WAVE);
+    const float mean = s / c;
+    float q = 0.f;
+    for (int i = lane; i < c; i += PTV3_WAVE) {
+        const float v = (MODE == 2 ? (float)out0[row * c + i] : (float)xr[i]) - mean;
+        q += v * v;
+    }
+#pragma unroll
+    for (int o = 1; o < PTV3_WAVE; o <<= 1) q += __shfl_xor(q, o, PTV3_WAVE);
+    const float rstd = rsqrtf(q / c + eps);
+    for (int i = lane; i < c; i += PTV3_WAVE) {
+        const float v = MODE == 2 ? (float)out0[row * c + i] : (float)xr[i];
+        float y = (v - mean) * rstd * (float)gamma[i] + (float)beta[i];
+        if (MODE == 1) y = (float)(T)y + (float)rr[i];
+        (MODE == 2 ? out1 : out0)[row * c + i] = (T)y;
+    }
+}
+
+template <typename T, int MODE>
+void launch(const void* x, const void* res, const void* gamma, const void* beta, const void* gamma2,
+            const void* beta2, int64_t n, int c, float eps, void* out0, void* out1, hipStream_t stream) {
+#define PTV3_LN(LPR)                                                                            \
+    hipLaunchKernelGGL((layer_norm_kernel<T, LPR, MODE>), dim3((unsigned)ptv3_ceil_div(n, 256 / LPR)), \
+                       dim3(256), 0, stream, (const T*)x, (const T*)res, (const T*)gamma,       \
+                       (const T*)beta, (const T*)gamma2, (const T*)beta2, n, eps, (T*)out0, (T*)out1)
+    switch (c) {
+        case 32: PTV3_LN(4); break;
+        case 64: PTV3_LN(8); break;
+        case 128: PTV3_LN(16); break;
+        case 256: PTV3_LN(32); break;
+        case 512: PTV3_LN(64); break;
+        default:
+            if (MODE == 3) {   // two generic passes: out0 = res + LN(x), then out1 = LN2(out0)
+                hipLaunchKernelGGL((layer_norm_generic_kernel<T, 1>), dim3((unsigned)ptv3_ceil_div(n, 4)),
+                                   dim3(256), 0, stream, (const T*)x, (const T*)res, (const T*)gamma,
+                                   (const T*)beta, n, c, eps, (T*)out0, (T*)nullptr);
+                hipLaunchKernelGGL((layer_norm_generic_kernel<T, 0>), dim3((unsigned)ptv3_ceil_div(n, 4)),
+                                   dim3(256), 0, stream, (const T*)out0, (const T*)nullptr, (const T*)gamma2,
+                                   (const T*)beta2, n, c, eps, (T*)out1, (T*)nullptr);
+            } else {
+                constexpr int GM = MODE == 3 ? 0 : MODE;
+                hipLaunchKernelGGL((layer_norm_generic_kernel<T, GM>), dim3((unsigned)ptv3_ceil_div(n, 4)),
+                                   dim3(256), 0, stream, (const T*)x, (const T*)res, (const T*)gamma,
+                                   (const T*)beta, n, c, eps, (T*)out0, (T*)out1);
+            }
+    }
+#undef PTV3_LN
+}
+
+template <typename T>
+void launch_mode(int mode, const void* x, const void* res, const void* gamma, const void* beta,
+                 const void* gamma2, const void* beta2, int64_t n, int c, float eps, void* out0,
+                 void* out1, hipStream_t stream) {
+    if (mode == 0) launch<T, 0>(x, res, gamma, beta, gamma2, beta2, n, c, eps, out0, out1, stream);
+    else if (mode == 1) launch<T, 1>(x, res, gamma, beta, gamma2, beta2, n, c, eps, out0, out1, stream);
+    else if (mode == 2) launch<T, 2>(x, res, gamma, beta, gamma2, beta2, n, c, eps, out0, out1, stream);
+    else launch<T, 3>(x, res, gamma, beta, gamma2, beta2, n, c, eps, out0, out1, stream);
+}
+
+}  // namespace
+
+extern "C" int ptv3_layer_norm(const void* x, const void* res, const void* gamma, const void* beta,
+                               const void* gamma2, const void* beta2, int dtype, int64_t n, int c,
+                               float eps, int mode, void* out0, void* out1, void* stream_) {
+    if (n < 0 || c < 1 || mode < 0 || mode > 3) return PTV3_EINVAL;
+    if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
+    if (n == 0) return PTV3_OK;
+    if (!x || !gamma || !beta || !out0) return PTV3_EINVAL;
+    if (mode != 0 && !res) return PTV3_EINVAL;
+    if (mode >= 2 && !out1) return PTV3_EINVAL;
+    if (mode == 3 && (!gamma2 || !beta2)) return PTV3_EINVAL;
+    hipStream_t stream = (hipStream_t)stream_;
+    if (dtype == PTV3_F32)
+        launch_mode<float>(mode, x, res, gamma, beta, gamma2, beta2, n, c, eps, out0, out1, stream);
+    else if (dtype == PTV3_F16)
+        launch_mode<_Float16>(mode, x, res, gamma, beta, gamma2, beta2, n, c, eps, out0, out1, stream);
+    else
+        launch_mode<__bf16>(mode, x, res, gamma, beta, gamma2, beta2, n, c, eps, out0, out1, stream);
+    PTV3_RETURN_LAUNCH();
+}

@@ -38,18 +38,25 @@ __global__ __launch_bounds__(SORT_THREADS) void tile_hist_kernel(
     tile_hist[((int64_t)row * tiles + tile) * RADIX + tid] = hist[tid];
 }
 
-// One block per row. Thread d owns digit d: serial exclusive scan over the tiles, then a
-// block-wide exclusive scan over the digit totals; the digit base is folded back in.
+// One block per row. Thread d owns digit d: exclusive scan over the tiles (loads issued 16 at
+// a time so they overlap), then a block-wide exclusive scan over the digit totals; the digit
+// base is folded back in.
 __global__ __launch_bounds__(RADIX) void tile_scan_kernel(uint32_t* __restrict__ tile_hist,
                                                           int tiles) {
     __shared__ uint32_t total[RADIX];
+    constexpr int CH = 16;
     const int row = blockIdx.x, d = threadIdx.x;
-    uint32_t* h = tile_hist + (int64_t)row * tiles * RADIX;
+    uint32_t* h = tile_hist + (int64_t)row * tiles * RADIX + d;
     uint32_t run = 0;
-    for (int t = 0; t < tiles; ++t) {
-        const uint32_t c = h[(int64_t)t * RADIX + d];
-        h[(int64_t)t * RADIX + d] = run;
-        run += c;
+    for (int t0 = 0; t0 < tiles; t0 += CH) {
+        uint32_t c[CH];
+#pragma unroll
+        for (int j = 0; j < CH; ++j) c[j] = (t0 + j < tiles) ? h[(int64_t)(t0 + j) * RADIX] : 0u;
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+            if (t0 + j < tiles) h[(int64_t)(t0 + j) * RADIX] = run;
+            run += c[j];
+        }
     }
     total[d] = run;
     __syncthreads();
@@ -61,8 +68,13 @@ __global__ __launch_bounds__(RADIX) void tile_scan_kernel(uint32_t* __restrict__
         __syncthreads();
     }
     const uint32_t dbase = total[d] - run;
-    if (dbase != 0)
-        for (int t = 0; t < tiles; ++t) h[(int64_t)t * RADIX + d] += dbase;
+    if (dbase != 0) {
+        for (int t0 = 0; t0 < tiles; t0 += CH) {
+#pragma unroll
+            for (int j = 0; j < CH; ++j)
+                if (t0 + j < tiles) h[(int64_t)(t0 + j) * RADIX] += dbase;
+        }
+    }
 }
 
 template <bool FIRST, bool LAST>

@@ -5,7 +5,7 @@ from functools import partial
 import torch
 import torch.nn as nn
 
-from .modules import (MLP, Block, DropPath, Embedding, PDNorm, PointModule, PointSequential,  # noqa: F401
+from .modules import (MLP, Block, DropPath, Embedding, LayerNorm, PDNorm, PointModule, PointSequential,  # noqa: F401
                       SerializedAttention, SerializedPooling, SerializedUnpooling)
 from .point import Point, batch2offset, offset2batch, offset2bincount  # noqa: F401
 from .sparse import SparseConvTensor, SubMConv3d  # noqa: F401
@@ -60,9 +60,9 @@ class PointTransformerV3(PointModule):
         if pdnorm_bn:
             bn = partial(PDNorm, norm_layer=partial(nn.BatchNorm1d, eps=1e-3, momentum=0.01,
                                                     affine=pdnorm_affine), **pd)
-        ln = nn.LayerNorm
+        ln = LayerNorm
         if pdnorm_ln:
-            ln = partial(PDNorm, norm_layer=partial(nn.LayerNorm, elementwise_affine=pdnorm_affine), **pd)
+            ln = partial(PDNorm, norm_layer=partial(LayerNorm, elementwise_affine=pdnorm_affine), **pd)
         act = nn.GELU
 
         def make_block(channels, heads, patch, rate, i, stage):

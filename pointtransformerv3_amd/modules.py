@@ -32,6 +32,15 @@ class DropPath(nn.Module):
         return x * mask
 
 
+class LayerNorm(nn.LayerNorm):
+    """nn.LayerNorm (same parameters and state_dict) evaluated by the row-wise HIP kernel."""
+
+    def forward(self, x):
+        if x.dim() != 2 or len(self.normalized_shape) != 1 or self.weight is None or self.bias is None:
+            return super().forward(x)
+        return ops.layer_norm(x, self.weight, self.bias, self.eps)
+
+
 class PointModule(nn.Module):
     """Marker base class: PointSequential hands the whole Point to subclasses (model.py:177-183)."""
 
@@ -217,7 +226,7 @@ class Block(PointModule):
     """xCPE conv + attention + MLP, each with a residual (model.py:519-606)."""
 
     def __init__(self, channels, num_heads, patch_size=48, mlp_ratio=4.0, qkv_bias=True, qk_scale=None,
-                 attn_drop=0.0, proj_drop=0.0, drop_path=0.0, norm_layer=nn.LayerNorm, act_layer=nn.GELU,
+                 attn_drop=0.0, proj_drop=0.0, drop_path=0.0, norm_layer=LayerNorm, act_layer=nn.GELU,
                  pre_norm=True, order_index=0, cpe_indice_key=None, enable_rpe=False, enable_flash=True,
                  upcast_attention=True, upcast_softmax=True):
         super().__init__()
@@ -238,7 +247,33 @@ class Block(PointModule):
                                        out_channels=channels, act_layer=act_layer, drop=proj_drop))
         self.drop_path = PointSequential(DropPath(drop_path) if drop_path > 0.0 else nn.Identity())
 
+    def _plain_layernorms(self):
+        """True when the three norms are affine LayerNorms this file can fuse with the residual
+        adds around them (the default model); PDNorm or post-norm blocks take the modular path."""
+        mods = (self.cpe[2], self.norm1[0], self.norm2[0])
+        return (self.pre_norm and all(type(m) is LayerNorm and m.weight is not None for m in mods)
+                and not (self.training and not isinstance(self.drop_path[0], nn.Identity)))
+
     def forward(self, point):
+        if not self._plain_layernorms():
+            return self._forward_modular(point)
+        ln_cpe, ln1, ln2 = self.cpe[2], self.norm1[0], self.norm2[0]
+        # xCPE: conv reads the sparse view, which lags behind feat in the first decoder block
+        conv = self.cpe[0](point.sparse_conv_feat).features
+        branch = self.cpe[1](conv)
+        # feat = shortcut + LN(branch) and its pre-norm for attention, in one pass
+        feat, normed = ops.layer_norm(branch, ln_cpe.weight, ln_cpe.bias, ln_cpe.eps, residual=point.feat,
+                                      mode=3, weight2=ln1.weight, bias2=ln1.bias)
+        point.feat = normed
+        point = self.attn(point)
+        # feat += attention branch, plus the pre-norm for the MLP
+        feat, normed = ops.layer_norm(point.feat, ln2.weight, ln2.bias, ln2.eps, residual=feat, mode=2)
+        feat = feat + self.mlp[0](normed)
+        point.feat = feat
+        point.sparse_conv_feat = point.sparse_conv_feat.replace_feature(feat)
+        return point
+
+    def _forward_modular(self, point):
         skip = point.feat
         point = self.cpe(point)
         point.feat = skip + point.feat
@@ -258,8 +293,8 @@ class Block(PointModule):
         point.feat = skip + point.feat
         if not self.pre_norm:
             point = self.norm2(point)
-        # the sparse view is refreshed only here (model.py:605); within the block the conv of
-        # the NEXT block therefore sees exactly this tensor
+        # the sparse view is refreshed only here (model.py:605); the conv of the NEXT block
+        # therefore sees exactly this tensor
         point.sparse_conv_feat = point.sparse_conv_feat.replace_feature(point.feat)
         return point
 
@@ -321,6 +356,8 @@ class SerializedPooling(PointModule):
         if self.traceable:
             fields["pooling_inverse"] = cluster
             fields["pooling_parent"] = point
+        # max(x >> d) == max(x) >> d: the pooled grid extent needs no reduction and no sync
+        fields["_grid_max_host"] = [v >> pooling_depth for v in point.grid_max_host()]
         pooled = Point(fields)
         if self.norm is not None:
             pooled = self.norm(pooled)

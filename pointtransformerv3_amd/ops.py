@@ -240,3 +240,25 @@ def unpool_add(parent, child, cluster):
                                    _ptr(cluster.contiguous()), child.shape[0], _ptr(out), _stream()),
                "ptv3_unpool_add")
     return out
+
+
+def layer_norm(x, weight, bias, eps=1e-5, residual=None, mode=0, weight2=None, bias2=None):
+    """Row-wise LayerNorm fused with neighbouring residual adds.
+
+    mode 0: LN(x).  mode 1: residual + LN(x).  mode 2: (s, LN(s)) with s = x + residual.
+    mode 3: (y, LN2(y)) with y = residual + LN(x) and LN2 using weight2/bias2."""
+    _dev(x, weight, bias, residual, weight2, bias2)
+    lib = _lib.load()
+    x = x.contiguous()
+    n, c = x.shape
+    dt = x.dtype
+    w, b = weight.to(dt).contiguous(), bias.to(dt).contiguous()
+    res = None if residual is None else residual.to(dt).contiguous()
+    w2 = None if weight2 is None else weight2.to(dt).contiguous()
+    b2 = None if bias2 is None else bias2.to(dt).contiguous()
+    out0 = torch.empty_like(x)
+    out1 = torch.empty_like(x) if mode >= 2 else None
+    _lib.check(lib.ptv3_layer_norm(_ptr(x), _ptr(res), _ptr(w), _ptr(b), _ptr(w2), _ptr(b2), _dtype_code(x),
+                                   n, c, float(eps), int(mode), _ptr(out0), _ptr(out1), _stream()),
+               "ptv3_layer_norm")
+    return out0 if mode < 2 else (out0, out1)

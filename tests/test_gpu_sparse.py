@@ -100,3 +100,30 @@ def test_segment_reduce_and_unpool(dtype):
     gotu = o.unpool_add(feat.to(DEV), child.to(DEV), to_dev(pc["cluster"]))
     wantu = OF.unpool_add(feat.float(), child.float(), pc["cluster"])
     assert rel_err(gotu, wantu) < (1e-6 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("c", [32, 64, 128, 256, 512, 48])
+def test_layer_norm_modes(dtype, c):
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(c)
+    n = 3001
+    x = (torch.randn(n, c, generator=g) * 2 + 0.5).to(dtype)
+    r = torch.randn(n, c, generator=g).to(dtype)
+    w, b = (torch.rand(c, generator=g) + 0.5).to(dtype), torch.randn(c, generator=g).to(dtype)
+    w2, b2 = (torch.rand(c, generator=g) + 0.5).to(dtype), torch.randn(c, generator=g).to(dtype)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+
+    def ln(v, ww, bb):
+        return F.layer_norm(v.float(), (c,), ww.float(), bb.float(), 1e-5)
+
+    o = ops()
+    dv = lambda t: t.to(DEV)
+    assert rel_err(o.layer_norm(dv(x), dv(w), dv(b)), ln(x, w, b)) < tol
+    assert rel_err(o.layer_norm(dv(x), dv(w), dv(b), residual=dv(r), mode=1), r.float() + ln(x, w, b).to(dtype).float()) < tol
+    s, z = o.layer_norm(dv(x), dv(w), dv(b), residual=dv(r), mode=2)
+    want_s = (x.float() + r.float()).to(dtype)
+    assert rel_err(s, want_s.float()) < tol and rel_err(z, ln(want_s, w, b)) < tol
+    y, z = o.layer_norm(dv(x), dv(w), dv(b), residual=dv(r), mode=3, weight2=dv(w2), bias2=dv(b2))
+    want_y = (r.float() + ln(x, w, b).to(dtype).float()).to(dtype)
+    assert rel_err(y, want_y.float()) < tol and rel_err(z, ln(want_y, w2, b2)) < tol
