@@ -14,6 +14,12 @@
 //     are already in operand layout for the second product O^T = V^T * P^T.
 //   * V^T only fills 16 of the 32 rows of that product; rows 16 and 20 are fed ones so the
 //     softmax denominator falls out of the same MFMA instead of costing VALU adds.
+//   * At head_dim 16 the kernel is bound by the exponentials (one quarter-rate v_exp_f32 per
+//     score against 64 MFMA flops), so everything else is taken off the VALU: q is scaled by
+//     scale*log2(e) once, the running reference maximum enters through the MFMA's C operand
+//     so scores arrive already shifted, and the reference only moves when a score exceeds it
+//     by 2^8 -- which a |q||k| bound rules out for most 64-key steps without looking at the
+//     scores.
 //   * Rows are read through slot_src and written through slot_dst, so the padded,
 //     permuted qkv tensor of the reference is never materialised.
 // fp32 kernel: one thread per query, K/V chunks staged in LDS, plain FMA arithmetic.
@@ -34,7 +40,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int HD = 16;             // head dim
-constexpr int ATT_THREADS = 256;   // 4 waves
+constexpr int ATT_THREADS = 512;   // 8 waves, two work-groups per CU -> 4 waves per SIMD
 constexpr int ATT_WAVES = ATT_THREADS / PTV3_WAVE;
 constexpr int VT_PAD_BYTES = 16;   // skews V^T rows across LDS banks
 
@@ -70,28 +76,66 @@ __device__ __forceinline__ int vt_pos(int kk) {
     return ((kk >> 2) & 1) * 16 + (kk >> 3) * 4 + (kk & 3);
 }
 
+// Scores may exceed the running reference maximum by this much (log2 units) before the
+// accumulators are rescaled: probabilities then stay below 2^8, safe for fp16 operands.
+constexpr float RESCALE_SLACK = 8.f;
+
 template <typename T>
-__global__ __launch_bounds__(ATT_THREADS, 2) void patch_attn_half_kernel(
+__device__ __forceinline__ float sum_sq8(u32x4 w) {
+    typedef typename Half<T>::v8 v8;
+    const v8 h = __builtin_bit_cast(v8, w);
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s = fmaf((float)h[i], (float)h[i], s);
+    return s;
+}
+
+template <typename T>
+__device__ __forceinline__ u32x4 scale8(u32x4 w, float c) {
+    typedef typename Half<T>::v8 v8;
+    const v8 h = __builtin_bit_cast(v8, w);
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = Half<T>::pack2((float)h[2 * i] * c, (float)h[2 * i + 1] * c);
+    return r;
+}
+
+// Work-group id -> (sequence, head) such that the heads of one sequence, which share cache
+// lines of the qkv rows, run on the same XCD (work-groups are dealt round-robin to 8 XCDs).
+__device__ __forceinline__ int xcd_chunked_id(int bid, int total) {
+    const int xcd = bid & 7, slot = bid >> 3;
+    const int per = total >> 3, rem = total & 7;
+    return xcd * per + min(xcd, rem) + slot;
+}
+
+template <typename T>
+__global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
     const T* __restrict__ qkv, int channels, int heads, const int32_t* __restrict__ slot_src,
     const int32_t* __restrict__ slot_dst, const int32_t* __restrict__ cu_seqlens, int lds_keys,
     float scale_log2e, T* __restrict__ out) {
     typedef typename Half<T>::v8 v8;
     extern __shared__ __align__(16) unsigned char smem[];
-    // K tile: lds_keys rows of 32 B. V^T tile: 16 rows of (lds_keys*2 + pad) B.
+    // K tile: lds_keys rows of 32 B. V^T tile: 16 rows of (lds_keys*2 + pad) B. Then one float
+    // per 64-key pair: the largest key norm of the pair.
     unsigned char* k_lds = smem;
     const int vt_stride = lds_keys * 2 + VT_PAD_BYTES;
     unsigned char* vt_lds = smem + (size_t)lds_keys * 32;
+    float* knorm_lds = (float*)(vt_lds + (size_t)HD * vt_stride);
 
-    const int seq = blockIdx.x / heads, head = blockIdx.x % heads;
+    const int wg = xcd_chunked_id(blockIdx.x, gridDim.x);
+    const int seq = wg / heads, head = wg % heads;
     const int s0 = cu_seqlens[seq];
     const int len = cu_seqlens[seq + 1] - s0;
     if (len <= 0) return;
-    const int len32 = (len + 31) & ~31;
+    const int len64 = (len + 63) & ~63;
+    const int n_pairs = len64 / 64;
     const int tid = threadIdx.x;
     const int64_t row_stride = 3 * (int64_t)channels;
 
+    for (int i = tid; i < n_pairs; i += ATT_THREADS) knorm_lds[i] = 0.f;
+    __syncthreads();
     // ---- stage K and V^T: thread handles (key, 8-channel half)
-    for (int e = tid; e < len32 * 2; e += ATT_THREADS) {
+    for (int e = tid; e < len64 * 2; e += ATT_THREADS) {
         const int key = e >> 1, part = e & 1;
         u32x4 kq = {0, 0, 0, 0}, vq = {0, 0, 0, 0};
         if (key < len) {
@@ -100,20 +144,23 @@ __global__ __launch_bounds__(ATT_THREADS, 2) void patch_attn_half_kernel(
             vq = *(const u32x4*)(base + 2 * channels);
         }
         *(u32x4*)(k_lds + key * 32 + part * 16) = kq;
+        float nsq = sum_sq8<T>(kq);
+        nsq += __shfl_xor(nsq, 1, PTV3_WAVE);   // the other half of the same key
+        if (part == 0) atomicMax((int*)&knorm_lds[key >> 6], __float_as_int(nsq));   // nsq >= 0
         const int pos = (key & ~31) + vt_pos(key & 31);
-        uint16_t* vt = (uint16_t*)(vt_lds + (size_t)(part * 8) * vt_stride) + pos;
+        unsigned char* vt = vt_lds + (size_t)(part * 8) * vt_stride + pos * 2;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const uint32_t w = vq[c];
-            *(uint16_t*)((unsigned char*)vt + (size_t)(2 * c) * vt_stride) = (uint16_t)(w & 0xffffu);
-            *(uint16_t*)((unsigned char*)vt + (size_t)(2 * c + 1) * vt_stride) = (uint16_t)(w >> 16);
+            *(uint16_t*)(vt + (size_t)(2 * c) * vt_stride) = (uint16_t)(w & 0xffffu);
+            *(uint16_t*)(vt + (size_t)(2 * c + 1) * vt_stride) = (uint16_t)(w >> 16);
         }
     }
     __syncthreads();
 
     const int wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
     const int col = lane & 31, hf = lane >> 5;
-    const int n_tiles = len32 / 32;
+    const int n_qtiles = (len + 31) / 32;
 
     // A operand rows of the second product: d < 16 read V^T, rows 16 and 20 are ones.
     u32x4 ones4;
@@ -121,8 +168,10 @@ __global__ __launch_bounds__(ATT_THREADS, 2) void patch_attn_half_kernel(
         const uint32_t o = (col == 16 || col == 20) ? (Half<T>::one() * 0x10001u) : 0u;
         ones4 = (u32x4){o, o, o, o};
     }
+    const unsigned char* k_base = k_lds + col * 32 + hf * 16;
+    const unsigned char* v_base = vt_lds + (size_t)(col & 15) * vt_stride + hf * 32;
 
-    for (int qt = wave; qt < n_tiles; qt += ATT_WAVES) {
+    for (int qt = wave; qt < n_qtiles; qt += ATT_WAVES) {
         const int qi = qt * 32 + col;   // my query inside the sequence
         int dst = -1;
         u32x4 qreg = {0, 0, 0, 0};
@@ -131,50 +180,73 @@ __global__ __launch_bounds__(ATT_THREADS, 2) void patch_attn_half_kernel(
             qreg = *(const u32x4*)(qkv + (int64_t)slot_src[s0 + qi] * row_stride + head * HD + hf * 8);
         }
         if (__ballot(dst >= 0) == 0) continue;   // tile of filler slots only
+        // scores come out of the MFMA in log2 units: q is scaled by scale * log2(e) up front
+        qreg = scale8<T>(qreg, scale_log2e);
         const v8 qfrag = __builtin_bit_cast(v8, qreg);
+        float qn = sum_sq8<T>(qreg);
+        qn += __shfl_xor(qn, 32, PTV3_WAVE);
+        const float qnorm = sqrtf(qn) * 1.0009765625f;   // margin for rounding in the bound
 
-        f32x16 acc;
+        f32x16 acc, cinit;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-        float m = -INFINITY;   // running max of raw scores (same in lane and lane^32)
+        for (int v = 0; v < 16; ++v) { acc[v] = 0.f; cinit[v] = 0.f; }
+        float m_ref = 0.f;   // reference maximum: the MFMA adds -m_ref to every score
 
-        for (int kt = 0; kt < n_tiles; ++kt) {
-            const v8 kfrag = __builtin_bit_cast(v8, *(const u32x4*)(k_lds + (kt * 32 + col) * 32 + hf * 16));
-            f32x16 s;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) s[v] = 0.f;
-            s = Half<T>::mfma(kfrag, qfrag, s);   // s[v] = <K[key_v], Q[q]>
-            if (kt == n_tiles - 1 && len != len32) {
+        for (int kp = 0; kp < n_pairs; ++kp) {
+            const v8 k0 = __builtin_bit_cast(v8, *(const u32x4*)(k_base + (kp * 64) * 32));
+            const v8 k1 = __builtin_bit_cast(v8, *(const u32x4*)(k_base + (kp * 64 + 32) * 32));
+            f32x16 sa = Half<T>::mfma(k0, qfrag, cinit);   // sa[v] = <K[key_v], Q[q]> - m_ref
+            f32x16 sb = Half<T>::mfma(k1, qfrag, cinit);
+            if (kp == n_pairs - 1 && len != len64) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const int key = kt * 32 + 8 * (v >> 2) + 4 * hf + (v & 3);
-                    if (key >= len) s[v] = -INFINITY;
+                    const int key = kp * 64 + 8 * (v >> 2) + 4 * hf + (v & 3);
+                    if (key >= len) sa[v] = -INFINITY;
+                    if (key + 32 >= len) sb[v] = -INFINITY;
                 }
             }
-            float mt = s[0];
+            // |score| <= |q| |k|: when even that bound stays within the slack nothing can
+            // overflow and the running reference is left alone (no max reduction at all)
+            const float bound = qnorm * sqrtf(knorm_lds[kp]) - m_ref;
+            const bool first = (kp == 0);
+            if (first || __ballot(bound > RESCALE_SLACK) != 0) {
+                float mx = fmaxf(sa[0], sb[0]);
 #pragma unroll
-            for (int v = 1; v < 16; ++v) mt = fmaxf(mt, s[v]);
-            mt = fmaxf(mt, __shfl_xor(mt, 32, PTV3_WAVE));
-            const float m_new = fmaxf(m, mt);
-            const float alpha = exp2f((m - m_new) * scale_log2e);
-            const float mc = m_new * scale_log2e;
-            m = m_new;
+                for (int v = 1; v < 16; ++v) mx = fmaxf(mx, fmaxf(sa[v], sb[v]));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, PTV3_WAVE));
+                const bool move = first || mx > RESCALE_SLACK;
+                if (__ballot(move) != 0) {
+                    const float delta = move ? mx : 0.f;
+                    const float alpha = first ? 1.f : exp2f(-delta);
+                    m_ref += delta;
 #pragma unroll
-            for (int v = 0; v < 9; ++v) acc[v] *= alpha;   // rows 0..15 (+ the denominator row)
-            uint32_t p[8];
+                    for (int v = 0; v < 16; ++v) {
+                        sa[v] -= delta;
+                        sb[v] -= delta;
+                        cinit[v] = -m_ref;
+                    }
 #pragma unroll
-            for (int v = 0; v < 8; ++v)
-                p[v] = Half<T>::pack2(exp2f(fmaf(s[2 * v], scale_log2e, -mc)),
-                                      exp2f(fmaf(s[2 * v + 1], scale_log2e, -mc)));
-            u32x4 va = ones4, vb = ones4;
-            if (col < HD) {
-                const unsigned char* vrow = vt_lds + (size_t)col * vt_stride + (kt * 32 + hf * 16) * 2;
-                va = *(const u32x4*)vrow;
-                vb = *(const u32x4*)(vrow + 16);
+                    for (int v = 0; v < 9; ++v) acc[v] *= alpha;   // rows 0..15 + denominator row
+                }
             }
-            const u32x4 pa = {p[0], p[1], p[2], p[3]}, pb = {p[4], p[5], p[6], p[7]};
-            acc = Half<T>::mfma(__builtin_bit_cast(v8, va), __builtin_bit_cast(v8, pa), acc);
-            acc = Half<T>::mfma(__builtin_bit_cast(v8, vb), __builtin_bit_cast(v8, pb), acc);
+            uint32_t pa[8], pb[8];
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                pa[v] = Half<T>::pack2(__builtin_amdgcn_exp2f(sa[2 * v]), __builtin_amdgcn_exp2f(sa[2 * v + 1]));
+                pb[v] = Half<T>::pack2(__builtin_amdgcn_exp2f(sb[2 * v]), __builtin_amdgcn_exp2f(sb[2 * v + 1]));
+            }
+            u32x4 va0 = ones4, va1 = ones4, vb0 = ones4, vb1 = ones4;
+            if (col < HD) {
+                const unsigned char* vrow = v_base + (kp * 64) * 2;
+                va0 = *(const u32x4*)vrow;
+                va1 = *(const u32x4*)(vrow + 16);
+                vb0 = *(const u32x4*)(vrow + 64);
+                vb1 = *(const u32x4*)(vrow + 80);
+            }
+            acc = Half<T>::mfma(__builtin_bit_cast(v8, va0), __builtin_bit_cast(v8, (u32x4){pa[0], pa[1], pa[2], pa[3]}), acc);
+            acc = Half<T>::mfma(__builtin_bit_cast(v8, va1), __builtin_bit_cast(v8, (u32x4){pa[4], pa[5], pa[6], pa[7]}), acc);
+            acc = Half<T>::mfma(__builtin_bit_cast(v8, vb0), __builtin_bit_cast(v8, (u32x4){pb[0], pb[1], pb[2], pb[3]}), acc);
+            acc = Half<T>::mfma(__builtin_bit_cast(v8, vb1), __builtin_bit_cast(v8, (u32x4){pb[4], pb[5], pb[6], pb[7]}), acc);
         }
         // acc[v]: d = 8*(v/4) + 4*hf + v%4; acc[8] = sum of probabilities (row 16 / 20)
         if (dst >= 0) {
@@ -263,12 +335,17 @@ template <typename T>
 int launch_half(const void* qkv, int channels, int heads, const int32_t* slot_src,
                 const int32_t* slot_dst, const int32_t* cu_seqlens, int64_t n_seq,
                 int64_t max_seqlen, float scale, void* out, hipStream_t stream) {
-    const int lds_keys = (int)((max_seqlen + 31) & ~31ll);
-    const size_t lds = (size_t)lds_keys * 32 + (size_t)HD * (lds_keys * 2 + VT_PAD_BYTES);
+    const int lds_keys = (int)((max_seqlen + 63) & ~63ll);
+    const size_t lds = (size_t)lds_keys * 32 + (size_t)HD * (lds_keys * 2 + VT_PAD_BYTES) +
+                       (size_t)(lds_keys / 64) * sizeof(float);
     if (lds > 160 * 1024) return PTV3_ESHAPE;
     auto kern = patch_attn_half_kernel<T>;
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
+    static size_t lds_allowed = 0;   // per instantiation; raised monotonically
+    if (lds > lds_allowed) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        lds_allowed = lds;
+    }
     const float scale_log2e = scale * 1.4426950408889634f;
     hipLaunchKernelGGL(kern, dim3((unsigned)(n_seq * heads)), dim3(ATT_THREADS), lds, stream,
                        (const T*)qkv, channels, heads, slot_src, slot_dst, cu_seqlens, lds_keys,
