@@ -85,18 +85,41 @@ int ptv3_patch_attn_fwd(const void *qkv, int dtype, int64_t n_rows, int channels
 
 /* spconv.SubMConv3d's index generation (call sites model.py:546-552, :767-774, tensor built
  * at :165-172). indices (n,4) int32 [batch,x,y,z], coordinates in [0, 65535];
- * nbr (n, ks^3) int32: nbr[i][(kx*ks+ky)*ks+kz] = row of the voxel at
- * (b, x+kx-ks/2, y+ky-ks/2, z+kz-ks/2) or -1. ks is 3 or 5. */
+ * nbr int32, entry (voxel i, tap t = (kx*ks+ky)*ks+kz) = row of the voxel at
+ * (b, x+kx-ks/2, y+ky-ks/2, z+kz-ks/2) or -1; stored voxel-major (n, ks^3) when tap_major == 0,
+ * tap-major (ks^3, n) otherwise (the layout the convolution kernels read coalesced; every
+ * function below that takes nbr also takes this flag). ks is 3 or 5. */
 size_t ptv3_kmap_workspace_bytes(int64_t n);
-int ptv3_kmap_build(const int32_t *indices, int64_t n, int ks, int32_t *nbr, void *workspace,
-                    size_t workspace_bytes, void *stream);
+int ptv3_kmap_build(const int32_t *indices, int64_t n, int ks, int tap_major, int32_t *nbr,
+                    void *workspace, size_t workspace_bytes, void *stream);
 
 /* spconv.SubMConv3d forward (same call sites): out[i] = bias + sum_k W[:,k,:] feat[nbr[i][k]].
  * feat (n,cin), weight (cout, V, cin) (spconv 2.x KRSC layout flattened over the taps),
  * bias (cout,) or NULL, out (n,cout); all of `dtype`, accumulation in fp32. */
 int ptv3_subm_conv_fwd(const void *feat, int dtype, int64_t n, int cin, const int32_t *nbr,
-                       int taps, const void *weight, const void *bias, int cout, void *out,
-                       void *stream);
+                       int taps, int tap_major, const void *weight, const void *bias, int cout,
+                       void *out, void *stream);
+
+/* Sparse-pair form of the same convolution, for maps where most taps of most voxels are empty
+ * (surface scans: 2-13 of 27 taps active). ptv3_conv_plan_count derives from nbr (n,taps) the
+ * number of active (input, output) pairs per tap (tap_ptr, taps+1 int32, exclusive) and in total
+ * (n_pairs, device int64); after reading n_pairs on the host, ptv3_conv_plan_fill writes
+ * row_ptr (n+1 int32: first output slot of every voxel), and per tap-major pair its input row
+ * (pair_in) and output slot (pair_slot), both (n_pairs,) int32. Same workspace for both calls,
+ * >= ptv3_conv_plan_workspace_bytes(n, taps); taps <= 128.
+ * ptv3_subm_conv_pairs_fwd multiplies every pair's input row by its tap's weight matrix with
+ * fully populated MFMA tiles into y (n_pairs, cout) and sums each voxel's slots (+bias) into
+ * out (n, cout). fp16/bf16 only; cin % 16 == 0, cout % 8 == 0. */
+size_t ptv3_conv_plan_workspace_bytes(int64_t n, int taps);
+int ptv3_conv_plan_count(const int32_t *nbr, int64_t n, int taps, int tap_major, int32_t *tap_ptr,
+                         int64_t *n_pairs, void *workspace, size_t workspace_bytes, void *stream);
+int ptv3_conv_plan_fill(const int32_t *nbr, int64_t n, int taps, int tap_major, const int32_t *tap_ptr,
+                        int32_t *row_ptr, int32_t *pair_in, int32_t *pair_slot, void *workspace,
+                        size_t workspace_bytes, void *stream);
+int ptv3_subm_conv_pairs_fwd(const void *feat, int dtype, int64_t n, int cin, int taps,
+                             int64_t n_pairs, const int32_t *tap_ptr, const int32_t *row_ptr,
+                             const int32_t *pair_in, const int32_t *pair_slot, const void *weight,
+                             const void *bias, int cout, void *y, void *out, void *stream);
 
 /* model.py:652-664,690-695: clusters of code0 >> shift walked in sorted order (order0 sorts
  * code0, so no further sort is needed). Outputs: cluster (n,) int64 [pooling_inverse],

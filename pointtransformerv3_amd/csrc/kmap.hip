@@ -2,12 +2,14 @@
 //
 // Replaces the index generation spconv performs for SubMConv3d (reference call sites
 // model.py:546-552 and :767-774 on the tensor built at :165-172). Canonical output:
-// nbr[i][(kx*ks+ky)*ks+kz] = row of the voxel at coord_i + (kx,ky,kz) - ks/2, or -1.
+// entry (voxel i, tap (kx*ks+ky)*ks+kz) = row of the voxel at coord_i + (kx,ky,kz) - ks/2, or -1,
+// stored voxel-major (n, taps) or tap-major (taps, n); the convolution kernels read the
+// tap-major form coalesced.
 //
 //   fill    : table keys <- EMPTY
 //   insert  : one thread per voxel, 64-bit CAS, linear probing (load factor <= 0.5)
-//   lookup  : one thread per (voxel, tap) so the int32 map is written fully coalesced;
-//             the 16 B voxel record is shared by the ks^3 threads of a voxel through L1
+//   lookup  : one thread per map entry in storage order, so the int32 map is written fully
+//             coalesced in either layout
 #include "common.h"
 
 namespace {
@@ -54,15 +56,17 @@ __global__ __launch_bounds__(256) void kmap_insert_kernel(const int32_t* __restr
     }
 }
 
+template <bool TAP_MAJOR>
 __global__ __launch_bounds__(256) void kmap_lookup_kernel(const int32_t* __restrict__ indices,
                                                           int64_t n, int ks, int taps,
                                                           const uint64_t* __restrict__ keys,
                                                           const int32_t* __restrict__ vals,
                                                           uint32_t mask, int32_t* __restrict__ nbr) {
+    // one thread per map entry, in the order the entries are stored, so writes coalesce
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= n * taps) return;
-    const int64_t i = e / taps;
-    const int t = (int)(e - i * taps);
+    const int64_t i = TAP_MAJOR ? e % n : e / taps;
+    const int t = (int)(TAP_MAJOR ? e / n : e - i * taps);
     const int r = ks >> 1;
     const int kz = t % ks, ky = (t / ks) % ks, kx = t / (ks * ks);
     const int4 v = ((const int4*)indices)[i];
@@ -96,7 +100,7 @@ extern "C" size_t ptv3_kmap_workspace_bytes(int64_t n) {
     return ptv3_align256((size_t)cap * sizeof(uint64_t)) + ptv3_align256((size_t)cap * sizeof(int32_t));
 }
 
-extern "C" int ptv3_kmap_build(const int32_t* indices, int64_t n, int ks, int32_t* nbr,
+extern "C" int ptv3_kmap_build(const int32_t* indices, int64_t n, int ks, int tap_major, int32_t* nbr,
                                void* workspace, size_t workspace_bytes, void* stream_) {
     if (n < 0 || n >= (1ll << 30)) return PTV3_EINVAL;
     if (ks != 3 && ks != 5) return PTV3_ESHAPE;
@@ -113,8 +117,11 @@ extern "C" int ptv3_kmap_build(const int32_t* indices, int64_t n, int ks, int32_
                        keys, cap);
     hipLaunchKernelGGL(kmap_insert_kernel, dim3((unsigned)ptv3_ceil_div(n, 256)), dim3(256), 0, stream,
                        indices, n, keys, vals, mask);
-    hipLaunchKernelGGL(kmap_lookup_kernel, dim3((unsigned)ptv3_ceil_div(n * taps, 256)), dim3(256), 0,
-                       stream, indices, n, ks, taps, (const uint64_t*)keys, (const int32_t*)vals, mask,
-                       nbr);
+    if (tap_major)
+        hipLaunchKernelGGL(kmap_lookup_kernel<true>, dim3((unsigned)ptv3_ceil_div(n * taps, 256)), dim3(256), 0,
+                           stream, indices, n, ks, taps, (const uint64_t*)keys, (const int32_t*)vals, mask, nbr);
+    else
+        hipLaunchKernelGGL(kmap_lookup_kernel<false>, dim3((unsigned)ptv3_ceil_div(n * taps, 256)), dim3(256), 0,
+                           stream, indices, n, ks, taps, (const uint64_t*)keys, (const int32_t*)vals, mask, nbr);
     PTV3_RETURN_LAUNCH();
 }

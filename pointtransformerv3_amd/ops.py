@@ -144,33 +144,92 @@ def patch_attention(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, 
     return out
 
 
-def kmap_build(indices, ks):
-    """(N, ks^3) int32 neighbour map of (N,4) int32 [batch,x,y,z] voxels."""
+def kmap_build(indices, ks, tap_major=False):
+    """int32 neighbour map of (N,4) int32 [batch,x,y,z] voxels: (N, ks^3), or (ks^3, N) when
+    tap_major (the layout the convolution kernels read coalesced)."""
     _dev(indices)
     lib = _lib.load()
     idx = indices.to(torch.int32).contiguous()
     n = idx.shape[0]
-    nbr = torch.empty((n, ks ** 3), dtype=torch.int32, device=idx.device)
+    shape = (ks ** 3, n) if tap_major else (n, ks ** 3)
+    nbr = torch.empty(shape, dtype=torch.int32, device=idx.device)
     nbytes = lib.ptv3_kmap_workspace_bytes(n)
     ws = _ws(nbytes, idx.device)
-    _lib.check(lib.ptv3_kmap_build(_ptr(idx), n, int(ks), _ptr(nbr), _ptr(ws), nbytes, _stream()),
-               "ptv3_kmap_build")
+    _lib.check(lib.ptv3_kmap_build(_ptr(idx), n, int(ks), int(bool(tap_major)), _ptr(nbr), _ptr(ws), nbytes,
+                                   _stream()), "ptv3_kmap_build")
     return nbr
 
 
-def subm_conv(feat, nbr, weight, bias=None):
-    """feat (N,Cin), nbr (N,V) int32, weight (Cout,V,Cin) or (Cout,k,k,k,Cin), bias (Cout,)."""
+def subm_conv(feat, nbr, weight, bias=None, tap_major=False):
+    """feat (N,Cin), nbr (N,V) int32 — or (V,N) when tap_major —, weight (Cout,V,Cin) or
+    (Cout,k,k,k,Cin), bias (Cout,). Dense output-stationary form (every tap of every voxel)."""
     _dev(feat, nbr, weight, bias)
+    lib = _lib.load()
+    feat = feat.contiguous()
+    nbr = nbr.contiguous()
+    n, cin = feat.shape
+    cout = weight.shape[0]
+    taps = nbr.shape[0] if tap_major else nbr.shape[1]
+    w = weight.reshape(cout, taps, cin).to(feat.dtype).contiguous()
+    b = None if bias is None else bias.to(feat.dtype).contiguous()
+    out = torch.empty((n, cout), dtype=feat.dtype, device=feat.device)
+    _lib.check(lib.ptv3_subm_conv_fwd(_ptr(feat), _dtype_code(feat), n, cin, _ptr(nbr), taps,
+                                      int(bool(tap_major)), _ptr(w), _ptr(b), cout, _ptr(out), _stream()),
+               "ptv3_subm_conv_fwd")
+    return out
+
+
+class ConvPlan:
+    """Active (input, output) pairs of a neighbour map, tap-major, plus each voxel's slots."""
+
+    __slots__ = ("n", "taps", "n_pairs", "tap_ptr", "row_ptr", "pair_in", "pair_slot")
+
+    def density(self):
+        return self.n_pairs / max(1, self.n * self.taps)
+
+
+def conv_plan(nbr, tap_major=False):
+    """Pair lists for subm_conv_pairs from a (N, taps) — or tap-major (taps, N) — neighbour map.
+    One host sync (the pair count)."""
+    _dev(nbr)
+    lib = _lib.load()
+    nbr = nbr.contiguous()
+    taps, n = nbr.shape if tap_major else nbr.shape[::-1]
+    tm = int(bool(tap_major))
+    dev = nbr.device
+    plan = ConvPlan()
+    plan.n, plan.taps = n, taps
+    plan.tap_ptr = torch.empty(taps + 1, dtype=torch.int32, device=dev)
+    count = torch.empty(1, dtype=torch.int64, device=dev)
+    nbytes = lib.ptv3_conv_plan_workspace_bytes(n, taps)
+    ws = _ws(nbytes, dev)
+    _lib.check(lib.ptv3_conv_plan_count(_ptr(nbr), n, taps, tm, _ptr(plan.tap_ptr), _ptr(count), _ptr(ws),
+                                        nbytes, _stream()), "ptv3_conv_plan_count")
+    plan.n_pairs = int(count.item())
+    plan.row_ptr = torch.empty(n + 1, dtype=torch.int32, device=dev)
+    plan.pair_in = torch.empty(max(plan.n_pairs, 1), dtype=torch.int32, device=dev)
+    plan.pair_slot = torch.empty(max(plan.n_pairs, 1), dtype=torch.int32, device=dev)
+    _lib.check(lib.ptv3_conv_plan_fill(_ptr(nbr), n, taps, tm, _ptr(plan.tap_ptr), _ptr(plan.row_ptr),
+                                       _ptr(plan.pair_in), _ptr(plan.pair_slot), _ptr(ws), nbytes, _stream()),
+               "ptv3_conv_plan_fill")
+    return plan
+
+
+def subm_conv_pairs(feat, plan, weight, bias=None):
+    """Submanifold convolution over the plan's active pairs only (fp16 / bf16)."""
+    _dev(feat, weight, bias)
     lib = _lib.load()
     feat = feat.contiguous()
     n, cin = feat.shape
     cout = weight.shape[0]
-    taps = nbr.shape[1]
-    w = weight.reshape(cout, taps, cin).to(feat.dtype).contiguous()
+    w = weight.reshape(cout, plan.taps, cin).to(feat.dtype).contiguous()
     b = None if bias is None else bias.to(feat.dtype).contiguous()
+    y = torch.empty((max(plan.n_pairs, 1), cout), dtype=feat.dtype, device=feat.device)
     out = torch.empty((n, cout), dtype=feat.dtype, device=feat.device)
-    _lib.check(lib.ptv3_subm_conv_fwd(_ptr(feat), _dtype_code(feat), n, cin, _ptr(nbr), taps, _ptr(w),
-                                      _ptr(b), cout, _ptr(out), _stream()), "ptv3_subm_conv_fwd")
+    _lib.check(lib.ptv3_subm_conv_pairs_fwd(_ptr(feat), _dtype_code(feat), n, cin, plan.taps, plan.n_pairs,
+                                            _ptr(plan.tap_ptr), _ptr(plan.row_ptr), _ptr(plan.pair_in),
+                                            _ptr(plan.pair_slot), _ptr(w), _ptr(b), cout, _ptr(y), _ptr(out),
+                                            _stream()), "ptv3_subm_conv_pairs_fwd")
     return out
 
 

@@ -26,19 +26,34 @@ class SparseConvTensor:
                                 self.indice_dict)
 
     def neighbour_map(self, kernel_size, indice_key=None):
+        """Tap-major (taps, N) int32 neighbour map, built once per indice_key."""
         key = (indice_key, kernel_size) if indice_key is not None else None
         if key is not None and key in self.indice_dict:
             return self.indice_dict[key]
-        nbr = ops.kmap_build(self.indices, kernel_size)
+        nbr = ops.kmap_build(self.indices, kernel_size, tap_major=True)   # (taps, N)
         if key is not None:
             self.indice_dict[key] = nbr
         return nbr
+
+    def conv_plan(self, kernel_size, indice_key=None):
+        """Pair lists of the neighbour map (see ops.conv_plan), cached like the map itself."""
+        key = ("plan", indice_key, kernel_size) if indice_key is not None else None
+        if key is not None and key in self.indice_dict:
+            return self.indice_dict[key]
+        plan = ops.conv_plan(self.neighbour_map(kernel_size, indice_key), tap_major=True)
+        if key is not None:
+            self.indice_dict[key] = plan
+        return plan
 
 
 class SubMConv3d(nn.Module):
     """Submanifold 3-D convolution: output sites = input sites. weight has spconv 2.x's
     (out, k, k, k, in) layout so checkpoints keep loading; `padding` is accepted and unused,
     as submanifold convolutions are centred by construction."""
+
+    # above this fraction of active (voxel, tap) pairs the dense output-stationary kernel wins
+    # (no pair buffer round trip); surface scans sit at 0.05-0.5
+    PAIR_MODE_MAX_DENSITY = 0.7
 
     def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
                  groups=1, bias=True, indice_key=None):
@@ -63,15 +78,23 @@ class SubMConv3d(nn.Module):
         feat = x.features
         if torch.is_autocast_enabled():
             feat = feat.to(torch.get_autocast_gpu_dtype())
-        nbr = x.neighbour_map(self.kernel_size, self.indice_key)
         weight = self.weight.reshape(self.out_channels, -1, self.in_channels)
         cin = self.in_channels
-        if feat.dtype != torch.float32 and cin % 16 != 0:
-            # the MFMA kernel consumes input channels 16 at a time: zero-pad the thin stem input
+        if feat.dtype == torch.float32:
+            nbr = x.neighbour_map(self.kernel_size, self.indice_key)
+            return x.replace_feature(ops.subm_conv(feat, nbr, weight, self.bias, tap_major=True))
+        if cin % 16 != 0:
+            # the MFMA kernels consume input channels 16 at a time: zero-pad the thin stem input
             pad = 16 - cin % 16
             feat = nn.functional.pad(feat, (0, pad))
             weight = nn.functional.pad(weight, (0, pad))
-        out = ops.subm_conv(feat, nbr, weight.to(feat.dtype), self.bias)
+        weight = weight.to(feat.dtype)
+        plan = x.conv_plan(self.kernel_size, self.indice_key)
+        if plan.density() <= self.PAIR_MODE_MAX_DENSITY and self.out_channels % 8 == 0:
+            out = ops.subm_conv_pairs(feat, plan, weight, self.bias)
+        else:
+            out = ops.subm_conv(feat, x.neighbour_map(self.kernel_size, self.indice_key), weight, self.bias,
+                                tap_major=True)
         return x.replace_feature(out)
 
 

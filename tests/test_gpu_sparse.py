@@ -127,3 +127,61 @@ def test_layer_norm_modes(dtype, c):
     y, z = o.layer_norm(dv(x), dv(w), dv(b), residual=dv(r), mode=3, weight2=dv(w2), bias2=dv(b2))
     want_y = (r.float() + ln(x, w, b).to(dtype).float()).to(dtype)
     assert rel_err(y, want_y.float()) < tol and rel_err(z, ln(want_y, w2, b2)) < tol
+
+
+@pytest.mark.parametrize("ks,n,extent", [(3, 1, 4), (3, 777, 12), (5, 3000, 20), (3, 40_000, 48)])
+def test_conv_plan_bit_exact(ks, n, extent):
+    rng = np.random.default_rng(n)
+    idx, *_ = _indices(rng, n, extent, 2)
+    nbr = OI.subm_kmap(idx, ks)
+    plan = ops().conv_plan(to_dev(nbr))
+    act = nbr >= 0
+    assert plan.n_pairs == int(act.sum())
+    # output-major slots: exclusive row-major rank of every active (voxel, tap)
+    want_row_ptr = np.concatenate([[0], np.cumsum(act.sum(1))])
+    assert np.array_equal(plan.row_ptr.cpu().numpy(), want_row_ptr)
+    assert np.array_equal(plan.tap_ptr.cpu().numpy(), np.concatenate([[0], np.cumsum(act.sum(0))]))
+    slot_of = np.cumsum(act.reshape(-1)).reshape(act.shape) - 1
+    vi, ti = np.nonzero(act.T)[1], np.nonzero(act.T)[0]    # tap-major enumeration, voxels ascending
+    assert np.array_equal(plan.pair_in.cpu().numpy()[:plan.n_pairs], nbr[vi, ti])
+    assert np.array_equal(plan.pair_slot.cpu().numpy()[:plan.n_pairs], slot_of[vi, ti])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("ks,cin,cout,n,extent", [(3, 32, 32, 3000, 20), (3, 64, 64, 50_000, 60), (3, 128, 128, 9000, 24),
+                                                  (3, 256, 256, 2000, 12), (3, 512, 512, 600, 8), (5, 16, 32, 20_000, 40)])
+def test_subm_conv_pairs_parity(dtype, ks, cin, cout, n, extent):
+    rng = np.random.default_rng(cin + n)
+    g = torch.Generator().manual_seed(cin + n)
+    idx, *_ = _indices(rng, n // 2, extent, 2)
+    nbr = OI.subm_kmap(idx, ks)
+    feat = torch.randn(len(idx), cin, generator=g).to(dtype)
+    bound = 1.0 / np.sqrt(ks ** 3 * cin)
+    w = ((torch.rand(cout, ks, ks, ks, cin, generator=g) * 2 - 1) * bound).to(dtype)
+    b = ((torch.rand(cout, generator=g) * 2 - 1) * bound).to(dtype) if ks == 3 else None
+    want = OF.subm_conv(feat.float(), nbr, w.float(), None if b is None else b.float())
+    o = ops()
+    plan = o.conv_plan(to_dev(nbr))
+    got = o.subm_conv_pairs(feat.to(DEV), plan, w.to(DEV), None if b is None else b.to(DEV))
+    assert got.dtype == dtype
+    assert rel_err(got, want) < TOL[dtype]
+
+
+def test_tap_major_layout_is_the_transpose():
+    rng = np.random.default_rng(12)
+    g = torch.Generator().manual_seed(12)
+    idx, *_ = _indices(rng, 5000, 24, 2)
+    o = ops()
+    for ks in (3, 5):
+        a = o.kmap_build(to_dev(idx), ks)
+        b = o.kmap_build(to_dev(idx), ks, tap_major=True)
+        assert b.shape == (ks ** 3, len(idx)) and torch.equal(a.t().contiguous(), b)
+        pa, pb = o.conv_plan(a), o.conv_plan(b, tap_major=True)
+        assert pa.n_pairs == pb.n_pairs
+        for f in ("tap_ptr", "row_ptr", "pair_in", "pair_slot"):
+            assert torch.equal(getattr(pa, f), getattr(pb, f)), f
+    nbr, nbr_t = o.kmap_build(to_dev(idx), 3), o.kmap_build(to_dev(idx), 3, tap_major=True)
+    for dtype in (torch.float32, torch.float16):
+        feat = torch.randn(len(idx), 64, generator=g).to(dtype).to(DEV)
+        w = (torch.randn(64, 27, 64, generator=g) * 0.05).to(dtype).to(DEV)
+        assert torch.equal(o.subm_conv(feat, nbr, w), o.subm_conv(feat, nbr_t, w, tap_major=True))
