@@ -75,6 +75,121 @@ def cpu_baseline(model, d, feat):
             "sample": f"one forward of the CPU oracle over scene 0 of the batch ({n0} points), {dt:.1f} s"}
 
 
+HBM_PEAK_GBS = 8000.0
+
+
+def _time_us(fn, iters=20, warmup=3):
+    """Average device time of fn() in microseconds (HIP events on the current stream)."""
+    for _ in range(warmup):
+        fn()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) * 1e3 / iters
+
+
+def kernel_rooflines(path):
+    """Per-kernel measurements at the sizes the baseline configs name, each against the roofline
+    that bounds it (algorithmic bytes or flops / measured time). Written to `path` as JSON."""
+    from oracle import indexing as OI
+    from pointtransformerv3_amd import ops, synthetic
+    dev = "cuda:0"
+    rows = []
+
+    def add(name, workload, bound, work, us, unit_work):
+        ach = work / (us * 1e-6) / (1e9 if bound == "hbm" else 1e12)
+        peak = HBM_PEAK_GBS if bound == "hbm" else MFMA_PEAK_TFLOPS
+        rows.append({"kernel": name, "workload": workload, "bound": bound, "us": us, "work": work,
+                     "work_unit": unit_work, "achieved": ach, "peak": peak,
+                     "unit": "GB/s" if bound == "hbm" else "TFLOP/s", "frac": ach / peak})
+
+    # ---- serialization: 4 room scenes, k = 4 orders, depth 9 (adaptive) and 16 (explicit)
+    d, _ = build_inputs(4, 106_000, 4000)
+    n = len(d["batch"])
+    g = torch.from_numpy(d["grid_coord"]).to(dev)
+    b = torch.from_numpy(d["batch"]).to(dev)
+    orders = ["z", "z-trans", "hilbert", "hilbert-trans"]
+    for depth in (9, 16):
+        us = _time_us(lambda: ops.encode_orders(g, b, depth, orders))
+        add("encode", f"{n} points, 4 orders, depth {depth}", "hbm", n * 52.0, us, "B (52 B/point)")
+        code = ops.encode_orders(g, b, depth, orders)
+        bits = 3 * depth + 2
+        passes = (bits + 7) // 8
+        us = _time_us(lambda: ops.argsort_rows(code, bits))
+        add("argsort+inverse", f"4 x {n} codes, {bits} significant bits, {passes} passes", "hbm",
+            4.0 * n * (passes * 24 + 16), us, f"B ({passes * 24 + 16} B per point and order)")
+    # ---- padding tables + slot tables
+    off_host = [int(v) for v in d["offset"]]
+    off = torch.from_numpy(d["offset"]).to(dev)
+    us = _time_us(lambda: ops.pad_index(off, off_host, 1024))
+    pad, unpad, cu = ops.pad_index(off, off_host, 1024)
+    add("pad_index", f"{n} points, patch 1024", "hbm", 8.0 * (len(pad) + n) + 4.0 * len(cu), us, "B")
+    # ---- config 2: patch attention alone, bf16, one 100k-point scene, C=512, H=32
+    sc = synthetic.room_scene(106_000, 2000, 0.02)
+    n2 = len(sc["grid_coord"])
+    g2 = torch.from_numpy(sc["grid_coord"]).to(dev)
+    b2 = torch.zeros(n2, dtype=torch.int64, device=dev)
+    code2 = ops.encode_orders(g2, b2, 9, ["hilbert"])
+    order2, inv2 = ops.argsort_rows(code2, 28)
+    off2 = torch.tensor([n2], device=dev)
+    pad2, unpad2, cu2 = ops.pad_index(off2, [n2], 1024)
+    src2, dst2 = ops.attn_slots(order2[0], inv2[0], pad2, unpad2)
+    gen = torch.Generator(device="cpu").manual_seed(2)
+    for dt, nm in ((torch.bfloat16, "bf16"), (torch.float16, "f16")):
+        qkv = (torch.randn(n2, 3 * 512, generator=gen) / 4).to(dt).to(dev)
+        us = _time_us(lambda: ops.patch_attention(qkv, 32, src2, dst2, cu2, 1024, 0.25), iters=10)
+        lens = torch.diff(cu2.long()).double()
+        fl = float(4.0 * (lens * lens).sum().item() * 512)
+        add(f"patch_attn<{nm}>", f"{n2} points (Hilbert order), patch 1024, C=512, 32 heads", "mfma", fl, us,
+            "FLOP (4 * sum len^2 * C)")
+    # ---- config 3: kmap + SubMConv3d 3x3x3 on 200k voxels, C=64, fp16
+    vox = synthetic.room_voxels(200_000, 3000)["grid_coord"]
+    idx = torch.from_numpy(np.concatenate([np.zeros((len(vox), 1), np.int32), vox], 1)).to(dev)
+    nv = len(vox)
+    us = _time_us(lambda: ops.kmap_build(idx, 3, tap_major=True))
+    add("kmap 3x3x3", f"{nv} voxels", "hbm", nv * 124.0, us, "B (124 B/voxel)")
+    nbr = ops.kmap_build(idx, 3, tap_major=True)
+    us = _time_us(lambda: ops.conv_plan(nbr, tap_major=True), iters=10)
+    plan = ops.conv_plan(nbr, tap_major=True)
+    add("conv_plan", f"{nv} voxels, {plan.n_pairs} active pairs", "hbm", nv * 27 * 4.0 * 2 + plan.n_pairs * 8.0 + nv * 4.0,
+        us, "B (map read twice, pair lists written)")
+    feat = torch.randn(nv, 64, generator=gen).half().to(dev)
+    w = ((torch.rand(64, 27, 64, generator=gen) * 2 - 1) / np.sqrt(27 * 64)).half().to(dev)
+    bias = torch.zeros(64).half().to(dev)
+    us = _time_us(lambda: ops.subm_conv_pairs(feat, plan, w, bias))
+    add("subm_conv pairs<f16>", f"{nv} voxels, {plan.n_pairs} pairs ({plan.n_pairs / nv:.2f}/voxel), 64->64", "mfma",
+        2.0 * plan.n_pairs * 64 * 64, us, "FLOP (2 * P_act * Cin * Cout)")
+    us = _time_us(lambda: ops.subm_conv(feat, nbr, w, bias, tap_major=True))
+    add("subm_conv dense<f16>", f"{nv} voxels, all 27 taps visited, 64->64", "mfma", 2.0 * plan.n_pairs * 64 * 64, us,
+        "FLOP (2 * P_act * Cin * Cout)")
+    # ---- pooling on the 4-scene batch
+    code = ops.encode_orders(g, b, 9, orders)
+    order, inverse = ops.argsort_rows(code, 29)
+    us = _time_us(lambda: ops.pool_clusters(code[0], order[0], 3), iters=10)
+    cluster, idx_ptr, head, m = ops.pool_clusters(code[0], order[0], 3)
+    add("pool_clusters", f"{n} points -> {m} clusters", "hbm", 24.0 * n + 16.0 * m, us, "B")
+    x = torch.randn(n, 64, generator=gen).half().to(dev)
+    us = _time_us(lambda: ops.segment_reduce(x, order[0], idx_ptr, "max"))
+    add("segment_reduce max<f16>", f"{n} x 64 -> {m} x 64", "hbm", (n * 64 + m * 64) * 2.0 + 8.0 * n, us, "B")
+    child = torch.randn(m, 64, generator=gen).half().to(dev)
+    us = _time_us(lambda: ops.unpool_add(x, child, cluster))
+    add("unpool_add<f16>", f"{n} x 64", "hbm", (2 * n * 64 + m * 64) * 2.0 + 8.0 * n, us, "B")
+    wln = torch.ones(64).half().to(dev)
+    us = _time_us(lambda: ops.layer_norm(x, wln, wln, 1e-5, residual=x, mode=2))
+    add("layer_norm mode 2<f16>", f"{n} x 64", "hbm", 4.0 * n * 64 * 2, us, "B (2 reads, 2 writes)")
+
+    os.makedirs(os.path.dirname(path) or ".", exist_ok=True)
+    with open(path, "w") as f:
+        json.dump(rows, f, indent=1)
+    for r in rows:
+        print(f"{r['kernel']:26s} {r['us']:9.1f} us  {r['achieved']:9.1f} {r['unit']:8s} {100 * r['frac']:5.1f}% of peak   {r['workload']}",
+              file=sys.stderr)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -83,6 +198,8 @@ def main():
     ap.add_argument("--scenes", type=int, default=4)
     ap.add_argument("--points", type=int, default=106_000, help="points drawn per scene before voxel dedup")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--kernels", metavar="PATH", default=None,
+                    help="also measure every kernel alone against its roofline and write the table to PATH")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (scenes would shard across "
@@ -144,6 +261,8 @@ def main():
                      "attn_ms_per_step": attn_ms / args.steps},
         "cpu_baseline": cpu,
     }
+    if args.kernels:
+        kernel_rooflines(args.kernels)
     print(json.dumps(result))
 
 

@@ -1,13 +1,24 @@
-// Submanifold sparse convolution forward as an output-stationary implicit GEMM over the
-// neighbour map.
+// Submanifold sparse convolution forward over the neighbour map, in two forms.
 //
 // Replaces spconv.SubMConv3d.forward at the reference call sites model.py:546-552 (xCPE,
 // 3x3x3, bias) and :767-774 (stem, 5x5x5, no bias).
 //
-// Half-precision path: one GEMM core (below) keeps a block of the output in MFMA accumulators,
-// stages weight tiles through double-buffered LDS and gathers neighbour rows straight into MFMA
-// operand registers. The product is taken transposed (rows = output channels, columns = voxels)
-// so a lane ends up holding 4 consecutive output channels of one voxel and stores 8 bytes.
+// Dense form (ptv3_subm_conv_fwd): output-stationary implicit GEMM. A work-group keeps a block
+// of the output in MFMA accumulators over all taps, so every output element is written once and
+// nothing is atomic; it pays MFMA work for every (voxel, tap) of the taps it visits. Best when a
+// good part of the taps is occupied (deep levels of a scan: 35-50 %).
+// Pair form (ptv3_subm_conv_pairs_fwd): rows of the GEMM are the ACTIVE (input, output) pairs,
+// grouped by tap, so every MFMA column is real work whatever the sparsity (a 2 cm surface scan
+// has 2-5 of 27 taps per voxel); one product row per pair goes to a scratch matrix and a segment
+// sum per voxel finishes. Costs a round trip of that matrix; best for sparse maps, thin channels.
+//
+// Both take the product transposed (rows = output channels, columns = voxels / pairs) with
+// v_mfma_f32_32x32x16: a lane's operand is then 8 consecutive input channels of one row, and its
+// results are 4 consecutive output channels of one row. Global traffic moves in whole row
+// segments (several lanes x 16 B per row) and a small wave-private LDS buffer converts between
+// that shape and the one-row-per-lane operand layout: touching 8-16 lines per memory instruction
+// instead of 32 is what keeps the address path from bounding the kernels.
+// fp32: one thread per output element, plain FMA (parity path, not tuned).
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 
@@ -50,25 +61,28 @@ template <> struct HalfOps<__bf16> {
 
 constexpr int CONV_THREADS = 256;
 constexpr int CONV_WAVES = CONV_THREADS / PTV3_WAVE;
-constexpr int W_PAD = 8;         // halfs of padding per LDS weight row
+constexpr int W_PAD = 8;           // halfs of padding per LDS weight row
+constexpr int XS_STRIDE = 72;      // halfs per staged row (64 + 8 of padding against bank conflicts)
 
-// Shared GEMM core. A work-group owns ROWS = 4 waves * MT * 32 rows and COUT_TILE = NT * 32
-// output channels; accumulators stay in registers. One "step" is (tap, 64-channel slice):
-// the W[couts, tap, slice] tile sits in LDS (double-buffered: the next tile is fetched into
-// registers while this one is multiplied), the rows' input features are gathered straight
-// into MFMA operand registers (8 consecutive channels of one row = one 16-byte load).
+// The staging buffer is private to a wave and LDS operations of one wave execute in program
+// order, so a write followed by a read of the same bytes needs no wait: only the compiler has
+// to be kept from reordering the two.
+__device__ __forceinline__ void lds_fence() { asm volatile("" ::: "memory"); }
+
+// Dense output-stationary form. A work-group owns ROWS = 4 waves * MT * 32 voxels and
+// COUT_TILE = NT * 32 output channels. One step is (tap, KC-channel slice): the
+// W[couts, tap, slice] tile sits in LDS, double-buffered (the next tile is fetched into registers
+// while this one is multiplied; one barrier per step); the neighbour rows of the step after are in
+// flight as well, and the neighbour indices of the tap after next. Taps no voxel of the
+// work-group has are skipped altogether; a wave skips the taps none of its voxels has.
 //
-// PAIRS == false: dense output-stationary mode. Row r is voxel row0 + r; for tap t its
-//   input row is nbr[voxel][t] (or nothing); all taps accumulate into the same registers and
-//   the voxel's output row is written once, with bias.
-// PAIRS == true: a work-group processes up to ROWS consecutive entries of a tap-major list of
-//   active (input row, output slot) pairs, all of ONE tap (tiles never straddle taps; the tap
-//   is found from tap_ptr), and writes one product row per pair to y[slot]; a segment sum over
-//   each voxel's slots finishes the convolution. Every MFMA column is a real pair, so the
-//   matrix work is proportional to the active pairs, not to taps * voxels.
-// KC: input channels per step (one LDS weight tile).
+// PAIRS == true turns the same kernel into a tile of the pair form: the work-group takes ROWS
+// consecutive entries of ONE tap of the tap-major pair list (found from tap_ptr), its rows are
+// pair_in[...], there is a single tap to visit, and product rows go to out[pair_slot[...]]
+// without bias. Used where the weight-stationary pair kernel would need most of the LDS for the
+// weights of one tap (256 and more input channels).
 template <typename T, int MT, int NT, int KC, bool PAIRS>
-__global__ __launch_bounds__(CONV_THREADS, 2) void subm_conv_gemm_kernel(
+__global__ __launch_bounds__(CONV_THREADS, 2) void subm_conv_dense_kernel(
     const T* __restrict__ feat, int64_t n, int cin, const int32_t* __restrict__ nbr, int taps,
     bool tap_major, const T* __restrict__ weight, const T* __restrict__ bias, int cout,
     T* __restrict__ out, const int32_t* __restrict__ pair_in, const int32_t* __restrict__ pair_slot,
@@ -78,63 +92,94 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void subm_conv_gemm_kernel(
     constexpr int COUT_TILE = NT * 32;
     constexpr int W_PIECES = COUT_TILE * (KC / 8);                 // 16-byte pieces per weight tile
     constexpr int W_LOADS = (W_PIECES + CONV_THREADS - 1) / CONV_THREADS;
+    constexpr int LPR = KC / 8;           // lanes per staged row segment
+    constexpr int RPI = 64 / LPR;         // rows per gather instruction
+    constexpr int ITS = 32 / RPI;         // gather instructions per 32-row group
     __shared__ __align__(16) T w_lds[2][COUT_TILE][KC + W_PAD];
-    __shared__ uint32_t wg_mask;
+    __shared__ __align__(16) T xs_all[CONV_WAVES][32 * XS_STRIDE];
+    __shared__ uint32_t wg_mask[4];
 
     const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
     const int col = lane & 31, hf = lane >> 5;
+    const int srow = lane / LPR, spc = lane % LPR;
+    T* xs = xs_all[wave];
     const int cout0 = blockIdx.y * COUT_TILE;
+    // dense: first voxel of the wave. pairs: first row of the wave inside the tile
+    const int64_t vox0 = (PAIRS ? 0 : (int64_t)blockIdx.x * ROWS) + wave * (MT * 32);
     // neighbour map entry (voxel i, tap t): voxel-major (n,taps) or tap-major (taps,n)
     auto nbr_at = [&](int64_t i, int t) { return tap_major ? nbr[(int64_t)t * n + i] : nbr[i * taps + t]; };
 
-    // ---- rows of this wave
-    int64_t row[MT];      // dense: voxel id; pairs: index into the pair list (or -1)
-    int32_t pin[MT];      // pairs: input row
-    int only_tap = 0;
-    uint32_t my_mask = 0;
+    int only_tap = -1, pstart = 0, pcount = 0;
+    uint32_t mask[4] = {0, 0, 0, 0};
     if (PAIRS) {
-        // which tap does tile blockIdx.x belong to? tiles never straddle taps
-        int tile = blockIdx.x, start = 0, count = 0;
-        only_tap = -1;
-        for (int tt = 0; tt < taps; ++tt) {
-            const int first = tap_ptr[tt], cnt = tap_ptr[tt + 1] - first;
-            const int tiles_here = (cnt + ROWS - 1) / ROWS;
-            if (tile < tiles_here) {
-                only_tap = tt;
-                start = first + tile * ROWS;
-                count = min(ROWS, cnt - tile * ROWS);
-                break;
+        // which tap does tile blockIdx.x belong to? lane l looks at taps l and l+64 (taps <= 128)
+        const int rid = blockIdx.x;
+        int first[2], cnt[2], nr[2], incl[2];
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const int tt = lane + 64 * k;
+            first[k] = tt < taps ? tap_ptr[tt] : 0;
+            cnt[k] = tt < taps ? tap_ptr[tt + 1] - first[k] : 0;
+            nr[k] = (cnt[k] + ROWS - 1) / ROWS;
+        }
+        int carry = 0;
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            int xsum = nr[k];
+#pragma unroll
+            for (int off = 1; off < PTV3_WAVE; off <<= 1) {
+                const int v = __shfl_up(xsum, off, PTV3_WAVE);
+                if (lane >= off) xsum += v;
             }
-            tile -= tiles_here;
+            incl[k] = xsum + carry;
+            carry += __shfl(xsum, PTV3_WAVE - 1, PTV3_WAVE);
         }
-        if (only_tap < 0) return;   // grid is an upper bound on the number of tiles
 #pragma unroll
-        for (int a = 0; a < MT; ++a) {
-            const int r = wave * (MT * 32) + a * 32 + col;
-            row[a] = r < count ? (int64_t)start + r : -1;
-            pin[a] = row[a] >= 0 ? pair_in[row[a]] : -1;
+        for (int k = 0; k < 2; ++k) {
+            const uint64_t hit = __ballot(nr[k] > 0 && rid < incl[k] && rid >= incl[k] - nr[k]);
+            if (hit && only_tap < 0) {
+                const int l = __ffsll((unsigned long long)hit) - 1;
+                const int rel = rid - (__shfl(incl[k], l, PTV3_WAVE) - __shfl(nr[k], l, PTV3_WAVE));
+                only_tap = 64 * k + l;
+                pstart = __shfl(first[k], l, PTV3_WAVE) + rel * ROWS;
+                pcount = min(ROWS, __shfl(cnt[k], l, PTV3_WAVE) - rel * ROWS);
+            }
         }
+        if (only_tap < 0) return;   // the grid is an upper bound on the number of tiles
     } else {
-        const int64_t row0 = (int64_t)blockIdx.x * ROWS + wave * (MT * 32);
-#pragma unroll
-        for (int a = 0; a < MT; ++a) {
-            row[a] = row0 + a * 32 + col;
-            pin[a] = -1;
-        }
-        // taps any voxel of the work-group has: the others are skipped altogether
-        if (tid == 0) wg_mask = 0;
+        // taps any voxel of the work-group has (bit t of a 128-bit mask)
+        if (tid < 4) wg_mask[tid] = 0;
         __syncthreads();
-        for (int t = 0; t < taps && taps <= 32; ++t) {
+        for (int t = 0; t < taps; ++t) {
             bool any = false;
 #pragma unroll
-            for (int a = 0; a < MT; ++a) any |= row[a] < n && nbr_at(row[a], t) >= 0;
-            if (__ballot(any) != 0) my_mask |= 1u << (t & 31);
+            for (int a = 0; a < MT; ++a) {
+                const int64_t v = vox0 + a * 32 + col;
+                any |= hf == 0 && v < n && nbr_at(v, t) >= 0;
+            }
+            if (__ballot(any) != 0 && lane == 0) atomicOr(&wg_mask[t >> 5], 1u << (t & 31));
         }
-        // 27 taps fit one word; for 125 taps (stem) the mask is not used: all taps are visited
-        if (taps <= 32 && lane == 0) atomicOr(&wg_mask, my_mask);
         __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 4; ++k) mask[k] = wg_mask[k];
     }
-    const uint32_t tap_mask = (PAIRS || taps > 32) ? 0xffffffffu : wg_mask;
+    // input rows of tap t in staging shape: lane (srow, spc) serves rows srow + RPI*it of each group
+    auto load_src = [&](int t, int32_t (&src)[MT][ITS]) {
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int it = 0; it < ITS; ++it) {
+                const int64_t v = vox0 + a * 32 + it * RPI + srow;
+                if (PAIRS) src[a][it] = (t == only_tap && v < pcount) ? pair_in[pstart + v] : -1;
+                else src[a][it] = (t < taps && v < n) ? nbr_at(v, t) : -1;
+            }
+    };
+    auto next_tap = [&](int t) {
+        if (PAIRS) return t < 0 ? only_tap : taps;
+        ++t;
+        while (t < taps && !((mask[t >> 5] >> (t & 31)) & 1u)) ++t;
+        return t;
+    };
 
     f32x16 acc[MT][NT];
 #pragma unroll
@@ -145,21 +190,6 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void subm_conv_gemm_kernel(
             for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
     const int chunks = (cin + KC - 1) / KC;
-    // next active tap after t (pairs mode has exactly one)
-    auto next_tap = [&](int t) {
-        if (PAIRS) return t < 0 ? only_tap : taps;
-        ++t;
-        while (t < taps && taps <= 32 && !((tap_mask >> t) & 1u)) ++t;
-        return t;
-    };
-    auto load_src = [&](int t, int32_t (&src)[MT]) {
-#pragma unroll
-        for (int a = 0; a < MT; ++a) {
-            if (PAIRS) src[a] = pin[a];
-            else src[a] = (t < taps && row[a] < n) ? nbr_at(row[a], t) : -1;
-        }
-    };
-    // global -> register fetch of one weight tile / of the rows' input slices
     auto fetch_w = [&](int t, int c0, u32x4 (&wreg)[W_LOADS]) {
 #pragma unroll
         for (int i = 0; i < W_LOADS; ++i) {
@@ -179,30 +209,36 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void subm_conv_gemm_kernel(
             if (e < W_PIECES) *(u32x4*)&w_lds[buf][co][pc * 8] = wreg[i];
         }
     };
-    auto gather_x = [&](const int32_t (&src)[MT], int c0, u32x4 (&x)[KC / 16][MT]) {
+    auto gather_raw = [&](const int32_t (&src)[MT][ITS], int c0, u32x4 (&raw)[MT][ITS]) {
 #pragma unroll
-        for (int ks = 0; ks < KC / 16; ++ks)
+        for (int a = 0; a < MT; ++a)
 #pragma unroll
-            for (int a = 0; a < MT; ++a) {
-                x[ks][a] = (u32x4){0, 0, 0, 0};
-                if (c0 + ks * 16 < cin && src[a] >= 0)
-                    x[ks][a] = *(const u32x4*)(feat + (int64_t)src[a] * cin + c0 + ks * 16 + hf * 8);
+            for (int it = 0; it < ITS; ++it) {
+                raw[a][it] = (u32x4){0, 0, 0, 0};
+                if (c0 + spc * 8 < cin && src[a][it] >= 0)
+                    raw[a][it] = *(const u32x4*)(feat + (int64_t)src[a][it] * cin + c0 + spc * 8);
             }
     };
+    auto wave_has = [&](const int32_t (&src)[MT][ITS]) {
+        bool any = false;
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int it = 0; it < ITS; ++it) any |= src[a][it] >= 0;
+        return __ballot(any) != 0;
+    };
 
-    // Pipeline: while the MFMAs of step s run, the weight tile and the gathered rows of step
-    // s+1 are in flight, and the neighbour indices of the tap after next are being fetched.
     int t = next_tap(-1);
     int tn = t < taps ? next_tap(t) : taps;
     int chunk = 0, buf = 0;
-    int32_t src_t[MT], src_tn[MT];
+    int32_t src_t[MT][ITS], src_tn[MT][ITS];
     u32x4 wreg[W_LOADS];
-    u32x4 x_cur[KC / 16][MT], x_nxt[KC / 16][MT];
+    u32x4 raw[MT][ITS];
     load_src(t, src_t);
     load_src(tn, src_tn);
     if (t < taps) {
         fetch_w(t, 0, wreg);
-        gather_x(src_t, 0, x_cur);
+        gather_raw(src_t, 0, raw);
         store_w(0, wreg);
     }
     __syncthreads();
@@ -211,23 +247,33 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void subm_conv_gemm_kernel(
         const int t2 = tap_ends ? tn : t;
         const int chunk2 = tap_ends ? 0 : chunk + 1;
         const bool has_next = t2 < taps;
-        int tnn = tn;
-        int32_t src_tnn[MT];
+        const bool active = wave_has(src_t);
+        // this step's rows: staging shape -> one row per lane
+        u32x4 x[KC / 16][MT];
+        if (active) {
 #pragma unroll
-        for (int a = 0; a < MT; ++a) src_tnn[a] = -1;
-        if (has_next) {
-            fetch_w(t2, chunk2 * KC, wreg);
-            if (tap_ends) gather_x(src_tn, 0, x_nxt);
-            else gather_x(src_t, chunk2 * KC, x_nxt);
-            if (tap_ends) {
-                tnn = next_tap(tn);
-                load_src(tnn, src_tnn);
+            for (int a = 0; a < MT; ++a) {
+#pragma unroll
+                for (int it = 0; it < ITS; ++it) *(u32x4*)(xs + (it * RPI + srow) * XS_STRIDE + spc * 8) = raw[a][it];
+                lds_fence();
+#pragma unroll
+                for (int ks = 0; ks < KC / 16; ++ks) x[ks][a] = *(const u32x4*)(xs + col * XS_STRIDE + ks * 16 + hf * 8);
+                lds_fence();
             }
         }
-        bool wave_any = false;
-#pragma unroll
-        for (int a = 0; a < MT; ++a) wave_any |= (__ballot(src_t[a] >= 0) != 0);
-        if (wave_any) {
+        // the step after this one: weights, rows, and (at a tap boundary) indices two taps ahead
+        int tnn = tn;
+        int32_t src_tnn[MT][ITS];
+        if (has_next) {
+            fetch_w(t2, chunk2 * KC, wreg);
+            if (tap_ends) gather_raw(src_tn, 0, raw);
+            else gather_raw(src_t, chunk2 * KC, raw);
+        }
+        if (tap_ends) {
+            tnn = has_next ? next_tap(tn) : taps;
+            load_src(tnn, src_tnn);
+        }
+        if (active) {
 #pragma unroll
             for (int ks = 0; ks < KC / 16; ++ks) {
                 if (chunk * KC + ks * 16 < cin) {
@@ -236,7 +282,7 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void subm_conv_gemm_kernel(
                         const v8 wfrag = __builtin_bit_cast(v8, *(const u32x4*)&w_lds[buf][b * 32 + col][ks * 16 + hf * 8]);
 #pragma unroll
                         for (int a = 0; a < MT; ++a)
-                            acc[a][b] = HalfOps<T>::mfma(wfrag, __builtin_bit_cast(v8, x_cur[ks][a]), acc[a][b]);
+                            acc[a][b] = HalfOps<T>::mfma(wfrag, __builtin_bit_cast(v8, x[ks][a]), acc[a][b]);
                     }
                 }
             }
@@ -244,102 +290,257 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void subm_conv_gemm_kernel(
         if (has_next) store_w(buf ^ 1, wreg);
         __syncthreads();
         buf ^= 1;
-#pragma unroll
-        for (int ks = 0; ks < KC / 16; ++ks)
-#pragma unroll
-            for (int a = 0; a < MT; ++a) x_cur[ks][a] = x_nxt[ks][a];
         if (tap_ends) {
 #pragma unroll
-            for (int a = 0; a < MT; ++a) { src_t[a] = src_tn[a]; src_tn[a] = src_tnn[a]; }
+            for (int a = 0; a < MT; ++a)
+#pragma unroll
+                for (int it = 0; it < ITS; ++it) { src_t[a][it] = src_tn[a][it]; src_tn[a][it] = src_tnn[a][it]; }
             t = tn;
             tn = tnn;
         }
         chunk = chunk2;
     }
 
-    // acc[a][b][v]: output channel cout0 + b*32 + 8*(v/4) + 4*hf + v%4 of row[a]
+    // acc[a][b][v]: output channel cout0 + b*32 + 8*(v/4) + 4*hf + v%4 of voxel vox0 + a*32 + col.
+    // Add the bias, go back to row-segment shape 64 channels at a time, store 16 bytes per lane.
 #pragma unroll
     for (int a = 0; a < MT; ++a) {
-        int64_t orow;
-        if (PAIRS) {
-            if (row[a] < 0) continue;
-            orow = pair_slot[row[a]];
-        } else {
-            if (row[a] >= n) continue;
-            orow = row[a];
+#pragma unroll
+        for (int b0 = 0; b0 < NT; b0 += 2) {
+#pragma unroll
+            for (int bb = 0; bb < 2 && b0 + bb < NT; ++bb)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int b = b0 + bb;
+                    const int co = cout0 + b * 32 + 8 * g + 4 * hf;
+                    float r[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        r[q] = acc[a][b][4 * g + q] +
+                               ((!PAIRS && bias && co + q < cout) ? HalfOps<T>::to_float(bias[co + q]) : 0.f);
+                    u32x2 pk = {HalfOps<T>::pack2(r[0], r[1]), HalfOps<T>::pack2(r[2], r[3])};
+                    *(u32x2*)(xs + col * XS_STRIDE + bb * 32 + 8 * g + 4 * hf) = pk;
+                }
+            lds_fence();
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const int orow = it * 8 + (lane >> 3), opc = lane & 7;
+                const int co = cout0 + b0 * 32 + opc * 8;
+                const int64_t v = vox0 + a * 32 + orow;
+                const u32x4 val = *(const u32x4*)(xs + orow * XS_STRIDE + opc * 8);
+                int64_t dst = -1;
+                if (PAIRS) { if (v < pcount) dst = pair_slot[pstart + v]; }
+                else if (v < n) dst = v;
+                if (dst >= 0 && co < cout && (NT - b0 >= 2 || opc < 4)) *(u32x4*)(out + dst * cout + co) = val;
+            }
+            lds_fence();
+        }
+    }
+}
+
+// Pair mode, weight-stationary. A work-group takes one tap and a range of up to `range_rows`
+// of that tap's pairs (tap-major list), keeps W[couts, tap, all input channels] in LDS for its
+// whole life and streams the range through it in tiles of ROWS pairs. Steps (tile, 64-channel
+// slice) are software-pipelined: the input rows of step s+1 and the pair indices of the tile after
+// next are in flight while the MFMAs of step s run; there is no block barrier after the weights
+// are staged.
+// Global traffic moves in whole 128-byte row segments: a gather instruction fetches 8 rows x 128 B
+// (8 lanes x 16 B per row) and a result store writes 8 rows x 128 B; a small wave-private LDS
+// buffer converts between that shape and the MFMA register layout (one row per lane). Touching 8
+// lines per instruction instead of 32 is what keeps the address path from bounding the kernel.
+// PKC: input channels per step (64, or 32 where the 128-register accumulator leaves no room for
+// a 64-channel prefetch). A staged row segment is PKC*2 bytes = LPR lanes x 16 B.
+template <typename T, int MT, int NT, int PKC>
+__global__ __launch_bounds__(CONV_THREADS, 2) void subm_conv_pairs_kernel(
+    const T* __restrict__ feat, int cin, int taps, const T* __restrict__ weight, int cout,
+    T* __restrict__ y, const int32_t* __restrict__ pair_in, const int32_t* __restrict__ pair_slot,
+    const int32_t* __restrict__ tap_ptr, int range_rows) {
+    typedef typename HalfOps<T>::v8 v8;
+    constexpr int ROWS = CONV_WAVES * MT * 32;
+    constexpr int COUT_TILE = NT * 32;
+    extern __shared__ __align__(16) unsigned char conv_smem[];
+    const int w_stride = cin + W_PAD;
+    T* w_lds = (T*)conv_smem;                                   // [COUT_TILE][cin + W_PAD]
+    const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
+    T* xs = w_lds + (size_t)COUT_TILE * w_stride + (size_t)wave * (32 * XS_STRIDE);   // wave-private [32][72]
+    const int col = lane & 31, hf = lane >> 5;
+    constexpr int LPR = PKC / 8;          // lanes per staged row segment
+    constexpr int RPI = 64 / LPR;         // rows per load/store instruction
+    constexpr int ITS = 32 / RPI;         // instructions per 32-row group
+    const int srow = lane / LPR, spc = lane % LPR;
+    const int cout0 = blockIdx.y * COUT_TILE;
+
+    // ---- which (tap, range) is blockIdx.x? ranges never straddle taps. Lane l looks at taps l
+    // and l+64 (taps <= 128): one round of loads, then a wave prefix sum of range counts.
+    int tap = -1, start = 0, count = 0;
+    {
+        const int rid = blockIdx.x;
+        int first[2], cnt[2], nr[2], incl[2];
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const int tt = lane + 64 * k;
+            first[k] = tt < taps ? tap_ptr[tt] : 0;
+            cnt[k] = tt < taps ? tap_ptr[tt + 1] - first[k] : 0;
+            nr[k] = (cnt[k] + range_rows - 1) / range_rows;
+        }
+        int carry = 0;
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            int x = nr[k];
+#pragma unroll
+            for (int off = 1; off < PTV3_WAVE; off <<= 1) {
+                const int v = __shfl_up(x, off, PTV3_WAVE);
+                if (lane >= off) x += v;
+            }
+            incl[k] = x + carry;
+            carry += __shfl(x, PTV3_WAVE - 1, PTV3_WAVE);
         }
 #pragma unroll
-        for (int b = 0; b < NT; ++b) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int co = cout0 + b * 32 + 8 * g + 4 * hf;
-                if (co >= cout) continue;
-                float r[4];
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    r[q] = acc[a][b][4 * g + q] + ((!PAIRS && bias) ? HalfOps<T>::to_float(bias[co + q]) : 0.f);
-                u32x2 pk = {HalfOps<T>::pack2(r[0], r[1]), HalfOps<T>::pack2(r[2], r[3])};
-                *(u32x2*)(out + orow * cout + co) = pk;
+        for (int k = 0; k < 2; ++k) {
+            const uint64_t hit = __ballot(nr[k] > 0 && rid < incl[k] && rid >= incl[k] - nr[k]);
+            if (hit && tap < 0) {
+                const int l = __ffsll((unsigned long long)hit) - 1;
+                const int rel = rid - (__shfl(incl[k], l, PTV3_WAVE) - __shfl(nr[k], l, PTV3_WAVE));
+                tap = 64 * k + l;
+                start = __shfl(first[k], l, PTV3_WAVE) + rel * range_rows;
+                count = min(range_rows, __shfl(cnt[k], l, PTV3_WAVE) - rel * range_rows);
             }
         }
     }
-}
+    if (tap < 0) return;   // the grid is an upper bound on the number of ranges
 
-// fp32: one thread per (voxel, output channel); a wave shares the voxel when cout >= 64.
-__global__ __launch_bounds__(256) void subm_conv_f32_kernel(
-    const float* __restrict__ feat, int64_t n, int cin, const int32_t* __restrict__ nbr, int taps,
-    bool tap_major, const float* __restrict__ weight, const float* __restrict__ bias, int cout,
-    float* __restrict__ out) {
-    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= n * cout) return;
-    const int64_t i = e / cout;
-    const int co = (int)(e - i * cout);
-    float acc = bias ? bias[co] : 0.f;
-    for (int t = 0; t < taps; ++t) {
-        const int32_t src = tap_major ? nbr[(int64_t)t * n + i] : nbr[i * taps + t];
-        if (src < 0) continue;
-        const float* x = feat + (int64_t)src * cin;
-        const float* w = weight + ((int64_t)co * taps + t) * cin;
-        float part = 0.f;
-        for (int c = 0; c < cin; ++c) part = fmaf(x[c], w[c], part);
-        acc += part;
+    // ---- stage W[cout0.., tap, :] once
+    {
+        const int pieces_per_row = cin / 8;
+        for (int e = tid; e < COUT_TILE * pieces_per_row; e += CONV_THREADS) {
+            const int co = e / pieces_per_row, pc = e % pieces_per_row;
+            u32x4 w = {0, 0, 0, 0};
+            if (cout0 + co < cout)
+                w = *(const u32x4*)(weight + ((int64_t)(cout0 + co) * taps + tap) * cin + pc * 8);
+            *(u32x4*)(w_lds + co * w_stride + pc * 8) = w;
+        }
     }
-    out[e] = acc;
-}
 
-template <typename T, int MT, int NT, int KC>
-void launch_dense_kc(const void* feat, int64_t n, int cin, const int32_t* nbr, int taps, bool tap_major,
-                  const void* weight, const void* bias, int cout, void* out, hipStream_t stream) {
-    constexpr int ROWS = CONV_WAVES * MT * 32, COUT_TILE = NT * 32;
-    dim3 grid((unsigned)ptv3_ceil_div(n, ROWS), (unsigned)ptv3_ceil_div(cout, COUT_TILE));
-    hipLaunchKernelGGL((subm_conv_gemm_kernel<T, MT, NT, KC, false>), grid, dim3(CONV_THREADS), 0, stream,
-                       (const T*)feat, n, cin, nbr, taps, tap_major, (const T*)weight, (const T*)bias, cout, (T*)out,
-                       (const int32_t*)nullptr, (const int32_t*)nullptr, (const int32_t*)nullptr);
-}
+    const int n_tiles = (count + ROWS - 1) / ROWS;
+    const int chunks = (cin + PKC - 1) / PKC;
+    const int wave_row0 = wave * (MT * 32);
+    // pair indices in staging shape: lane (srow, spc) serves rows srow + 8*it of every 32-row group
+    auto load_idx = [&](const int32_t* __restrict__ table, int tile, int32_t (&idx)[MT][ITS]) {
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int it = 0; it < ITS; ++it) {
+                const int r = tile * ROWS + wave_row0 + a * 32 + it * RPI + srow;
+                idx[a][it] = (tile < n_tiles && r < count) ? table[start + r] : -1;
+            }
+    };
+    // 64-channel slice of 32 rows per group: 4 instructions of 8 rows x 128 B
+    auto gather_raw = [&](const int32_t (&pin)[MT][ITS], int c0, u32x4 (&raw)[MT][ITS]) {
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int it = 0; it < ITS; ++it) {
+                raw[a][it] = (u32x4){0, 0, 0, 0};
+                if (c0 + spc * 8 < cin && pin[a][it] >= 0)
+                    raw[a][it] = *(const u32x4*)(feat + (int64_t)pin[a][it] * cin + c0 + spc * 8);
+            }
+    };
 
-template <typename T, int MT, int NT>
-void launch_dense(const void* feat, int64_t n, int cin, const int32_t* nbr, int taps, bool tap_major,
-                  const void* weight, const void* bias, int cout, void* out, hipStream_t stream) {
-    // wide channel slices cut the number of barriers; thin inputs would only pad them with zeros
-    if (cin >= 64) launch_dense_kc<T, MT, NT, 64>(feat, n, cin, nbr, taps, tap_major, weight, bias, cout, out, stream);
-    else launch_dense_kc<T, MT, NT, 32>(feat, n, cin, nbr, taps, tap_major, weight, bias, cout, out, stream);
-}
+    int32_t pin_c[MT][ITS], pin_n[MT][ITS];
+    u32x4 raw[MT][ITS];
+    load_idx(pair_in, 0, pin_c);
+    load_idx(pair_in, 1, pin_n);
+    gather_raw(pin_c, 0, raw);
+    __syncthreads();   // weights staged
 
-template <typename T>
-void dispatch_dense(const void* feat, int64_t n, int cin, const int32_t* nbr, int taps, bool tap_major,
-                    const void* weight, const void* bias, int cout, void* out, hipStream_t stream) {
-    // Rows per work-group: 256 while that still yields >= ~2 work-groups per CU, else 128.
-    const int64_t col_tiles = cout <= 32 ? 1 : (cout <= 64 ? 1 : ptv3_ceil_div(cout, 128));
-    const bool wide = ptv3_ceil_div(n, 256) * col_tiles >= 512;
-    if (cout <= 32) {
-        if (wide) launch_dense<T, 2, 1>(feat, n, cin, nbr, taps, tap_major, weight, bias, cout, out, stream);
-        else launch_dense<T, 1, 1>(feat, n, cin, nbr, taps, tap_major, weight, bias, cout, out, stream);
-    } else if (cout <= 64) {
-        if (wide) launch_dense<T, 2, 2>(feat, n, cin, nbr, taps, tap_major, weight, bias, cout, out, stream);
-        else launch_dense<T, 1, 2>(feat, n, cin, nbr, taps, tap_major, weight, bias, cout, out, stream);
-    } else {
-        if (wide) launch_dense<T, 2, 4>(feat, n, cin, nbr, taps, tap_major, weight, bias, cout, out, stream);
-        else launch_dense<T, 1, 4>(feat, n, cin, nbr, taps, tap_major, weight, bias, cout, out, stream);
+    f32x16 acc[MT][NT];
+    for (int tile = 0; tile < n_tiles; ++tile) {
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int b = 0; b < NT; ++b)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
+        // Narrow outputs (cin <= 64 in practice: one step per tile) fetch the input rows two tiles
+        // ahead so that index load and gather never sit in the same step; wide ones have several
+        // steps per tile to hide the index load and cannot spare the registers.
+        constexpr bool DEEP = NT <= 2;
+        int32_t pin_nn[MT][ITS], slot_c[MT][ITS];
+        if (DEEP) load_idx(pair_in, tile + 2, pin_nn);
+        for (int chunk = 0; chunk < chunks; ++chunk) {
+            if (!DEEP && chunk == 0) load_idx(pair_in, tile + 1, pin_n);
+            // output slots of this tile: needed after the last step's MFMAs
+            if (chunk == chunks - 1) load_idx(pair_slot, tile, slot_c);
+            // rows of this step: staging shape -> one row per lane, through the wave's LDS buffer
+            u32x4 x[PKC / 16][MT];
+#pragma unroll
+            for (int a = 0; a < MT; ++a) {
+#pragma unroll
+                for (int it = 0; it < ITS; ++it) *(u32x4*)(xs + (it * RPI + srow) * XS_STRIDE + spc * 8) = raw[a][it];
+                lds_fence();
+#pragma unroll
+                for (int ks = 0; ks < PKC / 16; ++ks) x[ks][a] = *(const u32x4*)(xs + col * XS_STRIDE + ks * 16 + hf * 8);
+                lds_fence();
+            }
+            // next step's rows
+            if (chunk + 1 < chunks) gather_raw(pin_c, (chunk + 1) * PKC, raw);
+            else gather_raw(pin_n, 0, raw);   // first slice of the next tile (nothing past the end)
+            const int c0 = chunk * PKC;
+#pragma unroll
+            for (int ks = 0; ks < PKC / 16; ++ks) {
+                if (c0 + ks * 16 < cin) {
+#pragma unroll
+                    for (int b = 0; b < NT; ++b) {
+                        const v8 wfrag = __builtin_bit_cast(
+                            v8, *(const u32x4*)(w_lds + (b * 32 + col) * w_stride + c0 + ks * 16 + hf * 8));
+#pragma unroll
+                        for (int a = 0; a < MT; ++a)
+                            acc[a][b] = HalfOps<T>::mfma(wfrag, __builtin_bit_cast(v8, x[ks][a]), acc[a][b]);
+                    }
+                }
+                // keep the scheduler from hoisting every weight fragment of the step up front
+                // (that costs 16 registers per 16-channel sub-step)
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // acc[a][b][v]: output channel cout0 + b*32 + 8*(v/4) + 4*hf + v%4 of the lane's row.
+        // Back to staging shape, 64 channels (two 32-channel tiles) at a time, then 16-byte stores.
+#pragma unroll
+        for (int a = 0; a < MT; ++a) {
+#pragma unroll
+            for (int b0 = 0; b0 < NT; b0 += 2) {
+#pragma unroll
+                for (int bb = 0; bb < 2 && b0 + bb < NT; ++bb)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int b = b0 + bb;
+                        u32x2 pk = {HalfOps<T>::pack2(acc[a][b][4 * g], acc[a][b][4 * g + 1]),
+                                    HalfOps<T>::pack2(acc[a][b][4 * g + 2], acc[a][b][4 * g + 3])};
+                        *(u32x2*)(xs + col * XS_STRIDE + bb * 32 + 8 * g + 4 * hf) = pk;
+                    }
+                lds_fence();
+                // 64 output channels of 32 rows = 8 lanes x 16 B per row, 8 rows per store
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    const int orow = it * 8 + (lane >> 3), opc = lane & 7;
+                    const int co = cout0 + b0 * 32 + opc * 8;
+                    const u32x4 v = *(const u32x4*)(xs + orow * XS_STRIDE + opc * 8);
+                    // the slot of row `orow` sits in the lane that staged it: group (it*8)/RPI, lane
+                    // (row within the group) * LPR
+                    const int32_t slot = __shfl(slot_c[a][(it * 8) / RPI], (((it * 8) % RPI) + (lane >> 3)) * LPR, PTV3_WAVE);
+                    if (slot >= 0 && co < cout && (NT - b0 >= 2 || opc < 4))
+                        *(u32x4*)(y + (int64_t)slot * cout + co) = v;
+                }
+                lds_fence();
+            }
+        }
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int it = 0; it < ITS; ++it) {
+                pin_c[a][it] = pin_n[a][it];
+                if (DEEP) pin_n[a][it] = pin_nn[a][it];
+            }
     }
 }
 
@@ -371,38 +572,102 @@ __global__ __launch_bounds__(256) void pair_segment_sum_kernel(const T* __restri
     *(u32x4*)(out + i * cout + c) = r;
 }
 
-template <typename T, int MT, int NT, int KC>
-void launch_pairs_kc(const void* feat, int cin, int taps, int64_t n_pairs, const int32_t* tap_ptr,
-                     const int32_t* pair_in, const int32_t* pair_slot, const void* weight, int cout,
-                     void* y, hipStream_t stream) {
-    constexpr int ROWS = CONV_WAVES * MT * 32, COUT_TILE = NT * 32;
-    // every tap may end with one partial tile
-    dim3 grid((unsigned)(n_pairs / ROWS + taps), (unsigned)ptv3_ceil_div(cout, COUT_TILE));
-    hipLaunchKernelGGL((subm_conv_gemm_kernel<T, MT, NT, KC, true>), grid, dim3(CONV_THREADS), 0, stream,
-                       (const T*)feat, (int64_t)0, cin, (const int32_t*)nullptr, taps, false, (const T*)weight,
-                       (const T*)nullptr, cout, (T*)y, pair_in, pair_slot, tap_ptr);
+// fp32: one thread per (voxel, output channel); a wave shares the voxel when cout >= 64.
+__global__ __launch_bounds__(256) void subm_conv_f32_kernel(
+    const float* __restrict__ feat, int64_t n, int cin, const int32_t* __restrict__ nbr, int taps,
+    bool tap_major, const float* __restrict__ weight, const float* __restrict__ bias, int cout,
+    float* __restrict__ out) {
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n * cout) return;
+    const int64_t i = e / cout;
+    const int co = (int)(e - i * cout);
+    float acc = bias ? bias[co] : 0.f;
+    for (int t = 0; t < taps; ++t) {
+        const int32_t src = tap_major ? nbr[(int64_t)t * n + i] : nbr[i * taps + t];
+        if (src < 0) continue;
+        const float* x = feat + (int64_t)src * cin;
+        const float* w = weight + ((int64_t)co * taps + t) * cin;
+        float part = 0.f;
+        for (int c = 0; c < cin; ++c) part = fmaf(x[c], w[c], part);
+        acc += part;
+    }
+    out[e] = acc;
 }
 
 template <typename T, int MT, int NT>
-void launch_pairs(const void* feat, int cin, int taps, int64_t n_pairs, const int32_t* tap_ptr,
-                  const int32_t* pair_in, const int32_t* pair_slot, const void* weight, int cout, void* y,
-                  hipStream_t stream) {
-    if (cin >= 64)
-        launch_pairs_kc<T, MT, NT, 64>(feat, cin, taps, n_pairs, tap_ptr, pair_in, pair_slot, weight, cout, y, stream);
-    else
-        launch_pairs_kc<T, MT, NT, 32>(feat, cin, taps, n_pairs, tap_ptr, pair_in, pair_slot, weight, cout, y, stream);
+void launch_dense(const void* feat, int64_t n, int cin, const int32_t* nbr, int taps, bool tap_major,
+                  const void* weight, const void* bias, int cout, void* out, hipStream_t stream) {
+    constexpr int ROWS = CONV_WAVES * MT * 32, COUT_TILE = NT * 32;
+    constexpr int KC = NT >= 4 ? 32 : 64;   // the 128-register accumulator leaves room for 32-channel prefetches only
+    dim3 grid((unsigned)ptv3_ceil_div(n, ROWS), (unsigned)ptv3_ceil_div(cout, COUT_TILE));
+    hipLaunchKernelGGL((subm_conv_dense_kernel<T, MT, NT, KC, false>), grid, dim3(CONV_THREADS), 0, stream,
+                       (const T*)feat, n, cin, nbr, taps, tap_major, (const T*)weight, (const T*)bias, cout, (T*)out,
+                       (const int32_t*)nullptr, (const int32_t*)nullptr, (const int32_t*)nullptr);
 }
 
 template <typename T>
-void dispatch_pairs(const void* feat, int cin, int taps, int64_t n_pairs, const int32_t* tap_ptr,
-                    const int32_t* pair_in, const int32_t* pair_slot, const void* weight, int cout, void* y,
-                    hipStream_t stream) {
+void dispatch_dense(const void* feat, int64_t n, int cin, const int32_t* nbr, int taps, bool tap_major,
+                    const void* weight, const void* bias, int cout, void* out, hipStream_t stream) {
+    // Rows per work-group: 256 while that still yields about two work-groups per CU, else 128.
     const int64_t col_tiles = cout <= 64 ? 1 : ptv3_ceil_div(cout, 128);
-    const bool wide = (n_pairs / 256 + taps) * col_tiles >= 512;
-#define PTV3_PAIRS(MT, NT) launch_pairs<T, MT, NT>(feat, cin, taps, n_pairs, tap_ptr, pair_in, pair_slot, weight, cout, y, stream)
-    if (cout <= 32) { if (wide) PTV3_PAIRS(2, 1); else PTV3_PAIRS(1, 1); }
-    else if (cout <= 64) { if (wide) PTV3_PAIRS(2, 2); else PTV3_PAIRS(1, 2); }
-    else { if (wide) PTV3_PAIRS(2, 4); else PTV3_PAIRS(1, 4); }
+    const bool wide = ptv3_ceil_div(n, 256) * col_tiles >= 512;
+#define PTV3_DENSE(MT, NT) launch_dense<T, MT, NT>(feat, n, cin, nbr, taps, tap_major, weight, bias, cout, out, stream)
+    if (cout <= 32) { if (wide) PTV3_DENSE(2, 1); else PTV3_DENSE(1, 1); }
+    else if (cout <= 64) { if (wide) PTV3_DENSE(2, 2); else PTV3_DENSE(1, 2); }
+    else { if (wide) PTV3_DENSE(2, 4); else PTV3_DENSE(1, 4); }
+#undef PTV3_DENSE
+}
+
+template <typename T, int MT, int NT>
+int launch_pairs(const void* feat, int cin, int taps, int64_t n_pairs, const int32_t* tap_ptr,
+                 const int32_t* pair_in, const int32_t* pair_slot, const void* weight, int cout, void* y,
+                 hipStream_t stream) {
+    constexpr int ROWS = CONV_WAVES * MT * 32, COUT_TILE = NT * 32;
+    const size_t lds = ((size_t)COUT_TILE * (cin + W_PAD) + (size_t)CONV_WAVES * 32 * XS_STRIDE) * sizeof(T);
+    if (lds > 160 * 1024) return PTV3_ESHAPE;
+    auto kern = subm_conv_pairs_kernel<T, MT, NT, (NT >= 4 ? 32 : 64)>;
+    static size_t lds_allowed = 0;   // per instantiation
+    if (lds > lds_allowed) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        lds_allowed = lds;
+    }
+    // Rows per work-group: long enough to amortise staging the weights, short enough to give
+    // every CU a few work-groups.
+    const int64_t col_tiles = ptv3_ceil_div(cout, COUT_TILE);
+    int64_t range_rows = ROWS * 8;
+    while (range_rows > ROWS && (n_pairs / range_rows + taps) * col_tiles < 1024) range_rows /= 2;
+    dim3 grid((unsigned)(n_pairs / range_rows + taps), (unsigned)col_tiles);   // every tap may end with a partial range
+    hipLaunchKernelGGL(kern, grid, dim3(CONV_THREADS), lds, stream, (const T*)feat, cin, taps, (const T*)weight, cout,
+                       (T*)y, pair_in, pair_slot, tap_ptr, (int)range_rows);
+    return PTV3_OK;
+}
+
+// pair tiles through the chunked kernel (55 KB of LDS whatever cin is)
+template <typename T>
+int launch_pairs_chunked(const void* feat, int cin, int taps, int64_t n_pairs, const int32_t* tap_ptr,
+                         const int32_t* pair_in, const int32_t* pair_slot, const void* weight, int cout, void* y,
+                         hipStream_t stream) {
+    constexpr int MT = 2, NT = 4, KC = 32, ROWS = CONV_WAVES * MT * 32, COUT_TILE = NT * 32;
+    dim3 grid((unsigned)(n_pairs / ROWS + taps), (unsigned)ptv3_ceil_div(cout, COUT_TILE));
+    hipLaunchKernelGGL((subm_conv_dense_kernel<T, MT, NT, KC, true>), grid, dim3(CONV_THREADS), 0, stream,
+                       (const T*)feat, (int64_t)0, cin, (const int32_t*)nullptr, taps, false, (const T*)weight,
+                       (const T*)nullptr, cout, (T*)y, pair_in, pair_slot, tap_ptr);
+    return PTV3_OK;
+}
+
+template <typename T>
+int dispatch_pairs(const void* feat, int cin, int taps, int64_t n_pairs, const int32_t* tap_ptr,
+                   const int32_t* pair_in, const int32_t* pair_slot, const void* weight, int cout, void* y,
+                   hipStream_t stream) {
+    // one tap's weights for 128 output channels: 34 KB at cin 128 (two or three work-groups per
+    // CU), 86 KB at 256 (one): from there on the chunked kernel keeps more waves in flight
+    if (cin >= 256 && cout > 64)
+        return launch_pairs_chunked<T>(feat, cin, taps, n_pairs, tap_ptr, pair_in, pair_slot, weight, cout, y, stream);
+#define PTV3_PAIRS(MT, NT) return launch_pairs<T, MT, NT>(feat, cin, taps, n_pairs, tap_ptr, pair_in, pair_slot, weight, cout, y, stream)
+    if (cout <= 32) PTV3_PAIRS(2, 1);
+    if (cout <= 64) PTV3_PAIRS(2, 2);
+    PTV3_PAIRS(2, 4);
 #undef PTV3_PAIRS
 }
 
@@ -424,7 +689,7 @@ extern "C" int ptv3_subm_conv_fwd(const void* feat, int dtype, int64_t n, int ci
         PTV3_RETURN_LAUNCH();
     }
     // operand registers are 8-channel pieces of 16-channel steps; stores are 4-channel pieces
-    if (cin % 16 != 0 || cout % 4 != 0) return PTV3_ESHAPE;
+    if (cin % 16 != 0 || cout % 8 != 0) return PTV3_ESHAPE;
     if (dtype == PTV3_F16)
         dispatch_dense<_Float16>(feat, n, cin, nbr, taps, tap_major, weight, bias, cout, out, stream);
     else
@@ -446,14 +711,17 @@ extern "C" int ptv3_subm_conv_pairs_fwd(const void* feat, int dtype, int64_t n, 
     if (n_pairs > 0 && (!pair_in || !pair_slot || !y)) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
     const dim3 sgrid((unsigned)ptv3_ceil_div(n * (cout / 8), 256)), sblock(256);
+    int rc = PTV3_OK;
     if (dtype == PTV3_F16) {
         if (n_pairs > 0)
-            dispatch_pairs<_Float16>(feat, cin, taps, n_pairs, tap_ptr, pair_in, pair_slot, weight, cout, y, stream);
+            rc = dispatch_pairs<_Float16>(feat, cin, taps, n_pairs, tap_ptr, pair_in, pair_slot, weight, cout, y, stream);
+        if (rc != PTV3_OK) return rc;
         hipLaunchKernelGGL(pair_segment_sum_kernel<_Float16>, sgrid, sblock, 0, stream, (const _Float16*)y,
                            row_ptr, n, cout, (const _Float16*)bias, (_Float16*)out);
     } else {
         if (n_pairs > 0)
-            dispatch_pairs<__bf16>(feat, cin, taps, n_pairs, tap_ptr, pair_in, pair_slot, weight, cout, y, stream);
+            rc = dispatch_pairs<__bf16>(feat, cin, taps, n_pairs, tap_ptr, pair_in, pair_slot, weight, cout, y, stream);
+        if (rc != PTV3_OK) return rc;
         hipLaunchKernelGGL(pair_segment_sum_kernel<__bf16>, sgrid, sblock, 0, stream, (const __bf16*)y, row_ptr,
                            n, cout, (const __bf16*)bias, (__bf16*)out);
     }

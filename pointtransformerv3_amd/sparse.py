@@ -51,9 +51,10 @@ class SubMConv3d(nn.Module):
     (out, k, k, k, in) layout so checkpoints keep loading; `padding` is accepted and unused,
     as submanifold convolutions are centred by construction."""
 
-    # above this fraction of active (voxel, tap) pairs the dense output-stationary kernel wins
-    # (no pair buffer round trip); surface scans sit at 0.05-0.5
-    PAIR_MODE_MAX_DENSITY = 0.7
+    # above this fraction of active (voxel, tap) pairs the dense output-stationary kernel is used
+    # (no pair-matrix round trip, but MFMA work for every tap); a 2 cm surface scan goes from 0.05
+    # at full resolution to 0.5 at the coarsest level, where the two forms measure about equal
+    PAIR_MODE_MAX_DENSITY = 0.6
 
     def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
                  groups=1, bias=True, indice_key=None):
