@@ -47,6 +47,10 @@ const char *ptv3_strerror(int rc);
 int ptv3_encode(const int32_t *grid_coord, const int64_t *batch, int64_t n, int depth,
                 const int32_t *order_ids_host, int k, int64_t *code, void *stream);
 
+/* model.py:100 (depth = bit length of the largest coordinate) and :162-164 (sparse_shape):
+ * per-axis maximum of grid_coord (n,3) int32 into out3 (3 int32, device). n >= 1. */
+int ptv3_grid_max(const int32_t *grid_coord, int64_t n, int32_t *out3, void *stream);
+
 /* model.py:119-126 and :667-674: per-row ascending argsort of (k,n) int64 codes plus the
  * inverse permutation. Only the low `key_bits` bits are sorted on (the rest must be equal
  * across a row, e.g. zero); ties keep their input order. */
@@ -151,12 +155,13 @@ int ptv3_unpool_add(const void *parent, const void *child, int dtype, int64_t n,
 /* nn.LayerNorm calls model.py:554,557,572 fused with the residual adds :589,:594,:602.
  * x,res,out0,out1 (n,c); gamma,beta (c,); all of dtype, statistics in fp32.
  * mode 0: out0 = LN(x).  mode 1: out0 = res + LN(x).
- * mode 2: out0 = x + res, out1 = LN(out0).
+ * mode 2: s = x + res, out1 = LN(s), out0 = s + shift (shift (c,) or NULL: the bias of a GEMM that
+ *         will accumulate onto out0).
  * mode 3: out0 = res + LN(x), out1 = LN(out0) with the second affine pair gamma2,beta2.
  * Intermediates are rounded to dtype where separate kernels would have stored them. */
 int ptv3_layer_norm(const void *x, const void *res, const void *gamma, const void *beta,
-                    const void *gamma2, const void *beta2, int dtype, int64_t n, int c, float eps,
-                    int mode, void *out0, void *out1, void *stream);
+                    const void *gamma2, const void *beta2, const void *shift, int dtype, int64_t n,
+                    int c, float eps, int mode, void *out0, void *out1, void *stream);
 
 #ifdef __cplusplus
 }

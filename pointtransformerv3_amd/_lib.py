@@ -16,6 +16,7 @@ SIGNATURES = {
     "ptv3_version": (_i32, []),
     "ptv3_strerror": (ctypes.c_char_p, [_i32]),
     "ptv3_encode": (_i32, [_vp, _vp, _i64, _i32, _vp, _i32, _vp, _vp]),
+    "ptv3_grid_max": (_i32, [_vp, _i64, _vp, _vp]),
     "ptv3_argsort_workspace_bytes": (_sz, [_i64, _i32]),
     "ptv3_argsort": (_i32, [_vp, _i64, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
     "ptv3_pad_sizes": (_i32, [_vp, _i32, _i64, _vp, _vp]),
@@ -38,7 +39,7 @@ SIGNATURES = {
                                 _vp]),
     "ptv3_segment_reduce": (_i32, [_vp, _i32, _i64, _i32, _vp, _vp, _i64, _i32, _vp, _vp]),
     "ptv3_unpool_add": (_i32, [_vp, _vp, _i32, _i64, _i32, _vp, _i64, _vp, _vp]),
-    "ptv3_layer_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _f32, _i32, _vp, _vp, _vp]),
+    "ptv3_layer_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _f32, _i32, _vp, _vp, _vp]),
 }
 
 _lib = None

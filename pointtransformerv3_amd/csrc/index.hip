@@ -59,7 +59,37 @@ __global__ __launch_bounds__(256) void attn_slots_kernel(
     slot_dst[i] = (unpad[inverse_row[row]] == i) ? (int32_t)row : -1;
 }
 
+// per-axis maximum of (n,3) int32 coordinates into out[3] (pre-set to INT_MIN by the caller's
+// first kernel below): wave reduce, then one atomic per wave and axis
+__global__ void grid_max_init_kernel(int32_t* __restrict__ out) {
+    if (threadIdx.x < 3) out[threadIdx.x] = INT32_MIN;
+}
+
+__global__ __launch_bounds__(256) void grid_max_kernel(const int32_t* __restrict__ grid_coord, int64_t n,
+                                                       int32_t* __restrict__ out) {
+    int32_t m[3] = {INT32_MIN, INT32_MIN, INT32_MIN};
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) m[a] = max(m[a], grid_coord[3 * i + a]);
+    }
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) m[a] = max(m[a], __shfl_xor(m[a], off, PTV3_WAVE));
+        if (threadIdx.x % PTV3_WAVE == 0) atomicMax(&out[a], m[a]);
+    }
+}
+
 }  // namespace
+
+extern "C" int ptv3_grid_max(const int32_t* grid_coord, int64_t n, int32_t* out3, void* stream_) {
+    if (n < 1 || !grid_coord || !out3) return PTV3_EINVAL;
+    hipStream_t stream = (hipStream_t)stream_;
+    hipLaunchKernelGGL(grid_max_init_kernel, dim3(1), dim3(64), 0, stream, out3);
+    const int64_t blocks = ptv3_ceil_div(n, 256 * 8) < 1024 ? ptv3_ceil_div(n, 256 * 8) : 1024;
+    hipLaunchKernelGGL(grid_max_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, grid_coord, n, out3);
+    PTV3_RETURN_LAUNCH();
+}
 
 extern "C" int ptv3_pad_sizes(const int64_t* offset_host, int nb, int64_t patch, int64_t* n_pad,
                               int64_t* n_seq) {

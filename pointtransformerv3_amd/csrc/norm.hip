@@ -9,6 +9,8 @@
 //   mode 0: out0 = LN(x)
 //   mode 1: out0 = res + LN(x)                      (cpe: shortcut + LN(Linear(conv)))
 //   mode 2: out0 = x + res; out1 = LN(out0)         (shortcut + branch, then pre-norm)
+//           with an optional per-channel `shift` added to the stored out0 only (the bias of the
+//           GEMM that will accumulate onto out0), out1 is still LN(x + res)
 //   mode 3: out0 = res + LN(x); out1 = LN2(out0)    (cpe residual, then the attention pre-norm)
 // Intermediate results are rounded to the storage type exactly where separate kernels would
 // have stored them, so fusing changes no value.
@@ -59,8 +61,8 @@ __device__ __forceinline__ void row_stats(const float (&v)[8], float eps, float&
 template <typename T, int LPR, int MODE>
 __global__ __launch_bounds__(256) void layer_norm_kernel(
     const T* __restrict__ x, const T* __restrict__ res, const T* __restrict__ gamma,
-    const T* __restrict__ beta, const T* __restrict__ gamma2, const T* __restrict__ beta2, int64_t n,
-    float eps, T* __restrict__ out0, T* __restrict__ out1) {
+    const T* __restrict__ beta, const T* __restrict__ gamma2, const T* __restrict__ beta2,
+    const T* __restrict__ shift, int64_t n, float eps, T* __restrict__ out0, T* __restrict__ out1) {
     constexpr int C = 8 * LPR;
     constexpr int ROWS_PER_BLOCK = 256 / LPR;
     const int sub = threadIdx.x % LPR;
@@ -79,7 +81,17 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(
     if (MODE == 2) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[i] = round_to<T>(v[i] + r[i]);
-        if (live) store8(out0 + off, v);
+        if (live) {
+            if (shift) {
+                float sh[8], w[8];
+                load8(shift + sub * 8, sh);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) w[i] = v[i] + sh[i];
+                store8(out0 + off, w);
+            } else {
+                store8(out0 + off, v);
+            }
+        }
     }
     float mean, rstd;
     row_stats<LPR>(v, eps, mean, rstd);
@@ -105,8 +117,8 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(
 template <typename T, int MODE>
 __global__ __launch_bounds__(256) void layer_norm_generic_kernel(
     const T* __restrict__ x, const T* __restrict__ res, const T* __restrict__ gamma,
-    const T* __restrict__ beta, int64_t n, int c, float eps, T* __restrict__ out0,
-    T* __restrict__ out1) {
+    const T* __restrict__ beta, const T* __restrict__ shift, int64_t n, int c, float eps,
+    T* __restrict__ out0, T* __restrict__ out1) {
     const int lane = threadIdx.x % PTV3_WAVE;
     const int64_t row = (int64_t)blockIdx.x * (256 / PTV3_WAVE) + threadIdx.x / PTV3_WAVE;
     if (row >= n) return;   // whole wave leaves together
@@ -117,7 +129,7 @@ __global__ __launch_bounds__(256) void layer_norm_generic_kernel(
         float v = (float)xr[i];
         if (MODE == 2) {
             const T t = (T)(v + (float)rr[i]);
-            out0[row * c + i] = t;
+            out1[row * c + i] = t;   // parked in out1 until the statistics are known
             v = (float)t;
         }
         s += v;
@@ -127,27 +139,30 @@ __global__ __launch_bounds__(256) void layer_norm_generic_kernel(
     const float mean = s / c;
     float q = 0.f;
     for (int i = lane; i < c; i += PTV3_WAVE) {
-        const float v = (MODE == 2 ? (float)out0[row * c + i] : (float)xr[i]) - mean;
+        const float v = (MODE == 2 ? (float)out1[row * c + i] : (float)xr[i]) - mean;
         q += v * v;
     }
 #pragma unroll
     for (int o = 1; o < PTV3_WAVE; o <<= 1) q += __shfl_xor(q, o, PTV3_WAVE);
     const float rstd = rsqrtf(q / c + eps);
     for (int i = lane; i < c; i += PTV3_WAVE) {
-        const float v = MODE == 2 ? (float)out0[row * c + i] : (float)xr[i];
+        const float v = MODE == 2 ? (float)out1[row * c + i] : (float)xr[i];
         float y = (v - mean) * rstd * (float)gamma[i] + (float)beta[i];
         if (MODE == 1) y = (float)(T)y + (float)rr[i];
+        if (MODE == 2) out0[row * c + i] = (T)(v + (shift ? (float)shift[i] : 0.f));
         (MODE == 2 ? out1 : out0)[row * c + i] = (T)y;
     }
 }
 
 template <typename T, int MODE>
 void launch(const void* x, const void* res, const void* gamma, const void* beta, const void* gamma2,
-            const void* beta2, int64_t n, int c, float eps, void* out0, void* out1, hipStream_t stream) {
+            const void* beta2, const void* shift, int64_t n, int c, float eps, void* out0, void* out1,
+            hipStream_t stream) {
 #define PTV3_LN(LPR)                                                                            \
     hipLaunchKernelGGL((layer_norm_kernel<T, LPR, MODE>), dim3((unsigned)ptv3_ceil_div(n, 256 / LPR)), \
                        dim3(256), 0, stream, (const T*)x, (const T*)res, (const T*)gamma,       \
-                       (const T*)beta, (const T*)gamma2, (const T*)beta2, n, eps, (T*)out0, (T*)out1)
+                       (const T*)beta, (const T*)gamma2, (const T*)beta2, (const T*)shift, n, eps, (T*)out0,  \
+                       (T*)out1)
     switch (c) {
         case 32: PTV3_LN(4); break;
         case 64: PTV3_LN(8); break;
@@ -158,15 +173,15 @@ void launch(const void* x, const void* res, const void* gamma, const void* beta,
             if (MODE == 3) {   // two generic passes: out0 = res + LN(x), then out1 = LN2(out0)
                 hipLaunchKernelGGL((layer_norm_generic_kernel<T, 1>), dim3((unsigned)ptv3_ceil_div(n, 4)),
                                    dim3(256), 0, stream, (const T*)x, (const T*)res, (const T*)gamma,
-                                   (const T*)beta, n, c, eps, (T*)out0, (T*)nullptr);
+                                   (const T*)beta, (const T*)nullptr, n, c, eps, (T*)out0, (T*)nullptr);
                 hipLaunchKernelGGL((layer_norm_generic_kernel<T, 0>), dim3((unsigned)ptv3_ceil_div(n, 4)),
                                    dim3(256), 0, stream, (const T*)out0, (const T*)nullptr, (const T*)gamma2,
-                                   (const T*)beta2, n, c, eps, (T*)out1, (T*)nullptr);
+                                   (const T*)beta2, (const T*)nullptr, n, c, eps, (T*)out1, (T*)nullptr);
             } else {
                 constexpr int GM = MODE == 3 ? 0 : MODE;
                 hipLaunchKernelGGL((layer_norm_generic_kernel<T, GM>), dim3((unsigned)ptv3_ceil_div(n, 4)),
                                    dim3(256), 0, stream, (const T*)x, (const T*)res, (const T*)gamma,
-                                   (const T*)beta, n, c, eps, (T*)out0, (T*)out1);
+                                   (const T*)beta, (const T*)shift, n, c, eps, (T*)out0, (T*)out1);
             }
     }
 #undef PTV3_LN
@@ -174,19 +189,20 @@ void launch(const void* x, const void* res, const void* gamma, const void* beta,
 
 template <typename T>
 void launch_mode(int mode, const void* x, const void* res, const void* gamma, const void* beta,
-                 const void* gamma2, const void* beta2, int64_t n, int c, float eps, void* out0,
-                 void* out1, hipStream_t stream) {
-    if (mode == 0) launch<T, 0>(x, res, gamma, beta, gamma2, beta2, n, c, eps, out0, out1, stream);
-    else if (mode == 1) launch<T, 1>(x, res, gamma, beta, gamma2, beta2, n, c, eps, out0, out1, stream);
-    else if (mode == 2) launch<T, 2>(x, res, gamma, beta, gamma2, beta2, n, c, eps, out0, out1, stream);
-    else launch<T, 3>(x, res, gamma, beta, gamma2, beta2, n, c, eps, out0, out1, stream);
+                 const void* gamma2, const void* beta2, const void* shift, int64_t n, int c, float eps,
+                 void* out0, void* out1, hipStream_t stream) {
+    if (mode == 0) launch<T, 0>(x, res, gamma, beta, gamma2, beta2, shift, n, c, eps, out0, out1, stream);
+    else if (mode == 1) launch<T, 1>(x, res, gamma, beta, gamma2, beta2, shift, n, c, eps, out0, out1, stream);
+    else if (mode == 2) launch<T, 2>(x, res, gamma, beta, gamma2, beta2, shift, n, c, eps, out0, out1, stream);
+    else launch<T, 3>(x, res, gamma, beta, gamma2, beta2, shift, n, c, eps, out0, out1, stream);
 }
 
 }  // namespace
 
 extern "C" int ptv3_layer_norm(const void* x, const void* res, const void* gamma, const void* beta,
-                               const void* gamma2, const void* beta2, int dtype, int64_t n, int c,
-                               float eps, int mode, void* out0, void* out1, void* stream_) {
+                               const void* gamma2, const void* beta2, const void* shift, int dtype,
+                               int64_t n, int c, float eps, int mode, void* out0, void* out1,
+                               void* stream_) {
     if (n < 0 || c < 1 || mode < 0 || mode > 3) return PTV3_EINVAL;
     if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
     if (n == 0) return PTV3_OK;
@@ -196,10 +212,10 @@ extern "C" int ptv3_layer_norm(const void* x, const void* res, const void* gamma
     if (mode == 3 && (!gamma2 || !beta2)) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
     if (dtype == PTV3_F32)
-        launch_mode<float>(mode, x, res, gamma, beta, gamma2, beta2, n, c, eps, out0, out1, stream);
+        launch_mode<float>(mode, x, res, gamma, beta, gamma2, beta2, shift, n, c, eps, out0, out1, stream);
     else if (dtype == PTV3_F16)
-        launch_mode<_Float16>(mode, x, res, gamma, beta, gamma2, beta2, n, c, eps, out0, out1, stream);
+        launch_mode<_Float16>(mode, x, res, gamma, beta, gamma2, beta2, shift, n, c, eps, out0, out1, stream);
     else
-        launch_mode<__bf16>(mode, x, res, gamma, beta, gamma2, beta2, n, c, eps, out0, out1, stream);
+        launch_mode<__bf16>(mode, x, res, gamma, beta, gamma2, beta2, shift, n, c, eps, out0, out1, stream);
     PTV3_RETURN_LAUNCH();
 }

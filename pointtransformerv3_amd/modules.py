@@ -266,9 +266,17 @@ class Block(PointModule):
                                       mode=3, weight2=ln1.weight, bias2=ln1.bias)
         point.feat = normed
         point = self.attn(point)
-        # feat += attention branch, plus the pre-norm for the MLP
-        feat, normed = ops.layer_norm(point.feat, ln2.weight, ln2.bias, ln2.eps, residual=feat, mode=2)
-        feat = feat + self.mlp[0](normed)
+        # feat += attention branch, plus the pre-norm for the MLP. When the MLP is the plain
+        # fc1-act-fc2 without dropout, fc2's bias is added to the stored sum here and fc2 itself
+        # accumulates onto it (GEMM with beta = 1): feat + fc2(h) + b2 without a separate add pass.
+        mlp = self.mlp[0]
+        plain_mlp = type(mlp) is MLP and mlp.fc2.bias is not None and not (self.training and mlp.drop.p > 0)
+        feat, normed = ops.layer_norm(point.feat, ln2.weight, ln2.bias, ln2.eps, residual=feat, mode=2,
+                                      shift=mlp.fc2.bias if plain_mlp else None)
+        if plain_mlp:
+            feat = torch.addmm(feat, mlp.act(mlp.fc1(normed)), mlp.fc2.weight.t())
+        else:
+            feat = feat + mlp(normed)
         point.feat = feat
         point.sparse_conv_feat = point.sparse_conv_feat.replace_feature(feat)
         return point

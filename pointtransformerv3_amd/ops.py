@@ -63,6 +63,16 @@ def encode_orders(grid_coord, batch, depth, orders):
     return code
 
 
+def grid_max(grid_coord):
+    """Per-axis maximum of (N,3) int32 coordinates as a (3,) int32 device tensor."""
+    _dev(grid_coord)
+    lib = _lib.load()
+    g = grid_coord.to(torch.int32).contiguous()
+    out = torch.empty(3, dtype=torch.int32, device=g.device)
+    _lib.check(lib.ptv3_grid_max(_ptr(g), g.shape[0], _ptr(out), _stream()), "ptv3_grid_max")
+    return out
+
+
 def argsort_rows(code, key_bits):
     """Row-wise ascending argsort of (k,N) int64 codes + inverse permutation."""
     _dev(code)
@@ -301,12 +311,14 @@ def unpool_add(parent, child, cluster):
     return out
 
 
-def layer_norm(x, weight, bias, eps=1e-5, residual=None, mode=0, weight2=None, bias2=None):
+def layer_norm(x, weight, bias, eps=1e-5, residual=None, mode=0, weight2=None, bias2=None, shift=None):
     """Row-wise LayerNorm fused with neighbouring residual adds.
 
-    mode 0: LN(x).  mode 1: residual + LN(x).  mode 2: (s, LN(s)) with s = x + residual.
+    mode 0: LN(x).  mode 1: residual + LN(x).
+    mode 2: (s + shift, LN(s)) with s = x + residual; shift (C,) is optional (the bias of a GEMM
+    that will accumulate onto the first result).
     mode 3: (y, LN2(y)) with y = residual + LN(x) and LN2 using weight2/bias2."""
-    _dev(x, weight, bias, residual, weight2, bias2)
+    _dev(x, weight, bias, residual, weight2, bias2, shift)
     lib = _lib.load()
     x = x.contiguous()
     n, c = x.shape
@@ -315,9 +327,10 @@ def layer_norm(x, weight, bias, eps=1e-5, residual=None, mode=0, weight2=None, b
     res = None if residual is None else residual.to(dt).contiguous()
     w2 = None if weight2 is None else weight2.to(dt).contiguous()
     b2 = None if bias2 is None else bias2.to(dt).contiguous()
+    sh = None if shift is None else shift.to(dt).contiguous()
     out0 = torch.empty_like(x)
     out1 = torch.empty_like(x) if mode >= 2 else None
-    _lib.check(lib.ptv3_layer_norm(_ptr(x), _ptr(res), _ptr(w), _ptr(b), _ptr(w2), _ptr(b2), _dtype_code(x),
-                                   n, c, float(eps), int(mode), _ptr(out0), _ptr(out1), _stream()),
+    _lib.check(lib.ptv3_layer_norm(_ptr(x), _ptr(res), _ptr(w), _ptr(b), _ptr(w2), _ptr(b2), _ptr(sh),
+                                   _dtype_code(x), n, c, float(eps), int(mode), _ptr(out0), _ptr(out1), _stream()),
                "ptv3_layer_norm")
     return out0 if mode < 2 else (out0, out1)

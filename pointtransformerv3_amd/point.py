@@ -77,7 +77,7 @@ class Point(AttrDict):
         """Per-axis maximum of grid_coord as a Python list of 3 ints."""
         if "_grid_max_host" not in self:
             self._ensure_grid_coord()
-            self["_grid_max_host"] = [int(v) for v in self["grid_coord"].max(0).values.tolist()]
+            self["_grid_max_host"] = [int(v) for v in ops.grid_max(self["grid_coord"]).tolist()]
         return self["_grid_max_host"]
 
     def _ensure_grid_coord(self):

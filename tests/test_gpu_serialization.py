@@ -113,3 +113,10 @@ def test_attn_slots():
     assert np.array_equal(src.cpu().numpy(), want_src)
     assert np.array_equal(dst.cpu().numpy(), np.where(primary, want_src, -1))
     assert primary.sum() == n
+
+
+def test_grid_max():
+    rng = np.random.default_rng(3)
+    for n in (1, 77, 300_001):
+        g = rng.integers(-5, 70_000, size=(n, 3)).astype(np.int32)
+        assert ops().grid_max(to_dev(g)).tolist() == g.max(0).tolist()

@@ -124,6 +124,8 @@ def test_layer_norm_modes(dtype, c):
     s, z = o.layer_norm(dv(x), dv(w), dv(b), residual=dv(r), mode=2)
     want_s = (x.float() + r.float()).to(dtype)
     assert rel_err(s, want_s.float()) < tol and rel_err(z, ln(want_s, w, b)) < tol
+    s2, z2 = o.layer_norm(dv(x), dv(w), dv(b), residual=dv(r), mode=2, shift=dv(b2))
+    assert rel_err(s2, want_s.float() + b2.float()) < tol and torch.equal(z2, z)
     y, z = o.layer_norm(dv(x), dv(w), dv(b), residual=dv(r), mode=3, weight2=dv(w2), bias2=dv(b2))
     want_y = (r.float() + ln(x, w, b).to(dtype).float()).to(dtype)
     assert rel_err(y, want_y.float()) < tol and rel_err(z, ln(want_y, w2, b2)) < tol
