@@ -163,6 +163,15 @@ int ptv3_layer_norm(const void *x, const void *res, const void *gamma, const voi
                     const void *gamma2, const void *beta2, const void *shift, int dtype, int64_t n,
                     int c, float eps, int mode, void *out0, void *out1, void *stream);
 
+/* MLP of a block plus its residual, model.py:510-516 and :602, in one kernel:
+ * out = resid + fc2(GELU(fc1(x))), exact (erf) GELU, intermediates rounded to dtype where the
+ * separate layers would have stored them. x, resid, out (n, channels); w1 (hidden, channels),
+ * b1 (hidden,), w2 (channels, hidden), b2 (channels,). fp16/bf16, channels 32 or 64,
+ * hidden = 4 * channels (PTV3_ESHAPE otherwise: use the separate layers). */
+int ptv3_mlp_fused(const void *x, const void *resid, const void *w1, const void *b1, const void *w2,
+                   const void *b2, int dtype, int64_t n, int channels, int hidden, void *out,
+                   void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -266,14 +266,22 @@ class Block(PointModule):
                                       mode=3, weight2=ln1.weight, bias2=ln1.bias)
         point.feat = normed
         point = self.attn(point)
-        # feat += attention branch, plus the pre-norm for the MLP. When the MLP is the plain
-        # fc1-act-fc2 without dropout, fc2's bias is added to the stored sum here and fc2 itself
-        # accumulates onto it (GEMM with beta = 1): feat + fc2(h) + b2 without a separate add pass.
+        # feat += attention branch, plus the pre-norm for the MLP
         mlp = self.mlp[0]
-        plain_mlp = type(mlp) is MLP and mlp.fc2.bias is not None and not (self.training and mlp.drop.p > 0)
+        plain_mlp = (type(mlp) is MLP and mlp.fc1.bias is not None and mlp.fc2.bias is not None
+                     and not (self.training and mlp.drop.p > 0))
+        exact_gelu = type(mlp.act) is nn.GELU and mlp.act.approximate == "none" if plain_mlp else False
+        fused = (plain_mlp and exact_gelu and self.channels in ops.MLP_FUSED_CHANNELS
+                 and mlp.fc1.out_features == 4 * self.channels and point.feat.dtype != torch.float32)
+        # when fc2 runs as a separate GEMM it accumulates onto the stored sum (beta = 1), so its
+        # bias is added to that sum here: feat + fc2(h) + b2 without a separate add pass
         feat, normed = ops.layer_norm(point.feat, ln2.weight, ln2.bias, ln2.eps, residual=feat, mode=2,
-                                      shift=mlp.fc2.bias if plain_mlp else None)
-        if plain_mlp:
+                                      shift=mlp.fc2.bias if (plain_mlp and not fused) else None)
+        if fused:
+            # thin channels, many points: fc1 + GELU + fc2 + residual in one kernel, the 4C-wide
+            # hidden tensor never leaves the CU
+            feat = ops.mlp_fused(normed, feat, mlp.fc1.weight, mlp.fc1.bias, mlp.fc2.weight, mlp.fc2.bias)
+        elif plain_mlp:
             feat = torch.addmm(feat, mlp.act(mlp.fc1(normed)), mlp.fc2.weight.t())
         else:
             feat = feat + mlp(normed)

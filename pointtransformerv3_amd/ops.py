@@ -334,3 +334,22 @@ def layer_norm(x, weight, bias, eps=1e-5, residual=None, mode=0, weight2=None, b
                                    _dtype_code(x), n, c, float(eps), int(mode), _ptr(out0), _ptr(out1), _stream()),
                "ptv3_layer_norm")
     return out0 if mode < 2 else (out0, out1)
+
+
+MLP_FUSED_CHANNELS = (32, 64)
+
+
+def mlp_fused(x, resid, w1, b1, w2, b2):
+    """resid + fc2(GELU(fc1(x))) in one kernel (exact GELU). x, resid (N,C) fp16/bf16 with C in
+    MLP_FUSED_CHANNELS; w1 (4C,C), b1 (4C,), w2 (C,4C), b2 (C,)."""
+    _dev(x, resid, w1, b1, w2, b2)
+    lib = _lib.load()
+    x = x.contiguous()
+    resid = resid.to(x.dtype).contiguous()
+    n, c = x.shape
+    dt = x.dtype
+    w1c, b1c, w2c, b2c = (t.to(dt).contiguous() for t in (w1, b1, w2, b2))
+    out = torch.empty_like(x)
+    _lib.check(lib.ptv3_mlp_fused(_ptr(x), _ptr(resid), _ptr(w1c), _ptr(b1c), _ptr(w2c), _ptr(b2c), _dtype_code(x),
+                                  n, c, w1c.shape[0], _ptr(out), _stream()), "ptv3_mlp_fused")
+    return out

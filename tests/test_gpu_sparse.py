@@ -187,3 +187,20 @@ def test_tap_major_layout_is_the_transpose():
         feat = torch.randn(len(idx), 64, generator=g).to(dtype).to(DEV)
         w = (torch.randn(64, 27, 64, generator=g) * 0.05).to(dtype).to(DEV)
         assert torch.equal(o.subm_conv(feat, nbr, w), o.subm_conv(feat, nbr_t, w, tap_major=True))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("c,n", [(32, 1), (32, 5000), (64, 33), (64, 70_001)])
+def test_mlp_fused_parity(dtype, c, n):
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(c + n)
+    x = torch.randn(n, c, generator=g).to(dtype)
+    r = torch.randn(n, c, generator=g).to(dtype)
+    w1 = (torch.randn(4 * c, c, generator=g) / c ** 0.5).to(dtype)
+    b1 = (torch.randn(4 * c, generator=g) * 0.5).to(dtype)
+    w2 = (torch.randn(c, 4 * c, generator=g) / (4 * c) ** 0.5).to(dtype)
+    b2 = (torch.randn(c, generator=g) * 0.5).to(dtype)
+    h = F.gelu(F.linear(x.float(), w1.float(), b1.float()))
+    want = r.float() + F.linear(h, w2.float(), b2.float())
+    got = ops().mlp_fused(*(t.to(DEV) for t in (x, r, w1, b1, w2, b2)))
+    assert got.dtype == dtype and rel_err(got, want) < TOL[dtype]
