@@ -52,6 +52,19 @@ def attention_flops(work):
     return float(4.0 * (lens * lens).sum().item() * channels)
 
 
+def recorded_traffic(n_points):
+    """HBM bytes per attention launch from the committed rocprofv3 --pmc summary of this same
+    workload (FETCH_SIZE and WRITE_SIZE runs, each scaled by a 1 GiB copy in the same process);
+    None when the summary is for another workload."""
+    path = os.path.join(ROOT, "profiles", "attention_traffic.json")
+    try:
+        with open(path) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None
+    return rec.get("traffic_bytes_per_launch") if rec.get("workload_points") == n_points else None
+
+
 def build_inputs(n_scenes, pts_per_scene, seed0):
     from pointtransformerv3_amd import synthetic
     scenes = [synthetic.room_scene(pts_per_scene, seed0 + i, 0.02) for i in range(n_scenes)]
@@ -198,6 +211,9 @@ def main():
     ap.add_argument("--scenes", type=int, default=4)
     ap.add_argument("--points", type=int, default=106_000, help="points drawn per scene before voxel dedup")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 1 GiB device copy (a kernel of known traffic) so that rocprofv3 --pmc "
+                         "FETCH_SIZE / WRITE_SIZE readings of this process can be scaled to bytes")
     ap.add_argument("--kernels", metavar="PATH", default=None,
                     help="also measure every kernel alone against its roofline and write the table to PATH")
     args = ap.parse_args()
@@ -255,12 +271,17 @@ def main():
                                f"scenes, {n_points} voxelised points, grid 0.02 m, 6-dim input, random-init weights"},
         "roofline": {"bound": "mfma", "kernel": "patch_attn_half_kernel<f16>", "achieved": achieved,
                      "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
-                     "traffic": None, "launches": launches,
+                     "traffic": recorded_traffic(n_points), "launches": launches,
                      "avg_launch_us": attn_ms * 1e3 / max(launches, 1),
                      "flops_per_launch": attn_flops / max(launches, 1),
                      "attn_ms_per_step": attn_ms / args.steps},
         "cpu_baseline": cpu,
     }
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)          # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
     if args.kernels:
         kernel_rooflines(args.kernels)
     print(json.dumps(result))

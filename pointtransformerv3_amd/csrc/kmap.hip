@@ -6,10 +6,14 @@
 // stored voxel-major (n, taps) or tap-major (taps, n); the convolution kernels read the
 // tap-major form coalesced.
 //
-//   fill    : table keys <- EMPTY
-//   insert  : one thread per voxel, 64-bit CAS, linear probing (load factor <= 0.5)
+//   fill    : table keys <- EMPTY, filter bits <- 0
+//   insert  : one thread per voxel, 64-bit CAS, linear probing (load factor <= 0.5); also sets the
+//             voxel's bit in a hashed bitmap of 16 bits per voxel
 //   lookup  : one thread per map entry in storage order, so the int32 map is written fully
-//             coalesced in either layout
+//             coalesced in either layout. On surface scans 90-97 % of the probed neighbours do not
+//             exist, and a probe of the table costs a whole cache line from HBM (the table does not
+//             fit L2); the bitmap (1 MB for 400k voxels, L2-resident) answers "absent" for ~94 % of
+//             those without touching the table.
 #include "common.h"
 
 namespace {
@@ -23,28 +27,35 @@ __device__ __forceinline__ uint64_t voxel_key(int b, int x, int y, int z) {
            ((uint64_t)(uint32_t)(y + 4) << 17) | (uint64_t)(uint32_t)(z + 4);
 }
 
-__device__ __forceinline__ uint32_t hash_slot(uint64_t k, uint32_t mask) {
+// 64-bit finaliser: the low bits pick the table slot, the high bits the filter bit
+__device__ __forceinline__ uint64_t mix64(uint64_t k) {
     k ^= k >> 33;
     k *= 0xff51afd7ed558ccdull;
     k ^= k >> 33;
     k *= 0xc4ceb9fe1a85ec53ull;
     k ^= k >> 33;
-    return (uint32_t)k & mask;
+    return k;
 }
 
-__global__ __launch_bounds__(256) void kmap_fill_kernel(uint64_t* __restrict__ keys, int64_t cap) {
+__global__ __launch_bounds__(256) void kmap_fill_kernel(uint64_t* __restrict__ keys, int64_t cap,
+                                                        uint32_t* __restrict__ filter, int64_t filter_words) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < cap) keys[i] = EMPTY_KEY;
+    if (i < filter_words) filter[i] = 0u;
 }
 
 __global__ __launch_bounds__(256) void kmap_insert_kernel(const int32_t* __restrict__ indices,
                                                           int64_t n, uint64_t* __restrict__ keys,
-                                                          int32_t* __restrict__ vals, uint32_t mask) {
+                                                          int32_t* __restrict__ vals, uint32_t mask,
+                                                          uint32_t* __restrict__ filter, uint32_t filter_mask) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const int4 v = ((const int4*)indices)[i];
     const uint64_t key = voxel_key(v.x, v.y, v.z, v.w);
-    uint32_t slot = hash_slot(key, mask);
+    const uint64_t h = mix64(key);
+    const uint32_t bit = (uint32_t)(h >> 32) & filter_mask;
+    atomicOr(&filter[bit >> 5], 1u << (bit & 31));
+    uint32_t slot = (uint32_t)h & mask;
     for (uint32_t probe = 0; probe <= mask; ++probe) {
         const uint64_t prev = atomicCAS((unsigned long long*)&keys[slot], (unsigned long long)EMPTY_KEY,
                                         (unsigned long long)key);
@@ -61,7 +72,8 @@ __global__ __launch_bounds__(256) void kmap_lookup_kernel(const int32_t* __restr
                                                           int64_t n, int ks, int taps,
                                                           const uint64_t* __restrict__ keys,
                                                           const int32_t* __restrict__ vals,
-                                                          uint32_t mask, int32_t* __restrict__ nbr) {
+                                                          uint32_t mask, const uint32_t* __restrict__ filter,
+                                                          uint32_t filter_mask, int32_t* __restrict__ nbr) {
     // one thread per map entry, in the order the entries are stored, so writes coalesce
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= n * taps) return;
@@ -75,8 +87,11 @@ __global__ __launch_bounds__(256) void kmap_lookup_kernel(const int32_t* __restr
         found = (int32_t)i;   // centre tap
     } else {
         const uint64_t key = voxel_key(v.x, v.y + kx - r, v.z + ky - r, v.w + kz - r);
-        uint32_t slot = hash_slot(key, mask);
-        for (uint32_t probe = 0; probe <= mask; ++probe) {
+        const uint64_t h = mix64(key);
+        const uint32_t bit = (uint32_t)(h >> 32) & filter_mask;
+        const bool maybe = (filter[bit >> 5] >> (bit & 31)) & 1u;
+        uint32_t slot = (uint32_t)h & mask;
+        for (uint32_t probe = 0; maybe && probe <= mask; ++probe) {
             const uint64_t cur = keys[slot];
             if (cur == key) { found = vals[slot]; break; }
             if (cur == EMPTY_KEY) break;
@@ -92,12 +107,19 @@ int64_t table_capacity(int64_t n) {
     return cap;
 }
 
+int64_t filter_bits(int64_t n) {
+    int64_t bits = 4096;
+    while (bits < 16 * n) bits <<= 1;
+    return bits;
+}
+
 }  // namespace
 
 extern "C" size_t ptv3_kmap_workspace_bytes(int64_t n) {
     if (n < 0) return 0;
     const int64_t cap = table_capacity(n);
-    return ptv3_align256((size_t)cap * sizeof(uint64_t)) + ptv3_align256((size_t)cap * sizeof(int32_t));
+    return ptv3_align256((size_t)cap * sizeof(uint64_t)) + ptv3_align256((size_t)cap * sizeof(int32_t)) +
+           ptv3_align256((size_t)filter_bits(n) / 8);
 }
 
 extern "C" int ptv3_kmap_build(const int32_t* indices, int64_t n, int ks, int tap_major, int32_t* nbr,
@@ -111,17 +133,22 @@ extern "C" int ptv3_kmap_build(const int32_t* indices, int64_t n, int ks, int ta
     const int64_t cap = table_capacity(n);
     uint64_t* keys = (uint64_t*)workspace;
     int32_t* vals = (int32_t*)((char*)workspace + ptv3_align256((size_t)cap * sizeof(uint64_t)));
+    uint32_t* filter = (uint32_t*)((char*)vals + ptv3_align256((size_t)cap * sizeof(int32_t)));
+    const int64_t fbits = filter_bits(n);
+    const uint32_t filter_mask = (uint32_t)(fbits - 1);
     const uint32_t mask = (uint32_t)(cap - 1);
     const int taps = ks * ks * ks;
     hipLaunchKernelGGL(kmap_fill_kernel, dim3((unsigned)ptv3_ceil_div(cap, 256)), dim3(256), 0, stream,
-                       keys, cap);
+                       keys, cap, filter, fbits / 32);
     hipLaunchKernelGGL(kmap_insert_kernel, dim3((unsigned)ptv3_ceil_div(n, 256)), dim3(256), 0, stream,
-                       indices, n, keys, vals, mask);
+                       indices, n, keys, vals, mask, filter, filter_mask);
     if (tap_major)
         hipLaunchKernelGGL(kmap_lookup_kernel<true>, dim3((unsigned)ptv3_ceil_div(n * taps, 256)), dim3(256), 0,
-                           stream, indices, n, ks, taps, (const uint64_t*)keys, (const int32_t*)vals, mask, nbr);
+                           stream, indices, n, ks, taps, (const uint64_t*)keys, (const int32_t*)vals, mask,
+                           (const uint32_t*)filter, filter_mask, nbr);
     else
         hipLaunchKernelGGL(kmap_lookup_kernel<false>, dim3((unsigned)ptv3_ceil_div(n * taps, 256)), dim3(256), 0,
-                           stream, indices, n, ks, taps, (const uint64_t*)keys, (const int32_t*)vals, mask, nbr);
+                           stream, indices, n, ks, taps, (const uint64_t*)keys, (const int32_t*)vals, mask,
+                           (const uint32_t*)filter, filter_mask, nbr);
     PTV3_RETURN_LAUNCH();
 }
