@@ -112,7 +112,7 @@ template <typename T>
 __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
     const T* __restrict__ qkv, int channels, int heads, const int32_t* __restrict__ slot_src,
     const int32_t* __restrict__ slot_dst, const int32_t* __restrict__ cu_seqlens, int lds_keys,
-    float scale_log2e, T* __restrict__ out) {
+    float scale_log2e, T* __restrict__ out, int full_items, int split) {
     typedef typename Half<T>::v8 v8;
     extern __shared__ __align__(16) unsigned char smem[];
     // K tile: lds_keys rows of 32 B. V^T tile: 16 rows of (lds_keys*2 + pad) B. Then one float
@@ -122,7 +122,18 @@ __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
     unsigned char* vt_lds = smem + (size_t)lds_keys * 32;
     float* knorm_lds = (float*)(vt_lds + (size_t)HD * vt_stride);
 
-    const int wg = xcd_chunked_id(blockIdx.x, gridDim.x);
+    // The first `full_items` work-groups take one (sequence, head) each. The items left over
+    // after the last full round of resident work-groups are cut into `split` query ranges, one
+    // work-group each, so that the partial round at the end of the launch is short.
+    int wg, part = 0, parts = 1;
+    if ((int)blockIdx.x < full_items) {
+        wg = xcd_chunked_id(blockIdx.x, full_items);
+    } else {
+        const int r = blockIdx.x - full_items;
+        wg = full_items + r / split;
+        part = r % split;
+        parts = split;
+    }
     const int seq = wg / heads, head = wg % heads;
     const int s0 = cu_seqlens[seq];
     const int len = cu_seqlens[seq + 1] - s0;
@@ -171,7 +182,8 @@ __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
     const unsigned char* k_base = k_lds + col * 32 + hf * 16;
     const unsigned char* v_base = vt_lds + (size_t)(col & 15) * vt_stride + hf * 32;
 
-    for (int qt = wave; qt < n_qtiles; qt += ATT_WAVES) {
+    const int qt_lo = (int)((int64_t)part * n_qtiles / parts), qt_hi = (int)((int64_t)(part + 1) * n_qtiles / parts);
+    for (int qt = qt_lo + wave; qt < qt_hi; qt += ATT_WAVES) {
         const int qi = qt * 32 + col;   // my query inside the sequence
         int dst = -1;
         u32x4 qreg = {0, 0, 0, 0};
@@ -347,9 +359,31 @@ int launch_half(const void* qkv, int channels, int heads, const int32_t* slot_sr
         lds_allowed = lds;
     }
     const float scale_log2e = scale * 1.4426950408889634f;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(n_seq * heads)), dim3(ATT_THREADS), lds, stream,
+    // resident work-groups: two per CU (LDS-bound)
+    static int slots = 0;
+    if (slots == 0) {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        slots = 2 * cus;
+    }
+    // Items beyond the last full round of resident work-groups are cut into `split` query ranges
+    // (each re-stages K/V, about a tenth of an item): pick the split that makes the tail shortest.
+    const int64_t total = n_seq * heads;
+    const int64_t rem = total % slots;
+    int64_t full = total - rem, split = 1;
+    if (rem != 0) {
+        double best = 1.0;
+        for (int64_t sp = 2; sp <= 4; ++sp) {
+            const double cost = (double)((rem * sp + slots - 1) / slots) / (double)sp + 0.1;
+            if (cost < best - 1e-9) { best = cost; split = sp; }
+        }
+    }
+    if (split == 1) full = total;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(full + (total - full) * split)), dim3(ATT_THREADS), lds, stream,
                        (const T*)qkv, channels, heads, slot_src, slot_dst, cu_seqlens, lds_keys,
-                       scale_log2e, (T*)out);
+                       scale_log2e, (T*)out, (int)full, (int)split);
     PTV3_RETURN_LAUNCH();
 }
 

@@ -109,35 +109,83 @@ __global__ __launch_bounds__(256) void pool_gather_kernel(
 template <typename T> __device__ __forceinline__ float ld(const T* p) { return (float)*p; }
 template <typename T> __device__ __forceinline__ void st(T* p, float v) { *p = (T)v; }
 
-template <typename T>
+// V consecutive channels per thread (V * sizeof(T) = 16 bytes when the channel count allows)
+template <typename T, int V> struct Pack { T v[V]; };
+
+template <typename T, int V>
 __global__ __launch_bounds__(256) void segment_reduce_kernel(
     const T* __restrict__ src, int c, const int64_t* __restrict__ indices,
     const int64_t* __restrict__ idx_ptr, int64_t m, int op, T* __restrict__ out) {
+    const int groups = c / V;
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= m * c) return;
-    const int64_t s = e / c;
-    const int ch = (int)(e - s * c);
+    if (e >= m * groups) return;
+    const int64_t s = e / groups;
+    const int ch = (int)(e - s * groups) * V;
     const int64_t b = idx_ptr[s], t = idx_ptr[s + 1];
-    float acc = (op == 0) ? -INFINITY : (op == 3 ? INFINITY : 0.f);
+    float acc[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) acc[k] = (op == 0) ? -INFINITY : (op == 3 ? INFINITY : 0.f);
     for (int64_t j = b; j < t; ++j) {
-        const float v = ld(src + indices[j] * c + ch);
-        acc = (op == 0) ? fmaxf(acc, v) : (op == 3 ? fminf(acc, v) : acc + v);
+        const Pack<T, V> p = *(const Pack<T, V>*)(src + indices[j] * c + ch);
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            const float v = (float)p.v[k];
+            acc[k] = (op == 0) ? fmaxf(acc[k], v) : (op == 3 ? fminf(acc[k], v) : acc[k] + v);
+        }
     }
-    if (op == 1 && t > b) acc /= (float)(t - b);
-    if (t == b) acc = 0.f;
-    st(out + e, acc);
+    Pack<T, V> r;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        float v = acc[k];
+        if (op == 1 && t > b) v /= (float)(t - b);
+        if (t == b) v = 0.f;
+        r.v[k] = (T)v;
+    }
+    *(Pack<T, V>*)(out + s * c + ch) = r;
 }
 
-template <typename T>
+template <typename T, int V>
 __global__ __launch_bounds__(256) void unpool_add_kernel(const T* __restrict__ parent,
                                                          const T* __restrict__ child, int64_t n,
                                                          int c, const int64_t* __restrict__ cluster,
                                                          T* __restrict__ out) {
+    const int groups = c / V;
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= n * c) return;
-    const int64_t i = e / c;
-    const int ch = (int)(e - i * c);
-    st(out + e, ld(parent + e) + ld(child + cluster[i] * c + ch));
+    if (e >= n * groups) return;
+    const int64_t i = e / groups;
+    const int ch = (int)(e - i * groups) * V;
+    const Pack<T, V> a = *(const Pack<T, V>*)(parent + i * c + ch);
+    const Pack<T, V> b = *(const Pack<T, V>*)(child + cluster[i] * c + ch);
+    Pack<T, V> r;
+#pragma unroll
+    for (int k = 0; k < V; ++k) r.v[k] = (T)((float)a.v[k] + (float)b.v[k]);
+    *(Pack<T, V>*)(out + i * c + ch) = r;
+}
+
+template <typename T>
+void launch_segment_reduce(const void* src, int c, const int64_t* indices, const int64_t* idx_ptr, int64_t m,
+                           int op, void* out, hipStream_t stream) {
+    constexpr int V = 16 / sizeof(T);
+    if (c % V == 0) {
+        hipLaunchKernelGGL((segment_reduce_kernel<T, V>), dim3((unsigned)ptv3_ceil_div(m * (c / V), 256)), dim3(256), 0,
+                           stream, (const T*)src, c, indices, idx_ptr, m, op, (T*)out);
+    } else {
+        hipLaunchKernelGGL((segment_reduce_kernel<T, 1>), dim3((unsigned)ptv3_ceil_div(m * c, 256)), dim3(256), 0,
+                           stream, (const T*)src, c, indices, idx_ptr, m, op, (T*)out);
+    }
+}
+
+template <typename T>
+void launch_unpool_add(const void* parent, const void* child, int64_t n, int c, const int64_t* cluster, void* out,
+                       hipStream_t stream) {
+    constexpr int V = 16 / sizeof(T);
+    if (c % V == 0) {
+        hipLaunchKernelGGL((unpool_add_kernel<T, V>), dim3((unsigned)ptv3_ceil_div(n * (c / V), 256)), dim3(256), 0,
+                           stream, (const T*)parent, (const T*)child, n, c, cluster, (T*)out);
+    } else {
+        hipLaunchKernelGGL((unpool_add_kernel<T, 1>), dim3((unsigned)ptv3_ceil_div(n * c, 256)), dim3(256), 0, stream,
+                           (const T*)parent, (const T*)child, n, c, cluster, (T*)out);
+    }
 }
 
 }  // namespace
@@ -188,16 +236,9 @@ extern "C" int ptv3_segment_reduce(const void* src, int dtype, int64_t n, int c,
     if (m == 0) return PTV3_OK;
     if (!src || !indices || !idx_ptr || !out) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
-    const dim3 grid((unsigned)ptv3_ceil_div(m * c, 256)), block(256);
-    if (dtype == PTV3_F32)
-        hipLaunchKernelGGL(segment_reduce_kernel<float>, grid, block, 0, stream, (const float*)src, c,
-                           indices, idx_ptr, m, op, (float*)out);
-    else if (dtype == PTV3_F16)
-        hipLaunchKernelGGL(segment_reduce_kernel<_Float16>, grid, block, 0, stream, (const _Float16*)src,
-                           c, indices, idx_ptr, m, op, (_Float16*)out);
-    else
-        hipLaunchKernelGGL(segment_reduce_kernel<__bf16>, grid, block, 0, stream, (const __bf16*)src, c,
-                           indices, idx_ptr, m, op, (__bf16*)out);
+    if (dtype == PTV3_F32) launch_segment_reduce<float>(src, c, indices, idx_ptr, m, op, out, stream);
+    else if (dtype == PTV3_F16) launch_segment_reduce<_Float16>(src, c, indices, idx_ptr, m, op, out, stream);
+    else launch_segment_reduce<__bf16>(src, c, indices, idx_ptr, m, op, out, stream);
     PTV3_RETURN_LAUNCH();
 }
 
@@ -208,15 +249,8 @@ extern "C" int ptv3_unpool_add(const void* parent, const void* child, int dtype,
     if (n == 0) return PTV3_OK;
     if (!parent || !child || !cluster || !out) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
-    const dim3 grid((unsigned)ptv3_ceil_div(n * c, 256)), block(256);
-    if (dtype == PTV3_F32)
-        hipLaunchKernelGGL(unpool_add_kernel<float>, grid, block, 0, stream, (const float*)parent,
-                           (const float*)child, n, c, cluster, (float*)out);
-    else if (dtype == PTV3_F16)
-        hipLaunchKernelGGL(unpool_add_kernel<_Float16>, grid, block, 0, stream, (const _Float16*)parent,
-                           (const _Float16*)child, n, c, cluster, (_Float16*)out);
-    else
-        hipLaunchKernelGGL(unpool_add_kernel<__bf16>, grid, block, 0, stream, (const __bf16*)parent,
-                           (const __bf16*)child, n, c, cluster, (__bf16*)out);
+    if (dtype == PTV3_F32) launch_unpool_add<float>(parent, child, n, c, cluster, out, stream);
+    else if (dtype == PTV3_F16) launch_unpool_add<_Float16>(parent, child, n, c, cluster, out, stream);
+    else launch_unpool_add<__bf16>(parent, child, n, c, cluster, out, stream);
     PTV3_RETURN_LAUNCH();
 }

@@ -70,9 +70,10 @@ def room_voxels(n_voxels, seed, grid_size=0.02):
 
 
 def lidar_scene(seed, grid_size=0.05, beams=64, az_step_deg=0.2, max_range=75.0, n_boxes=30):
-    """One spinning-LiDAR sweep: `beams` elevations in [-25,+3] deg, azimuth step 0.2 deg,
-    rays cast against the ground plane z=-1.8 m and random boxes; returns past `max_range`
-    are dropped. Density falls off with range as for a real sweep."""
+    """One spinning-LiDAR sweep: `beams` elevations in [-25,+3] deg, azimuth step 0.2 deg
+    (115,200 rays), cast against the ground plane z=-1.8 m, random boxes (vehicles, buildings) and
+    a ring of walls near 60-70 m that catches the upper beams; returns past `max_range` are
+    dropped. Point density falls off with range as for a real sweep."""
     rng = np.random.default_rng(seed)
     elev = np.deg2rad(np.linspace(-25.0, 3.0, beams))
     az = np.deg2rad(np.arange(0.0, 360.0, az_step_deg))
@@ -81,17 +82,32 @@ def lidar_scene(seed, grid_size=0.05, beams=64, az_step_deg=0.2, max_range=75.0,
     t = np.full(len(d), np.inf)
     down = d[:, 2] < -1e-6
     t[down] = -1.8 / d[down, 2]
-    for _ in range(n_boxes):
-        c = np.array([rng.uniform(-60, 60), rng.uniform(-60, 60), 0.0])
-        if np.hypot(c[0], c[1]) < 4.0:
-            continue
-        half = np.array([rng.uniform(0.8, 4.0), rng.uniform(0.8, 4.0), rng.uniform(0.8, 2.5)])
-        lo, hi = c - half - np.array([0, 0, 1.8 - half[2]]), c + half - np.array([0, 0, 1.8 - half[2]])
+
+    def hit_box(lo, hi):
         with np.errstate(divide="ignore", invalid="ignore"):
             t0, t1 = lo / d, hi / d
         tn, tf = np.minimum(t0, t1).max(1), np.maximum(t0, t1).min(1)
-        hit = (tn <= tf) & (tn > 0)
-        t = np.where(hit & (tn < t), tn, t)
+        return np.where((tn <= tf) & (tn > 0), tn, np.inf)
+
+    boxes = []
+    for _ in range(n_boxes):
+        c = np.array([rng.uniform(-55, 55), rng.uniform(-55, 55)])
+        if np.hypot(c[0], c[1]) < 4.0:
+            continue
+        half = np.array([rng.uniform(0.8, 4.0), rng.uniform(0.8, 4.0)])
+        height = rng.uniform(1.5, 6.0)
+        boxes.append((np.array([c[0] - half[0], c[1] - half[1], -1.8]), np.array([c[0] + half[0], c[1] + half[1], -1.8 + height])))
+    # perimeter: four 12 m high walls at a random distance of 58-68 m
+    for axis, sign in ((0, 1), (0, -1), (1, 1), (1, -1)):
+        dist = rng.uniform(58, 68)
+        lo, hi = np.array([-70.0, -70.0, -1.8]), np.array([70.0, 70.0, 10.2])
+        if sign > 0:
+            lo[axis], hi[axis] = dist, dist + 1.0
+        else:
+            lo[axis], hi[axis] = -dist - 1.0, -dist
+        boxes.append((lo, hi))
+    for lo, hi in boxes:
+        t = np.minimum(t, hit_box(lo, hi))
     ok = t < max_range
     pts = d[ok] * t[ok, None] + rng.normal(0, 0.01, size=(int(ok.sum()), 3))
     g, keep = voxelize_unique(pts, grid_size)
