@@ -163,6 +163,15 @@ int ptv3_layer_norm(const void *x, const void *res, const void *gamma, const voi
                     const void *gamma2, const void *beta2, const void *shift, int dtype, int64_t n,
                     int c, float eps, int mode, void *out0, void *out1, void *stream);
 
+/* Inference-mode nn.BatchNorm1d (model.py:848) and the nn.GELU that follows it at model.py:776-779,
+ * :707-710 and :729-735 in one pass: out = act((x - mean) * rsqrt(var + eps) * gamma + beta) per
+ * channel; act 0 = none, 1 = exact GELU. x, out (n,c) of dtype; running_mean/var (c,) float32 when
+ * stats_f32 != 0, else of dtype (a module cast with .half()); gamma, beta (c,) of dtype or NULL.
+ * c % 8 == 0. */
+int ptv3_bn_act(const void *x, const void *running_mean, const void *running_var, int stats_f32,
+                const void *gamma, const void *beta, int dtype, int64_t n, int c, float eps, int act,
+                void *out, void *stream);
+
 /* MLP of a block plus its residual, model.py:510-516 and :602, in one kernel:
  * out = resid + fc2(GELU(fc1(x))), exact (erf) GELU, intermediates rounded to dtype where the
  * separate layers would have stored them. x, resid, out (n, channels); w1 (hidden, channels),

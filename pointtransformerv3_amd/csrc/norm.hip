@@ -154,6 +154,45 @@ __global__ __launch_bounds__(256) void layer_norm_generic_kernel(
     }
 }
 
+// Inference-mode BatchNorm1d followed (optionally) by exact GELU: y = act((x - mean) * rstd * gamma
+// + beta), per channel, 8 channels per thread. The normalised value is rounded to the storage type
+// before the activation, as two separate layers would round it.
+__device__ __forceinline__ float gelu_exact(float x) {
+    // 0.5 x (1 + erf(x / sqrt 2)); erf by Abramowitz-Stegun 7.1.26, |error| < 1.5e-7
+    const float z = fabsf(x) * 0.70710678118654752f;
+    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
+    float p = fmaf(1.061405429f, t, -1.453152027f);
+    p = fmaf(p, t, 1.421413741f);
+    p = fmaf(p, t, -0.284496736f);
+    p = fmaf(p, t, 0.254829592f);
+    const float e = __builtin_amdgcn_exp2f(-z * z * 1.4426950408889634f);
+    const float erf_abs = fmaf(-p * t, e, 1.0f);
+    const float half_x = 0.5f * x;
+    return fmaf(copysignf(erf_abs, x), half_x, half_x);
+}
+
+template <typename T, typename S>
+__global__ __launch_bounds__(256) void bn_act_kernel(const T* __restrict__ x, const S* __restrict__ mean,
+                                                     const S* __restrict__ var, const T* __restrict__ gamma,
+                                                     const T* __restrict__ beta, float eps, int act, int64_t n,
+                                                     int c, T* __restrict__ out) {
+    const int groups = c / 8;
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n * groups) return;
+    const int ch = (int)(e % groups) * 8;
+    float v[8], g[8], b[8];
+    load8(x + e * 8, v);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { g[i] = gamma ? (float)gamma[ch + i] : 1.f; b[i] = beta ? (float)beta[ch + i] : 0.f; }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float rstd = rsqrtf((float)var[ch + i] + eps);
+        float y = round_to<T>((v[i] - (float)mean[ch + i]) * rstd * g[i] + b[i]);
+        v[i] = act == 1 ? gelu_exact(y) : y;
+    }
+    store8(out + e * 8, v);
+}
+
 template <typename T, int MODE>
 void launch(const void* x, const void* res, const void* gamma, const void* beta, const void* gamma2,
             const void* beta2, const void* shift, int64_t n, int c, float eps, void* out0, void* out1,
@@ -217,5 +256,34 @@ extern "C" int ptv3_layer_norm(const void* x, const void* res, const void* gamma
         launch_mode<_Float16>(mode, x, res, gamma, beta, gamma2, beta2, shift, n, c, eps, out0, out1, stream);
     else
         launch_mode<__bf16>(mode, x, res, gamma, beta, gamma2, beta2, shift, n, c, eps, out0, out1, stream);
+    PTV3_RETURN_LAUNCH();
+}
+
+template <typename T, typename S>
+void launch_bn_act(const void* x, const void* mean, const void* var, const void* gamma, const void* beta, float eps,
+                   int act, int64_t n, int c, void* out, hipStream_t stream) {
+    hipLaunchKernelGGL((bn_act_kernel<T, S>), dim3((unsigned)ptv3_ceil_div(n * (c / 8), 256)), dim3(256), 0, stream,
+                       (const T*)x, (const S*)mean, (const S*)var, (const T*)gamma, (const T*)beta, eps, act, n, c,
+                       (T*)out);
+}
+
+extern "C" int ptv3_bn_act(const void* x, const void* running_mean, const void* running_var, int stats_f32,
+                           const void* gamma, const void* beta, int dtype, int64_t n, int c, float eps, int act,
+                           void* out, void* stream_) {
+    if (n < 0 || c < 1 || act < 0 || act > 1) return PTV3_EINVAL;
+    if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
+    if (c % 8 != 0) return PTV3_ESHAPE;
+    if (n == 0) return PTV3_OK;
+    if (!x || !running_mean || !running_var || !out) return PTV3_EINVAL;
+    hipStream_t stream = (hipStream_t)stream_;
+#define PTV3_BN(T)                                                                                          \
+    do {                                                                                                    \
+        if (stats_f32) launch_bn_act<T, float>(x, running_mean, running_var, gamma, beta, eps, act, n, c, out, stream); \
+        else launch_bn_act<T, T>(x, running_mean, running_var, gamma, beta, eps, act, n, c, out, stream);   \
+    } while (0)
+    if (dtype == PTV3_F32) PTV3_BN(float);
+    else if (dtype == PTV3_F16) PTV3_BN(_Float16);
+    else PTV3_BN(__bf16);
+#undef PTV3_BN
     PTV3_RETURN_LAUNCH();
 }

@@ -41,6 +41,16 @@ class LayerNorm(nn.LayerNorm):
         return ops.layer_norm(x, self.weight, self.bias, self.eps)
 
 
+def _fusable_bn(module, feat):
+    """Inference-mode BatchNorm1d over (N, C) GPU features that the one-pass kernel covers."""
+    return (type(module) is nn.BatchNorm1d and not module.training and module.track_running_stats
+            and module.running_mean is not None and feat.is_cuda and feat.dim() == 2 and feat.shape[1] % 8 == 0)
+
+
+def _exact_gelu(module):
+    return type(module) is nn.GELU and module.approximate == "none"
+
+
 class PointModule(nn.Module):
     """Marker base class: PointSequential hands the whole Point to subclasses (model.py:177-183)."""
 
@@ -79,7 +89,21 @@ class PointSequential(PointModule):
         self.add_module(name, module)
 
     def forward(self, input):
-        for module in self._modules.values():
+        modules = list(self._modules.values())
+        skip = False
+        for i, module in enumerate(modules):
+            if skip:   # activation already applied together with the normalisation before it
+                skip = False
+                continue
+            nxt = modules[i + 1] if i + 1 < len(modules) else None
+            if isinstance(input, Point) and _fusable_bn(module, input.feat):
+                with_act = _exact_gelu(nxt)
+                input.feat = ops.bn_act(input.feat, module.running_mean, module.running_var, module.weight,
+                                        module.bias, module.eps, with_act)
+                if "sparse_conv_feat" in input:
+                    input.sparse_conv_feat = input.sparse_conv_feat.replace_feature(input.feat)
+                skip = with_act
+                continue
             if isinstance(module, PointModule):
                 input = module(input)
             elif is_spconv_module(module):
@@ -375,10 +399,16 @@ class SerializedPooling(PointModule):
         # max(x >> d) == max(x) >> d: the pooled grid extent needs no reduction and no sync
         fields["_grid_max_host"] = [v >> pooling_depth for v in point.grid_max_host()]
         pooled = Point(fields)
-        if self.norm is not None:
-            pooled = self.norm(pooled)
-        if self.act is not None:
-            pooled = self.act(pooled)
+        norm = self.norm[0] if self.norm is not None and len(self.norm) == 1 else None
+        act = self.act[0] if self.act is not None and len(self.act) == 1 else None
+        if norm is not None and _fusable_bn(norm, pooled.feat) and _exact_gelu(act):
+            pooled.feat = ops.bn_act(pooled.feat, norm.running_mean, norm.running_var, norm.weight, norm.bias,
+                                     norm.eps, True)
+        else:
+            if self.norm is not None:
+                pooled = self.norm(pooled)
+            if self.act is not None:
+                pooled = self.act(pooled)
         pooled.sparsify()
         return pooled
 

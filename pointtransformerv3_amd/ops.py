@@ -353,3 +353,23 @@ def mlp_fused(x, resid, w1, b1, w2, b2):
     _lib.check(lib.ptv3_mlp_fused(_ptr(x), _ptr(resid), _ptr(w1c), _ptr(b1c), _ptr(w2c), _ptr(b2c), _dtype_code(x),
                                   n, c, w1c.shape[0], _ptr(out), _stream()), "ptv3_mlp_fused")
     return out
+
+
+def bn_act(x, running_mean, running_var, weight, bias, eps, gelu):
+    """Inference-mode BatchNorm1d, optionally followed by exact GELU, in one pass. The running
+    statistics may be float32 or of x's dtype."""
+    _dev(x, running_mean, running_var, weight, bias)
+    lib = _lib.load()
+    x = x.contiguous()
+    n, c = x.shape
+    dt = x.dtype
+    stats_f32 = running_mean.dtype == torch.float32
+    if not stats_f32 and running_mean.dtype != dt:
+        running_mean, running_var, stats_f32 = running_mean.float(), running_var.float(), True
+    w = None if weight is None else weight.to(dt).contiguous()
+    b = None if bias is None else bias.to(dt).contiguous()
+    out = torch.empty_like(x)
+    _lib.check(lib.ptv3_bn_act(_ptr(x), _ptr(running_mean.contiguous()), _ptr(running_var.contiguous()),
+                               int(stats_f32), _ptr(w), _ptr(b), _dtype_code(x), n, c, float(eps), int(bool(gelu)),
+                               _ptr(out), _stream()), "ptv3_bn_act")
+    return out

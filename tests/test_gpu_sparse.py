@@ -204,3 +204,22 @@ def test_mlp_fused_parity(dtype, c, n):
     want = r.float() + F.linear(h, w2.float(), b2.float())
     got = ops().mlp_fused(*(t.to(DEV) for t in (x, r, w1, b1, w2, b2)))
     assert got.dtype == dtype and rel_err(got, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("half_stats", [False, True])
+def test_bn_act_parity(dtype, half_stats):
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(3)
+    n, c = 4097, 64
+    x = (torch.randn(n, c, generator=g) * 2).to(dtype)
+    mean, var = torch.randn(c, generator=g), torch.rand(c, generator=g) + 0.5
+    w, b = (torch.rand(c, generator=g) + 0.5).to(dtype), torch.randn(c, generator=g).to(dtype)
+    sd = dtype if half_stats else torch.float32
+    mean, var = mean.to(sd), var.to(sd)
+    y = F.batch_norm(x.float(), mean.float(), var.float(), w.float(), b.float(), False, 0.0, 1e-3)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    o = ops()
+    dv = lambda t: t.to(DEV)
+    assert rel_err(o.bn_act(dv(x), dv(mean), dv(var), dv(w), dv(b), 1e-3, False), y) < tol
+    assert rel_err(o.bn_act(dv(x), dv(mean), dv(var), dv(w), dv(b), 1e-3, True), F.gelu(y.to(dtype).float())) < tol
