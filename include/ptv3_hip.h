@@ -142,6 +142,16 @@ int ptv3_pool_gather(const int64_t *code, int64_t n, int k, int shift, const int
                      int64_t *code_out, int32_t *grid_coord_out, int64_t *batch_out,
                      void *stream);
 
+/* model.py:667-674 without a sort: the pooled order of every curve is the sequence of distinct
+ * clusters met when walking the parent points along that curve (order (k,n): the parent's
+ * serialized_order; cluster (n,): pooling_inverse; m clusters). Writes order_out, inverse_out
+ * (k,m) int64, identical to argsort of the pooled codes and its inverse. Requires what the
+ * reference's pooling relies on too: a point's code shifted right is its cluster's code. */
+size_t ptv3_pool_orders_workspace_bytes(int64_t n, int k);
+int ptv3_pool_orders(const int64_t *order, const int64_t *cluster, int64_t n, int k, int64_t m,
+                     int64_t *order_out, int64_t *inverse_out, void *workspace,
+                     size_t workspace_bytes, void *stream);
+
 /* torch_scatter.segment_csr call sites model.py:684-689: reduce src[indices[j]] over
  * j in [idx_ptr[s], idx_ptr[s+1]). op 0 = max, 1 = mean, 2 = sum, 3 = min.
  * src (n,c) of dtype, out (m,c) of dtype. */

@@ -90,6 +90,60 @@ __global__ __launch_bounds__(PB) void cluster_assign_kernel(
     if (i == n - 1) idx_ptr[cid + 1] = n;
 }
 
+// ---- pooled serialization orders without sorting.
+// Walking the parent points along any of their serialization orders visits the clusters of the
+// coarser level as runs (a point's code shifted right by 3 bits per pooled level is its cluster's
+// code on the same curve), in ascending order of that cluster code. The sequence of run heads is
+// therefore the pooled order of that curve: flags + scan per row, all rows in one launch.
+__device__ __forceinline__ bool order_run_start(const int64_t* __restrict__ order_row,
+                                                const int64_t* __restrict__ cluster, int64_t i) {
+    if (i == 0) return true;
+    return cluster[order_row[i]] != cluster[order_row[i - 1]];
+}
+
+__global__ __launch_bounds__(PB) void order_count_kernel(const int64_t* __restrict__ order,
+                                                         const int64_t* __restrict__ cluster, int64_t n,
+                                                         uint32_t* __restrict__ block_cnt) {
+    const int64_t i = (int64_t)blockIdx.x * PB + threadIdx.x;
+    const int64_t* row = order + (int64_t)blockIdx.y * n;
+    const uint32_t f = (i < n && order_run_start(row, cluster, i)) ? 1u : 0u;
+    uint32_t total;
+    block_inclusive_scan(f, &total);
+    if (threadIdx.x == 0) block_cnt[(int64_t)blockIdx.y * gridDim.x + blockIdx.x] = total;
+}
+
+// one block per row: exclusive scan of the row's block counts in place
+__global__ __launch_bounds__(PB) void order_scan_kernel(uint32_t* __restrict__ block_cnt, int64_t blocks) {
+    uint32_t* cnt = block_cnt + (int64_t)blockIdx.x * blocks;
+    uint32_t carry = 0;
+    for (int64_t b0 = 0; b0 < blocks; b0 += PB) {
+        const int64_t b = b0 + threadIdx.x;
+        const uint32_t v = b < blocks ? cnt[b] : 0u;
+        uint32_t total;
+        const uint32_t inc = block_inclusive_scan(v, &total);
+        if (b < blocks) cnt[b] = carry + inc - v;
+        carry += total;
+    }
+}
+
+__global__ __launch_bounds__(PB) void order_assign_kernel(const int64_t* __restrict__ order,
+                                                          const int64_t* __restrict__ cluster, int64_t n,
+                                                          int64_t m, const uint32_t* __restrict__ block_base,
+                                                          int64_t* __restrict__ order_out,
+                                                          int64_t* __restrict__ inverse_out) {
+    const int64_t i = (int64_t)blockIdx.x * PB + threadIdx.x;
+    const int64_t* row = order + (int64_t)blockIdx.y * n;
+    const bool f = i < n && order_run_start(row, cluster, i);
+    uint32_t total;
+    const uint32_t inc = block_inclusive_scan(f ? 1u : 0u, &total);
+    if (!f) return;
+    const int64_t pos = (int64_t)block_base[(int64_t)blockIdx.y * gridDim.x + blockIdx.x] + inc - 1;
+    if (pos >= m) return;   // cannot happen when the codes form a hierarchy; keeps writes in bounds
+    const int64_t c = cluster[row[i]];
+    order_out[(int64_t)blockIdx.y * m + pos] = c;
+    inverse_out[(int64_t)blockIdx.y * m + c] = pos;
+}
+
 __global__ __launch_bounds__(256) void pool_gather_kernel(
     const int64_t* __restrict__ code, int64_t n, int k, int shift,
     const int32_t* __restrict__ grid_coord, int pool_depth, const int64_t* __restrict__ batch,
@@ -252,5 +306,27 @@ extern "C" int ptv3_unpool_add(const void* parent, const void* child, int dtype,
     if (dtype == PTV3_F32) launch_unpool_add<float>(parent, child, n, c, cluster, out, stream);
     else if (dtype == PTV3_F16) launch_unpool_add<_Float16>(parent, child, n, c, cluster, out, stream);
     else launch_unpool_add<__bf16>(parent, child, n, c, cluster, out, stream);
+    PTV3_RETURN_LAUNCH();
+}
+
+extern "C" size_t ptv3_pool_orders_workspace_bytes(int64_t n, int k) {
+    if (n < 0 || k < 1) return 0;
+    return ptv3_align256((size_t)k * ptv3_ceil_div(n > 0 ? n : 1, PB) * sizeof(uint32_t));
+}
+
+extern "C" int ptv3_pool_orders(const int64_t* order, const int64_t* cluster, int64_t n, int k, int64_t m,
+                                int64_t* order_out, int64_t* inverse_out, void* workspace,
+                                size_t workspace_bytes, void* stream_) {
+    if (n < 1 || n >= (1ll << 31) || k < 1 || k > 65535 || m < 1 || m > n) return PTV3_EINVAL;
+    if (!order || !cluster || !order_out || !inverse_out || !workspace) return PTV3_EINVAL;
+    if (workspace_bytes < ptv3_pool_orders_workspace_bytes(n, k)) return PTV3_EWORKSPACE;
+    hipStream_t stream = (hipStream_t)stream_;
+    const int64_t blocks = ptv3_ceil_div(n, PB);
+    uint32_t* block_cnt = (uint32_t*)workspace;
+    const dim3 grid((unsigned)blocks, (unsigned)k);
+    hipLaunchKernelGGL(order_count_kernel, grid, dim3(PB), 0, stream, order, cluster, n, block_cnt);
+    hipLaunchKernelGGL(order_scan_kernel, dim3((unsigned)k), dim3(PB), 0, stream, block_cnt, blocks);
+    hipLaunchKernelGGL(order_assign_kernel, grid, dim3(PB), 0, stream, order, cluster, n, m,
+                       (const uint32_t*)block_cnt, order_out, inverse_out);
     PTV3_RETURN_LAUNCH();
 }

@@ -38,41 +38,54 @@ __global__ __launch_bounds__(SORT_THREADS) void tile_hist_kernel(
     tile_hist[((int64_t)row * tiles + tile) * RADIX + tid] = hist[tid];
 }
 
-// One block per row. Thread d owns digit d: exclusive scan over the tiles (loads issued 16 at
-// a time so they overlap), then a block-wide exclusive scan over the digit totals; the digit
-// base is folded back in.
-__global__ __launch_bounds__(RADIX) void tile_scan_kernel(uint32_t* __restrict__ tile_hist,
-                                                          int tiles) {
+// One block of 1024 threads per row: thread (q, d) owns digit d over the q-th quarter of the
+// tiles. Quarter sums -> digit totals -> exclusive scan over digits; then every thread rescans
+// its quarter once, writing the final start of each (tile, digit) run.
+constexpr int SCAN_Q = 4;
+__global__ __launch_bounds__(RADIX * SCAN_Q) void tile_scan_kernel(uint32_t* __restrict__ tile_hist,
+                                                                   int tiles) {
+    __shared__ uint32_t part[SCAN_Q][RADIX];
     __shared__ uint32_t total[RADIX];
-    constexpr int CH = 16;
-    const int row = blockIdx.x, d = threadIdx.x;
+    constexpr int CH = 8;
+    const int row = blockIdx.x, d = threadIdx.x % RADIX, q = threadIdx.x / RADIX;
+    const int per = (tiles + SCAN_Q - 1) / SCAN_Q;
+    const int t_lo = min(q * per, tiles), t_hi = min(t_lo + per, tiles);
     uint32_t* h = tile_hist + (int64_t)row * tiles * RADIX + d;
-    uint32_t run = 0;
-    for (int t0 = 0; t0 < tiles; t0 += CH) {
+    uint32_t sum = 0;
+    for (int t0 = t_lo; t0 < t_hi; t0 += CH) {
         uint32_t c[CH];
 #pragma unroll
-        for (int j = 0; j < CH; ++j) c[j] = (t0 + j < tiles) ? h[(int64_t)(t0 + j) * RADIX] : 0u;
+        for (int j = 0; j < CH; ++j) c[j] = (t0 + j < t_hi) ? h[(int64_t)(t0 + j) * RADIX] : 0u;
+#pragma unroll
+        for (int j = 0; j < CH; ++j) sum += c[j];
+    }
+    part[q][d] = sum;
+    __syncthreads();
+    uint32_t qbase = 0, dtotal = 0;
+#pragma unroll
+    for (int k = 0; k < SCAN_Q; ++k) {
+        const uint32_t v = part[k][d];
+        if (k < q) qbase += v;
+        dtotal += v;
+    }
+    if (q == 0) total[d] = dtotal;
+    __syncthreads();
+    // Hillis-Steele inclusive scan over the 256 digit totals (first 256 threads; all hit the barriers)
+    for (int off = 1; off < RADIX; off <<= 1) {
+        const uint32_t v = (q == 0 && d >= off) ? total[d - off] : 0u;
+        __syncthreads();
+        if (q == 0) total[d] += v;
+        __syncthreads();
+    }
+    uint32_t run = total[d] - dtotal + qbase;   // digit base + tiles of earlier quarters
+    for (int t0 = t_lo; t0 < t_hi; t0 += CH) {
+        uint32_t c[CH];
+#pragma unroll
+        for (int j = 0; j < CH; ++j) c[j] = (t0 + j < t_hi) ? h[(int64_t)(t0 + j) * RADIX] : 0u;
 #pragma unroll
         for (int j = 0; j < CH; ++j) {
-            if (t0 + j < tiles) h[(int64_t)(t0 + j) * RADIX] = run;
+            if (t0 + j < t_hi) h[(int64_t)(t0 + j) * RADIX] = run;
             run += c[j];
-        }
-    }
-    total[d] = run;
-    __syncthreads();
-    // Hillis-Steele inclusive scan over 256 digit totals
-    for (int off = 1; off < RADIX; off <<= 1) {
-        const uint32_t v = (d >= off) ? total[d - off] : 0u;
-        __syncthreads();
-        total[d] += v;
-        __syncthreads();
-    }
-    const uint32_t dbase = total[d] - run;
-    if (dbase != 0) {
-        for (int t0 = 0; t0 < tiles; t0 += CH) {
-#pragma unroll
-            for (int j = 0; j < CH; ++j)
-                if (t0 + j < tiles) h[(int64_t)(t0 + j) * RADIX] += dbase;
         }
     }
 }
@@ -199,7 +212,7 @@ extern "C" int ptv3_argsort(const int64_t* code, int64_t n, int k, int key_bits,
         int64_t* kout = w.keys[p & 1];
         int32_t* iout = w.idx[p & 1];
         hipLaunchKernelGGL(tile_hist_kernel, grid, block, 0, stream, kin, n, shift, w.tile_hist, tiles);
-        hipLaunchKernelGGL(tile_scan_kernel, dim3((unsigned)k), dim3(RADIX), 0, stream, w.tile_hist, tiles);
+        hipLaunchKernelGGL(tile_scan_kernel, dim3((unsigned)k), dim3(RADIX * SCAN_Q), 0, stream, w.tile_hist, tiles);
 #define PTV3_SCATTER(F, L)                                                                    \
     hipLaunchKernelGGL((scatter_kernel<F, L>), grid, block, 0, stream, kin, iin, n, shift,    \
                        (const uint32_t*)w.tile_hist, tiles, kout, iout, order, inverse)

@@ -373,8 +373,9 @@ class SerializedPooling(PointModule):
         cluster, idx_ptr, head, m = ops.pool_clusters(point.serialized_code[0], indices, shift)
         code, grid_coord, batch = ops.pool_gather(point.serialized_code, shift, point.grid_coord,
                                                   pooling_depth, point.batch, head)
-        n_scenes = len(point.offset_host())
-        order, inverse = ops.argsort_rows(code, 3 * depth + max(1, (n_scenes - 1).bit_length()))
+        # pooled orders: the distinct clusters met when walking the parent along each curve (same
+        # result as argsort of the pooled codes, model.py:667-674, without sorting)
+        order, inverse = ops.pool_orders(point.serialized_order, cluster, m)
         if self.shuffle_orders:
             perm = torch.randperm(code.shape[0]).to(code.device)   # CPU generator (model.py:677)
             code, order, inverse = code[perm], order[perm], inverse[perm]

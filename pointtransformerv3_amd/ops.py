@@ -283,6 +283,23 @@ def pool_gather(code, shift, grid_coord, pool_depth, batch, head):
     return code_out, gc_out, b_out
 
 
+def pool_orders(order, cluster, m):
+    """Pooled serialization orders and inverses (k,M) from the parent's orders (k,N) and the
+    cluster of every parent point — no sort (see ptv3_pool_orders)."""
+    _dev(order, cluster)
+    lib = _lib.load()
+    order = order.contiguous()
+    k, n = order.shape
+    dev = order.device
+    order_out = torch.empty((k, m), dtype=torch.int64, device=dev)
+    inverse_out = torch.empty((k, m), dtype=torch.int64, device=dev)
+    nbytes = lib.ptv3_pool_orders_workspace_bytes(n, k)
+    ws = _ws(nbytes, dev)
+    _lib.check(lib.ptv3_pool_orders(_ptr(order), _ptr(cluster.contiguous()), n, k, int(m), _ptr(order_out),
+                                    _ptr(inverse_out), _ptr(ws), nbytes, _stream()), "ptv3_pool_orders")
+    return order_out, inverse_out
+
+
 def segment_reduce(src, indices, idx_ptr, reduce="max"):
     """reduce(src[indices[idx_ptr[s]:idx_ptr[s+1]]]) per segment."""
     _dev(src, indices, idx_ptr)

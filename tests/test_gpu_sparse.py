@@ -223,3 +223,23 @@ def test_bn_act_parity(dtype, half_stats):
     dv = lambda t: t.to(DEV)
     assert rel_err(o.bn_act(dv(x), dv(mean), dv(var), dv(w), dv(b), 1e-3, False), y) < tol
     assert rel_err(o.bn_act(dv(x), dv(mean), dv(var), dv(w), dv(b), 1e-3, True), F.gelu(y.to(dtype).float())) < tol
+
+
+@pytest.mark.parametrize("n,extent,nb", [(1, 4, 1), (3000, 16, 2), (60_000, 64, 3)])
+def test_pool_orders_equal_argsort_of_pooled_codes(n, extent, nb):
+    rng = np.random.default_rng(n)
+    idx, g, batch, offset = _indices(rng, n, extent, nb)
+    depth, code, order, inverse = OS.serialize(g, batch)
+    want = OI.pool_clusters(code, g, batch, 1)
+    o = ops()
+    # also with the rows in another order than (z, z-trans, hilbert, hilbert-trans)
+    for perm in ([0, 1, 2, 3], [2, 0, 3, 1]):
+        c, od = code[perm], order[perm]
+        w = OI.pool_clusters(c, g, batch, 1)
+        cluster, idx_ptr, head, m = o.pool_clusters(to_dev(c[0]), to_dev(od[0]), 3)
+        po, pi = o.pool_orders(to_dev(od), cluster, m)
+        assert np.array_equal(po.cpu().numpy(), w["order"]) and np.array_equal(pi.cpu().numpy(), w["inverse"])
+        pc, _, _ = o.pool_gather(to_dev(c), 3, to_dev(g), 1, to_dev(batch), head)
+        so, si = o.argsort_rows(pc, 3 * (depth - 1) + 2)
+        assert torch.equal(so, po) and torch.equal(si, pi)
+    assert m == len(want["counts"])
