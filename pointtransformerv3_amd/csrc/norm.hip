@@ -180,14 +180,18 @@ __global__ __launch_bounds__(256) void bn_act_kernel(const T* __restrict__ x, co
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= n * groups) return;
     const int ch = (int)(e % groups) * 8;
-    float v[8], g[8], b[8];
+    float v[8], g[8], b[8], mu[8], va[8];
     load8(x + e * 8, v);
+    load8(mean + ch, mu);
+    load8(var + ch, va);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { g[i] = gamma ? (float)gamma[ch + i] : 1.f; b[i] = beta ? (float)beta[ch + i] : 0.f; }
+    for (int i = 0; i < 8; ++i) { g[i] = 1.f; b[i] = 0.f; }
+    if (gamma) load8(gamma + ch, g);
+    if (beta) load8(beta + ch, b);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        const float rstd = rsqrtf((float)var[ch + i] + eps);
-        float y = round_to<T>((v[i] - (float)mean[ch + i]) * rstd * g[i] + b[i]);
+        const float rstd = rsqrtf(va[i] + eps);
+        float y = round_to<T>((v[i] - mu[i]) * rstd * g[i] + b[i]);
         v[i] = act == 1 ? gelu_exact(y) : y;
     }
     store8(out + e * 8, v);
