@@ -191,6 +191,31 @@ int ptv3_mlp_fused(const void *x, const void *resid, const void *w1, const void 
                    const void *b2, int dtype, int64_t n, int channels, int hidden, void *out,
                    void *stream);
 
+/* Head of a block for thin channels, model.py:541-545, :587-589, :592-593 and :450 in one kernel:
+ *   feat = shortcut + LayerNorm_cpe(conv @ w_cpe^T + b_cpe)
+ *   qkv  = LayerNorm_1(feat) @ w_qkv^T + b_qkv
+ * (cpe.1, cpe.2, the residual, norm1 and attn.qkv), intermediates rounded to dtype where the
+ * separate layers would have stored them. conv, shortcut, feat (n, channels); qkv (n, 3*channels);
+ * w_cpe (channels, channels); w_qkv (3*channels, channels); biases and LayerNorm parameters of
+ * dtype, NULL = 0 (bias, beta) or 1 (gamma). fp16/bf16, channels 32 or 64 (PTV3_ESHAPE otherwise:
+ * use the separate layers). */
+int ptv3_block_head_fused(const void *conv, const void *shortcut, const void *w_cpe, const void *b_cpe,
+                          const void *ln_cpe_gamma, const void *ln_cpe_beta, float ln_cpe_eps,
+                          const void *ln1_gamma, const void *ln1_beta, float ln1_eps, const void *w_qkv,
+                          const void *b_qkv, int dtype, int64_t n, int channels, void *feat, void *qkv,
+                          void *stream);
+
+/* Tail of a block for thin channels, model.py:485-487, :594-595 and :599-602 in one kernel:
+ *   feat = shortcut + (attn @ w_proj^T + b_proj)
+ *   out  = feat + fc2(GELU(fc1(LayerNorm_2(feat))))
+ * (attn.proj, the residual, norm2, the MLP and its residual; exact GELU), rounded like the separate
+ * layers. attn, shortcut, out (n, channels); w_proj (channels, channels); w1 (hidden, channels);
+ * w2 (channels, hidden); fp16/bf16, channels 32 or 64, hidden = 4 * channels. */
+int ptv3_block_tail_fused(const void *attn, const void *shortcut, const void *w_proj, const void *b_proj,
+                          const void *ln2_gamma, const void *ln2_beta, float ln2_eps, const void *w1,
+                          const void *b1, const void *w2, const void *b2, int dtype, int64_t n,
+                          int channels, int hidden, void *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,67 @@
+// Shared pieces of the row-tile kernels (fused MLP, fused block head / tail): a wave owns 32 rows,
+// products are taken transposed with v_mfma_f32_32x32x16 so that every lane owns one row.
+#pragma once
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+
+#include "common.h"
+
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <typename T> struct H16;
+template <> struct H16<_Float16> {
+    typedef f16x8 v8;
+    static __device__ __forceinline__ f32x16 mfma(v8 a, v8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+        f32x2 f = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
+    }
+    static __device__ __forceinline__ float round(float v) { return (float)(_Float16)v; }
+    static __device__ __forceinline__ float lo(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[0]; }
+    static __device__ __forceinline__ float hi(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[1]; }
+};
+template <> struct H16<__bf16> {
+    typedef bf16x8 v8;
+    static __device__ __forceinline__ f32x16 mfma(v8 a, v8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+        f32x2 f = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+    }
+    static __device__ __forceinline__ float round(float v) { return (float)(__bf16)v; }
+    static __device__ __forceinline__ float lo(uint32_t w) { return (float)__builtin_bit_cast(bf16x2, w)[0]; }
+    static __device__ __forceinline__ float hi(uint32_t w) { return (float)__builtin_bit_cast(bf16x2, w)[1]; }
+};
+
+// position of hidden unit kk (0..31) of a 32-block in W2's LDS row: registers 0..15 of a lane of
+// half h hold rows 8*(v/4) + 4*h + v%4 of the first product
+__device__ __forceinline__ int perm32(int kk) { return ((kk >> 2) & 1) * 16 + (kk >> 3) * 4 + (kk & 3); }
+
+__device__ __forceinline__ float gelu_erf(float x) {
+    // 0.5 x (1 + erf(x / sqrt 2)), erf(z) = sign(z) (1 - poly(t) exp(-z^2)), t = 1 / (1 + p |z|)
+    const float z = fabsf(x) * 0.70710678118654752f;
+    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
+    float p = fmaf(1.061405429f, t, -1.453152027f);
+    p = fmaf(p, t, 1.421413741f);
+    p = fmaf(p, t, -0.284496736f);
+    p = fmaf(p, t, 0.254829592f);
+    const float e = __builtin_amdgcn_exp2f(-z * z * 1.4426950408889634f);
+    const float erf_abs = fmaf(-p * t, e, 1.0f);
+    const float half_x = 0.5f * x;
+    return fmaf(copysignf(erf_abs, x), half_x, half_x);
+}
+
+}  // namespace

@@ -209,21 +209,23 @@ class SerializedAttention(PointModule):
                                         point.serialized_inverse[self.order_index], pad, unpad)
         return point[key]
 
-    def forward(self, point):
+    def attend(self, point, qkv):
+        """softmax(q k^T * scale) v inside the patches of this layer's order, for packed
+        qkv (N, 3C) in point order; returns (N, C) in point order (model.py:452-484)."""
         if not self.enable_flash:
             sizes = offset2bincount(torch.as_tensor(point.offset_host()))
             self.patch_size = min(int(sizes.min()), self.patch_size_max)
         _, _, cu_seqlens = self.get_padding_and_inverse(point)
         slot_src, slot_dst = self._slots(point)
-
-        qkv = self.qkv(point.feat)
         if self.enable_flash and qkv.dtype == torch.float32:
             # the fused path of the reference always computes in half precision (model.py:477,483)
-            feat = ops.patch_attention(qkv.half(), self.num_heads, slot_src, slot_dst, cu_seqlens,
+            return ops.patch_attention(qkv.half(), self.num_heads, slot_src, slot_dst, cu_seqlens,
                                        self.patch_size, self.scale).to(qkv.dtype)
-        else:
-            feat = ops.patch_attention(qkv, self.num_heads, slot_src, slot_dst, cu_seqlens,
-                                       self.patch_size, self.scale)
+        return ops.patch_attention(qkv, self.num_heads, slot_src, slot_dst, cu_seqlens,
+                                   self.patch_size, self.scale)
+
+    def forward(self, point):
+        feat = self.attend(point, self.qkv(point.feat))
         feat = self.proj(feat)
         feat = self.proj_drop(feat)
         point.feat = feat
@@ -282,28 +284,36 @@ class Block(PointModule):
         if not self._plain_layernorms():
             return self._forward_modular(point)
         ln_cpe, ln1, ln2 = self.cpe[2], self.norm1[0], self.norm2[0]
-        # xCPE: conv reads the sparse view, which lags behind feat in the first decoder block
-        conv = self.cpe[0](point.sparse_conv_feat).features
-        branch = self.cpe[1](conv)
-        # feat = shortcut + LN(branch) and its pre-norm for attention, in one pass
-        feat, normed = ops.layer_norm(branch, ln_cpe.weight, ln_cpe.bias, ln_cpe.eps, residual=point.feat,
-                                      mode=3, weight2=ln1.weight, bias2=ln1.bias)
-        point.feat = normed
-        point = self.attn(point)
-        # feat += attention branch, plus the pre-norm for the MLP
         mlp = self.mlp[0]
         plain_mlp = (type(mlp) is MLP and mlp.fc1.bias is not None and mlp.fc2.bias is not None
                      and not (self.training and mlp.drop.p > 0))
         exact_gelu = type(mlp.act) is nn.GELU and mlp.act.approximate == "none" if plain_mlp else False
         fused = (plain_mlp and exact_gelu and self.channels in ops.MLP_FUSED_CHANNELS
                  and mlp.fc1.out_features == 4 * self.channels and point.feat.dtype != torch.float32)
-        # when fc2 runs as a separate GEMM it accumulates onto the stored sum (beta = 1), so its
+        # xCPE: conv reads the sparse view, which lags behind feat in the first decoder block
+        conv = self.cpe[0](point.sparse_conv_feat).features
+        if fused and type(self.cpe[1]) is nn.Linear and not (self.training and self.attn.proj_drop.p > 0):
+            # thin channels, many points: every dense layer is bound by its N x C tensors going to
+            # HBM and back, so the block runs as conv, head kernel, attention, tail kernel
+            feat, qkv = ops.block_head_fused(conv, point.feat, self.cpe[1], ln_cpe, ln1, self.attn.qkv)
+            attn = self.attn.attend(point, qkv)
+            feat = ops.block_tail_fused(attn, feat, self.attn.proj, ln2, mlp.fc1, mlp.fc2)
+            point.feat = feat
+            point.sparse_conv_feat = point.sparse_conv_feat.replace_feature(feat)
+            return point
+        branch = self.cpe[1](conv)
+        # feat = shortcut + LN(branch) and its pre-norm for attention, in one pass
+        feat, normed = ops.layer_norm(branch, ln_cpe.weight, ln_cpe.bias, ln_cpe.eps, residual=point.feat,
+                                      mode=3, weight2=ln1.weight, bias2=ln1.bias)
+        point.feat = normed
+        point = self.attn(point)
+        # feat += attention branch, plus the pre-norm for the MLP.
+        # When fc2 runs as a separate GEMM it accumulates onto the stored sum (beta = 1), so its
         # bias is added to that sum here: feat + fc2(h) + b2 without a separate add pass
         feat, normed = ops.layer_norm(point.feat, ln2.weight, ln2.bias, ln2.eps, residual=feat, mode=2,
                                       shift=mlp.fc2.bias if (plain_mlp and not fused) else None)
         if fused:
-            # thin channels, many points: fc1 + GELU + fc2 + residual in one kernel, the 4C-wide
-            # hidden tensor never leaves the CU
+            # fc1 + GELU + fc2 + residual in one kernel, the 4C-wide hidden tensor never leaves the CU
             feat = ops.mlp_fused(normed, feat, mlp.fc1.weight, mlp.fc1.bias, mlp.fc2.weight, mlp.fc2.bias)
         elif plain_mlp:
             feat = torch.addmm(feat, mlp.act(mlp.fc1(normed)), mlp.fc2.weight.t())

@@ -372,6 +372,50 @@ def mlp_fused(x, resid, w1, b1, w2, b2):
     return out
 
 
+def _opt(t, dt):
+    return None if t is None else t.to(dt).contiguous()
+
+
+def block_head_fused(conv, shortcut, cpe_linear, ln_cpe, ln1, qkv_linear):
+    """feat = shortcut + ln_cpe(cpe_linear(conv)); qkv = qkv_linear(ln1(feat)) in one kernel.
+    conv, shortcut (N,C) fp16/bf16 with C in MLP_FUSED_CHANNELS; the modules are a Linear C->C,
+    two LayerNorms and a Linear C->3C. Returns (feat, qkv)."""
+    _dev(conv, shortcut, cpe_linear.weight, qkv_linear.weight)
+    lib = _lib.load()
+    conv = conv.contiguous()
+    dt = conv.dtype
+    shortcut = shortcut.to(dt).contiguous()
+    n, c = conv.shape
+    keep = [_opt(t, dt) for t in (cpe_linear.weight, cpe_linear.bias, ln_cpe.weight, ln_cpe.bias, ln1.weight,
+                                   ln1.bias, qkv_linear.weight, qkv_linear.bias)]
+    feat = torch.empty_like(conv)
+    qkv = torch.empty((n, 3 * c), dtype=dt, device=conv.device)
+    _lib.check(lib.ptv3_block_head_fused(_ptr(conv), _ptr(shortcut), _ptr(keep[0]), _ptr(keep[1]), _ptr(keep[2]),
+                                         _ptr(keep[3]), float(ln_cpe.eps), _ptr(keep[4]), _ptr(keep[5]),
+                                         float(ln1.eps), _ptr(keep[6]), _ptr(keep[7]), _dtype_code(conv), n, c,
+                                         _ptr(feat), _ptr(qkv), _stream()), "ptv3_block_head_fused")
+    return feat, qkv
+
+
+def block_tail_fused(attn, shortcut, proj, ln2, fc1, fc2):
+    """feat = shortcut + proj(attn); returns feat + fc2(GELU(fc1(ln2(feat)))) from one kernel.
+    attn, shortcut (N,C) fp16/bf16 with C in MLP_FUSED_CHANNELS and fc1: C->4C."""
+    _dev(attn, shortcut, proj.weight, fc1.weight, fc2.weight)
+    lib = _lib.load()
+    attn = attn.contiguous()
+    dt = attn.dtype
+    shortcut = shortcut.to(dt).contiguous()
+    n, c = attn.shape
+    keep = [_opt(t, dt) for t in (proj.weight, proj.bias, ln2.weight, ln2.bias, fc1.weight, fc1.bias, fc2.weight,
+                                   fc2.bias)]
+    out = torch.empty_like(attn)
+    _lib.check(lib.ptv3_block_tail_fused(_ptr(attn), _ptr(shortcut), _ptr(keep[0]), _ptr(keep[1]), _ptr(keep[2]),
+                                         _ptr(keep[3]), float(ln2.eps), _ptr(keep[4]), _ptr(keep[5]), _ptr(keep[6]),
+                                         _ptr(keep[7]), _dtype_code(attn), n, c, keep[4].shape[0], _ptr(out),
+                                         _stream()), "ptv3_block_tail_fused")
+    return out
+
+
 def bn_act(x, running_mean, running_var, weight, bias, eps, gelu):
     """Inference-mode BatchNorm1d, optionally followed by exact GELU, in one pass. The running
     statistics may be float32 or of x's dtype."""

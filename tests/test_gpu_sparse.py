@@ -206,6 +206,69 @@ def test_mlp_fused_parity(dtype, c, n):
     assert got.dtype == dtype and rel_err(got, want) < TOL[dtype]
 
 
+def _lin(cin, cout, g, dtype, bias=True):
+    m = torch.nn.Linear(cin, cout, bias=bias)
+    with torch.no_grad():
+        m.weight.copy_(torch.randn(cout, cin, generator=g) / cin ** 0.5)
+        if bias:
+            m.bias.copy_(torch.randn(cout, generator=g) * 0.5)
+    return m.to(dtype)
+
+
+def _ln(c, g, dtype):
+    m = torch.nn.LayerNorm(c)
+    with torch.no_grad():
+        m.weight.copy_(torch.rand(c, generator=g) + 0.5)
+        m.bias.copy_(torch.randn(c, generator=g) * 0.3)
+    return m.to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("c", [32, 64])
+@pytest.mark.parametrize("n", [1, 33, 5000, 70_001])
+def test_block_head_fused_parity(dtype, c, n):
+    """shortcut + LN(Linear(conv)) and Linear(LN(that)) against the separate fp32 layers."""
+    g = torch.Generator().manual_seed(11 * c + n)
+    conv = torch.randn(n, c, generator=g).to(dtype)
+    short = torch.randn(n, c, generator=g).to(dtype)
+    cpe1, lnc, ln1 = _lin(c, c, g, dtype), _ln(c, g, dtype), _ln(c, g, dtype)
+    qkv = _lin(c, 3 * c, g, dtype, bias=(n % 2 == 1))
+    with torch.no_grad():
+        f32 = lambda m: m.float()
+        want_feat = short.float() + f32(_clone(lnc))(f32(_clone(cpe1))(conv.float()))
+        want_qkv = f32(_clone(qkv))(f32(_clone(ln1))(want_feat))
+        mods = [m.to(DEV) for m in (cpe1, lnc, ln1, qkv)]
+        feat, out = ops().block_head_fused(conv.to(DEV), short.to(DEV), *mods)
+    assert feat.dtype == dtype and out.shape == (n, 3 * c)
+    assert rel_err(feat, want_feat) < TOL[dtype]
+    assert rel_err(out, want_qkv) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("c", [32, 64])
+@pytest.mark.parametrize("n", [1, 33, 5000, 70_001])
+def test_block_tail_fused_parity(dtype, c, n):
+    """feat = shortcut + proj(attn); feat + fc2(GELU(fc1(LN(feat)))) against the separate fp32 layers."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(13 * c + n)
+    attn = torch.randn(n, c, generator=g).to(dtype)
+    short = torch.randn(n, c, generator=g).to(dtype)
+    proj, ln2 = _lin(c, c, g, dtype), _ln(c, g, dtype)
+    fc1, fc2 = _lin(c, 4 * c, g, dtype), _lin(4 * c, c, g, dtype)
+    with torch.no_grad():
+        f32 = lambda m: _clone(m).float()
+        feat = short.float() + f32(proj)(attn.float())
+        want = feat + f32(fc2)(F.gelu(f32(fc1)(f32(ln2)(feat))))
+        mods = [m.to(DEV) for m in (proj, ln2, fc1, fc2)]
+        got = ops().block_tail_fused(attn.to(DEV), short.to(DEV), *mods)
+    assert got.dtype == dtype and rel_err(got, want) < TOL[dtype]
+
+
+def _clone(module):
+    import copy
+    return copy.deepcopy(module)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("half_stats", [False, True])
 def test_bn_act_parity(dtype, half_stats):
