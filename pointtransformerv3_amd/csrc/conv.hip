@@ -338,6 +338,209 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void subm_conv_dense_kernel(
     }
 }
 
+// Pair mode for wide inputs (cin a multiple of 32 * DEPTH), persistent work-groups.
+// A tile is ROWS consecutive entries of ONE tap of the tap-major pair list times COUT_TILE output
+// channels; the contraction runs in 32-channel steps. Both a step's MFMA work (a few hundred
+// cycles) and a whole tile (cin / 32 steps) are short against the latency of the dependent loads
+// that feed them (tap bounds -> pair indices -> input rows), so
+//   * the input rows and the weight tile of the next DEPTH steps are in flight in a ring of
+//     registers, and the ring runs on across tile boundaries: the last DEPTH steps of a tile
+//     already fetch the first steps of the work-group's next tile;
+//   * the pair indices of the next tile are fetched while this tile is multiplied;
+//   * addresses are per-lane pointers set up once per tile (a step adds a constant), and the
+//     loop body has no branches: rows past the end of a tile and output channels past cout read
+//     a valid address and their products are never stored.
+template <typename T, int MT, int NT, int DEPTH>
+__global__ __launch_bounds__(CONV_THREADS, 2) void pair_gemm_kernel(
+    const T* __restrict__ feat, int cin, int taps, const T* __restrict__ weight, int cout,
+    T* __restrict__ y, const int32_t* __restrict__ pair_in, const int32_t* __restrict__ pair_slot,
+    const int32_t* __restrict__ tap_ptr) {
+    typedef typename HalfOps<T>::v8 v8;
+    constexpr int KC = 32;
+    constexpr int ROWS = CONV_WAVES * MT * 32;
+    constexpr int COUT_TILE = NT * 32;
+    constexpr int W_LOADS = COUT_TILE * (KC / 8) / CONV_THREADS;
+    static_assert(W_LOADS >= 1 && COUT_TILE * (KC / 8) % CONV_THREADS == 0, "weight tile must split evenly");
+    static_assert(DEPTH % 2 == 0, "the weight double buffer alternates with the ring");
+    constexpr int LPR = KC / 8, RPI = 64 / LPR, ITS = 32 / RPI;
+    __shared__ __align__(16) T w_lds[2][COUT_TILE][KC + W_PAD];
+    __shared__ __align__(16) T xs_all[CONV_WAVES][32 * XS_STRIDE];
+
+    const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
+    const int col = lane & 31, hf = lane >> 5;
+    const int srow = lane / LPR, spc = lane % LPR;
+    T* xs = xs_all[wave];
+    const int row0 = wave * (MT * 32);   // first row of the wave inside a tile
+
+    // Row tiles per tap, as an inclusive prefix over the taps: lane l holds taps l and l+64.
+    int first[2], cnt[2], nr[2], incl[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const int tt = lane + 64 * k;
+        first[k] = tt < taps ? tap_ptr[tt] : 0;
+        cnt[k] = tt < taps ? tap_ptr[tt + 1] - first[k] : 0;
+        nr[k] = (cnt[k] + ROWS - 1) / ROWS;
+    }
+    int row_tiles = 0;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        int xsum = nr[k];
+#pragma unroll
+        for (int off = 1; off < PTV3_WAVE; off <<= 1) {
+            const int v = __shfl_up(xsum, off, PTV3_WAVE);
+            if (lane >= off) xsum += v;
+        }
+        incl[k] = xsum + row_tiles;
+        row_tiles += __shfl(xsum, PTV3_WAVE - 1, PTV3_WAVE);
+    }
+    const int col_tiles = (cout + COUT_TILE - 1) / COUT_TILE;
+    const int total = row_tiles * col_tiles;
+    if ((int)blockIdx.x >= total) return;
+
+    struct Tile {
+        const T* xptr[MT][ITS];   // input rows, staging shape: lane (srow, spc) serves rows srow + RPI*it
+        const T* wptr[W_LOADS];   // weight pieces: thread e -> output channel e / 4, 8-channel piece e % 4
+        int32_t slot[MT][4];      // y rows of the pairs this lane stores in the epilogue, -1 past the end
+        int cout0;
+    };
+    auto setup = [&](int g, Tile& tl) {
+        const int rid = g / col_tiles;
+        tl.cout0 = (g % col_tiles) * COUT_TILE;
+        int tap = 0, pstart = 0, pcount = 1;
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const uint64_t hit = __ballot(nr[k] > 0 && rid < incl[k] && rid >= incl[k] - nr[k]);
+            if (hit) {
+                const int l = __ffsll((unsigned long long)hit) - 1;
+                const int rel = rid - (__shfl(incl[k], l, PTV3_WAVE) - __shfl(nr[k], l, PTV3_WAVE));
+                tap = 64 * k + l;
+                pstart = __shfl(first[k], l, PTV3_WAVE) + rel * ROWS;
+                pcount = min(ROWS, __shfl(cnt[k], l, PTV3_WAVE) - rel * ROWS);
+            }
+        }
+#pragma unroll
+        for (int a = 0; a < MT; ++a) {
+#pragma unroll
+            for (int it = 0; it < ITS; ++it) {
+                const int v = row0 + a * 32 + it * RPI + srow;
+                const int32_t idx = pair_in[pstart + min(v, pcount - 1)];
+                tl.xptr[a][it] = feat + (int64_t)idx * cin + spc * 8;
+            }
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const int v = row0 + a * 32 + it * 8 + (lane >> 3);
+                tl.slot[a][it] = v < pcount ? pair_slot[pstart + v] : -1;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < W_LOADS; ++i) {
+            const int e = tid + i * CONV_THREADS;
+            const int co = min(tl.cout0 + e / (KC / 8), cout - 1), pc = e % (KC / 8);
+            tl.wptr[i] = weight + ((int64_t)co * taps + tap) * cin + pc * 8;
+        }
+    };
+
+    u32x4 raw[DEPTH][MT][ITS], wreg[DEPTH][W_LOADS];
+    auto issue = [&](const Tile& tl, int step, u32x4 (&r)[MT][ITS], u32x4 (&w)[W_LOADS]) {
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int it = 0; it < ITS; ++it) r[a][it] = *(const u32x4*)(tl.xptr[a][it] + step * KC);
+#pragma unroll
+        for (int i = 0; i < W_LOADS; ++i) w[i] = *(const u32x4*)(tl.wptr[i] + step * KC);
+    };
+    auto store_w = [&](int buf, const u32x4 (&w)[W_LOADS]) {
+#pragma unroll
+        for (int i = 0; i < W_LOADS; ++i) {
+            const int e = tid + i * CONV_THREADS;
+            *(u32x4*)&w_lds[buf][e / (KC / 8)][(e % (KC / 8)) * 8] = w[i];
+        }
+    };
+    f32x16 acc[MT][NT];
+    // DEPTH steps starting at s0; afterwards the ring holds steps ahead .. ahead + DEPTH - 1 of `src`
+    auto run_steps = [&](const Tile& src, int ahead) {
+#pragma unroll
+        for (int j = 0; j < DEPTH; ++j) {
+            const int buf = j & 1;
+            u32x4 x[KC / 16][MT];
+#pragma unroll
+            for (int a = 0; a < MT; ++a) {
+#pragma unroll
+                for (int it = 0; it < ITS; ++it) *(u32x4*)(xs + (it * RPI + srow) * XS_STRIDE + spc * 8) = raw[j][a][it];
+                lds_fence();
+#pragma unroll
+                for (int ks = 0; ks < KC / 16; ++ks) x[ks][a] = *(const u32x4*)(xs + col * XS_STRIDE + ks * 16 + hf * 8);
+                lds_fence();
+            }
+            store_w(buf ^ 1, wreg[(j + 1) % DEPTH]);   // weights of the step after this one
+            issue(src, ahead + j, raw[j], wreg[j]);
+            u32x4 wf[KC / 16][NT];
+#pragma unroll
+            for (int ks = 0; ks < KC / 16; ++ks)
+#pragma unroll
+                for (int b = 0; b < NT; ++b) wf[ks][b] = *(const u32x4*)&w_lds[buf][b * 32 + col][ks * 16 + hf * 8];
+#pragma unroll
+            for (int ks = 0; ks < KC / 16; ++ks)
+#pragma unroll
+                for (int b = 0; b < NT; ++b)
+#pragma unroll
+                    for (int a = 0; a < MT; ++a)
+                        acc[a][b] = HalfOps<T>::mfma(__builtin_bit_cast(v8, wf[ks][b]), __builtin_bit_cast(v8, x[ks][a]), acc[a][b]);
+            __syncthreads();
+        }
+    };
+
+    const int steps = cin / KC;   // a multiple of DEPTH
+    Tile cur, nxt;
+    setup(blockIdx.x, cur);
+#pragma unroll
+    for (int j = 0; j < DEPTH; ++j) issue(cur, j, raw[j], wreg[j]);
+    store_w(0, wreg[0]);
+    __syncthreads();
+
+    for (int g = blockIdx.x; g < total; g += gridDim.x) {
+        const int gn = g + (int)gridDim.x;
+        setup(gn < total ? gn : g, nxt);   // without a next tile the ring re-reads this one (never used)
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int b = 0; b < NT; ++b)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
+        for (int s0 = 0; s0 + DEPTH < steps; s0 += DEPTH) run_steps(cur, s0 + DEPTH);
+        run_steps(nxt, 0);
+
+        // acc[a][b][v]: output channel cout0 + b*32 + 8*(v/4) + 4*hf + v%4 of pair row0 + a*32 + col.
+        // Back to row-segment shape 64 channels at a time, 16 bytes per lane to y[slot].
+#pragma unroll
+        for (int a = 0; a < MT; ++a) {
+#pragma unroll
+            for (int b0 = 0; b0 < NT; b0 += 2) {
+#pragma unroll
+                for (int bb = 0; bb < 2 && b0 + bb < NT; ++bb)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int b = b0 + bb;
+                        u32x2 pk = {HalfOps<T>::pack2(acc[a][b][4 * q], acc[a][b][4 * q + 1]),
+                                    HalfOps<T>::pack2(acc[a][b][4 * q + 2], acc[a][b][4 * q + 3])};
+                        *(u32x2*)(xs + col * XS_STRIDE + bb * 32 + 8 * q + 4 * hf) = pk;
+                    }
+                lds_fence();
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    const int orow = it * 8 + (lane >> 3), opc = lane & 7;
+                    const int co = cur.cout0 + b0 * 32 + opc * 8;
+                    const u32x4 val = *(const u32x4*)(xs + orow * XS_STRIDE + opc * 8);
+                    if (cur.slot[a][it] >= 0 && co < cout && (NT - b0 >= 2 || opc < 4))
+                        *(u32x4*)(y + (int64_t)cur.slot[a][it] * cout + co) = val;
+                }
+                lds_fence();
+            }
+        }
+        cur = nxt;
+    }
+}
+
 // Pair mode, weight-stationary. A work-group takes one tap and a range of up to `range_rows`
 // of that tap's pairs (tap-major list), keeps W[couts, tap, all input channels] in LDS for its
 // whole life and streams the range through it in tiles of ROWS pairs. Steps (tile, 64-channel
@@ -561,10 +764,23 @@ __global__ __launch_bounds__(256) void pair_segment_sum_kernel(const T* __restri
 #pragma unroll
     for (int k = 0; k < 8; ++k) acc[k] = bias ? HalfOps<T>::to_float(bias[c + k]) : 0.f;
     const int s0 = row_ptr[i], s1 = row_ptr[i + 1];
-    for (int s = s0; s < s1; ++s) {
-        const v8 v = __builtin_bit_cast(v8, *(const u32x4*)(y + (int64_t)s * cout + c));
+    // four rows in flight per thread; the additions keep the order s0, s0+1, ...
+    const T* src = y + (int64_t)s0 * cout + c;
+    for (int s = s0; s < s1; s += 4, src += 4 * (int64_t)cout) {
+        u32x4 raw[4];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) acc[k] += (float)v[k];
+        for (int j = 0; j < 4; ++j) {
+            raw[j] = (u32x4){0, 0, 0, 0};
+            if (s + j < s1) raw[j] = *(const u32x4*)(src + (int64_t)j * cout);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (s + j < s1) {
+                const v8 v = __builtin_bit_cast(v8, raw[j]);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) acc[k] += (float)v[k];
+            }
+        }
     }
     u32x4 r;
 #pragma unroll
@@ -644,25 +860,47 @@ int launch_pairs(const void* feat, int cin, int taps, int64_t n_pairs, const int
 }
 
 // pair tiles through the chunked kernel (55 KB of LDS whatever cin is)
-template <typename T>
-int launch_pairs_chunked(const void* feat, int cin, int taps, int64_t n_pairs, const int32_t* tap_ptr,
+template <typename T, int MT, int NT, int KC>
+int launch_pairs_chunked_v(const void* feat, int cin, int taps, int64_t n_pairs, const int32_t* tap_ptr,
                          const int32_t* pair_in, const int32_t* pair_slot, const void* weight, int cout, void* y,
                          hipStream_t stream) {
-    constexpr int MT = 2, NT = 4, KC = 32, ROWS = CONV_WAVES * MT * 32, COUT_TILE = NT * 32;
+    constexpr int ROWS = CONV_WAVES * MT * 32, COUT_TILE = NT * 32;
     dim3 grid((unsigned)(n_pairs / ROWS + taps), (unsigned)ptv3_ceil_div(cout, COUT_TILE));
     hipLaunchKernelGGL((subm_conv_dense_kernel<T, MT, NT, KC, true>), grid, dim3(CONV_THREADS), 0, stream,
                        (const T*)feat, (int64_t)0, cin, (const int32_t*)nullptr, taps, false, (const T*)weight,
                        (const T*)nullptr, cout, (T*)y, pair_in, pair_slot, tap_ptr);
     return PTV3_OK;
 }
+template <typename T, int MT, int NT, int DEPTH>
+int launch_pair_gemm(const void* feat, int cin, int taps, int64_t n_pairs, const int32_t* tap_ptr,
+                     const int32_t* pair_in, const int32_t* pair_slot, const void* weight, int cout, void* y,
+                     hipStream_t stream) {
+    constexpr int ROWS = CONV_WAVES * MT * 32, COUT_TILE = NT * 32;
+    // persistent work-groups: as many as the machine holds at a time (or as there can be tiles)
+    const int64_t tiles_max = (n_pairs / ROWS + taps) * ptv3_ceil_div(cout, COUT_TILE);
+    const int64_t resident = 256 * 2;
+    dim3 grid((unsigned)(tiles_max < resident ? tiles_max : resident));
+    hipLaunchKernelGGL((pair_gemm_kernel<T, MT, NT, DEPTH>), grid, dim3(CONV_THREADS), 0, stream, (const T*)feat, cin,
+                       taps, (const T*)weight, cout, (T*)y, pair_in, pair_slot, tap_ptr);
+    return PTV3_OK;
+}
+template <typename T>
+int launch_pairs_chunked(const void* feat, int cin, int taps, int64_t n_pairs, const int32_t* tap_ptr,
+                         const int32_t* pair_in, const int32_t* pair_slot, const void* weight, int cout, void* y,
+                         hipStream_t stream) {
+    // the ring of the persistent kernel is four 32-channel steps deep
+    if (cin % 128 == 0 && taps <= 128)
+        return launch_pair_gemm<T, 1, 4, 4>(feat, cin, taps, n_pairs, tap_ptr, pair_in, pair_slot, weight, cout, y, stream);
+    return launch_pairs_chunked_v<T, 2, 4, 32>(feat, cin, taps, n_pairs, tap_ptr, pair_in, pair_slot, weight, cout, y, stream);
+}
 
 template <typename T>
 int dispatch_pairs(const void* feat, int cin, int taps, int64_t n_pairs, const int32_t* tap_ptr,
                    const int32_t* pair_in, const int32_t* pair_slot, const void* weight, int cout, void* y,
                    hipStream_t stream) {
-    // one tap's weights for 128 output channels: 34 KB at cin 128 (two or three work-groups per
-    // CU), 86 KB at 256 (one): from there on the chunked kernel keeps more waves in flight
-    if (cin >= 256 && cout > 64)
+    // from 128 input channels on a tile is long enough (4+ contraction steps) for the persistent
+    // tile kernel, which keeps more waves in flight than one tap's weights in LDS allow
+    if (cin >= 128 && cout > 64)
         return launch_pairs_chunked<T>(feat, cin, taps, n_pairs, tap_ptr, pair_in, pair_slot, weight, cout, y, stream);
 #define PTV3_PAIRS(MT, NT) return launch_pairs<T, MT, NT>(feat, cin, taps, n_pairs, tap_ptr, pair_in, pair_slot, weight, cout, y, stream)
     if (cout <= 32) PTV3_PAIRS(2, 1);
