@@ -56,6 +56,8 @@ template <> struct Half<_Float16> {
         return __builtin_bit_cast(uint32_t, h);
     }
     static __device__ __forceinline__ uint16_t one() { return 0x3C00; }
+    // |score| (log2 units) up to which 2^score needs no shift: normal fp16 numbers are 2^-14 .. 2^15
+    static __device__ __forceinline__ float plain_limit() { return 14.f; }
 };
 template <> struct Half<__bf16> {
     typedef bf16x8 v8;
@@ -68,6 +70,8 @@ template <> struct Half<__bf16> {
         return __builtin_bit_cast(uint32_t, h);
     }
     static __device__ __forceinline__ uint16_t one() { return 0x3F80; }
+    // bf16 has fp32's exponent range; 1024 keys of 2^100 still sum within fp32
+    static __device__ __forceinline__ float plain_limit() { return 100.f; }
 };
 
 // position of key kk (0..31) inside its 32-key block of the transposed V tile: the keys a
@@ -108,6 +112,86 @@ __device__ __forceinline__ int xcd_chunked_id(int bid, int total) {
     return xcd * per + min(xcd, rem) + slot;
 }
 
+// One 32-query tile of one wave against every key of the sequence in LDS.
+// SHIFT = false: the caller has checked that no score can leave [-limit, limit] (|q||k| bound),
+// so probabilities 2^score are representable as they are, the MFMA's C operand is the constant
+// zero and the loop holds nothing but loads, MFMAs, exponentials and conversions.
+// SHIFT = true: scores arrive shifted by a running reference maximum that enters through the C
+// operand; the reference moves (and the accumulators are rescaled) only when a score exceeds it
+// by RESCALE_SLACK, which the per-step |q||k| bound rules out without looking at the scores.
+template <typename T, bool SHIFT>
+__device__ __forceinline__ f32x16 attend_tile(typename Half<T>::v8 qfrag, float qnorm, float kn_reg,
+                                              const unsigned char* k_ptr, const unsigned char* v_ptr,
+                                              int v_step, int n_pairs, int len, int hf) {
+    typedef typename Half<T>::v8 v8;
+    f32x16 acc, cinit;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) { acc[v] = 0.f; cinit[v] = 0.f; }
+    float m_ref = 0.f;   // reference maximum: the MFMA adds -m_ref to every score
+    const bool ragged = (len & 63) != 0;
+    v8 k0 = __builtin_bit_cast(v8, *(const u32x4*)k_ptr);
+    v8 k1 = __builtin_bit_cast(v8, *(const u32x4*)(k_ptr + 32 * 32));
+    for (int kp = 0; kp < n_pairs; ++kp) {
+        f32x16 sa = Half<T>::mfma(k0, qfrag, cinit);   // sa[v] = <K[key_v], Q[q]> - m_ref
+        f32x16 sb = Half<T>::mfma(k1, qfrag, cinit);
+        // operands of the second product: 16 value rows, a row of ones (the denominator), zeros
+        const u32x4 va0 = *(const u32x4*)v_ptr;
+        const u32x4 va1 = *(const u32x4*)(v_ptr + 16);
+        const u32x4 vb0 = *(const u32x4*)(v_ptr + 64);
+        const u32x4 vb1 = *(const u32x4*)(v_ptr + 80);
+        v_ptr += v_step;
+        // keys of the next step (the tile is padded by one step, so the address is always valid)
+        k_ptr += 64 * 32;
+        k0 = __builtin_bit_cast(v8, *(const u32x4*)k_ptr);
+        k1 = __builtin_bit_cast(v8, *(const u32x4*)(k_ptr + 32 * 32));
+        if (ragged && kp == n_pairs - 1) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int key = kp * 64 + 8 * (v >> 2) + 4 * hf + (v & 3);
+                if (key >= len) sa[v] = -INFINITY;
+                if (key + 32 >= len) sb[v] = -INFINITY;
+            }
+        }
+        if (SHIFT) {
+            // |score| <= |q| |k|: when even that bound stays within the slack nothing can
+            // overflow and the running reference is left alone (no max reduction at all)
+            const float kn = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, kn_reg), kp));
+            const bool first = (kp == 0);
+            if (first || __ballot(qnorm * kn - m_ref > RESCALE_SLACK) != 0) {
+                float mx = fmaxf(sa[0], sb[0]);
+#pragma unroll
+                for (int v = 1; v < 16; ++v) mx = fmaxf(mx, fmaxf(sa[v], sb[v]));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, PTV3_WAVE));
+                const bool move = first || mx > RESCALE_SLACK;
+                if (__ballot(move) != 0) {
+                    const float delta = move ? mx : 0.f;
+                    const float alpha = first ? 1.f : exp2f(-delta);
+                    m_ref += delta;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        sa[v] -= delta;
+                        sb[v] -= delta;
+                        cinit[v] = -m_ref;
+                    }
+#pragma unroll
+                    for (int v = 0; v < 9; ++v) acc[v] *= alpha;   // rows 0..15 + denominator row
+                }
+            }
+        }
+        uint32_t pa[8], pb[8];
+#pragma unroll
+        for (int v = 0; v < 8; ++v) {
+            pa[v] = Half<T>::pack2(__builtin_amdgcn_exp2f(sa[2 * v]), __builtin_amdgcn_exp2f(sa[2 * v + 1]));
+            pb[v] = Half<T>::pack2(__builtin_amdgcn_exp2f(sb[2 * v]), __builtin_amdgcn_exp2f(sb[2 * v + 1]));
+        }
+        acc = Half<T>::mfma(__builtin_bit_cast(v8, va0), __builtin_bit_cast(v8, (u32x4){pa[0], pa[1], pa[2], pa[3]}), acc);
+        acc = Half<T>::mfma(__builtin_bit_cast(v8, va1), __builtin_bit_cast(v8, (u32x4){pa[4], pa[5], pa[6], pa[7]}), acc);
+        acc = Half<T>::mfma(__builtin_bit_cast(v8, vb0), __builtin_bit_cast(v8, (u32x4){pb[0], pb[1], pb[2], pb[3]}), acc);
+        acc = Half<T>::mfma(__builtin_bit_cast(v8, vb1), __builtin_bit_cast(v8, (u32x4){pb[4], pb[5], pb[6], pb[7]}), acc);
+    }
+    return acc;
+}
+
 template <typename T>
 __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
     const T* __restrict__ qkv, int channels, int heads, const int32_t* __restrict__ slot_src,
@@ -115,12 +199,14 @@ __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
     float scale_log2e, T* __restrict__ out, int full_items, int split) {
     typedef typename Half<T>::v8 v8;
     extern __shared__ __align__(16) unsigned char smem[];
-    // K tile: lds_keys rows of 32 B. V^T tile: 16 rows of (lds_keys*2 + pad) B. Then one float
-    // per 64-key pair: the largest key norm of the pair.
+    // K tile: lds_keys + 64 rows of 32 B (the last 64 are only ever prefetched). V^T tile: 16 rows
+    // of (lds_keys*2 + pad) B. One float per 64-key step: the largest squared key norm of the
+    // step. Then 96 B of ones and 96 B of zeros: rows 16.. of the second product's A operand.
     unsigned char* k_lds = smem;
     const int vt_stride = lds_keys * 2 + VT_PAD_BYTES;
-    unsigned char* vt_lds = smem + (size_t)lds_keys * 32;
+    unsigned char* vt_lds = smem + (size_t)(lds_keys + 64) * 32;
     float* knorm_lds = (float*)(vt_lds + (size_t)HD * vt_stride);
+    unsigned char* const_lds = (unsigned char*)knorm_lds + ((lds_keys / 64 * 4 + 15) & ~15);
 
     // The first `full_items` work-groups take one (sequence, head) each. The items left over
     // after the last full round of resident work-groups are cut into `split` query ranges, one
@@ -144,27 +230,44 @@ __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
     const int64_t row_stride = 3 * (int64_t)channels;
 
     for (int i = tid; i < n_pairs; i += ATT_THREADS) knorm_lds[i] = 0.f;
+    if (tid < 48) ((uint32_t*)const_lds)[tid] = tid < 24 ? Half<T>::one() * 0x10001u : 0u;
     __syncthreads();
-    // ---- stage K and V^T: thread handles (key, 8-channel half)
-    for (int e = tid; e < len64 * 2; e += ATT_THREADS) {
-        const int key = e >> 1, part = e & 1;
-        u32x4 kq = {0, 0, 0, 0}, vq = {0, 0, 0, 0};
-        if (key < len) {
-            const T* base = qkv + (int64_t)slot_src[s0 + key] * row_stride + head * HD + part * 8;
-            kq = *(const u32x4*)(base + channels);
-            vq = *(const u32x4*)(base + 2 * channels);
-        }
-        *(u32x4*)(k_lds + key * 32 + part * 16) = kq;
-        float nsq = sum_sq8<T>(kq);
-        nsq += __shfl_xor(nsq, 1, PTV3_WAVE);   // the other half of the same key
-        if (part == 0) atomicMax((int*)&knorm_lds[key >> 6], __float_as_int(nsq));   // nsq >= 0
-        const int pos = (key & ~31) + vt_pos(key & 31);
-        unsigned char* vt = vt_lds + (size_t)(part * 8) * vt_stride + pos * 2;
+    // ---- stage K and V^T: a thread handles (key, 8-channel half); four items in flight per thread
+    for (int e0 = tid; e0 < len64 * 2; e0 += 4 * ATT_THREADS) {
+        int32_t row[4];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const uint32_t w = vq[c];
-            *(uint16_t*)(vt + (size_t)(2 * c) * vt_stride) = (uint16_t)(w & 0xffffu);
-            *(uint16_t*)(vt + (size_t)(2 * c + 1) * vt_stride) = (uint16_t)(w >> 16);
+        for (int j = 0; j < 4; ++j) {
+            const int key = (e0 + j * ATT_THREADS) >> 1;
+            row[j] = key < len ? slot_src[s0 + key] : -1;
+        }
+        u32x4 kq[4], vq[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            kq[j] = (u32x4){0, 0, 0, 0};
+            vq[j] = (u32x4){0, 0, 0, 0};
+            if (row[j] >= 0) {
+                const T* base = qkv + (int64_t)row[j] * row_stride + head * HD + (tid & 1) * 8;
+                kq[j] = *(const u32x4*)(base + channels);
+                vq[j] = *(const u32x4*)(base + 2 * channels);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int e = e0 + j * ATT_THREADS;
+            if (e >= len64 * 2) break;
+            const int key = e >> 1, half8 = e & 1;   // == tid & 1: the stride is even
+            *(u32x4*)(k_lds + key * 32 + half8 * 16) = kq[j];
+            float nsq = sum_sq8<T>(kq[j]);
+            nsq += __shfl_xor(nsq, 1, PTV3_WAVE);   // the other half of the same key
+            if (half8 == 0) atomicMax((int*)&knorm_lds[key >> 6], __float_as_int(nsq));   // nsq >= 0
+            const int pos = (key & ~31) + vt_pos(key & 31);
+            unsigned char* vt = vt_lds + (size_t)(half8 * 8) * vt_stride + pos * 2;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t w = vq[j][c];
+                *(uint16_t*)(vt + (size_t)(2 * c) * vt_stride) = (uint16_t)(w & 0xffffu);
+                *(uint16_t*)(vt + (size_t)(2 * c + 1) * vt_stride) = (uint16_t)(w >> 16);
+            }
         }
     }
     __syncthreads();
@@ -173,14 +276,18 @@ __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
     const int col = lane & 31, hf = lane >> 5;
     const int n_qtiles = (len + 31) / 32;
 
-    // A operand rows of the second product: d < 16 read V^T, rows 16 and 20 are ones.
-    u32x4 ones4;
-    {
-        const uint32_t o = (col == 16 || col == 20) ? (Half<T>::one() * 0x10001u) : 0u;
-        ones4 = (u32x4){o, o, o, o};
-    }
+    // lane l keeps the largest key norm of step l (at most 37 steps fit the LDS); the largest of all
+    float kn_reg = lane < n_pairs ? sqrtf(knorm_lds[lane]) * 1.0009765625f : 0.f;   // margin for rounding in the bound
+    float kn_all = kn_reg;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) kn_all = fmaxf(kn_all, __shfl_xor(kn_all, off, PTV3_WAVE));
+
+    // A operand rows of the second product: d < 16 read V^T and advance 128 B per step; rows 16
+    // and 20 read ones and the others zeros, without advancing.
     const unsigned char* k_base = k_lds + col * 32 + hf * 16;
-    const unsigned char* v_base = vt_lds + (size_t)(col & 15) * vt_stride + hf * 32;
+    const unsigned char* v_base = col < HD ? vt_lds + (size_t)col * vt_stride + hf * 32
+                                           : const_lds + ((col == 16 || col == 20) ? 0 : 96);
+    const int v_step = col < HD ? 128 : 0;
 
     const int qt_lo = (int)((int64_t)part * n_qtiles / parts), qt_hi = (int)((int64_t)(part + 1) * n_qtiles / parts);
     for (int qt = qt_lo + wave; qt < qt_hi; qt += ATT_WAVES) {
@@ -197,69 +304,13 @@ __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
         const v8 qfrag = __builtin_bit_cast(v8, qreg);
         float qn = sum_sq8<T>(qreg);
         qn += __shfl_xor(qn, 32, PTV3_WAVE);
-        const float qnorm = sqrtf(qn) * 1.0009765625f;   // margin for rounding in the bound
+        const float qnorm = sqrtf(qn) * 1.0009765625f;
 
-        f32x16 acc, cinit;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) { acc[v] = 0.f; cinit[v] = 0.f; }
-        float m_ref = 0.f;   // reference maximum: the MFMA adds -m_ref to every score
-
-        for (int kp = 0; kp < n_pairs; ++kp) {
-            const v8 k0 = __builtin_bit_cast(v8, *(const u32x4*)(k_base + (kp * 64) * 32));
-            const v8 k1 = __builtin_bit_cast(v8, *(const u32x4*)(k_base + (kp * 64 + 32) * 32));
-            f32x16 sa = Half<T>::mfma(k0, qfrag, cinit);   // sa[v] = <K[key_v], Q[q]> - m_ref
-            f32x16 sb = Half<T>::mfma(k1, qfrag, cinit);
-            if (kp == n_pairs - 1 && len != len64) {
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int key = kp * 64 + 8 * (v >> 2) + 4 * hf + (v & 3);
-                    if (key >= len) sa[v] = -INFINITY;
-                    if (key + 32 >= len) sb[v] = -INFINITY;
-                }
-            }
-            // |score| <= |q| |k|: when even that bound stays within the slack nothing can
-            // overflow and the running reference is left alone (no max reduction at all)
-            const float bound = qnorm * sqrtf(knorm_lds[kp]) - m_ref;
-            const bool first = (kp == 0);
-            if (first || __ballot(bound > RESCALE_SLACK) != 0) {
-                float mx = fmaxf(sa[0], sb[0]);
-#pragma unroll
-                for (int v = 1; v < 16; ++v) mx = fmaxf(mx, fmaxf(sa[v], sb[v]));
-                mx = fmaxf(mx, __shfl_xor(mx, 32, PTV3_WAVE));
-                const bool move = first || mx > RESCALE_SLACK;
-                if (__ballot(move) != 0) {
-                    const float delta = move ? mx : 0.f;
-                    const float alpha = first ? 1.f : exp2f(-delta);
-                    m_ref += delta;
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        sa[v] -= delta;
-                        sb[v] -= delta;
-                        cinit[v] = -m_ref;
-                    }
-#pragma unroll
-                    for (int v = 0; v < 9; ++v) acc[v] *= alpha;   // rows 0..15 + denominator row
-                }
-            }
-            uint32_t pa[8], pb[8];
-#pragma unroll
-            for (int v = 0; v < 8; ++v) {
-                pa[v] = Half<T>::pack2(__builtin_amdgcn_exp2f(sa[2 * v]), __builtin_amdgcn_exp2f(sa[2 * v + 1]));
-                pb[v] = Half<T>::pack2(__builtin_amdgcn_exp2f(sb[2 * v]), __builtin_amdgcn_exp2f(sb[2 * v + 1]));
-            }
-            u32x4 va0 = ones4, va1 = ones4, vb0 = ones4, vb1 = ones4;
-            if (col < HD) {
-                const unsigned char* vrow = v_base + (kp * 64) * 2;
-                va0 = *(const u32x4*)vrow;
-                va1 = *(const u32x4*)(vrow + 16);
-                vb0 = *(const u32x4*)(vrow + 64);
-                vb1 = *(const u32x4*)(vrow + 80);
-            }
-            acc = Half<T>::mfma(__builtin_bit_cast(v8, va0), __builtin_bit_cast(v8, (u32x4){pa[0], pa[1], pa[2], pa[3]}), acc);
-            acc = Half<T>::mfma(__builtin_bit_cast(v8, va1), __builtin_bit_cast(v8, (u32x4){pa[4], pa[5], pa[6], pa[7]}), acc);
-            acc = Half<T>::mfma(__builtin_bit_cast(v8, vb0), __builtin_bit_cast(v8, (u32x4){pb[0], pb[1], pb[2], pb[3]}), acc);
-            acc = Half<T>::mfma(__builtin_bit_cast(v8, vb1), __builtin_bit_cast(v8, (u32x4){pb[4], pb[5], pb[6], pb[7]}), acc);
-        }
+        f32x16 acc;
+        if (__ballot(qnorm * kn_all > Half<T>::plain_limit()) == 0)
+            acc = attend_tile<T, false>(qfrag, qnorm, kn_reg, k_base, v_base, v_step, n_pairs, len, hf);
+        else
+            acc = attend_tile<T, true>(qfrag, qnorm, kn_reg, k_base, v_base, v_step, n_pairs, len, hf);
         // acc[v]: d = 8*(v/4) + 4*hf + v%4; acc[8] = sum of probabilities (row 16 / 20)
         if (dst >= 0) {
             const float inv = 1.f / acc[8];
@@ -348,8 +399,9 @@ int launch_half(const void* qkv, int channels, int heads, const int32_t* slot_sr
                 const int32_t* slot_dst, const int32_t* cu_seqlens, int64_t n_seq,
                 int64_t max_seqlen, float scale, void* out, hipStream_t stream) {
     const int lds_keys = (int)((max_seqlen + 63) & ~63ll);
-    const size_t lds = (size_t)lds_keys * 32 + (size_t)HD * (lds_keys * 2 + VT_PAD_BYTES) +
-                       (size_t)(lds_keys / 64) * sizeof(float);
+    // K (+ one prefetch-only step), V^T, per-step key norms (padded to 16 B), ones and zeros
+    const size_t lds = (size_t)(lds_keys + 64) * 32 + (size_t)HD * (lds_keys * 2 + VT_PAD_BYTES) +
+                       (size_t)(lds_keys / 64) * sizeof(float) + 12 + 192;
     if (lds > 160 * 1024) return PTV3_ESHAPE;
     auto kern = patch_attn_half_kernel<T>;
     static size_t lds_allowed = 0;   // per instantiation; raised monotonically

@@ -60,23 +60,53 @@ __global__ __launch_bounds__(256) void attn_slots_kernel(
 }
 
 // per-axis maximum of (n,3) int32 coordinates into out[3] (pre-set to INT_MIN by the caller's
-// first kernel below): wave reduce, then one atomic per wave and axis
+// first kernel below): wave and block reduce, then one atomic per block and axis
 __global__ void grid_max_init_kernel(int32_t* __restrict__ out) {
     if (threadIdx.x < 3) out[threadIdx.x] = INT32_MIN;
 }
 
 __global__ __launch_bounds__(256) void grid_max_kernel(const int32_t* __restrict__ grid_coord, int64_t n,
-                                                       int32_t* __restrict__ out) {
+                                                       int head, int32_t* __restrict__ out) {
+    // the (n,3) array as a flat stream of 3n values, value f being axis f % 3: `head` values up to
+    // the first 16-byte boundary, then four per load, then the last few
+    typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+    __shared__ int32_t part[4][3];
     int32_t m[3] = {INT32_MIN, INT32_MIN, INT32_MIN};
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t total = 3 * n, quads = (total - head) / 4;
+    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += (int64_t)gridDim.x * blockDim.x) {
+        const i32x4 v = *(const i32x4*)(grid_coord + head + 4 * q);
+        const int a0 = (int)((head + 4 * q) % 3);   // axis of v[0] and v[3]; v[1], v[2] follow cyclically
+        const int a1 = a0 == 2 ? 0 : a0 + 1;
+        const int32_t first = max(v[0], v[3]);
 #pragma unroll
-        for (int a = 0; a < 3; ++a) m[a] = max(m[a], grid_coord[3 * i + a]);
+        for (int a = 0; a < 3; ++a) {
+            const int32_t c = a == a0 ? first : (a == a1 ? v[1] : v[2]);
+            m[a] = max(m[a], c);
+        }
     }
+    if (blockIdx.x == 0) {   // at most 3 + 3 leftover values
+        const int64_t rest = total - head - 4 * quads;
+        int64_t f = -1;
+        if ((int)threadIdx.x < head) f = threadIdx.x;
+        else if ((int64_t)threadIdx.x - head < rest) f = 4 * quads + threadIdx.x;
+        if (f >= 0) {
+            const int a = (int)(f % 3);
+            const int32_t v = grid_coord[f];
+#pragma unroll
+            for (int k = 0; k < 3; ++k) if (k == a) m[k] = max(m[k], v);
+        }
+    }
+    const int wave = threadIdx.x / PTV3_WAVE, lane = threadIdx.x % PTV3_WAVE;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) m[a] = max(m[a], __shfl_xor(m[a], off, PTV3_WAVE));
-        if (threadIdx.x % PTV3_WAVE == 0) atomicMax(&out[a], m[a]);
+        if (lane == 0) part[wave][a] = m[a];
+    }
+    __syncthreads();
+    if (threadIdx.x < 3) {
+        const int a = threadIdx.x;
+        atomicMax(&out[a], max(max(part[0][a], part[1][a]), max(part[2][a], part[3][a])));
     }
 }
 
@@ -86,8 +116,11 @@ extern "C" int ptv3_grid_max(const int32_t* grid_coord, int64_t n, int32_t* out3
     if (n < 1 || !grid_coord || !out3) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
     hipLaunchKernelGGL(grid_max_init_kernel, dim3(1), dim3(64), 0, stream, out3);
-    const int64_t blocks = ptv3_ceil_div(n, 256 * 8) < 1024 ? ptv3_ceil_div(n, 256 * 8) : 1024;
-    hipLaunchKernelGGL(grid_max_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, grid_coord, n, out3);
+    const int64_t want = ptv3_ceil_div(3 * n, 4 * 256);   // one 16-byte load per thread, at most 512 blocks
+    const int64_t blocks = want < 512 ? want : 512;
+    int head = (int)(((16 - ((uintptr_t)grid_coord & 15)) & 15) / 4);
+    if (head > 3 * n) head = (int)(3 * n);
+    hipLaunchKernelGGL(grid_max_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, grid_coord, n, head, out3);
     PTV3_RETURN_LAUNCH();
 }
 

@@ -380,15 +380,16 @@ class SerializedPooling(PointModule):
 
         # clusters in ascending order of the (shifted) row-0 code
         indices = point.serialized_order[0]
-        cluster, idx_ptr, head, m = ops.pool_clusters(point.serialized_code[0], indices, shift)
+        cluster, idx_ptr, head, m, offset, offset_host = ops.pool_clusters(point.serialized_code[0], indices, shift,
+                                                                           point.offset)
         code, grid_coord, batch = ops.pool_gather(point.serialized_code, shift, point.grid_coord,
                                                   pooling_depth, point.batch, head)
         # pooled orders: the distinct clusters met when walking the parent along each curve (same
         # result as argsort of the pooled codes, model.py:667-674, without sorting)
         order, inverse = ops.pool_orders(point.serialized_order, cluster, m)
         if self.shuffle_orders:
-            perm = torch.randperm(code.shape[0]).to(code.device)   # CPU generator (model.py:677)
-            code, order, inverse = code[perm], order[perm], inverse[perm]
+            perm = torch.randperm(code.shape[0]).tolist()   # CPU generator (model.py:677)
+            code, order, inverse = ops.permute_rows(perm, code, order, inverse)
 
         fields = AttrDict(
             feat=ops.segment_reduce(self.proj(point.feat), indices, idx_ptr, self.reduce),
@@ -398,6 +399,8 @@ class SerializedPooling(PointModule):
             serialized_inverse=inverse,
             serialized_depth=depth,
             batch=batch,
+            offset=offset,   # what batch2offset(batch) would compute (model.py:66-67), without its host syncs
+            _offset_host=offset_host,
         )
         if "coord" in point:
             fields["coord"] = ops.segment_reduce(point.coord.float(), indices, idx_ptr, "mean")

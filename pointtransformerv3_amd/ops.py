@@ -243,25 +243,41 @@ def subm_conv_pairs(feat, plan, weight, bias=None):
     return out
 
 
-def pool_clusters(code0, order0, shift):
+def pool_clusters(code0, order0, shift, offset=None):
     """Clusters of code0 >> shift in sorted order. One host sync (the cluster count).
 
-    Returns cluster (N,), idx_ptr (M+1,), head (M,), M."""
-    _dev(code0, order0)
+    Returns cluster (N,), idx_ptr (M+1,), head (M,), M; with `offset` (the parent's cumulative
+    scene ends, on the device) also the pooled scene ends as a device tensor and as a Python
+    list, read in the same device->host copy as the count. Scenes are runs of the sorted order
+    (the scene id is the top of every code), so scene b ends with the cluster of its last point."""
+    _dev(code0, order0, offset)
     lib = _lib.load()
     n = code0.shape[0]
     dev = code0.device
+    order0 = order0.contiguous()
     cluster = torch.empty(n, dtype=torch.int64, device=dev)
     idx_ptr = torch.empty(n + 1, dtype=torch.int64, device=dev)
     head = torch.empty(n, dtype=torch.int64, device=dev)
     count = torch.empty(1, dtype=torch.int64, device=dev)
     nbytes = lib.ptv3_pool_clusters_workspace_bytes(n)
     ws = _ws(nbytes, dev)
-    _lib.check(lib.ptv3_pool_clusters(_ptr(code0.contiguous()), _ptr(order0.contiguous()), n, int(shift),
+    _lib.check(lib.ptv3_pool_clusters(_ptr(code0.contiguous()), _ptr(order0), n, int(shift),
                                       _ptr(cluster), _ptr(idx_ptr), _ptr(head), _ptr(count), _ptr(ws),
                                       nbytes, _stream()), "ptv3_pool_clusters")
-    m = int(count.item())
-    return cluster, idx_ptr[: m + 1], head[:m], m
+    if offset is None:
+        m = int(count.item())
+        return cluster, idx_ptr[: m + 1], head[:m], m
+    last = offset.long() - 1   # sorted position of each scene's last point (-1: no point so far)
+    pooled_offset = torch.where(last >= 0, cluster[order0[last.clamp(min=0)]] + 1, torch.zeros_like(last))
+    host = torch.cat([count, pooled_offset]).tolist()
+    m = int(host[0])
+    return cluster, idx_ptr[: m + 1], head[:m], m, pooled_offset, [int(v) for v in host[1:]]
+
+
+def permute_rows(rows, *tensors):
+    """tensor[rows] for a short host list of row indices, as one concatenation per tensor: an
+    index tensor would first have to be copied to the device, which waits for the stream."""
+    return tuple(torch.stack([t[i] for i in rows]) for t in tensors)
 
 
 def pool_gather(code, shift, grid_coord, pool_depth, batch, head):

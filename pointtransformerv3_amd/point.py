@@ -20,11 +20,12 @@ def offset2bincount(offset):
 
 
 @torch.inference_mode()
-def offset2batch(offset):
-    """Scene id per point from cumulative scene ends (model.py:35-40)."""
+def offset2batch(offset, n=None):
+    """Scene id per point from cumulative scene ends (model.py:35-40). With the number of points
+    given, the result is sized without reading the offsets back to the host."""
     sizes = offset2bincount(offset)
     ids = torch.arange(sizes.numel(), device=offset.device, dtype=torch.long)
-    return ids.repeat_interleave(sizes)
+    return ids.repeat_interleave(sizes, output_size=n)
 
 
 @torch.inference_mode()
@@ -62,22 +63,38 @@ class Point(AttrDict):
     def __init__(self, *args, **kwargs):
         super().__init__(*args, **kwargs)
         if "batch" not in self and "offset" in self:
-            self["batch"] = offset2batch(self["offset"])
+            n = next((self[k].shape[0] for k in ("feat", "coord", "grid_coord") if k in self), None)
+            self["batch"] = offset2batch(self["offset"], n)
         elif "offset" not in self and "batch" in self:
             self["offset"] = batch2offset(self["batch"])
 
-    # ---- host-side facts, one device->host copy each, cached -------------------------
+    # ---- host-side facts: scene ends and grid extent, read in one device->host copy, cached
+    def _fetch_host(self):
+        want_offset = "_offset_host" not in self
+        want_grid = "_grid_max_host" not in self and ("grid_coord" in self or {"grid_size", "coord"} <= self.keys())
+        parts = []
+        if want_offset:
+            parts.append(self["offset"].long())
+        if want_grid:
+            self._ensure_grid_coord()
+            parts.append(ops.grid_max(self["grid_coord"]).long())
+        host = [int(v) for v in (torch.cat(parts) if len(parts) > 1 else parts[0]).tolist()]
+        if want_offset:
+            nb = self["offset"].shape[0]
+            self["_offset_host"], host = host[:nb], host[nb:]
+        if want_grid:
+            self["_grid_max_host"] = host
+
     def offset_host(self):
         """Cumulative scene ends as a Python list."""
         if "_offset_host" not in self:
-            self["_offset_host"] = [int(v) for v in self["offset"].tolist()]
+            self._fetch_host()
         return self["_offset_host"]
 
     def grid_max_host(self):
         """Per-axis maximum of grid_coord as a Python list of 3 ints."""
         if "_grid_max_host" not in self:
-            self._ensure_grid_coord()
-            self["_grid_max_host"] = [int(v) for v in ops.grid_max(self["grid_coord"]).tolist()]
+            self._fetch_host()
         return self["_grid_max_host"]
 
     def _ensure_grid_coord(self):
@@ -108,9 +125,8 @@ class Point(AttrDict):
         sort_order, inverse = ops.argsort_rows(code, key_bits)
 
         if shuffle_orders:
-            perm = torch.randperm(code.shape[0])              # CPU generator, as model.py:129
-            perm = perm.to(code.device)
-            code, sort_order, inverse = code[perm], sort_order[perm], inverse[perm]
+            perm = torch.randperm(code.shape[0]).tolist()     # CPU generator, as model.py:129
+            code, sort_order, inverse = ops.permute_rows(perm, code, sort_order, inverse)
 
         self["serialized_code"] = code
         self["serialized_order"] = sort_order

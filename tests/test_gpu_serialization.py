@@ -120,3 +120,8 @@ def test_grid_max():
     for n in (1, 77, 300_001):
         g = rng.integers(-5, 70_000, size=(n, 3)).astype(np.int32)
         assert ops().grid_max(to_dev(g)).tolist() == g.max(0).tolist()
+    # rows of a larger tensor: the first value is not on a 16-byte boundary
+    g = rng.integers(-5, 70_000, size=(5003, 3)).astype(np.int32)
+    dev = to_dev(g)
+    for skip in (1, 2, 3, 5000, 5002):
+        assert ops().grid_max(dev[skip:]).tolist() == g[skip:].max(0).tolist()
