@@ -120,6 +120,18 @@ int ptv3_conv_plan_count(const int32_t *nbr, int64_t n, int taps, int tap_major,
 int ptv3_conv_plan_fill(const int32_t *nbr, int64_t n, int taps, int tap_major, const int32_t *tap_ptr,
                         int32_t *row_ptr, int32_t *pair_in, int32_t *pair_slot, void *workspace,
                         size_t workspace_bytes, void *stream);
+/* The same pair lists straight from the voxel coordinates (indices as for ptv3_kmap_build), without
+ * a stored neighbour map: bit-identical to ptv3_conv_plan_count / _fill applied to the map
+ * ptv3_kmap_build returns. The count call builds the voxel hash in the workspace, the fill call
+ * (after n_pairs has been read on the host) reuses it: same workspace, untouched in between,
+ * >= ptv3_kmap_plan_workspace_bytes(n, ks); ks is 3 or 5. Replaces spconv's indice-pair generation
+ * for SubMConv3d (call sites model.py:546-552, :767-774). */
+size_t ptv3_kmap_plan_workspace_bytes(int64_t n, int ks);
+int ptv3_kmap_plan_count(const int32_t *indices, int64_t n, int ks, int32_t *tap_ptr, int64_t *n_pairs,
+                         void *workspace, size_t workspace_bytes, void *stream);
+int ptv3_kmap_plan_fill(const int32_t *indices, int64_t n, int ks, const int32_t *tap_ptr,
+                        int32_t *row_ptr, int32_t *pair_in, int32_t *pair_slot, void *workspace,
+                        size_t workspace_bytes, void *stream);
 int ptv3_subm_conv_pairs_fwd(const void *feat, int dtype, int64_t n, int cin, int taps,
                              int64_t n_pairs, const int32_t *tap_ptr, const int32_t *row_ptr,
                              const int32_t *pair_in, const int32_t *pair_slot, const void *weight,

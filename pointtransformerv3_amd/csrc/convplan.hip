@@ -10,7 +10,12 @@
 //     writes pair q's product row to y[pair_slot[q]], and a segment sum over
 //     [row_ptr[i], row_ptr[i+1]) finishes voxel i without atomics.
 // Both ranks are exclusive scans of the same activity mask, one row-major, one tap-major.
-#include "common.h"
+//
+// The pair lists can also be built straight from the voxel coordinates (ptv3_kmap_plan_*): the same
+// two scans, with the activity mask looked up in the voxel hash on the fly instead of read from a
+// stored map. For a 5x5x5 stem on 400k voxels the stored map is 200 MB written once and read twice
+// for ~6 active taps of 125 per voxel; the direct form never materialises it.
+#include "voxelhash.h"
 
 namespace {
 
@@ -149,8 +154,8 @@ struct PlanWs {
     size_t bytes;
 };
 
-PlanWs carve_plan(void* base, int64_t n, int taps) {
-    const int64_t blocks = ptv3_ceil_div(n > 0 ? n : 1, PLAN_THREADS);
+PlanWs carve_plan(void* base, int64_t n, int taps, int block_threads = PLAN_THREADS) {
+    const int64_t blocks = ptv3_ceil_div(n > 0 ? n : 1, block_threads);
     PlanWs w;
     char* p = (char*)base;
     size_t off = 0;
@@ -164,6 +169,203 @@ PlanWs carve_plan(void* base, int64_t n, int taps) {
     off += ptv3_align256((size_t)MAX_TAPS * 4);
     w.bytes = off;
     return w;
+}
+
+
+// ---- pair lists straight from the voxel hash: one wave per block of 64 voxels, thread = voxel.
+// A lane reads the headers of the (at most 8) voxel blocks around its voxel, all in flight
+// together, and knows from their masks which taps exist. Found taps are published as per-tap lane
+// masks in LDS, which give the block's per-tap counts (count pass) and every pair's rank inside
+// (block, tap) (fill pass); the fill pass then reads one row index per existing neighbour.
+constexpr int DIRECT_THREADS = PTV3_WAVE;
+
+struct TapSet {
+    uint64_t lo, hi;   // bit t <-> tap t (< 128)
+    __device__ __forceinline__ void set(int t) {
+        if (t < 64) lo |= 1ull << t; else hi |= 1ull << (t - 64);
+    }
+    __device__ __forceinline__ int count() const { return __popcll(lo) + __popcll(hi); }
+    __device__ __forceinline__ int rank(int t) const {   // members below t
+        return t < 64 ? __popcll(lo & ((1ull << t) - 1ull)) : __popcll(lo) + __popcll(hi & ((1ull << (t - 64)) - 1ull));
+    }
+};
+
+__device__ __forceinline__ uint32_t wave_scan_incl(uint32_t v, uint32_t* total) {
+    const int lane = threadIdx.x % PTV3_WAVE;
+    uint32_t x = v;
+#pragma unroll
+    for (int off = 1; off < PTV3_WAVE; off <<= 1) {
+        const uint32_t y = __shfl_up(x, off, PTV3_WAVE);
+        if (lane >= off) x += y;
+    }
+    *total = __shfl(x, PTV3_WAVE - 1, PTV3_WAVE);
+    return x;
+}
+
+// taps of the window that exist, also published in lane_mask[t]
+template <int KS>
+__device__ __forceinline__ TapSet publish_taps(const VoxelWindow& w, int4 v, unsigned long long* lane_mask) {
+    const int lane = threadIdx.x;
+    TapSet found = {0, 0};
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        uint64_t m = w.hits[k];
+        while (m) {
+            const int bit = __builtin_ctzll(m);
+            m &= m - 1;
+            const int t = vh_tap_of<KS / 2>(w, k, bit, v.y, v.z, v.w);
+            found.set(t);
+            atomicOr(&lane_mask[t], 1ull << lane);
+        }
+    }
+    return found;
+}
+
+// what the count pass leaves per voxel for the fill pass: the header slots of its 8 blocks and
+// its found taps, as arrays over the voxels (coalesced both ways)
+struct DirectNotes {
+    uint32_t* slot;     // [8][n]
+    uint64_t* found;    // [2][n]
+};
+
+template <int KS>
+__global__ __launch_bounds__(DIRECT_THREADS) void direct_count_kernel(
+    const int32_t* __restrict__ indices, int64_t n, VoxelHash h, DirectNotes notes, uint32_t* __restrict__ row_cnt,
+    uint32_t* __restrict__ blk_row_sum, uint32_t* __restrict__ blk_tap_cnt) {
+    constexpr int TAPS = KS * KS * KS;
+    __shared__ unsigned long long lane_mask[MAX_TAPS];
+    const int lane = threadIdx.x;
+    const int64_t i = (int64_t)blockIdx.x * DIRECT_THREADS + lane;
+    lane_mask[lane] = 0;
+    lane_mask[lane + 64] = 0;
+    __syncthreads();
+    uint32_t cnt = 0;
+    if (i < n) {
+        const int4 v = ((const int4*)indices)[i];
+        const VoxelWindow w = vh_window<KS / 2>(h, v.x, v.y, v.z, v.w);
+        const TapSet found = publish_taps<KS>(w, v, lane_mask);
+        cnt = (uint32_t)found.count();
+        row_cnt[i] = cnt;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) notes.slot[(int64_t)k * n + i] = w.slot[k];
+        notes.found[i] = found.lo;
+        notes.found[n + i] = found.hi;
+    }
+    uint32_t total;
+    wave_scan_incl(cnt, &total);
+    if (lane == 0) blk_row_sum[blockIdx.x] = total;
+    __syncthreads();
+    for (int t = lane; t < TAPS; t += DIRECT_THREADS)
+        blk_tap_cnt[(int64_t)blockIdx.x * TAPS + t] = (uint32_t)__popcll(lane_mask[t]);
+}
+
+constexpr int DIRECT_STAGE = 1024;   // pairs of one 64-voxel block staged in LDS for coalesced writes
+
+template <int KS>
+__global__ __launch_bounds__(DIRECT_THREADS) void direct_fill_kernel(
+    const int32_t* __restrict__ indices, int64_t n, VoxelHash h, DirectNotes notes, const uint32_t* __restrict__ row_cnt,
+    const uint32_t* __restrict__ blk_row_off, const uint32_t* __restrict__ blk_tap_off,
+    const int32_t* __restrict__ tap_ptr, int32_t* __restrict__ row_ptr, int32_t* __restrict__ pair_in,
+    int32_t* __restrict__ pair_slot) {
+    constexpr int R = KS / 2, TAPS = KS * KS * KS, CENTRE = TAPS / 2;
+    __shared__ unsigned long long lane_mask[MAX_TAPS];
+    __shared__ uint32_t tap_base[MAX_TAPS];    // first pair of (block, tap) in the tap-major lists
+    __shared__ uint32_t tap_start[MAX_TAPS];   // first pair of (block, tap) in the staging buffer
+    __shared__ uint32_t blk_slot[8][DIRECT_THREADS];
+    __shared__ uint32_t stage_q[DIRECT_STAGE];
+    __shared__ int32_t stage_in[DIRECT_STAGE], stage_slot[DIRECT_STAGE];
+    const int lane = threadIdx.x;
+    const int64_t i = (int64_t)blockIdx.x * DIRECT_THREADS + lane;
+    const uint64_t below = (1ull << lane) - 1ull;
+    lane_mask[lane] = 0;
+    lane_mask[lane + 64] = 0;
+    for (int t = lane; t < TAPS; t += DIRECT_THREADS)
+        tap_base[t] = (uint32_t)tap_ptr[t] + blk_tap_off[(int64_t)blockIdx.x * TAPS + t];
+    const uint32_t cnt = i < n ? row_cnt[i] : 0u;
+    uint32_t total;
+    const uint32_t inc = wave_scan_incl(cnt, &total);
+    const uint32_t slot0 = blk_row_off[blockIdx.x] + inc - cnt;   // first output slot of my voxel
+    if (i < n) row_ptr[i] = (int32_t)slot0;
+    if (i == n - 1) row_ptr[n] = (int32_t)(slot0 + cnt);
+    int4 v = {0, 0, 0, 0};
+    TapSet found = {0, 0};
+    if (i < n) {
+        v = ((const int4*)indices)[i];
+        found.lo = notes.found[i];
+        found.hi = notes.found[n + i];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) blk_slot[k][lane] = notes.slot[(int64_t)k * n + i];
+    }
+    __syncthreads();
+    // per-tap lane masks from the found sets
+    {
+        TapSet f = found;
+        while (f.lo) { const int t = __builtin_ctzll(f.lo); f.lo &= f.lo - 1; atomicOr(&lane_mask[t], 1ull << lane); }
+        while (f.hi) { const int t = 64 + __builtin_ctzll(f.hi); f.hi &= f.hi - 1; atomicOr(&lane_mask[t], 1ull << lane); }
+    }
+    __syncthreads();
+    // staging position of every tap's first pair: exclusive scan of the per-tap counts
+    {
+        const uint32_t c0 = (uint32_t)__popcll(lane_mask[lane]), c1 = (uint32_t)__popcll(lane_mask[lane + 64]);
+        uint32_t t0, t1;
+        const uint32_t i0 = wave_scan_incl(c0, &t0);
+        const uint32_t i1 = wave_scan_incl(c1, &t1);
+        tap_start[lane] = i0 - c0;
+        tap_start[lane + 64] = t0 + i1 - c1;
+    }
+    __syncthreads();
+    const bool staged = total <= (uint32_t)DIRECT_STAGE;   // total = pairs of this block
+    // a voxel's slots follow tap order, a tap's pairs voxel order: both ranks come from the masks
+    const int xs = v.y + VH_SHIFT, ys = v.z + VH_SHIFT, zs = v.w + VH_SHIFT;
+    const int bx0 = (xs - R) >> 2, by0 = (ys - R) >> 2, bz0 = (zs - R) >> 2;
+    TapSet f = found;
+    uint32_t slot = slot0;
+    while (f.lo | f.hi) {
+        int t;
+        if (f.lo) { t = __builtin_ctzll(f.lo); f.lo &= f.lo - 1; }
+        else { t = 64 + __builtin_ctzll(f.hi); f.hi &= f.hi - 1; }
+        int32_t src = (int32_t)i;
+        if (t != CENTRE) {
+            const int cx = xs + t / (KS * KS) - R, cy = ys + (t / KS) % KS - R, cz = zs + t % KS - R;
+            const int k = ((cx >> 2) - bx0) << 2 | ((cy >> 2) - by0) << 1 | ((cz >> 2) - bz0);
+            const int bit = (cx & 3) << 4 | (cy & 3) << 2 | (cz & 3);
+            src = h.rows[(int64_t)blk_slot[k][lane] * 64 + bit];
+        }
+        const uint32_t rank = (uint32_t)__popcll(lane_mask[t] & below);
+        const uint32_t q = tap_base[t] + rank;
+        if (staged) {
+            const uint32_t e = tap_start[t] + rank;
+            stage_q[e] = q;
+            stage_in[e] = src;
+            stage_slot[e] = (int32_t)slot;
+        } else {
+            pair_in[q] = src;
+            pair_slot[q] = (int32_t)slot;
+        }
+        ++slot;
+    }
+    if (!staged) return;   // uniform: `total` is the same in every lane
+    __syncthreads();
+    for (uint32_t e = lane; e < total; e += DIRECT_THREADS) {
+        const uint32_t q = stage_q[e];
+        pair_in[q] = stage_in[e];
+        pair_slot[q] = stage_slot[e];
+    }
+}
+
+size_t direct_notes_bytes(int64_t n) {
+    return ptv3_align256((size_t)n * 8 * sizeof(uint32_t)) + ptv3_align256((size_t)n * 2 * sizeof(uint64_t));
+}
+
+DirectNotes carve_notes(void* base, int64_t n) {
+    DirectNotes d;
+    d.slot = (uint32_t*)base;
+    d.found = (uint64_t*)((char*)base + ptv3_align256((size_t)n * 8 * sizeof(uint32_t)));
+    return d;
+}
+
+size_t direct_plan_bytes(int64_t n, int taps) {
+    return vh_bytes(n) + direct_notes_bytes(n) + carve_plan(nullptr, n, taps, DIRECT_THREADS).bytes;
 }
 
 }  // namespace
@@ -202,5 +404,59 @@ extern "C" int ptv3_conv_plan_fill(const int32_t* nbr, int64_t n, int taps, int 
     hipLaunchKernelGGL(plan_fill_kernel, dim3((unsigned)blocks), dim3(PLAN_THREADS), 0, (hipStream_t)stream_,
                        nbr, n, taps, tap_major != 0, (const uint32_t*)w.row_cnt, (const uint32_t*)w.blk_row_sum,
                        (const uint32_t*)w.blk_tap_cnt, tap_ptr, row_ptr, pair_in, pair_slot);
+    PTV3_RETURN_LAUNCH();
+}
+
+extern "C" size_t ptv3_kmap_plan_workspace_bytes(int64_t n, int ks) {
+    if (n < 0 || (ks != 3 && ks != 5)) return 0;
+    return direct_plan_bytes(n, ks * ks * ks);
+}
+
+extern "C" int ptv3_kmap_plan_count(const int32_t* indices, int64_t n, int ks, int32_t* tap_ptr, int64_t* n_pairs,
+                                    void* workspace, size_t workspace_bytes, void* stream_) {
+    if (n < 1 || n >= (1ll << 31) / 128) return PTV3_EINVAL;
+    if (ks != 3 && ks != 5) return PTV3_ESHAPE;
+    if (!indices || !tap_ptr || !n_pairs || !workspace) return PTV3_EINVAL;
+    const int taps = ks * ks * ks;
+    if (workspace_bytes < direct_plan_bytes(n, taps)) return PTV3_EWORKSPACE;
+    hipStream_t stream = (hipStream_t)stream_;
+    const VoxelHash h = vh_build(workspace, indices, n, stream);
+    const DirectNotes notes = carve_notes((char*)workspace + vh_bytes(n), n);
+    PlanWs w = carve_plan((char*)workspace + vh_bytes(n) + direct_notes_bytes(n), n, taps, DIRECT_THREADS);
+    const int64_t blocks = ptv3_ceil_div(n, DIRECT_THREADS);
+    if (ks == 3)
+        hipLaunchKernelGGL(direct_count_kernel<3>, dim3((unsigned)blocks), dim3(DIRECT_THREADS), 0, stream, indices, n,
+                           h, notes, w.row_cnt, w.blk_row_sum, w.blk_tap_cnt);
+    else
+        hipLaunchKernelGGL(direct_count_kernel<5>, dim3((unsigned)blocks), dim3(DIRECT_THREADS), 0, stream, indices, n,
+                           h, notes, w.row_cnt, w.blk_row_sum, w.blk_tap_cnt);
+    hipLaunchKernelGGL(plan_scan_kernel, dim3((unsigned)(taps + 1)), dim3(PLAN_THREADS), 0, stream,
+                       w.blk_tap_cnt, w.blk_row_sum, blocks, taps, w.tap_total, n_pairs);
+    hipLaunchKernelGGL(plan_tap_ptr_kernel, dim3(1), dim3(PLAN_THREADS), 0, stream,
+                       (const uint32_t*)w.tap_total, taps, tap_ptr);
+    PTV3_RETURN_LAUNCH();
+}
+
+extern "C" int ptv3_kmap_plan_fill(const int32_t* indices, int64_t n, int ks, const int32_t* tap_ptr,
+                                   int32_t* row_ptr, int32_t* pair_in, int32_t* pair_slot, void* workspace,
+                                   size_t workspace_bytes, void* stream_) {
+    if (n < 1 || n >= (1ll << 31) / 128) return PTV3_EINVAL;
+    if (ks != 3 && ks != 5) return PTV3_ESHAPE;
+    if (!indices || !tap_ptr || !row_ptr || !pair_in || !pair_slot || !workspace) return PTV3_EINVAL;
+    const int taps = ks * ks * ks;
+    if (workspace_bytes < direct_plan_bytes(n, taps)) return PTV3_EWORKSPACE;
+    hipStream_t stream = (hipStream_t)stream_;
+    const VoxelHash h = vh_view(workspace, n);   // built by ptv3_kmap_plan_count in this workspace
+    const DirectNotes notes = carve_notes((char*)workspace + vh_bytes(n), n);
+    PlanWs w = carve_plan((char*)workspace + vh_bytes(n) + direct_notes_bytes(n), n, taps, DIRECT_THREADS);
+    const int64_t blocks = ptv3_ceil_div(n, DIRECT_THREADS);
+    if (ks == 3)
+        hipLaunchKernelGGL(direct_fill_kernel<3>, dim3((unsigned)blocks), dim3(DIRECT_THREADS), 0, stream, indices, n, h,
+                           notes, (const uint32_t*)w.row_cnt, (const uint32_t*)w.blk_row_sum, (const uint32_t*)w.blk_tap_cnt,
+                           tap_ptr, row_ptr, pair_in, pair_slot);
+    else
+        hipLaunchKernelGGL(direct_fill_kernel<5>, dim3((unsigned)blocks), dim3(DIRECT_THREADS), 0, stream, indices, n, h,
+                           notes, (const uint32_t*)w.row_cnt, (const uint32_t*)w.blk_row_sum, (const uint32_t*)w.blk_tap_cnt,
+                           tap_ptr, row_ptr, pair_in, pair_slot);
     PTV3_RETURN_LAUNCH();
 }

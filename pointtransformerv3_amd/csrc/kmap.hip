@@ -6,120 +6,42 @@
 // stored voxel-major (n, taps) or tap-major (taps, n); the convolution kernels read the
 // tap-major form coalesced.
 //
-//   fill    : table keys <- EMPTY, filter bits <- 0
-//   insert  : one thread per voxel, 64-bit CAS, linear probing (load factor <= 0.5); also sets the
-//             voxel's bit in a hashed bitmap of 16 bits per voxel
-//   lookup  : one thread per map entry in storage order, so the int32 map is written fully
-//             coalesced in either layout. On surface scans 90-97 % of the probed neighbours do not
-//             exist, and a probe of the table costs a whole cache line from HBM (the table does not
-//             fit L2); the bitmap (1 MB for 400k voxels, L2-resident) answers "absent" for ~94 % of
-//             those without touching the table.
-#include "common.h"
+//   fill, insert : the block-keyed voxel hash (voxelhash.h)
+//   lookup       : one thread per voxel: at most 8 block headers tell which neighbours exist, one row
+//                  read per existing neighbour; the voxel's taps are first set to -1 (in the
+//                  tap-major layout consecutive lanes write consecutive voxels of one tap).
+#include "voxelhash.h"
 
 namespace {
 
-constexpr uint64_t EMPTY_KEY = ~0ull;
-
-__device__ __forceinline__ uint64_t voxel_key(int b, int x, int y, int z) {
-    // 17 bits per axis after a +4 shift: neighbours of coordinate 0 stay distinct and
-    // nothing wraps for coordinates up to 65535 and kernel sizes up to 9.
-    return ((uint64_t)(uint32_t)b << 51) | ((uint64_t)(uint32_t)(x + 4) << 34) |
-           ((uint64_t)(uint32_t)(y + 4) << 17) | (uint64_t)(uint32_t)(z + 4);
-}
-
-// 64-bit finaliser: the low bits pick the table slot, the high bits the filter bit
-__device__ __forceinline__ uint64_t mix64(uint64_t k) {
-    k ^= k >> 33;
-    k *= 0xff51afd7ed558ccdull;
-    k ^= k >> 33;
-    k *= 0xc4ceb9fe1a85ec53ull;
-    k ^= k >> 33;
-    return k;
-}
-
-__global__ __launch_bounds__(256) void kmap_fill_kernel(uint64_t* __restrict__ keys, int64_t cap,
-                                                        uint32_t* __restrict__ filter, int64_t filter_words) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < cap) keys[i] = EMPTY_KEY;
-    if (i < filter_words) filter[i] = 0u;
-}
-
-__global__ __launch_bounds__(256) void kmap_insert_kernel(const int32_t* __restrict__ indices,
-                                                          int64_t n, uint64_t* __restrict__ keys,
-                                                          int32_t* __restrict__ vals, uint32_t mask,
-                                                          uint32_t* __restrict__ filter, uint32_t filter_mask) {
+template <bool TAP_MAJOR, int KS>
+__global__ __launch_bounds__(256) void kmap_lookup_kernel(const int32_t* __restrict__ indices, int64_t n,
+                                                          VoxelHash h, int32_t* __restrict__ nbr) {
+    constexpr int R = KS / 2, TAPS = KS * KS * KS;
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const int4 v = ((const int4*)indices)[i];
-    const uint64_t key = voxel_key(v.x, v.y, v.z, v.w);
-    const uint64_t h = mix64(key);
-    const uint32_t bit = (uint32_t)(h >> 32) & filter_mask;
-    atomicOr(&filter[bit >> 5], 1u << (bit & 31));
-    uint32_t slot = (uint32_t)h & mask;
-    for (uint32_t probe = 0; probe <= mask; ++probe) {
-        const uint64_t prev = atomicCAS((unsigned long long*)&keys[slot], (unsigned long long)EMPTY_KEY,
-                                        (unsigned long long)key);
-        if (prev == EMPTY_KEY || prev == key) {
-            vals[slot] = (int32_t)i;
-            return;
-        }
-        slot = (slot + 1) & mask;
-    }
-}
-
-template <bool TAP_MAJOR>
-__global__ __launch_bounds__(256) void kmap_lookup_kernel(const int32_t* __restrict__ indices,
-                                                          int64_t n, int ks, int taps,
-                                                          const uint64_t* __restrict__ keys,
-                                                          const int32_t* __restrict__ vals,
-                                                          uint32_t mask, const uint32_t* __restrict__ filter,
-                                                          uint32_t filter_mask, int32_t* __restrict__ nbr) {
-    // one thread per map entry, in the order the entries are stored, so writes coalesce
-    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= n * taps) return;
-    const int64_t i = TAP_MAJOR ? e % n : e / taps;
-    const int t = (int)(TAP_MAJOR ? e / n : e - i * taps);
-    const int r = ks >> 1;
-    const int kz = t % ks, ky = (t / ks) % ks, kx = t / (ks * ks);
-    const int4 v = ((const int4*)indices)[i];
-    int32_t found = -1;
-    if (t == taps / 2) {
-        found = (int32_t)i;   // centre tap
-    } else {
-        const uint64_t key = voxel_key(v.x, v.y + kx - r, v.z + ky - r, v.w + kz - r);
-        const uint64_t h = mix64(key);
-        const uint32_t bit = (uint32_t)(h >> 32) & filter_mask;
-        const bool maybe = (filter[bit >> 5] >> (bit & 31)) & 1u;
-        uint32_t slot = (uint32_t)h & mask;
-        for (uint32_t probe = 0; maybe && probe <= mask; ++probe) {
-            const uint64_t cur = keys[slot];
-            if (cur == key) { found = vals[slot]; break; }
-            if (cur == EMPTY_KEY) break;
-            slot = (slot + 1) & mask;
+    const VoxelWindow w = vh_window<R>(h, v.x, v.y, v.z, v.w);
+#pragma unroll 1
+    for (int t = 0; t < TAPS; ++t) nbr[TAP_MAJOR ? (int64_t)t * n + i : i * TAPS + t] = -1;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        uint64_t m = w.hits[k];
+        while (m) {
+            const int bit = __builtin_ctzll(m);
+            m &= m - 1;
+            const int t = vh_tap_of<R>(w, k, bit, v.y, v.z, v.w);
+            const int32_t row = t == TAPS / 2 ? (int32_t)i : h.rows[(int64_t)w.slot[k] * 64 + bit];
+            nbr[TAP_MAJOR ? (int64_t)t * n + i : i * TAPS + t] = row;
         }
     }
-    nbr[e] = found;
-}
-
-int64_t table_capacity(int64_t n) {
-    int64_t cap = 1024;
-    while (cap < 2 * n) cap <<= 1;
-    return cap;
-}
-
-int64_t filter_bits(int64_t n) {
-    int64_t bits = 4096;
-    while (bits < 16 * n) bits <<= 1;
-    return bits;
 }
 
 }  // namespace
 
 extern "C" size_t ptv3_kmap_workspace_bytes(int64_t n) {
     if (n < 0) return 0;
-    const int64_t cap = table_capacity(n);
-    return ptv3_align256((size_t)cap * sizeof(uint64_t)) + ptv3_align256((size_t)cap * sizeof(int32_t)) +
-           ptv3_align256((size_t)filter_bits(n) / 8);
+    return vh_bytes(n);
 }
 
 extern "C" int ptv3_kmap_build(const int32_t* indices, int64_t n, int ks, int tap_major, int32_t* nbr,
@@ -128,27 +50,16 @@ extern "C" int ptv3_kmap_build(const int32_t* indices, int64_t n, int ks, int ta
     if (ks != 3 && ks != 5) return PTV3_ESHAPE;
     if (n == 0) return PTV3_OK;
     if (!indices || !nbr || !workspace) return PTV3_EINVAL;
-    if (workspace_bytes < ptv3_kmap_workspace_bytes(n)) return PTV3_EWORKSPACE;
+    if (workspace_bytes < vh_bytes(n)) return PTV3_EWORKSPACE;
     hipStream_t stream = (hipStream_t)stream_;
-    const int64_t cap = table_capacity(n);
-    uint64_t* keys = (uint64_t*)workspace;
-    int32_t* vals = (int32_t*)((char*)workspace + ptv3_align256((size_t)cap * sizeof(uint64_t)));
-    uint32_t* filter = (uint32_t*)((char*)vals + ptv3_align256((size_t)cap * sizeof(int32_t)));
-    const int64_t fbits = filter_bits(n);
-    const uint32_t filter_mask = (uint32_t)(fbits - 1);
-    const uint32_t mask = (uint32_t)(cap - 1);
-    const int taps = ks * ks * ks;
-    hipLaunchKernelGGL(kmap_fill_kernel, dim3((unsigned)ptv3_ceil_div(cap, 256)), dim3(256), 0, stream,
-                       keys, cap, filter, fbits / 32);
-    hipLaunchKernelGGL(kmap_insert_kernel, dim3((unsigned)ptv3_ceil_div(n, 256)), dim3(256), 0, stream,
-                       indices, n, keys, vals, mask, filter, filter_mask);
-    if (tap_major)
-        hipLaunchKernelGGL(kmap_lookup_kernel<true>, dim3((unsigned)ptv3_ceil_div(n * taps, 256)), dim3(256), 0,
-                           stream, indices, n, ks, taps, (const uint64_t*)keys, (const int32_t*)vals, mask,
-                           (const uint32_t*)filter, filter_mask, nbr);
-    else
-        hipLaunchKernelGGL(kmap_lookup_kernel<false>, dim3((unsigned)ptv3_ceil_div(n * taps, 256)), dim3(256), 0,
-                           stream, indices, n, ks, taps, (const uint64_t*)keys, (const int32_t*)vals, mask,
-                           (const uint32_t*)filter, filter_mask, nbr);
+    const VoxelHash h = vh_build(workspace, indices, n, stream);
+    const dim3 grid((unsigned)ptv3_ceil_div(n, 256)), block(256);
+#define PTV3_LOOKUP(TM, KS) hipLaunchKernelGGL((kmap_lookup_kernel<TM, KS>), grid, block, 0, stream, indices, n, h, nbr)
+    if (tap_major) {
+        if (ks == 3) PTV3_LOOKUP(true, 3); else PTV3_LOOKUP(true, 5);
+    } else {
+        if (ks == 3) PTV3_LOOKUP(false, 3); else PTV3_LOOKUP(false, 5);
+    }
+#undef PTV3_LOOKUP
     PTV3_RETURN_LAUNCH();
 }

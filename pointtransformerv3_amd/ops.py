@@ -225,6 +225,32 @@ def conv_plan(nbr, tap_major=False):
     return plan
 
 
+def conv_plan_direct(indices, ks):
+    """The pair lists of conv_plan(kmap_build(indices, ks)) straight from the (N,4) int32
+    [batch,x,y,z] voxel coordinates, without storing the neighbour map. One host sync (the pair count)."""
+    _dev(indices)
+    lib = _lib.load()
+    idx = indices.to(torch.int32).contiguous()
+    n, taps = idx.shape[0], ks ** 3
+    dev = idx.device
+    plan = ConvPlan()
+    plan.n, plan.taps = n, taps
+    plan.tap_ptr = torch.empty(taps + 1, dtype=torch.int32, device=dev)
+    count = torch.empty(1, dtype=torch.int64, device=dev)
+    nbytes = lib.ptv3_kmap_plan_workspace_bytes(n, int(ks))
+    ws = _ws(nbytes, dev)
+    _lib.check(lib.ptv3_kmap_plan_count(_ptr(idx), n, int(ks), _ptr(plan.tap_ptr), _ptr(count), _ptr(ws), nbytes,
+                                        _stream()), "ptv3_kmap_plan_count")
+    plan.n_pairs = int(count.item())
+    plan.row_ptr = torch.empty(n + 1, dtype=torch.int32, device=dev)
+    plan.pair_in = torch.empty(max(plan.n_pairs, 1), dtype=torch.int32, device=dev)
+    plan.pair_slot = torch.empty(max(plan.n_pairs, 1), dtype=torch.int32, device=dev)
+    _lib.check(lib.ptv3_kmap_plan_fill(_ptr(idx), n, int(ks), _ptr(plan.tap_ptr), _ptr(plan.row_ptr),
+                                       _ptr(plan.pair_in), _ptr(plan.pair_slot), _ptr(ws), nbytes, _stream()),
+               "ptv3_kmap_plan_fill")
+    return plan
+
+
 def subm_conv_pairs(feat, plan, weight, bias=None):
     """Submanifold convolution over the plan's active pairs only (fp16 / bf16)."""
     _dev(feat, weight, bias)

@@ -36,11 +36,15 @@ class SparseConvTensor:
         return nbr
 
     def conv_plan(self, kernel_size, indice_key=None):
-        """Pair lists of the neighbour map (see ops.conv_plan), cached like the map itself."""
+        """Pair lists of the neighbour map (see ops.conv_plan), cached like the map itself; built
+        straight from the coordinates unless the map has been built already."""
         key = ("plan", indice_key, kernel_size) if indice_key is not None else None
         if key is not None and key in self.indice_dict:
             return self.indice_dict[key]
-        plan = ops.conv_plan(self.neighbour_map(kernel_size, indice_key), tap_major=True)
+        if indice_key is not None and (indice_key, kernel_size) in self.indice_dict:
+            plan = ops.conv_plan(self.indice_dict[(indice_key, kernel_size)], tap_major=True)
+        else:
+            plan = ops.conv_plan_direct(self.indices, kernel_size)
         if key is not None:
             self.indice_dict[key] = plan
         return plan

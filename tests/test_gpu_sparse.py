@@ -149,6 +149,27 @@ def test_conv_plan_bit_exact(ks, n, extent):
     assert np.array_equal(plan.pair_slot.cpu().numpy()[:plan.n_pairs], slot_of[vi, ti])
 
 
+@pytest.mark.parametrize("ks,n,extent,nb", [(3, 1, 4, 1), (3, 777, 12, 2), (5, 3000, 20, 2), (3, 40_000, 48, 3),
+                                            (5, 30_000, 40, 2), (3, 5000, 300, 1)])
+def test_conv_plan_direct_equals_plan_of_map(ks, n, extent, nb):
+    # the pair lists built straight from the coordinates are those of the stored map, bit for bit
+    rng = np.random.default_rng(ks * 1000 + n)
+    idx, *_ = _indices(rng, n, extent, nb)
+    o = ops()
+    dev_idx = to_dev(idx)
+    ref = o.conv_plan(o.kmap_build(dev_idx, ks, tap_major=True), tap_major=True)
+    got = o.conv_plan_direct(dev_idx, ks)
+    assert got.n_pairs == ref.n_pairs and got.taps == ref.taps and got.n == ref.n
+    assert torch.equal(got.tap_ptr, ref.tap_ptr) and torch.equal(got.row_ptr, ref.row_ptr)
+    assert torch.equal(got.pair_in[:got.n_pairs], ref.pair_in[:ref.n_pairs])
+    assert torch.equal(got.pair_slot[:got.n_pairs], ref.pair_slot[:ref.n_pairs])
+    # and the oracle's map, tap-major, lists the same pairs
+    nbr = OI.subm_kmap(idx, ks)
+    t_idx, v_idx = np.nonzero(nbr.T >= 0)
+    assert got.n_pairs == len(t_idx)
+    assert np.array_equal(got.pair_in[:got.n_pairs].cpu().numpy(), nbr.T[t_idx, v_idx])
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("ks,cin,cout,n,extent", [(3, 32, 32, 3000, 20), (3, 64, 64, 50_000, 60), (3, 128, 128, 9000, 24),
                                                   (3, 256, 256, 2000, 12), (3, 512, 512, 600, 8), (5, 16, 32, 20_000, 40),
