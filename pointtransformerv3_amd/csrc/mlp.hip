@@ -177,15 +177,21 @@ int launch_mlp(const void* x, const void* resid, const void* w1, const void* b1,
 
 }  // namespace
 
+// wide channels (128, 256, 512): mlpwide.hip
+int mlp_wide_dispatch(const void* x, const void* resid, const void* w1, const void* b1, const void* w2, const void* b2,
+                      int dtype, int64_t n, int channels, void* out, hipStream_t stream);
+
 extern "C" int ptv3_mlp_fused(const void* x, const void* resid, const void* w1, const void* b1, const void* w2,
                               const void* b2, int dtype, int64_t n, int channels, int hidden, void* out,
                               void* stream_) {
     if (n < 0 || channels < 1 || hidden < 1) return PTV3_EINVAL;
     if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
-    if ((channels != 32 && channels != 64) || hidden != 4 * channels) return PTV3_ESHAPE;
+    const bool thin = channels == 32 || channels == 64, wide = channels == 128 || channels == 256 || channels == 512;
+    if ((!thin && !wide) || hidden != 4 * channels) return PTV3_ESHAPE;
     if (n == 0) return PTV3_OK;
     if (!x || !resid || !w1 || !b1 || !w2 || !b2 || !out) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
+    if (wide) return mlp_wide_dispatch(x, resid, w1, b1, w2, b2, dtype, n, channels, out, stream);
     if (dtype == PTV3_F16) {
         if (channels == 32) return launch_mlp<_Float16, 32>(x, resid, w1, b1, w2, b2, n, out, stream);
         return launch_mlp<_Float16, 64>(x, resid, w1, b1, w2, b2, n, out, stream);

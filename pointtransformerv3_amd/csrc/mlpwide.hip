@@ -1,0 +1,220 @@
+// Fused MLP for wide channels (C = 128, 256, 512; hidden = 4C; half precision):
+//   out = resid + fc2(GELU(fc1(x)))                       (model.py:493-516, :599-602)
+// As separate kernels this is three passes over an N x 4C tensor (fc1 writes it, GELU rewrites it,
+// fc2 reads it); here a work-group keeps a tile of rows on the CU for the whole chain.
+//
+// A work-group of 8 waves owns R = 64 or 128 rows. The hidden axis is cut into four chunks of C
+// units; per chunk, stage A computes GELU(x W1_chunk^T + b1) for the tile into LDS and stage B adds
+// its product with W2's chunk to the output accumulators, which stay in registers across the
+// chunks. Products are taken transposed with v_mfma_f32_32x32x16 (rows of the A operand = output
+// units, columns = points); a wave owns 64 points x 32*MT output units in both stages, reads the
+// point-side operand from LDS (the x tile in stage A, the hidden chunk in stage B) and streams
+// its own rows of W1 / W2 straight from L2 into operand registers, 64 contiguous bytes per weight
+// row and step. No two waves of a work-group with the same points share weight rows, so nothing
+// is fetched into LDS twice, and the weight stream runs DEPTH steps ahead in a ring of registers
+// that is never drained: its addresses do not depend on the tile, so it runs on across stages,
+// chunks and tiles of the persistent work-group.
+// Intermediates are rounded to the storage type where the separate layers would have stored them.
+#include "rowtile.h"
+
+namespace {
+
+constexpr int MW_THREADS = 512;
+constexpr int MW_WAVES = MW_THREADS / PTV3_WAVE;
+constexpr int MW_PAD = 8;   // halfs of padding per LDS row
+
+template <typename T, int C, int WM, int WN, int MT, int DEPTH>
+__global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
+    const T* __restrict__ x, const T* __restrict__ resid, const T* __restrict__ w1, const T* __restrict__ b1,
+    const T* __restrict__ w2, const T* __restrict__ b2, int64_t n, T* __restrict__ out) {
+    typedef typename H16<T>::v8 v8;
+    static_assert(WM * WN == MW_WAVES && C == 32 * MT * WN, "8 waves cover R x C");
+    constexpr int R = 64 * WM, H = 4 * C, XS = C + MW_PAD;
+    constexpr int KU = C / 32;            // 32-wide contraction steps per stage
+    constexpr int UNITS = 4 * 2 * KU;     // weight steps per tile: 4 chunks x (stage A, stage B)
+    static_assert(KU % DEPTH == 0, "the ring is indexed statically");
+    constexpr int PPR = C / 8;            // 16-byte pieces per row
+    constexpr int PIECES = R * PPR / MW_THREADS;
+    extern __shared__ __align__(16) unsigned char mw_smem[];
+    T* xt = (T*)mw_smem;      // [R][XS] input tile
+    T* ht = xt + R * XS;      // [R][XS] hidden chunk, then the output tile
+
+    const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
+    const int col = lane & 31, hf = lane >> 5;
+    const int wm = wave % WM, wn = wave / WM;
+    const int ch0 = wn * 32 * MT;   // first output unit of this wave (hidden unit inside a chunk / channel)
+    const int r0 = wm * 64;         // first row of this wave inside the tile
+
+    // weight step u: chunk u / (2 KU), stage (u / KU) & 1, 32-wide step u % KU; lane (col, hf) of
+    // output tile a takes 2 x 8 consecutive inputs of weight row ch0 + 32 a + col
+    auto issue = [&](int u, u32x4 (&r)[MT][2]) {
+        const int chunk = u / (2 * KU), st = (u / KU) & 1, kk = u % KU;
+#pragma unroll
+        for (int a = 0; a < MT; ++a) {
+            const int unit = ch0 + a * 32 + col;
+            const T* p = st == 0 ? w1 + (int64_t)(chunk * C + unit) * C + kk * 32 + hf * 16
+                                 : w2 + (int64_t)unit * H + chunk * C + kk * 32 + hf * 16;
+            r[a][0] = *(const u32x4*)p;
+            r[a][1] = *(const u32x4*)(p + 8);
+        }
+    };
+    u32x4 ring[DEPTH][MT][2];
+#pragma unroll
+    for (int j = 0; j < DEPTH; ++j) issue(j, ring[j]);
+
+    // one stage: acc[a][rt] += W rows (ring) x tile rows (LDS `src`); u0 = first weight step
+    auto stage = [&](const T* src, f32x16 (&acc)[MT][2], int u0) {
+        const T* brow = src + (r0 + col) * XS + hf * 16;
+        for (int kk0 = 0; kk0 < KU; kk0 += DEPTH) {
+#pragma unroll
+            for (int j = 0; j < DEPTH; ++j) {
+                const int kk = kk0 + j;
+                u32x4 bf[2][2];
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt) {
+                    bf[rt][0] = *(const u32x4*)(brow + rt * 32 * XS + kk * 32);
+                    bf[rt][1] = *(const u32x4*)(brow + rt * 32 * XS + kk * 32 + 8);
+                }
+                u32x4 af[MT][2];
+#pragma unroll
+                for (int a = 0; a < MT; ++a) {
+                    af[a][0] = ring[j][a][0];
+                    af[a][1] = ring[j][a][1];
+                }
+                int un = u0 + kk + DEPTH;
+                if (un >= UNITS) un -= UNITS;   // the stream of the next tile is the same
+                issue(un, ring[j]);
+#pragma unroll
+                for (int a = 0; a < MT; ++a)
+#pragma unroll
+                    for (int rt = 0; rt < 2; ++rt) {
+                        acc[a][rt] = H16<T>::mfma(__builtin_bit_cast(v8, af[a][0]), __builtin_bit_cast(v8, bf[rt][0]), acc[a][rt]);
+                        acc[a][rt] = H16<T>::mfma(__builtin_bit_cast(v8, af[a][1]), __builtin_bit_cast(v8, bf[rt][1]), acc[a][rt]);
+                    }
+            }
+        }
+    };
+
+    const int64_t n_tiles = (n + R - 1) / R;
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t row0 = tile * R;
+        // ---- x tile -> LDS
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            const int p = tid + i * MW_THREADS;
+            const int rr = p / PPR, pc = p % PPR;
+            u32x4 v = {0, 0, 0, 0};
+            if (row0 + rr < n) v = *(const u32x4*)(x + (row0 + rr) * C + pc * 8);
+            *(u32x4*)(xt + rr * XS + pc * 8) = v;
+        }
+        __syncthreads();
+
+        f32x16 acc[MT][2];
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[a][rt][v] = 0.f;
+
+        for (int chunk = 0; chunk < 4; ++chunk) {
+            f32x16 hacc[MT][2];
+#pragma unroll
+            for (int a = 0; a < MT; ++a)
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) hacc[a][rt][v] = 0.f;
+            stage(xt, hacc, chunk * 2 * KU);
+            // hacc[a][rt][v]: hidden unit ch0 + 32 a + 8 (v / 4) + 4 hf + v % 4 of row r0 + 32 rt + col
+#pragma unroll
+            for (int a = 0; a < MT; ++a)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int hh = ch0 + a * 32 + 8 * g + 4 * hf;
+                    const u32x2 bb = *(const u32x2*)(b1 + chunk * C + hh);
+                    const float bias[4] = {H16<T>::lo(bb[0]), H16<T>::hi(bb[0]), H16<T>::lo(bb[1]), H16<T>::hi(bb[1])};
+#pragma unroll
+                    for (int rt = 0; rt < 2; ++rt) {
+                        float hv[4];
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) hv[q] = gelu_erf(H16<T>::round(hacc[a][rt][4 * g + q] + bias[q]));
+                        *(u32x2*)(ht + (r0 + rt * 32 + col) * XS + hh) =
+                            (u32x2){H16<T>::pack2(hv[0], hv[1]), H16<T>::pack2(hv[2], hv[3])};
+                    }
+                }
+            __syncthreads();
+            stage(ht, acc, chunk * 2 * KU + KU);
+            __syncthreads();
+        }
+
+        // ---- fc2 + bias, rounded, parked in LDS; then resid + that in contiguous 16-byte pieces
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int cc = ch0 + a * 32 + 8 * g + 4 * hf;
+                const u32x2 bb = *(const u32x2*)(b2 + cc);
+                const float bias[4] = {H16<T>::lo(bb[0]), H16<T>::hi(bb[0]), H16<T>::lo(bb[1]), H16<T>::hi(bb[1])};
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt)
+                    *(u32x2*)(ht + (r0 + rt * 32 + col) * XS + cc) =
+                        (u32x2){H16<T>::pack2(acc[a][rt][4 * g] + bias[0], acc[a][rt][4 * g + 1] + bias[1]),
+                                H16<T>::pack2(acc[a][rt][4 * g + 2] + bias[2], acc[a][rt][4 * g + 3] + bias[3])};
+            }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            const int p = tid + i * MW_THREADS;
+            const int rr = p / PPR, pc = p % PPR;
+            if (row0 + rr < n) {
+                const u32x4 o = *(const u32x4*)(ht + rr * XS + pc * 8);
+                const u32x4 s = *(const u32x4*)(resid + (row0 + rr) * C + pc * 8);
+                u32x4 r;
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    r[k] = H16<T>::pack2(H16<T>::lo(o[k]) + H16<T>::lo(s[k]), H16<T>::hi(o[k]) + H16<T>::hi(s[k]));
+                *(u32x4*)(out + (row0 + rr) * C + pc * 8) = r;
+            }
+        }
+        // the next tile's first write to ht comes after the barrier that follows its x tile load
+    }
+}
+
+template <typename T, int C, int WM, int WN, int MT, int DEPTH>
+int launch_mlp_wide(const void* x, const void* resid, const void* w1, const void* b1, const void* w2, const void* b2,
+                    int64_t n, void* out, hipStream_t stream) {
+    constexpr int R = 64 * WM;
+    const size_t lds = (size_t)2 * R * (C + MW_PAD) * sizeof(T);
+    auto kern = mlp_wide_kernel<T, C, WM, WN, MT, DEPTH>;
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        configured = true;
+    }
+    // persistent work-groups: as many as the machine holds at a time
+    const int64_t tiles = (n + R - 1) / R;
+    const int64_t resident = 256;   // one work-group per CU: two waves per SIMD at this register count
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles < resident ? tiles : resident)), dim3(MW_THREADS), lds, stream,
+                       (const T*)x, (const T*)resid, (const T*)w1, (const T*)b1, (const T*)w2, (const T*)b2, n, (T*)out);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? PTV3_OK : (int)e;
+}
+
+}  // namespace
+
+// called by ptv3_mlp_fused for channels 128, 256 and 512
+int mlp_wide_dispatch(const void* x, const void* resid, const void* w1, const void* b1, const void* w2, const void* b2,
+                  int dtype, int64_t n, int channels, void* out, hipStream_t stream) {
+#define PTV3_MW(T)                                                                                                  \
+    do {                                                                                                            \
+        if (channels == 128) return launch_mlp_wide<T, 128, 2, 4, 1, 4>(x, resid, w1, b1, w2, b2, n, out, stream);   \
+        if (channels == 256) return launch_mlp_wide<T, 256, 1, 8, 1, 4>(x, resid, w1, b1, w2, b2, n, out, stream);   \
+        if (channels == 512) return launch_mlp_wide<T, 512, 1, 8, 2, 2>(x, resid, w1, b1, w2, b2, n, out, stream);   \
+    } while (0)
+    if (dtype == PTV3_F16) PTV3_MW(_Float16);
+    if (dtype == PTV3_BF16) PTV3_MW(__bf16);
+#undef PTV3_MW
+    return PTV3_ESHAPE;
+}

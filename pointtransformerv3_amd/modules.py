@@ -288,8 +288,10 @@ class Block(PointModule):
         plain_mlp = (type(mlp) is MLP and mlp.fc1.bias is not None and mlp.fc2.bias is not None
                      and not (self.training and mlp.drop.p > 0))
         exact_gelu = type(mlp.act) is nn.GELU and mlp.act.approximate == "none" if plain_mlp else False
-        fused = (plain_mlp and exact_gelu and self.channels in ops.MLP_FUSED_CHANNELS
-                 and mlp.fc1.out_features == 4 * self.channels and point.feat.dtype != torch.float32)
+        fusable = (plain_mlp and exact_gelu and mlp.fc1.out_features == 4 * self.channels
+                   and point.feat.dtype != torch.float32)
+        fused = fusable and self.channels in ops.MLP_FUSED_CHANNELS            # whole block head and tail
+        fused_mlp = fusable and self.channels in ops.MLP_ONLY_FUSED_PAYS          # the MLP alone
         # xCPE: conv reads the sparse view, which lags behind feat in the first decoder block
         conv = self.cpe[0](point.sparse_conv_feat).features
         if fused and type(self.cpe[1]) is nn.Linear and not (self.training and self.attn.proj_drop.p > 0):
@@ -311,8 +313,8 @@ class Block(PointModule):
         # When fc2 runs as a separate GEMM it accumulates onto the stored sum (beta = 1), so its
         # bias is added to that sum here: feat + fc2(h) + b2 without a separate add pass
         feat, normed = ops.layer_norm(point.feat, ln2.weight, ln2.bias, ln2.eps, residual=feat, mode=2,
-                                      shift=mlp.fc2.bias if (plain_mlp and not fused) else None)
-        if fused:
+                                      shift=mlp.fc2.bias if (plain_mlp and not fused_mlp) else None)
+        if fused_mlp:
             # fc1 + GELU + fc2 + residual in one kernel, the 4C-wide hidden tensor never leaves the CU
             feat = ops.mlp_fused(normed, feat, mlp.fc1.weight, mlp.fc1.bias, mlp.fc2.weight, mlp.fc2.bias)
         elif plain_mlp:

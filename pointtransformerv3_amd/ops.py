@@ -395,12 +395,14 @@ def layer_norm(x, weight, bias, eps=1e-5, residual=None, mode=0, weight2=None, b
     return out0 if mode < 2 else (out0, out1)
 
 
-MLP_FUSED_CHANNELS = (32, 64)
+MLP_FUSED_CHANNELS = (32, 64)             # widths of the fused block head / tail kernels
+MLP_ONLY_FUSED_CHANNELS = (32, 64, 128, 256, 512)   # widths the fused MLP kernel supports
+MLP_ONLY_FUSED_PAYS = (32, 64, 128)                 # widths at which it beats fc1, GELU and fc2 as three launches
 
 
 def mlp_fused(x, resid, w1, b1, w2, b2):
     """resid + fc2(GELU(fc1(x))) in one kernel (exact GELU). x, resid (N,C) fp16/bf16 with C in
-    MLP_FUSED_CHANNELS; w1 (4C,C), b1 (4C,), w2 (C,4C), b2 (C,)."""
+    MLP_ONLY_FUSED_CHANNELS; w1 (4C,C), b1 (4C,), w2 (C,4C), b2 (C,)."""
     _dev(x, resid, w1, b1, w2, b2)
     lib = _lib.load()
     x = x.contiguous()

@@ -213,7 +213,8 @@ def test_tap_major_layout_is_the_transpose():
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("c,n", [(32, 1), (32, 5000), (64, 33), (64, 70_001)])
+@pytest.mark.parametrize("c,n", [(32, 1), (32, 5000), (64, 33), (64, 70_001), (128, 1), (128, 300), (128, 40_001),
+                                 (256, 63), (256, 64), (256, 20_001), (512, 65), (512, 9000)])
 def test_mlp_fused_parity(dtype, c, n):
     import torch.nn.functional as F
     g = torch.Generator().manual_seed(c + n)
