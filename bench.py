@@ -105,6 +105,26 @@ def _time_us(fn, iters=20, warmup=3):
     return s.elapsed_time(e) * 1e3 / iters
 
 
+def attention_config2(reps):
+    """Baseline config 2 alone: Hilbert order of one room scene, patch 1024, C=512, 32 heads, fp16."""
+    from pointtransformerv3_amd import ops, synthetic
+    dev = "cuda:0"
+    sc = synthetic.room_scene(106_000, 2000, 0.02)
+    n2 = len(sc["grid_coord"])
+    g2 = torch.from_numpy(sc["grid_coord"]).to(dev)
+    b2 = torch.zeros(n2, dtype=torch.int64, device=dev)
+    order2, inv2 = ops.argsort_rows(ops.encode_orders(g2, b2, 9, ["hilbert"]), 28)
+    pad2, unpad2, cu2 = ops.pad_index(torch.tensor([n2], device=dev), [n2], 1024)
+    src2, dst2 = ops.attn_slots(order2[0], inv2[0], pad2, unpad2)
+    gen = torch.Generator(device="cpu").manual_seed(2)
+    qkv = (torch.randn(n2, 3 * 512, generator=gen) / 4).half().to(dev)
+    us = _time_us(lambda: ops.patch_attention(qkv, 32, src2, dst2, cu2, 1024, 0.25), iters=reps, warmup=1)
+    lens = torch.diff(cu2.long()).double()
+    fl = float(4.0 * (lens * lens).sum().item() * 512)
+    print(json.dumps({"kernel": "patch_attn_half_kernel<f16>", "points": n2, "sequences": int(len(cu2) - 1), "heads": 32,
+                      "us": us, "flops": fl, "tflops": fl / us / 1e6, "frac_mfma_peak": fl / us / 1e6 / MFMA_PEAK_TFLOPS}))
+
+
 def kernel_rooflines(path):
     """Per-kernel measurements at the sizes the baseline configs name, each against the roofline
     that bounds it (algorithmic bytes or flops / measured time). Written to `path` as JSON."""
@@ -135,6 +155,21 @@ def kernel_rooflines(path):
         us = _time_us(lambda: ops.argsort_rows(code, bits))
         add("argsort+inverse", f"4 x {n} codes, {bits} significant bits, {passes} passes", "hbm",
             4.0 * n * (passes * 24 + 16), us, f"B ({passes * 24 + 16} B per point and order)")
+    # ---- the same two at 16x the points (64 scenes): at 400k points these kernels run for a few
+    # microseconds each, a size at which launch and ramp-up, not bandwidth, set the time
+    reps = 16
+    g_big = g.repeat(reps, 1)
+    b_big = (b[None, :] + 4 * torch.arange(reps, device=dev)[:, None]).reshape(-1)
+    nb = n * reps
+    us = _time_us(lambda: ops.encode_orders(g_big, b_big, 9, orders), iters=10)
+    add("encode", f"{nb} points (64 scenes), 4 orders, depth 9", "hbm", nb * 52.0, us, "B (52 B/point)")
+    code_big = ops.encode_orders(g_big, b_big, 9, orders)
+    bits = 27 + 6
+    passes = (bits + 7) // 8
+    us = _time_us(lambda: ops.argsort_rows(code_big, bits), iters=5)
+    add("argsort+inverse", f"4 x {nb} codes, {bits} significant bits, {passes} passes", "hbm",
+        4.0 * nb * (passes * 24 + 16), us, f"B ({passes * 24 + 16} B per point and order)")
+    del code_big
     # ---- padding tables + slot tables
     off_host = [int(v) for v in d["offset"]]
     off = torch.from_numpy(d["offset"]).to(dev)
@@ -170,6 +205,17 @@ def kernel_rooflines(path):
     plan = ops.conv_plan(nbr, tap_major=True)
     add("conv_plan", f"{nv} voxels, {plan.n_pairs} active pairs", "hbm", nv * 27 * 4.0 * 2 + plan.n_pairs * 8.0 + nv * 4.0,
         us, "B (map read twice, pair lists written)")
+    us = _time_us(lambda: ops.conv_plan_direct(idx, 3), iters=10)
+    add("kmap+plan direct 3x3x3", f"{nv} voxels, {plan.n_pairs} active pairs", "hbm", nv * 16.0 + plan.n_pairs * 8.0 + nv * 4.0,
+        us, "B (coordinates read, pair lists written; no stored map)")
+    idx_big = torch.cat([torch.cat([b_big[:, None].int(), g_big.int()], 1)]).contiguous()
+    for ks in (3, 5):
+        us = _time_us(lambda: ops.conv_plan_direct(idx_big, ks), iters=5)
+        pb = ops.conv_plan_direct(idx_big, ks)
+        add(f"kmap+plan direct {ks}x{ks}x{ks}", f"{nb} voxels (64 scenes), {pb.n_pairs} active pairs", "hbm",
+            nb * 16.0 + pb.n_pairs * 8.0 + nb * 4.0, us, "B (coordinates read, pair lists written; no stored map)")
+        del pb
+    del idx_big
     feat = torch.randn(nv, 64, generator=gen).half().to(dev)
     w = ((torch.rand(64, 27, 64, generator=gen) * 2 - 1) / np.sqrt(27 * 64)).half().to(dev)
     bias = torch.zeros(64).half().to(dev)
@@ -191,6 +237,14 @@ def kernel_rooflines(path):
     child = torch.randn(m, 64, generator=gen).half().to(dev)
     us = _time_us(lambda: ops.unpool_add(x, child, cluster))
     add("unpool_add<f16>", f"{n} x 64", "hbm", (2 * n * 64 + m * 64) * 2.0 + 8.0 * n, us, "B")
+    # ---- fused MLP (fc1 + GELU + fc2 + residual) at the widths and sizes of the model's levels
+    for nm, cm in ((n, 64), (148_000, 128)):
+        xm = torch.randn(nm, cm, generator=gen).half().to(dev)
+        w1 = (torch.randn(4 * cm, cm, generator=gen) / cm ** 0.5).half().to(dev)
+        w2 = (torch.randn(cm, 4 * cm, generator=gen) / (4 * cm) ** 0.5).half().to(dev)
+        bm1, bm2 = torch.zeros(4 * cm).half().to(dev), torch.zeros(cm).half().to(dev)
+        us = _time_us(lambda: ops.mlp_fused(xm, xm, w1, bm1, w2, bm2))
+        add("mlp_fused<f16>", f"{nm} x {cm}, hidden {4 * cm}", "mfma", 16.0 * nm * cm * cm, us, "FLOP (16 N C^2)")
     wln = torch.ones(64).half().to(dev)
     us = _time_us(lambda: ops.layer_norm(x, wln, wln, 1e-5, residual=x, mode=2))
     add("layer_norm mode 2<f16>", f"{n} x 64", "hbm", 4.0 * n * 64 * 2, us, "B (2 reads, 2 writes)")
@@ -214,6 +268,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device copy (a kernel of known traffic) so that rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings of this process can be scaled to bytes")
+    ap.add_argument("--attention-config2", metavar="REPS", type=int, default=0,
+                    help="only run the patch attention kernel at baseline config 2 (one 100k-point scene, C=512, 32 "
+                         "heads, fp16) REPS times and print its rate: the command to put under rocprofv3 --pmc")
     ap.add_argument("--kernels", metavar="PATH", default=None,
                     help="also measure every kernel alone against its roofline and write the table to PATH")
     args = ap.parse_args()
@@ -224,6 +281,9 @@ def main():
 
     from pointtransformerv3_amd import PointTransformerV3, ops
 
+    if args.attention_config2 > 0:
+        attention_config2(args.attention_config2)
+        return
     dev = "cuda:0"
     torch.manual_seed(0)
     model = PointTransformerV3().eval().half()

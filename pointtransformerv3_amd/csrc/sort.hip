@@ -4,10 +4,12 @@
 // Replaces torch.argsort + scatter_ at model.py:119-126 and :667-674 of the reference.
 // Only the significant low bits are sorted (3*depth + batch bits, e.g. 29 instead of 64),
 // 8 bits per pass; all k rows share every launch (blockIdx.y = row). A pass is
-//   tile_hist  : per-tile digit histogram (LDS atomics)
-//   tile_scan  : per row, exclusive scan over (digit, tile) -> global start of every
-//                (tile, digit) run
-//   scatter    : stable rank inside the tile by wave-level digit matching, then one write
+//   tile_hist  : per-tile digit histogram (LDS atomics), digit totals of the row (global atomics)
+//   tile_scan  : global start of every (tile, digit) run: exclusive scan of the 256 digit totals,
+//                then per digit a running sum over the tiles; 16 blocks per row, 16 digits each
+//   scatter    : stable rank inside the tile by wave-level digit matching; the tile is put in
+//                digit order in LDS first, so that the global writes of one digit are contiguous
+//                runs instead of 4096 scattered 12-byte stores
 // The payload between passes is a 32-bit point index; int64 order/inverse appear only in
 // the last pass.
 #include "common.h"
@@ -17,12 +19,18 @@ namespace {
 constexpr int RADIX = 256;
 constexpr int SORT_THREADS = 256;
 constexpr int SORT_WAVES = SORT_THREADS / PTV3_WAVE;
-constexpr int SORT_ITEMS = 8;
+constexpr int SORT_ITEMS = 16;
 constexpr int SORT_TILE = SORT_THREADS * SORT_ITEMS;
+constexpr int MAX_PASSES = 8;
+
+__global__ __launch_bounds__(SORT_THREADS) void zero_totals_kernel(uint32_t* __restrict__ totals, int count) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) totals[i] = 0u;
+}
 
 __global__ __launch_bounds__(SORT_THREADS) void tile_hist_kernel(
     const int64_t* __restrict__ keys, int64_t n, int shift, uint32_t* __restrict__ tile_hist,
-    int tiles) {
+    int tiles, uint32_t* __restrict__ totals) {
     __shared__ uint32_t hist[RADIX];
     const int row = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
     hist[tid] = 0;
@@ -35,22 +43,35 @@ __global__ __launch_bounds__(SORT_THREADS) void tile_hist_kernel(
         if (i < n) atomicAdd(&hist[(uint32_t)((uint64_t)src[i] >> shift) & 255u], 1u);
     }
     __syncthreads();
-    tile_hist[((int64_t)row * tiles + tile) * RADIX + tid] = hist[tid];
+    const uint32_t c = hist[tid];
+    tile_hist[((int64_t)row * tiles + tile) * RADIX + tid] = c;
+    if (c) atomicAdd(&totals[row * RADIX + tid], c);
 }
 
-// One block of 1024 threads per row: thread (q, d) owns digit d over the q-th quarter of the
-// tiles. Quarter sums -> digit totals -> exclusive scan over digits; then every thread rescans
-// its quarter once, writing the final start of each (tile, digit) run.
-constexpr int SCAN_Q = 4;
-__global__ __launch_bounds__(RADIX * SCAN_Q) void tile_scan_kernel(uint32_t* __restrict__ tile_hist,
-                                                                   int tiles) {
-    __shared__ uint32_t part[SCAN_Q][RADIX];
-    __shared__ uint32_t total[RADIX];
+// grid (k, 16): block (row, dg) turns the counts of digits 16 dg .. 16 dg + 15 into global starts.
+// Thread (slice, d) owns one digit over one sixteenth of the tiles.
+constexpr int SCAN_SLICES = 16, SCAN_DIGITS = RADIX / SCAN_SLICES;
+__global__ __launch_bounds__(RADIX) void tile_scan_kernel(uint32_t* __restrict__ tile_hist, int tiles,
+                                                          const uint32_t* __restrict__ totals) {
+    __shared__ uint32_t base[RADIX];
+    __shared__ uint32_t part[SCAN_SLICES][SCAN_DIGITS];
     constexpr int CH = 8;
-    const int row = blockIdx.x, d = threadIdx.x % RADIX, q = threadIdx.x / RADIX;
-    const int per = (tiles + SCAN_Q - 1) / SCAN_Q;
-    const int t_lo = min(q * per, tiles), t_hi = min(t_lo + per, tiles);
-    uint32_t* h = tile_hist + (int64_t)row * tiles * RADIX + d;
+    const int row = blockIdx.x, dg = blockIdx.y, tid = threadIdx.x;
+    // exclusive scan of the row's digit totals (Hillis-Steele over 256 threads)
+    const uint32_t mine = totals[row * RADIX + tid];
+    base[tid] = mine;
+    __syncthreads();
+    for (int off = 1; off < RADIX; off <<= 1) {
+        const uint32_t v = tid >= off ? base[tid - off] : 0u;
+        __syncthreads();
+        base[tid] += v;
+        __syncthreads();
+    }
+    const int d = tid % SCAN_DIGITS, slice = tid / SCAN_DIGITS;
+    const int digit = dg * SCAN_DIGITS + d;
+    const int per = (tiles + SCAN_SLICES - 1) / SCAN_SLICES;
+    const int t_lo = min(slice * per, tiles), t_hi = min(t_lo + per, tiles);
+    uint32_t* h = tile_hist + (int64_t)row * tiles * RADIX + digit;
     uint32_t sum = 0;
     for (int t0 = t_lo; t0 < t_hi; t0 += CH) {
         uint32_t c[CH];
@@ -59,25 +80,10 @@ __global__ __launch_bounds__(RADIX * SCAN_Q) void tile_scan_kernel(uint32_t* __r
 #pragma unroll
         for (int j = 0; j < CH; ++j) sum += c[j];
     }
-    part[q][d] = sum;
+    part[slice][d] = sum;
     __syncthreads();
-    uint32_t qbase = 0, dtotal = 0;
-#pragma unroll
-    for (int k = 0; k < SCAN_Q; ++k) {
-        const uint32_t v = part[k][d];
-        if (k < q) qbase += v;
-        dtotal += v;
-    }
-    if (q == 0) total[d] = dtotal;
-    __syncthreads();
-    // Hillis-Steele inclusive scan over the 256 digit totals (first 256 threads; all hit the barriers)
-    for (int off = 1; off < RADIX; off <<= 1) {
-        const uint32_t v = (q == 0 && d >= off) ? total[d - off] : 0u;
-        __syncthreads();
-        if (q == 0) total[d] += v;
-        __syncthreads();
-    }
-    uint32_t run = total[d] - dtotal + qbase;   // digit base + tiles of earlier quarters
+    uint32_t run = base[digit] - totals[row * RADIX + digit];   // exclusive digit base
+    for (int k = 0; k < slice; ++k) run += part[k][d];
     for (int t0 = t_lo; t0 < t_hi; t0 += CH) {
         uint32_t c[CH];
 #pragma unroll
@@ -95,14 +101,19 @@ __global__ __launch_bounds__(SORT_THREADS) void scatter_kernel(
     const int64_t* __restrict__ keys_in, const int32_t* __restrict__ idx_in, int64_t n, int shift,
     const uint32_t* __restrict__ tile_off, int tiles, int64_t* __restrict__ keys_out,
     int32_t* __restrict__ idx_out, int64_t* __restrict__ order, int64_t* __restrict__ inverse) {
-    __shared__ uint32_t whist[SORT_WAVES][RADIX];
+    __shared__ uint32_t whist[SORT_WAVES][RADIX];   // per wave and digit: count, then start inside the sorted tile
+    __shared__ uint32_t gdelta[RADIX];              // global start of the digit's run minus its start inside the tile
+    __shared__ uint32_t wsum[SORT_WAVES];
+    __shared__ int64_t skey[SORT_TILE];
+    __shared__ int32_t sidx[SORT_TILE];
     const int row = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
     const int wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
     for (int w = 0; w < SORT_WAVES; ++w) whist[w][tid] = 0;
     __syncthreads();
 
     const int64_t rbase = (int64_t)row * n;
-    const int64_t wbase = (int64_t)tile * SORT_TILE + (int64_t)wave * (PTV3_WAVE * SORT_ITEMS);
+    const int64_t tbase = (int64_t)tile * SORT_TILE;
+    const int64_t wbase = tbase + (int64_t)wave * (PTV3_WAVE * SORT_ITEMS);
     int64_t key[SORT_ITEMS];
     int32_t idx[SORT_ITEMS];
     uint32_t rank[SORT_ITEMS];
@@ -114,6 +125,10 @@ __global__ __launch_bounds__(SORT_THREADS) void scatter_kernel(
         const bool valid = i < n;
         key[j] = valid ? keys_in[rbase + i] : 0;
         idx[j] = FIRST ? (int32_t)i : (valid ? idx_in[rbase + i] : 0);
+    }
+#pragma unroll
+    for (int j = 0; j < SORT_ITEMS; ++j) {
+        const bool valid = wbase + j * PTV3_WAVE + lane < n;
         const uint32_t digit = (uint32_t)((uint64_t)key[j] >> shift) & 255u;
         uint64_t peers = __ballot(valid);
 #pragma unroll
@@ -131,27 +146,51 @@ __global__ __launch_bounds__(SORT_THREADS) void scatter_kernel(
     }
     __syncthreads();
     {
-        // digit `tid`: turn per-wave counts into global starts of each wave's run
-        uint32_t run = tile_off[((int64_t)row * tiles + tile) * RADIX + tid];
-        for (int w = 0; w < SORT_WAVES; ++w) {
-            const uint32_t c = whist[w][tid];
-            whist[w][tid] = run;
-            run += c;
+        // digit `tid`: its start inside the sorted tile (exclusive scan of the tile histogram over
+        // the digits), the starts of each wave's run of it, and where the run goes globally
+        uint32_t c[SORT_WAVES], total = 0;
+#pragma unroll
+        for (int w = 0; w < SORT_WAVES; ++w) { c[w] = whist[w][tid]; total += c[w]; }
+        uint32_t x = total;
+#pragma unroll
+        for (int off = 1; off < PTV3_WAVE; off <<= 1) {
+            const uint32_t y = __shfl_up(x, off, PTV3_WAVE);
+            if (lane >= off) x += y;
         }
+        if (lane == PTV3_WAVE - 1) wsum[wave] = x;
+        __syncthreads();
+        uint32_t start = x - total;
+        for (int w = 0; w < wave; ++w) start += wsum[w];
+        gdelta[tid] = tile_off[((int64_t)row * tiles + tile) * RADIX + tid] - start;
+#pragma unroll
+        for (int w = 0; w < SORT_WAVES; ++w) { whist[w][tid] = start; start += c[w]; }
     }
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < SORT_ITEMS; ++j) {
-        const int64_t i = wbase + j * PTV3_WAVE + lane;
-        if (i < n) {
+        if (wbase + j * PTV3_WAVE + lane < n) {
             const uint32_t digit = (uint32_t)((uint64_t)key[j] >> shift) & 255u;
-            const int64_t pos = (int64_t)whist[wave][digit] + rank[j];
+            const uint32_t lp = whist[wave][digit] + rank[j];
+            skey[lp] = key[j];
+            sidx[lp] = idx[j];
+        }
+    }
+    __syncthreads();
+    const int count = (int)(n - tbase < SORT_TILE ? n - tbase : SORT_TILE);
+#pragma unroll
+    for (int j = 0; j < SORT_ITEMS; ++j) {
+        const int lp = j * SORT_THREADS + tid;
+        if (lp < count) {
+            const int64_t kv = skey[lp];
+            const int32_t iv = sidx[lp];
+            const uint32_t digit = (uint32_t)((uint64_t)kv >> shift) & 255u;
+            const int64_t pos = (int64_t)(uint32_t)(gdelta[digit] + (uint32_t)lp);
             if (LAST) {
-                order[rbase + pos] = idx[j];
-                inverse[rbase + idx[j]] = pos;
+                order[rbase + pos] = iv;
+                inverse[rbase + iv] = pos;
             } else {
-                keys_out[rbase + pos] = key[j];
-                idx_out[rbase + pos] = idx[j];
+                keys_out[rbase + pos] = kv;
+                idx_out[rbase + pos] = iv;
             }
         }
     }
@@ -161,6 +200,7 @@ struct SortWs {
     int64_t* keys[2];
     int32_t* idx[2];
     uint32_t* tile_hist;
+    uint32_t* totals;   // [MAX_PASSES][k][RADIX]
     size_t bytes;
 };
 
@@ -179,6 +219,8 @@ SortWs carve(void* base, int64_t n, int k) {
     }
     w.tile_hist = (uint32_t*)(p + off);
     off += ptv3_align256((size_t)k * tiles * RADIX * sizeof(uint32_t));
+    w.totals = (uint32_t*)(p + off);
+    off += ptv3_align256((size_t)MAX_PASSES * k * RADIX * sizeof(uint32_t));
     w.bytes = off;
     return w;
 }
@@ -203,6 +245,9 @@ extern "C" int ptv3_argsort(const int64_t* code, int64_t n, int k, int key_bits,
     const int tiles = (int)ptv3_ceil_div(n, SORT_TILE);
     const int passes = (key_bits + 7) / 8;
     const dim3 grid((unsigned)tiles, (unsigned)k), block(SORT_THREADS);
+    const int n_totals = passes * k * RADIX;
+    hipLaunchKernelGGL(zero_totals_kernel, dim3((unsigned)ptv3_ceil_div(n_totals, SORT_THREADS)), block, 0, stream,
+                       w.totals, n_totals);
 
     const int64_t* kin = code;
     const int32_t* iin = nullptr;
@@ -211,8 +256,10 @@ extern "C" int ptv3_argsort(const int64_t* code, int64_t n, int k, int key_bits,
         const bool first = (p == 0), last = (p == passes - 1);
         int64_t* kout = w.keys[p & 1];
         int32_t* iout = w.idx[p & 1];
-        hipLaunchKernelGGL(tile_hist_kernel, grid, block, 0, stream, kin, n, shift, w.tile_hist, tiles);
-        hipLaunchKernelGGL(tile_scan_kernel, dim3((unsigned)k), dim3(RADIX * SCAN_Q), 0, stream, w.tile_hist, tiles);
+        uint32_t* totals = w.totals + (size_t)p * k * RADIX;
+        hipLaunchKernelGGL(tile_hist_kernel, grid, block, 0, stream, kin, n, shift, w.tile_hist, tiles, totals);
+        hipLaunchKernelGGL(tile_scan_kernel, dim3((unsigned)k, SCAN_SLICES), dim3(RADIX), 0, stream, w.tile_hist, tiles,
+                           (const uint32_t*)totals);
 #define PTV3_SCATTER(F, L)                                                                    \
     hipLaunchKernelGGL((scatter_kernel<F, L>), grid, block, 0, stream, kin, iin, n, shift,    \
                        (const uint32_t*)w.tile_hist, tiles, kout, iout, order, inverse)
