@@ -107,3 +107,48 @@ def test_serialization_method_matches_oracle():
     p.sparsify()
     assert p.sparse_shape == [int(v) + 96 for v in d["grid_coord"].max(0)]
     assert p.sparse_conv_feat.indices.dtype == torch.int32 and p.sparse_conv_feat.batch_size == 3
+
+
+def _full_size_inputs(lidar):
+    if lidar:
+        d, feat = _data(0, 2, grid=0.05, seed=5000, lidar=True)     # baseline config 5: two ~120k-point sweeps
+    else:
+        d, feat = _data(106_000, 4, grid=0.02, seed=4000)           # baseline config 4: four ~100k-point rooms
+    return d, feat.astype(np.float16).astype(np.float32)
+
+
+@pytest.mark.parametrize("lidar", [False, True])
+def test_full_size_forward_properties(lidar):
+    """Baseline configs 4 and 5 at full size, where the CPU oracle takes minutes: properties that do
+    not depend on the size. (a) The order in which the points are stored is immaterial: every step
+    of the model is defined on coordinates (curve codes, voxel neighbours, grid clusters), so a
+    forward over shuffled rows gives the shuffled result. (b) Scenes of a batch do not interact in
+    inference (the scene id tops every code, patches and voxel neighbourhoods stay inside a
+    scene): scene 0 alone gives the rows of scene 0. (c) Two runs agree bit for bit."""
+    from pointtransformerv3_amd import PointTransformerV3
+    torch.manual_seed(4)
+    model = PointTransformerV3(in_channels=4 if lidar else 6, shuffle_orders=False).eval().half().to(DEV)
+    d, feat = _full_size_inputs(lidar)
+    n = len(feat)
+    assert n > 150_000
+
+    def run(dd, ff):
+        _draw_perms(11, False)   # same pooling row shuffles in every run
+        return _run(model, dd, ff, torch.float16).feat.float().cpu()
+
+    base = run(d, feat)
+    assert base.shape == (n, 64) and torch.isfinite(base).all()
+    assert torch.equal(run(d, feat), base)                                   # (c)
+    # (a) shuffle the rows inside every scene
+    rng = np.random.default_rng(1)
+    starts = np.concatenate([[0], d["offset"][:-1]])
+    perm = np.concatenate([s + rng.permutation(e - s) for s, e in zip(starts, d["offset"])])
+    dp = dict(d, grid_coord=d["grid_coord"][perm], coord=d["coord"][perm])
+    got = run(dp, feat[perm])
+    scale = float(base.abs().max())
+    assert float((got - base[perm]).abs().max()) / scale < 2e-2
+    # (b) the first scene alone
+    n0 = int(d["offset"][0])
+    d0 = dict(grid_coord=d["grid_coord"][:n0], coord=d["coord"][:n0], offset=d["offset"][:1])
+    alone = run(d0, feat[:n0])
+    assert float((alone - base[:n0]).abs().max()) / scale < 2e-2
