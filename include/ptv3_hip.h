@@ -87,6 +87,17 @@ int ptv3_patch_attn_fwd(const void *qkv, int dtype, int64_t n_rows, int channels
                         const int32_t *cu_seqlens, int64_t n_seq, int64_t max_seqlen,
                         float scale, void *out, void *stream);
 
+/* The same with the relative position bias of model.py:297-316, :468-469 (fp32 only: the reference
+ * applies it on its non-fused path, in float): score(query i, key j, head h) +=
+ * sum over the axes a of rpe_table[a * R + clamp(g_i[a] - g_j[a], -pos_bnd, pos_bnd) + pos_bnd][h],
+ * R = 2 * pos_bnd + 1; grid_coord (n_rows, 3) int32 in point order, rpe_table (3 * R, heads) fp32,
+ * pos_bnd <= 128. */
+int ptv3_patch_attn_rpe_fwd(const float *qkv, int64_t n_rows, int channels, int heads,
+                            const int32_t *slot_src, const int32_t *slot_dst,
+                            const int32_t *cu_seqlens, int64_t n_seq, int64_t max_seqlen, float scale,
+                            const int32_t *grid_coord, const float *rpe_table, int pos_bnd, float *out,
+                            void *stream);
+
 /* spconv.SubMConv3d's index generation (call sites model.py:546-552, :767-774, tensor built
  * at :165-172). indices (n,4) int32 [batch,x,y,z], coordinates in [0, 65535];
  * nbr int32, entry (voxel i, tap t = (kx*ks+ky)*ks+kz) = row of the voxel at

@@ -50,6 +50,10 @@ def _kmap(level, ks):
 
 
 def _attention(sd, name, level, x, heads, patch, order_index):
+    rpe = None
+    if name + ".rpe.rpe_table" in sd:
+        # the table is sized by the configured patch size, whatever the patch shrinks to (model.py:298-303, :371)
+        rpe = (level["grid_coord"], sd[name + ".rpe.rpe_table"], int((4 * patch) ** (1 / 3) * 2))
     if not level["flash"]:
         # without the fused path the patch shrinks to the smallest scene (model.py:441-444)
         patch = min(int(OI.offset2bincount(level["offset"]).min()), patch)
@@ -59,7 +63,7 @@ def _attention(sd, name, level, x, heads, patch, order_index):
     pad, unpad, cu = level[key]
     qkv = _linear(sd, name + ".qkv", x)
     out = OF.serialized_attention_core(qkv, level["order"][order_index], level["inverse"][order_index],
-                                       pad, unpad, cu, heads)
+                                       pad, unpad, cu, heads, rpe=rpe)
     return _linear(sd, name + ".proj", out)
 
 

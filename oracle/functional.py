@@ -17,9 +17,22 @@ import torch
 import torch.nn.functional as F
 
 
-def patch_attention(qkv, cu_seqlens, num_heads, scale=None):
+def rpe_bias(coord, table, pos_bnd):
+    """Relative position bias of one patch (model.py:297-316, :375-379): coord (L, 3) integer grid
+    coordinates in patch order, table (3 * R, H) with R = 2 * pos_bnd + 1. Returns (H, L, L) with
+    entry [h, i, j] = sum over axes a of table[a * R + clamp(coord[i, a] - coord[j, a]) + pos_bnd, h]."""
+    coord = torch.as_tensor(np.asarray(coord), dtype=torch.int64)
+    table = torch.as_tensor(table, dtype=torch.float32)
+    rnum = 2 * pos_bnd + 1
+    rel = coord[:, None, :] - coord[None, :, :]                                   # (L, L, 3): query - key
+    idx = rel.clamp(-pos_bnd, pos_bnd) + pos_bnd + torch.arange(3) * rnum
+    return table[idx.reshape(-1)].reshape(idx.shape + (-1,)).sum(2).permute(2, 0, 1)
+
+
+def patch_attention(qkv, cu_seqlens, num_heads, scale=None, rpe=None):
     """qkv: (Npad, 3*C) fp32 rows already in padded serialized order, channel layout
-    [3][H][D] (model.py:461,477). Returns (Npad, C)."""
+    [3][H][D] (model.py:461,477). rpe = (coord (Npad, 3) in the same order, table, pos_bnd) adds the
+    relative position bias to the scores (model.py:468-469). Returns (Npad, C)."""
     qkv = torch.as_tensor(qkv, dtype=torch.float32)
     npad, c3 = qkv.shape
     C = c3 // 3
@@ -30,7 +43,10 @@ def patch_attention(qkv, cu_seqlens, num_heads, scale=None):
     for s, e in zip(cu[:-1], cu[1:]):
         blk = qkv[s:e].reshape(e - s, 3, num_heads, D).permute(1, 2, 0, 3)  # (3,H,L,D)
         q, k, v = blk[0], blk[1], blk[2]
-        attn = torch.softmax((q * scale) @ k.transpose(-2, -1), dim=-1)
+        score = (q * scale) @ k.transpose(-2, -1)
+        if rpe is not None:
+            score = score + rpe_bias(np.asarray(rpe[0])[s:e], rpe[1], rpe[2])
+        attn = torch.softmax(score, dim=-1)
         out[s:e] = (attn @ v).transpose(0, 1).reshape(e - s, C)
     return out
 
@@ -57,13 +73,16 @@ def patch_attention_bruteforce(qkv, cu_seqlens, num_heads, scale=None):
 
 
 def serialized_attention_core(feat_qkv, order, inverse, pad, unpad, cu_seqlens, num_heads,
-                              scale=None):
+                              scale=None, rpe=None):
     """model.py:452-484: gather rows into padded serialized order, attend inside each
-    patch, keep each point's primary slot. feat_qkv: (N, 3C). Returns (N, C)."""
+    patch, keep each point's primary slot. feat_qkv: (N, 3C); rpe = (grid_coord (N, 3) in point
+    order, table, pos_bnd). Returns (N, C)."""
     feat_qkv = torch.as_tensor(feat_qkv, dtype=torch.float32)
     gidx = torch.as_tensor(np.asarray(order)[np.asarray(pad)])
     back = torch.as_tensor(np.asarray(unpad)[np.asarray(inverse)])
-    out = patch_attention(feat_qkv[gidx], cu_seqlens, num_heads, scale)
+    if rpe is not None:
+        rpe = (np.asarray(rpe[0])[gidx.numpy()], rpe[1], rpe[2])
+    out = patch_attention(feat_qkv[gidx], cu_seqlens, num_heads, scale, rpe)
     return out[back]
 
 

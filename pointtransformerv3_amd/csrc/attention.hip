@@ -394,6 +394,94 @@ __global__ __launch_bounds__(F32_QB) void patch_attn_f32_kernel(
     }
 }
 
+// ---- fp32 with relative position bias (model.py:297-316, :468-469): as above, and every score
+// gets table[clamp(dx) + b][h] + table[R + clamp(dy) + b][h] + table[2R + clamp(dz) + b][h] for the
+// grid offset (dx, dy, dz) = query - key, b = pos_bnd, R = 2 b + 1. The head's 3R table entries and
+// the chunk's key coordinates sit in LDS.
+constexpr int RPE_MAX_BND = 128;
+
+__global__ __launch_bounds__(F32_QB) void patch_attn_rpe_f32_kernel(
+    const float* __restrict__ qkv, int channels, int heads, const int32_t* __restrict__ slot_src,
+    const int32_t* __restrict__ slot_dst, const int32_t* __restrict__ cu_seqlens, int q_blocks,
+    float scale, const int32_t* __restrict__ grid_coord, const float* __restrict__ rpe_table, int pos_bnd,
+    float* __restrict__ out) {
+    __shared__ float k_lds[F32_KC][HD];
+    __shared__ float v_lds[F32_KC][HD];
+    __shared__ int32_t c_lds[F32_KC][3];
+    __shared__ float t_lds[3 * (2 * RPE_MAX_BND + 1)];
+    const int seq = blockIdx.x / (heads * q_blocks);
+    const int rem = blockIdx.x % (heads * q_blocks);
+    const int head = rem / q_blocks, qb = rem % q_blocks;
+    const int s0 = cu_seqlens[seq];
+    const int len = cu_seqlens[seq + 1] - s0;
+    if (qb * F32_QB >= len) return;
+    const int tid = threadIdx.x;
+    const int qi = qb * F32_QB + tid;
+    const int64_t row_stride = 3 * (int64_t)channels;
+    const int rnum = 2 * pos_bnd + 1;
+    for (int e = tid; e < 3 * rnum; e += F32_QB) t_lds[e] = rpe_table[(int64_t)e * heads + head];
+
+    float q[HD], o[HD];
+    int dst = -1, qx = 0, qy = 0, qz = 0;
+#pragma unroll
+    for (int d = 0; d < HD; ++d) { q[d] = 0.f; o[d] = 0.f; }
+    if (qi < len) {
+        dst = slot_dst[s0 + qi];
+        const int64_t r = slot_src[s0 + qi];
+        const float* src = qkv + r * row_stride + head * HD;
+#pragma unroll
+        for (int d = 0; d < HD; ++d) q[d] = src[d] * scale;
+        qx = grid_coord[3 * r];
+        qy = grid_coord[3 * r + 1];
+        qz = grid_coord[3 * r + 2];
+    }
+    float m = -INFINITY, l = 0.f;
+    for (int c0 = 0; c0 < len; c0 += F32_KC) {
+        __syncthreads();
+        for (int e = tid; e < F32_KC * HD; e += F32_QB) {
+            const int key = e / HD, d = e % HD;
+            float kv = 0.f, vv = 0.f;
+            if (c0 + key < len) {
+                const int64_t r = slot_src[s0 + c0 + key];
+                const float* src = qkv + r * row_stride + head * HD + d;
+                kv = src[channels];
+                vv = src[2 * channels];
+                if (d < 3) c_lds[key][d] = grid_coord[3 * r + d];
+            }
+            k_lds[key][d] = kv;
+            v_lds[key][d] = vv;
+        }
+        __syncthreads();
+        const int kn = min(F32_KC, len - c0);
+        for (int key = 0; key < kn; ++key) {
+            float s = 0.f;
+#pragma unroll
+            for (int d = 0; d < HD; ++d) s = fmaf(q[d], k_lds[key][d], s);
+            const int dx = min(max(qx - c_lds[key][0], -pos_bnd), pos_bnd) + pos_bnd;
+            const int dy = min(max(qy - c_lds[key][1], -pos_bnd), pos_bnd) + pos_bnd;
+            const int dz = min(max(qz - c_lds[key][2], -pos_bnd), pos_bnd) + pos_bnd;
+            s += t_lds[dx] + t_lds[rnum + dy] + t_lds[2 * rnum + dz];
+            if (s > m) {
+                const float a = __expf(m - s);
+                l *= a;
+#pragma unroll
+                for (int d = 0; d < HD; ++d) o[d] *= a;
+                m = s;
+            }
+            const float p = __expf(s - m);
+            l += p;
+#pragma unroll
+            for (int d = 0; d < HD; ++d) o[d] = fmaf(p, v_lds[key][d], o[d]);
+        }
+    }
+    if (dst >= 0) {
+        const float inv = 1.f / l;
+        float* dstp = out + (int64_t)dst * channels + head * HD;
+#pragma unroll
+        for (int d = 0; d < HD; ++d) dstp[d] = o[d] * inv;
+    }
+}
+
 template <typename T>
 int launch_half(const void* qkv, int channels, int heads, const int32_t* slot_src,
                 const int32_t* slot_dst, const int32_t* cu_seqlens, int64_t n_seq,
@@ -463,5 +551,23 @@ extern "C" int ptv3_patch_attn_fwd(const void* qkv, int dtype, int64_t n_rows, i
     hipLaunchKernelGGL(patch_attn_f32_kernel, dim3((unsigned)(n_seq * heads * q_blocks)), dim3(F32_QB),
                        0, stream, (const float*)qkv, channels, heads, slot_src, slot_dst, cu_seqlens,
                        q_blocks, scale, (float*)out);
+    PTV3_RETURN_LAUNCH();
+}
+
+extern "C" int ptv3_patch_attn_rpe_fwd(const float* qkv, int64_t n_rows, int channels, int heads,
+                                       const int32_t* slot_src, const int32_t* slot_dst,
+                                       const int32_t* cu_seqlens, int64_t n_seq, int64_t max_seqlen, float scale,
+                                       const int32_t* grid_coord, const float* rpe_table, int pos_bnd, float* out,
+                                       void* stream_) {
+    if (n_rows < 0 || n_seq < 0 || channels < 1 || heads < 1 || max_seqlen < 1) return PTV3_EINVAL;
+    if (pos_bnd < 0 || pos_bnd > RPE_MAX_BND) return PTV3_ESHAPE;
+    if (channels % heads != 0 || channels / heads != HD) return PTV3_ESHAPE;
+    if (n_seq == 0 || n_rows == 0) return PTV3_OK;
+    if (!qkv || !slot_src || !slot_dst || !cu_seqlens || !grid_coord || !rpe_table || !out) return PTV3_EINVAL;
+    const int q_blocks = (int)ptv3_ceil_div(max_seqlen, F32_QB);
+    if (n_seq * heads * q_blocks >= (1ll << 31)) return PTV3_EINVAL;
+    hipLaunchKernelGGL(patch_attn_rpe_f32_kernel, dim3((unsigned)(n_seq * heads * q_blocks)), dim3(F32_QB), 0,
+                       (hipStream_t)stream_, qkv, channels, heads, slot_src, slot_dst, cu_seqlens, q_blocks, scale,
+                       grid_coord, rpe_table, pos_bnd, out);
     PTV3_RETURN_LAUNCH();
 }

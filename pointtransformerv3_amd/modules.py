@@ -154,6 +154,26 @@ class PDNorm(PointModule):
         return point
 
 
+class RPE(nn.Module):
+    """Relative position bias table (model.py:297-316): one learned value per axis, clamped grid
+    offset and head. The attention kernel reads the table directly; forward() is the reference's
+    dense (N, H, K, K) bias for callers that want it."""
+
+    def __init__(self, patch_size, num_heads):
+        super().__init__()
+        self.patch_size, self.num_heads = patch_size, num_heads
+        self.pos_bnd = int((4 * patch_size) ** (1 / 3) * 2)
+        self.rpe_num = 2 * self.pos_bnd + 1
+        self.rpe_table = nn.Parameter(torch.zeros(3 * self.rpe_num, num_heads))
+        nn.init.trunc_normal_(self.rpe_table, std=0.02)
+
+    def forward(self, coord):
+        idx = (coord.clamp(-self.pos_bnd, self.pos_bnd) + self.pos_bnd
+               + torch.arange(3, device=coord.device) * self.rpe_num)
+        out = self.rpe_table.index_select(0, idx.reshape(-1))
+        return out.view(idx.shape + (-1,)).sum(3).permute(0, 3, 1, 2)
+
+
 class SerializedAttention(PointModule):
     """Attention inside patches of the serialized point sequence (model.py:319-490).
 
@@ -172,11 +192,8 @@ class SerializedAttention(PointModule):
         self.order_index = order_index
         self.upcast_attention, self.upcast_softmax = upcast_attention, upcast_softmax
         self.enable_rpe, self.enable_flash = enable_rpe, enable_flash
-        if enable_rpe:
-            raise NotImplementedError(
-                "relative position bias is not covered by the HIP attention kernel; it is "
-                "mutually exclusive with the flash path every released PTv3 config uses")
         if enable_flash:
+            assert enable_rpe is False, "Set enable_rpe to False when enable Flash Attention"
             assert upcast_attention is False, "Set upcast_attention to False when enable Flash Attention"
             assert upcast_softmax is False, "Set upcast_softmax to False when enable Flash Attention"
             self.patch_size = patch_size
@@ -190,6 +207,7 @@ class SerializedAttention(PointModule):
         self.qkv = nn.Linear(channels, channels * 3, bias=qkv_bias)
         self.proj = nn.Linear(channels, channels)
         self.proj_drop = nn.Dropout(proj_drop)
+        self.rpe = RPE(patch_size, num_heads) if enable_rpe else None
 
     @torch.no_grad()
     def get_padding_and_inverse(self, point):
@@ -217,6 +235,12 @@ class SerializedAttention(PointModule):
             self.patch_size = min(int(sizes.min()), self.patch_size_max)
         _, _, cu_seqlens = self.get_padding_and_inverse(point)
         slot_src, slot_dst = self._slots(point)
+        if self.enable_rpe:
+            # bias from the grid offsets of (query, key) inside the patch, added before the softmax; the
+            # reference takes this path in float (upcast_attention / upcast_softmax, model.py:463-471)
+            out = ops.patch_attention_rpe(qkv.float(), self.num_heads, slot_src, slot_dst, cu_seqlens, self.patch_size,
+                                          self.scale, point.grid_coord, self.rpe.rpe_table, self.rpe.pos_bnd)
+            return out.to(qkv.dtype)
         if self.enable_flash and qkv.dtype == torch.float32:
             # the fused path of the reference always computes in half precision (model.py:477,483)
             return ops.patch_attention(qkv.half(), self.num_heads, slot_src, slot_dst, cu_seqlens,

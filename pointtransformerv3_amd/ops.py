@@ -154,6 +154,29 @@ def patch_attention(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, 
     return out
 
 
+def patch_attention_rpe(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale, grid_coord, rpe_table,
+                        pos_bnd):
+    """patch_attention with the relative position bias of model.py:297-316 added to every score:
+    fp32 qkv (N, 3C), grid_coord (N, 3) in point order, rpe_table (3 * (2 * pos_bnd + 1), H)."""
+    _dev(qkv, slot_src, slot_dst, cu_seqlens, grid_coord, rpe_table)
+    lib = _lib.load()
+    if qkv.dtype != torch.float32:
+        raise _lib.Ptv3Error("the relative position bias path computes in float32, as the reference's does")
+    qkv = qkv.contiguous()
+    n, c3 = qkv.shape
+    c = c3 // 3
+    g = grid_coord.to(torch.int32).contiguous()
+    t = rpe_table.to(torch.float32).contiguous()
+    if t.shape != (3 * (2 * pos_bnd + 1), num_heads) or g.shape != (n, 3):
+        raise _lib.Ptv3Error("rpe_table must be (3 * (2 * pos_bnd + 1), heads) and grid_coord (N, 3)")
+    out = torch.empty((n, c), dtype=torch.float32, device=qkv.device)
+    _lib.check(lib.ptv3_patch_attn_rpe_fwd(_ptr(qkv), n, c, int(num_heads), _ptr(slot_src), _ptr(slot_dst),
+                                           _ptr(cu_seqlens), cu_seqlens.shape[0] - 1, int(max_seqlen), float(scale),
+                                           _ptr(g), _ptr(t), int(pos_bnd), _ptr(out), _stream()),
+               "ptv3_patch_attn_rpe_fwd")
+    return out
+
+
 def kmap_build(indices, ks, tap_major=False):
     """int32 neighbour map of (N,4) int32 [batch,x,y,z] voxels: (N, ks^3), or (ks^3, N) when
     tap_major (the layout the convolution kernels read coalesced)."""

@@ -95,3 +95,64 @@ def test_attention_config2_shape_bf16_sampled():
         sel = torch.as_tensor(rows[s:e][primary])
         err = (got[sel] - want[torch.as_tensor(primary)]).abs().max() / want.abs().max()
         assert err < 2e-2, (p, float(err))
+
+
+@pytest.mark.parametrize("counts,patch", [([64], 64), ([700, 300], 256), ([2500], 1024)])
+def test_attention_rpe_parity_fp32(counts, patch):
+    """Relative position bias path (fp32): kernel vs the CPU oracle, table drawn like the reference's."""
+    heads, seed = 4, 31
+    rng = np.random.default_rng(seed)
+    g = torch.Generator().manual_seed(seed)
+    n = int(sum(counts))
+    C = heads * 16
+    offset = np.cumsum(counts).astype(np.int64)
+    starts = np.concatenate([[0], offset[:-1]])
+    order = np.concatenate([s + rng.permutation(c) for s, c in zip(starts, counts)]).astype(np.int64)
+    inverse = np.empty(n, np.int64)
+    inverse[order] = np.arange(n)
+    qkv = torch.randn(n, 3 * C, generator=g)
+    grid = rng.integers(0, 60, size=(n, 3)).astype(np.int32)
+    pos_bnd = int((4 * patch) ** (1 / 3) * 2)
+    table = torch.randn(3 * (2 * pos_bnd + 1), heads, generator=g) * 0.5
+    pad, unpad, cu = OI.padding_tables(offset, patch)
+    want = OF.serialized_attention_core(qkv, order, inverse, pad, unpad, cu, heads, rpe=(grid, table, pos_bnd))
+    o = ops()
+    gp, gu, gc = o.pad_index(to_dev(offset), offset.tolist(), patch)
+    src, dst = o.attn_slots(to_dev(order), to_dev(inverse), gp, gu)
+    got = o.patch_attention_rpe(qkv.to(DEV), heads, src, dst, gc, patch, 16 ** -0.5, to_dev(grid), table.to(DEV), pos_bnd)
+    assert rel_err(got, want) < 1e-4
+    zero = o.patch_attention_rpe(qkv.to(DEV), heads, src, dst, gc, patch, 16 ** -0.5, to_dev(grid),
+                                 torch.zeros_like(table).to(DEV), pos_bnd)
+    plain = o.patch_attention(qkv.to(DEV), heads, src, dst, gc, patch, 16 ** -0.5)
+    assert rel_err(zero, plain.cpu()) < 1e-5
+
+
+def test_attention_module_with_rpe():
+    """SerializedAttention(enable_rpe=True, enable_flash=False) as the reference builds it (model.py:319-490):
+    the patch shrinks to the smallest scene, the bias table is the module's parameter `rpe.rpe_table`."""
+    from pointtransformerv3_amd import Point
+    from pointtransformerv3_amd.modules import SerializedAttention
+    rng = np.random.default_rng(8)
+    torch.manual_seed(8)
+    C, heads = 64, 4
+    attn = SerializedAttention(C, heads, patch_size=128, order_index=0, enable_rpe=True, enable_flash=False).eval()
+    assert attn.rpe.rpe_table.shape == (3 * (2 * int((4 * 128) ** (1 / 3) * 2) + 1), heads)
+    assert "rpe.rpe_table" in attn.state_dict()
+    counts = [150, 260]
+    n = sum(counts)
+    grid = rng.integers(0, 40, size=(n, 3)).astype(np.int32)
+    offset = np.cumsum(counts).astype(np.int64)
+    feat = torch.randn(n, C)
+    p = Point(feat=feat.to(DEV), grid_coord=torch.from_numpy(grid).to(DEV), offset=torch.from_numpy(offset).to(DEV))
+    p.serialization(order=["z"])
+    with torch.inference_mode():
+        got = attn.to(DEV)(p).feat.cpu()
+    patch = 128                                              # min(150, 260, 128)
+    order, inverse = p.serialized_order[0].cpu().numpy(), p.serialized_inverse[0].cpu().numpy()
+    pad, unpad, cu = OI.padding_tables(offset, patch)
+    sd = {k: v.cpu() for k, v in attn.state_dict().items()}
+    qkv = torch.nn.functional.linear(feat, sd["qkv.weight"], sd["qkv.bias"])
+    core = OF.serialized_attention_core(qkv, order, inverse, pad, unpad, cu, heads,
+                                        rpe=(grid, sd["rpe.rpe_table"], attn.rpe.pos_bnd))
+    want = torch.nn.functional.linear(core, sd["proj.weight"], sd["proj.bias"])
+    assert rel_err(got, want) < 1e-4

@@ -152,3 +152,28 @@ def test_full_size_forward_properties(lidar):
     d0 = dict(grid_coord=d["grid_coord"][:n0], coord=d["coord"][:n0], offset=d["offset"][:1])
     alone = run(d0, feat[:n0])
     assert float((alone - base[:n0]).abs().max()) / scale < 2e-2
+
+
+def test_forward_fp32_with_relative_position_bias():
+    """enable_rpe=True on the non-fused attention path (model.py:297-316, :468-469): every block owns a
+    table `attn.rpe.rpe_table`; the whole forward against the CPU oracle."""
+    from pointtransformerv3_amd import PointTransformerV3
+    kw = dict(enc_depths=(1, 1, 1, 1, 1), dec_depths=(1, 1, 1, 1), enc_patch_size=(256,) * 5, dec_patch_size=(256,) * 4)
+    torch.manual_seed(6)
+    model = PointTransformerV3(shuffle_orders=False, enable_flash=False, enable_rpe=True, upcast_attention=True,
+                               upcast_softmax=True, **kw).eval()
+    sd = model.state_dict()
+    assert "enc.enc0.block0.attn.rpe.rpe_table" in sd and "dec.dec3.block0.attn.rpe.rpe_table" in sd
+    with torch.no_grad():
+        for k, v in sd.items():
+            if k.endswith("rpe_table"):
+                v.mul_(60.0)     # the initial std of 0.02 would hide the bias below the tolerance
+    d, feat = _data(2500, 2)
+    perms = _draw_perms(9, False)
+    want = ptv3_forward(model.state_dict(), d["grid_coord"], feat, d["offset"], enable_flash=False, perms=perms, **kw)
+    without = ptv3_forward({k: v for k, v in model.state_dict().items() if not k.endswith("rpe_table")},
+                           d["grid_coord"], feat, d["offset"], enable_flash=False, perms=perms, **kw)
+    assert float((want - without).abs().max() / want.abs().max()) > 1e-2     # the bias matters in this test
+    _draw_perms(9, False)
+    point = _run(model.to(DEV), d, feat, torch.float32)
+    assert rel_err(point.feat, want) < 1e-4

@@ -176,3 +176,35 @@ def test_segment_csr_and_unpool():
         np.allclose(OF.segment_csr(src, indices, ptr, "mean").numpy(), [[0., 7.], [8 / 3, 7 / 3]])
     out = OF.unpool_add(torch.ones(3, 2), torch.tensor([[1., 2.], [10., 20.]]), [1, 0, 1])
     assert out.tolist() == [[11., 21.], [2., 3.], [11., 21.]]
+
+
+def test_rpe_bias_and_attention_with_bias():
+    """Relative position bias (model.py:297-316, :468-469). Pins: a per-pair loop straight from the
+    definition; a hand case (offset (+1, 0, -40) with pos_bnd 3 reads table rows 4, 7+3, 14+0); the
+    clamp; a zero table changes nothing; softmax with the bias equals torch's
+    scaled_dot_product_attention with the bias passed as an additive mask."""
+    rng = np.random.default_rng(5)
+    g = torch.Generator().manual_seed(5)
+    L, H, bnd = 37, 3, 3
+    rnum = 2 * bnd + 1
+    coord = rng.integers(0, 12, size=(L, 3))
+    table = torch.randn(3 * rnum, H, generator=g)
+    bias = OF.rpe_bias(coord, table, bnd)
+    assert bias.shape == (H, L, L)
+    for i, j in ((0, 0), (3, 17), (36, 5), (11, 30)):
+        want = torch.zeros(H)
+        for a in range(3):
+            d = int(np.clip(coord[i, a] - coord[j, a], -bnd, bnd))
+            want += table[a * rnum + d + bnd]
+        assert torch.allclose(bias[:, i, j], want, atol=1e-6)
+    two = OF.rpe_bias(np.array([[5, 2, 0], [4, 2, 40]]), table, bnd)     # query 0 - key 1 = (+1, 0, -40)
+    assert torch.allclose(two[:, 0, 1], table[4] + table[rnum + 3] + table[2 * rnum + 0], atol=1e-6)
+    assert torch.allclose(two[:, 1, 0], table[2] + table[rnum + 3] + table[2 * rnum + 6], atol=1e-6)
+    qkv = torch.randn(L, 3 * H * 16, generator=g)
+    plain = OF.patch_attention(qkv, [0, L], H)
+    assert torch.allclose(OF.patch_attention(qkv, [0, L], H, rpe=(coord, torch.zeros_like(table), bnd)), plain, atol=1e-6)
+    got = OF.patch_attention(qkv, [0, L], H, rpe=(coord, table, bnd))
+    assert not torch.allclose(got, plain, atol=1e-3)
+    q, k, v = qkv.reshape(L, 3, H, 16).permute(1, 2, 0, 3)
+    want = F.scaled_dot_product_attention(q[None], k[None], v[None], attn_mask=bias[None])[0]
+    assert torch.allclose(got, want.transpose(0, 1).reshape(L, H * 16), atol=1e-5)
