@@ -12,14 +12,18 @@
 //     query (column) and 16 keys (rows). Row max / rescale are then lane-local apart from a
 //     single exchange with lane^32, and the fp32 result registers, converted to 16-bit,
 //     are already in operand layout for the second product O^T = V^T * P^T.
-//   * V^T only fills 16 of the 32 rows of that product; rows 16 and 20 are fed ones so the
-//     softmax denominator falls out of the same MFMA instead of costing VALU adds.
-//   * At head_dim 16 the kernel is bound by the exponentials (one quarter-rate v_exp_f32 per
-//     score against 64 MFMA flops), so everything else is taken off the VALU: q is scaled by
-//     scale*log2(e) once, the running reference maximum enters through the MFMA's C operand
-//     so scores arrive already shifted, and the reference only moves when a score exceeds it
-//     by 2^8 -- which a |q||k| bound rules out for most 64-key steps without looking at the
-//     scores.
+//   * V^T only fills 16 of the 32 rows of that product; rows 16 and 20 are fed ones (from a small
+//     LDS constant, by per-lane addressing) so the softmax denominator falls out of the same MFMA
+//     instead of costing VALU adds.
+//   * At head_dim 16 the kernel is bound by the softmax arithmetic, not by the MFMAs: per 64 keys x
+//     32 queries a wave issues 6 MFMAs (128 useful MFMA cycles) but 32 v_exp_f32 (8 issue cycles
+//     each on this part) and 16 packed conversions (4 each), 320 VALU cycles. Everything else is
+//     therefore taken off the VALU: q is scaled by scale*log2(e) once; a |q||k| bound (key norms are
+//     reduced while K is staged) decides per query tile whether probabilities can be taken as
+//     2^score with no running maximum at all (C operand = constant zero); otherwise the running
+//     reference maximum enters through the MFMA's C operand so scores arrive already shifted, and
+//     the reference only moves when a score exceeds it by 2^8 -- which the same bound rules out
+//     for most 64-key steps without looking at the scores.
 //   * Rows are read through slot_src and written through slot_dst, so the padded,
 //     permuted qkv tensor of the reference is never materialised.
 // fp32 kernel: one thread per query, K/V chunks staged in LDS, plain FMA arithmetic.

@@ -372,3 +372,25 @@ def test_subm_conv_config3_full_size_fp16():
     twice = o.subm_conv_pairs((feat * 2).to(DEV), plan, w.to(DEV), None)
     once = o.subm_conv_pairs(feat.to(DEV), plan, w.to(DEV), None)
     assert rel_err(twice, 2 * once.float().cpu()) < 2e-3                  # (c)
+
+
+@pytest.mark.parametrize("ks", [3, 5])
+def test_voxel_hash_edge_coordinates(ks):
+    """Voxels at the corners of the coordinate range (0 and 65535), many scene ids, neighbours across
+    4x4x4 block borders in every direction, a lone voxel: map and direct pair lists against the oracle."""
+    rng = np.random.default_rng(ks)
+    parts = []
+    for b, base in ((0, 0), (1, 65535 - 7), (37, 4), (1023, 32760)):
+        g = rng.integers(0, 8, size=(150, 3)) + base
+        parts.append(np.concatenate([np.full((150, 1), b), g], 1))
+    parts.append(np.array([[5, 0, 0, 0], [5, 65535, 65535, 65535], [5, 3, 4, 3], [5, 4, 4, 4], [6, 100, 200, 300]]))
+    idx = np.unique(np.concatenate(parts).astype(np.int32), axis=0)
+    idx = idx[rng.permutation(len(idx))]
+    want = OI.subm_kmap(idx, ks)
+    o = ops()
+    assert np.array_equal(o.kmap_build(to_dev(idx), ks).cpu().numpy(), want)
+    plan = o.conv_plan_direct(to_dev(idx), ks)
+    t_idx, v_idx = np.nonzero(want.T >= 0)
+    assert plan.n_pairs == len(t_idx)
+    assert np.array_equal(plan.pair_in[:plan.n_pairs].cpu().numpy(), want.T[t_idx, v_idx])
+    assert np.array_equal(plan.row_ptr.cpu().numpy(), np.concatenate([[0], np.cumsum((want >= 0).sum(1))]))
