@@ -205,11 +205,19 @@ int ptv3_bn_act(const void *x, const void *running_mean, const void *running_var
                 const void *gamma, const void *beta, int dtype, int64_t n, int c, float eps, int act,
                 void *out, void *stream);
 
+/* nn.Linear of the wide blocks (model.py:541-545 cpe.1, :450 qkv, :487 proj, :510-512 fc1 + GELU):
+ * out = act(x w^T + bias), x (n, k), w (nout, k), bias (nout,) or NULL, out (n, nout), act = exact
+ * (erf) GELU when gelu != 0. fp16/bf16, k in {128, 256, 512}, nout a multiple of 32 (PTV3_ESHAPE
+ * otherwise: use a library GEMM). Tall-and-skinny form: rows held in MFMA operand registers, no loop
+ * over memory along k. */
+int ptv3_linear_fwd(const void *x, const void *w, const void *bias, int dtype, int64_t n, int k, int nout,
+                    int gelu, void *out, void *stream);
+
 /* MLP of a block plus its residual, model.py:510-516 and :602, in one kernel:
  * out = resid + fc2(GELU(fc1(x))), exact (erf) GELU, intermediates rounded to dtype where the
  * separate layers would have stored them. x, resid, out (n, channels); w1 (hidden, channels),
- * b1 (hidden,), w2 (channels, hidden), b2 (channels,). fp16/bf16, channels 32 or 64,
- * hidden = 4 * channels (PTV3_ESHAPE otherwise: use the separate layers). */
+ * b1 (hidden,), w2 (channels, hidden), b2 (channels,). fp16/bf16, channels 32, 64, 128, 256 or
+ * 512, hidden = 4 * channels (PTV3_ESHAPE otherwise: use the separate layers). */
 int ptv3_mlp_fused(const void *x, const void *resid, const void *w1, const void *b1, const void *w2,
                    const void *b2, int dtype, int64_t n, int channels, int hidden, void *out,
                    void *stream);

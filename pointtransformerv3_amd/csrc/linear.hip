@@ -1,0 +1,176 @@
+// Linear layer for many rows and few channels: out = act(x W^T + b), x (n, K) with K = 128, 256
+// or 512, W (N, K) as nn.Linear stores it, half precision.
+//
+// The Linear layers of the wide blocks (model.py:541-545 cpe.1, :450 qkv, :487 proj, :510-512
+// fc1 + GELU) are tall and skinny: 9k-150k rows against 128-512 input channels. A library GEMM
+// spends most of its time in the prologue and epilogue of its K loop there. Here the contraction
+// has no loop over memory at all: a wave owns 32 rows, converts them once to MFMA operand
+// registers (K / 16 fragments) and multiplies them with one 32-channel tile of W after the other,
+// W's chunk of output channels sitting in LDS for the life of the persistent work-group
+// (products are taken transposed, rows of the A operand = output channels, so a lane ends up with
+// 4 consecutive output channels of one row). x is read once per chunk of output channels, out is
+// written once; rows move between global memory and registers as contiguous 16-byte pieces
+// through a wave-private LDS buffer. The bias, and for fc1 the exact GELU, are applied on the
+// accumulators; results are rounded to the storage type once, as the separate layers round.
+#include "rowtile.h"
+
+namespace {
+
+constexpr int LIN_THREADS = 512;
+constexpr int LIN_WAVES = LIN_THREADS / PTV3_WAVE;
+constexpr int LIN_PAD = 8;                 // halfs of padding per LDS row
+constexpr int LIN_XSS = 64 + LIN_PAD;      // tile buffer row stride: 64 channels at a time
+// LDS budget for the weight chunk: at 128 inputs small enough for two work-groups per CU
+constexpr size_t lin_w_bytes(int k) { return k <= 128 ? 40 * 1024 : 105 * 1024; }
+
+template <typename T, int K, bool GELU>
+__global__ __launch_bounds__(LIN_THREADS, 2) void linear_rows_kernel(
+    const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ bias, int64_t n, int nout, int chunk,
+    T* __restrict__ out) {
+    typedef typename H16<T>::v8 v8;
+    constexpr int KS = K / 16, WS = K + LIN_PAD;
+    extern __shared__ __align__(16) unsigned char lin_smem[];
+    T* w_lds = (T*)lin_smem;                               // [chunk][WS]
+    float* b_lds = (float*)(w_lds + (size_t)chunk * WS);   // [chunk]
+    T* xs_all = (T*)(b_lds + chunk);                       // [waves][32][LIN_XSS]
+
+    const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
+    const int col = lane & 31, hf = lane >> 5;
+    T* xs = xs_all + wave * (32 * LIN_XSS);
+    const int c0 = blockIdx.y * chunk;                     // first output channel of this work-group
+    const int cn = min(chunk, nout - c0);                  // its output channels (a multiple of 32)
+
+    // ---- weight chunk and bias -> LDS (rows past cn are never read)
+    {
+        constexpr int PPR = K / 8;
+        for (int e = tid; e < cn * PPR; e += LIN_THREADS) {
+            const int r = e / PPR, pc = e % PPR;
+            *(u32x4*)(w_lds + r * WS + pc * 8) = *(const u32x4*)(w + (int64_t)(c0 + r) * K + pc * 8);
+        }
+        for (int e = tid; e < cn; e += LIN_THREADS) b_lds[e] = bias ? (float)bias[c0 + e] : 0.f;
+    }
+    __syncthreads();
+
+    const int64_t n_tiles = (n + 31) / 32;
+    for (int64_t tile = (int64_t)blockIdx.x * LIN_WAVES + wave; tile < n_tiles; tile += (int64_t)gridDim.x * LIN_WAVES) {
+        const int64_t row0 = tile * 32;
+        // ---- 32 rows -> operand fragments, 64 channels at a time: lane (r, piece) moves 16 bytes
+        v8 xf[KS];
+#pragma unroll
+        for (int part = 0; part < K / 64; ++part) {
+            u32x4 raw[4];
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const int pidx = it * PTV3_WAVE + lane;    // 32 rows x 8 pieces
+                const int64_t r = row0 + pidx / 8;
+                raw[it] = (u32x4){0, 0, 0, 0};
+                if (r < n) raw[it] = *(const u32x4*)(x + r * K + part * 64 + (pidx % 8) * 8);
+            }
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const int pidx = it * PTV3_WAVE + lane;
+                *(u32x4*)(xs + (pidx / 8) * LIN_XSS + (pidx % 8) * 8) = raw[it];
+            }
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+                xf[part * 4 + ks] = __builtin_bit_cast(v8, *(const u32x4*)(xs + col * LIN_XSS + ks * 16 + hf * 8));
+            asm volatile("" ::: "memory");
+        }
+        // ---- output channels two 32-tiles (64 channels) at a time
+        for (int o0 = 0; o0 < cn; o0 += 64) {
+            const int nt = (cn - o0) >= 64 ? 2 : 1;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                if (t >= nt) break;
+                f32x16 d;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) d[v] = 0.f;
+                const T* wrow = w_lds + (o0 + t * 32 + col) * WS + hf * 8;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    d = H16<T>::mfma(__builtin_bit_cast(v8, *(const u32x4*)(wrow + ks * 16)), xf[ks], d);
+                // d[v]: output channel o0 + 32 t + 8 (v / 4) + 4 hf + v % 4 of row `col`
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const f32x4 bb = *(const f32x4*)(b_lds + o0 + t * 32 + 8 * g + 4 * hf);
+                    float r[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        r[q] = d[4 * g + q] + bb[q];
+                        if (GELU) r[q] = gelu_erf(H16<T>::round(r[q]));
+                    }
+                    *(u32x2*)(xs + col * LIN_XSS + t * 32 + 8 * g + 4 * hf) =
+                        (u32x2){H16<T>::pack2(r[0], r[1]), H16<T>::pack2(r[2], r[3])};
+                }
+            }
+            asm volatile("" ::: "memory");
+            const int ppr_g = nt * 4;                        // 16-byte pieces per row of this group
+            const int its = 32 * ppr_g / PTV3_WAVE;          // 4 or 2
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                if (it >= its) break;
+                const int pidx = it * PTV3_WAVE + lane;
+                const int rr = pidx / ppr_g, pc = pidx % ppr_g;
+                const int64_t r = row0 + rr;
+                const u32x4 o4 = *(const u32x4*)(xs + rr * LIN_XSS + pc * 8);
+                if (r < n) *(u32x4*)(out + r * nout + c0 + o0 + pc * 8) = o4;
+            }
+            asm volatile("" ::: "memory");
+        }
+    }
+}
+
+template <typename T, int K, bool GELU>
+int launch_linear(const void* x, const void* w, const void* bias, int64_t n, int nout, void* out, hipStream_t stream) {
+    // output channels per work-group: as many 32-tiles as the LDS budget holds, spread evenly
+    const int cap = (int)(lin_w_bytes(K) / ((K + LIN_PAD) * sizeof(T))) / 32 * 32;
+    const int n_chunks = (nout + cap - 1) / cap;
+    const int chunk = ((nout + n_chunks - 1) / n_chunks + 31) / 32 * 32;
+    const size_t lds = (size_t)chunk * (K + LIN_PAD) * sizeof(T) + (size_t)chunk * sizeof(float) +
+                       (size_t)LIN_WAVES * 32 * LIN_XSS * sizeof(T);
+    auto kern = linear_rows_kernel<T, K, GELU>;
+    static size_t lds_allowed = 0;
+    if (lds > lds_allowed) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        lds_allowed = lds;
+    }
+    // persistent work-groups: as many as the LDS lets a CU hold, shared out between the chunks
+    const int64_t tiles = (n + 31) / 32;
+    int64_t per_chunk = (lds <= 80 * 1024 ? 512 : 256) / n_chunks;
+    if (per_chunk < 1) per_chunk = 1;
+    const int64_t need = (tiles + LIN_WAVES - 1) / LIN_WAVES;
+    if (per_chunk > need) per_chunk = need;
+    hipLaunchKernelGGL(kern, dim3((unsigned)per_chunk, (unsigned)n_chunks), dim3(LIN_THREADS), lds, stream, (const T*)x,
+                       (const T*)w, (const T*)bias, n, nout, chunk, (T*)out);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? PTV3_OK : (int)e;
+}
+
+}  // namespace
+
+extern "C" int ptv3_linear_fwd(const void* x, const void* w, const void* bias, int dtype, int64_t n, int k, int nout,
+                               int gelu, void* out, void* stream_) {
+    if (n < 0 || k < 1 || nout < 1) return PTV3_EINVAL;
+    if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
+    if ((k != 128 && k != 256 && k != 512) || nout % 32 != 0) return PTV3_ESHAPE;
+    if (n == 0) return PTV3_OK;
+    if (!x || !w || !out) return PTV3_EINVAL;
+    hipStream_t stream = (hipStream_t)stream_;
+#define PTV3_LIN(T, K)                                                                          \
+    if (k == K)                                                                                 \
+        return gelu ? launch_linear<T, K, true>(x, w, bias, n, nout, out, stream)               \
+                    : launch_linear<T, K, false>(x, w, bias, n, nout, out, stream)
+    if (dtype == PTV3_F16) {
+        PTV3_LIN(_Float16, 128);
+        PTV3_LIN(_Float16, 256);
+        PTV3_LIN(_Float16, 512);
+    } else {
+        PTV3_LIN(__bf16, 128);
+        PTV3_LIN(__bf16, 256);
+        PTV3_LIN(__bf16, 512);
+    }
+#undef PTV3_LIN
+    return PTV3_ESHAPE;
+}

@@ -249,8 +249,8 @@ class SerializedAttention(PointModule):
                                    self.patch_size, self.scale)
 
     def forward(self, point):
-        feat = self.attend(point, self.qkv(point.feat))
-        feat = self.proj(feat)
+        feat = self.attend(point, ops.linear(point.feat, self.qkv))
+        feat = ops.linear(feat, self.proj)
         feat = self.proj_drop(feat)
         point.feat = feat
         return point
@@ -327,7 +327,7 @@ class Block(PointModule):
             point.feat = feat
             point.sparse_conv_feat = point.sparse_conv_feat.replace_feature(feat)
             return point
-        branch = self.cpe[1](conv)
+        branch = ops.linear(conv, self.cpe[1]) if type(self.cpe[1]) is nn.Linear else self.cpe[1](conv)
         # feat = shortcut + LN(branch) and its pre-norm for attention, in one pass
         feat, normed = ops.layer_norm(branch, ln_cpe.weight, ln_cpe.bias, ln_cpe.eps, residual=point.feat,
                                       mode=3, weight2=ln1.weight, bias2=ln1.bias)
@@ -342,7 +342,8 @@ class Block(PointModule):
             # fc1 + GELU + fc2 + residual in one kernel, the 4C-wide hidden tensor never leaves the CU
             feat = ops.mlp_fused(normed, feat, mlp.fc1.weight, mlp.fc1.bias, mlp.fc2.weight, mlp.fc2.bias)
         elif plain_mlp:
-            feat = torch.addmm(feat, mlp.act(mlp.fc1(normed)), mlp.fc2.weight.t())
+            hidden = ops.linear(normed, mlp.fc1, gelu=True) if exact_gelu else mlp.act(mlp.fc1(normed))
+            feat = torch.addmm(feat, hidden, mlp.fc2.weight.t())
         else:
             feat = feat + mlp(normed)
         point.feat = feat

@@ -418,6 +418,48 @@ def layer_norm(x, weight, bias, eps=1e-5, residual=None, mode=0, weight2=None, b
     return out0 if mode < 2 else (out0, out1)
 
 
+LINEAR_ROWS_IN = (128, 256, 512)          # input widths of the tall-and-skinny Linear kernel
+
+
+def linear_rows_ok(x, weight):
+    """True when linear_rows covers this layer: half precision, 128 / 256 / 512 inputs, outputs in 32s."""
+    return (x.is_cuda and x.dtype in (torch.float16, torch.bfloat16) and x.dim() == 2
+            and weight.shape[1] in LINEAR_ROWS_IN and weight.shape[0] % 32 == 0)
+
+
+def linear_rows_pays(x, weight, gelu=False):
+    """Where the tall-and-skinny kernel measured faster than the library GEMM (+ GELU launch) on MI355X:
+    everything at 128 inputs, the wider outputs at 256, all but the 3x-wide qkv at 512."""
+    if not linear_rows_ok(x, weight):
+        return False
+    nout, k = weight.shape
+    if k == 128 or gelu:
+        return True
+    return nout >= 3 * k if k == 256 else nout <= k
+
+
+def linear(x, mod, gelu=False):
+    """mod(x) for an nn.Linear (followed by exact GELU if gelu), on whichever path is faster."""
+    if linear_rows_pays(x, mod.weight, gelu):
+        return linear_rows(x, mod.weight, mod.bias, gelu)
+    y = torch.nn.functional.linear(x, mod.weight, mod.bias)
+    return torch.nn.functional.gelu(y) if gelu else y
+
+
+def linear_rows(x, weight, bias=None, gelu=False):
+    """act(x W^T + b) for many rows and few channels (see ptv3_linear_fwd); act = exact GELU if gelu."""
+    _dev(x, weight, bias)
+    lib = _lib.load()
+    x = x.contiguous()
+    n, k = x.shape
+    w = weight.to(x.dtype).contiguous()
+    b = None if bias is None else bias.to(x.dtype).contiguous()
+    out = torch.empty((n, w.shape[0]), dtype=x.dtype, device=x.device)
+    _lib.check(lib.ptv3_linear_fwd(_ptr(x), _ptr(w), _ptr(b), _dtype_code(x), n, k, w.shape[0], int(bool(gelu)),
+                                   _ptr(out), _stream()), "ptv3_linear_fwd")
+    return out
+
+
 MLP_FUSED_CHANNELS = (32, 64)             # widths of the fused block head / tail kernels
 MLP_ONLY_FUSED_CHANNELS = (32, 64, 128, 256, 512)   # widths the fused MLP kernel supports
 MLP_ONLY_FUSED_PAYS = (32, 64, 128)                 # widths at which it beats fc1, GELU and fc2 as three launches

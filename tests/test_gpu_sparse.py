@@ -394,3 +394,21 @@ def test_voxel_hash_edge_coordinates(ks):
     assert plan.n_pairs == len(t_idx)
     assert np.array_equal(plan.pair_in[:plan.n_pairs].cpu().numpy(), want.T[t_idx, v_idx])
     assert np.array_equal(plan.row_ptr.cpu().numpy(), np.concatenate([[0], np.cumsum((want >= 0).sum(1))]))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("k,nout,n,gelu,bias", [(128, 128, 1, False, True), (128, 384, 40_001, False, True), (128, 512, 777, True, True),
+                                                (256, 768, 9000, False, True), (256, 1024, 5000, True, True), (256, 96, 33, False, False),
+                                                (512, 512, 2500, False, True), (512, 2048, 1000, True, True), (512, 1536, 64, False, True)])
+def test_linear_rows_parity(dtype, k, nout, n, gelu, bias):
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(k + nout + n)
+    x = torch.randn(n, k, generator=g).to(dtype)
+    w = (torch.randn(nout, k, generator=g) / k ** 0.5).to(dtype)
+    b = (torch.randn(nout, generator=g) * 0.5).to(dtype) if bias else None
+    want = F.linear(x.float(), w.float(), None if b is None else b.float())
+    if gelu:
+        want = F.gelu(want)
+    got = ops().linear_rows(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), gelu)
+    assert got.dtype == dtype and got.shape == (n, nout)
+    assert rel_err(got, want) < TOL[dtype]
