@@ -207,7 +207,7 @@ int ptv3_bn_act(const void *x, const void *running_mean, const void *running_var
 
 /* nn.Linear of the wide blocks (model.py:541-545 cpe.1, :450 qkv, :487 proj, :510-512 fc1 + GELU):
  * out = act(x w^T + bias), x (n, k), w (nout, k), bias (nout,) or NULL, out (n, nout), act = exact
- * (erf) GELU when gelu != 0. fp16/bf16, k in {128, 256, 512}, nout a multiple of 32 (PTV3_ESHAPE
+ * (erf) GELU when gelu != 0. fp16/bf16, k in {32, 64, 128, 256, 512}, nout a multiple of 32 (PTV3_ESHAPE
  * otherwise: use a library GEMM). Tall-and-skinny form: rows held in MFMA operand registers, no loop
  * over memory along k. */
 int ptv3_linear_fwd(const void *x, const void *w, const void *bias, int dtype, int64_t n, int k, int nout,

@@ -1,5 +1,5 @@
-// Linear layer for many rows and few channels: out = act(x W^T + b), x (n, K) with K = 128, 256
-// or 512, W (N, K) as nn.Linear stores it, half precision.
+// Linear layer for many rows and few channels: out = act(x W^T + b), x (n, K) with K = 32, 64, 128,
+// 256 or 512, W (N, K) as nn.Linear stores it, half precision.
 //
 // The Linear layers of the wide blocks (model.py:541-545 cpe.1, :450 qkv, :487 proj, :510-512
 // fc1 + GELU) are tall and skinny: 9k-150k rows against 128-512 input channels. A library GEMM
@@ -56,25 +56,28 @@ __global__ __launch_bounds__(LIN_THREADS, 2) void linear_rows_kernel(
         const int64_t row0 = tile * 32;
         // ---- 32 rows -> operand fragments, 64 channels at a time: lane (r, piece) moves 16 bytes
         v8 xf[KS];
+        constexpr int PART = K < 64 ? K : 64;             // channels staged at a time
+        constexpr int PPP = PART / 8;                     // 16-byte pieces per row and part
+        constexpr int ITS = 32 * PPP / PTV3_WAVE;         // pieces per lane and part
 #pragma unroll
-        for (int part = 0; part < K / 64; ++part) {
-            u32x4 raw[4];
+        for (int part = 0; part < K / PART; ++part) {
+            u32x4 raw[ITS];
 #pragma unroll
-            for (int it = 0; it < 4; ++it) {
-                const int pidx = it * PTV3_WAVE + lane;    // 32 rows x 8 pieces
-                const int64_t r = row0 + pidx / 8;
+            for (int it = 0; it < ITS; ++it) {
+                const int pidx = it * PTV3_WAVE + lane;    // 32 rows x PPP pieces
+                const int64_t r = row0 + pidx / PPP;
                 raw[it] = (u32x4){0, 0, 0, 0};
-                if (r < n) raw[it] = *(const u32x4*)(x + r * K + part * 64 + (pidx % 8) * 8);
+                if (r < n) raw[it] = *(const u32x4*)(x + r * K + part * PART + (pidx % PPP) * 8);
             }
 #pragma unroll
-            for (int it = 0; it < 4; ++it) {
+            for (int it = 0; it < ITS; ++it) {
                 const int pidx = it * PTV3_WAVE + lane;
-                *(u32x4*)(xs + (pidx / 8) * LIN_XSS + (pidx % 8) * 8) = raw[it];
+                *(u32x4*)(xs + (pidx / PPP) * LIN_XSS + (pidx % PPP) * 8) = raw[it];
             }
             asm volatile("" ::: "memory");
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
-                xf[part * 4 + ks] = __builtin_bit_cast(v8, *(const u32x4*)(xs + col * LIN_XSS + ks * 16 + hf * 8));
+            for (int ks = 0; ks < PART / 16; ++ks)
+                xf[part * (PART / 16) + ks] = __builtin_bit_cast(v8, *(const u32x4*)(xs + col * LIN_XSS + ks * 16 + hf * 8));
             asm volatile("" ::: "memory");
         }
         // ---- output channels two 32-tiles (64 channels) at a time
@@ -154,7 +157,7 @@ extern "C" int ptv3_linear_fwd(const void* x, const void* w, const void* bias, i
                                int gelu, void* out, void* stream_) {
     if (n < 0 || k < 1 || nout < 1) return PTV3_EINVAL;
     if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
-    if ((k != 128 && k != 256 && k != 512) || nout % 32 != 0) return PTV3_ESHAPE;
+    if ((k != 32 && k != 64 && k != 128 && k != 256 && k != 512) || nout % 32 != 0) return PTV3_ESHAPE;
     if (n == 0) return PTV3_OK;
     if (!x || !w || !out) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
@@ -163,10 +166,14 @@ extern "C" int ptv3_linear_fwd(const void* x, const void* w, const void* bias, i
         return gelu ? launch_linear<T, K, true>(x, w, bias, n, nout, out, stream)               \
                     : launch_linear<T, K, false>(x, w, bias, n, nout, out, stream)
     if (dtype == PTV3_F16) {
+        PTV3_LIN(_Float16, 32);
+        PTV3_LIN(_Float16, 64);
         PTV3_LIN(_Float16, 128);
         PTV3_LIN(_Float16, 256);
         PTV3_LIN(_Float16, 512);
     } else {
+        PTV3_LIN(__bf16, 32);
+        PTV3_LIN(__bf16, 64);
         PTV3_LIN(__bf16, 128);
         PTV3_LIN(__bf16, 256);
         PTV3_LIN(__bf16, 512);

@@ -113,7 +113,7 @@ class PointSequential(PointModule):
                 else:
                     input = module(input)
             elif isinstance(input, Point):
-                input.feat = module(input.feat)
+                input.feat = ops.linear(input.feat, module) if type(module) is nn.Linear else module(input.feat)
                 if "sparse_conv_feat" in input:
                     input.sparse_conv_feat = input.sparse_conv_feat.replace_feature(input.feat)
             elif isinstance(input, SparseConvTensor):
@@ -419,7 +419,7 @@ class SerializedPooling(PointModule):
             code, order, inverse = ops.permute_rows(perm, code, order, inverse)
 
         fields = AttrDict(
-            feat=ops.segment_reduce(self.proj(point.feat), indices, idx_ptr, self.reduce),
+            feat=ops.segment_reduce(ops.linear(point.feat, self.proj), indices, idx_ptr, self.reduce),
             grid_coord=grid_coord,
             serialized_code=code,
             serialized_order=order,

@@ -418,24 +418,22 @@ def layer_norm(x, weight, bias, eps=1e-5, residual=None, mode=0, weight2=None, b
     return out0 if mode < 2 else (out0, out1)
 
 
-LINEAR_ROWS_IN = (128, 256, 512)          # input widths of the tall-and-skinny Linear kernel
+LINEAR_ROWS_IN = (32, 64, 128, 256, 512)   # input widths of the tall-and-skinny Linear kernel
 
 
 def linear_rows_ok(x, weight):
-    """True when linear_rows covers this layer: half precision, 128 / 256 / 512 inputs, outputs in 32s."""
+    """True when linear_rows covers this layer: half precision, 32 ... 512 inputs, outputs in 32s."""
     return (x.is_cuda and x.dtype in (torch.float16, torch.bfloat16) and x.dim() == 2
             and weight.shape[1] in LINEAR_ROWS_IN and weight.shape[0] % 32 == 0)
 
 
 def linear_rows_pays(x, weight, gelu=False):
-    """Where the tall-and-skinny kernel measured faster than the library GEMM (+ GELU launch) on MI355X:
-    everything at 128 inputs, the wider outputs at 256, all but the 3x-wide qkv at 512."""
+    """Where the tall-and-skinny kernel measured at least as fast as the library GEMM (+ GELU launch) on
+    MI355X: everything up to 256 inputs (3-4x at 32 and 64), all but the 3x-wide qkv at 512."""
     if not linear_rows_ok(x, weight):
         return False
     nout, k = weight.shape
-    if k == 128 or gelu:
-        return True
-    return nout >= 3 * k if k == 256 else nout <= k
+    return k <= 256 or gelu or nout <= 2 * k
 
 
 def linear(x, mod, gelu=False):

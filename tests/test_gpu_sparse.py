@@ -397,7 +397,8 @@ def test_voxel_hash_edge_coordinates(ks):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("k,nout,n,gelu,bias", [(128, 128, 1, False, True), (128, 384, 40_001, False, True), (128, 512, 777, True, True),
+@pytest.mark.parametrize("k,nout,n,gelu,bias", [(32, 64, 50_001, False, True), (64, 64, 31, False, True), (64, 128, 4000, True, False),
+                                                (128, 128, 1, False, True), (128, 384, 40_001, False, True), (128, 512, 777, True, True),
                                                 (256, 768, 9000, False, True), (256, 1024, 5000, True, True), (256, 96, 33, False, False),
                                                 (512, 512, 2500, False, True), (512, 2048, 1000, True, True), (512, 1536, 64, False, True)])
 def test_linear_rows_parity(dtype, k, nout, n, gelu, bias):
