@@ -212,6 +212,12 @@ int ptv3_bn_act(const void *x, const void *running_mean, const void *running_var
  * over memory along k. */
 int ptv3_linear_fwd(const void *x, const void *w, const void *bias, int dtype, int64_t n, int k, int nout,
                     int gelu, void *out, void *stream);
+/* The same followed by an inference-mode nn.BatchNorm1d and optionally the GELU, the projections of
+ * model.py:726-735 (Linear -> BatchNorm1d -> GELU) in one kernel; statistics and affine parameters as
+ * for ptv3_bn_act. The Linear's result is rounded to dtype before the normalisation, as when stored. */
+int ptv3_linear_bn_act_fwd(const void *x, const void *w, const void *bias, const void *running_mean,
+                           const void *running_var, int stats_f32, const void *gamma, const void *beta,
+                           float eps, int dtype, int64_t n, int k, int nout, int gelu, void *out, void *stream);
 
 /* MLP of a block plus its residual, model.py:510-516 and :602, in one kernel:
  * out = resid + fc2(GELU(fc1(x))), exact (erf) GELU, intermediates rounded to dtype where the

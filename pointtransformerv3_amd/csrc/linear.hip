@@ -23,16 +23,29 @@ constexpr int LIN_XSS = 64 + LIN_PAD;      // tile buffer row stride: 64 channel
 // LDS budget for the weight chunk: at 128 inputs small enough for two work-groups per CU
 constexpr size_t lin_w_bytes(int k) { return k <= 128 ? 40 * 1024 : 105 * 1024; }
 
-template <typename T, int K, bool GELU>
+// inference BatchNorm folded into the epilogue (model.py:726-735: Linear -> BatchNorm1d -> GELU)
+struct LinBn {
+    const void* mean;    // running statistics: float32 when stats_f32, else of the data type
+    const void* var;
+    const void* gamma;   // of the data type, or null
+    const void* beta;
+    float eps;
+    int stats_f32;
+};
+
+template <typename T, int K, bool GELU, bool BN>
 __global__ __launch_bounds__(LIN_THREADS, 2) void linear_rows_kernel(
-    const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ bias, int64_t n, int nout, int chunk,
-    T* __restrict__ out) {
+    const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ bias, LinBn bn, int64_t n, int nout,
+    int chunk, T* __restrict__ out) {
     typedef typename H16<T>::v8 v8;
     constexpr int KS = K / 16, WS = K + LIN_PAD;
     extern __shared__ __align__(16) unsigned char lin_smem[];
     T* w_lds = (T*)lin_smem;                               // [chunk][WS]
     float* b_lds = (float*)(w_lds + (size_t)chunk * WS);   // [chunk]
-    T* xs_all = (T*)(b_lds + chunk);                       // [waves][32][LIN_XSS]
+    float* mu_lds = b_lds + chunk;                         // [chunk] x 3 with BN: mean, rstd * gamma, beta
+    float* sc_lds = mu_lds + (BN ? chunk : 0);
+    float* be_lds = sc_lds + (BN ? chunk : 0);
+    T* xs_all = (T*)(be_lds + (BN ? chunk : 0));           // [waves][32][LIN_XSS]
 
     const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
     const int col = lane & 31, hf = lane >> 5;
@@ -47,7 +60,17 @@ __global__ __launch_bounds__(LIN_THREADS, 2) void linear_rows_kernel(
             const int r = e / PPR, pc = e % PPR;
             *(u32x4*)(w_lds + r * WS + pc * 8) = *(const u32x4*)(w + (int64_t)(c0 + r) * K + pc * 8);
         }
-        for (int e = tid; e < cn; e += LIN_THREADS) b_lds[e] = bias ? (float)bias[c0 + e] : 0.f;
+        for (int e = tid; e < cn; e += LIN_THREADS) {
+            b_lds[e] = bias ? (float)bias[c0 + e] : 0.f;
+            if (BN) {
+                const int c = c0 + e;
+                const float mu = bn.stats_f32 ? ((const float*)bn.mean)[c] : (float)((const T*)bn.mean)[c];
+                const float va = bn.stats_f32 ? ((const float*)bn.var)[c] : (float)((const T*)bn.var)[c];
+                mu_lds[e] = mu;
+                sc_lds[e] = rsqrtf(va + bn.eps) * (bn.gamma ? (float)((const T*)bn.gamma)[c] : 1.f);
+                be_lds[e] = bn.beta ? (float)((const T*)bn.beta)[c] : 0.f;
+            }
+        }
     }
     __syncthreads();
 
@@ -101,6 +124,10 @@ __global__ __launch_bounds__(LIN_THREADS, 2) void linear_rows_kernel(
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         r[q] = d[4 * g + q] + bb[q];
+                        if (BN) {
+                            const int c = o0 + t * 32 + 8 * g + 4 * hf + q;
+                            r[q] = (H16<T>::round(r[q]) - mu_lds[c]) * sc_lds[c] + be_lds[c];
+                        }
                         if (GELU) r[q] = gelu_erf(H16<T>::round(r[q]));
                     }
                     *(u32x2*)(xs + col * LIN_XSS + t * 32 + 8 * g + 4 * hf) =
@@ -124,15 +151,16 @@ __global__ __launch_bounds__(LIN_THREADS, 2) void linear_rows_kernel(
     }
 }
 
-template <typename T, int K, bool GELU>
-int launch_linear(const void* x, const void* w, const void* bias, int64_t n, int nout, void* out, hipStream_t stream) {
+template <typename T, int K, bool GELU, bool BN>
+int launch_linear(const void* x, const void* w, const void* bias, LinBn bn, int64_t n, int nout, void* out,
+                  hipStream_t stream) {
     // output channels per work-group: as many 32-tiles as the LDS budget holds, spread evenly
     const int cap = (int)(lin_w_bytes(K) / ((K + LIN_PAD) * sizeof(T))) / 32 * 32;
     const int n_chunks = (nout + cap - 1) / cap;
     const int chunk = ((nout + n_chunks - 1) / n_chunks + 31) / 32 * 32;
-    const size_t lds = (size_t)chunk * (K + LIN_PAD) * sizeof(T) + (size_t)chunk * sizeof(float) +
+    const size_t lds = (size_t)chunk * (K + LIN_PAD) * sizeof(T) + (size_t)chunk * sizeof(float) * (BN ? 4 : 1) +
                        (size_t)LIN_WAVES * 32 * LIN_XSS * sizeof(T);
-    auto kern = linear_rows_kernel<T, K, GELU>;
+    auto kern = linear_rows_kernel<T, K, GELU, BN>;
     static size_t lds_allowed = 0;
     if (lds > lds_allowed) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -146,38 +174,56 @@ int launch_linear(const void* x, const void* w, const void* bias, int64_t n, int
     const int64_t need = (tiles + LIN_WAVES - 1) / LIN_WAVES;
     if (per_chunk > need) per_chunk = need;
     hipLaunchKernelGGL(kern, dim3((unsigned)per_chunk, (unsigned)n_chunks), dim3(LIN_THREADS), lds, stream, (const T*)x,
-                       (const T*)w, (const T*)bias, n, nout, chunk, (T*)out);
+                       (const T*)w, (const T*)bias, bn, n, nout, chunk, (T*)out);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? PTV3_OK : (int)e;
+}
+
+int dispatch_linear(const void* x, const void* w, const void* bias, const LinBn* bn, int dtype, int64_t n, int k,
+                    int nout, int gelu, void* out, hipStream_t stream) {
+    const LinBn none = {nullptr, nullptr, nullptr, nullptr, 0.f, 0};
+#define PTV3_LIN(T, K)                                                                                       \
+    if (k == K) {                                                                                            \
+        if (bn) return gelu ? launch_linear<T, K, true, true>(x, w, bias, *bn, n, nout, out, stream)         \
+                            : launch_linear<T, K, false, true>(x, w, bias, *bn, n, nout, out, stream);       \
+        return gelu ? launch_linear<T, K, true, false>(x, w, bias, none, n, nout, out, stream)               \
+                    : launch_linear<T, K, false, false>(x, w, bias, none, n, nout, out, stream);             \
+    }
+    if (dtype == PTV3_F16) {
+        PTV3_LIN(_Float16, 32) PTV3_LIN(_Float16, 64) PTV3_LIN(_Float16, 128) PTV3_LIN(_Float16, 256) PTV3_LIN(_Float16, 512)
+    } else {
+        PTV3_LIN(__bf16, 32) PTV3_LIN(__bf16, 64) PTV3_LIN(__bf16, 128) PTV3_LIN(__bf16, 256) PTV3_LIN(__bf16, 512)
+    }
+#undef PTV3_LIN
+    return PTV3_ESHAPE;
+}
+
+int check_linear(int dtype, int64_t n, int k, int nout) {
+    if (n < 0 || k < 1 || nout < 1) return PTV3_EINVAL;
+    if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
+    if ((k != 32 && k != 64 && k != 128 && k != 256 && k != 512) || nout % 32 != 0) return PTV3_ESHAPE;
+    return PTV3_OK;
 }
 
 }  // namespace
 
 extern "C" int ptv3_linear_fwd(const void* x, const void* w, const void* bias, int dtype, int64_t n, int k, int nout,
                                int gelu, void* out, void* stream_) {
-    if (n < 0 || k < 1 || nout < 1) return PTV3_EINVAL;
-    if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
-    if ((k != 32 && k != 64 && k != 128 && k != 256 && k != 512) || nout % 32 != 0) return PTV3_ESHAPE;
+    const int rc = check_linear(dtype, n, k, nout);
+    if (rc != PTV3_OK) return rc;
     if (n == 0) return PTV3_OK;
     if (!x || !w || !out) return PTV3_EINVAL;
-    hipStream_t stream = (hipStream_t)stream_;
-#define PTV3_LIN(T, K)                                                                          \
-    if (k == K)                                                                                 \
-        return gelu ? launch_linear<T, K, true>(x, w, bias, n, nout, out, stream)               \
-                    : launch_linear<T, K, false>(x, w, bias, n, nout, out, stream)
-    if (dtype == PTV3_F16) {
-        PTV3_LIN(_Float16, 32);
-        PTV3_LIN(_Float16, 64);
-        PTV3_LIN(_Float16, 128);
-        PTV3_LIN(_Float16, 256);
-        PTV3_LIN(_Float16, 512);
-    } else {
-        PTV3_LIN(__bf16, 32);
-        PTV3_LIN(__bf16, 64);
-        PTV3_LIN(__bf16, 128);
-        PTV3_LIN(__bf16, 256);
-        PTV3_LIN(__bf16, 512);
-    }
-#undef PTV3_LIN
-    return PTV3_ESHAPE;
+    return dispatch_linear(x, w, bias, nullptr, dtype, n, k, nout, gelu, out, (hipStream_t)stream_);
+}
+
+extern "C" int ptv3_linear_bn_act_fwd(const void* x, const void* w, const void* bias, const void* running_mean,
+                                      const void* running_var, int stats_f32, const void* gamma, const void* beta,
+                                      float eps, int dtype, int64_t n, int k, int nout, int gelu, void* out,
+                                      void* stream_) {
+    const int rc = check_linear(dtype, n, k, nout);
+    if (rc != PTV3_OK) return rc;
+    if (n == 0) return PTV3_OK;
+    if (!x || !w || !running_mean || !running_var || !out) return PTV3_EINVAL;
+    const LinBn bn = {running_mean, running_var, gamma, beta, eps, stats_f32};
+    return dispatch_linear(x, w, bias, &bn, dtype, n, k, nout, gelu, out, (hipStream_t)stream_);
 }

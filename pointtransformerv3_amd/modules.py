@@ -90,19 +90,28 @@ class PointSequential(PointModule):
 
     def forward(self, input):
         modules = list(self._modules.values())
-        skip = False
+        skip = 0
         for i, module in enumerate(modules):
-            if skip:   # activation already applied together with the normalisation before it
-                skip = False
+            if skip:   # already applied together with the module(s) before it
+                skip -= 1
                 continue
             nxt = modules[i + 1] if i + 1 < len(modules) else None
+            if (isinstance(input, Point) and type(module) is nn.Linear and ops.linear_rows_pays(input.feat, module.weight)
+                    and _fusable_bn(nxt, input.feat)):
+                # Linear -> BatchNorm1d (-> GELU), the projections of the unpooling stages, in one kernel
+                with_act = _exact_gelu(modules[i + 2] if i + 2 < len(modules) else None)
+                input.feat = ops.linear_bn_act(input.feat, module, nxt, with_act)
+                if "sparse_conv_feat" in input:
+                    input.sparse_conv_feat = input.sparse_conv_feat.replace_feature(input.feat)
+                skip = 2 if with_act else 1
+                continue
             if isinstance(input, Point) and _fusable_bn(module, input.feat):
                 with_act = _exact_gelu(nxt)
                 input.feat = ops.bn_act(input.feat, module.running_mean, module.running_var, module.weight,
                                         module.bias, module.eps, with_act)
                 if "sparse_conv_feat" in input:
                     input.sparse_conv_feat = input.sparse_conv_feat.replace_feature(input.feat)
-                skip = with_act
+                skip = int(with_act)
                 continue
             if isinstance(module, PointModule):
                 input = module(input)

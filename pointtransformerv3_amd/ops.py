@@ -458,6 +458,28 @@ def linear_rows(x, weight, bias=None, gelu=False):
     return out
 
 
+def linear_bn_act(x, lin, bn, gelu):
+    """gelu?(BatchNorm1d_inference(lin(x))) in one kernel for the layers linear_rows covers."""
+    _dev(x, lin.weight, bn.running_mean)
+    lib = _lib.load()
+    x = x.contiguous()
+    n, k = x.shape
+    dt = x.dtype
+    w = lin.weight.to(dt).contiguous()
+    b = None if lin.bias is None else lin.bias.to(dt).contiguous()
+    mean, var = bn.running_mean, bn.running_var
+    stats_f32 = mean.dtype == torch.float32
+    if not stats_f32 and mean.dtype != dt:
+        mean, var, stats_f32 = mean.float(), var.float(), True
+    g = None if bn.weight is None else bn.weight.to(dt).contiguous()
+    be = None if bn.bias is None else bn.bias.to(dt).contiguous()
+    out = torch.empty((n, w.shape[0]), dtype=dt, device=x.device)
+    _lib.check(lib.ptv3_linear_bn_act_fwd(_ptr(x), _ptr(w), _ptr(b), _ptr(mean.contiguous()), _ptr(var.contiguous()),
+                                          int(stats_f32), _ptr(g), _ptr(be), float(bn.eps), _dtype_code(x), n, k,
+                                          w.shape[0], int(bool(gelu)), _ptr(out), _stream()), "ptv3_linear_bn_act_fwd")
+    return out
+
+
 MLP_FUSED_CHANNELS = (32, 64)             # widths of the fused block head / tail kernels
 MLP_ONLY_FUSED_CHANNELS = (32, 64, 128, 256, 512)   # widths the fused MLP kernel supports
 MLP_ONLY_FUSED_PAYS = (32, 64, 128)                 # widths at which it beats fc1, GELU and fc2 as three launches

@@ -413,3 +413,36 @@ def test_linear_rows_parity(dtype, k, nout, n, gelu, bias):
     got = ops().linear_rows(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), gelu)
     assert got.dtype == dtype and got.shape == (n, nout)
     assert rel_err(got, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("k,nout,n,gelu,stats_f32,affine", [(512, 256, 3001, True, True, True), (256, 256, 777, True, False, True),
+                                                            (64, 64, 40_001, True, True, True), (128, 64, 5, False, True, False),
+                                                            (32, 128, 1000, True, True, True), (256, 128, 2048, False, False, True)])
+def test_linear_bn_act_parity(dtype, k, nout, n, gelu, stats_f32, affine):
+    """Linear -> BatchNorm1d (inference) -> GELU in one kernel (model.py:726-735) against torch in fp32."""
+    import torch.nn.functional as F
+    torch.manual_seed(k * 7 + nout + n)
+    lin = torch.nn.Linear(k, nout)
+    bn = torch.nn.BatchNorm1d(nout, affine=affine).eval()
+    bn.running_mean.normal_(0, 0.3)
+    bn.running_var.uniform_(0.5, 2.0)
+    if affine:
+        bn.weight.data.uniform_(0.5, 1.5)
+        bn.bias.data.normal_(0, 0.3)
+    x = torch.randn(n, k).to(dtype)
+    lin_h = lin.to(dtype)
+    with torch.no_grad():
+        want = bn(F.linear(x.float(), lin_h.weight.float(), lin_h.bias.float()))
+        if gelu:
+            want = F.gelu(want)
+    lin_d, bn_d = lin_h.to(DEV), bn.to(DEV)
+    if not stats_f32:
+        bn_d = bn_d.to(dtype)
+    got = ops().linear_bn_act(x.to(DEV), lin_d, bn_d, gelu)
+    assert got.dtype == dtype and got.shape == (n, nout)
+    assert rel_err(got, want) < TOL[dtype]
+    # the same as the two-kernel path it replaces, up to one rounding of the intermediate
+    two = ops().bn_act(ops().linear_rows(x.to(DEV), lin_d.weight, lin_d.bias), bn_d.running_mean, bn_d.running_var,
+                       bn_d.weight, bn_d.bias, bn_d.eps, gelu)
+    assert rel_err(got, two.float().cpu()) < (2e-3 if dtype == torch.float16 else 1.6e-2)
