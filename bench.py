@@ -225,6 +225,26 @@ def kernel_rooflines(path):
     us = _time_us(lambda: ops.subm_conv(feat, nbr, w, bias, tap_major=True))
     add("subm_conv dense<f16>", f"{nv} voxels, all 27 taps visited, 64->64", "mfma", 2.0 * plan.n_pairs * 64 * 64, us,
         "FLOP (2 * P_act * Cin * Cout)")
+    packed = ops.conv_pack_weight(w, 27, torch.float16)
+    plan.tiles()
+    us = _time_us(lambda: ops.subm_conv_tiles(feat, plan, packed, bias))
+    add("subm_conv tiles<f16>", f"{nv} voxels, {plan.n_pairs} pairs ({plan.n_pairs / nv:.2f}/voxel), 64->64", "mfma",
+        2.0 * plan.n_pairs * 64 * 64, us, "FLOP (2 * P_act * Cin * Cout)")
+    # the level the forward runs the tile form on: the 4-scene batch pooled twice (8 cm voxels), 128 channels
+    lvl = torch.unique(torch.cat([b[:, None].int(), (g >> 2).int()], 1), dim=0).contiguous()
+    nl = len(lvl)
+    plan2 = ops.conv_plan_direct(lvl, 3)
+    plan2.tiles()
+    feat2 = torch.randn(nl, 128, generator=gen).half().to(dev)
+    w2 = ((torch.rand(128, 27, 128, generator=gen) * 2 - 1) / np.sqrt(27 * 128)).half().to(dev)
+    bias2 = torch.zeros(128).half().to(dev)
+    packed2 = ops.conv_pack_weight(w2, 27, torch.float16)
+    for name, fn in (("subm_conv pairs<f16>", lambda: ops.subm_conv_pairs(feat2, plan2, w2, bias2)),
+                     ("subm_conv tiles<f16>", lambda: ops.subm_conv_tiles(feat2, plan2, packed2, bias2))):
+        us = _time_us(fn)
+        add(name, f"{nl} voxels (4 scenes at 8 cm), {plan2.n_pairs} pairs ({plan2.n_pairs / nl:.2f}/voxel), 128->128", "mfma",
+            2.0 * plan2.n_pairs * 128 * 128, us, "FLOP (2 * P_act * Cin * Cout)")
+    del plan2, feat2, w2, packed2, lvl
     # ---- pooling on the 4-scene batch
     code = ops.encode_orders(g, b, 9, orders)
     order, inverse = ops.argsort_rows(code, 29)

@@ -148,6 +148,29 @@ int ptv3_subm_conv_pairs_fwd(const void *feat, int dtype, int64_t n, int cin, in
                              const int32_t *pair_in, const int32_t *pair_slot, const void *weight,
                              const void *bias, int cout, void *y, void *out, void *stream);
 
+/* Tile form of the 3x3x3 convolution with cin == cout == channels in {32, 64, 128, 256} (the xCPE of
+ * every block, model.py:546-552), fp16/bf16: a work-group keeps the fp32 sums of a tile of 128
+ * consecutive output voxels on chip and walks their pairs tap by tap, so no product row per pair
+ * goes through memory; sums in tap order, nothing atomic, same result on every run.
+ * Lists, made once per plan (n < 2^24, taps == 27):
+ *   ptv3_conv_plan_slots: the tap-major lists of a plan -> output-major words slot_pair (n_pairs,)
+ *     int32, slot_pair[pair_slot[q]] = tap(q) << 24 | pair_in[q];
+ *   ptv3_conv_plan_tiles: per tile its pairs sorted by tap. tile_tap (ptv3_conv_plan_tile_count(n),
+ *     32) int32: [t] = first pair of tap t relative to the tile's first pair, [27] = pairs of the
+ *     tile, [28] = the tile's first pair; tile_pair (n_pairs,) int32 = voxel inside the tile << 24 |
+ *     input row (the order inside a tap is unspecified; no result depends on it).
+ * ptv3_subm_conv_pack_weight stores the (channels, taps, channels) weight in MFMA fragment order
+ * (same size); do it once per weight. */
+int ptv3_conv_plan_slots(const int32_t *tap_ptr, int taps, const int32_t *pair_in, const int32_t *pair_slot,
+                         int64_t n_pairs, int32_t *slot_pair, void *stream);
+int64_t ptv3_conv_plan_tile_count(int64_t n);
+int ptv3_conv_plan_tiles(const int32_t *row_ptr, const int32_t *slot_pair, int64_t n, int taps,
+                         int32_t *tile_tap, int32_t *tile_pair, int32_t *vox_taps, void *stream);
+int ptv3_subm_conv_pack_weight(const void *weight, int dtype, int channels, int taps, void *packed, void *stream);
+int ptv3_subm_conv_tiles_fwd(const void *feat, int dtype, int64_t n, int channels, int taps,
+                             const void *packed_weight, const void *bias, const int32_t *tile_tap,
+                             const int32_t *tile_pair, const int32_t *vox_taps, void *out, void *stream);
+
 /* model.py:652-664,690-695: clusters of code0 >> shift walked in sorted order (order0 sorts
  * code0, so no further sort is needed). Outputs: cluster (n,) int64 [pooling_inverse],
  * indices (n,) int64 (= order0: points grouped by cluster), idx_ptr (n+1 allocated, m+1 used),

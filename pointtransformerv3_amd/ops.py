@@ -215,10 +215,34 @@ def subm_conv(feat, nbr, weight, bias=None, tap_major=False):
 class ConvPlan:
     """Active (input, output) pairs of a neighbour map, tap-major, plus each voxel's slots."""
 
-    __slots__ = ("n", "taps", "n_pairs", "tap_ptr", "row_ptr", "pair_in", "pair_slot")
+    __slots__ = ("n", "taps", "n_pairs", "tap_ptr", "row_ptr", "pair_in", "pair_slot", "_slot_pair", "_tiles")
 
     def density(self):
         return self.n_pairs / max(1, self.n * self.taps)
+
+    def slot_pair(self):
+        """Output-major pair words (tap << 24 | input row) for subm_conv_tiles, made on first use."""
+        if getattr(self, "_slot_pair", None) is None:
+            lib = _lib.load()
+            sp = torch.empty(max(self.n_pairs, 1), dtype=torch.int32, device=self.pair_in.device)
+            _lib.check(lib.ptv3_conv_plan_slots(_ptr(self.tap_ptr), self.taps, _ptr(self.pair_in), _ptr(self.pair_slot),
+                                                self.n_pairs, _ptr(sp), _stream()), "ptv3_conv_plan_slots")
+            self._slot_pair = sp
+        return self._slot_pair
+
+    def tiles(self):
+        """(tile_tap, tile_pair): every tile's pairs sorted by tap for subm_conv_tiles, made on first use."""
+        if getattr(self, "_tiles", None) is None:
+            lib = _lib.load()
+            dev = self.pair_in.device
+            tile_tap = torch.empty((lib.ptv3_conv_plan_tile_count(self.n), 32), dtype=torch.int32, device=dev)
+            tile_pair = torch.empty(max(self.n_pairs, 1), dtype=torch.int32, device=dev)
+            vox_taps = torch.empty(max(self.n, 1), dtype=torch.int32, device=dev)
+            _lib.check(lib.ptv3_conv_plan_tiles(_ptr(self.row_ptr), _ptr(self.slot_pair()), self.n, self.taps,
+                                                _ptr(tile_tap), _ptr(tile_pair), _ptr(vox_taps), _stream()),
+                       "ptv3_conv_plan_tiles")
+            self._tiles = (tile_tap, tile_pair, vox_taps)
+        return self._tiles
 
 
 def conv_plan(nbr, tap_major=False):
@@ -289,6 +313,37 @@ def subm_conv_pairs(feat, plan, weight, bias=None):
                                             _ptr(plan.tap_ptr), _ptr(plan.row_ptr), _ptr(plan.pair_in),
                                             _ptr(plan.pair_slot), _ptr(w), _ptr(b), cout, _ptr(y), _ptr(out),
                                             _stream()), "ptv3_subm_conv_pairs_fwd")
+    return out
+
+
+CONV_TILE_CHANNELS = (64, 128)   # cin == cout widths of the tile form of the 3x3x3 convolution
+
+
+def conv_pack_weight(weight, taps, dtype):
+    """(cout, taps, cin) weight with cin == cout in MFMA fragment order for subm_conv_tiles."""
+    _dev(weight)
+    lib = _lib.load()
+    c = weight.shape[0]
+    w = weight.reshape(c, taps, c).to(dtype).contiguous()
+    packed = torch.empty_like(w)
+    _lib.check(lib.ptv3_subm_conv_pack_weight(_ptr(w), _dtype_code(w), c, taps, _ptr(packed), _stream()),
+               "ptv3_subm_conv_pack_weight")
+    return packed
+
+
+def subm_conv_tiles(feat, plan, packed_weight, bias=None):
+    """3x3x3 submanifold convolution with cin == cout, sums kept on chip per tile of outputs (fp16 / bf16)."""
+    _dev(feat, packed_weight, bias)
+    lib = _lib.load()
+    feat = feat.contiguous()
+    n, c = feat.shape
+    assert packed_weight.dtype == feat.dtype and packed_weight.numel() == plan.taps * c * c
+    b = None if bias is None else bias.to(feat.dtype).contiguous()
+    out = torch.empty((n, c), dtype=feat.dtype, device=feat.device)
+    tile_tap, tile_pair, vox_taps = plan.tiles()
+    _lib.check(lib.ptv3_subm_conv_tiles_fwd(_ptr(feat), _dtype_code(feat), n, c, plan.taps, _ptr(packed_weight), _ptr(b),
+                                            _ptr(tile_tap), _ptr(tile_pair), _ptr(vox_taps), _ptr(out), _stream()),
+               "ptv3_subm_conv_tiles_fwd")
     return out
 
 

@@ -59,6 +59,9 @@ class SubMConv3d(nn.Module):
     # (no pair-matrix round trip, but MFMA work for every tap); a 2 cm surface scan goes from 0.05
     # at full resolution to 0.5 at the coarsest level, where the two forms measure about equal
     PAIR_MODE_MAX_DENSITY = 0.6
+    # from this many pairs per voxel on, the tile form (sums kept on chip, no pair matrix through memory)
+    # measured faster than the pair form at 64 and 128 channels; sparser levels stay on the pair form
+    TILE_MODE_MIN_PAIRS_PER_VOXEL = 4.0
 
     def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
                  groups=1, bias=True, indice_key=None):
@@ -79,6 +82,16 @@ class SubMConv3d(nn.Module):
         if self.bias is not None:
             nn.init.uniform_(self.bias, -bound, bound)
 
+    def _packed_weight(self, dtype):
+        """The weight in the tile kernel's fragment order, repacked when the parameter changes."""
+        w = self.weight
+        key = (w.data_ptr(), w._version, dtype, w.device)
+        cached = getattr(self, "_packed", None)
+        if cached is None or cached[0] != key:
+            packed = ops.conv_pack_weight(w.detach().reshape(self.out_channels, -1, self.in_channels), 27, dtype)
+            self._packed = cached = (key, packed)
+        return cached[1]
+
     def forward(self, x):
         feat = x.features
         if torch.is_autocast_enabled():
@@ -93,8 +106,11 @@ class SubMConv3d(nn.Module):
             pad = 16 - cin % 16
             feat = nn.functional.pad(feat, (0, pad))
             weight = nn.functional.pad(weight, (0, pad))
-        weight = weight.to(feat.dtype)
         plan = x.conv_plan(self.kernel_size, self.indice_key)
+        if (self.kernel_size == 3 and cin == self.out_channels and cin in ops.CONV_TILE_CHANNELS
+                and plan.n < (1 << 24) and plan.n_pairs >= self.TILE_MODE_MIN_PAIRS_PER_VOXEL * plan.n):
+            return x.replace_feature(ops.subm_conv_tiles(feat, plan, self._packed_weight(feat.dtype), self.bias))
+        weight = weight.to(feat.dtype)
         if plan.density() <= self.PAIR_MODE_MAX_DENSITY and self.out_channels % 8 == 0:
             out = ops.subm_conv_pairs(feat, plan, weight, self.bias)
         else:

@@ -446,3 +446,34 @@ def test_linear_bn_act_parity(dtype, k, nout, n, gelu, stats_f32, affine):
     two = ops().bn_act(ops().linear_rows(x.to(DEV), lin_d.weight, lin_d.bias), bn_d.running_mean, bn_d.running_var,
                        bn_d.weight, bn_d.bias, bn_d.eps, gelu)
     assert rel_err(got, two.float().cpu()) < (2e-3 if dtype == torch.float16 else 1.6e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("c,n,extent", [(64, 3000, 20), (64, 50_000, 60), (128, 9000, 24), (128, 2000, 12), (64, 2, 4),
+                                        (128, 900, 8), (64, 40_001, 90), (128, 6000, 40), (64, 400, 6)])
+def test_subm_conv_tiles_parity(dtype, c, n, extent):
+    """Tile form of the xCPE convolution (sums kept on chip) against the oracle, from sparse scans to
+    nearly full grids (every tap of most voxels present), and the same bits on every run."""
+    rng = np.random.default_rng(c + n)
+    g = torch.Generator().manual_seed(c + n)
+    idx, *_ = _indices(rng, n // 2, extent, 2)
+    nbr = OI.subm_kmap(idx, 3)
+    feat = torch.randn(len(idx), c, generator=g).to(dtype)
+    bound = 1.0 / np.sqrt(27 * c)
+    w = ((torch.rand(c, 3, 3, 3, c, generator=g) * 2 - 1) * bound * 3).to(dtype)
+    b = ((torch.rand(c, generator=g) * 2 - 1) * 0.2).to(dtype)
+    want = OF.subm_conv(feat.float(), nbr, w.float(), b.float())
+    o = ops()
+    plan = o.conv_plan_direct(to_dev(idx), 3)
+    # the output-major words list every voxel's neighbours in tap order
+    sp = plan.slot_pair().cpu().numpy()[:plan.n_pairs]
+    v_idx, t_idx = np.nonzero(nbr >= 0)
+    assert np.array_equal(sp >> 24, t_idx) and np.array_equal(sp & 0xFFFFFF, nbr[v_idx, t_idx])
+    packed = o.conv_pack_weight(w.to(DEV), 27, dtype)
+    got = o.subm_conv_tiles(feat.to(DEV), plan, packed, b.to(DEV))
+    assert got.dtype == dtype and got.shape == (len(idx), c)
+    assert rel_err(got, want) < TOL[dtype]
+    again = o.subm_conv_tiles(feat.to(DEV), plan, packed, b.to(DEV))
+    assert torch.equal(got, again)
+    nob = o.subm_conv_tiles(feat.to(DEV), plan, packed, None)
+    assert rel_err(nob, OF.subm_conv(feat.float(), nbr, w.float(), None)) < TOL[dtype]
