@@ -206,11 +206,13 @@ __global__ __launch_bounds__(TileShape<C>::THREADS, TileShape<C>::OCC) void conv
     const int col = lane & 31, hf = lane >> 5;
     const int cw = wave % CW, pw = wave / CW;
     const int cout0 = blockIdx.y * COUT_WG;             // first output channel of the work-group
-    const int64_t v0 = (int64_t)blockIdx.x * TV;
+    // (giving each XCD one contiguous range of tiles instead of round-robin measured no faster)
+    const int tile = blockIdx.x;
+    const int64_t v0 = (int64_t)tile * TV;
     const int nv = (int)min((int64_t)TV, n - v0);
 
     // ---- the tile's pair list and chunk table
-    const int32_t* tt = tile_tap + (int64_t)blockIdx.x * CT_TILE_WORDS;
+    const int32_t* tt = tile_tap + (int64_t)tile * CT_TILE_WORDS;
     const int total = tt[CT_TAPS];
     const uint32_t* tp = tile_pair + tt[28];
     for (int e = tid; e < total; e += THREADS) plist[e] = tp[e];
@@ -290,6 +292,7 @@ __global__ __launch_bounds__(TileShape<C>::THREADS, TileShape<C>::OCC) void conv
             if (g * 32 + 31 >= lo && g * 32 <= hi) {   // uniform: the chunk has outputs in this group
                 const int o = g * 32 + col;
                 const bool present = ((taps_of[gi] >> t) & 1u) && o >= lo && o <= hi;
+                if (__ballot(present) == 0) continue;   // none of the group's outputs has this tap
                 // an absent neighbour reads the row of zeros: no branch, no registers to clear
                 const T* row = present ? xb + o * C : zero_row;
                 const int sw = present ? (o & 7) : 0;
