@@ -51,6 +51,10 @@ int ptv3_encode(const int32_t *grid_coord, const int64_t *batch, int64_t n, int 
  * per-axis maximum of grid_coord (n,3) int32 into out3 (3 int32, device). n >= 1. */
 int ptv3_grid_max(const int32_t *grid_coord, int64_t n, int32_t *out3, void *stream);
 
+/* model.py:35-40 (offset2batch): scene id of each of the n points from the cumulative scene ends
+ * offset (n_scenes,) int64 on the device, n = offset[n_scenes - 1] known to the caller. */
+int ptv3_offset2batch(const int64_t *offset, int n_scenes, int64_t n, int64_t *batch, void *stream);
+
 /* model.py:119-126 and :667-674: per-row ascending argsort of (k,n) int64 codes plus the
  * inverse permutation. Only the low `key_bits` bits are sorted on (the rest must be equal
  * across a row, e.g. zero); ties keep their input order. */
@@ -174,28 +178,35 @@ int ptv3_subm_conv_tiles_fwd(const void *feat, int dtype, int64_t n, int channel
 /* model.py:652-664,690-695: clusters of code0 >> shift walked in sorted order (order0 sorts
  * code0, so no further sort is needed). Outputs: cluster (n,) int64 [pooling_inverse],
  * indices (n,) int64 (= order0: points grouped by cluster), idx_ptr (n+1 allocated, m+1 used),
- * head (n allocated, m used), n_clusters (1,) int64 on the device. */
+ * head (n allocated, m used), n_clusters (1 + n_scenes,) int64 on the device: the cluster count,
+ * then (model.py:66-67 for the pooled point, without a bincount) the pooled cumulative scene ends
+ * from the parent's offset (n_scenes,) int64 on the device; n_scenes may be 0 (offset unused). */
 size_t ptv3_pool_clusters_workspace_bytes(int64_t n);
 int ptv3_pool_clusters(const int64_t *code0, const int64_t *order0, int64_t n, int shift,
-                       int64_t *cluster, int64_t *idx_ptr, int64_t *head, int64_t *n_clusters,
-                       void *workspace, size_t workspace_bytes, void *stream);
+                       const int64_t *offset, int n_scenes, int64_t *cluster, int64_t *idx_ptr,
+                       int64_t *head, int64_t *n_clusters, void *workspace, size_t workspace_bytes,
+                       void *stream);
 
 /* model.py:666-674,690,695 once the cluster count m is known on the host: pooled codes
  * (k,m) = code[:, head] >> shift, pooled grid_coord (m,3) = grid_coord[head] >> pool_depth,
- * pooled batch (m,) = batch[head]. */
+ * pooled batch (m,) = batch[head]; indices_out (m,4) int32 = [batch, x, y, z] of the pooled
+ * points, the sparse tensor's indices (model.py:165-167), or NULL. row_perm: host array of k ints,
+ * output row r is made from input row row_perm[r] (the shuffle of model.py:675-679 applied while
+ * writing; k <= 16), or NULL for the identity. */
 int ptv3_pool_gather(const int64_t *code, int64_t n, int k, int shift, const int32_t *grid_coord,
                      int pool_depth, const int64_t *batch, const int64_t *head, int64_t m,
-                     int64_t *code_out, int32_t *grid_coord_out, int64_t *batch_out,
-                     void *stream);
+                     const int32_t *row_perm, int64_t *code_out, int32_t *grid_coord_out,
+                     int64_t *batch_out, int32_t *indices_out, void *stream);
 
 /* model.py:667-674 without a sort: the pooled order of every curve is the sequence of distinct
  * clusters met when walking the parent points along that curve (order (k,n): the parent's
  * serialized_order; cluster (n,): pooling_inverse; m clusters). Writes order_out, inverse_out
  * (k,m) int64, identical to argsort of the pooled codes and its inverse. Requires what the
- * reference's pooling relies on too: a point's code shifted right is its cluster's code. */
+ * reference's pooling relies on too: a point's code shifted right is its cluster's code.
+ * row_perm as for ptv3_pool_gather. */
 size_t ptv3_pool_orders_workspace_bytes(int64_t n, int k);
 int ptv3_pool_orders(const int64_t *order, const int64_t *cluster, int64_t n, int k, int64_t m,
-                     int64_t *order_out, int64_t *inverse_out, void *workspace,
+                     const int32_t *row_perm, int64_t *order_out, int64_t *inverse_out, void *workspace,
                      size_t workspace_bytes, void *stream);
 
 /* torch_scatter.segment_csr call sites model.py:684-689: reduce src[indices[j]] over

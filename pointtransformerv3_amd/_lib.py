@@ -17,6 +17,7 @@ SIGNATURES = {
     "ptv3_strerror": (ctypes.c_char_p, [_i32]),
     "ptv3_encode": (_i32, [_vp, _vp, _i64, _i32, _vp, _i32, _vp, _vp]),
     "ptv3_grid_max": (_i32, [_vp, _i64, _vp, _vp]),
+    "ptv3_offset2batch": (_i32, [_vp, _i32, _i64, _vp, _vp]),
     "ptv3_argsort_workspace_bytes": (_sz, [_i64, _i32]),
     "ptv3_argsort": (_i32, [_vp, _i64, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
     "ptv3_pad_sizes": (_i32, [_vp, _i32, _i64, _vp, _vp]),
@@ -43,11 +44,11 @@ SIGNATURES = {
     "ptv3_subm_conv_pairs_fwd": (_i32, [_vp, _i32, _i64, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp,
                                         _i32, _vp, _vp, _vp]),
     "ptv3_pool_clusters_workspace_bytes": (_sz, [_i64]),
-    "ptv3_pool_clusters": (_i32, [_vp, _vp, _i64, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
-    "ptv3_pool_gather": (_i32, [_vp, _i64, _i32, _i32, _vp, _i32, _vp, _vp, _i64, _vp, _vp, _vp,
+    "ptv3_pool_clusters": (_i32, [_vp, _vp, _i64, _i32, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "ptv3_pool_gather": (_i32, [_vp, _i64, _i32, _i32, _vp, _i32, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp,
                                 _vp]),
     "ptv3_pool_orders_workspace_bytes": (_sz, [_i64, _i32]),
-    "ptv3_pool_orders": (_i32, [_vp, _vp, _i64, _i32, _i64, _vp, _vp, _vp, _sz, _vp]),
+    "ptv3_pool_orders": (_i32, [_vp, _vp, _i64, _i32, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "ptv3_segment_reduce": (_i32, [_vp, _i32, _i64, _i32, _vp, _vp, _i64, _i32, _vp, _vp]),
     "ptv3_unpool_add": (_i32, [_vp, _vp, _i32, _i64, _i32, _vp, _i64, _vp, _vp]),
     "ptv3_bn_act": (_i32, [_vp, _vp, _vp, _i32, _vp, _vp, _i32, _i64, _i32, _f32, _i32, _vp, _vp]),

@@ -110,7 +110,29 @@ __global__ __launch_bounds__(256) void grid_max_kernel(const int32_t* __restrict
     }
 }
 
+// scene id of every point from the cumulative scene ends: the number of ends <= i
+__global__ __launch_bounds__(256) void offset2batch_kernel(const int64_t* __restrict__ offset, int nb, int64_t n,
+                                                           int64_t* __restrict__ batch) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    int lo = 0, hi = nb;   // first scene whose end is > i
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (offset[mid] <= i) lo = mid + 1; else hi = mid;
+    }
+    batch[i] = lo;
+}
+
 }  // namespace
+
+extern "C" int ptv3_offset2batch(const int64_t* offset, int n_scenes, int64_t n, int64_t* batch, void* stream_) {
+    if (n < 0 || n_scenes < 1) return PTV3_EINVAL;
+    if (n == 0) return PTV3_OK;
+    if (!offset || !batch) return PTV3_EINVAL;
+    hipLaunchKernelGGL(offset2batch_kernel, dim3((unsigned)ptv3_ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream_,
+                       offset, n_scenes, n, batch);
+    PTV3_RETURN_LAUNCH();
+}
 
 extern "C" int ptv3_grid_max(const int32_t* grid_coord, int64_t n, int32_t* out3, void* stream_) {
     if (n < 1 || !grid_coord || !out3) return PTV3_EINVAL;

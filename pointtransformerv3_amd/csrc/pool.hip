@@ -101,11 +101,35 @@ __device__ __forceinline__ bool order_run_start(const int64_t* __restrict__ orde
     return cluster[order_row[i]] != cluster[order_row[i - 1]];
 }
 
+// Output row r of the pooled tables comes from input row src[r] (the reference permutes the rows
+// after pooling, model.py:675-679: the same tables, written once).
+constexpr int MAX_PERM_ROWS = 16;
+struct RowPerm {
+    int32_t src[MAX_PERM_ROWS];
+    int use;
+    __device__ __forceinline__ int of(int r) const { return use ? src[r] : r; }
+};
+
+RowPerm make_row_perm(const int32_t* host_perm, int k) {
+    RowPerm p;
+    p.use = host_perm != nullptr;
+    for (int r = 0; r < MAX_PERM_ROWS; ++r) p.src[r] = (host_perm && r < k) ? host_perm[r] : r;
+    return p;
+}
+
+bool row_perm_ok(const int32_t* host_perm, int k) {
+    if (!host_perm) return true;
+    if (k > MAX_PERM_ROWS) return false;
+    for (int r = 0; r < k; ++r)
+        if (host_perm[r] < 0 || host_perm[r] >= k) return false;
+    return true;
+}
+
 __global__ __launch_bounds__(PB) void order_count_kernel(const int64_t* __restrict__ order,
                                                          const int64_t* __restrict__ cluster, int64_t n,
-                                                         uint32_t* __restrict__ block_cnt) {
+                                                         RowPerm perm, uint32_t* __restrict__ block_cnt) {
     const int64_t i = (int64_t)blockIdx.x * PB + threadIdx.x;
-    const int64_t* row = order + (int64_t)blockIdx.y * n;
+    const int64_t* row = order + (int64_t)perm.of(blockIdx.y) * n;
     const uint32_t f = (i < n && order_run_start(row, cluster, i)) ? 1u : 0u;
     uint32_t total;
     block_inclusive_scan(f, &total);
@@ -128,11 +152,12 @@ __global__ __launch_bounds__(PB) void order_scan_kernel(uint32_t* __restrict__ b
 
 __global__ __launch_bounds__(PB) void order_assign_kernel(const int64_t* __restrict__ order,
                                                           const int64_t* __restrict__ cluster, int64_t n,
-                                                          int64_t m, const uint32_t* __restrict__ block_base,
+                                                          int64_t m, RowPerm perm,
+                                                          const uint32_t* __restrict__ block_base,
                                                           int64_t* __restrict__ order_out,
                                                           int64_t* __restrict__ inverse_out) {
     const int64_t i = (int64_t)blockIdx.x * PB + threadIdx.x;
-    const int64_t* row = order + (int64_t)blockIdx.y * n;
+    const int64_t* row = order + (int64_t)perm.of(blockIdx.y) * n;
     const bool f = i < n && order_run_start(row, cluster, i);
     uint32_t total;
     const uint32_t inc = block_inclusive_scan(f ? 1u : 0u, &total);
@@ -147,17 +172,35 @@ __global__ __launch_bounds__(PB) void order_assign_kernel(const int64_t* __restr
 __global__ __launch_bounds__(256) void pool_gather_kernel(
     const int64_t* __restrict__ code, int64_t n, int k, int shift,
     const int32_t* __restrict__ grid_coord, int pool_depth, const int64_t* __restrict__ batch,
-    const int64_t* __restrict__ head, int64_t m, int64_t* __restrict__ code_out,
-    int32_t* __restrict__ grid_coord_out, int64_t* __restrict__ batch_out) {
+    const int64_t* __restrict__ head, int64_t m, RowPerm perm, int64_t* __restrict__ code_out,
+    int32_t* __restrict__ grid_coord_out, int64_t* __restrict__ batch_out, int32_t* __restrict__ indices_out) {
     const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (j >= m) return;
     const int64_t h = head[j];
-    for (int r = 0; r < k; ++r) code_out[(int64_t)r * m + j] = code[(int64_t)r * n + h] >> shift;
+    for (int r = 0; r < k; ++r) code_out[(int64_t)r * m + j] = code[(int64_t)perm.of(r) * n + h] >> shift;
+    int32_t g[3] = {0, 0, 0};
+    if (grid_coord) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) g[a] = grid_coord[3 * h + a] >> pool_depth;
+    }
+    const int64_t b = batch ? batch[h] : 0;
     if (grid_coord_out) {
 #pragma unroll
-        for (int a = 0; a < 3; ++a) grid_coord_out[3 * j + a] = grid_coord[3 * h + a] >> pool_depth;
+        for (int a = 0; a < 3; ++a) grid_coord_out[3 * j + a] = g[a];
     }
-    if (batch_out) batch_out[j] = batch[h];
+    if (batch_out) batch_out[j] = b;
+    if (indices_out) ((int4*)indices_out)[j] = make_int4((int32_t)b, g[0], g[1], g[2]);
+}
+
+// pooled scene ends: scene s ends with the cluster of its last point in sorted order
+__global__ __launch_bounds__(256) void pool_offsets_kernel(const int64_t* __restrict__ offset, int nb,
+                                                           const int64_t* __restrict__ order0,
+                                                           const int64_t* __restrict__ cluster,
+                                                           int64_t* __restrict__ out) {
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= nb) return;
+    const int64_t last = offset[j] - 1;   // -1: no point so far
+    out[j] = last >= 0 ? cluster[order0[last]] + 1 : 0;
 }
 
 template <typename T> __device__ __forceinline__ float ld(const T* p) { return (float)*p; }
@@ -250,10 +293,11 @@ extern "C" size_t ptv3_pool_clusters_workspace_bytes(int64_t n) {
 }
 
 extern "C" int ptv3_pool_clusters(const int64_t* code0, const int64_t* order0, int64_t n, int shift,
-                                  int64_t* cluster, int64_t* idx_ptr, int64_t* head,
-                                  int64_t* n_clusters, void* workspace, size_t workspace_bytes,
+                                  const int64_t* offset, int n_scenes, int64_t* cluster, int64_t* idx_ptr,
+                                  int64_t* head, int64_t* n_clusters, void* workspace, size_t workspace_bytes,
                                   void* stream_) {
-    if (n < 1 || n >= (1ll << 31) || shift < 0 || shift > 62) return PTV3_EINVAL;
+    if (n < 1 || n >= (1ll << 31) || shift < 0 || shift > 62 || n_scenes < 0) return PTV3_EINVAL;
+    if (n_scenes > 0 && !offset) return PTV3_EINVAL;
     if (!code0 || !order0 || !cluster || !idx_ptr || !head || !n_clusters || !workspace) return PTV3_EINVAL;
     if (workspace_bytes < ptv3_pool_clusters_workspace_bytes(n)) return PTV3_EWORKSPACE;
     hipStream_t stream = (hipStream_t)stream_;
@@ -264,21 +308,26 @@ extern "C" int ptv3_pool_clusters(const int64_t* code0, const int64_t* order0, i
     hipLaunchKernelGGL(cluster_scan_kernel, dim3(1), dim3(PB), 0, stream, block_cnt, blocks, n_clusters);
     hipLaunchKernelGGL(cluster_assign_kernel, dim3((unsigned)blocks), dim3(PB), 0, stream, code0, order0, n,
                        shift, (const uint32_t*)block_cnt, cluster, idx_ptr, head);
+    if (n_scenes > 0)
+        hipLaunchKernelGGL(pool_offsets_kernel, dim3((unsigned)ptv3_ceil_div(n_scenes, 256)), dim3(256), 0, stream,
+                           offset, n_scenes, order0, (const int64_t*)cluster, n_clusters + 1);
     PTV3_RETURN_LAUNCH();
 }
 
 extern "C" int ptv3_pool_gather(const int64_t* code, int64_t n, int k, int shift,
                                 const int32_t* grid_coord, int pool_depth, const int64_t* batch,
-                                const int64_t* head, int64_t m, int64_t* code_out,
-                                int32_t* grid_coord_out, int64_t* batch_out, void* stream) {
+                                const int64_t* head, int64_t m, const int32_t* row_perm, int64_t* code_out,
+                                int32_t* grid_coord_out, int64_t* batch_out, int32_t* indices_out, void* stream) {
     if (n < 0 || m < 0 || m > n || k < 1 || shift < 0 || shift > 62 || pool_depth < 0 || pool_depth > 31)
         return PTV3_EINVAL;
+    if (!row_perm_ok(row_perm, k)) return PTV3_EINVAL;
     if (m == 0) return PTV3_OK;
     if (!code || !head || !code_out) return PTV3_EINVAL;
-    if ((grid_coord_out && !grid_coord) || (batch_out && !batch)) return PTV3_EINVAL;
+    if ((grid_coord_out && !grid_coord) || (batch_out && !batch) || (indices_out && (!grid_coord || !batch)))
+        return PTV3_EINVAL;
     hipLaunchKernelGGL(pool_gather_kernel, dim3((unsigned)ptv3_ceil_div(m, 256)), dim3(256), 0,
                        (hipStream_t)stream, code, n, k, shift, grid_coord, pool_depth, batch, head, m,
-                       code_out, grid_coord_out, batch_out);
+                       make_row_perm(row_perm, k), code_out, grid_coord_out, batch_out, indices_out);
     PTV3_RETURN_LAUNCH();
 }
 
@@ -315,18 +364,20 @@ extern "C" size_t ptv3_pool_orders_workspace_bytes(int64_t n, int k) {
 }
 
 extern "C" int ptv3_pool_orders(const int64_t* order, const int64_t* cluster, int64_t n, int k, int64_t m,
-                                int64_t* order_out, int64_t* inverse_out, void* workspace,
+                                const int32_t* row_perm, int64_t* order_out, int64_t* inverse_out, void* workspace,
                                 size_t workspace_bytes, void* stream_) {
     if (n < 1 || n >= (1ll << 31) || k < 1 || k > 65535 || m < 1 || m > n) return PTV3_EINVAL;
+    if (!row_perm_ok(row_perm, k)) return PTV3_EINVAL;
+    const RowPerm perm = make_row_perm(row_perm, k);
     if (!order || !cluster || !order_out || !inverse_out || !workspace) return PTV3_EINVAL;
     if (workspace_bytes < ptv3_pool_orders_workspace_bytes(n, k)) return PTV3_EWORKSPACE;
     hipStream_t stream = (hipStream_t)stream_;
     const int64_t blocks = ptv3_ceil_div(n, PB);
     uint32_t* block_cnt = (uint32_t*)workspace;
     const dim3 grid((unsigned)blocks, (unsigned)k);
-    hipLaunchKernelGGL(order_count_kernel, grid, dim3(PB), 0, stream, order, cluster, n, block_cnt);
+    hipLaunchKernelGGL(order_count_kernel, grid, dim3(PB), 0, stream, order, cluster, n, perm, block_cnt);
     hipLaunchKernelGGL(order_scan_kernel, dim3((unsigned)k), dim3(PB), 0, stream, block_cnt, blocks);
-    hipLaunchKernelGGL(order_assign_kernel, grid, dim3(PB), 0, stream, order, cluster, n, m,
+    hipLaunchKernelGGL(order_assign_kernel, grid, dim3(PB), 0, stream, order, cluster, n, m, perm,
                        (const uint32_t*)block_cnt, order_out, inverse_out);
     PTV3_RETURN_LAUNCH();
 }

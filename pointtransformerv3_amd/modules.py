@@ -352,7 +352,7 @@ class Block(PointModule):
             feat = ops.mlp_fused(normed, feat, mlp.fc1.weight, mlp.fc1.bias, mlp.fc2.weight, mlp.fc2.bias)
         elif plain_mlp:
             hidden = ops.linear(normed, mlp.fc1, gelu=True) if exact_gelu else mlp.act(mlp.fc1(normed))
-            feat = torch.addmm(feat, hidden, mlp.fc2.weight.t())
+            feat = feat.addmm_(hidden, mlp.fc2.weight.to(hidden.dtype).t())   # onto the stored sum, no copy of it
         else:
             feat = feat + mlp(normed)
         point.feat = feat
@@ -418,14 +418,13 @@ class SerializedPooling(PointModule):
         indices = point.serialized_order[0]
         cluster, idx_ptr, head, m, offset, offset_host = ops.pool_clusters(point.serialized_code[0], indices, shift,
                                                                            point.offset)
-        code, grid_coord, batch = ops.pool_gather(point.serialized_code, shift, point.grid_coord,
-                                                  pooling_depth, point.batch, head)
+        # the shuffle of the orders (model.py:675-679) is applied while the pooled tables are written
+        perm = torch.randperm(point.serialized_code.shape[0]).tolist() if self.shuffle_orders else None   # CPU generator
+        code, grid_coord, batch, indices4 = ops.pool_gather(point.serialized_code, shift, point.grid_coord,
+                                                            pooling_depth, point.batch, head, perm)
         # pooled orders: the distinct clusters met when walking the parent along each curve (same
         # result as argsort of the pooled codes, model.py:667-674, without sorting)
-        order, inverse = ops.pool_orders(point.serialized_order, cluster, m)
-        if self.shuffle_orders:
-            perm = torch.randperm(code.shape[0]).tolist()   # CPU generator (model.py:677)
-            code, order, inverse = ops.permute_rows(perm, code, order, inverse)
+        order, inverse = ops.pool_orders(point.serialized_order, cluster, m, perm)
 
         fields = AttrDict(
             feat=ops.segment_reduce(ops.linear(point.feat, self.proj), indices, idx_ptr, self.reduce),
@@ -437,6 +436,7 @@ class SerializedPooling(PointModule):
             batch=batch,
             offset=offset,   # what batch2offset(batch) would compute (model.py:66-67), without its host syncs
             _offset_host=offset_host,
+            _sparse_indices=indices4,   # [batch, x, y, z] int32, what sparsify() would concatenate
         )
         if "coord" in point:
             fields["coord"] = ops.segment_reduce(point.coord.float(), indices, idx_ptr, "mean")

@@ -73,6 +73,16 @@ def grid_max(grid_coord):
     return out
 
 
+def offset2batch(offset, n):
+    """Scene id (int64) of each of n points from the cumulative scene ends on the device."""
+    _dev(offset)
+    lib = _lib.load()
+    off = offset.to(torch.int64).contiguous()
+    batch = torch.empty(int(n), dtype=torch.int64, device=off.device)
+    _lib.check(lib.ptv3_offset2batch(_ptr(off), off.shape[0], int(n), _ptr(batch), _stream()), "ptv3_offset2batch")
+    return batch
+
+
 def argsort_rows(code, key_bits):
     """Row-wise ascending argsort of (k,N) int64 codes + inverse permutation."""
     _dev(code)
@@ -362,30 +372,34 @@ def pool_clusters(code0, order0, shift, offset=None):
     cluster = torch.empty(n, dtype=torch.int64, device=dev)
     idx_ptr = torch.empty(n + 1, dtype=torch.int64, device=dev)
     head = torch.empty(n, dtype=torch.int64, device=dev)
-    count = torch.empty(1, dtype=torch.int64, device=dev)
+    nb = 0 if offset is None else offset.shape[0]
+    count = torch.empty(1 + nb, dtype=torch.int64, device=dev)   # cluster count, then the pooled scene ends
+    off = None if offset is None else offset.to(torch.int64).contiguous()
     nbytes = lib.ptv3_pool_clusters_workspace_bytes(n)
     ws = _ws(nbytes, dev)
-    _lib.check(lib.ptv3_pool_clusters(_ptr(code0.contiguous()), _ptr(order0), n, int(shift),
+    _lib.check(lib.ptv3_pool_clusters(_ptr(code0.contiguous()), _ptr(order0), n, int(shift), _ptr(off), nb,
                                       _ptr(cluster), _ptr(idx_ptr), _ptr(head), _ptr(count), _ptr(ws),
                                       nbytes, _stream()), "ptv3_pool_clusters")
-    if offset is None:
-        m = int(count.item())
-        return cluster, idx_ptr[: m + 1], head[:m], m
-    last = offset.long() - 1   # sorted position of each scene's last point (-1: no point so far)
-    pooled_offset = torch.where(last >= 0, cluster[order0[last.clamp(min=0)]] + 1, torch.zeros_like(last))
-    host = torch.cat([count, pooled_offset]).tolist()
+    host = count.tolist()
     m = int(host[0])
-    return cluster, idx_ptr[: m + 1], head[:m], m, pooled_offset, [int(v) for v in host[1:]]
+    if offset is None:
+        return cluster, idx_ptr[: m + 1], head[:m], m
+    return cluster, idx_ptr[: m + 1], head[:m], m, count[1:], [int(v) for v in host[1:]]
 
 
-def permute_rows(rows, *tensors):
-    """tensor[rows] for a short host list of row indices, as one concatenation per tensor: an
-    index tensor would first have to be copied to the device, which waits for the stream."""
-    return tuple(torch.stack([t[i] for i in rows]) for t in tensors)
+def _row_perm(rows, k):
+    """Host int32 array for the row_perm argument of the pooling kernels (None: identity)."""
+    if rows is None:
+        return None, None
+    assert len(rows) == k
+    arr = (ctypes.c_int32 * k)(*[int(r) for r in rows])
+    return arr, ctypes.cast(arr, ctypes.c_void_p)
 
 
-def pool_gather(code, shift, grid_coord, pool_depth, batch, head):
-    """Pooled code (k,M), grid_coord (M,3) int32, batch (M,) at the cluster heads."""
+def pool_gather(code, shift, grid_coord, pool_depth, batch, head, rows=None):
+    """Pooled code (k,M), grid_coord (M,3) int32, batch (M,) at the cluster heads, and the (M,4)
+    int32 [batch, x, y, z] indices of the pooled sparse tensor. With rows (a host list), output
+    row r of the code comes from input row rows[r]."""
     _dev(code, grid_coord, batch, head)
     lib = _lib.load()
     code = code.contiguous()
@@ -397,15 +411,18 @@ def pool_gather(code, shift, grid_coord, pool_depth, batch, head):
     gc_out = torch.empty((m, 3), dtype=torch.int32, device=dev)
     b = batch.to(torch.int64).contiguous()
     b_out = torch.empty(m, dtype=torch.int64, device=dev)
+    idx_out = torch.empty((m, 4), dtype=torch.int32, device=dev)
+    keep, perm = _row_perm(rows, k)
     _lib.check(lib.ptv3_pool_gather(_ptr(code), n, k, int(shift), _ptr(gc), int(pool_depth), _ptr(b),
-                                    _ptr(head.contiguous()), m, _ptr(code_out), _ptr(gc_out), _ptr(b_out),
-                                    _stream()), "ptv3_pool_gather")
-    return code_out, gc_out, b_out
+                                    _ptr(head.contiguous()), m, perm, _ptr(code_out), _ptr(gc_out), _ptr(b_out),
+                                    _ptr(idx_out), _stream()), "ptv3_pool_gather")
+    return code_out, gc_out, b_out, idx_out
 
 
-def pool_orders(order, cluster, m):
+def pool_orders(order, cluster, m, rows=None):
     """Pooled serialization orders and inverses (k,M) from the parent's orders (k,N) and the
-    cluster of every parent point — no sort (see ptv3_pool_orders)."""
+    cluster of every parent point — no sort (see ptv3_pool_orders). With rows (a host list),
+    output row r comes from input row rows[r]."""
     _dev(order, cluster)
     lib = _lib.load()
     order = order.contiguous()
@@ -415,7 +432,8 @@ def pool_orders(order, cluster, m):
     inverse_out = torch.empty((k, m), dtype=torch.int64, device=dev)
     nbytes = lib.ptv3_pool_orders_workspace_bytes(n, k)
     ws = _ws(nbytes, dev)
-    _lib.check(lib.ptv3_pool_orders(_ptr(order), _ptr(cluster.contiguous()), n, k, int(m), _ptr(order_out),
+    keep, perm = _row_perm(rows, k)
+    _lib.check(lib.ptv3_pool_orders(_ptr(order), _ptr(cluster.contiguous()), n, k, int(m), perm, _ptr(order_out),
                                     _ptr(inverse_out), _ptr(ws), nbytes, _stream()), "ptv3_pool_orders")
     return order_out, inverse_out
 

@@ -23,6 +23,8 @@ def offset2bincount(offset):
 def offset2batch(offset, n=None):
     """Scene id per point from cumulative scene ends (model.py:35-40). With the number of points
     given, the result is sized without reading the offsets back to the host."""
+    if n is not None and offset.is_cuda:
+        return ops.offset2batch(offset, n)
     sizes = offset2bincount(offset)
     ids = torch.arange(sizes.numel(), device=offset.device, dtype=torch.long)
     return ids.repeat_interleave(sizes, output_size=n)
@@ -120,13 +122,14 @@ class Point(AttrDict):
         assert depth * 3 + n_scenes.bit_length() <= 63       # model.py:103
         assert depth <= 16                                    # model.py:108
 
+        if shuffle_orders:
+            # model.py:127-132 permutes the rows of code / order / inverse afterwards; a row depends
+            # on nothing but its order, so encoding the orders in permuted sequence gives the same tables
+            perm = torch.randperm(len(orders)).tolist()       # CPU generator, as model.py:129
+            orders = [orders[i] for i in perm]
         code = ops.encode_orders(self["grid_coord"], self["batch"], depth, orders)
         key_bits = 3 * depth + max(1, (n_scenes - 1).bit_length())
         sort_order, inverse = ops.argsort_rows(code, key_bits)
-
-        if shuffle_orders:
-            perm = torch.randperm(code.shape[0]).tolist()     # CPU generator, as model.py:129
-            code, sort_order, inverse = ops.permute_rows(perm, code, sort_order, inverse)
 
         self["serialized_code"] = code
         self["serialized_order"] = sort_order
@@ -143,7 +146,9 @@ class Point(AttrDict):
             sparse_shape = self["sparse_shape"]
         else:
             sparse_shape = [v + pad for v in self.grid_max_host()]
-        indices = torch.cat([self["batch"].unsqueeze(-1).int(), self["grid_coord"].int()], dim=1).contiguous()
+        indices = self.get("_sparse_indices")
+        if indices is None:
+            indices = torch.cat([self["batch"].unsqueeze(-1).int(), self["grid_coord"].int()], dim=1).contiguous()
         self["sparse_shape"] = sparse_shape
         self["sparse_conv_feat"] = SparseConvTensor(
             features=self["feat"], indices=indices, spatial_shape=sparse_shape,

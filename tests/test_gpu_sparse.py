@@ -75,10 +75,33 @@ def test_pool_clusters_and_gather_bit_exact():
     # the reference takes whichever member an unstable sort puts first (model.py:660-664);
     # only values shared by all members are read through it, so membership is the contract
     assert np.array_equal(want["cluster"][head.cpu().numpy()], np.arange(m))
-    pc, pg, pb = o.pool_gather(to_dev(code), 3, to_dev(g), 1, to_dev(batch), head)
+    pc, pg, pb, p4 = o.pool_gather(to_dev(code), 3, to_dev(g), 1, to_dev(batch), head)
     assert np.array_equal(pc.cpu().numpy(), want["code"])
     assert np.array_equal(pg.cpu().numpy(), want["grid_coord"])
     assert np.array_equal(pb.cpu().numpy(), want["batch"])
+    # the sparse tensor's indices are [batch, x, y, z] of the pooled points (model.py:165-167)
+    assert np.array_equal(p4.cpu().numpy(), np.concatenate([want["batch"][:, None], want["grid_coord"]], 1))
+    # pooled scene ends, read back with the cluster count, equal bincount(batch).cumsum (model.py:43-45, :66-67)
+    res = o.pool_clusters(to_dev(code[0]), to_dev(order[0]), 3, to_dev(offset))
+    assert res[3] == m and torch.equal(res[0], cluster)
+    want_off = np.cumsum(np.bincount(want["batch"], minlength=len(offset)))
+    assert np.array_equal(res[4].cpu().numpy(), want_off) and res[5] == want_off.tolist()
+    # rows written in shuffled order (model.py:675-679) are the rows of the unshuffled tables
+    rows = [2, 0, 3, 1]
+    po, pi = o.pool_orders(to_dev(order), cluster, m)
+    qc, _, _, _ = o.pool_gather(to_dev(code), 3, to_dev(g), 1, to_dev(batch), head, rows)
+    qo, qi = o.pool_orders(to_dev(order), cluster, m, rows)
+    assert torch.equal(qc, pc[rows]) and torch.equal(qo, po[rows]) and torch.equal(qi, pi[rows])
+
+
+def test_offset2batch_matches_repeat_interleave():
+    from pointtransformerv3_amd import point as P
+    for sizes in ([5], [3, 0, 4], [1000, 1, 70_000, 12], [0, 0, 9]):
+        offset = torch.tensor(sizes).cumsum(0)
+        n = int(offset[-1])
+        want = torch.arange(len(sizes)).repeat_interleave(torch.tensor(sizes))
+        got = P.offset2batch(offset.to(DEV), n)
+        assert got.dtype == torch.int64 and torch.equal(got.cpu(), want)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
@@ -326,7 +349,7 @@ def test_pool_orders_equal_argsort_of_pooled_codes(n, extent, nb):
         cluster, idx_ptr, head, m = o.pool_clusters(to_dev(c[0]), to_dev(od[0]), 3)
         po, pi = o.pool_orders(to_dev(od), cluster, m)
         assert np.array_equal(po.cpu().numpy(), w["order"]) and np.array_equal(pi.cpu().numpy(), w["inverse"])
-        pc, _, _ = o.pool_gather(to_dev(c), 3, to_dev(g), 1, to_dev(batch), head)
+        pc, _, _, _ = o.pool_gather(to_dev(c), 3, to_dev(g), 1, to_dev(batch), head)
         so, si = o.argsort_rows(pc, 3 * (depth - 1) + 2)
         assert torch.equal(so, po) and torch.equal(si, pi)
     assert m == len(want["counts"])
