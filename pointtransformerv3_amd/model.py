@@ -75,6 +75,7 @@ class PointTransformerV3(PointModule):
 
         self.embedding = Embedding(in_channels=in_channels, embed_channels=enc_channels[0],
                                    norm_layer=bn, act_layer=act)
+        self.stride = tuple(stride)
 
         # encoder: stochastic-depth rate grows linearly over all encoder blocks
         rates = [r.item() for r in torch.linspace(0, drop_path, sum(enc_depths))]
@@ -82,8 +83,10 @@ class PointTransformerV3(PointModule):
         for s in range(n):
             stage = PointSequential()
             if s > 0:
-                stage.add(SerializedPooling(in_channels=enc_channels[s - 1], out_channels=enc_channels[s],
-                                            stride=stride[s - 1], norm_layer=bn, act_layer=act), name="down")
+                down = SerializedPooling(in_channels=enc_channels[s - 1], out_channels=enc_channels[s],
+                                         stride=stride[s - 1], norm_layer=bn, act_layer=act)
+                down.next_stride = stride[s] if s < n - 1 else None   # the pooling that follows on its output
+                stage.add(down, name="down")
             first = sum(enc_depths[:s])
             for i in range(enc_depths[s]):
                 stage.add(make_block(enc_channels[s], enc_num_head[s], enc_patch_size[s], rates[first + i], i, s),
@@ -107,11 +110,21 @@ class PointTransformerV3(PointModule):
                               name=f"block{i}")
                 self.dec.add(module=stage, name=f"dec{s}")
 
+    def _level0_kernel_sizes(self):
+        from .sparse import SubMConv3d
+        mods = list(self.embedding.modules()) + list(next(iter(self.enc._modules.values())).modules())
+        return tuple(sorted({m.kernel_size for m in mods if isinstance(m, SubMConv3d)}, reverse=True))
+
     def forward(self, data_dict):
         """data_dict: feat, grid_coord (or coord + grid_size), offset or batch. Returns the Point
         whose feat is (N, dec_channels[0]) in the original point order."""
         point = Point(data_dict)
+        # the pair lists of the stem and of the first stage's xCPE depend on the coordinates only:
+        # their first halves are queued behind the first host read-back and run while the host waits
+        point.plan_ahead(self._level0_kernel_sizes())
         point.serialization(order=self.order, shuffle_orders=self.shuffle_orders)
+        if self.stride:
+            point.pool_ahead(self.stride[0])   # the first pooling's clusters need the codes only
         point.sparsify()
         point = self.embedding(point)
         point = self.enc(point)

@@ -393,6 +393,13 @@ class SerializedPooling(PointModule):
     numbers them (no unique, no sort), a gather kernel produces the pooled codes, coordinates
     and scene ids, and a segment kernel reduces the projected features."""
 
+    # kernel sizes of the convolutions that follow on the pooled points (the xCPE of every Block is
+    # 3x3x3, model.py:546-552): their pair lists are started as soon as the pooled coordinates exist
+    plan_kernel_sizes = (3,)
+    # stride of the pooling module that follows on this one's output, if any: its clusters are started
+    # as soon as the pooled codes exist
+    next_stride = None
+
     def __init__(self, in_channels, out_channels, stride=2, norm_layer=None, act_layer=None,
                  reduce="max", shuffle_orders=True, traceable=True):
         super().__init__()
@@ -416,18 +423,23 @@ class SerializedPooling(PointModule):
 
         # clusters in ascending order of the (shifted) row-0 code
         indices = point.serialized_order[0]
-        cluster, idx_ptr, head, m, offset, offset_host = ops.pool_clusters(point.serialized_code[0], indices, shift,
-                                                                           point.offset)
+        ahead = point.pop("_pending_pool", None)   # started when the codes came into being (Point.pool_ahead)
+        pending = ahead[1] if ahead is not None and ahead[0] == shift else \
+            ops.pool_clusters_start(point.serialized_code[0], indices, shift, point.offset)
+        projected = ops.linear(point.feat, self.proj)   # needs no cluster count: runs while the count travels
+        cluster, idx_ptr, head, m, offset, offset_host = ops.pool_clusters_finish(pending)
         # the shuffle of the orders (model.py:675-679) is applied while the pooled tables are written
         perm = torch.randperm(point.serialized_code.shape[0]).tolist() if self.shuffle_orders else None   # CPU generator
         code, grid_coord, batch, indices4 = ops.pool_gather(point.serialized_code, shift, point.grid_coord,
                                                             pooling_depth, point.batch, head, perm)
         # pooled orders: the distinct clusters met when walking the parent along each curve (same
         # result as argsort of the pooled codes, model.py:667-674, without sorting)
+        # pair lists of the convolutions on the pooled points: first half queued now, finished at first use
+        plans = {ks: ops.conv_plan_direct_start(indices4, ks) for ks in self.plan_kernel_sizes}
         order, inverse = ops.pool_orders(point.serialized_order, cluster, m, perm)
 
         fields = AttrDict(
-            feat=ops.segment_reduce(ops.linear(point.feat, self.proj), indices, idx_ptr, self.reduce),
+            feat=ops.segment_reduce(projected, indices, idx_ptr, self.reduce),
             grid_coord=grid_coord,
             serialized_code=code,
             serialized_order=order,
@@ -437,6 +449,7 @@ class SerializedPooling(PointModule):
             offset=offset,   # what batch2offset(batch) would compute (model.py:66-67), without its host syncs
             _offset_host=offset_host,
             _sparse_indices=indices4,   # [batch, x, y, z] int32, what sparsify() would concatenate
+            _pending_plans=plans,
         )
         if "coord" in point:
             fields["coord"] = ops.segment_reduce(point.coord.float(), indices, idx_ptr, "mean")
@@ -460,6 +473,8 @@ class SerializedPooling(PointModule):
             if self.act is not None:
                 pooled = self.act(pooled)
         pooled.sparsify()
+        if self.next_stride is not None:
+            pooled.pool_ahead(self.next_stride)
         return pooled
 
 

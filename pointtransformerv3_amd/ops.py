@@ -38,6 +38,33 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
+class Readback:
+    """Device -> host read of a small tensor that does not drain the stream.
+
+    A plain .tolist() / .item() waits for everything queued on the stream and leaves the GPU idle
+    until the host has queued new work. Here the copy into pinned memory is queued right behind the
+    producing kernels, followed by an event; get() waits for that event only, so whatever the host
+    queued on the stream in between keeps the GPU busy while the value travels."""
+
+    blocking = False   # True: plain stream-draining copy at get() (for comparison)
+
+    def __init__(self, tensor):
+        if Readback.blocking:
+            self.tensor = tensor
+            return
+        self.host = torch.empty(tensor.shape, dtype=tensor.dtype, pin_memory=True)
+        self.host.copy_(tensor, non_blocking=True)
+        self.done = torch.cuda.Event()
+        self.done.record(torch.cuda.current_stream(tensor.device))
+
+    def get(self):
+        """The values as a Python list (waits for the copy only)."""
+        if Readback.blocking:
+            return self.tensor.tolist()
+        self.done.synchronize()
+        return self.host.tolist()
+
+
 def _ws(nbytes, device):
     return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
 
@@ -282,9 +309,16 @@ def conv_plan(nbr, tap_major=False):
     return plan
 
 
-def conv_plan_direct(indices, ks):
-    """The pair lists of conv_plan(kmap_build(indices, ks)) straight from the (N,4) int32
-    [batch,x,y,z] voxel coordinates, without storing the neighbour map. One host sync (the pair count)."""
+class PendingPlan:
+    """conv_plan_direct between its two kernels: the pair count is on its way to the host."""
+
+    __slots__ = ("plan", "idx", "ks", "ws", "nbytes", "count")
+
+
+def conv_plan_direct_start(indices, ks):
+    """First half of conv_plan_direct: voxel hash and pair counts are queued and the total starts its
+    way to the host; conv_plan_direct_finish completes the lists. Work queued in between overlaps
+    the read-back instead of waiting behind it."""
     _dev(indices)
     lib = _lib.load()
     idx = indices.to(torch.int32).contiguous()
@@ -298,14 +332,30 @@ def conv_plan_direct(indices, ks):
     ws = _ws(nbytes, dev)
     _lib.check(lib.ptv3_kmap_plan_count(_ptr(idx), n, int(ks), _ptr(plan.tap_ptr), _ptr(count), _ptr(ws), nbytes,
                                         _stream()), "ptv3_kmap_plan_count")
-    plan.n_pairs = int(count.item())
+    pend = PendingPlan()
+    pend.plan, pend.idx, pend.ks, pend.ws, pend.nbytes = plan, idx, int(ks), ws, nbytes
+    pend.count = Readback(count)
+    return pend
+
+
+def conv_plan_direct_finish(pend):
+    lib = _lib.load()
+    plan, idx, n = pend.plan, pend.idx, pend.plan.n
+    dev = idx.device
+    plan.n_pairs = int(pend.count.get()[0])
     plan.row_ptr = torch.empty(n + 1, dtype=torch.int32, device=dev)
     plan.pair_in = torch.empty(max(plan.n_pairs, 1), dtype=torch.int32, device=dev)
     plan.pair_slot = torch.empty(max(plan.n_pairs, 1), dtype=torch.int32, device=dev)
-    _lib.check(lib.ptv3_kmap_plan_fill(_ptr(idx), n, int(ks), _ptr(plan.tap_ptr), _ptr(plan.row_ptr),
-                                       _ptr(plan.pair_in), _ptr(plan.pair_slot), _ptr(ws), nbytes, _stream()),
+    _lib.check(lib.ptv3_kmap_plan_fill(_ptr(idx), n, pend.ks, _ptr(plan.tap_ptr), _ptr(plan.row_ptr),
+                                       _ptr(plan.pair_in), _ptr(plan.pair_slot), _ptr(pend.ws), pend.nbytes, _stream()),
                "ptv3_kmap_plan_fill")
     return plan
+
+
+def conv_plan_direct(indices, ks):
+    """The pair lists of conv_plan(kmap_build(indices, ks)) straight from the (N,4) int32
+    [batch,x,y,z] voxel coordinates, without storing the neighbour map. One read-back (the pair count)."""
+    return conv_plan_direct_finish(conv_plan_direct_start(indices, ks))
 
 
 def subm_conv_pairs(feat, plan, weight, bias=None):
@@ -357,34 +407,51 @@ def subm_conv_tiles(feat, plan, packed_weight, bias=None):
     return out
 
 
-def pool_clusters(code0, order0, shift, offset=None):
-    """Clusters of code0 >> shift in sorted order. One host sync (the cluster count).
+class PendingClusters:
+    __slots__ = ("cluster", "idx_ptr", "head", "count", "read", "with_offset")
 
-    Returns cluster (N,), idx_ptr (M+1,), head (M,), M; with `offset` (the parent's cumulative
-    scene ends, on the device) also the pooled scene ends as a device tensor and as a Python
-    list, read in the same device->host copy as the count. Scenes are runs of the sorted order
-    (the scene id is the top of every code), so scene b ends with the cluster of its last point."""
+
+def pool_clusters_start(code0, order0, shift, offset=None):
+    """Queues the cluster kernels of pool_clusters and starts the read-back of the cluster count
+    (and the pooled scene ends); pool_clusters_finish returns what pool_clusters does."""
     _dev(code0, order0, offset)
     lib = _lib.load()
     n = code0.shape[0]
     dev = code0.device
     order0 = order0.contiguous()
-    cluster = torch.empty(n, dtype=torch.int64, device=dev)
-    idx_ptr = torch.empty(n + 1, dtype=torch.int64, device=dev)
-    head = torch.empty(n, dtype=torch.int64, device=dev)
+    pend = PendingClusters()
+    pend.cluster = torch.empty(n, dtype=torch.int64, device=dev)
+    pend.idx_ptr = torch.empty(n + 1, dtype=torch.int64, device=dev)
+    pend.head = torch.empty(n, dtype=torch.int64, device=dev)
     nb = 0 if offset is None else offset.shape[0]
-    count = torch.empty(1 + nb, dtype=torch.int64, device=dev)   # cluster count, then the pooled scene ends
+    pend.count = torch.empty(1 + nb, dtype=torch.int64, device=dev)   # cluster count, then the pooled scene ends
+    pend.with_offset = offset is not None
     off = None if offset is None else offset.to(torch.int64).contiguous()
     nbytes = lib.ptv3_pool_clusters_workspace_bytes(n)
     ws = _ws(nbytes, dev)
     _lib.check(lib.ptv3_pool_clusters(_ptr(code0.contiguous()), _ptr(order0), n, int(shift), _ptr(off), nb,
-                                      _ptr(cluster), _ptr(idx_ptr), _ptr(head), _ptr(count), _ptr(ws),
+                                      _ptr(pend.cluster), _ptr(pend.idx_ptr), _ptr(pend.head), _ptr(pend.count), _ptr(ws),
                                       nbytes, _stream()), "ptv3_pool_clusters")
-    host = count.tolist()
+    pend.read = Readback(pend.count)
+    return pend
+
+
+def pool_clusters_finish(pend):
+    host = pend.read.get()
     m = int(host[0])
-    if offset is None:
-        return cluster, idx_ptr[: m + 1], head[:m], m
-    return cluster, idx_ptr[: m + 1], head[:m], m, count[1:], [int(v) for v in host[1:]]
+    if not pend.with_offset:
+        return pend.cluster, pend.idx_ptr[: m + 1], pend.head[:m], m
+    return pend.cluster, pend.idx_ptr[: m + 1], pend.head[:m], m, pend.count[1:], [int(v) for v in host[1:]]
+
+
+def pool_clusters(code0, order0, shift, offset=None):
+    """Clusters of code0 >> shift in sorted order. One read-back (the cluster count).
+
+    Returns cluster (N,), idx_ptr (M+1,), head (M,), M; with `offset` (the parent's cumulative
+    scene ends, on the device) also the pooled scene ends as a device tensor and as a Python
+    list, read in the same device->host copy as the count. Scenes are runs of the sorted order
+    (the scene id is the top of every code), so scene b ends with the cluster of its last point."""
+    return pool_clusters_finish(pool_clusters_start(code0, order0, shift, offset))
 
 
 def _row_perm(rows, k):

@@ -8,6 +8,8 @@ batched radix sort, and the host learns the three things it needs (grid extent, 
 and sparse shape, and scene sizes) from a single device->host copy that is cached on the
 Point.
 """
+import math
+
 import torch
 
 from . import ops
@@ -80,7 +82,14 @@ class Point(AttrDict):
         if want_grid:
             self._ensure_grid_coord()
             parts.append(ops.grid_max(self["grid_coord"]).long())
-        host = [int(v) for v in (torch.cat(parts) if len(parts) > 1 else parts[0]).tolist()]
+        both = torch.cat(parts) if len(parts) > 1 else parts[0]
+        if both.is_cuda:
+            read = ops.Readback(both)
+            for ks in self.pop("_plan_ahead", ()):   # queued behind the read-back, runs while the host waits
+                self.start_plan(ks)
+            host = [int(v) for v in read.get()]
+        else:
+            host = [int(v) for v in both.tolist()]
         if want_offset:
             nb = self["offset"].shape[0]
             self["_offset_host"], host = host[:nb], host[nb:]
@@ -135,6 +144,42 @@ class Point(AttrDict):
         self["serialized_order"] = sort_order
         self["serialized_inverse"] = inverse
 
+    # ---- pair lists of the convolutions, started ahead of their first use ------------------
+    def _sparse_indices_tensor(self):
+        indices = self.get("_sparse_indices")
+        if indices is None:
+            indices = torch.cat([self["batch"].unsqueeze(-1).int(), self["grid_coord"].int()], dim=1).contiguous()
+            self["_sparse_indices"] = indices
+        return indices
+
+    def plan_ahead(self, kernel_sizes):
+        """Ask for the pair lists of these kernel sizes to be started at the next host read-back (or now
+        if the host facts are cached already): they depend on the coordinates only."""
+        if "_offset_host" in self and "_grid_max_host" in self:
+            for ks in kernel_sizes:
+                self.start_plan(ks)
+        else:
+            self["_plan_ahead"] = tuple(kernel_sizes)
+
+    def start_plan(self, ks):
+        if not self["feat"].is_cuda:
+            return
+        self._ensure_grid_coord()
+        pending = self.setdefault("_pending_plans", {})
+        if ks not in pending:
+            pending[ks] = ops.conv_plan_direct_start(self._sparse_indices_tensor(), ks)
+
+    def pool_ahead(self, stride):
+        """Queue the cluster kernels of the grid pooling with this stride now (model.py:652-664 reads
+        nothing but the serialized codes): when the pooling module runs, the cluster count is on the host."""
+        if "serialized_code" not in self or not self["serialized_code"].is_cuda:
+            return
+        depth = (math.ceil(stride) - 1).bit_length()
+        if depth > self["serialized_depth"]:
+            depth = 0
+        self["_pending_pool"] = (3 * depth, ops.pool_clusters_start(self["serialized_code"][0], self["serialized_order"][0],
+                                                                     3 * depth, self["offset"]))
+
     # ---- sparsify --------------------------------------------------------------------
     def sparsify(self, pad=96):
         """Attach the sparse-conv view of the features (model.py:138-174)."""
@@ -146,10 +191,10 @@ class Point(AttrDict):
             sparse_shape = self["sparse_shape"]
         else:
             sparse_shape = [v + pad for v in self.grid_max_host()]
-        indices = self.get("_sparse_indices")
-        if indices is None:
-            indices = torch.cat([self["batch"].unsqueeze(-1).int(), self["grid_coord"].int()], dim=1).contiguous()
+        indices = self._sparse_indices_tensor()
         self["sparse_shape"] = sparse_shape
-        self["sparse_conv_feat"] = SparseConvTensor(
-            features=self["feat"], indices=indices, spatial_shape=sparse_shape,
-            batch_size=len(self.offset_host()))
+        sct = SparseConvTensor(features=self["feat"], indices=indices, spatial_shape=sparse_shape,
+                               batch_size=len(self.offset_host()))
+        for ks, pend in self.pop("_pending_plans", {}).items():
+            sct.indice_dict[("pending", ks)] = pend
+        self["sparse_conv_feat"] = sct

@@ -43,6 +43,8 @@ class SparseConvTensor:
             return self.indice_dict[key]
         if indice_key is not None and (indice_key, kernel_size) in self.indice_dict:
             plan = ops.conv_plan(self.indice_dict[(indice_key, kernel_size)], tap_major=True)
+        elif ("pending", kernel_size) in self.indice_dict:
+            plan = ops.conv_plan_direct_finish(self.indice_dict.pop(("pending", kernel_size)))
         else:
             plan = ops.conv_plan_direct(self.indices, kernel_size)
         if key is not None:
