@@ -177,3 +177,62 @@ def test_forward_fp32_with_relative_position_bias():
     _draw_perms(9, False)
     point = _run(model.to(DEV), d, feat, torch.float32)
     assert rel_err(point.feat, want) < 1e-4
+
+
+def test_forward_cls_mode_encoder_only_fp16():
+    """cls_mode (model.py:817, :976-981) stops after the encoder: the pooled points of the last stage."""
+    from pointtransformerv3_amd import PointTransformerV3
+    torch.manual_seed(4)
+    model = PointTransformerV3(cls_mode=True, shuffle_orders=False).eval().half()
+    d, feat = _data(9000, 2, grid=0.03)
+    f16 = feat.astype(np.float16).astype(np.float32)
+    perms = _draw_perms(21, False)
+    sd = {k: v.float() for k, v in model.state_dict().items()}
+    point = _run(model.to(DEV), d, f16, torch.float16)
+    want = ptv3_forward(sd, d["grid_coord"], f16, d["offset"], perms=perms, cls_mode=True)
+    assert point.feat.shape == want.shape and point.feat.shape[1] == 512
+    assert rel_err(point.feat, want) < 2e-2
+    assert "pooling_parent" in point   # the decoder never ran
+
+
+def test_forward_pdnorm_picks_the_conditions_norms():
+    """PDNorm (model.py:255-294) with decoupled norms is the plain model carrying that condition's norm
+    parameters: same forward, bit for bit, through whichever kernels each of them takes."""
+    from pointtransformerv3_amd import PointTransformerV3
+    kw = dict(enc_depths=(1, 1, 1, 1, 1), dec_depths=(1, 1, 1, 1), shuffle_orders=False)
+    torch.manual_seed(5)
+    pd = PointTransformerV3(pdnorm_bn=True, pdnorm_ln=True, **kw).eval()
+    for name, buf in pd.named_buffers():   # distinct statistics per condition
+        if name.endswith("running_mean"):
+            buf.normal_(0, 0.2)
+        elif name.endswith("running_var"):
+            buf.uniform_(0.6, 1.6)
+    plain = PointTransformerV3(**kw).eval()
+    cond = "S3DIS"
+    idx = pd.embedding.stem.norm.conditions.index(cond) if hasattr(pd.embedding.stem, "norm") else 1
+    pd_sd = pd.state_dict()
+    sd = {}
+    for key in plain.state_dict():
+        if key in pd_sd:
+            sd[key] = pd_sd[key]
+            continue
+        head, leaf = key.rsplit(".", 1)
+        cand = f"{head}.norm.{idx}.{leaf}"
+        assert cand in pd_sd, (key, cand)
+        sd[key] = pd_sd[cand]
+    plain.load_state_dict(sd)
+    d, feat = _data(5000, 2, grid=0.04)
+    f16 = feat.astype(np.float16).astype(np.float32)
+
+    def run(model, extra):
+        data = dict(feat=torch.from_numpy(f16).to(DEV, torch.float16), grid_coord=torch.from_numpy(d["grid_coord"]).to(DEV),
+                    coord=torch.from_numpy(d["coord"]).to(DEV), offset=torch.from_numpy(d["offset"]).to(DEV), **extra)
+        with torch.inference_mode():
+            return model(data).feat
+    got = run(pd.half().to(DEV), dict(condition=cond))
+    want = run(plain.half().to(DEV), {})
+    assert torch.isfinite(got.float()).all()
+    # PDNorm modules run in torch, the plain model's norms in the fused kernels: same math, other rounding points
+    assert rel_err(got, want.float().cpu()) < 2e-2
+    other = run(pd, dict(condition="ScanNet"))
+    assert rel_err(other, want.float().cpu()) > 1e-3   # another condition's statistics do change the result
