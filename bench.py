@@ -245,6 +245,16 @@ def kernel_rooflines(path):
         add(name, f"{nl} voxels (4 scenes at 8 cm), {plan2.n_pairs} pairs ({plan2.n_pairs / nl:.2f}/voxel), 128->128", "mfma",
             2.0 * plan2.n_pairs * 128 * 128, us, "FLOP (2 * P_act * Cin * Cout)")
     del plan2, feat2, w2, packed2, lvl
+    # ---- voxelisation in front of the model: the 4 rooms' raw points (before the one-point-per-voxel cut)
+    raw = [synthetic.room_points(106_000, 4000 + i).astype(np.float32) for i in range(4)]
+    raw_coord = torch.from_numpy(np.concatenate(raw)).to(dev)
+    raw_off = torch.from_numpy(np.cumsum([len(r) for r in raw])).to(dev)
+    us = _time_us(lambda: ops.voxelize(raw_coord, raw_off, 0.02), iters=10)
+    kept = len(ops.voxelize(raw_coord, raw_off, 0.02)["index"])
+    nr = len(raw_coord)
+    add("voxelize", f"{nr} points (4 rooms) -> {kept} voxels at 2 cm", "hbm", 20.0 * nr + 20.0 * kept, us,
+        "B (12 B coordinates read + 8 B inverse written per point, 20 B grid_coord + index per voxel)")
+    del raw, raw_coord
     # ---- pooling on the 4-scene batch
     code = ops.encode_orders(g, b, 9, orders)
     order, inverse = ops.argsort_rows(code, 29)

@@ -51,6 +51,21 @@ int ptv3_encode(const int32_t *grid_coord, const int64_t *batch, int64_t n, int 
  * per-axis maximum of grid_coord (n,3) int32 into out3 (3 int32, device). n >= 1. */
 int ptv3_grid_max(const int32_t *grid_coord, int64_t n, int32_t *out3, void *stream);
 
+/* Voxelisation in front of the model (what Pointcept's data pipeline does on the host before
+ * PointTransformerV3.forward, model.py:966-973, sees a batch; model.py:88-96 is the model's own
+ * fallback for grid_coord alone): per scene, grid_coord = floor((coord - scene minimum) / grid_size),
+ * and the first point in input order of every voxel is kept. coord (n,3) float32, offset (n_scenes,)
+ * int64 cumulative scene ends, all on the device. Outputs, sized for n by the caller: grid_coord
+ * (m,3) int32 and index (m,) int64 of the kept points in input order, inverse (n,) int64 = position
+ * of every input point's voxel among the kept ones (or NULL), offset_out (n_scenes,) int64 = scene
+ * ends of the kept points, counts (2,) int64 on the device = {m, status}; status 1 means a grid
+ * coordinate needs more than 16 bits (the serialization's limit, model.py:108) and the rest is
+ * meaningless. n < 2^30. */
+size_t ptv3_voxelize_workspace_bytes(int64_t n, int n_scenes);
+int ptv3_voxelize(const float *coord, int64_t n, const int64_t *offset, int n_scenes, float grid_size,
+                  int32_t *grid_coord, int64_t *index, int64_t *inverse, int64_t *offset_out,
+                  int64_t *counts, void *workspace, size_t workspace_bytes, void *stream);
+
 /* model.py:35-40 (offset2batch): scene id of each of the n points from the cumulative scene ends
  * offset (n_scenes,) int64 on the device, n = offset[n_scenes - 1] known to the caller. */
 int ptv3_offset2batch(const int64_t *offset, int n_scenes, int64_t n, int64_t *batch, void *stream);

@@ -132,3 +132,35 @@ def subm_kmap_bruteforce(indices, ks=3):
         for k, (dx, dy, dz) in enumerate(off):
             nbr[i, k] = table.get((b, x + dx, y + dy, z + dz), -1)
     return nbr
+
+
+def voxelize(coord, offset, grid_size):
+    """Voxelisation in front of the model: per scene grid_coord = floor((p - scene min) / grid_size)
+    in float32, the first point (input order) of every voxel kept.
+
+    The reference checkout has no file for this step (it is Pointcept's GridSample + collate, outside
+    the checkout; model.py:88-96 is only the fallback that derives grid_coord): parity with it is
+    unpinned. What is pinned is this function against a dictionary brute force and against the
+    generator of the benchmark scenes (tests/test_oracle_indexing.py).
+    Returns grid_coord (M,3) int32, index (M,) kept input rows ascending, inverse (N,) voxel of every
+    point, ends (B,) cumulative kept counts."""
+    coord = np.asarray(coord, np.float32)
+    grids, index, inverse, ends = [], [], np.empty(len(coord), np.int64), []
+    start, kept = 0, 0
+    for end in offset:
+        p = coord[start:end]
+        if len(p):
+            g = np.floor((p - p.min(0)) / np.float32(grid_size)).astype(np.int64)
+            key = (g[:, 0] << 42) | (g[:, 1] << 21) | g[:, 2]
+            _, first, inv = np.unique(key, return_index=True, return_inverse=True)
+            rank = np.argsort(np.argsort(first))          # voxels numbered by their first point
+            order = np.sort(first)
+            grids.append(g[order].astype(np.int32))
+            index.append(order + start)
+            inverse[start:end] = rank[inv] + kept
+            kept += len(order)
+        ends.append(kept)
+        start = end
+    g_all = np.concatenate(grids) if grids else np.zeros((0, 3), np.int32)
+    i_all = np.concatenate(index) if index else np.zeros(0, np.int64)
+    return g_all, i_all, inverse, np.array(ends, np.int64)

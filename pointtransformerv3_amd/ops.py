@@ -100,6 +100,36 @@ def grid_max(grid_coord):
     return out
 
 
+def voxelize(coord, offset, grid_size, with_inverse=True):
+    """Per scene grid_coord = floor((coord - scene minimum) / grid_size), first point of every voxel kept.
+
+    coord (N,3) float32 and offset (B,) cumulative scene ends on the device. Returns a dict:
+    grid_coord (M,3) int32 and index (M,) int64 of the kept points in input order, offset (B,) int64
+    scene ends of the kept points, inverse (N,) int64 voxel of every input point. One read-back (M)."""
+    _dev(coord, offset)
+    lib = _lib.load()
+    coord = coord.to(torch.float32).contiguous()
+    off = offset.to(torch.int64).contiguous()
+    n, nb = coord.shape[0], off.shape[0]
+    dev = coord.device
+    grid = torch.empty((n, 3), dtype=torch.int32, device=dev)
+    index = torch.empty(n, dtype=torch.int64, device=dev)
+    inverse = torch.empty(n, dtype=torch.int64, device=dev) if with_inverse else None
+    off_out = torch.empty(nb, dtype=torch.int64, device=dev)
+    counts = torch.empty(2, dtype=torch.int64, device=dev)
+    nbytes = lib.ptv3_voxelize_workspace_bytes(n, nb)
+    ws = _ws(nbytes, dev)
+    _lib.check(lib.ptv3_voxelize(_ptr(coord), n, _ptr(off), nb, float(grid_size), _ptr(grid), _ptr(index), _ptr(inverse),
+                                 _ptr(off_out), _ptr(counts), _ptr(ws), nbytes, _stream()), "ptv3_voxelize")
+    m, status = Readback(counts).get()
+    if status:
+        raise RuntimeError("voxelize: a grid coordinate does not fit 16 bits (grid_size too small for the scene extent)")
+    out = dict(grid_coord=grid[:m], index=index[:m], offset=off_out)
+    if with_inverse:
+        out["inverse"] = inverse
+    return out
+
+
 def offset2batch(offset, n):
     """Scene id (int64) of each of n points from the cumulative scene ends on the device."""
     _dev(offset)

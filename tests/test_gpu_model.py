@@ -236,3 +236,30 @@ def test_forward_pdnorm_picks_the_conditions_norms():
     assert rel_err(got, want.float().cpu()) < 2e-2
     other = run(pd, dict(condition="ScanNet"))
     assert rel_err(other, want.float().cpu()) > 1e-3   # another condition's statistics do change the result
+
+
+def test_raw_points_through_grid_sample_and_forward():
+    """Raw, unvoxelised scenes -> device voxelisation -> forward: the same output as handing the model
+    the host-voxelised batch (the scene generator keeps the same first points)."""
+    from pointtransformerv3_amd import PointTransformerV3, synthetic, voxelize
+    grid = 0.04
+    raw = [synthetic.room_points(15_000, 50 + i).astype(np.float32) for i in range(2)]
+    coord = torch.from_numpy(np.concatenate(raw)).to(DEV)
+    offset = torch.from_numpy(np.cumsum([len(r) for r in raw])).to(DEV)
+    rng = np.random.default_rng(8)
+    feat = torch.from_numpy(rng.random((len(coord), 6)).astype(np.float32)).to(DEV).half()
+    batch = voxelize.grid_sample(coord, offset, grid, feat=feat)
+    # host path: voxelize every scene with numpy, concatenate
+    parts = [synthetic.voxelize_unique(r, np.float32(grid)) for r in raw]
+    g_host = np.concatenate([p[0] for p in parts])
+    starts = np.concatenate([[0], np.cumsum([len(r) for r in raw])[:-1]])
+    keep = np.concatenate([p[1] + s for p, s in zip(parts, starts)])
+    assert np.array_equal(batch["grid_coord"].cpu().numpy(), g_host) and np.array_equal(batch["index"].cpu().numpy(), keep)
+    torch.manual_seed(6)
+    model = PointTransformerV3(enc_depths=(1, 1, 1, 1, 1), dec_depths=(1, 1, 1, 1), shuffle_orders=False).eval().half().to(DEV)
+    host = dict(feat=feat[torch.from_numpy(keep).to(DEV)], grid_coord=torch.from_numpy(g_host).to(DEV),
+                coord=coord[torch.from_numpy(keep).to(DEV)], offset=torch.from_numpy(np.cumsum([len(p[1]) for p in parts])).to(DEV))
+    with torch.inference_mode():
+        torch.manual_seed(9); a = model({k: batch[k] for k in ("feat", "grid_coord", "coord", "offset")}).feat
+        torch.manual_seed(9); b = model(host).feat
+    assert a.shape[0] == len(keep) and torch.equal(a, b)

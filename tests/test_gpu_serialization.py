@@ -125,3 +125,33 @@ def test_grid_max():
     dev = to_dev(g)
     for skip in (1, 2, 3, 5000, 5002):
         assert ops().grid_max(dev[skip:]).tolist() == g[skip:].max(0).tolist()
+
+
+@pytest.mark.parametrize("sizes,grid", [([5000], 0.05), ([30_000, 1, 0, 12_345], 0.02), ([0, 700, 0], 0.1),
+                                        ([200_000, 150_000], 0.02)])
+def test_voxelize_matches_numpy(sizes, grid):
+    from pointtransformerv3_amd import ops, voxelize
+    rng = np.random.default_rng(sum(sizes))
+    # points on a few planes plus noise, shifted per scene; duplicates of voxels are common
+    coord = np.concatenate([np.concatenate([rng.random((n, 2)) * 6, rng.integers(0, 3, (n, 1)) + rng.normal(0, 0.004, (n, 1))], 1)
+                            + rng.normal(0, 50, 3) for n in sizes]).astype(np.float32)
+    offset = np.cumsum(sizes).astype(np.int64)
+    wg, wi, winv, wends = OI.voxelize(coord, offset, grid)
+    got = ops.voxelize(torch.from_numpy(coord).to(DEV), torch.from_numpy(offset).to(DEV), grid)
+    assert np.array_equal(got["grid_coord"].cpu().numpy(), wg)
+    assert np.array_equal(got["index"].cpu().numpy(), wi)
+    assert np.array_equal(got["inverse"].cpu().numpy(), winv)
+    assert np.array_equal(got["offset"].cpu().numpy(), wends)
+    assert len(wi) < len(coord) or min(s for s in sizes if s) == 1   # the cases do merge points
+    # the batch dictionary it makes runs through the model's own serialization
+    feat = torch.from_numpy(rng.random((len(coord), 4)).astype(np.float32)).to(DEV)
+    batch = voxelize.grid_sample(torch.from_numpy(coord).to(DEV), torch.from_numpy(offset).to(DEV), grid, feat=feat)
+    assert batch["feat"].shape == (len(wi), 4) and torch.equal(batch["feat"], feat[batch["index"]])
+    assert torch.equal(batch["coord"], torch.from_numpy(coord).to(DEV)[batch["index"]])
+
+
+def test_voxelize_rejects_extents_beyond_16_bits():
+    from pointtransformerv3_amd import ops
+    coord = torch.tensor([[0.0, 0.0, 0.0], [700.0, 0.0, 0.0]], device=DEV)
+    with pytest.raises(RuntimeError, match="16 bits"):
+        ops.voxelize(coord, torch.tensor([2], device=DEV), 0.01)

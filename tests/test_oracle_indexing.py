@@ -208,3 +208,33 @@ def test_rpe_bias_and_attention_with_bias():
     q, k, v = qkv.reshape(L, 3, H, 16).permute(1, 2, 0, 3)
     want = F.scaled_dot_product_attention(q[None], k[None], v[None], attn_mask=bias[None])[0]
     assert torch.allclose(got, want.transpose(0, 1).reshape(L, H * 16), atol=1e-5)
+
+
+def test_voxelize_against_dictionary_and_scene_generator():
+    from pointtransformerv3_amd import synthetic
+    rng = np.random.default_rng(31)
+    sizes = [400, 0, 1, 900]
+    coord = np.concatenate([rng.random((n, 3)) * 2 + rng.normal(0, 20, 3) for n in sizes]).astype(np.float32)
+    offset = np.cumsum(sizes)
+    grid = 0.25
+    g, index, inverse, ends = OI.voxelize(coord, offset, grid)
+    # brute force: walk the points, remember the first of every (scene, cell)
+    seen, want_g, want_i, want_inv, want_ends, start = {}, [], [], [], [], 0
+    for s, end in enumerate(offset):
+        lo = coord[start:end].min(0) if end > start else None
+        for i in range(start, end):
+            cell = tuple(np.floor((coord[i] - lo) / np.float32(grid)).astype(np.int64))
+            if (s, cell) not in seen:
+                seen[(s, cell)] = len(want_i)
+                want_g.append(cell); want_i.append(i)
+            want_inv.append(seen[(s, cell)])
+        want_ends.append(len(want_i))
+        start = end
+    assert np.array_equal(g, np.array(want_g)) and np.array_equal(index, want_i)
+    assert np.array_equal(inverse, want_inv) and np.array_equal(ends, want_ends)
+    assert len(index) < len(coord)
+    # one scene: the generator of the benchmark scenes does the same (in the precision of its points)
+    pts = synthetic.room_points(5000, 3).astype(np.float32)
+    g1, keep = synthetic.voxelize_unique(pts, np.float32(0.05))
+    g2, i2, _, _ = OI.voxelize(pts, [len(pts)], 0.05)
+    assert np.array_equal(g1, g2) and np.array_equal(keep, i2)
