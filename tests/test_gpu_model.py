@@ -263,3 +263,18 @@ def test_raw_points_through_grid_sample_and_forward():
         torch.manual_seed(9); a = model({k: batch[k] for k in ("feat", "grid_coord", "coord", "offset")}).feat
         torch.manual_seed(9); b = model(host).feat
     assert a.shape[0] == len(keep) and torch.equal(a, b)
+
+
+def test_forward_bf16_default_model():
+    """The whole forward in bf16 (8 mantissa bits per stored activation) stays inside the same bound."""
+    from pointtransformerv3_amd import PointTransformerV3
+    torch.manual_seed(1)
+    model = PointTransformerV3(shuffle_orders=False).eval().to(torch.bfloat16)
+    d, feat = _data(20000, 2, grid=0.02)
+    f = torch.from_numpy(feat).to(torch.bfloat16).float().numpy()
+    perms = _draw_perms(77, False)
+    sd = {k: v.float() for k, v in model.state_dict().items()}
+    point = _run(model.to(DEV), d, f, torch.bfloat16)
+    want = ptv3_forward(sd, d["grid_coord"], f, d["offset"], perms=perms)
+    assert point.feat.dtype == torch.bfloat16
+    assert rel_err(point.feat, want) < 2e-2
