@@ -274,6 +274,16 @@ int ptv3_linear_fwd(const void *x, const void *w, const void *bias, int dtype, i
 int ptv3_linear_bn_act_fwd(const void *x, const void *w, const void *bias, const void *running_mean,
                            const void *running_var, int stats_f32, const void *gamma, const void *beta,
                            float eps, int dtype, int64_t n, int k, int nout, int gelu, void *out, void *stream);
+/* Square Linear (channels in and out, 128 or 256; fp16/bf16) fused with the LayerNorms and residual
+ * additions that follow it in a block, semantics and rounding points of ptv3_layer_norm's modes with
+ * x replaced by Linear(x):
+ *   mode 2 (proj, model.py:487,594-597): s = res + Linear(x); out0 = s (+ shift); out1 = LN(s)
+ *   mode 3 (cpe.1 + cpe.2, model.py:541-545,587-593): s = res + LN(Linear(x)); out0 = s; out1 = LN2(s)
+ * w (channels, channels) as nn.Linear stores it, bias / shift (channels,) or NULL, gamma2 / beta2
+ * for mode 3 only. */
+int ptv3_linear_ln_fwd(const void *x, const void *w, const void *bias, const void *res, const void *gamma,
+                       const void *beta, const void *gamma2, const void *beta2, const void *shift, int dtype,
+                       int64_t n, int channels, int mode, float eps, void *out0, void *out1, void *stream);
 
 /* MLP of a block plus its residual, model.py:510-516 and :602, in one kernel:
  * out = resid + fc2(GELU(fc1(x))), exact (erf) GELU, intermediates rounded to dtype where the

@@ -336,17 +336,27 @@ class Block(PointModule):
             point.feat = feat
             point.sparse_conv_feat = point.sparse_conv_feat.replace_feature(feat)
             return point
-        branch = ops.linear(conv, self.cpe[1]) if type(self.cpe[1]) is nn.Linear else self.cpe[1](conv)
-        # feat = shortcut + LN(branch) and its pre-norm for attention, in one pass
-        feat, normed = ops.layer_norm(branch, ln_cpe.weight, ln_cpe.bias, ln_cpe.eps, residual=point.feat,
-                                      mode=3, weight2=ln1.weight, bias2=ln1.bias)
-        point.feat = normed
-        point = self.attn(point)
+        same_eps = ln_cpe.eps == ln1.eps
+        if ops.linear_ln_ok(conv, self.cpe[1]) and same_eps:
+            # cpe Linear, its LayerNorm, the residual and the attention's pre-norm in one kernel
+            feat, normed = ops.linear_ln(conv, self.cpe[1], point.feat, ln_cpe, 3, ln2=ln1)
+        else:
+            branch = ops.linear(conv, self.cpe[1]) if type(self.cpe[1]) is nn.Linear else self.cpe[1](conv)
+            # feat = shortcut + LN(branch) and its pre-norm for attention, in one pass
+            feat, normed = ops.layer_norm(branch, ln_cpe.weight, ln_cpe.bias, ln_cpe.eps, residual=point.feat,
+                                          mode=3, weight2=ln1.weight, bias2=ln1.bias)
         # feat += attention branch, plus the pre-norm for the MLP.
         # When fc2 runs as a separate GEMM it accumulates onto the stored sum (beta = 1), so its
         # bias is added to that sum here: feat + fc2(h) + b2 without a separate add pass
-        feat, normed = ops.layer_norm(point.feat, ln2.weight, ln2.bias, ln2.eps, residual=feat, mode=2,
-                                      shift=mlp.fc2.bias if (plain_mlp and not fused_mlp) else None)
+        shift = mlp.fc2.bias if (plain_mlp and not fused_mlp) else None
+        point.feat = normed
+        attn_out = self.attn.attend(point, ops.linear(normed, self.attn.qkv))
+        if ops.linear_ln_ok(attn_out, self.attn.proj) and not (self.training and self.attn.proj_drop.p > 0):
+            # proj, the residual and the MLP's pre-norm in one kernel
+            feat, normed = ops.linear_ln(attn_out, self.attn.proj, feat, ln2, 2, shift=shift)
+        else:
+            branch = self.attn.proj_drop(ops.linear(attn_out, self.attn.proj))
+            feat, normed = ops.layer_norm(branch, ln2.weight, ln2.bias, ln2.eps, residual=feat, mode=2, shift=shift)
         if fused_mlp:
             # fc1 + GELU + fc2 + residual in one kernel, the 4C-wide hidden tensor never leaves the CU
             feat = ops.mlp_fused(normed, feat, mlp.fc1.weight, mlp.fc1.bias, mlp.fc2.weight, mlp.fc2.bias)

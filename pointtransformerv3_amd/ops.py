@@ -610,6 +610,38 @@ def layer_norm(x, weight, bias, eps=1e-5, residual=None, mode=0, weight2=None, b
     return out0 if mode < 2 else (out0, out1)
 
 
+LINEAR_LN_CHANNELS = (128, 256)   # square Linear + LayerNorm(s) + residual in one kernel
+# where that kernel measured faster than Linear kernel + LayerNorm kernel on MI355X: at 128 channels
+# (146k rows: 35 us against 42-49); at 256 the C x C weights fill the LDS, four waves per CU remain
+# and the two kernels win (38k rows: 44-67 us against 33-35)
+LINEAR_LN_PAYS = (128,)
+
+
+def linear_ln_ok(x, lin):
+    return (x.is_cuda and x.dtype in (torch.float16, torch.bfloat16) and x.dim() == 2 and type(lin) is torch.nn.Linear
+            and lin.in_features == lin.out_features and lin.in_features in LINEAR_LN_PAYS)
+
+
+def linear_ln(x, lin, residual, ln, mode, ln2=None, shift=None):
+    """layer_norm(lin(x), ..., residual=residual, mode=mode, ...) for a square nn.Linear in one kernel
+    (modes 2 and 3 of layer_norm; same rounding points). Returns (out0, out1)."""
+    _dev(x, lin.weight, residual, ln.weight)
+    lib = _lib.load()
+    x = x.contiguous()
+    n, c = x.shape
+    dt = x.dtype
+    cast = lambda t: None if t is None else t.to(dt).contiguous()
+    w, b, res = cast(lin.weight), cast(lin.bias), cast(residual)
+    g1, b1 = cast(ln.weight), cast(ln.bias)
+    g2, b2 = (cast(ln2.weight), cast(ln2.bias)) if ln2 is not None else (None, None)
+    sh = cast(shift)
+    out0, out1 = torch.empty_like(x), torch.empty_like(x)
+    _lib.check(lib.ptv3_linear_ln_fwd(_ptr(x), _ptr(w), _ptr(b), _ptr(res), _ptr(g1), _ptr(b1), _ptr(g2), _ptr(b2), _ptr(sh),
+                                      _dtype_code(x), n, c, int(mode), float(ln.eps), _ptr(out0), _ptr(out1), _stream()),
+               "ptv3_linear_ln_fwd")
+    return out0, out1
+
+
 LINEAR_ROWS_IN = (32, 64, 128, 256, 512)   # input widths of the tall-and-skinny Linear kernel
 
 

@@ -531,3 +531,43 @@ def test_segment_reduce_bn_act_equals_the_separate_kernels(dtype, gelu):
     two = o.bn_act(o.segment_reduce(*args), bn_d.running_mean, bn_d.running_var, bn_d.weight, bn_d.bias, bn_d.eps, gelu)
     assert got.dtype == dtype and torch.equal(got, two)
     assert rel_err(got, want) < (1e-5 if dtype == torch.float32 else TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("c,n,mode", [(128, 5001, 3), (128, 77, 2), (256, 3000, 3), (256, 40_001, 2), (256, 1, 3), (128, 33, 3)])
+def test_linear_ln_parity(dtype, c, n, mode):
+    """Square Linear + LayerNorm(s) + residual in one kernel (model.py:541-545,587-597) against torch in
+    fp32 and against the two kernels it replaces (same rounding points, other summation order)."""
+    import torch.nn.functional as F
+    torch.manual_seed(c + n + mode)
+    lin = torch.nn.Linear(c, c).to(dtype)
+    ln1, ln2 = torch.nn.LayerNorm(c), torch.nn.LayerNorm(c)
+    for ln in (ln1, ln2):
+        ln.weight.data.uniform_(0.5, 1.5)
+        ln.bias.data.normal_(0, 0.3)
+    ln1, ln2 = ln1.to(dtype), ln2.to(dtype)
+    x = torch.randn(n, c).to(dtype)
+    res = torch.randn(n, c).to(dtype)
+    shift = (torch.randn(c) * 0.2).to(dtype)
+    o = ops()
+    with torch.no_grad():
+        y = F.linear(x.float(), lin.weight.float(), lin.bias.float())
+        if mode == 3:
+            s = res.float() + F.layer_norm(y, (c,), ln1.weight.float(), ln1.bias.float(), ln1.eps)
+            want0, want1 = s, F.layer_norm(s, (c,), ln2.weight.float(), ln2.bias.float(), ln2.eps)
+        else:
+            s = res.float() + y
+            want0, want1 = s + shift.float(), F.layer_norm(s, (c,), ln1.weight.float(), ln1.bias.float(), ln1.eps)
+        lin_d, l1, l2 = lin.to(DEV), ln1.to(DEV), ln2.to(DEV)   # (moves the modules)
+        if mode == 3:
+            got0, got1 = o.linear_ln(x.to(DEV), lin_d, res.to(DEV), l1, 3, ln2=l2)
+            two0, two1 = o.layer_norm(o.linear_rows(x.to(DEV), lin_d.weight, lin_d.bias), l1.weight, l1.bias, l1.eps,
+                                      residual=res.to(DEV), mode=3, weight2=l2.weight, bias2=l2.bias)
+        else:
+            got0, got1 = o.linear_ln(x.to(DEV), lin_d, res.to(DEV), l1, 2, shift=shift.to(DEV))
+            two0, two1 = o.layer_norm(o.linear_rows(x.to(DEV), lin_d.weight, lin_d.bias), l1.weight, l1.bias, l1.eps,
+                                      residual=res.to(DEV), mode=2, shift=shift.to(DEV))
+    assert got0.dtype == dtype and got0.shape == (n, c) and got1.shape == (n, c)
+    assert rel_err(got0, want0) < TOL[dtype] and rel_err(got1, want1) < TOL[dtype]
+    ulp = 2e-3 if dtype == torch.float16 else 1.6e-2
+    assert rel_err(got0, two0.float().cpu()) < ulp and rel_err(got1, two1.float().cpu()) < ulp
