@@ -78,21 +78,44 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_count_kernel(
 
 // blockIdx.x < taps: exclusive scan of column t of blk_tap_cnt over the blocks, total to
 // tap_total[t]. blockIdx.x == taps: exclusive scan of blk_row_sum, grand total to *n_pairs.
-__global__ __launch_bounds__(PLAN_THREADS) void plan_scan_kernel(uint32_t* __restrict__ blk_tap_cnt,
+// A column is one sequential chain of block scans, so the work-group is as wide as it gets
+// (1024 threads: a 400k-voxel level is 7 steps instead of 25).
+constexpr int SCAN_THREADS = 1024;
+constexpr int SCAN_WAVES = SCAN_THREADS / PTV3_WAVE;
+
+__global__ __launch_bounds__(SCAN_THREADS) void plan_scan_kernel(uint32_t* __restrict__ blk_tap_cnt,
                                                                  uint32_t* __restrict__ blk_row_sum,
                                                                  int64_t blocks, int taps,
                                                                  uint32_t* __restrict__ tap_total,
                                                                  int64_t* __restrict__ n_pairs) {
+    __shared__ uint32_t wsum[SCAN_WAVES];
     const int col = blockIdx.x;
+    const int lane = threadIdx.x % PTV3_WAVE, wave = threadIdx.x / PTV3_WAVE;
     uint32_t carry = 0;
-    for (int64_t b0 = 0; b0 < blocks; b0 += PLAN_THREADS) {
+    for (int64_t b0 = 0; b0 < blocks; b0 += SCAN_THREADS) {
         const int64_t b = b0 + threadIdx.x;
         uint32_t* p = col < taps ? &blk_tap_cnt[b * taps + col] : &blk_row_sum[b];
         const uint32_t v = b < blocks ? *p : 0u;
-        uint32_t total;
-        const uint32_t inc = block_scan_incl(v, &total);
-        if (b < blocks) *p = carry + inc - v;
+        uint32_t x = v;
+#pragma unroll
+        for (int off = 1; off < PTV3_WAVE; off <<= 1) {
+            const uint32_t y = __shfl_up(x, off, PTV3_WAVE);
+            if (lane >= off) x += y;
+        }
+        if (lane == PTV3_WAVE - 1) wsum[wave] = x;
+        __syncthreads();
+        // the 16 wave totals: every wave scans them itself (lanes 0..15)
+        uint32_t ws = lane < SCAN_WAVES ? wsum[lane] : 0u;
+#pragma unroll
+        for (int off = 1; off < SCAN_WAVES; off <<= 1) {
+            const uint32_t y = __shfl_up(ws, off, PTV3_WAVE);
+            if (lane >= off) ws += y;
+        }
+        const uint32_t total = __shfl(ws, SCAN_WAVES - 1, PTV3_WAVE);
+        const uint32_t base = wave == 0 ? 0u : __shfl(ws, wave - 1, PTV3_WAVE);
+        if (b < blocks) *p = carry + base + x - v;
         carry += total;
+        __syncthreads();
     }
     if (threadIdx.x == 0) {
         if (col < taps) tap_total[col] = carry;
@@ -386,7 +409,7 @@ extern "C" int ptv3_conv_plan_count(const int32_t* nbr, int64_t n, int taps, int
     const int64_t blocks = ptv3_ceil_div(n, PLAN_THREADS);
     hipLaunchKernelGGL(plan_count_kernel, dim3((unsigned)blocks), dim3(PLAN_THREADS), 0, stream, nbr, n, taps,
                        tap_major != 0, w.row_cnt, w.blk_row_sum, w.blk_tap_cnt);
-    hipLaunchKernelGGL(plan_scan_kernel, dim3((unsigned)(taps + 1)), dim3(PLAN_THREADS), 0, stream,
+    hipLaunchKernelGGL(plan_scan_kernel, dim3((unsigned)(taps + 1)), dim3(SCAN_THREADS), 0, stream,
                        w.blk_tap_cnt, w.blk_row_sum, blocks, taps, w.tap_total, n_pairs);
     hipLaunchKernelGGL(plan_tap_ptr_kernel, dim3(1), dim3(PLAN_THREADS), 0, stream,
                        (const uint32_t*)w.tap_total, taps, tap_ptr);
@@ -430,7 +453,7 @@ extern "C" int ptv3_kmap_plan_count(const int32_t* indices, int64_t n, int ks, i
     else
         hipLaunchKernelGGL(direct_count_kernel<5>, dim3((unsigned)blocks), dim3(DIRECT_THREADS), 0, stream, indices, n,
                            h, notes, w.row_cnt, w.blk_row_sum, w.blk_tap_cnt);
-    hipLaunchKernelGGL(plan_scan_kernel, dim3((unsigned)(taps + 1)), dim3(PLAN_THREADS), 0, stream,
+    hipLaunchKernelGGL(plan_scan_kernel, dim3((unsigned)(taps + 1)), dim3(SCAN_THREADS), 0, stream,
                        w.blk_tap_cnt, w.blk_row_sum, blocks, taps, w.tap_total, n_pairs);
     hipLaunchKernelGGL(plan_tap_ptr_kernel, dim3(1), dim3(PLAN_THREADS), 0, stream,
                        (const uint32_t*)w.tap_total, taps, tap_ptr);
