@@ -229,13 +229,6 @@ int ptv3_pool_orders(const int64_t *order, const int64_t *cluster, int64_t n, in
  * src (n,c) of dtype, out (m,c) of dtype. */
 int ptv3_segment_reduce(const void *src, int dtype, int64_t n, int c, const int64_t *indices,
                         const int64_t *idx_ptr, int64_t m, int op, void *out, void *stream);
-/* The same followed by the inference-mode nn.BatchNorm1d and optional exact GELU that the pooling
- * applies to the reduced features (model.py:690-695): statistics float32 when stats_f32 (always for
- * float32 data) else of dtype, gamma / beta of dtype or NULL; every stage rounds to dtype. */
-int ptv3_segment_reduce_bn_act(const void *src, int dtype, int64_t n, int c, const int64_t *indices,
-                               const int64_t *idx_ptr, int64_t m, int op, const void *running_mean,
-                               const void *running_var, int stats_f32, const void *gamma, const void *beta,
-                               float eps, int gelu, void *out, void *stream);
 
 /* model.py:746: out[i] = parent[i] + child[cluster[i]]; parent,out (n,c), child (m,c). */
 int ptv3_unpool_add(const void *parent, const void *child, int dtype, int64_t n, int c,

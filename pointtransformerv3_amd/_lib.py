@@ -52,8 +52,6 @@ SIGNATURES = {
     "ptv3_pool_orders_workspace_bytes": (_sz, [_i64, _i32]),
     "ptv3_pool_orders": (_i32, [_vp, _vp, _i64, _i32, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "ptv3_segment_reduce": (_i32, [_vp, _i32, _i64, _i32, _vp, _vp, _i64, _i32, _vp, _vp]),
-    "ptv3_segment_reduce_bn_act": (_i32, [_vp, _i32, _i64, _i32, _vp, _vp, _i64, _i32, _vp, _vp, _i32, _vp, _vp, _f32,
-                                          _i32, _vp, _vp]),
     "ptv3_unpool_add": (_i32, [_vp, _vp, _i32, _i64, _i32, _vp, _i64, _vp, _vp]),
     "ptv3_bn_act": (_i32, [_vp, _vp, _vp, _i32, _vp, _vp, _i32, _i64, _i32, _f32, _i32, _vp, _vp]),
     "ptv3_linear_fwd": (_i32, [_vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp]),

@@ -209,36 +209,10 @@ template <typename T> __device__ __forceinline__ void st(T* p, float v) { *p = (
 // V consecutive channels per thread (V * sizeof(T) = 16 bytes when the channel count allows)
 template <typename T, int V> struct Pack { T v[V]; };
 
-// inference BatchNorm1d (+ exact GELU) applied to the reduced row before it is stored: the
-// norm and activation that follow the pooling's segment_csr (model.py:684-695)
-struct SegBn {
-    const void* mean;    // running statistics: float32 when stats_f32, else of the data type
-    const void* var;
-    const void* gamma;   // of the data type, or null
-    const void* beta;
-    float eps;
-    int stats_f32;
-    int gelu;
-};
-
-__device__ __forceinline__ float seg_gelu(float x) {
-    // 0.5 x (1 + erf(x / sqrt 2)); erf by Abramowitz-Stegun 7.1.26, |error| < 1.5e-7
-    const float z = fabsf(x) * 0.70710678118654752f;
-    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
-    float p = fmaf(1.061405429f, t, -1.453152027f);
-    p = fmaf(p, t, 1.421413741f);
-    p = fmaf(p, t, -0.284496736f);
-    p = fmaf(p, t, 0.254829592f);
-    const float e = __builtin_amdgcn_exp2f(-z * z * 1.4426950408889634f);
-    const float erf_abs = fmaf(-p * t, e, 1.0f);
-    const float half_x = 0.5f * x;
-    return fmaf(copysignf(erf_abs, x), half_x, half_x);
-}
-
-template <typename T, int V, bool BN>
+template <typename T, int V>
 __global__ __launch_bounds__(256) void segment_reduce_kernel(
     const T* __restrict__ src, int c, const int64_t* __restrict__ indices,
-    const int64_t* __restrict__ idx_ptr, int64_t m, int op, SegBn bn, T* __restrict__ out) {
+    const int64_t* __restrict__ idx_ptr, int64_t m, int op, T* __restrict__ out) {
     const int groups = c / V;
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= m * groups) return;
@@ -262,16 +236,6 @@ __global__ __launch_bounds__(256) void segment_reduce_kernel(
         float v = acc[k];
         if (op == 1 && t > b) v /= (float)(t - b);
         if (t == b) v = 0.f;
-        if (BN) {
-            // every stage rounds to the storage type, as the separate layers would
-            const int cc = ch + k;
-            const float mu = bn.stats_f32 ? ((const float*)bn.mean)[cc] : (float)((const T*)bn.mean)[cc];
-            const float va = bn.stats_f32 ? ((const float*)bn.var)[cc] : (float)((const T*)bn.var)[cc];
-            const float g = bn.gamma ? (float)((const T*)bn.gamma)[cc] : 1.f;
-            const float be = bn.beta ? (float)((const T*)bn.beta)[cc] : 0.f;
-            v = (float)(T)(((float)(T)v - mu) * rsqrtf(va + bn.eps) * g + be);
-            if (bn.gelu) v = seg_gelu(v);
-        }
         r.v[k] = (T)v;
     }
     *(Pack<T, V>*)(out + s * c + ch) = r;
@@ -295,25 +259,17 @@ __global__ __launch_bounds__(256) void unpool_add_kernel(const T* __restrict__ p
     *(Pack<T, V>*)(out + i * c + ch) = r;
 }
 
-template <typename T, bool BN>
-void launch_segment_reduce_v(const void* src, int c, const int64_t* indices, const int64_t* idx_ptr, int64_t m,
-                             int op, const SegBn& bn, void* out, hipStream_t stream) {
-    constexpr int V = 16 / sizeof(T);
-    if (c % V == 0) {
-        hipLaunchKernelGGL((segment_reduce_kernel<T, V, BN>), dim3((unsigned)ptv3_ceil_div(m * (c / V), 256)), dim3(256),
-                           0, stream, (const T*)src, c, indices, idx_ptr, m, op, bn, (T*)out);
-    } else {
-        hipLaunchKernelGGL((segment_reduce_kernel<T, 1, BN>), dim3((unsigned)ptv3_ceil_div(m * c, 256)), dim3(256), 0,
-                           stream, (const T*)src, c, indices, idx_ptr, m, op, bn, (T*)out);
-    }
-}
-
 template <typename T>
 void launch_segment_reduce(const void* src, int c, const int64_t* indices, const int64_t* idx_ptr, int64_t m,
-                           int op, const SegBn* bn, void* out, hipStream_t stream) {
-    const SegBn none = {nullptr, nullptr, nullptr, nullptr, 0.f, 0, 0};
-    if (bn) launch_segment_reduce_v<T, true>(src, c, indices, idx_ptr, m, op, *bn, out, stream);
-    else launch_segment_reduce_v<T, false>(src, c, indices, idx_ptr, m, op, none, out, stream);
+                           int op, void* out, hipStream_t stream) {
+    constexpr int V = 16 / sizeof(T);
+    if (c % V == 0) {
+        hipLaunchKernelGGL((segment_reduce_kernel<T, V>), dim3((unsigned)ptv3_ceil_div(m * (c / V), 256)), dim3(256), 0,
+                           stream, (const T*)src, c, indices, idx_ptr, m, op, (T*)out);
+    } else {
+        hipLaunchKernelGGL((segment_reduce_kernel<T, 1>), dim3((unsigned)ptv3_ceil_div(m * c, 256)), dim3(256), 0,
+                           stream, (const T*)src, c, indices, idx_ptr, m, op, (T*)out);
+    }
 }
 
 template <typename T>
@@ -383,25 +339,9 @@ extern "C" int ptv3_segment_reduce(const void* src, int dtype, int64_t n, int c,
     if (m == 0) return PTV3_OK;
     if (!src || !indices || !idx_ptr || !out) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
-    if (dtype == PTV3_F32) launch_segment_reduce<float>(src, c, indices, idx_ptr, m, op, nullptr, out, stream);
-    else if (dtype == PTV3_F16) launch_segment_reduce<_Float16>(src, c, indices, idx_ptr, m, op, nullptr, out, stream);
-    else launch_segment_reduce<__bf16>(src, c, indices, idx_ptr, m, op, nullptr, out, stream);
-    PTV3_RETURN_LAUNCH();
-}
-
-extern "C" int ptv3_segment_reduce_bn_act(const void* src, int dtype, int64_t n, int c, const int64_t* indices,
-                                          const int64_t* idx_ptr, int64_t m, int op, const void* running_mean,
-                                          const void* running_var, int stats_f32, const void* gamma,
-                                          const void* beta, float eps, int gelu, void* out, void* stream_) {
-    if (n < 0 || m < 0 || c < 1 || op < 0 || op > 3) return PTV3_EINVAL;
-    if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
-    if (m == 0) return PTV3_OK;
-    if (!src || !indices || !idx_ptr || !running_mean || !running_var || !out) return PTV3_EINVAL;
-    hipStream_t stream = (hipStream_t)stream_;
-    const SegBn bn = {running_mean, running_var, gamma, beta, eps, (dtype == PTV3_F32) ? 1 : stats_f32, gelu};
-    if (dtype == PTV3_F32) launch_segment_reduce<float>(src, c, indices, idx_ptr, m, op, &bn, out, stream);
-    else if (dtype == PTV3_F16) launch_segment_reduce<_Float16>(src, c, indices, idx_ptr, m, op, &bn, out, stream);
-    else launch_segment_reduce<__bf16>(src, c, indices, idx_ptr, m, op, &bn, out, stream);
+    if (dtype == PTV3_F32) launch_segment_reduce<float>(src, c, indices, idx_ptr, m, op, out, stream);
+    else if (dtype == PTV3_F16) launch_segment_reduce<_Float16>(src, c, indices, idx_ptr, m, op, out, stream);
+    else launch_segment_reduce<__bf16>(src, c, indices, idx_ptr, m, op, out, stream);
     PTV3_RETURN_LAUNCH();
 }
 

@@ -448,16 +448,8 @@ class SerializedPooling(PointModule):
         plans = {ks: ops.conv_plan_direct_start(indices4, ks) for ks in self.plan_kernel_sizes}
         order, inverse = ops.pool_orders(point.serialized_order, cluster, m, perm)
 
-        # the BatchNorm + GELU that follow (model.py:690-695) ride in the reduction's epilogue when they can
-        norm = self.norm[0] if self.norm is not None and len(self.norm) == 1 else None
-        act = self.act[0] if self.act is not None and len(self.act) == 1 else None
-        fuse_norm = norm is not None and _fusable_bn(norm, projected) and (act is None or _exact_gelu(act))
-        if fuse_norm:
-            pooled_feat = ops.segment_reduce_bn_act(projected, indices, idx_ptr, self.reduce, norm, act is not None)
-        else:
-            pooled_feat = ops.segment_reduce(projected, indices, idx_ptr, self.reduce)
         fields = AttrDict(
-            feat=pooled_feat,
+            feat=ops.segment_reduce(projected, indices, idx_ptr, self.reduce),
             grid_coord=grid_coord,
             serialized_code=code,
             serialized_order=order,
@@ -480,9 +472,9 @@ class SerializedPooling(PointModule):
         # max(x >> d) == max(x) >> d: the pooled grid extent needs no reduction and no sync
         fields["_grid_max_host"] = [v >> pooling_depth for v in point.grid_max_host()]
         pooled = Point(fields)
-        if fuse_norm:
-            pass
-        elif norm is not None and _fusable_bn(norm, pooled.feat) and _exact_gelu(act):
+        norm = self.norm[0] if self.norm is not None and len(self.norm) == 1 else None
+        act = self.act[0] if self.act is not None and len(self.act) == 1 else None
+        if norm is not None and _fusable_bn(norm, pooled.feat) and _exact_gelu(act):
             pooled.feat = ops.bn_act(pooled.feat, norm.running_mean, norm.running_var, norm.weight, norm.bias,
                                      norm.eps, True)
         else:

@@ -549,28 +549,6 @@ def segment_reduce(src, indices, idx_ptr, reduce="max"):
     return out
 
 
-def segment_reduce_bn_act(src, indices, idx_ptr, reduce, bn, gelu):
-    """gelu?(BatchNorm1d_inference(segment_reduce(src, ...))) in one kernel (bn: an nn.BatchNorm1d in eval mode)."""
-    _dev(src, indices, idx_ptr, bn.running_mean)
-    lib = _lib.load()
-    src = src.contiguous()
-    n, c = src.shape
-    dt = src.dtype
-    m = idx_ptr.shape[0] - 1
-    mean, var = bn.running_mean, bn.running_var
-    stats_f32 = mean.dtype == torch.float32
-    if not stats_f32 and mean.dtype != dt:
-        mean, var, stats_f32 = mean.float(), var.float(), True
-    g = None if bn.weight is None else bn.weight.to(dt).contiguous()
-    be = None if bn.bias is None else bn.bias.to(dt).contiguous()
-    out = torch.empty((m, c), dtype=dt, device=src.device)
-    _lib.check(lib.ptv3_segment_reduce_bn_act(_ptr(src), _dtype_code(src), n, c, _ptr(indices.contiguous()),
-                                              _ptr(idx_ptr.contiguous()), m, REDUCE_OPS[reduce], _ptr(mean.contiguous()),
-                                              _ptr(var.contiguous()), int(stats_f32), _ptr(g), _ptr(be), float(bn.eps),
-                                              int(bool(gelu)), _ptr(out), _stream()), "ptv3_segment_reduce_bn_act")
-    return out
-
-
 def unpool_add(parent, child, cluster):
     """parent + child[cluster]."""
     _dev(parent, child, cluster)

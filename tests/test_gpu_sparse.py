@@ -502,37 +502,6 @@ def test_subm_conv_tiles_parity(dtype, c, n, extent):
     assert rel_err(nob, OF.subm_conv(feat.float(), nbr, w.float(), None)) < TOL[dtype]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("gelu", [True, False])
-def test_segment_reduce_bn_act_equals_the_separate_kernels(dtype, gelu):
-    """Pooling's segment max followed by BatchNorm1d (+ GELU) (model.py:684-695) in one kernel: the same
-    bits as segment_reduce then bn_act, and within tolerance of torch in fp32."""
-    import torch.nn.functional as F
-    rng = np.random.default_rng(16)
-    g0 = torch.Generator().manual_seed(16)
-    idx, g, batch, offset = _indices(rng, 9000, 30, 2)
-    depth, code, order, inverse = OS.serialize(g, batch)
-    pc = OI.pool_clusters(code, g, batch, 1)
-    c = 72
-    feat = torch.randn(len(g), c, generator=g0).to(dtype)
-    bn = torch.nn.BatchNorm1d(c).eval()
-    bn.running_mean.normal_(0, 0.3, generator=g0)
-    bn.running_var.uniform_(0.5, 2.0, generator=g0)
-    bn.weight.data.uniform_(0.5, 1.5, generator=g0)
-    bn.bias.data.normal_(0, 0.3, generator=g0)
-    with torch.no_grad():
-        want = bn(OF.segment_csr(feat.float(), pc["indices"], pc["idx_ptr"], "max"))
-        if gelu:
-            want = F.gelu(want)
-    o = ops()
-    bn_d = bn.to(DEV)
-    args = (feat.to(DEV), to_dev(pc["indices"]), to_dev(pc["idx_ptr"]), "max")
-    got = o.segment_reduce_bn_act(*args, bn_d, gelu)
-    two = o.bn_act(o.segment_reduce(*args), bn_d.running_mean, bn_d.running_var, bn_d.weight, bn_d.bias, bn_d.eps, gelu)
-    assert got.dtype == dtype and torch.equal(got, two)
-    assert rel_err(got, want) < (1e-5 if dtype == torch.float32 else TOL[dtype])
-
-
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("c,n,mode", [(128, 5001, 3), (128, 77, 2), (256, 3000, 3), (256, 40_001, 2), (256, 1, 3), (128, 33, 3)])
 def test_linear_ln_parity(dtype, c, n, mode):
