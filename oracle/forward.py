@@ -81,8 +81,12 @@ def _block(sd, name, level, heads, patch, order_index):
     level["sparse_feat"] = feat
 
 
-def _pool(sd, name, parent, perm):
-    pc = OI.pool_clusters(parent["code"], parent["grid_coord"], parent["batch"], 1)
+def _pool(sd, name, parent, perm, stride=2):
+    # model.py:640-651: pooling depth = bit length of (stride - 1), 0 when deeper than the codes
+    pooling_depth = (int(np.ceil(stride)) - 1).bit_length()
+    if pooling_depth > parent["depth"]:
+        pooling_depth = 0
+    pc = OI.pool_clusters(parent["code"], parent["grid_coord"], parent["batch"], pooling_depth)
     code, order, inverse = pc["code"], pc["order"], pc["inverse"]
     if perm is not None:
         code, order, inverse = code[perm], order[perm], inverse[perm]
@@ -90,7 +94,7 @@ def _pool(sd, name, parent, perm):
     feat = F.gelu(_bn(sd, name + ".norm.0", feat))
     return dict(feat=feat, sparse_feat=feat, grid_coord=pc["grid_coord"], batch=pc["batch"],
                 offset=OI.batch2offset(pc["batch"]), code=code, order=order, inverse=inverse,
-                depth=parent["depth"] - 1, kmaps={}, cluster=pc["cluster"], parent=parent,
+                depth=parent["depth"] - pooling_depth, kmaps={}, cluster=pc["cluster"], parent=parent,
                 flash=parent["flash"])
 
 
@@ -138,11 +142,11 @@ def ptv3_forward(state_dict, grid_coord, feat, offset, perms=None, trace=None, *
 
     note("embedding", level)
 
-    assert all(st == 2 for st in cfg["stride"]), "the oracle pools by 2 per stage"
+    assert all(st == 2 ** ((int(st) - 1).bit_length()) for st in cfg["stride"])   # model.py:646
     n_stage = len(cfg["enc_depths"])
     for s in range(n_stage):
         if s > 0:
-            level = _pool(sd, f"enc.enc{s}.down", level, perms[s])
+            level = _pool(sd, f"enc.enc{s}.down", level, perms[s], cfg["stride"][s - 1])
             note(f"enc.enc{s}.down", level)
         for i in range(cfg["enc_depths"][s]):
             _block(sd, f"enc.enc{s}.block{i}", level, cfg["enc_num_head"][s], cfg["enc_patch_size"][s], i % k)

@@ -278,3 +278,19 @@ def test_forward_bf16_default_model():
     want = ptv3_forward(sd, d["grid_coord"], f, d["offset"], perms=perms)
     assert point.feat.dtype == torch.bfloat16
     assert rel_err(point.feat, want) < 2e-2
+
+
+def test_forward_other_pooling_strides_fp32():
+    """Strides 4 and 1 among the poolings (model.py:640-651: two levels at once, and none): the clusters
+    started ahead of the pooling module and the pair lists of the coarser levels follow the stride."""
+    from pointtransformerv3_amd import PointTransformerV3
+    kw = dict(stride=(2, 4, 1, 2), enc_depths=(1, 1, 1, 1, 1), dec_depths=(1, 1, 1, 1),
+              enc_patch_size=(256,) * 5, dec_patch_size=(256,) * 4)
+    torch.manual_seed(12)
+    model = PointTransformerV3(shuffle_orders=False, enable_flash=False, **kw).eval()
+    d, feat = _data(6000, 2, grid=0.02)
+    perms = _draw_perms(31, False)
+    want = ptv3_forward(model.state_dict(), d["grid_coord"], feat, d["offset"], enable_flash=False, perms=perms, **kw)
+    point = _run(model.to(DEV), d, feat, torch.float32)
+    assert point.feat.shape == want.shape
+    assert rel_err(point.feat, want) < 1e-4
