@@ -342,7 +342,23 @@ def conv_plan(nbr, tap_major=False):
 class PendingPlan:
     """conv_plan_direct between its two kernels: the pair count is on its way to the host."""
 
-    __slots__ = ("plan", "idx", "ks", "ws", "nbytes", "count")
+    __slots__ = ("plan", "idx", "ks", "ws", "nbytes", "count", "side_done")
+
+
+# The first halves of the pair lists are queued on a second stream: chains of small, latency-bound
+# kernels that depend on the coordinates only, they run beside the main stream's work (serialization,
+# projections) instead of in front of it (0.08 ms per forward; the pooling clusters gained nothing there).
+AHEAD_ON_SIDE_STREAM = True
+_SIDE_STREAMS = {}
+
+
+def _side_stream(dev):
+    """The second stream of this device (default priority), made to wait for what the main stream holds."""
+    side = _SIDE_STREAMS.get(dev)
+    if side is None:
+        side = _SIDE_STREAMS[dev] = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    return side
 
 
 def conv_plan_direct_start(indices, ks):
@@ -360,10 +376,22 @@ def conv_plan_direct_start(indices, ks):
     count = torch.empty(1, dtype=torch.int64, device=dev)
     nbytes = lib.ptv3_kmap_plan_workspace_bytes(n, int(ks))
     ws = _ws(nbytes, dev)
-    _lib.check(lib.ptv3_kmap_plan_count(_ptr(idx), n, int(ks), _ptr(plan.tap_ptr), _ptr(count), _ptr(ws), nbytes,
-                                        _stream()), "ptv3_kmap_plan_count")
     pend = PendingPlan()
     pend.plan, pend.idx, pend.ks, pend.ws, pend.nbytes = plan, idx, int(ks), ws, nbytes
+    pend.side_done = None
+    if AHEAD_ON_SIDE_STREAM and not Readback.blocking:
+        side = _side_stream(dev)
+        with torch.cuda.stream(side):
+            _lib.check(lib.ptv3_kmap_plan_count(_ptr(idx), n, int(ks), _ptr(plan.tap_ptr), _ptr(count), _ptr(ws), nbytes,
+                                                _stream()), "ptv3_kmap_plan_count")
+            pend.count = Readback(count)
+            pend.side_done = torch.cuda.Event()
+            pend.side_done.record(side)
+        for t in (idx, plan.tap_ptr, count, ws):   # not to be reused before the second stream is through
+            t.record_stream(side)
+        return pend
+    _lib.check(lib.ptv3_kmap_plan_count(_ptr(idx), n, int(ks), _ptr(plan.tap_ptr), _ptr(count), _ptr(ws), nbytes,
+                                        _stream()), "ptv3_kmap_plan_count")
     pend.count = Readback(count)
     return pend
 
@@ -373,6 +401,8 @@ def conv_plan_direct_finish(pend):
     plan, idx, n = pend.plan, pend.idx, pend.plan.n
     dev = idx.device
     plan.n_pairs = int(pend.count.get()[0])
+    if pend.side_done is not None:
+        torch.cuda.current_stream(dev).wait_event(pend.side_done)
     plan.row_ptr = torch.empty(n + 1, dtype=torch.int32, device=dev)
     plan.pair_in = torch.empty(max(plan.n_pairs, 1), dtype=torch.int32, device=dev)
     plan.pair_slot = torch.empty(max(plan.n_pairs, 1), dtype=torch.int32, device=dev)
@@ -459,7 +489,8 @@ def pool_clusters_start(code0, order0, shift, offset=None):
     off = None if offset is None else offset.to(torch.int64).contiguous()
     nbytes = lib.ptv3_pool_clusters_workspace_bytes(n)
     ws = _ws(nbytes, dev)
-    _lib.check(lib.ptv3_pool_clusters(_ptr(code0.contiguous()), _ptr(order0), n, int(shift), _ptr(off), nb,
+    code0 = code0.contiguous()
+    _lib.check(lib.ptv3_pool_clusters(_ptr(code0), _ptr(order0), n, int(shift), _ptr(off), nb,
                                       _ptr(pend.cluster), _ptr(pend.idx_ptr), _ptr(pend.head), _ptr(pend.count), _ptr(ws),
                                       nbytes, _stream()), "ptv3_pool_clusters")
     pend.read = Readback(pend.count)
