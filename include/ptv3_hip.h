@@ -162,6 +162,22 @@ int ptv3_kmap_plan_count(const int32_t *indices, int64_t n, int ks, int32_t *tap
 int ptv3_kmap_plan_fill(const int32_t *indices, int64_t n, int ks, const int32_t *tap_ptr,
                         int32_t *row_ptr, int32_t *pair_in, int32_t *pair_slot, void *workspace,
                         size_t workspace_bytes, void *stream);
+/* The 3x3x3 pair lists of a voxel set from its 5x5x5 lists (a 5x5x5 stem and 3x3x3 blocks on the same
+ * level, model.py:767-774 and :546-552): the inner 27 taps of the 5x5x5 neighbourhood are the 3x3x3
+ * neighbourhood, so one voxel hash and one neighbour search serve both. Bit-identical to
+ * ptv3_kmap_plan_count / _fill with ks = 3.
+ * _inner_count reads what ptv3_kmap_plan_count(ks = 5) left in its workspace (workspace5, untouched
+ * since) and writes found3 (n,) int32 [bit t: voxel has tap t], row_cnt3 (n,) int32 [pairs per voxel],
+ * tap_ptr3 (28,) int32 and n_pairs3 (device int64). The caller turns row_cnt3 into row_ptr3 (n+1,
+ * exclusive prefix sum) and, with the 5x5x5 lists of ptv3_kmap_plan_fill, _inner_fill writes pair_in3 /
+ * pair_slot3 (allocate n_pairs5 entries: the 3x3x3 lists are never longer). */
+int ptv3_kmap_plan_inner_count(const int32_t *tap_ptr5, int64_t n, const void *workspace5,
+                               size_t workspace5_bytes, int32_t *found3, int32_t *row_cnt3,
+                               int32_t *tap_ptr3, int64_t *n_pairs3, void *stream);
+int ptv3_kmap_plan_inner_fill(const int32_t *tap_ptr5, const int32_t *row_ptr5, const int32_t *pair_in5,
+                              const int32_t *pair_slot5, int64_t n, int64_t n_pairs5, const int32_t *found3,
+                              const int32_t *tap_ptr3, const int32_t *row_ptr3, int32_t *pair_in3,
+                              int32_t *pair_slot3, void *stream);
 int ptv3_subm_conv_pairs_fwd(const void *feat, int dtype, int64_t n, int cin, int taps,
                              int64_t n_pairs, const int32_t *tap_ptr, const int32_t *row_ptr,
                              const int32_t *pair_in, const int32_t *pair_slot, const void *weight,

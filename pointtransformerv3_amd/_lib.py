@@ -38,6 +38,8 @@ SIGNATURES = {
     "ptv3_kmap_plan_workspace_bytes": (_sz, [_i64, _i32]),
     "ptv3_kmap_plan_count": (_i32, [_vp, _i64, _i32, _vp, _vp, _vp, _sz, _vp]),
     "ptv3_kmap_plan_fill": (_i32, [_vp, _i64, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "ptv3_kmap_plan_inner_count": (_i32, [_vp, _i64, _vp, _sz, _vp, _vp, _vp, _vp, _vp]),
+    "ptv3_kmap_plan_inner_fill": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
     "ptv3_conv_plan_slots": (_i32, [_vp, _i32, _vp, _vp, _i64, _vp, _vp]),
     "ptv3_conv_plan_tile_count": (_i64, [_i64]),
     "ptv3_conv_plan_tiles": (_i32, [_vp, _vp, _i64, _i32, _vp, _vp, _vp, _vp]),

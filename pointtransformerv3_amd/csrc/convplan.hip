@@ -391,6 +391,86 @@ size_t direct_plan_bytes(int64_t n, int taps) {
     return vh_bytes(n) + direct_notes_bytes(n) + carve_plan(nullptr, n, taps, DIRECT_THREADS).bytes;
 }
 
+// ---- the 3x3x3 pair lists of a voxel set from its 5x5x5 lists: the inner 27 taps of the 5x5x5
+// neighbourhood ARE the 3x3x3 neighbourhood, so their tap-major segments are copied and only the
+// output-major slots are renumbered (a stem with a 5x5x5 kernel and blocks with 3x3x3 kernels share
+// level 0: one voxel hash and one neighbour search instead of two).
+__device__ __forceinline__ int inner_tap5(int t3) {   // index among the 125 taps of 3x3x3 tap t3
+    const int dx = t3 / 9, dy = (t3 / 3) % 3, dz = t3 % 3;
+    return ((dx + 1) * 5 + (dy + 1)) * 5 + (dz + 1);
+}
+
+// thread = voxel: its 3x3x3 taps (bit t3) and their number, from the tap set the 5x5x5 count pass left
+__global__ __launch_bounds__(PLAN_THREADS) void inner_count_kernel(DirectNotes notes, int64_t n,
+                                                                   uint32_t* __restrict__ found3,
+                                                                   int32_t* __restrict__ row_cnt3) {
+    const int64_t i = (int64_t)blockIdx.x * PLAN_THREADS + threadIdx.x;
+    if (i >= n) return;
+    const uint64_t lo = notes.found[i], hi = notes.found[n + i];
+    uint32_t f = 0;
+#pragma unroll
+    for (int t3 = 0; t3 < 27; ++t3) {
+        const int t5 = inner_tap5(t3);
+        const uint64_t bit = t5 < 64 ? (lo >> t5) & 1ull : (hi >> (t5 - 64)) & 1ull;
+        f |= (uint32_t)bit << t3;
+    }
+    found3[i] = f;
+    row_cnt3[i] = __popc(f);
+}
+
+// one work-group: tap_ptr3 = exclusive scan of the inner taps' counts, total to *n_pairs3
+__global__ __launch_bounds__(64) void inner_tap_ptr_kernel(const int32_t* __restrict__ tap_ptr5,
+                                                           int32_t* __restrict__ tap_ptr3,
+                                                           int64_t* __restrict__ n_pairs3) {
+    const int lane = threadIdx.x;
+    int c = 0;
+    if (lane < 27) {
+        const int t5 = inner_tap5(lane);
+        c = tap_ptr5[t5 + 1] - tap_ptr5[t5];
+    }
+    int x = c;
+#pragma unroll
+    for (int off = 1; off < 32; off <<= 1) {
+        const int y = __shfl_up(x, off, PTV3_WAVE);
+        if (lane >= off) x += y;
+    }
+    if (lane < 27) tap_ptr3[lane] = x - c;
+    if (lane == 26) {
+        tap_ptr3[27] = x;
+        *n_pairs3 = x;
+    }
+}
+
+// thread = pair of the 3x3x3 lists: copy its input row, renumber its output slot
+__global__ __launch_bounds__(PLAN_THREADS) void inner_fill_kernel(
+    const int32_t* __restrict__ tap_ptr5, const int32_t* __restrict__ row_ptr5, const int32_t* __restrict__ pair_in5,
+    const int32_t* __restrict__ pair_slot5, int64_t n, const uint32_t* __restrict__ found3,
+    const int32_t* __restrict__ tap_ptr3, const int32_t* __restrict__ row_ptr3, int32_t* __restrict__ pair_in3,
+    int32_t* __restrict__ pair_slot3) {
+    __shared__ int32_t tp3[28], base5[27];
+    if (threadIdx.x < 28) tp3[threadIdx.x] = tap_ptr3[threadIdx.x];
+    if (threadIdx.x < 27) base5[threadIdx.x] = tap_ptr5[inner_tap5(threadIdx.x)];
+    __syncthreads();
+    const int64_t q3 = (int64_t)blockIdx.x * PLAN_THREADS + threadIdx.x;
+    if (q3 >= tp3[27]) return;
+    int lo = 0, hi = 27;   // the (non-empty) tap whose segment holds q3
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (tp3[mid] <= (int32_t)q3) lo = mid; else hi = mid;
+    }
+    const int t3 = lo;
+    const int64_t q5 = (int64_t)base5[t3] + (q3 - tp3[t3]);
+    pair_in3[q3] = pair_in5[q5];
+    // output voxel of the pair: the row whose 5x5x5 slot range holds its slot
+    const int32_t slot5 = pair_slot5[q5];
+    int64_t a = 0, b = n;   // largest i with row_ptr5[i] <= slot5
+    while (b - a > 1) {
+        const int64_t mid = (a + b) >> 1;
+        if (row_ptr5[mid] <= slot5) a = mid; else b = mid;
+    }
+    pair_slot3[q3] = row_ptr3[a] + __popc(found3[a] & ((1u << t3) - 1u));
+}
+
 }  // namespace
 
 extern "C" size_t ptv3_conv_plan_workspace_bytes(int64_t n, int taps) {
@@ -481,5 +561,33 @@ extern "C" int ptv3_kmap_plan_fill(const int32_t* indices, int64_t n, int ks, co
         hipLaunchKernelGGL(direct_fill_kernel<5>, dim3((unsigned)blocks), dim3(DIRECT_THREADS), 0, stream, indices, n, h,
                            notes, (const uint32_t*)w.row_cnt, (const uint32_t*)w.blk_row_sum, (const uint32_t*)w.blk_tap_cnt,
                            tap_ptr, row_ptr, pair_in, pair_slot);
+    PTV3_RETURN_LAUNCH();
+}
+
+extern "C" int ptv3_kmap_plan_inner_count(const int32_t* tap_ptr5, int64_t n, const void* workspace5,
+                                          size_t workspace5_bytes, int32_t* found3, int32_t* row_cnt3,
+                                          int32_t* tap_ptr3, int64_t* n_pairs3, void* stream_) {
+    if (n < 1 || n >= (1ll << 31) / 128) return PTV3_EINVAL;
+    if (!tap_ptr5 || !workspace5 || !found3 || !row_cnt3 || !tap_ptr3 || !n_pairs3) return PTV3_EINVAL;
+    if (workspace5_bytes < direct_plan_bytes(n, 125)) return PTV3_EWORKSPACE;
+    hipStream_t stream = (hipStream_t)stream_;
+    const DirectNotes notes = carve_notes((char*)workspace5 + vh_bytes(n), n);   // left by ptv3_kmap_plan_count(ks = 5)
+    hipLaunchKernelGGL(inner_count_kernel, dim3((unsigned)ptv3_ceil_div(n, PLAN_THREADS)), dim3(PLAN_THREADS), 0, stream,
+                       notes, n, (uint32_t*)found3, row_cnt3);
+    hipLaunchKernelGGL(inner_tap_ptr_kernel, dim3(1), dim3(64), 0, stream, tap_ptr5, tap_ptr3, n_pairs3);
+    PTV3_RETURN_LAUNCH();
+}
+
+extern "C" int ptv3_kmap_plan_inner_fill(const int32_t* tap_ptr5, const int32_t* row_ptr5, const int32_t* pair_in5,
+                                         const int32_t* pair_slot5, int64_t n, int64_t n_pairs5, const int32_t* found3,
+                                         const int32_t* tap_ptr3, const int32_t* row_ptr3, int32_t* pair_in3,
+                                         int32_t* pair_slot3, void* stream_) {
+    if (n < 1 || n_pairs5 < 1) return PTV3_EINVAL;
+    if (!tap_ptr5 || !row_ptr5 || !pair_in5 || !pair_slot5 || !found3 || !tap_ptr3 || !row_ptr3 || !pair_in3 || !pair_slot3)
+        return PTV3_EINVAL;
+    // the 3x3x3 lists are at most as long as the 5x5x5 ones: threads past their end leave at once
+    hipLaunchKernelGGL(inner_fill_kernel, dim3((unsigned)ptv3_ceil_div(n_pairs5, PLAN_THREADS)), dim3(PLAN_THREADS), 0,
+                       (hipStream_t)stream_, tap_ptr5, row_ptr5, pair_in5, pair_slot5, n, (const uint32_t*)found3, tap_ptr3,
+                       row_ptr3, pair_in3, pair_slot3);
     PTV3_RETURN_LAUNCH();
 }

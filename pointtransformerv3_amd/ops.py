@@ -282,7 +282,18 @@ def subm_conv(feat, nbr, weight, bias=None, tap_major=False):
 class ConvPlan:
     """Active (input, output) pairs of a neighbour map, tap-major, plus each voxel's slots."""
 
-    __slots__ = ("n", "taps", "n_pairs", "tap_ptr", "row_ptr", "pair_in", "pair_slot", "_slot_pair", "_tiles")
+    __slots__ = ("n", "taps", "_n_pairs", "tap_ptr", "row_ptr", "pair_in", "pair_slot", "_slot_pair", "_tiles")
+
+    @property
+    def n_pairs(self):
+        """Number of active pairs; a plan derived from another one learns it from a read-back at first use."""
+        if isinstance(self._n_pairs, Readback):
+            self._n_pairs = int(self._n_pairs.get()[0])
+        return self._n_pairs
+
+    @n_pairs.setter
+    def n_pairs(self, value):
+        self._n_pairs = value
 
     def density(self):
         return self.n_pairs / max(1, self.n * self.taps)
@@ -409,6 +420,36 @@ def conv_plan_direct_finish(pend):
     _lib.check(lib.ptv3_kmap_plan_fill(_ptr(idx), n, pend.ks, _ptr(plan.tap_ptr), _ptr(plan.row_ptr),
                                        _ptr(plan.pair_in), _ptr(plan.pair_slot), _ptr(pend.ws), pend.nbytes, _stream()),
                "ptv3_kmap_plan_fill")
+    return plan
+
+
+def conv_plan_inner(plan5, pend5):
+    """The 3x3x3 pair lists of the voxel set whose 5x5x5 lists plan5 holds, derived from them and from what
+    the 5x5x5 count pass left in its workspace (pend5, the PendingPlan plan5 was finished from): no second
+    voxel hash, no second neighbour search. Bit-identical to conv_plan_direct(indices, 3)."""
+    lib = _lib.load()
+    n, dev = plan5.n, plan5.tap_ptr.device
+    assert plan5.taps == 125 and pend5.ks == 5
+    plan = ConvPlan()
+    plan.n, plan.taps = n, 27
+    plan.tap_ptr = torch.empty(28, dtype=torch.int32, device=dev)
+    found3 = torch.empty(n, dtype=torch.int32, device=dev)
+    row_cnt = torch.empty(n, dtype=torch.int32, device=dev)
+    row_ptr = torch.zeros(n + 1, dtype=torch.int32, device=dev)
+    count = torch.empty(1, dtype=torch.int64, device=dev)
+    _lib.check(lib.ptv3_kmap_plan_inner_count(_ptr(plan5.tap_ptr), n, _ptr(pend5.ws), pend5.nbytes, _ptr(found3),
+                                              _ptr(row_cnt), _ptr(plan.tap_ptr), _ptr(count), _stream()),
+               "ptv3_kmap_plan_inner_count")
+    plan.n_pairs = Readback(count)
+    torch.cumsum(row_cnt, 0, dtype=torch.int32, out=row_ptr[1:])
+    plan.row_ptr = row_ptr
+    cap = max(plan5.n_pairs, 1)
+    plan.pair_in = torch.empty(cap, dtype=torch.int32, device=dev)
+    plan.pair_slot = torch.empty(cap, dtype=torch.int32, device=dev)
+    _lib.check(lib.ptv3_kmap_plan_inner_fill(_ptr(plan5.tap_ptr), _ptr(plan5.row_ptr), _ptr(plan5.pair_in),
+                                             _ptr(plan5.pair_slot), n, plan5.n_pairs, _ptr(found3), _ptr(plan.tap_ptr),
+                                             _ptr(plan.row_ptr), _ptr(plan.pair_in), _ptr(plan.pair_slot), _stream()),
+               "ptv3_kmap_plan_inner_fill")
     return plan
 
 

@@ -166,7 +166,10 @@ class Point(AttrDict):
             return
         self._ensure_grid_coord()
         pending = self.setdefault("_pending_plans", {})
-        if ks not in pending:
+        if ks == 3 and 5 in pending:
+            # the 3x3x3 lists are the inner taps of the 5x5x5 ones: derived when those are finished
+            self.setdefault("_derived_plans", {})[3] = 5
+        elif ks not in pending:
             pending[ks] = ops.conv_plan_direct_start(self._sparse_indices_tensor(), ks)
 
     def pool_ahead(self, stride):
@@ -197,4 +200,6 @@ class Point(AttrDict):
                                batch_size=len(self.offset_host()))
         for ks, pend in self.pop("_pending_plans", {}).items():
             sct.indice_dict[("pending", ks)] = pend
+        for ks, src in self.pop("_derived_plans", {}).items():
+            sct.indice_dict[("derive", ks)] = src
         self["sparse_conv_feat"] = sct

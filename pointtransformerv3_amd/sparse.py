@@ -35,6 +35,16 @@ class SparseConvTensor:
             self.indice_dict[key] = nbr
         return nbr
 
+    def _finish_pending(self, kernel_size):
+        """Second half of a pair-list construction started ahead; the 3x3x3 lists that were asked to be
+        derived from these 5x5x5 lists are made right behind them and parked under ("ready", 3)."""
+        pend = self.indice_dict.pop(("pending", kernel_size))
+        plan = ops.conv_plan_direct_finish(pend)
+        for k in [k for k in self.indice_dict if isinstance(k, tuple) and k[0] == "derive" and self.indice_dict[k] == kernel_size]:
+            self.indice_dict[("ready", k[1])] = ops.conv_plan_inner(plan, pend)
+            del self.indice_dict[k]
+        return plan
+
     def conv_plan(self, kernel_size, indice_key=None):
         """Pair lists of the neighbour map (see ops.conv_plan), cached like the map itself; built
         straight from the coordinates unless the map has been built already."""
@@ -43,8 +53,15 @@ class SparseConvTensor:
             return self.indice_dict[key]
         if indice_key is not None and (indice_key, kernel_size) in self.indice_dict:
             plan = ops.conv_plan(self.indice_dict[(indice_key, kernel_size)], tap_major=True)
+        elif ("ready", kernel_size) in self.indice_dict:
+            plan = self.indice_dict.pop(("ready", kernel_size))
         elif ("pending", kernel_size) in self.indice_dict:
-            plan = ops.conv_plan_direct_finish(self.indice_dict.pop(("pending", kernel_size)))
+            plan = self._finish_pending(kernel_size)
+        elif ("derive", kernel_size) in self.indice_dict and ("pending", self.indice_dict[("derive", kernel_size)]) in self.indice_dict:
+            # asked for before the lists it derives from were finished: finish those (kept for their own conv)
+            src = self.indice_dict[("derive", kernel_size)]
+            self.indice_dict[("ready", src)] = self._finish_pending(src)
+            plan = self.indice_dict.pop(("ready", kernel_size))
         else:
             plan = ops.conv_plan_direct(self.indices, kernel_size)
         if key is not None:

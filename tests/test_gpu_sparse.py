@@ -540,3 +540,20 @@ def test_linear_ln_parity(dtype, c, n, mode):
     assert rel_err(got0, want0) < TOL[dtype] and rel_err(got1, want1) < TOL[dtype]
     ulp = 2e-3 if dtype == torch.float16 else 1.6e-2
     assert rel_err(got0, two0.float().cpu()) < ulp and rel_err(got1, two1.float().cpu()) < ulp
+
+
+@pytest.mark.parametrize("n,extent,nb", [(1, 4, 1), (2500, 14, 2), (50_000, 60, 3), (20_000, 300, 1)])
+def test_conv_plan_inner_equals_direct_3x3x3(n, extent, nb):
+    """The 3x3x3 pair lists derived from the 5x5x5 ones (their inner 27 taps) are the lists built directly."""
+    rng = np.random.default_rng(n + extent)
+    idx, *_ = _indices(rng, n, extent, nb)
+    o = ops()
+    dev_idx = to_dev(idx)
+    pend5 = o.conv_plan_direct_start(dev_idx, 5)
+    plan5 = o.conv_plan_direct_finish(pend5)
+    got = o.conv_plan_inner(plan5, pend5)
+    ref = o.conv_plan_direct(dev_idx, 3)
+    assert got.n_pairs == ref.n_pairs and got.taps == 27 and got.n == ref.n
+    assert torch.equal(got.tap_ptr, ref.tap_ptr) and torch.equal(got.row_ptr, ref.row_ptr)
+    assert torch.equal(got.pair_in[:got.n_pairs], ref.pair_in[:ref.n_pairs])
+    assert torch.equal(got.pair_slot[:got.n_pairs], ref.pair_slot[:ref.n_pairs])
