@@ -363,13 +363,17 @@ AHEAD_ON_SIDE_STREAM = True
 _SIDE_STREAMS = {}
 
 
-def _side_stream(dev):
-    """The second stream of this device (default priority), made to wait for what the main stream holds."""
-    side = _SIDE_STREAMS.get(dev)
+def side_stream(dev, index=0):
+    """Side stream `index` of this device (default priority), made to wait for what the current stream holds."""
+    side = _SIDE_STREAMS.get((dev, index))
     if side is None:
-        side = _SIDE_STREAMS[dev] = torch.cuda.Stream(device=dev)
+        side = _SIDE_STREAMS[(dev, index)] = torch.cuda.Stream(device=dev)
     side.wait_stream(torch.cuda.current_stream(dev))
     return side
+
+
+def _side_stream(dev):
+    return side_stream(dev, 0)
 
 
 def conv_plan_direct_start(indices, ks):
