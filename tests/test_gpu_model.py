@@ -294,3 +294,23 @@ def test_forward_other_pooling_strides_fp32():
     point = _run(model.to(DEV), d, feat, torch.float32)
     assert point.feat.shape == want.shape
     assert rel_err(point.feat, want) < 1e-4
+
+
+@pytest.mark.parametrize("sizes", [[50], [1, 3000], [200, 2, 70]])
+def test_forward_tiny_and_ragged_scenes_fp32(sizes):
+    """Scenes smaller than a patch, single-point scenes, very unequal scenes in one batch."""
+    from pointtransformerv3_amd import PointTransformerV3, synthetic
+    kw = dict(enc_depths=(1, 1, 1, 1, 1), dec_depths=(1, 1, 1, 1), enc_patch_size=(128,) * 5, dec_patch_size=(128,) * 4)
+    torch.manual_seed(0)
+    model = PointTransformerV3(shuffle_orders=False, enable_flash=False, **kw).eval()
+    scenes = []
+    for i, n in enumerate(sizes):
+        sc = synthetic.room_scene(max(n * 2, 4), 100 + i, 0.05)
+        scenes.append(dict(coord=sc["coord"][:n], grid_coord=sc["grid_coord"][:n]))
+    d = synthetic.collate(scenes)
+    assert [len(s["grid_coord"]) for s in scenes] == sizes
+    feat = synthetic.room_features(d["coord"], 1)
+    perms = _draw_perms(3, False)
+    want = ptv3_forward(model.state_dict(), d["grid_coord"], feat, d["offset"], enable_flash=False, perms=perms, **kw)
+    point = _run(model.to(DEV), d, feat, torch.float32)
+    assert rel_err(point.feat, want) < 1e-4
