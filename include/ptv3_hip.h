@@ -117,6 +117,17 @@ int ptv3_patch_attn_rpe_fwd(const float *qkv, int64_t n_rows, int channels, int 
                             const int32_t *grid_coord, const float *rpe_table, int pos_bnd, float *out,
                             void *stream);
 
+/* Backward of ptv3_patch_attn_fwd: what autograd derives for model.py:456-484 (the backward of the
+ * flash_attn_varlen_qkvpacked_func call at :476-482 and of the row gathers around it). out is the
+ * forward result, dout its gradient (n_rows, C); dqkv (n_rows, 3*C) receives [dq | dk | dv] per row,
+ * every element written. Filler slots take no gradient as queries; as keys their share is added to
+ * the row they repeat. n_pad = cu_seqlens[n_seq], the number of slots. */
+size_t ptv3_patch_attn_bwd_workspace_bytes(int dtype, int64_t n_pad, int channels, int heads);
+int ptv3_patch_attn_bwd(const void *qkv, const void *out, const void *dout, int dtype, int64_t n_rows,
+                        int channels, int heads, const int32_t *slot_src, const int32_t *slot_dst,
+                        const int32_t *cu_seqlens, int64_t n_seq, int64_t max_seqlen, int64_t n_pad,
+                        float scale, void *dqkv, void *workspace, size_t workspace_bytes, void *stream);
+
 /* spconv.SubMConv3d's index generation (call sites model.py:546-552, :767-774, tensor built
  * at :165-172). indices (n,4) int32 [batch,x,y,z], coordinates in [0, 65535];
  * nbr int32, entry (voxel i, tap t = (kx*ks+ky)*ks+kz) = row of the voxel at
@@ -133,6 +144,13 @@ int ptv3_kmap_build(const int32_t *indices, int64_t n, int ks, int tap_major, in
 int ptv3_subm_conv_fwd(const void *feat, int dtype, int64_t n, int cin, const int32_t *nbr,
                        int taps, int tap_major, const void *weight, const void *bias, int cout,
                        void *out, void *stream);
+
+/* Weight gradient of spconv.SubMConv3d (same call sites): dweight[co][t][ci] += sum over voxels i with
+ * nbr[t][i] >= 0 of dout[i][co] * feat[nbr[t][i]][ci]. nbr is tap-major (taps, n); dweight
+ * (cout, taps, cin) fp32 is accumulated into (zero it first). The input gradient needs no kernel of
+ * its own: it is ptv3_subm_conv_fwd of dout with weight'[ci][t][co] = weight[co][taps-1-t][ci]. */
+int ptv3_subm_conv_wgrad(const void *feat, const void *dout, int dtype, int64_t n, int cin, int cout,
+                         const int32_t *nbr, int taps, float *dweight, void *stream);
 
 /* Sparse-pair form of the same convolution, for maps where most taps of most voxels are empty
  * (surface scans: 2-13 of 27 taps active). ptv3_conv_plan_count derives from nbr (n,taps) the
@@ -245,6 +263,14 @@ int ptv3_pool_orders(const int64_t *order, const int64_t *cluster, int64_t n, in
  * src (n,c) of dtype, out (m,c) of dtype. */
 int ptv3_segment_reduce(const void *src, int dtype, int64_t n, int c, const int64_t *indices,
                         const int64_t *idx_ptr, int64_t m, int op, void *out, void *stream);
+
+/* Backward of ptv3_segment_reduce (torch_scatter.segment_csr's, model.py:684-689): dsrc (n,c).
+ * max / min: the gradient of a cluster goes to the first member in list order whose value equals
+ * out; sum: to every member; mean: divided by the cluster size. Every row of src must belong to
+ * exactly one cluster (true for grid pooling), so every element of dsrc is written. */
+int ptv3_segment_reduce_bwd(const void *src, const void *out, const void *dout, int dtype, int64_t n, int c,
+                            const int64_t *indices, const int64_t *idx_ptr, int64_t m, int op, void *dsrc,
+                            void *stream);
 
 /* model.py:746: out[i] = parent[i] + child[cluster[i]]; parent,out (n,c), child (m,c). */
 int ptv3_unpool_add(const void *parent, const void *child, int dtype, int64_t n, int c,

@@ -129,7 +129,11 @@ def subm_conv_dense(feat, indices, weight, bias=None):
 
 def segment_csr(src, indices, idx_ptr, reduce="max"):
     """reduce(src[indices[idx_ptr[m]:idx_ptr[m+1]]]) per segment m (model.py:684-689).
-    Segments are never empty on this path."""
+    Segments are never empty on this path. A src that takes a gradient goes through torch operators
+    (same values) so that autograd can differentiate it: the gradient of max / min lands on the
+    attaining member, split evenly should several tie (torch_scatter picks one of them)."""
+    if isinstance(src, torch.Tensor) and src.requires_grad:
+        return _segment_csr_autograd(src, indices, idx_ptr, reduce)
     src = np.asarray(torch.as_tensor(src, dtype=torch.float32))[np.asarray(indices)]
     starts = np.asarray(idx_ptr[:-1], dtype=np.int64)
     if reduce == "max":
@@ -142,6 +146,15 @@ def segment_csr(src, indices, idx_ptr, reduce="max"):
             out = out / np.diff(np.asarray(idx_ptr, dtype=np.int64))[:, None]
         out = out.astype(np.float32)
     return torch.from_numpy(np.ascontiguousarray(out))
+
+
+def _segment_csr_autograd(src, indices, idx_ptr, reduce):
+    ptr = torch.as_tensor(np.asarray(idx_ptr), dtype=torch.int64)
+    rows = src[torch.as_tensor(np.asarray(indices), dtype=torch.int64)]
+    m = ptr.numel() - 1
+    seg = torch.repeat_interleave(torch.arange(m), ptr[1:] - ptr[:-1])[:, None].expand_as(rows)
+    op = {"max": "amax", "min": "amin", "sum": "sum", "mean": "mean"}[reduce]
+    return torch.zeros(m, src.shape[1], dtype=src.dtype).scatter_reduce(0, seg, rows, op, include_self=False)
 
 
 def unpool_add(parent_feat, child_feat, cluster):

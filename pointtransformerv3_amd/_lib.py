@@ -29,9 +29,13 @@ SIGNATURES = {
     "ptv3_patch_attn_fwd": (_i32, [_vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _f32,
                                    _vp, _vp]),
     "ptv3_patch_attn_rpe_fwd": (_i32, [_vp, _i64, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _f32, _vp, _vp, _i32, _vp, _vp]),
+    "ptv3_patch_attn_bwd_workspace_bytes": (_sz, [_i32, _i64, _i32, _i32]),
+    "ptv3_patch_attn_bwd": (_i32, [_vp, _vp, _vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _vp,
+                                   _vp, _sz, _vp]),
     "ptv3_kmap_workspace_bytes": (_sz, [_i64]),
     "ptv3_kmap_build": (_i32, [_vp, _i64, _i32, _i32, _vp, _vp, _sz, _vp]),
     "ptv3_subm_conv_fwd": (_i32, [_vp, _i32, _i64, _i32, _vp, _i32, _i32, _vp, _vp, _i32, _vp, _vp]),
+    "ptv3_subm_conv_wgrad": (_i32, [_vp, _vp, _i32, _i64, _i32, _i32, _vp, _i32, _vp, _vp]),
     "ptv3_conv_plan_workspace_bytes": (_sz, [_i64, _i32]),
     "ptv3_conv_plan_count": (_i32, [_vp, _i64, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
     "ptv3_conv_plan_fill": (_i32, [_vp, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
@@ -54,6 +58,7 @@ SIGNATURES = {
     "ptv3_pool_orders_workspace_bytes": (_sz, [_i64, _i32]),
     "ptv3_pool_orders": (_i32, [_vp, _vp, _i64, _i32, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "ptv3_segment_reduce": (_i32, [_vp, _i32, _i64, _i32, _vp, _vp, _i64, _i32, _vp, _vp]),
+    "ptv3_segment_reduce_bwd": (_i32, [_vp, _vp, _vp, _i32, _i64, _i32, _vp, _vp, _i64, _i32, _vp, _vp]),
     "ptv3_unpool_add": (_i32, [_vp, _vp, _i32, _i64, _i32, _vp, _i64, _vp, _vp]),
     "ptv3_bn_act": (_i32, [_vp, _vp, _vp, _i32, _vp, _vp, _i32, _i64, _i32, _f32, _i32, _vp, _vp]),
     "ptv3_linear_fwd": (_i32, [_vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp]),

@@ -1,0 +1,88 @@
+"""torch.autograd.Function wrappers of the sparse operators that have HIP backward kernels: patch
+attention (the reference relies on flash_attn's backward, model.py:476-482), submanifold convolution
+(spconv's, model.py:546-552, :767-774), segment reduction (torch_scatter's, model.py:684-689) and the
+unpooling add (index_select's, model.py:746). Dense layers keep torch's own autograd."""
+import torch
+
+from . import ops
+
+
+class PatchAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale):
+        out = ops.patch_attention(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale)
+        ctx.save_for_backward(qkv, out)
+        ctx.args = (num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        qkv, out = ctx.saved_tensors
+        return (ops.patch_attention_bwd(qkv, out, dout, *ctx.args),) + (None,) * 6
+
+
+class SubMConv(torch.autograd.Function):
+    """module is the SubMConv3d whose forward dispatch (pair, tile or dense form) is reused for the
+    input gradient; sparse is the SparseConvTensor that owns the neighbour maps."""
+
+    @staticmethod
+    def forward(ctx, feat, weight, bias, sparse, module):
+        cout, cin = weight.shape[0], weight.shape[-1]
+        w = weight.detach().reshape(cout, -1, cin)
+        out = module.convolve(sparse, feat.detach(), w, None if bias is None else bias.detach())
+        ctx.save_for_backward(feat, weight)
+        ctx.sparse, ctx.module, ctx.has_bias = sparse, module, bias is not None
+        ctx.bias_dtype = None if bias is None else bias.dtype
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        feat, weight = ctx.saved_tensors
+        sparse, module = ctx.sparse, ctx.module
+        cout, cin = weight.shape[0], weight.shape[-1]
+        dout = dout.contiguous()
+        dfeat = dweight = dbias = None
+        if ctx.needs_input_grad[0]:
+            # the same convolution with mirrored taps and the weight transposed
+            wt = weight.detach().reshape(cout, -1, cin).flip(1).permute(2, 1, 0).contiguous()
+            pad = -cin % 16 if dout.dtype != torch.float32 else 0   # the half-precision forms write outputs in 16s
+            if pad:
+                wt = torch.nn.functional.pad(wt, (0, 0, 0, 0, 0, pad))
+            dfeat = module.convolve(sparse, dout, wt, None)[:, :cin].to(feat.dtype)
+        if ctx.needs_input_grad[1]:
+            nbr = sparse.neighbour_map(module.kernel_size, module.indice_key)
+            dweight = ops.subm_conv_wgrad(feat, dout, nbr).reshape(weight.shape).to(weight.dtype)
+        if ctx.has_bias and ctx.needs_input_grad[2]:
+            dbias = dout.sum(0, dtype=torch.float32).to(ctx.bias_dtype)
+        return dfeat, dweight, dbias, None, None
+
+
+class SegmentReduce(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, src, indices, idx_ptr, reduce):
+        out = ops.segment_reduce(src, indices, idx_ptr, reduce)
+        ctx.save_for_backward(src, out)
+        ctx.args = (indices, idx_ptr, reduce)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        src, out = ctx.saved_tensors
+        return ops.segment_reduce_bwd(src, out, dout, *ctx.args), None, None, None
+
+
+class UnpoolAdd(torch.autograd.Function):
+    """parent + child[cluster]; indices / idx_ptr are the pooling's member lists of the clusters, over which
+    the gradient of child is a segment sum (no atomics)."""
+
+    @staticmethod
+    def forward(ctx, parent, child, cluster, indices, idx_ptr):
+        ctx.args = (indices, idx_ptr)
+        ctx.child_dtype = child.dtype
+        return ops.unpool_add(parent, child, cluster)
+
+    @staticmethod
+    def backward(ctx, dout):
+        dout = dout.contiguous()
+        dchild = ops.segment_reduce(dout, *ctx.args, "sum").to(ctx.child_dtype) if ctx.needs_input_grad[1] else None
+        return dout, dchild, None, None, None

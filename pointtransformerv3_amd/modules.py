@@ -11,6 +11,7 @@ import torch
 import torch.nn as nn
 
 from . import ops
+from .autograd import SegmentReduce, UnpoolAdd
 from .point import AttrDict, Point, offset2bincount
 from .sparse import SparseConvTensor, SubMConv3d, is_spconv_module
 
@@ -36,7 +37,8 @@ class LayerNorm(nn.LayerNorm):
     """nn.LayerNorm (same parameters and state_dict) evaluated by the row-wise HIP kernel."""
 
     def forward(self, x):
-        if x.dim() != 2 or len(self.normalized_shape) != 1 or self.weight is None or self.bias is None:
+        if (x.dim() != 2 or len(self.normalized_shape) != 1 or self.weight is None or self.bias is None
+                or ops.wants_grad(x, self.weight, self.bias)):
             return super().forward(x)
         return ops.layer_norm(x, self.weight, self.bias, self.eps)
 
@@ -44,7 +46,8 @@ class LayerNorm(nn.LayerNorm):
 def _fusable_bn(module, feat):
     """Inference-mode BatchNorm1d over (N, C) GPU features that the one-pass kernel covers."""
     return (type(module) is nn.BatchNorm1d and not module.training and module.track_running_stats
-            and module.running_mean is not None and feat.is_cuda and feat.dim() == 2 and feat.shape[1] % 8 == 0)
+            and module.running_mean is not None and feat.is_cuda and feat.dim() == 2 and feat.shape[1] % 8 == 0
+            and not ops.wants_grad(feat, module.weight, module.bias))
 
 
 def _exact_gelu(module):
@@ -244,6 +247,14 @@ class SerializedAttention(PointModule):
             self.patch_size = min(int(sizes.min()), self.patch_size_max)
         _, _, cu_seqlens = self.get_padding_and_inverse(point)
         slot_src, slot_dst = self._slots(point)
+        grad = ops.wants_grad(qkv)
+        if grad and self.enable_rpe:
+            raise NotImplementedError("the relative position bias has no backward kernel: train with enable_rpe=False")
+        if grad:
+            from .autograd import PatchAttention
+            half = qkv.half() if (self.enable_flash and qkv.dtype == torch.float32) else qkv
+            return PatchAttention.apply(half, self.num_heads, slot_src, slot_dst, cu_seqlens, self.patch_size,
+                                        self.scale).to(qkv.dtype)
         if self.enable_rpe:
             # bias from the grid offsets of (query, key) inside the patch, added before the softmax; the
             # reference takes this path in float (upcast_attention / upcast_softmax, model.py:463-471)
@@ -314,8 +325,8 @@ class Block(PointModule):
                 and not (self.training and not isinstance(self.drop_path[0], nn.Identity)))
 
     def forward(self, point):
-        if not self._plain_layernorms():
-            return self._forward_modular(point)
+        if not self._plain_layernorms() or (torch.is_grad_enabled() and ops.wants_grad(point.feat, *self.parameters())):
+            return self._forward_modular(point)   # module by module: every one of them has a backward
         ln_cpe, ln1, ln2 = self.cpe[2], self.norm1[0], self.norm2[0]
         mlp = self.mlp[0]
         plain_mlp = (type(mlp) is MLP and mlp.fc1.bias is not None and mlp.fc2.bias is not None
@@ -449,7 +460,8 @@ class SerializedPooling(PointModule):
         order, inverse = ops.pool_orders(point.serialized_order, cluster, m, perm)
 
         fields = AttrDict(
-            feat=ops.segment_reduce(projected, indices, idx_ptr, self.reduce),
+            feat=(SegmentReduce.apply(projected, indices, idx_ptr, self.reduce) if ops.wants_grad(projected)
+                  else ops.segment_reduce(projected, indices, idx_ptr, self.reduce)),
             grid_coord=grid_coord,
             serialized_code=code,
             serialized_order=order,
@@ -460,6 +472,7 @@ class SerializedPooling(PointModule):
             _offset_host=offset_host,
             _sparse_indices=indices4,   # [batch, x, y, z] int32, what sparsify() would concatenate
             _pending_plans=plans,
+            _pool_members=(indices, idx_ptr),   # the clusters' member lists: the unpooling's backward sums over them
         )
         if "coord" in point:
             fields["coord"] = ops.segment_reduce(point.coord.float(), indices, idx_ptr, "mean")
@@ -513,7 +526,10 @@ class SerializedUnpooling(PointModule):
         parent = self.proj_skip(parent)
         # only .feat is updated; parent.sparse_conv_feat keeps the skip projection, which is
         # what the first decoder block's conv reads in the reference as well (model.py:746)
-        parent.feat = ops.unpool_add(parent.feat, point.feat, inverse)
+        if ops.wants_grad(parent.feat, point.feat):
+            parent.feat = UnpoolAdd.apply(parent.feat, point.feat, inverse, *point["_pool_members"])
+        else:
+            parent.feat = ops.unpool_add(parent.feat, point.feat, inverse)
         if self.traceable:
             parent["unpooling_parent"] = point
         return parent

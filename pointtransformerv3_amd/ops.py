@@ -38,6 +38,12 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
+def wants_grad(*tensors):
+    """True when autograd is recording and one of the tensors (or parameters) takes a gradient: the fused
+    inference kernels are then left for the operators that have a backward."""
+    return torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors)
+
+
 class Readback:
     """Device -> host read of a small tensor that does not drain the stream.
 
@@ -221,6 +227,26 @@ def patch_attention(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, 
     return out
 
 
+def patch_attention_bwd(qkv, out, dout, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale):
+    """Gradient of patch_attention with respect to qkv, (N, 3C) laid out [dq | dk | dv]."""
+    _dev(qkv, out, dout, slot_src, slot_dst, cu_seqlens)
+    lib = _lib.load()
+    qkv, out = qkv.contiguous(), out.contiguous()
+    dout = dout.to(qkv.dtype).contiguous()
+    n, c3 = qkv.shape
+    c = c3 // 3
+    n_pad = slot_src.shape[0]
+    dqkv = torch.empty_like(qkv)
+    code = _dtype_code(qkv)
+    nbytes = lib.ptv3_patch_attn_bwd_workspace_bytes(code, n_pad, c, int(num_heads))
+    ws = _ws(nbytes, qkv.device)
+    _lib.check(lib.ptv3_patch_attn_bwd(_ptr(qkv), _ptr(out), _ptr(dout), code, n, c, int(num_heads), _ptr(slot_src),
+                                       _ptr(slot_dst), _ptr(cu_seqlens), cu_seqlens.shape[0] - 1, int(max_seqlen),
+                                       n_pad, float(scale), _ptr(dqkv), _ptr(ws), nbytes, _stream()),
+               "ptv3_patch_attn_bwd")
+    return dqkv
+
+
 def patch_attention_rpe(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale, grid_coord, rpe_table,
                         pos_bnd):
     """patch_attention with the relative position bias of model.py:297-316 added to every score:
@@ -277,6 +303,22 @@ def subm_conv(feat, nbr, weight, bias=None, tap_major=False):
                                       int(bool(tap_major)), _ptr(w), _ptr(b), cout, _ptr(out), _stream()),
                "ptv3_subm_conv_fwd")
     return out
+
+
+def subm_conv_wgrad(feat, dout, nbr):
+    """Weight gradient (Cout, V, Cin) in fp32 of the submanifold convolution; nbr is the tap-major (V, N) map."""
+    _dev(feat, dout, nbr)
+    lib = _lib.load()
+    feat = feat.contiguous()
+    dout = dout.to(feat.dtype).contiguous()
+    nbr = nbr.contiguous()
+    n, cin = feat.shape
+    cout = dout.shape[1]
+    taps = nbr.shape[0]
+    dw = torch.zeros((cout, taps, cin), dtype=torch.float32, device=feat.device)
+    _lib.check(lib.ptv3_subm_conv_wgrad(_ptr(feat), _ptr(dout), _dtype_code(feat), n, cin, cout, _ptr(nbr), taps,
+                                        _ptr(dw), _stream()), "ptv3_subm_conv_wgrad")
+    return dw
 
 
 class ConvPlan:
@@ -625,6 +667,21 @@ def segment_reduce(src, indices, idx_ptr, reduce="max"):
     return out
 
 
+def segment_reduce_bwd(src, out, dout, indices, idx_ptr, reduce="max"):
+    """Gradient of segment_reduce with respect to src (every row of src belongs to one segment)."""
+    _dev(src, out, dout, indices, idx_ptr)
+    lib = _lib.load()
+    src, out = src.contiguous(), out.contiguous()
+    dout = dout.to(src.dtype).contiguous()
+    n, c = src.shape
+    m = idx_ptr.shape[0] - 1
+    dsrc = torch.empty_like(src)
+    _lib.check(lib.ptv3_segment_reduce_bwd(_ptr(src), _ptr(out), _ptr(dout), _dtype_code(src), n, c,
+                                           _ptr(indices.contiguous()), _ptr(idx_ptr.contiguous()), m,
+                                           REDUCE_OPS[reduce], _ptr(dsrc), _stream()), "ptv3_segment_reduce_bwd")
+    return dsrc
+
+
 def unpool_add(parent, child, cluster):
     """parent + child[cluster]."""
     _dev(parent, child, cluster)
@@ -716,6 +773,12 @@ def linear_rows_pays(x, weight, gelu=False):
 
 def linear(x, mod, gelu=False):
     """mod(x) for an nn.Linear (followed by exact GELU if gelu), on whichever path is faster."""
+    if wants_grad(x, mod.weight, mod.bias):
+        w, b = mod.weight, mod.bias
+        if not torch.is_autocast_enabled() and w.dtype != x.dtype:
+            w, b = w.to(x.dtype), None if b is None else b.to(x.dtype)
+        y = torch.nn.functional.linear(x, w, b)
+        return torch.nn.functional.gelu(y) if gelu else y
     if linear_rows_pays(x, mod.weight, gelu):
         return linear_rows(x, mod.weight, mod.bias, gelu)
     y = torch.nn.functional.linear(x, mod.weight, mod.bias)

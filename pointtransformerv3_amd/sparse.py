@@ -111,31 +111,38 @@ class SubMConv3d(nn.Module):
             self._packed = cached = (key, packed)
         return cached[1]
 
-    def forward(self, x):
-        feat = x.features
-        if torch.is_autocast_enabled():
-            feat = feat.to(torch.get_autocast_gpu_dtype())
-        weight = self.weight.reshape(self.out_channels, -1, self.in_channels)
-        cin = self.in_channels
+    def convolve(self, x, feat, weight, bias, packed=None):
+        """The convolution of feat (N, Cin) over x's neighbourhoods with weight (Cout, V, Cin), on whichever
+        form fits: dense output-stationary (fp32, or many active taps), pair lists, or tiles. packed() hands
+        out the weight in the tile kernel's order when the caller has it cached."""
+        cout, _, cin = weight.shape
         if feat.dtype == torch.float32:
             nbr = x.neighbour_map(self.kernel_size, self.indice_key)
-            return x.replace_feature(ops.subm_conv(feat, nbr, weight, self.bias, tap_major=True))
+            return ops.subm_conv(feat, nbr, weight, bias, tap_major=True)
         if cin % 16 != 0:
             # the MFMA kernels consume input channels 16 at a time: zero-pad the thin stem input
             pad = 16 - cin % 16
             feat = nn.functional.pad(feat, (0, pad))
             weight = nn.functional.pad(weight, (0, pad))
         plan = x.conv_plan(self.kernel_size, self.indice_key)
-        if (self.kernel_size == 3 and cin == self.out_channels and cin in ops.CONV_TILE_CHANNELS
+        if (self.kernel_size == 3 and cin == cout and cin in ops.CONV_TILE_CHANNELS
                 and plan.n < (1 << 24) and plan.n_pairs >= self.TILE_MODE_MIN_PAIRS_PER_VOXEL * plan.n):
-            return x.replace_feature(ops.subm_conv_tiles(feat, plan, self._packed_weight(feat.dtype), self.bias))
+            tiles = packed() if packed is not None else ops.conv_pack_weight(weight, 27, feat.dtype)
+            return ops.subm_conv_tiles(feat, plan, tiles, bias)
         weight = weight.to(feat.dtype)
-        if plan.density() <= self.PAIR_MODE_MAX_DENSITY and self.out_channels % 8 == 0:
-            out = ops.subm_conv_pairs(feat, plan, weight, self.bias)
-        else:
-            out = ops.subm_conv(feat, x.neighbour_map(self.kernel_size, self.indice_key), weight, self.bias,
-                                tap_major=True)
-        return x.replace_feature(out)
+        if plan.density() <= self.PAIR_MODE_MAX_DENSITY and cout % 8 == 0:
+            return ops.subm_conv_pairs(feat, plan, weight, bias)
+        return ops.subm_conv(feat, x.neighbour_map(self.kernel_size, self.indice_key), weight, bias, tap_major=True)
+
+    def forward(self, x):
+        feat = x.features
+        if torch.is_autocast_enabled():
+            feat = feat.to(torch.get_autocast_dtype("cuda"))
+        if ops.wants_grad(feat, self.weight, self.bias):
+            from .autograd import SubMConv
+            return x.replace_feature(SubMConv.apply(feat, self.weight, self.bias, x, self))
+        weight = self.weight.reshape(self.out_channels, -1, self.in_channels)
+        return x.replace_feature(self.convolve(x, feat, weight, self.bias, lambda: self._packed_weight(feat.dtype)))
 
 
 def is_spconv_module(module):

@@ -15,7 +15,7 @@ def to_dev(a, dtype=None):
 def rel_err(got, want):
     """max |got-want| / max |want| — the 'max-abs relative' measure of the parity bar."""
     got = got.detach().float().cpu()
-    want = torch.as_tensor(want).float()
+    want = torch.as_tensor(want).detach().float()
     return float((got - want).abs().max() / want.abs().max().clamp_min(1e-12))
 
 
