@@ -264,6 +264,12 @@ int ptv3_pool_orders(const int64_t *order, const int64_t *cluster, int64_t n, in
 int ptv3_segment_reduce(const void *src, int dtype, int64_t n, int c, const int64_t *indices,
                         const int64_t *idx_ptr, int64_t m, int op, void *out, void *stream);
 
+/* Weight gradient of nn.Linear (model.py:366-367, :505-507, :553, :633, :726-727 under autograd):
+ * dweight[o][i] += sum over rows r of dout[r][o] * x[r][i]. x (n,k), dout (n,nout) fp16 / bf16 with k and
+ * nout multiples of 8; dweight (nout,k) fp32 is accumulated into (zero it first). */
+int ptv3_linear_wgrad(const void *x, const void *dout, int dtype, int64_t n, int k, int nout, float *dweight,
+                      void *stream);
+
 /* Backward of ptv3_segment_reduce (torch_scatter.segment_csr's, model.py:684-689): dsrc (n,c).
  * max / min: the gradient of a cluster goes to the first member in list order whose value equals
  * out; sum: to every member; mean: divided by the cluster size. Every row of src must belong to

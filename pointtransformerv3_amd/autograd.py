@@ -57,6 +57,33 @@ class SubMConv(torch.autograd.Function):
         return dfeat, dweight, dbias, None, None
 
 
+class Linear(torch.autograd.Function):
+    """x W^T + b for half-precision rows; weight and bias may be fp32 masters (autocast)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        w = weight.detach().to(x.dtype)
+        b = None if bias is None else bias.detach().to(x.dtype)
+        if ops.linear_rows_pays(x, w):
+            out = ops.linear_rows(x, w, b)
+        else:
+            out = torch.nn.functional.linear(x, w, b)
+        ctx.save_for_backward(x, weight)
+        ctx.bias_dtype = None if bias is None else bias.dtype
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        x, weight = ctx.saved_tensors
+        dout = dout.contiguous()
+        dx = dout @ weight.detach().to(dout.dtype) if ctx.needs_input_grad[0] else None
+        dw = ops.linear_wgrad(x, dout).to(weight.dtype) if ctx.needs_input_grad[1] else None
+        db = None
+        if ctx.bias_dtype is not None and ctx.needs_input_grad[2]:
+            db = dout.sum(0, dtype=torch.float32).to(ctx.bias_dtype)
+        return dx, dw, db
+
+
 class SegmentReduce(torch.autograd.Function):
     @staticmethod
     def forward(ctx, src, indices, idx_ptr, reduce):

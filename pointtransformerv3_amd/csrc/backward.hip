@@ -5,8 +5,13 @@
 //   the input gradient is the same convolution with the taps mirrored and the weight transposed
 //   (nbr[i][t] = j  <=>  nbr[j][V-1-t] = i), which the forward kernels already compute; what is new
 //   is   dW[co][t][ci] = sum_i dy[i][co] * x[nbr[i][t]][ci],   here per (tap, 64x64 weight block, range of
-//   voxels): both operands go through LDS 32 voxels at a time, every thread keeps a 4x4 block of sums
-//   in fp32 and adds it to the fp32 result with atomics at the end.
+//   voxels). Half precision: the valid (voxel, neighbour) pairs of the range are compacted into LDS, each wave
+//   takes 32 of them per step, writes both operands transposed into LDS (the MFMA wants the summed
+//   index contiguous per lane) and accumulates up to 2x2 tiles of v_mfma_f32_32x32x16; fp32 atomics at
+//   the end. fp32 and channel counts that are not multiples of 8: the same on plain FMAs, 4x4 sums per thread.
+// * nn.Linear's weight gradient dW = dy^T x (the qkv / proj / fc1 / fc2 / cpe Linears, model.py:366-367,
+//   :505-507, :553): the same kernel without the gather -- a reduction over several hundred thousand rows
+//   into a weight of a few dozen channels, which a general GEMM handles badly.
 // * torch_scatter.segment_csr (model.py:684-689): max / min send the gradient of a cluster to the first
 //   member that attains the value, sum copies it to every member, mean divides it by the cluster size.
 #include <hip/hip_bf16.h>
@@ -15,6 +20,9 @@
 #include "common.h"
 
 namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int WG_T = 64;     // weight block: WG_T output x WG_T input channels
 constexpr int WG_P = 32;     // voxels per staging step
@@ -86,6 +94,135 @@ __global__ __launch_bounds__(256) void conv_wgrad_kernel(const T* __restrict__ x
         }
 }
 
+// ---- d[m][tap][k] += sum over rows of a[row][m] * b[src(row)][k] on the matrix cores.
+// A work-group covers a 64 x 64 block of d and a range of rows; each of its four waves takes 32 rows per
+// step: 16-byte pieces of the two operands are written transposed into the wave's LDS tiles (rows of
+// OR_S halves, 16-byte chunks swizzled by the channel group so that the writes spread over the banks),
+// then read back as MFMA operands.
+constexpr int OR_S = 40;      // halves per LDS row: 32 summed rows + padding that spreads the operand reads
+constexpr int OR_C = 64;      // channels per block side
+constexpr int OR_LIST = 4096; // most rows per work-group with GATHER (the compacted pair list lives in LDS)
+
+template <typename T> struct Mfma16;
+template <> struct Mfma16<_Float16> {
+    typedef _Float16 v8 __attribute__((ext_vector_type(8)));
+    static __device__ __forceinline__ f32x16 mfma(v8 a, v8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
+template <> struct Mfma16<__bf16> {
+    typedef __bf16 v8 __attribute__((ext_vector_type(8)));
+    static __device__ __forceinline__ f32x16 mfma(v8 a, v8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+};
+
+// writes the 8 channels of piece (row r of the step, channel group g) transposed: tile[8 g + c][r]
+__device__ __forceinline__ void put_transposed(uint16_t* tile, int g, int r, u32x4 w) {
+    uint16_t* base = tile + (8 * g) * OR_S + (((r >> 3) ^ (g & 3)) << 3) + (r & 7);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        base[(2 * c) * OR_S] = (uint16_t)(w[c] & 0xffffu);
+        base[(2 * c + 1) * OR_S] = (uint16_t)(w[c] >> 16);
+    }
+}
+
+template <typename T, bool GATHER>
+__global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a, const T* __restrict__ b, int64_t n,
+                                                         int m_total, int k_total, const int32_t* __restrict__ nbr,
+                                                         int taps, int splits, int64_t rows_per_split,
+                                                         float* __restrict__ d) {
+    typedef typename Mfma16<T>::v8 v8;
+    __shared__ __align__(16) uint16_t tiles[4][2][OR_C * OR_S];
+    __shared__ int32_t list_a[GATHER ? OR_LIST : 1], list_b[GATHER ? OR_LIST : 1];
+    __shared__ int list_n;
+    const int tap = blockIdx.x / splits, split = blockIdx.x % splits;
+    const int m0 = blockIdx.y * OR_C, k0 = blockIdx.z * OR_C;
+    const int tm = min(2, (m_total - m0 + 31) / 32), tk = min(2, (k_total - k0 + 31) / 32);
+    const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
+    const int64_t r0 = (int64_t)split * rows_per_split;
+    const int64_t r1 = min(n, r0 + rows_per_split);
+    int count = (int)(r1 - r0);
+    if (GATHER) {
+        // compact the voxels of the range that have this neighbour: (output row, input row) pairs
+        if (tid == 0) list_n = 0;
+        __syncthreads();
+        const int32_t* nb = nbr + (int64_t)tap * n;
+        for (int64_t e = r0 + tid; e < r0 + ((r1 - r0 + 255) / 256) * 256; e += 256) {
+            const int32_t src = e < r1 ? nb[e] : -1;
+            const uint64_t mask = __ballot(src >= 0);
+            int base = 0;
+            if (lane == 0 && mask) base = atomicAdd(&list_n, __popcll(mask));
+            base = __shfl(base, 0, PTV3_WAVE);
+            if (src >= 0) {
+                const int pos = base + __popcll(mask & ((1ull << lane) - 1));
+                list_a[pos] = (int32_t)(e - r0);
+                list_b[pos] = src;
+            }
+        }
+        __syncthreads();
+        count = list_n;
+    }
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    uint16_t* ta = tiles[wave][0];
+    uint16_t* tb = tiles[wave][1];
+    const int g = lane & 7, rr = lane >> 3;   // piece: channel group g, rows rr + 8 j
+    const bool a_in = m0 + 8 * g < m_total, b_in = k0 + 8 * g < k_total;
+    const int col = lane & 31, hf = lane >> 5;
+    for (int base = 0; base < count; base += 4 * 32) {   // the same trip count for every wave
+        const int mine = base + wave * 32;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int r = rr + 8 * j;
+            const int idx = mine + r;
+            u32x4 wa = {0, 0, 0, 0}, wb = {0, 0, 0, 0};
+            if (idx < count) {
+                const int64_t ra = r0 + (GATHER ? list_a[idx] : idx);
+                const int64_t rb = GATHER ? (int64_t)list_b[idx] : ra;
+                if (a_in) wa = *(const u32x4*)(a + ra * m_total + m0 + 8 * g);
+                if (b_in) wb = *(const u32x4*)(b + rb * k_total + k0 + 8 * g);
+            }
+            put_transposed(ta, g, r, wa);
+            put_transposed(tb, g, r, wb);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            v8 fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int ch = 32 * i + col;
+                const int chunk = (2 * ks + hf) ^ ((ch >> 3) & 3);
+                fa[i] = __builtin_bit_cast(v8, *(const u32x4*)(ta + ch * OR_S + 8 * chunk));
+                fb[i] = __builtin_bit_cast(v8, *(const u32x4*)(tb + ch * OR_S + 8 * chunk));
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    if (i < tm && j < tk) acc[i][j] = Mfma16<T>::mfma(fa[i], fb[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+    // acc[i][j][v]: m = m0 + 32 i + 8 (v / 4) + 4 hf + v % 4, k = k0 + 32 j + col
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            if (i >= tm || j >= tk) continue;
+            const int k = k0 + 32 * j + col;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + 32 * i + 8 * (v >> 2) + 4 * hf + (v & 3);
+                if (m < m_total && k < k_total && acc[i][j][v] != 0.f)
+                    atomicAdd(d + ((int64_t)m * taps + tap) * k_total + k, acc[i][j][v]);
+            }
+        }
+}
+
 // one thread per (cluster, channel): walks the members in list order
 template <typename T>
 __global__ __launch_bounds__(256) void segment_reduce_bwd_kernel(const T* __restrict__ src, const T* __restrict__ out,
@@ -112,6 +249,31 @@ __global__ __launch_bounds__(256) void segment_reduce_bwd_kernel(const T* __rest
         const T v = (T)(op == 1 ? g / (float)(t - b) : g);
         for (int64_t j = b; j < t; ++j) dsrc[indices[j] * c + ch] = v;
     }
+}
+
+// rows of the reduction per work-group: enough work-groups to fill the part a few times, few enough that the
+// atomics at the end stay cheap next to the rows read
+void outer_split(int64_t n, int64_t blocks_per_split, int64_t cap, int64_t* splits, int64_t* rows) {
+    int64_t sp = ptv3_ceil_div(1024, blocks_per_split);
+    const int64_t most = ptv3_ceil_div(n, 512);
+    if (sp > most) sp = most;
+    if (sp < 1) sp = 1;
+    int64_t r = ptv3_ceil_div(ptv3_ceil_div(n, sp), 128) * 128;
+    if (cap > 0 && r > cap) r = cap;
+    *rows = r;
+    *splits = ptv3_ceil_div(n, r);
+}
+
+template <typename T, bool GATHER>
+int launch_outer(const void* a, const void* b, int64_t n, int m_total, int k_total, const int32_t* nbr, int taps,
+                 float* d, hipStream_t stream) {
+    const int64_t bm = ptv3_ceil_div(m_total, OR_C), bk = ptv3_ceil_div(k_total, OR_C);
+    int64_t splits, rows;
+    outer_split(n, (int64_t)taps * bm * bk, GATHER ? OR_LIST : 0, &splits, &rows);
+    if ((int64_t)taps * splits >= (1ll << 31)) return PTV3_EINVAL;
+    hipLaunchKernelGGL((outer_rows_kernel<T, GATHER>), dim3((unsigned)(taps * splits), (unsigned)bm, (unsigned)bk),
+                       dim3(256), 0, stream, (const T*)a, (const T*)b, n, m_total, k_total, nbr, taps, (int)splits, rows, d);
+    PTV3_RETURN_LAUNCH();
 }
 
 template <typename T>
@@ -149,9 +311,25 @@ extern "C" int ptv3_subm_conv_wgrad(const void* feat, const void* dout, int dtyp
     if (!feat || !dout || !nbr || !dweight) return PTV3_EINVAL;
     if ((int64_t)taps * ptv3_ceil_div(n, 256) >= (1ll << 31)) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
+    if (dtype != PTV3_F32 && cin % 8 == 0 && cout % 8 == 0) {
+        if (dtype == PTV3_F16) return launch_outer<_Float16, true>(dout, feat, n, cout, cin, nbr, taps, dweight, stream);
+        return launch_outer<__bf16, true>(dout, feat, n, cout, cin, nbr, taps, dweight, stream);
+    }
     if (dtype == PTV3_F16) return launch_wgrad<_Float16>(feat, dout, n, cin, cout, nbr, taps, dweight, stream);
     if (dtype == PTV3_BF16) return launch_wgrad<__bf16>(feat, dout, n, cin, cout, nbr, taps, dweight, stream);
     return launch_wgrad<float>(feat, dout, n, cin, cout, nbr, taps, dweight, stream);
+}
+
+extern "C" int ptv3_linear_wgrad(const void* x, const void* dout, int dtype, int64_t n, int k, int nout, float* dweight,
+                                 void* stream_) {
+    if (n < 0 || k < 1 || nout < 1) return PTV3_EINVAL;
+    if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
+    if (k % 8 != 0 || nout % 8 != 0) return PTV3_ESHAPE;
+    if (n == 0) return PTV3_OK;
+    if (!x || !dout || !dweight) return PTV3_EINVAL;
+    hipStream_t stream = (hipStream_t)stream_;
+    if (dtype == PTV3_F16) return launch_outer<_Float16, false>(dout, x, n, nout, k, nullptr, 1, dweight, stream);
+    return launch_outer<__bf16, false>(dout, x, n, nout, k, nullptr, 1, dweight, stream);
 }
 
 extern "C" int ptv3_segment_reduce_bwd(const void* src, const void* out, const void* dout, int dtype, int64_t n, int c,

@@ -289,7 +289,7 @@ class MLP(nn.Module):
         self.drop = nn.Dropout(drop)
 
     def forward(self, x):
-        return self.drop(self.fc2(self.drop(self.act(self.fc1(x)))))
+        return self.drop(ops.linear(self.drop(self.act(ops.linear(x, self.fc1))), self.fc2))
 
 
 class Block(PointModule):

@@ -775,6 +775,12 @@ def linear(x, mod, gelu=False):
     """mod(x) for an nn.Linear (followed by exact GELU if gelu), on whichever path is faster."""
     if wants_grad(x, mod.weight, mod.bias):
         w, b = mod.weight, mod.bias
+        xa = x.to(torch.get_autocast_dtype("cuda")) if (torch.is_autocast_enabled() and x.is_cuda) else x
+        if (xa.is_cuda and xa.dim() == 2 and xa.dtype in (torch.float16, torch.bfloat16)
+                and w.shape[0] % 8 == 0 and w.shape[1] % 8 == 0):
+            from .autograd import Linear
+            y = Linear.apply(xa, w, b)   # the weight gradient is a reduction over all rows: own kernel
+            return torch.nn.functional.gelu(y) if gelu else y
         if not torch.is_autocast_enabled() and w.dtype != x.dtype:
             w, b = w.to(x.dtype), None if b is None else b.to(x.dtype)
         y = torch.nn.functional.linear(x, w, b)
@@ -797,6 +803,20 @@ def linear_rows(x, weight, bias=None, gelu=False):
     _lib.check(lib.ptv3_linear_fwd(_ptr(x), _ptr(w), _ptr(b), _dtype_code(x), n, k, w.shape[0], int(bool(gelu)),
                                    _ptr(out), _stream()), "ptv3_linear_fwd")
     return out
+
+
+def linear_wgrad(x, dout):
+    """dout^T x in fp32, (Nout, K): the weight gradient of a Linear over many rows (fp16 / bf16)."""
+    _dev(x, dout)
+    lib = _lib.load()
+    x = x.contiguous()
+    dout = dout.to(x.dtype).contiguous()
+    n, k = x.shape
+    nout = dout.shape[1]
+    dw = torch.zeros((nout, k), dtype=torch.float32, device=x.device)
+    _lib.check(lib.ptv3_linear_wgrad(_ptr(x), _ptr(dout), _dtype_code(x), n, k, nout, _ptr(dw), _stream()),
+               "ptv3_linear_wgrad")
+    return dw
 
 
 def linear_bn_act(x, lin, bn, gelu):

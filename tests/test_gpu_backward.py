@@ -81,6 +81,28 @@ def test_subm_conv_backward_parity(dtype, cin, cout, ks, n):
     assert rel_err(conv.bias.grad, db) < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n,k,nout", [(5000, 32, 96), (70001, 128, 512), (333, 512, 64), (1, 8, 8), (20000, 72, 40)])
+def test_linear_backward_parity(dtype, n, k, nout):
+    """The Linear autograd function (row kernel forward, row-reduction kernel for the weight gradient)
+    against torch CPU autograd in fp32 on the same rounded inputs."""
+    from pointtransformerv3_amd.autograd import Linear
+    g = torch.Generator().manual_seed(n + k)
+    x = torch.randn(n, k, generator=g).to(dtype)
+    w = (torch.randn(nout, k, generator=g) / k ** 0.5).to(dtype)
+    b = torch.randn(nout, generator=g).to(dtype)
+    dout = torch.randn(n, nout, generator=g).to(dtype)
+    xr, wr, br = (t.float().requires_grad_(True) for t in (x, w, b))
+    torch.nn.functional.linear(xr, wr, br).backward(dout.float())
+    xg, wg, bg = (t.to(DEV).requires_grad_(True) for t in (x, w, b))
+    out = Linear.apply(xg, wg, bg)
+    out.backward(dout.to(DEV))
+    assert rel_err(out, torch.nn.functional.linear(x.float(), w.float(), b.float())) < TOL[dtype]
+    assert rel_err(xg.grad, xr.grad) < TOL[dtype]
+    assert rel_err(wg.grad, wr.grad) < TOL[dtype]
+    assert rel_err(bg.grad, br.grad) < TOL[dtype]
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("reduce", ["max", "min", "sum", "mean"])
 def test_segment_reduce_backward_parity(dtype, reduce):
