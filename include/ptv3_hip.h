@@ -270,6 +270,12 @@ int ptv3_segment_reduce(const void *src, int dtype, int64_t n, int c, const int6
 int ptv3_linear_wgrad(const void *x, const void *dout, int dtype, int64_t n, int k, int nout, float *dweight,
                       void *stream);
 
+/* Backward of nn.LayerNorm over rows (model.py:554, :557, :572 under autograd): x, dout, dx (n,c) and
+ * gamma (c,) of dtype, c in {32, 64, 128, 256, 512}; mean and rstd are recomputed from x.
+ * dgamma, dbeta (c,) fp32 are accumulated into (zero them first). */
+int ptv3_layer_norm_bwd(const void *x, const void *dout, const void *gamma, int dtype, int64_t n, int c,
+                        float eps, void *dx, float *dgamma, float *dbeta, void *stream);
+
 /* Backward of ptv3_segment_reduce (torch_scatter.segment_csr's, model.py:684-689): dsrc (n,c).
  * max / min: the gradient of a cluster goes to the first member in list order whose value equals
  * out; sum: to every member; mean: divided by the cluster size. Every row of src must belong to

@@ -84,6 +84,23 @@ class Linear(torch.autograd.Function):
         return dx, dw, db
 
 
+class LayerNorm(torch.autograd.Function):
+    """Row-wise LayerNorm in the dtype of x (statistics in fp32); mean and rstd are not kept, the backward
+    kernel recomputes them from x."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, eps):
+        ctx.save_for_backward(x, weight)
+        ctx.eps, ctx.bias_dtype = eps, bias.dtype
+        return ops.layer_norm(x, weight.detach(), bias.detach(), eps)
+
+    @staticmethod
+    def backward(ctx, dout):
+        x, weight = ctx.saved_tensors
+        dx, dw, db = ops.layer_norm_bwd(x, dout, weight.detach(), ctx.eps)
+        return dx, dw.to(weight.dtype), db.to(ctx.bias_dtype), None
+
+
 class SegmentReduce(torch.autograd.Function):
     @staticmethod
     def forward(ctx, src, indices, idx_ptr, reduce):

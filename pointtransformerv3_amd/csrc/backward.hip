@@ -12,6 +12,11 @@
 // * nn.Linear's weight gradient dW = dy^T x (the qkv / proj / fc1 / fc2 / cpe Linears, model.py:366-367,
 //   :505-507, :553): the same kernel without the gather -- a reduction over several hundred thousand rows
 //   into a weight of a few dozen channels, which a general GEMM handles badly.
+// * nn.LayerNorm (model.py:554, :557, :572): with xhat = (x - mean) * rstd and g = dy * gamma,
+//   dx = rstd * (g - mean(g) - xhat * mean(g * xhat)), dgamma = sum_rows dy * xhat, dbeta = sum_rows dy. Mean and
+//   rstd are recomputed from x (two passes over the registers, like the forward kernel); 8 channels per
+//   lane, a row per C / 8 lanes, column sums kept per lane over the rows and combined through LDS and
+//   one atomic per work-group and channel.
 // * torch_scatter.segment_csr (model.py:684-689): max / min send the gradient of a cluster to the first
 //   member that attains the value, sum copies it to every member, mean divides it by the cluster size.
 #include <hip/hip_bf16.h>
@@ -223,6 +228,133 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
         }
 }
 
+template <typename T> struct Row8;
+template <> struct Row8<float> {
+    static __device__ __forceinline__ void load(const float* p, float* v) {
+        const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    }
+    static __device__ __forceinline__ void store(float* p, const float* v) {
+        *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
+        *(float4*)(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+};
+template <typename H> struct Row8Half {
+    typedef H h8 __attribute__((ext_vector_type(8)));
+    static __device__ __forceinline__ void load(const H* p, float* v) {
+        const h8 a = *(const h8*)p;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (float)a[i];
+    }
+    static __device__ __forceinline__ void store(H* p, const float* v) {
+        h8 a;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) a[i] = (H)v[i];
+        *(h8*)p = a;
+    }
+};
+template <> struct Row8<_Float16> : Row8Half<_Float16> {};
+template <> struct Row8<__bf16> : Row8Half<__bf16> {};
+
+template <int LPR>
+__device__ __forceinline__ float row_sum(float v) {
+#pragma unroll
+    for (int off = 1; off < LPR; off <<= 1) v += __shfl_xor(v, off, PTV3_WAVE);
+    return v;
+}
+
+template <typename T, int LPR>
+__global__ __launch_bounds__(256) void layer_norm_bwd_kernel(const T* __restrict__ x, const T* __restrict__ dy,
+                                                             const T* __restrict__ gamma, int64_t n, float eps,
+                                                             T* __restrict__ dx, float* __restrict__ dgamma,
+                                                             float* __restrict__ dbeta) {
+    constexpr int C = LPR * 8, RPW = PTV3_WAVE / LPR;
+    __shared__ float part[2][4][C];
+    const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
+    const int sub = lane % LPR, rsub = lane / LPR;
+    float g[8], ag[8], ab[8];
+    Row8<T>::load(gamma + sub * 8, g);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { ag[i] = 0.f; ab[i] = 0.f; }
+    const int64_t stride = (int64_t)gridDim.x * 4 * RPW;
+    for (int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * RPW; row0 < n; row0 += stride) {
+        const int64_t row = row0 + rsub;
+        const bool valid = row < n;
+        float xv[8], gv[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { xv[i] = 0.f; gv[i] = 0.f; }
+        if (valid) {
+            Row8<T>::load(x + row * C + sub * 8, xv);
+            Row8<T>::load(dy + row * C + sub * 8, gv);
+        }
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s += xv[i];
+        const float mean = row_sum<LPR>(s) * (1.f / C);
+        float q = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { xv[i] -= mean; q = fmaf(xv[i], xv[i], q); }
+        const float rstd = rsqrtf(row_sum<LPR>(q) * (1.f / C) + eps);
+        float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            xv[i] *= rstd;                      // xhat
+            ag[i] = fmaf(gv[i], xv[i], ag[i]);  // rows beyond n carry zeros
+            ab[i] += gv[i];
+            gv[i] *= g[i];
+            s1 += gv[i];
+            s2 = fmaf(gv[i], xv[i], s2);
+        }
+        s1 = row_sum<LPR>(s1) * (1.f / C);
+        s2 = row_sum<LPR>(s2) * (1.f / C);
+        if (valid) {
+            float o[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o[i] = rstd * (gv[i] - s1 - xv[i] * s2);
+            Row8<T>::store(dx + row * C + sub * 8, o);
+        }
+    }
+    // column sums: over the rows a wave holds side by side, then over the waves, then one atomic per channel
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+#pragma unroll
+        for (int off = LPR; off < PTV3_WAVE; off <<= 1) {
+            ag[i] += __shfl_xor(ag[i], off, PTV3_WAVE);
+            ab[i] += __shfl_xor(ab[i], off, PTV3_WAVE);
+        }
+    }
+    if (rsub == 0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            part[0][wave][sub * 8 + i] = ag[i];
+            part[1][wave][sub * 8 + i] = ab[i];
+        }
+    }
+    __syncthreads();
+    for (int c = tid; c < 2 * C; c += 256) {
+        const int which = c / C, ch = c % C;
+        const float v = part[which][0][ch] + part[which][1][ch] + part[which][2][ch] + part[which][3][ch];
+        atomicAdd((which ? dbeta : dgamma) + ch, v);
+    }
+}
+
+template <typename T>
+int launch_ln_bwd(const void* x, const void* dy, const void* gamma, int64_t n, int c, float eps, void* dx, float* dgamma,
+                  float* dbeta, hipStream_t stream) {
+    const int64_t rows_per_wg = 4 * (PTV3_WAVE / (c / 8));
+    int64_t grid = ptv3_ceil_div(n, rows_per_wg);
+    if (grid > 2048) grid = 2048;
+#define PTV3_LNB(L)                                                                                                   \
+    if (c == 8 * L) {                                                                                                 \
+        hipLaunchKernelGGL((layer_norm_bwd_kernel<T, L>), dim3((unsigned)grid), dim3(256), 0, stream, (const T*)x,    \
+                           (const T*)dy, (const T*)gamma, n, eps, (T*)dx, dgamma, dbeta);                             \
+        PTV3_RETURN_LAUNCH();                                                                                         \
+    }
+    PTV3_LNB(4) PTV3_LNB(8) PTV3_LNB(16) PTV3_LNB(32) PTV3_LNB(64)
+#undef PTV3_LNB
+    return PTV3_ESHAPE;
+}
+
 // one thread per (cluster, channel): walks the members in list order
 template <typename T>
 __global__ __launch_bounds__(256) void segment_reduce_bwd_kernel(const T* __restrict__ src, const T* __restrict__ out,
@@ -330,6 +462,19 @@ extern "C" int ptv3_linear_wgrad(const void* x, const void* dout, int dtype, int
     hipStream_t stream = (hipStream_t)stream_;
     if (dtype == PTV3_F16) return launch_outer<_Float16, false>(dout, x, n, nout, k, nullptr, 1, dweight, stream);
     return launch_outer<__bf16, false>(dout, x, n, nout, k, nullptr, 1, dweight, stream);
+}
+
+extern "C" int ptv3_layer_norm_bwd(const void* x, const void* dout, const void* gamma, int dtype, int64_t n, int c,
+                                   float eps, void* dx, float* dgamma, float* dbeta, void* stream_) {
+    if (n < 0 || c < 1) return PTV3_EINVAL;
+    if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
+    if (c != 32 && c != 64 && c != 128 && c != 256 && c != 512) return PTV3_ESHAPE;
+    if (n == 0) return PTV3_OK;
+    if (!x || !dout || !gamma || !dx || !dgamma || !dbeta) return PTV3_EINVAL;
+    hipStream_t stream = (hipStream_t)stream_;
+    if (dtype == PTV3_F16) return launch_ln_bwd<_Float16>(x, dout, gamma, n, c, eps, dx, dgamma, dbeta, stream);
+    if (dtype == PTV3_BF16) return launch_ln_bwd<__bf16>(x, dout, gamma, n, c, eps, dx, dgamma, dbeta, stream);
+    return launch_ln_bwd<float>(x, dout, gamma, n, c, eps, dx, dgamma, dbeta, stream);
 }
 
 extern "C" int ptv3_segment_reduce_bwd(const void* src, const void* out, const void* dout, int dtype, int64_t n, int c,

@@ -11,7 +11,7 @@ import torch
 import torch.nn as nn
 
 from . import ops
-from .autograd import SegmentReduce, UnpoolAdd
+from .autograd import LayerNorm as LayerNormFn, SegmentReduce, UnpoolAdd
 from .point import AttrDict, Point, offset2bincount
 from .sparse import SparseConvTensor, SubMConv3d, is_spconv_module
 
@@ -37,8 +37,11 @@ class LayerNorm(nn.LayerNorm):
     """nn.LayerNorm (same parameters and state_dict) evaluated by the row-wise HIP kernel."""
 
     def forward(self, x):
-        if (x.dim() != 2 or len(self.normalized_shape) != 1 or self.weight is None or self.bias is None
-                or ops.wants_grad(x, self.weight, self.bias)):
+        if x.dim() != 2 or len(self.normalized_shape) != 1 or self.weight is None or self.bias is None:
+            return super().forward(x)
+        if ops.wants_grad(x, self.weight, self.bias):
+            if x.is_cuda and x.shape[1] in ops.LAYER_NORM_BWD_CHANNELS:
+                return LayerNormFn.apply(x, self.weight, self.bias, self.eps)
             return super().forward(x)
         return ops.layer_norm(x, self.weight, self.bias, self.eps)
 

@@ -721,6 +721,24 @@ def layer_norm(x, weight, bias, eps=1e-5, residual=None, mode=0, weight2=None, b
     return out0 if mode < 2 else (out0, out1)
 
 
+LAYER_NORM_BWD_CHANNELS = (32, 64, 128, 256, 512)
+
+
+def layer_norm_bwd(x, dout, weight, eps=1e-5):
+    """(dx, dweight, dbias) of LayerNorm over the rows of x; dweight and dbias in fp32."""
+    _dev(x, dout, weight)
+    lib = _lib.load()
+    x = x.contiguous()
+    dout = dout.to(x.dtype).contiguous()
+    n, c = x.shape
+    dx = torch.empty_like(x)
+    dwb = torch.zeros((2, c), dtype=torch.float32, device=x.device)
+    _lib.check(lib.ptv3_layer_norm_bwd(_ptr(x), _ptr(dout), _ptr(weight.to(x.dtype).contiguous()), _dtype_code(x), n, c,
+                                       float(eps), _ptr(dx), _ptr(dwb[0]), _ptr(dwb[1]), _stream()),
+               "ptv3_layer_norm_bwd")
+    return dx, dwb[0], dwb[1]
+
+
 LINEAR_LN_CHANNELS = (128, 256)   # square Linear + LayerNorm(s) + residual in one kernel
 # where that kernel measured faster than Linear kernel + LayerNorm kernel on MI355X: at 128 channels
 # (146k rows: 35 us against 42-49); at 256 the C x C weights fill the LDS, four waves per CU remain

@@ -92,12 +92,33 @@ def test_linear_backward_parity(dtype, n, k, nout):
     w = (torch.randn(nout, k, generator=g) / k ** 0.5).to(dtype)
     b = torch.randn(nout, generator=g).to(dtype)
     dout = torch.randn(n, nout, generator=g).to(dtype)
-    xr, wr, br = (t.float().requires_grad_(True) for t in (x, w, b))
+    xr, wr, br = (t.float().clone().requires_grad_(True) for t in (x, w, b))
     torch.nn.functional.linear(xr, wr, br).backward(dout.float())
-    xg, wg, bg = (t.to(DEV).requires_grad_(True) for t in (x, w, b))
+    xg, wg, bg = (t.detach().to(DEV).requires_grad_(True) for t in (x, w, b))
     out = Linear.apply(xg, wg, bg)
     out.backward(dout.to(DEV))
     assert rel_err(out, torch.nn.functional.linear(x.float(), w.float(), b.float())) < TOL[dtype]
+    assert rel_err(xg.grad, xr.grad) < TOL[dtype]
+    assert rel_err(wg.grad, wr.grad) < TOL[dtype]
+    assert rel_err(bg.grad, br.grad) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n,c", [(1, 32), (4097, 32), (3000, 64), (2500, 128), (1111, 256), (700, 512)])
+def test_layer_norm_backward_parity(dtype, n, c):
+    from pointtransformerv3_amd.autograd import LayerNorm
+    g = torch.Generator().manual_seed(n + c)
+    x = (torch.randn(n, c, generator=g) * 2 + 0.5).to(dtype)
+    w = (torch.rand(c, generator=g) + 0.5).to(dtype)
+    b = torch.randn(c, generator=g).to(dtype)
+    dout = torch.randn(n, c, generator=g).to(dtype)
+    xr, wr, br = (t.float().clone().requires_grad_(True) for t in (x, w, b))
+    want = torch.nn.functional.layer_norm(xr, (c,), wr, br, 1e-5)
+    want.backward(dout.float())
+    xg, wg, bg = (t.detach().to(DEV).requires_grad_(True) for t in (x, w, b))
+    out = LayerNorm.apply(xg, wg, bg, 1e-5)
+    out.backward(dout.to(DEV))
+    assert rel_err(out, want) < TOL[dtype]
     assert rel_err(xg.grad, xr.grad) < TOL[dtype]
     assert rel_err(wg.grad, wr.grad) < TOL[dtype]
     assert rel_err(bg.grad, br.grad) < TOL[dtype]
