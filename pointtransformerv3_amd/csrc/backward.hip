@@ -118,13 +118,18 @@ template <> struct Mfma16<__bf16> {
     static __device__ __forceinline__ f32x16 mfma(v8 a, v8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
 };
 
-// writes the 8 channels of piece (row r of the step, channel group g) transposed: tile[8 g + c][r]
-__device__ __forceinline__ void put_transposed(uint16_t* tile, int g, int r, u32x4 w) {
-    uint16_t* base = tile + (8 * g) * OR_S + (((r >> 3) ^ (g & 3)) << 3) + (r & 7);
+// writes pieces of four consecutive rows 4 q .. 4 q + 3 (8 channels of group g each) transposed: per channel the
+// four halves are one 8-byte word at tile[8 g + c][4 q], chunks of 8 rows swizzled by the channel group
+__device__ __forceinline__ void put_transposed4(uint16_t* tile, int g, int q, const u32x4* w) {
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    uint16_t* base = tile + (8 * g) * OR_S + (((q >> 1) ^ (g & 3)) << 3) + ((q & 1) << 2);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        base[(2 * c) * OR_S] = (uint16_t)(w[c] & 0xffffu);
-        base[(2 * c + 1) * OR_S] = (uint16_t)(w[c] >> 16);
+    for (int p = 0; p < 4; ++p) {
+        // words w[j][p] hold channels (2 p, 2 p + 1) of row j
+        const u32x2 even = {__builtin_amdgcn_perm(w[1][p], w[0][p], 0x05040100u), __builtin_amdgcn_perm(w[3][p], w[2][p], 0x05040100u)};
+        const u32x2 odd = {__builtin_amdgcn_perm(w[1][p], w[0][p], 0x07060302u), __builtin_amdgcn_perm(w[3][p], w[2][p], 0x07060302u)};
+        *(u32x2*)(base + (2 * p) * OR_S) = even;
+        *(u32x2*)(base + (2 * p + 1) * OR_S) = odd;
     }
 }
 
@@ -174,25 +179,26 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
 
     uint16_t* ta = tiles[wave][0];
     uint16_t* tb = tiles[wave][1];
-    const int g = lane & 7, rr = lane >> 3;   // piece: channel group g, rows rr + 8 j
+    const int g = lane & 7, rq = lane >> 3;   // pieces: channel group g, rows 4 rq + j
     const bool a_in = m0 + 8 * g < m_total, b_in = k0 + 8 * g < k_total;
     const int col = lane & 31, hf = lane >> 5;
     for (int base = 0; base < count; base += 4 * 32) {   // the same trip count for every wave
         const int mine = base + wave * 32;
+        u32x4 wa[4], wb[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int r = rr + 8 * j;
-            const int idx = mine + r;
-            u32x4 wa = {0, 0, 0, 0}, wb = {0, 0, 0, 0};
+            const int idx = mine + 4 * rq + j;
+            wa[j] = (u32x4){0, 0, 0, 0};
+            wb[j] = (u32x4){0, 0, 0, 0};
             if (idx < count) {
                 const int64_t ra = r0 + (GATHER ? list_a[idx] : idx);
                 const int64_t rb = GATHER ? (int64_t)list_b[idx] : ra;
-                if (a_in) wa = *(const u32x4*)(a + ra * m_total + m0 + 8 * g);
-                if (b_in) wb = *(const u32x4*)(b + rb * k_total + k0 + 8 * g);
+                if (a_in) wa[j] = *(const u32x4*)(a + ra * m_total + m0 + 8 * g);
+                if (b_in) wb[j] = *(const u32x4*)(b + rb * k_total + k0 + 8 * g);
             }
-            put_transposed(ta, g, r, wa);
-            put_transposed(tb, g, r, wb);
         }
+        put_transposed4(ta, g, rq, wa);
+        put_transposed4(tb, g, rq, wb);
         __syncthreads();
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {

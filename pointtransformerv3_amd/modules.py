@@ -41,6 +41,8 @@ class LayerNorm(nn.LayerNorm):
             return super().forward(x)
         if ops.wants_grad(x, self.weight, self.bias):
             if x.is_cuda and x.shape[1] in ops.LAYER_NORM_BWD_CHANNELS:
+                if torch.is_autocast_enabled():
+                    x = x.float()   # autocast runs layer_norm in float and hands out a float result
                 return LayerNormFn.apply(x, self.weight, self.bias, self.eps)
             return super().forward(x)
         return ops.layer_norm(x, self.weight, self.bias, self.eps)
