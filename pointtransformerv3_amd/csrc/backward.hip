@@ -137,7 +137,7 @@ template <typename T, bool GATHER>
 __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a, const T* __restrict__ b, int64_t n,
                                                          int m_total, int k_total, const int32_t* __restrict__ nbr,
                                                          int taps, int splits, int64_t rows_per_split,
-                                                         float* __restrict__ d) {
+                                                         int64_t slab_stride, float* __restrict__ d) {
     typedef typename Mfma16<T>::v8 v8;
     __shared__ __align__(16) uint16_t tiles[4][2][OR_C * OR_S];
     __shared__ int32_t list_a[GATHER ? OR_LIST : 1], list_b[GATHER ? OR_LIST : 1];
@@ -218,20 +218,44 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
         }
         __syncthreads();
     }
-    // acc[i][j][v]: m = m0 + 32 i + 8 (v / 4) + 4 hf + v % 4, k = k0 + 32 j + col
+    // the four waves hold sums over different rows: add them up in LDS (the operand tiles are free now), then
+    // every thread stores 16 of the block's 64 x 64 values into this split's slab, without atomics.
+    // acc[i][j][v]: m = 32 i + 8 (v / 4) + 4 hf + v % 4, k = 32 j + col
+    float* sum = (float*)&tiles[0][0][0];   // 64 x 64 floats = 16 KB of the 40 KB
+    for (int w = 0; w < 4; ++w) {
+        if (wave == w) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            if (i >= tm || j >= tk) continue;
-            const int k = k0 + 32 * j + col;
+                for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int m = m0 + 32 * i + 8 * (v >> 2) + 4 * hf + (v & 3);
-                if (m < m_total && k < k_total && acc[i][j][v] != 0.f)
-                    atomicAdd(d + ((int64_t)m * taps + tap) * k_total + k, acc[i][j][v]);
-            }
+                    for (int v = 0; v < 16; ++v) {
+                        float* at = sum + (32 * i + 8 * (v >> 2) + 4 * hf + (v & 3)) * OR_C + 32 * j + col;
+                        *at = (w == 0 ? 0.f : *at) + acc[i][j][v];
+                    }
         }
+        __syncthreads();
+    }
+    float* slab = d + (int64_t)split * slab_stride;
+    for (int e = tid; e < OR_C * OR_C; e += 256) {
+        const int m = m0 + e / OR_C, k = k0 + e % OR_C;
+        if (m < m_total && k < k_total) slab[((int64_t)m * taps + tap) * k_total + k] = sum[e];
+    }
+}
+
+// out[i] = sum over the splits' slabs
+__global__ __launch_bounds__(256) void slab_sum_kernel(const float* __restrict__ slabs, int64_t count, int splits,
+                                                       float* __restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    float v = 0.f;
+    for (int s = 0; s < splits; ++s) v += slabs[(int64_t)s * count + i];
+    out[i] = v;
+}
+
+__global__ __launch_bounds__(256) void zero_kernel(float* __restrict__ out, int64_t count) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) out[i] = 0.f;
 }
 
 template <typename T> struct Row8;
@@ -389,11 +413,11 @@ __global__ __launch_bounds__(256) void segment_reduce_bwd_kernel(const T* __rest
     }
 }
 
-// rows of the reduction per work-group: enough work-groups to fill the part a few times, few enough that the
-// atomics at the end stay cheap next to the rows read
+// Rows of the reduction per work-group: enough work-groups to fill the part, but at least 1024 rows each so
+// that the 64 x 64 block a work-group hands in is small next to what it read.
 void outer_split(int64_t n, int64_t blocks_per_split, int64_t cap, int64_t* splits, int64_t* rows) {
     int64_t sp = ptv3_ceil_div(1024, blocks_per_split);
-    const int64_t most = ptv3_ceil_div(n, 512);
+    const int64_t most = ptv3_ceil_div(n, 1024);
     if (sp > most) sp = most;
     if (sp < 1) sp = 1;
     int64_t r = ptv3_ceil_div(ptv3_ceil_div(n, sp), 128) * 128;
@@ -402,15 +426,31 @@ void outer_split(int64_t n, int64_t blocks_per_split, int64_t cap, int64_t* spli
     *splits = ptv3_ceil_div(n, r);
 }
 
+template <bool GATHER>
+size_t outer_workspace(int64_t n, int m_total, int k_total, int taps) {
+    int64_t splits, rows;
+    outer_split(n, (int64_t)taps * ptv3_ceil_div(m_total, OR_C) * ptv3_ceil_div(k_total, OR_C), GATHER ? OR_LIST : 0,
+                &splits, &rows);
+    return splits > 1 ? ptv3_align256((size_t)splits * m_total * taps * k_total * sizeof(float)) : 0;
+}
+
+// d (m_total, taps, k_total) fp32 is written in full
 template <typename T, bool GATHER>
 int launch_outer(const void* a, const void* b, int64_t n, int m_total, int k_total, const int32_t* nbr, int taps,
-                 float* d, hipStream_t stream) {
+                 float* d, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     const int64_t bm = ptv3_ceil_div(m_total, OR_C), bk = ptv3_ceil_div(k_total, OR_C);
     int64_t splits, rows;
     outer_split(n, (int64_t)taps * bm * bk, GATHER ? OR_LIST : 0, &splits, &rows);
     if ((int64_t)taps * splits >= (1ll << 31)) return PTV3_EINVAL;
+    const int64_t count = (int64_t)m_total * taps * k_total;
+    if (splits > 1 && (!workspace || workspace_bytes < (size_t)splits * count * sizeof(float))) return PTV3_EWORKSPACE;
+    float* slabs = splits > 1 ? (float*)workspace : d;
     hipLaunchKernelGGL((outer_rows_kernel<T, GATHER>), dim3((unsigned)(taps * splits), (unsigned)bm, (unsigned)bk),
-                       dim3(256), 0, stream, (const T*)a, (const T*)b, n, m_total, k_total, nbr, taps, (int)splits, rows, d);
+                       dim3(256), 0, stream, (const T*)a, (const T*)b, n, m_total, k_total, nbr, taps, (int)splits, rows,
+                       count, slabs);
+    if (splits > 1)
+        hipLaunchKernelGGL(slab_sum_kernel, dim3((unsigned)ptv3_ceil_div(count, 256)), dim3(256), 0, stream,
+                           (const float*)slabs, count, (int)splits, d);
     PTV3_RETURN_LAUNCH();
 }
 
@@ -425,6 +465,8 @@ int launch_wgrad(const void* x, const void* dy, int64_t n, int cin, int cout, co
     if (splits < 1) splits = 1;
     const int64_t rows = ptv3_ceil_div(ptv3_ceil_div(n, splits), WG_P) * WG_P;
     splits = ptv3_ceil_div(n, rows);
+    const int64_t count = (int64_t)cout * taps * cin;
+    hipLaunchKernelGGL(zero_kernel, dim3((unsigned)ptv3_ceil_div(count, 256)), dim3(256), 0, stream, dw, count);
     hipLaunchKernelGGL(conv_wgrad_kernel<T>, dim3((unsigned)(taps * splits), (unsigned)ptv3_ceil_div(cout, WG_T),
                                                   (unsigned)ptv3_ceil_div(cin, WG_T)),
                        dim3(256), 0, stream, (const T*)x, (const T*)dy, n, cin, cout, nbr, taps, (int)splits, rows, dw);
@@ -441,33 +483,60 @@ int launch_segment_bwd(const void* src, const void* out, const void* dout, int c
 
 }  // namespace
 
+static bool wgrad_on_mfma(int dtype, int cin, int cout) {
+    return dtype != PTV3_F32 && cin % 8 == 0 && cout % 8 == 0;
+}
+
+extern "C" size_t ptv3_subm_conv_wgrad_workspace_bytes(int dtype, int64_t n, int cin, int cout, int taps) {
+    if (n < 1 || cin < 1 || cout < 1 || taps < 1 || !wgrad_on_mfma(dtype, cin, cout)) return 0;
+    return outer_workspace<true>(n, cout, cin, taps);
+}
+
 extern "C" int ptv3_subm_conv_wgrad(const void* feat, const void* dout, int dtype, int64_t n, int cin, int cout,
-                                    const int32_t* nbr, int taps, float* dweight, void* stream_) {
+                                    const int32_t* nbr, int taps, float* dweight, void* workspace,
+                                    size_t workspace_bytes, void* stream_) {
     if (n < 0 || cin < 1 || cout < 1 || taps < 1) return PTV3_EINVAL;
     if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
-    if (n == 0) return PTV3_OK;
-    if (!feat || !dout || !nbr || !dweight) return PTV3_EINVAL;
-    if ((int64_t)taps * ptv3_ceil_div(n, 256) >= (1ll << 31)) return PTV3_EINVAL;
+    if (!dweight) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
-    if (dtype != PTV3_F32 && cin % 8 == 0 && cout % 8 == 0) {
-        if (dtype == PTV3_F16) return launch_outer<_Float16, true>(dout, feat, n, cout, cin, nbr, taps, dweight, stream);
-        return launch_outer<__bf16, true>(dout, feat, n, cout, cin, nbr, taps, dweight, stream);
+    if (n == 0) {
+        const int64_t count = (int64_t)cout * taps * cin;
+        hipLaunchKernelGGL(zero_kernel, dim3((unsigned)ptv3_ceil_div(count, 256)), dim3(256), 0, stream, dweight, count);
+        PTV3_RETURN_LAUNCH();
+    }
+    if (!feat || !dout || !nbr) return PTV3_EINVAL;
+    if ((int64_t)taps * ptv3_ceil_div(n, 256) >= (1ll << 31)) return PTV3_EINVAL;
+    if (wgrad_on_mfma(dtype, cin, cout)) {
+        if (dtype == PTV3_F16)
+            return launch_outer<_Float16, true>(dout, feat, n, cout, cin, nbr, taps, dweight, workspace, workspace_bytes, stream);
+        return launch_outer<__bf16, true>(dout, feat, n, cout, cin, nbr, taps, dweight, workspace, workspace_bytes, stream);
     }
     if (dtype == PTV3_F16) return launch_wgrad<_Float16>(feat, dout, n, cin, cout, nbr, taps, dweight, stream);
     if (dtype == PTV3_BF16) return launch_wgrad<__bf16>(feat, dout, n, cin, cout, nbr, taps, dweight, stream);
     return launch_wgrad<float>(feat, dout, n, cin, cout, nbr, taps, dweight, stream);
 }
 
+extern "C" size_t ptv3_linear_wgrad_workspace_bytes(int64_t n, int k, int nout) {
+    if (n < 1 || k < 1 || nout < 1) return 0;
+    return outer_workspace<false>(n, nout, k, 1);
+}
+
 extern "C" int ptv3_linear_wgrad(const void* x, const void* dout, int dtype, int64_t n, int k, int nout, float* dweight,
-                                 void* stream_) {
+                                 void* workspace, size_t workspace_bytes, void* stream_) {
     if (n < 0 || k < 1 || nout < 1) return PTV3_EINVAL;
     if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
     if (k % 8 != 0 || nout % 8 != 0) return PTV3_ESHAPE;
-    if (n == 0) return PTV3_OK;
-    if (!x || !dout || !dweight) return PTV3_EINVAL;
+    if (!dweight) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
-    if (dtype == PTV3_F16) return launch_outer<_Float16, false>(dout, x, n, nout, k, nullptr, 1, dweight, stream);
-    return launch_outer<__bf16, false>(dout, x, n, nout, k, nullptr, 1, dweight, stream);
+    if (n == 0) {
+        const int64_t count = (int64_t)nout * k;
+        hipLaunchKernelGGL(zero_kernel, dim3((unsigned)ptv3_ceil_div(count, 256)), dim3(256), 0, stream, dweight, count);
+        PTV3_RETURN_LAUNCH();
+    }
+    if (!x || !dout) return PTV3_EINVAL;
+    if (dtype == PTV3_F16)
+        return launch_outer<_Float16, false>(dout, x, n, nout, k, nullptr, 1, dweight, workspace, workspace_bytes, stream);
+    return launch_outer<__bf16, false>(dout, x, n, nout, k, nullptr, 1, dweight, workspace, workspace_bytes, stream);
 }
 
 extern "C" int ptv3_layer_norm_bwd(const void* x, const void* dout, const void* gamma, int dtype, int64_t n, int c,

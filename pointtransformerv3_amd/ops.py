@@ -315,9 +315,11 @@ def subm_conv_wgrad(feat, dout, nbr):
     n, cin = feat.shape
     cout = dout.shape[1]
     taps = nbr.shape[0]
-    dw = torch.zeros((cout, taps, cin), dtype=torch.float32, device=feat.device)
+    dw = torch.empty((cout, taps, cin), dtype=torch.float32, device=feat.device)
+    nbytes = lib.ptv3_subm_conv_wgrad_workspace_bytes(_dtype_code(feat), n, cin, cout, taps)
+    ws = _ws(nbytes, feat.device) if nbytes else None
     _lib.check(lib.ptv3_subm_conv_wgrad(_ptr(feat), _ptr(dout), _dtype_code(feat), n, cin, cout, _ptr(nbr), taps,
-                                        _ptr(dw), _stream()), "ptv3_subm_conv_wgrad")
+                                        _ptr(dw), _ptr(ws), nbytes, _stream()), "ptv3_subm_conv_wgrad")
     return dw
 
 
@@ -831,9 +833,11 @@ def linear_wgrad(x, dout):
     dout = dout.to(x.dtype).contiguous()
     n, k = x.shape
     nout = dout.shape[1]
-    dw = torch.zeros((nout, k), dtype=torch.float32, device=x.device)
-    _lib.check(lib.ptv3_linear_wgrad(_ptr(x), _ptr(dout), _dtype_code(x), n, k, nout, _ptr(dw), _stream()),
-               "ptv3_linear_wgrad")
+    dw = torch.empty((nout, k), dtype=torch.float32, device=x.device)
+    nbytes = lib.ptv3_linear_wgrad_workspace_bytes(n, k, nout)
+    ws = _ws(nbytes, x.device) if nbytes else None
+    _lib.check(lib.ptv3_linear_wgrad(_ptr(x), _ptr(dout), _dtype_code(x), n, k, nout, _ptr(dw), _ptr(ws), nbytes,
+                                     _stream()), "ptv3_linear_wgrad")
     return dw
 
 
