@@ -51,7 +51,10 @@ class SubMConv(torch.autograd.Function):
             dfeat = module.convolve(sparse, dout, wt, None)[:, :cin].to(feat.dtype)
         if ctx.needs_input_grad[1]:
             nbr = sparse.neighbour_map(module.kernel_size, module.indice_key)
-            dweight = ops.subm_conv_wgrad(feat, dout, nbr).reshape(weight.shape).to(weight.dtype)
+            x = feat.detach()
+            if x.dtype != torch.float32 and cin % 8:
+                x = torch.nn.functional.pad(x, (0, -cin % 8))   # the matrix-core kernel reads channels 8 at a time
+            dweight = ops.subm_conv_wgrad(x, dout, nbr)[:, :, :cin].reshape(weight.shape).to(weight.dtype)
         if ctx.has_bias and ctx.needs_input_grad[2]:
             dbias = dout.sum(0, dtype=torch.float32).to(ctx.bias_dtype)
         return dfeat, dweight, dbias, None, None

@@ -243,14 +243,32 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
     }
 }
 
-// out[i] = sum over the splits' slabs
+// out[i] = sum over the splits' slabs: a work-group takes 32 neighbouring values, its 8 thread rows share
+// out the splits (four loads in flight each) and meet in LDS
 __global__ __launch_bounds__(256) void slab_sum_kernel(const float* __restrict__ slabs, int64_t count, int splits,
                                                        float* __restrict__ out) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= count) return;
-    float v = 0.f;
-    for (int s = 0; s < splits; ++s) v += slabs[(int64_t)s * count + i];
-    out[i] = v;
+    __shared__ float part[8][32];
+    const int e = threadIdx.x % 32, lane_s = threadIdx.x / 32;
+    const int64_t i = (int64_t)blockIdx.x * 32 + e;
+    float v0 = 0.f, v1 = 0.f, v2 = 0.f, v3 = 0.f;
+    if (i < count) {
+        int s = lane_s;
+        for (; s + 24 < splits; s += 32) {
+            v0 += slabs[(int64_t)s * count + i];
+            v1 += slabs[(int64_t)(s + 8) * count + i];
+            v2 += slabs[(int64_t)(s + 16) * count + i];
+            v3 += slabs[(int64_t)(s + 24) * count + i];
+        }
+        for (; s < splits; s += 8) v0 += slabs[(int64_t)s * count + i];
+    }
+    part[lane_s][e] = (v0 + v1) + (v2 + v3);
+    __syncthreads();
+    if (lane_s == 0 && i < count) {
+        float v = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v += part[k][e];
+        out[i] = v;
+    }
 }
 
 __global__ __launch_bounds__(256) void zero_kernel(float* __restrict__ out, int64_t count) {
@@ -449,7 +467,7 @@ int launch_outer(const void* a, const void* b, int64_t n, int m_total, int k_tot
                        dim3(256), 0, stream, (const T*)a, (const T*)b, n, m_total, k_total, nbr, taps, (int)splits, rows,
                        count, slabs);
     if (splits > 1)
-        hipLaunchKernelGGL(slab_sum_kernel, dim3((unsigned)ptv3_ceil_div(count, 256)), dim3(256), 0, stream,
+        hipLaunchKernelGGL(slab_sum_kernel, dim3((unsigned)ptv3_ceil_div(count, 32)), dim3(256), 0, stream,
                            (const float*)slabs, count, (int)splits, d);
     PTV3_RETURN_LAUNCH();
 }
