@@ -117,16 +117,26 @@ int ptv3_patch_attn_rpe_fwd(const float *qkv, int64_t n_rows, int channels, int 
                             const int32_t *grid_coord, const float *rpe_table, int pos_bnd, float *out,
                             void *stream);
 
+/* ptv3_patch_attn_fwd (fp16 / bf16) that also keeps what the backward pass needs: lse (heads, n_pad) fp32,
+ * lse[h][slot] = log2 of the sum over the slot's sequence of 2^(score * log2(e)) for every real slot
+ * (filler slots are left unwritten). n_pad = cu_seqlens[n_seq]. */
+int ptv3_patch_attn_fwd_lse(const void *qkv, int dtype, int64_t n_rows, int channels, int heads,
+                            const int32_t *slot_src, const int32_t *slot_dst, const int32_t *cu_seqlens,
+                            int64_t n_seq, int64_t max_seqlen, int64_t n_pad, float scale, void *out,
+                            float *lse, void *stream);
+
 /* Backward of ptv3_patch_attn_fwd: what autograd derives for model.py:456-484 (the backward of the
  * flash_attn_varlen_qkvpacked_func call at :476-482 and of the row gathers around it). out is the
  * forward result, dout its gradient (n_rows, C); dqkv (n_rows, 3*C) receives [dq | dk | dv] per row,
  * every element written. Filler slots take no gradient as queries; as keys their share is added to
- * the row they repeat. n_pad = cu_seqlens[n_seq], the number of slots. */
+ * the row they repeat. n_pad = cu_seqlens[n_seq], the number of slots. lse: what ptv3_patch_attn_fwd_lse
+ * wrote for the same inputs (fp16 / bf16 only), or NULL to have it recomputed. */
 size_t ptv3_patch_attn_bwd_workspace_bytes(int dtype, int64_t n_pad, int channels, int heads);
 int ptv3_patch_attn_bwd(const void *qkv, const void *out, const void *dout, int dtype, int64_t n_rows,
                         int channels, int heads, const int32_t *slot_src, const int32_t *slot_dst,
                         const int32_t *cu_seqlens, int64_t n_seq, int64_t max_seqlen, int64_t n_pad,
-                        float scale, void *dqkv, void *workspace, size_t workspace_bytes, void *stream);
+                        float scale, const float *lse, void *dqkv, void *workspace, size_t workspace_bytes,
+                        void *stream);
 
 /* spconv.SubMConv3d's index generation (call sites model.py:546-552, :767-774, tensor built
  * at :165-172). indices (n,4) int32 [batch,x,y,z], coordinates in [0, 65535];

@@ -10,15 +10,19 @@ from . import ops
 class PatchAttention(torch.autograd.Function):
     @staticmethod
     def forward(ctx, qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale):
-        out = ops.patch_attention(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale)
+        args = (num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale)
+        if qkv.dtype == torch.float32:
+            out, ctx.lse = ops.patch_attention(qkv, *args), None
+        else:
+            out, ctx.lse = ops.patch_attention_lse(qkv, *args)
         ctx.save_for_backward(qkv, out)
-        ctx.args = (num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale)
+        ctx.args = args
         return out
 
     @staticmethod
     def backward(ctx, dout):
         qkv, out = ctx.saved_tensors
-        return (ops.patch_attention_bwd(qkv, out, dout, *ctx.args),) + (None,) * 6
+        return (ops.patch_attention_bwd(qkv, out, dout, *ctx.args, lse=ctx.lse),) + (None,) * 6
 
 
 class SubMConv(torch.autograd.Function):

@@ -50,7 +50,7 @@ __device__ __forceinline__ int xcd_chunked_id(int bid, int total) {
 // SHIFT = true: scores arrive shifted by a running reference maximum that enters through the C
 // operand; the reference moves (and the accumulators are rescaled) only when a score exceeds it
 // by RESCALE_SLACK, which the per-step |q||k| bound rules out without looking at the scores.
-template <typename T, bool SHIFT>
+template <typename T, bool SHIFT, bool LSE>
 __device__ __forceinline__ f32x16 attend_tile(typename Half<T>::v8 qfrag, float qnorm, float kn_reg,
                                               const unsigned char* k_ptr, const unsigned char* v_ptr,
                                               int v_step, int n_pairs, int len, int hf) {
@@ -120,14 +120,18 @@ __device__ __forceinline__ f32x16 attend_tile(typename Half<T>::v8 qfrag, float 
         acc = Half<T>::mfma(__builtin_bit_cast(v8, vb0), __builtin_bit_cast(v8, (u32x4){pb[0], pb[1], pb[2], pb[3]}), acc);
         acc = Half<T>::mfma(__builtin_bit_cast(v8, vb1), __builtin_bit_cast(v8, (u32x4){pb[4], pb[5], pb[6], pb[7]}), acc);
     }
+    // result row 17 / 21 multiplies zeros: its register carries the reference maximum to the caller
+    if (SHIFT && LSE) acc[9] = m_ref;
     return acc;
 }
 
-template <typename T>
+// LSE: also write log2(sum_j 2^score_ij) of every real query, scores in log2 units (scale * log2(e) folded into
+// q), to lse[head * lse_stride + slot]: what the backward kernels need to rebuild the probabilities.
+template <typename T, bool LSE>
 __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
     const T* __restrict__ qkv, int channels, int heads, const int32_t* __restrict__ slot_src,
     const int32_t* __restrict__ slot_dst, const int32_t* __restrict__ cu_seqlens, int lds_keys,
-    float scale_log2e, T* __restrict__ out, int full_items, int split) {
+    float scale_log2e, T* __restrict__ out, int full_items, int split, float* __restrict__ lse, int64_t lse_stride) {
     typedef typename Half<T>::v8 v8;
     extern __shared__ __align__(16) unsigned char smem[];
     // K tile: lds_keys + 64 rows of 32 B (the last 64 are only ever prefetched). V^T tile: 16 rows
@@ -239,9 +243,9 @@ __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
 
         f32x16 acc;
         if (__ballot(qnorm * kn_all > Half<T>::plain_limit()) == 0)
-            acc = attend_tile<T, false>(qfrag, qnorm, kn_reg, k_base, v_base, v_step, n_pairs, len, hf);
+            acc = attend_tile<T, false, LSE>(qfrag, qnorm, kn_reg, k_base, v_base, v_step, n_pairs, len, hf);
         else
-            acc = attend_tile<T, true>(qfrag, qnorm, kn_reg, k_base, v_base, v_step, n_pairs, len, hf);
+            acc = attend_tile<T, true, LSE>(qfrag, qnorm, kn_reg, k_base, v_base, v_step, n_pairs, len, hf);
         // acc[v]: d = 8*(v/4) + 4*hf + v%4; acc[8] = sum of probabilities (row 16 / 20)
         if (dst >= 0) {
             const float inv = 1.f / acc[8];
@@ -250,6 +254,7 @@ __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
             u32x2 hi = {Half<T>::pack2(acc[4] * inv, acc[5] * inv), Half<T>::pack2(acc[6] * inv, acc[7] * inv)};
             *(u32x2*)o = lo;
             *(u32x2*)(o + 8) = hi;
+            if (LSE && hf == 0) lse[(int64_t)head * lse_stride + s0 + qi] = acc[9] + __builtin_amdgcn_logf(acc[8]);
         }
     }
 }
@@ -413,16 +418,16 @@ __global__ __launch_bounds__(F32_QB) void patch_attn_rpe_f32_kernel(
     }
 }
 
-template <typename T>
+template <typename T, bool LSE>
 int launch_half(const void* qkv, int channels, int heads, const int32_t* slot_src,
                 const int32_t* slot_dst, const int32_t* cu_seqlens, int64_t n_seq,
-                int64_t max_seqlen, float scale, void* out, hipStream_t stream) {
+                int64_t max_seqlen, float scale, void* out, float* lse, int64_t lse_stride, hipStream_t stream) {
     const int lds_keys = (int)((max_seqlen + 63) & ~63ll);
     // K (+ one prefetch-only step), V^T, per-step key norms (padded to 16 B), ones and zeros
     const size_t lds = (size_t)(lds_keys + 64) * 32 + (size_t)HD * (lds_keys * 2 + VT_PAD_BYTES) +
                        (size_t)(lds_keys / 64) * sizeof(float) + 12 + 192;
     if (lds > 160 * 1024) return PTV3_ESHAPE;
-    auto kern = patch_attn_half_kernel<T>;
+    auto kern = patch_attn_half_kernel<T, LSE>;
     static size_t lds_allowed = 0;   // per instantiation; raised monotonically
     if (lds > lds_allowed) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -454,7 +459,7 @@ int launch_half(const void* qkv, int channels, int heads, const int32_t* slot_sr
     if (split == 1) full = total;
     hipLaunchKernelGGL(kern, dim3((unsigned)(full + (total - full) * split)), dim3(ATT_THREADS), lds, stream,
                        (const T*)qkv, channels, heads, slot_src, slot_dst, cu_seqlens, lds_keys,
-                       scale_log2e, (T*)out, (int)full, (int)split);
+                       scale_log2e, (T*)out, (int)full, (int)split, lse, lse_stride);
     PTV3_RETURN_LAUNCH();
 }
 
@@ -472,17 +477,35 @@ extern "C" int ptv3_patch_attn_fwd(const void* qkv, int dtype, int64_t n_rows, i
     if (!qkv || !slot_src || !slot_dst || !cu_seqlens || !out) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
     if (dtype == PTV3_F16)
-        return launch_half<_Float16>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
-                                     max_seqlen, scale, out, stream);
+        return launch_half<_Float16, false>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
+                                            max_seqlen, scale, out, nullptr, 0, stream);
     if (dtype == PTV3_BF16)
-        return launch_half<__bf16>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
-                                   max_seqlen, scale, out, stream);
+        return launch_half<__bf16, false>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
+                                          max_seqlen, scale, out, nullptr, 0, stream);
     const int q_blocks = (int)ptv3_ceil_div(max_seqlen, F32_QB);
     if (n_seq * heads * q_blocks >= (1ll << 31)) return PTV3_EINVAL;
     hipLaunchKernelGGL(patch_attn_f32_kernel, dim3((unsigned)(n_seq * heads * q_blocks)), dim3(F32_QB),
                        0, stream, (const float*)qkv, channels, heads, slot_src, slot_dst, cu_seqlens,
                        q_blocks, scale, (float*)out);
     PTV3_RETURN_LAUNCH();
+}
+
+extern "C" int ptv3_patch_attn_fwd_lse(const void* qkv, int dtype, int64_t n_rows, int channels, int heads,
+                                       const int32_t* slot_src, const int32_t* slot_dst, const int32_t* cu_seqlens,
+                                       int64_t n_seq, int64_t max_seqlen, int64_t n_pad, float scale, void* out,
+                                       float* lse, void* stream_) {
+    if (n_rows < 0 || n_seq < 0 || n_pad < 0 || channels < 1 || heads < 1 || max_seqlen < 1) return PTV3_EINVAL;
+    if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
+    if (channels % heads != 0 || channels / heads != HD) return PTV3_ESHAPE;
+    if (n_seq * heads >= (1ll << 31)) return PTV3_EINVAL;
+    if (n_seq == 0 || n_rows == 0) return PTV3_OK;
+    if (!qkv || !slot_src || !slot_dst || !cu_seqlens || !out || !lse) return PTV3_EINVAL;
+    hipStream_t stream = (hipStream_t)stream_;
+    if (dtype == PTV3_F16)
+        return launch_half<_Float16, true>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq, max_seqlen,
+                                           scale, out, lse, n_pad, stream);
+    return launch_half<__bf16, true>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq, max_seqlen, scale,
+                                     out, lse, n_pad, stream);
 }
 
 extern "C" int ptv3_patch_attn_rpe_fwd(const float* qkv, int64_t n_rows, int channels, int heads,

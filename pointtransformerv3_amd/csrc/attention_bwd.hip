@@ -83,12 +83,12 @@ __device__ __forceinline__ f32x16 splat16(float x) {
 }
 
 // ---- kernel 1: one work-group per (sequence, head), a wave per 32-query tile
-template <typename T>
+template <typename T, bool HAVE_LSE>
 __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_q_kernel(
     const T* __restrict__ qkv, const T* __restrict__ out, const T* __restrict__ dout, int channels, int heads,
     const int32_t* __restrict__ slot_src, const int32_t* __restrict__ slot_dst,
     const int32_t* __restrict__ cu_seqlens, int lds_keys, float scale, int64_t n_pad, T* __restrict__ dqkv,
-    float* __restrict__ lse_ws, float* __restrict__ d_ws) {
+    float* lse_ws, float* __restrict__ d_ws) {
     typedef typename Half<T>::v8 v8;
     extern __shared__ __align__(16) unsigned char smem[];
     // K rows, V rows, K^T, 96 B of zeros
@@ -149,41 +149,47 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_q_kernel(
         const v8 qfrag = __builtin_bit_cast(v8, scale8<T>(qreg, scale_log2e));   // scores in log2 units
         const v8 dofrag = __builtin_bit_cast(v8, doreg);
 
-        // first sweep: log-sum-exp of the query's score row (this lane sees half of the keys)
+        // log-sum-exp of the query's score row: kept by the forward pass, or a first sweep over the keys
+        // (this lane sees half of them)
         const f32x16 zero = splat16(0.f);
-        float m = -INFINITY, l = 0.f;
-        for (int kp = 0; kp < n_pairs; ++kp) {
-            const v8 k0 = __builtin_bit_cast(v8, *(const u32x4*)(k_base + (size_t)kp * 64 * 32));
-            const v8 k1 = __builtin_bit_cast(v8, *(const u32x4*)(k_base + (size_t)kp * 64 * 32 + 32 * 32));
-            f32x16 sa = Half<T>::mfma(k0, qfrag, zero);
-            f32x16 sb = Half<T>::mfma(k1, qfrag, zero);
-            if (ragged && kp == n_pairs - 1) {
+        float lse = 0.f;
+        if (HAVE_LSE) {
+            if (dst >= 0) lse = lse_ws[(int64_t)head * n_pad + s0 + qi];
+        } else {
+            float m = -INFINITY, l = 0.f;
+            for (int kp = 0; kp < n_pairs; ++kp) {
+                const v8 k0 = __builtin_bit_cast(v8, *(const u32x4*)(k_base + (size_t)kp * 64 * 32));
+                const v8 k1 = __builtin_bit_cast(v8, *(const u32x4*)(k_base + (size_t)kp * 64 * 32 + 32 * 32));
+                f32x16 sa = Half<T>::mfma(k0, qfrag, zero);
+                f32x16 sb = Half<T>::mfma(k1, qfrag, zero);
+                if (ragged && kp == n_pairs - 1) {
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int key = kp * 64 + 8 * (v >> 2) + 4 * hf + (v & 3);
-                    if (key >= len) sa[v] = -INFINITY;
-                    if (key + 32 >= len) sb[v] = -INFINITY;
+                    for (int v = 0; v < 16; ++v) {
+                        const int key = kp * 64 + 8 * (v >> 2) + 4 * hf + (v & 3);
+                        if (key >= len) sa[v] = -INFINITY;
+                        if (key + 32 >= len) sb[v] = -INFINITY;
+                    }
                 }
+                float mx = fmaxf(sa[0], sb[0]);
+#pragma unroll
+                for (int v = 1; v < 16; ++v) mx = fmaxf(mx, fmaxf(sa[v], sb[v]));
+                const float m_new = fmaxf(m, mx);
+                const float ms = m_new == -INFINITY ? 0.f : m_new;
+                float add = 0.f;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) add += __builtin_amdgcn_exp2f(sa[v] - ms) + __builtin_amdgcn_exp2f(sb[v] - ms);
+                l = l * __builtin_amdgcn_exp2f(m - ms) + add;
+                m = m_new;
             }
-            float mx = fmaxf(sa[0], sb[0]);
-#pragma unroll
-            for (int v = 1; v < 16; ++v) mx = fmaxf(mx, fmaxf(sa[v], sb[v]));
-            const float m_new = fmaxf(m, mx);
-            const float ms = m_new == -INFINITY ? 0.f : m_new;
-            float add = 0.f;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) add += __builtin_amdgcn_exp2f(sa[v] - ms) + __builtin_amdgcn_exp2f(sb[v] - ms);
-            l = l * __builtin_amdgcn_exp2f(m - ms) + add;
-            m = m_new;
+            {
+                const float mo = __shfl_xor(m, 32, PTV3_WAVE), lo = __shfl_xor(l, 32, PTV3_WAVE);
+                const float mm = fmaxf(m, mo);
+                const float ms = mm == -INFINITY ? 0.f : mm;
+                l = l * __builtin_amdgcn_exp2f(m - ms) + lo * __builtin_amdgcn_exp2f(mo - ms);
+                m = ms;
+            }
+            lse = dst >= 0 ? m + __builtin_amdgcn_logf(l) : 0.f;   // log2 units
         }
-        {
-            const float mo = __shfl_xor(m, 32, PTV3_WAVE), lo = __shfl_xor(l, 32, PTV3_WAVE);
-            const float mm = fmaxf(m, mo);
-            const float ms = mm == -INFINITY ? 0.f : mm;
-            l = l * __builtin_amdgcn_exp2f(m - ms) + lo * __builtin_amdgcn_exp2f(mo - ms);
-            m = ms;
-        }
-        const float lse = dst >= 0 ? m + __builtin_amdgcn_logf(l) : 0.f;   // log2 units
 
         // second sweep: P, dS and dQ^T
         const f32x16 c_lse = splat16(-lse), c_d = splat16(-dsum);
@@ -230,7 +236,7 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_q_kernel(
             *(u32x2*)o = lo;
             *(u32x2*)(o + 8) = hi;
             if (hf == 0) {
-                lse_ws[(int64_t)head * n_pad + s0 + qi] = lse;
+                if (!HAVE_LSE) lse_ws[(int64_t)head * n_pad + s0 + qi] = lse;
                 d_ws[(int64_t)head * n_pad + s0 + qi] = dsum;
             }
         }
@@ -590,19 +596,21 @@ BwdWs carve(void* base, int dtype, int64_t n_pad, int channels, int heads) {
 template <typename T>
 int launch_half_bwd(const void* qkv, const void* out, const void* dout, int channels, int heads,
                     const int32_t* slot_src, const int32_t* slot_dst, const int32_t* cu_seqlens, int64_t n_seq,
-                    int64_t max_seqlen, int64_t n_pad, float scale, void* dqkv, const BwdWs& ws, hipStream_t stream) {
+                    int64_t max_seqlen, int64_t n_pad, float scale, void* dqkv, const BwdWs& ws, float* lse,
+                    hipStream_t stream) {
     const int lds_keys = (int)((max_seqlen + 63) & ~63ll);
     const size_t t_bytes = (size_t)HD * (lds_keys * 2 + VT_PAD_BYTES);
     const size_t lds_q = 2 * (size_t)lds_keys * 32 + t_bytes + 96;
     const size_t lds_kv = 2 * (size_t)lds_keys * 32 + 2 * t_bytes + 2 * (size_t)lds_keys * sizeof(float) + 96;
     if (lds_q > 160 * 1024 || lds_kv > 160 * 1024) return PTV3_ESHAPE;
-    auto kq = attn_bwd_q_kernel<T>;
+    auto kq = lse ? attn_bwd_q_kernel<T, true> : attn_bwd_q_kernel<T, false>;
+    float* lse_buf = lse ? lse : ws.lse;
     auto kkv = attn_bwd_kv_kernel<T>;
-    static size_t allowed_q = 0, allowed_kv = 0;
-    if (lds_q > allowed_q) {
+    static size_t allowed_q[2] = {0, 0}, allowed_kv = 0;
+    if (lds_q > allowed_q[lse != nullptr]) {
         hipError_t e = hipFuncSetAttribute((const void*)kq, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_q);
         if (e != hipSuccess) return (int)e;
-        allowed_q = lds_q;
+        allowed_q[lse != nullptr] = lds_q;
     }
     if (lds_kv > allowed_kv) {
         hipError_t e = hipFuncSetAttribute((const void*)kkv, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_kv);
@@ -611,9 +619,9 @@ int launch_half_bwd(const void* qkv, const void* out, const void* dout, int chan
     }
     const unsigned grid = (unsigned)(n_seq * heads);
     hipLaunchKernelGGL(kq, dim3(grid), dim3(BWD_THREADS), lds_q, stream, (const T*)qkv, (const T*)out, (const T*)dout,
-                       channels, heads, slot_src, slot_dst, cu_seqlens, lds_keys, scale, n_pad, (T*)dqkv, ws.lse, ws.d);
+                       channels, heads, slot_src, slot_dst, cu_seqlens, lds_keys, scale, n_pad, (T*)dqkv, lse_buf, ws.d);
     hipLaunchKernelGGL(kkv, dim3(grid), dim3(BWD_THREADS), lds_kv, stream, (const T*)qkv, (const T*)dout, channels,
-                       heads, slot_src, slot_dst, cu_seqlens, lds_keys, scale, n_pad, ws.lse, ws.d, (T*)dqkv,
+                       heads, slot_src, slot_dst, cu_seqlens, lds_keys, scale, n_pad, lse_buf, ws.d, (T*)dqkv,
                        (T*)ws.fill);
     const int64_t items = n_pad * (2 * channels / 8);
     hipLaunchKernelGGL(attn_bwd_fill_kernel<T>, dim3((unsigned)ptv3_ceil_div(items, 256)), dim3(256), 0, stream,
@@ -631,7 +639,8 @@ extern "C" size_t ptv3_patch_attn_bwd_workspace_bytes(int dtype, int64_t n_pad, 
 extern "C" int ptv3_patch_attn_bwd(const void* qkv, const void* out, const void* dout, int dtype, int64_t n_rows,
                                    int channels, int heads, const int32_t* slot_src, const int32_t* slot_dst,
                                    const int32_t* cu_seqlens, int64_t n_seq, int64_t max_seqlen, int64_t n_pad,
-                                   float scale, void* dqkv, void* workspace, size_t workspace_bytes, void* stream_) {
+                                   float scale, const float* lse, void* dqkv, void* workspace, size_t workspace_bytes,
+                                   void* stream_) {
     if (n_rows < 0 || n_seq < 0 || n_pad < 0 || channels < 1 || heads < 1 || max_seqlen < 1) return PTV3_EINVAL;
     if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
     if (channels % heads != 0 || channels / heads != HD) return PTV3_ESHAPE;
@@ -643,10 +652,10 @@ extern "C" int ptv3_patch_attn_bwd(const void* qkv, const void* out, const void*
     hipStream_t stream = (hipStream_t)stream_;
     if (dtype == PTV3_F16)
         return launch_half_bwd<_Float16>(qkv, out, dout, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
-                                         max_seqlen, n_pad, scale, dqkv, ws, stream);
+                                         max_seqlen, n_pad, scale, dqkv, ws, (float*)lse, stream);
     if (dtype == PTV3_BF16)
         return launch_half_bwd<__bf16>(qkv, out, dout, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
-                                       max_seqlen, n_pad, scale, dqkv, ws, stream);
+                                       max_seqlen, n_pad, scale, dqkv, ws, (float*)lse, stream);
     const int blocks = (int)ptv3_ceil_div(max_seqlen, F32_B);
     if (n_seq * heads * blocks >= (1ll << 31)) return PTV3_EINVAL;
     const unsigned grid = (unsigned)(n_seq * heads * blocks);

@@ -227,8 +227,26 @@ def patch_attention(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, 
     return out
 
 
-def patch_attention_bwd(qkv, out, dout, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale):
-    """Gradient of patch_attention with respect to qkv, (N, 3C) laid out [dq | dk | dv]."""
+def patch_attention_lse(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale):
+    """patch_attention (fp16 / bf16) that also returns the (heads, n_pad) log-sum-exp rows the backward uses."""
+    _dev(qkv, slot_src, slot_dst, cu_seqlens)
+    lib = _lib.load()
+    qkv = qkv.contiguous()
+    n, c3 = qkv.shape
+    c = c3 // 3
+    n_pad = slot_src.shape[0]
+    out = torch.empty((n, c), dtype=qkv.dtype, device=qkv.device)
+    lse = torch.empty((int(num_heads), n_pad), dtype=torch.float32, device=qkv.device)
+    _lib.check(lib.ptv3_patch_attn_fwd_lse(_ptr(qkv), _dtype_code(qkv), n, c, int(num_heads), _ptr(slot_src),
+                                           _ptr(slot_dst), _ptr(cu_seqlens), cu_seqlens.shape[0] - 1, int(max_seqlen),
+                                           n_pad, float(scale), _ptr(out), _ptr(lse), _stream()),
+               "ptv3_patch_attn_fwd_lse")
+    return out, lse
+
+
+def patch_attention_bwd(qkv, out, dout, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale, lse=None):
+    """Gradient of patch_attention with respect to qkv, (N, 3C) laid out [dq | dk | dv]; lse from
+    patch_attention_lse saves the backward kernel a sweep over the keys."""
     _dev(qkv, out, dout, slot_src, slot_dst, cu_seqlens)
     lib = _lib.load()
     qkv, out = qkv.contiguous(), out.contiguous()
@@ -242,7 +260,7 @@ def patch_attention_bwd(qkv, out, dout, num_heads, slot_src, slot_dst, cu_seqlen
     ws = _ws(nbytes, qkv.device)
     _lib.check(lib.ptv3_patch_attn_bwd(_ptr(qkv), _ptr(out), _ptr(dout), code, n, c, int(num_heads), _ptr(slot_src),
                                        _ptr(slot_dst), _ptr(cu_seqlens), cu_seqlens.shape[0] - 1, int(max_seqlen),
-                                       n_pad, float(scale), _ptr(dqkv), _ptr(ws), nbytes, _stream()),
+                                       n_pad, float(scale), _ptr(lse), _ptr(dqkv), _ptr(ws), nbytes, _stream()),
                "ptv3_patch_attn_bwd")
     return dqkv
 

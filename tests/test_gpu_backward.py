@@ -54,6 +54,30 @@ def test_attention_backward_parity(dtype, counts, patch):
         assert rel_err(x.grad[:, sl], want[:, sl]) < TOL[dtype], part
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_attention_backward_recomputes_lse_when_not_kept(dtype):
+    """The backward entry point without the forward's log-sum-exp rows: same result as with them."""
+    heads, patch, counts = 2, 128, [300, 77]
+    rng = np.random.default_rng(7)
+    g = torch.Generator().manual_seed(7)
+    n, C = sum(counts), heads * 16
+    offset = np.cumsum(counts).astype(np.int64)
+    order = np.concatenate([s + rng.permutation(c) for s, c in zip([0, counts[0]], counts)]).astype(np.int64)
+    inverse = np.empty(n, np.int64)
+    inverse[order] = np.arange(n)
+    o = ops()
+    gp, gu, gc = o.pad_index(to_dev(offset), offset.tolist(), patch)
+    src, dst = o.attn_slots(to_dev(order), to_dev(inverse), gp, gu)
+    qkv = torch.randn(n, 3 * C, generator=g).to(dtype).to(DEV)
+    dout = torch.randn(n, C, generator=g).to(dtype).to(DEV)
+    args = (heads, src, dst, gc, patch, 0.25)
+    out, lse = o.patch_attention_lse(qkv, *args)
+    assert torch.equal(out, o.patch_attention(qkv, *args))
+    kept = o.patch_attention_bwd(qkv, out, dout, *args, lse=lse)
+    redone = o.patch_attention_bwd(qkv, out, dout, *args)
+    assert rel_err(redone, kept.float().cpu()) < TOL[dtype]
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("cin,cout,ks,n", [(6, 32, 5, 1500), (32, 32, 3, 2000), (64, 64, 3, 3000), (128, 128, 3, 1200),
                                            (48, 80, 3, 700)])
