@@ -304,20 +304,34 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_kv_kernel(
     const unsigned char* dot_base = col < HD ? dot_lds + (size_t)col * t_stride + hf * 32 : zero_lds;
     const int t_step = col < HD ? 128 : 0;
 
-    for (int kt = wave; kt < n_ktiles; kt += BWD_WAVES) {
-        const int key = kt * 32 + col;
-        const bool valid = key < len;
-        int64_t row = 0;
-        int kdst = -1;
-        u32x4 kreg = {0, 0, 0, 0}, vreg = {0, 0, 0, 0};
-        if (valid) {
-            row = slot_src[s0 + key];
-            kdst = slot_dst[s0 + key];
-            kreg = *(const u32x4*)(qkv + row * row_stride + channels + head * HD + hf * 8);
-            vreg = *(const u32x4*)(qkv + row * row_stride + 2 * channels + head * HD + hf * 8);
+    // Two key tiles per sweep over the queries: the query-side operands of a step (Q and dO rows, their
+    // transposes, -lse and -D: 28 16-byte LDS reads) are fetched once and used for both, which halves the
+    // LDS traffic per MFMA -- with one tile the kernel is bound by LDS bandwidth.
+    for (int kt = wave; kt < n_ktiles; kt += 2 * BWD_WAVES) {
+        int key[2], kdst[2];
+        int64_t row[2];
+        bool valid[2];
+        v8 kfrag[2], vfrag[2];
+        f32x16 acc_v[2], acc_k[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            key[t] = (kt + t * BWD_WAVES) * 32 + col;
+            valid[t] = key[t] < len;
+            row[t] = 0;
+            kdst[t] = -1;
+            u32x4 kreg = {0, 0, 0, 0}, vreg = {0, 0, 0, 0};
+            if (valid[t]) {
+                row[t] = slot_src[s0 + key[t]];
+                kdst[t] = slot_dst[s0 + key[t]];
+                kreg = *(const u32x4*)(qkv + row[t] * row_stride + channels + head * HD + hf * 8);
+                vreg = *(const u32x4*)(qkv + row[t] * row_stride + 2 * channels + head * HD + hf * 8);
+            }
+            kfrag[t] = __builtin_bit_cast(v8, kreg);
+            vfrag[t] = __builtin_bit_cast(v8, vreg);
+            acc_v[t] = splat16(0.f);
+            acc_k[t] = splat16(0.f);
         }
-        const v8 kfrag = __builtin_bit_cast(v8, kreg), vfrag = __builtin_bit_cast(v8, vreg);
-        f32x16 acc_v = splat16(0.f), acc_k = splat16(0.f);
+        const bool two = kt + BWD_WAVES < n_ktiles;   // the same for every lane of the wave
         const unsigned char* qt_ptr = qt_base;
         const unsigned char* dot_ptr = dot_base;
         for (int st = 0; st < n_pairs; ++st) {
@@ -340,44 +354,55 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_kv_kernel(
                     cdb[4 * a + r] = db[r];
                 }
             }
-            const f32x16 sa = Half<T>::mfma(q0, kfrag, cla);    // S - lse, [query, this lane's key]
-            const f32x16 sb = Half<T>::mfma(q1, kfrag, clb);
-            const f32x16 da = Half<T>::mfma(g0, vfrag, cda);    // dP - D
-            const f32x16 db = Half<T>::mfma(g1, vfrag, cdb);
-            const u32x4 ga0 = *(const u32x4*)dot_ptr, ga1 = *(const u32x4*)(dot_ptr + 16);
-            const u32x4 gb0 = *(const u32x4*)(dot_ptr + 64), gb1 = *(const u32x4*)(dot_ptr + 80);
-            const u32x4 qa0 = *(const u32x4*)qt_ptr, qa1 = *(const u32x4*)(qt_ptr + 16);
-            const u32x4 qb0 = *(const u32x4*)(qt_ptr + 64), qb1 = *(const u32x4*)(qt_ptr + 80);
+            const v8 ga0 = __builtin_bit_cast(v8, *(const u32x4*)dot_ptr);
+            const v8 ga1 = __builtin_bit_cast(v8, *(const u32x4*)(dot_ptr + 16));
+            const v8 gb0 = __builtin_bit_cast(v8, *(const u32x4*)(dot_ptr + 64));
+            const v8 gb1 = __builtin_bit_cast(v8, *(const u32x4*)(dot_ptr + 80));
+            const v8 qa0 = __builtin_bit_cast(v8, *(const u32x4*)qt_ptr);
+            const v8 qa1 = __builtin_bit_cast(v8, *(const u32x4*)(qt_ptr + 16));
+            const v8 qb0 = __builtin_bit_cast(v8, *(const u32x4*)(qt_ptr + 64));
+            const v8 qb1 = __builtin_bit_cast(v8, *(const u32x4*)(qt_ptr + 80));
             dot_ptr += t_step;
             qt_ptr += t_step;
-            float pa[16], pb[16], dsa[16], dsb[16];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                pa[v] = __builtin_amdgcn_exp2f(sa[v]);
-                pb[v] = __builtin_amdgcn_exp2f(sb[v]);
-                dsa[v] = pa[v] * da[v];
-                dsb[v] = pb[v] * db[v];
+            for (int t = 0; t < 2; ++t) {
+                if (t == 1 && !two) break;
+                const f32x16 sa = Half<T>::mfma(q0, kfrag[t], cla);    // S - lse, [query, this lane's key]
+                const f32x16 sb = Half<T>::mfma(q1, kfrag[t], clb);
+                const f32x16 da = Half<T>::mfma(g0, vfrag[t], cda);    // dP - D
+                const f32x16 db = Half<T>::mfma(g1, vfrag[t], cdb);
+                float pa[16], pb[16], dsa[16], dsb[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    pa[v] = __builtin_amdgcn_exp2f(sa[v]);
+                    pb[v] = __builtin_amdgcn_exp2f(sb[v]);
+                    dsa[v] = pa[v] * da[v];
+                    dsb[v] = pb[v] * db[v];
+                }
+                acc_v[t] = Half<T>::mfma(ga0, pack8<T>(pa), acc_v[t]);
+                acc_v[t] = Half<T>::mfma(ga1, pack8<T>(pa + 8), acc_v[t]);
+                acc_v[t] = Half<T>::mfma(gb0, pack8<T>(pb), acc_v[t]);
+                acc_v[t] = Half<T>::mfma(gb1, pack8<T>(pb + 8), acc_v[t]);
+                acc_k[t] = Half<T>::mfma(qa0, pack8<T>(dsa), acc_k[t]);
+                acc_k[t] = Half<T>::mfma(qa1, pack8<T>(dsa + 8), acc_k[t]);
+                acc_k[t] = Half<T>::mfma(qb0, pack8<T>(dsb), acc_k[t]);
+                acc_k[t] = Half<T>::mfma(qb1, pack8<T>(dsb + 8), acc_k[t]);
             }
-            acc_v = Half<T>::mfma(__builtin_bit_cast(v8, ga0), pack8<T>(pa), acc_v);
-            acc_v = Half<T>::mfma(__builtin_bit_cast(v8, ga1), pack8<T>(pa + 8), acc_v);
-            acc_v = Half<T>::mfma(__builtin_bit_cast(v8, gb0), pack8<T>(pb), acc_v);
-            acc_v = Half<T>::mfma(__builtin_bit_cast(v8, gb1), pack8<T>(pb + 8), acc_v);
-            acc_k = Half<T>::mfma(__builtin_bit_cast(v8, qa0), pack8<T>(dsa), acc_k);
-            acc_k = Half<T>::mfma(__builtin_bit_cast(v8, qa1), pack8<T>(dsa + 8), acc_k);
-            acc_k = Half<T>::mfma(__builtin_bit_cast(v8, qb0), pack8<T>(dsb), acc_k);
-            acc_k = Half<T>::mfma(__builtin_bit_cast(v8, qb1), pack8<T>(dsb + 8), acc_k);
         }
-        if (valid) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            if (!valid[t]) continue;
             // a real slot owns its row of dqkv; a filler's share is parked per slot and added afterwards.
             // Q^T was staged times scale * log2(e): dK = scale * dS^T Q = (dS^T Q_staged) * ln 2
-            T* base = kdst >= 0 ? dqkv + row * row_stride + channels + head * HD + 4 * hf
-                                : fill + (int64_t)(s0 + key) * 2 * channels + head * HD + 4 * hf;
-            u32x2 lo = {Half<T>::pack2(acc_k[0] * LN2, acc_k[1] * LN2), Half<T>::pack2(acc_k[2] * LN2, acc_k[3] * LN2)};
-            u32x2 hi = {Half<T>::pack2(acc_k[4] * LN2, acc_k[5] * LN2), Half<T>::pack2(acc_k[6] * LN2, acc_k[7] * LN2)};
+            T* base = kdst[t] >= 0 ? dqkv + row[t] * row_stride + channels + head * HD + 4 * hf
+                                   : fill + (int64_t)(s0 + key[t]) * 2 * channels + head * HD + 4 * hf;
+            const f32x16 ak = acc_k[t], av = acc_v[t];
+            u32x2 lo = {Half<T>::pack2(ak[0] * LN2, ak[1] * LN2), Half<T>::pack2(ak[2] * LN2, ak[3] * LN2)};
+            u32x2 hi = {Half<T>::pack2(ak[4] * LN2, ak[5] * LN2), Half<T>::pack2(ak[6] * LN2, ak[7] * LN2)};
             *(u32x2*)base = lo;
             *(u32x2*)(base + 8) = hi;
-            lo = (u32x2){Half<T>::pack2(acc_v[0], acc_v[1]), Half<T>::pack2(acc_v[2], acc_v[3])};
-            hi = (u32x2){Half<T>::pack2(acc_v[4], acc_v[5]), Half<T>::pack2(acc_v[6], acc_v[7])};
+            lo = (u32x2){Half<T>::pack2(av[0], av[1]), Half<T>::pack2(av[2], av[3])};
+            hi = (u32x2){Half<T>::pack2(av[4], av[5]), Half<T>::pack2(av[6], av[7])};
             *(u32x2*)(base + channels) = lo;
             *(u32x2*)(base + channels + 8) = hi;
         }
