@@ -287,6 +287,51 @@ def kernel_rooflines(path):
               file=sys.stderr)
 
 
+def training_step(args):
+    """Forward + backward + AdamW of the default model in training mode (batch-norm batch statistics,
+    stochastic depth 0.3, order shuffling) on the benchmark's input, cross-entropy against random labels
+    through a 13-class linear head. Not the headline metric: reported beside it."""
+    from pointtransformerv3_amd import PointTransformerV3
+    dev = "cuda:0"
+    dtype = getattr(torch, args.train)
+    torch.manual_seed(0)
+    model = PointTransformerV3().to(dev).train()
+    head = torch.nn.Linear(64, 13).to(dev)
+    opt = torch.optim.AdamW(list(model.parameters()) + list(head.parameters()), lr=1e-3)
+    d, feat = build_inputs(args.scenes, args.points, 4000)
+    n_points = len(feat)
+    data = dict(feat=torch.from_numpy(feat).to(dev), grid_coord=torch.from_numpy(d["grid_coord"]).to(dev),
+                offset=torch.from_numpy(d["offset"]).to(dev))
+    target = torch.randint(0, 13, (n_points,), device=dev)
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        with torch.autocast("cuda", dtype=dtype):
+            out = model(dict(data)).feat
+            loss = torch.nn.functional.cross_entropy(head(out).float(), target)
+        loss.backward()
+        opt.step()
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    assert torch.isfinite(loss.detach())
+    print(json.dumps({
+        "metric": "PTv3 training step points/sec (4x100k-pt scenes)", "value": n_points / (ms * 1e-3), "unit": "points/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": {"bfloat16": "bf16", "float16": "f16"}[args.train],
+        "data": "synthetic",
+        "config": {"workload": f"forward + backward + AdamW, default architecture in training mode, autocast, "
+                               f"{args.scenes} room scenes, {n_points} voxelised points, grid 0.02 m"},
+        "peak_memory_gib": torch.cuda.max_memory_allocated() / 2 ** 30}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -301,6 +346,9 @@ def main():
     ap.add_argument("--attention-config2", metavar="REPS", type=int, default=0,
                     help="only run the patch attention kernel at baseline config 2 (one 100k-point scene, C=512, 32 "
                          "heads, fp16) REPS times and print its rate: the command to put under rocprofv3 --pmc")
+    ap.add_argument("--train", metavar="DTYPE", default=None, choices=["bfloat16", "float16"],
+                    help="instead of the forward benchmark, time a training step (forward, backward, AdamW) of the "
+                         "same model and input under autocast to DTYPE and print its own JSON line")
     ap.add_argument("--kernels", metavar="PATH", default=None,
                     help="also measure every kernel alone against its roofline and write the table to PATH")
     args = ap.parse_args()
@@ -313,6 +361,9 @@ def main():
 
     if args.attention_config2 > 0:
         attention_config2(args.attention_config2)
+        return
+    if args.train:
+        training_step(args)
         return
     dev = "cuda:0"
     torch.manual_seed(0)

@@ -157,11 +157,12 @@ int ptv3_subm_conv_fwd(const void *feat, int dtype, int64_t n, int cin, const in
 
 /* Weight gradient of spconv.SubMConv3d (same call sites): dweight[co][t][ci] = sum over voxels i with
  * nbr[t][i] >= 0 of dout[i][co] * feat[nbr[t][i]][ci]. nbr is tap-major (taps, n); dweight
- * (cout, taps, cin) fp32, every element written. The input gradient needs no kernel of its own: it is
- * ptv3_subm_conv_fwd of dout with weight'[ci][t][co] = weight[co][taps-1-t][ci]. */
+ * (cout, taps, cin) fp32, every element written; dbias (cout,) fp32 or NULL: sum over the voxels of dout
+ * (fp16 / bf16 with cin and cout multiples of 8 only, PTV3_ESHAPE otherwise). The input gradient needs
+ * no kernel of its own: it is ptv3_subm_conv_fwd of dout with weight'[ci][t][co] = weight[co][taps-1-t][ci]. */
 size_t ptv3_subm_conv_wgrad_workspace_bytes(int dtype, int64_t n, int cin, int cout, int taps);
 int ptv3_subm_conv_wgrad(const void *feat, const void *dout, int dtype, int64_t n, int cin, int cout,
-                         const int32_t *nbr, int taps, float *dweight, void *workspace,
+                         const int32_t *nbr, int taps, float *dweight, float *dbias, void *workspace,
                          size_t workspace_bytes, void *stream);
 
 /* Sparse-pair form of the same convolution, for maps where most taps of most voxels are empty
@@ -278,10 +279,11 @@ int ptv3_segment_reduce(const void *src, int dtype, int64_t n, int c, const int6
 
 /* Weight gradient of nn.Linear (model.py:366-367, :505-507, :553, :633, :726-727 under autograd):
  * dweight[o][i] = sum over rows r of dout[r][o] * x[r][i]. x (n,k), dout (n,nout) fp16 / bf16 with k and
- * nout multiples of 8; dweight (nout,k) fp32, every element written. */
+ * nout multiples of 8; dweight (nout,k) fp32, every element written; dbias (nout,) fp32 or NULL: the
+ * column sums of dout, taken from the same pass over its rows. */
 size_t ptv3_linear_wgrad_workspace_bytes(int64_t n, int k, int nout);
 int ptv3_linear_wgrad(const void *x, const void *dout, int dtype, int64_t n, int k, int nout, float *dweight,
-                      void *workspace, size_t workspace_bytes, void *stream);
+                      float *dbias, void *workspace, size_t workspace_bytes, void *stream);
 
 /* Backward of nn.LayerNorm over rows (model.py:554, :557, :572 under autograd): x, dout, dx (n,c) and
  * gamma (c,) of dtype, c in {32, 64, 128, 256, 512}; mean and rstd are recomputed from x.

@@ -38,7 +38,7 @@ SIGNATURES = {
     "ptv3_kmap_build": (_i32, [_vp, _i64, _i32, _i32, _vp, _vp, _sz, _vp]),
     "ptv3_subm_conv_fwd": (_i32, [_vp, _i32, _i64, _i32, _vp, _i32, _i32, _vp, _vp, _i32, _vp, _vp]),
     "ptv3_subm_conv_wgrad_workspace_bytes": (_sz, [_i32, _i64, _i32, _i32, _i32]),
-    "ptv3_subm_conv_wgrad": (_i32, [_vp, _vp, _i32, _i64, _i32, _i32, _vp, _i32, _vp, _vp, _sz, _vp]),
+    "ptv3_subm_conv_wgrad": (_i32, [_vp, _vp, _i32, _i64, _i32, _i32, _vp, _i32, _vp, _vp, _vp, _sz, _vp]),
     "ptv3_conv_plan_workspace_bytes": (_sz, [_i64, _i32]),
     "ptv3_conv_plan_count": (_i32, [_vp, _i64, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
     "ptv3_conv_plan_fill": (_i32, [_vp, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
@@ -68,7 +68,7 @@ SIGNATURES = {
     "ptv3_linear_bn_act_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _f32, _i32, _i64, _i32, _i32, _i32, _vp, _vp]),
     "ptv3_layer_norm_bwd": (_i32, [_vp, _vp, _vp, _i32, _i64, _i32, _f32, _vp, _vp, _vp, _vp]),
     "ptv3_linear_wgrad_workspace_bytes": (_sz, [_i64, _i32, _i32]),
-    "ptv3_linear_wgrad": (_i32, [_vp, _vp, _i32, _i64, _i32, _i32, _vp, _vp, _sz, _vp]),
+    "ptv3_linear_wgrad": (_i32, [_vp, _vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
     "ptv3_linear_ln_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _f32, _vp, _vp, _vp]),
     "ptv3_mlp_fused": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _vp, _vp]),
     "ptv3_block_head_fused": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _vp, _f32, _vp, _vp, _i32, _i64, _i32,

@@ -58,8 +58,12 @@ class SubMConv(torch.autograd.Function):
             x = feat.detach()
             if x.dtype != torch.float32 and cin % 8:
                 x = torch.nn.functional.pad(x, (0, -cin % 8))   # the matrix-core kernel reads channels 8 at a time
-            dweight = ops.subm_conv_wgrad(x, dout, nbr)[:, :, :cin].reshape(weight.shape).to(weight.dtype)
-        if ctx.has_bias and ctx.needs_input_grad[2]:
+            want_bias = ctx.has_bias and ctx.needs_input_grad[2]
+            dw, db = ops.subm_conv_wgrad(x, dout, nbr, with_bias=True)
+            dweight = dw[:, :, :cin].reshape(weight.shape).to(weight.dtype)
+            if want_bias and db is not None:
+                dbias = db.to(ctx.bias_dtype)
+        if dbias is None and ctx.has_bias and ctx.needs_input_grad[2]:
             dbias = dout.sum(0, dtype=torch.float32).to(ctx.bias_dtype)
         return dfeat, dweight, dbias, None, None
 
@@ -84,11 +88,14 @@ class Linear(torch.autograd.Function):
         x, weight = ctx.saved_tensors
         dout = dout.contiguous()
         dx = dout @ weight.detach().to(dout.dtype) if ctx.needs_input_grad[0] else None
-        dw = ops.linear_wgrad(x, dout).to(weight.dtype) if ctx.needs_input_grad[1] else None
-        db = None
-        if ctx.bias_dtype is not None and ctx.needs_input_grad[2]:
-            db = dout.sum(0, dtype=torch.float32).to(ctx.bias_dtype)
-        return dx, dw, db
+        want_bias = ctx.bias_dtype is not None and ctx.needs_input_grad[2]
+        dw = db = None
+        if ctx.needs_input_grad[1]:
+            dw, db = ops.linear_wgrad(x, dout, with_bias=True)
+            dw = dw.to(weight.dtype)
+        if want_bias:
+            db = db.to(ctx.bias_dtype) if db is not None else dout.sum(0, dtype=torch.float32).to(ctx.bias_dtype)
+        return dx, dw, db if want_bias else None
 
 
 class LayerNorm(torch.autograd.Function):

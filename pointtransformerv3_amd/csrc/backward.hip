@@ -137,8 +137,10 @@ template <typename T, bool GATHER>
 __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a, const T* __restrict__ b, int64_t n,
                                                          int m_total, int k_total, const int32_t* __restrict__ nbr,
                                                          int taps, int splits, int64_t rows_per_split,
-                                                         int64_t slab_stride, float* __restrict__ d) {
+                                                         int64_t slab_stride, float* __restrict__ d,
+                                                         float* __restrict__ colsum) {
     typedef typename Mfma16<T>::v8 v8;
+    __shared__ float wave_cols[4][OR_C];
     __shared__ __align__(16) uint16_t tiles[4][2][OR_C * OR_S];
     __shared__ int32_t list_a[GATHER ? OR_LIST : 1], list_b[GATHER ? OR_LIST : 1];
     __shared__ int list_n;
@@ -182,6 +184,12 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
     const int g = lane & 7, rq = lane >> 3;   // pieces: channel group g, rows 4 rq + j
     const bool a_in = m0 + 8 * g < m_total, b_in = k0 + 8 * g < k_total;
     const int col = lane & 31, hf = lane >> 5;
+    // column sums of a (the bias gradient) ride along in the blocks that read each of a's rows exactly once:
+    // the first block along k, and with GATHER the centre tap, whose pairs are (i, i) for every voxel
+    const bool sum_cols = colsum != nullptr && blockIdx.z == 0 && (!GATHER || tap == taps / 2);
+    float cs[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) cs[c] = 0.f;
     for (int base = 0; base < count; base += 4 * 32) {   // the same trip count for every wave
         const int mine = base + wave * 32;
         u32x4 wa[4], wb[4];
@@ -195,6 +203,14 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
                 const int64_t rb = GATHER ? (int64_t)list_b[idx] : ra;
                 if (a_in) wa[j] = *(const u32x4*)(a + ra * m_total + m0 + 8 * g);
                 if (b_in) wb[j] = *(const u32x4*)(b + rb * k_total + k0 + 8 * g);
+            }
+        }
+        if (sum_cols) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const v8 h = __builtin_bit_cast(v8, wa[j]);
+#pragma unroll
+                for (int c = 0; c < 8; ++c) cs[c] += (float)h[c];
             }
         }
         put_transposed4(ta, g, rq, wa);
@@ -241,33 +257,50 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
         const int m = m0 + e / OR_C, k = k0 + e % OR_C;
         if (m < m_total && k < k_total) slab[((int64_t)m * taps + tap) * k_total + k] = sum[e];
     }
+    if (sum_cols) {   // the same for the whole work-group
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            cs[c] += __shfl_xor(cs[c], 8, PTV3_WAVE);
+            cs[c] += __shfl_xor(cs[c], 16, PTV3_WAVE);
+            cs[c] += __shfl_xor(cs[c], 32, PTV3_WAVE);
+        }
+        if (rq == 0) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) wave_cols[wave][8 * g + c] = cs[c];
+        }
+        __syncthreads();
+        if (tid < OR_C && m0 + tid < m_total)
+            colsum[(int64_t)split * slab_stride + m0 + tid] =
+                wave_cols[0][tid] + wave_cols[1][tid] + wave_cols[2][tid] + wave_cols[3][tid];
+    }
 }
 
-// out[i] = sum over the splits' slabs: a work-group takes 32 neighbouring values, its 8 thread rows share
+// out[i] = sum over the splits' slabs (of `stride` floats, the first `total` of them summed): a work-group takes 32 neighbouring values, its 8 thread rows share
 // out the splits (four loads in flight each) and meet in LDS
-__global__ __launch_bounds__(256) void slab_sum_kernel(const float* __restrict__ slabs, int64_t count, int splits,
-                                                       float* __restrict__ out) {
+__global__ __launch_bounds__(256) void slab_sum_kernel(const float* __restrict__ slabs, int64_t stride, int64_t total,
+                                                       int splits, float* __restrict__ out, int64_t first,
+                                                       float* __restrict__ out2) {
     __shared__ float part[8][32];
     const int e = threadIdx.x % 32, lane_s = threadIdx.x / 32;
     const int64_t i = (int64_t)blockIdx.x * 32 + e;
     float v0 = 0.f, v1 = 0.f, v2 = 0.f, v3 = 0.f;
-    if (i < count) {
+    if (i < total) {
         int s = lane_s;
         for (; s + 24 < splits; s += 32) {
-            v0 += slabs[(int64_t)s * count + i];
-            v1 += slabs[(int64_t)(s + 8) * count + i];
-            v2 += slabs[(int64_t)(s + 16) * count + i];
-            v3 += slabs[(int64_t)(s + 24) * count + i];
+            v0 += slabs[(int64_t)s * stride + i];
+            v1 += slabs[(int64_t)(s + 8) * stride + i];
+            v2 += slabs[(int64_t)(s + 16) * stride + i];
+            v3 += slabs[(int64_t)(s + 24) * stride + i];
         }
-        for (; s < splits; s += 8) v0 += slabs[(int64_t)s * count + i];
+        for (; s < splits; s += 8) v0 += slabs[(int64_t)s * stride + i];
     }
     part[lane_s][e] = (v0 + v1) + (v2 + v3);
     __syncthreads();
-    if (lane_s == 0 && i < count) {
+    if (lane_s == 0 && i < total) {
         float v = 0.f;
 #pragma unroll
         for (int k = 0; k < 8; ++k) v += part[k][e];
-        out[i] = v;
+        if (i < first) out[i] = v; else out2[i - first] = v;   // a slab's tail goes to the second result
     }
 }
 
@@ -449,26 +482,30 @@ size_t outer_workspace(int64_t n, int m_total, int k_total, int taps) {
     int64_t splits, rows;
     outer_split(n, (int64_t)taps * ptv3_ceil_div(m_total, OR_C) * ptv3_ceil_div(k_total, OR_C), GATHER ? OR_LIST : 0,
                 &splits, &rows);
-    return splits > 1 ? ptv3_align256((size_t)splits * m_total * taps * k_total * sizeof(float)) : 0;
+    return splits > 1 ? ptv3_align256((size_t)splits * ((size_t)m_total * taps * k_total + m_total) * sizeof(float)) : 0;
 }
 
-// d (m_total, taps, k_total) fp32 is written in full
+// d (m_total, taps, k_total) fp32 is written in full; so is colsum (m_total,) when given: the column sums of a
 template <typename T, bool GATHER>
 int launch_outer(const void* a, const void* b, int64_t n, int m_total, int k_total, const int32_t* nbr, int taps,
-                 float* d, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                 float* d, float* colsum, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     const int64_t bm = ptv3_ceil_div(m_total, OR_C), bk = ptv3_ceil_div(k_total, OR_C);
     int64_t splits, rows;
     outer_split(n, (int64_t)taps * bm * bk, GATHER ? OR_LIST : 0, &splits, &rows);
     if ((int64_t)taps * splits >= (1ll << 31)) return PTV3_EINVAL;
     const int64_t count = (int64_t)m_total * taps * k_total;
-    if (splits > 1 && (!workspace || workspace_bytes < (size_t)splits * count * sizeof(float))) return PTV3_EWORKSPACE;
+    const int64_t stride = count + m_total;
+    if (splits > 1 && (!workspace || workspace_bytes < (size_t)splits * stride * sizeof(float))) return PTV3_EWORKSPACE;
     float* slabs = splits > 1 ? (float*)workspace : d;
+    float* cols = !colsum ? nullptr : (splits > 1 ? slabs + count : colsum);
     hipLaunchKernelGGL((outer_rows_kernel<T, GATHER>), dim3((unsigned)(taps * splits), (unsigned)bm, (unsigned)bk),
                        dim3(256), 0, stream, (const T*)a, (const T*)b, n, m_total, k_total, nbr, taps, (int)splits, rows,
-                       count, slabs);
-    if (splits > 1)
-        hipLaunchKernelGGL(slab_sum_kernel, dim3((unsigned)ptv3_ceil_div(count, 32)), dim3(256), 0, stream,
-                           (const float*)slabs, count, (int)splits, d);
+                       stride, slabs, cols);
+    if (splits > 1) {
+        const int64_t total = colsum ? stride : count;
+        hipLaunchKernelGGL(slab_sum_kernel, dim3((unsigned)ptv3_ceil_div(total, 32)), dim3(256), 0, stream,
+                           (const float*)slabs, stride, total, (int)splits, d, count, colsum);
+    }
     PTV3_RETURN_LAUNCH();
 }
 
@@ -511,23 +548,25 @@ extern "C" size_t ptv3_subm_conv_wgrad_workspace_bytes(int dtype, int64_t n, int
 }
 
 extern "C" int ptv3_subm_conv_wgrad(const void* feat, const void* dout, int dtype, int64_t n, int cin, int cout,
-                                    const int32_t* nbr, int taps, float* dweight, void* workspace,
+                                    const int32_t* nbr, int taps, float* dweight, float* dbias, void* workspace,
                                     size_t workspace_bytes, void* stream_) {
     if (n < 0 || cin < 1 || cout < 1 || taps < 1) return PTV3_EINVAL;
     if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
     if (!dweight) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
+    if (dbias && !wgrad_on_mfma(dtype, cin, cout)) return PTV3_ESHAPE;   // the bias sum rides on the matrix-core kernel only
     if (n == 0) {
         const int64_t count = (int64_t)cout * taps * cin;
         hipLaunchKernelGGL(zero_kernel, dim3((unsigned)ptv3_ceil_div(count, 256)), dim3(256), 0, stream, dweight, count);
+        if (dbias) hipLaunchKernelGGL(zero_kernel, dim3((unsigned)ptv3_ceil_div(cout, 256)), dim3(256), 0, stream, dbias, (int64_t)cout);
         PTV3_RETURN_LAUNCH();
     }
     if (!feat || !dout || !nbr) return PTV3_EINVAL;
     if ((int64_t)taps * ptv3_ceil_div(n, 256) >= (1ll << 31)) return PTV3_EINVAL;
     if (wgrad_on_mfma(dtype, cin, cout)) {
         if (dtype == PTV3_F16)
-            return launch_outer<_Float16, true>(dout, feat, n, cout, cin, nbr, taps, dweight, workspace, workspace_bytes, stream);
-        return launch_outer<__bf16, true>(dout, feat, n, cout, cin, nbr, taps, dweight, workspace, workspace_bytes, stream);
+            return launch_outer<_Float16, true>(dout, feat, n, cout, cin, nbr, taps, dweight, dbias, workspace, workspace_bytes, stream);
+        return launch_outer<__bf16, true>(dout, feat, n, cout, cin, nbr, taps, dweight, dbias, workspace, workspace_bytes, stream);
     }
     if (dtype == PTV3_F16) return launch_wgrad<_Float16>(feat, dout, n, cin, cout, nbr, taps, dweight, stream);
     if (dtype == PTV3_BF16) return launch_wgrad<__bf16>(feat, dout, n, cin, cout, nbr, taps, dweight, stream);
@@ -540,7 +579,7 @@ extern "C" size_t ptv3_linear_wgrad_workspace_bytes(int64_t n, int k, int nout) 
 }
 
 extern "C" int ptv3_linear_wgrad(const void* x, const void* dout, int dtype, int64_t n, int k, int nout, float* dweight,
-                                 void* workspace, size_t workspace_bytes, void* stream_) {
+                                 float* dbias, void* workspace, size_t workspace_bytes, void* stream_) {
     if (n < 0 || k < 1 || nout < 1) return PTV3_EINVAL;
     if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
     if (k % 8 != 0 || nout % 8 != 0) return PTV3_ESHAPE;
@@ -549,12 +588,13 @@ extern "C" int ptv3_linear_wgrad(const void* x, const void* dout, int dtype, int
     if (n == 0) {
         const int64_t count = (int64_t)nout * k;
         hipLaunchKernelGGL(zero_kernel, dim3((unsigned)ptv3_ceil_div(count, 256)), dim3(256), 0, stream, dweight, count);
+        if (dbias) hipLaunchKernelGGL(zero_kernel, dim3((unsigned)ptv3_ceil_div(nout, 256)), dim3(256), 0, stream, dbias, (int64_t)nout);
         PTV3_RETURN_LAUNCH();
     }
     if (!x || !dout) return PTV3_EINVAL;
     if (dtype == PTV3_F16)
-        return launch_outer<_Float16, false>(dout, x, n, nout, k, nullptr, 1, dweight, workspace, workspace_bytes, stream);
-    return launch_outer<__bf16, false>(dout, x, n, nout, k, nullptr, 1, dweight, workspace, workspace_bytes, stream);
+        return launch_outer<_Float16, false>(dout, x, n, nout, k, nullptr, 1, dweight, dbias, workspace, workspace_bytes, stream);
+    return launch_outer<__bf16, false>(dout, x, n, nout, k, nullptr, 1, dweight, dbias, workspace, workspace_bytes, stream);
 }
 
 extern "C" int ptv3_layer_norm_bwd(const void* x, const void* dout, const void* gamma, int dtype, int64_t n, int c,

@@ -323,8 +323,9 @@ def subm_conv(feat, nbr, weight, bias=None, tap_major=False):
     return out
 
 
-def subm_conv_wgrad(feat, dout, nbr):
-    """Weight gradient (Cout, V, Cin) in fp32 of the submanifold convolution; nbr is the tap-major (V, N) map."""
+def subm_conv_wgrad(feat, dout, nbr, with_bias=False):
+    """Weight gradient (Cout, V, Cin) in fp32 of the submanifold convolution; nbr is the tap-major (V, N) map.
+    with_bias: also the bias gradient (Cout,), summed in the same pass where the kernel allows (None otherwise)."""
     _dev(feat, dout, nbr)
     lib = _lib.load()
     feat = feat.contiguous()
@@ -334,11 +335,13 @@ def subm_conv_wgrad(feat, dout, nbr):
     cout = dout.shape[1]
     taps = nbr.shape[0]
     dw = torch.empty((cout, taps, cin), dtype=torch.float32, device=feat.device)
+    fused = with_bias and feat.dtype != torch.float32 and cin % 8 == 0 and cout % 8 == 0
+    db = torch.empty(cout, dtype=torch.float32, device=feat.device) if fused else None
     nbytes = lib.ptv3_subm_conv_wgrad_workspace_bytes(_dtype_code(feat), n, cin, cout, taps)
     ws = _ws(nbytes, feat.device) if nbytes else None
     _lib.check(lib.ptv3_subm_conv_wgrad(_ptr(feat), _ptr(dout), _dtype_code(feat), n, cin, cout, _ptr(nbr), taps,
-                                        _ptr(dw), _ptr(ws), nbytes, _stream()), "ptv3_subm_conv_wgrad")
-    return dw
+                                        _ptr(dw), _ptr(db), _ptr(ws), nbytes, _stream()), "ptv3_subm_conv_wgrad")
+    return (dw, db) if with_bias else dw
 
 
 class ConvPlan:
@@ -843,8 +846,9 @@ def linear_rows(x, weight, bias=None, gelu=False):
     return out
 
 
-def linear_wgrad(x, dout):
-    """dout^T x in fp32, (Nout, K): the weight gradient of a Linear over many rows (fp16 / bf16)."""
+def linear_wgrad(x, dout, with_bias=False):
+    """dout^T x in fp32, (Nout, K): the weight gradient of a Linear over many rows (fp16 / bf16); with_bias:
+    also the column sums of dout (Nout,), the bias gradient, from the same pass."""
     _dev(x, dout)
     lib = _lib.load()
     x = x.contiguous()
@@ -852,11 +856,12 @@ def linear_wgrad(x, dout):
     n, k = x.shape
     nout = dout.shape[1]
     dw = torch.empty((nout, k), dtype=torch.float32, device=x.device)
+    db = torch.empty(nout, dtype=torch.float32, device=x.device) if with_bias else None
     nbytes = lib.ptv3_linear_wgrad_workspace_bytes(n, k, nout)
     ws = _ws(nbytes, x.device) if nbytes else None
-    _lib.check(lib.ptv3_linear_wgrad(_ptr(x), _ptr(dout), _dtype_code(x), n, k, nout, _ptr(dw), _ptr(ws), nbytes,
-                                     _stream()), "ptv3_linear_wgrad")
-    return dw
+    _lib.check(lib.ptv3_linear_wgrad(_ptr(x), _ptr(dout), _dtype_code(x), n, k, nout, _ptr(dw), _ptr(db), _ptr(ws),
+                                     nbytes, _stream()), "ptv3_linear_wgrad")
+    return (dw, db) if with_bias else dw
 
 
 def linear_bn_act(x, lin, bn, gelu):
