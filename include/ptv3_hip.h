@@ -286,10 +286,11 @@ int ptv3_linear_wgrad(const void *x, const void *dout, int dtype, int64_t n, int
                       float *dbias, void *workspace, size_t workspace_bytes, void *stream);
 
 /* Backward of nn.LayerNorm over rows (model.py:554, :557, :572 under autograd): x, dout, dx (n,c) and
- * gamma (c,) of dtype, c in {32, 64, 128, 256, 512}; mean and rstd are recomputed from x.
- * dgamma, dbeta (c,) fp32 are accumulated into (zero them first). */
-int ptv3_layer_norm_bwd(const void *x, const void *dout, const void *gamma, int dtype, int64_t n, int c,
-                        float eps, void *dx, float *dgamma, float *dbeta, void *stream);
+ * gamma (c,) of dtype, c in {32, 64, 128, 256, 512}; mean and rstd are recomputed from x. dres (n,c) or
+ * NULL is added to dx: the gradient that reaches x past the LayerNorm (the residual connection of
+ * model.py:589-604). dgamma, dbeta (c,) fp32 are accumulated into (zero them first). */
+int ptv3_layer_norm_bwd(const void *x, const void *dout, const void *gamma, const void *dres, int dtype,
+                        int64_t n, int c, float eps, void *dx, float *dgamma, float *dbeta, void *stream);
 
 /* Backward of ptv3_segment_reduce (torch_scatter.segment_csr's, model.py:684-689): dsrc (n,c).
  * max / min: the gradient of a cluster goes to the first member in list order whose value equals

@@ -115,6 +115,28 @@ class LayerNorm(torch.autograd.Function):
         return dx, dw.to(weight.dtype), db.to(ctx.bias_dtype), None
 
 
+class AddLayerNorm(torch.autograd.Function):
+    """s = skip + branch * mask, y = LayerNorm(s): a residual connection followed by the next pre-norm
+    (model.py:589-604; mask is the stochastic-depth factor per row, or None). Returns (s, y); the backward
+    kernel adds the gradient arriving at s to the LayerNorm's own, so autograd has nothing to accumulate."""
+
+    @staticmethod
+    def forward(ctx, skip, branch, mask, weight, bias, eps):
+        s = skip + branch if mask is None else torch.addcmul(skip, branch, mask)   # promotes like skip + branch * mask
+        y = ops.layer_norm(s, weight.detach(), bias.detach(), eps)
+        ctx.save_for_backward(s, weight, mask)
+        ctx.eps, ctx.dtypes = eps, (skip.dtype, branch.dtype, bias.dtype)
+        return s, y
+
+    @staticmethod
+    def backward(ctx, ds, dy):
+        s, weight, mask = ctx.saved_tensors
+        g, dw, db = ops.layer_norm_bwd(s, dy, weight.detach(), ctx.eps, dres=ds)
+        skip_dtype, branch_dtype, bias_dtype = ctx.dtypes
+        dbranch = g if mask is None else g * mask.to(g.dtype)
+        return g.to(skip_dtype), dbranch.to(branch_dtype), None, dw.to(weight.dtype), db.to(bias_dtype), None
+
+
 class SegmentReduce(torch.autograd.Function):
     @staticmethod
     def forward(ctx, src, indices, idx_ptr, reduce):

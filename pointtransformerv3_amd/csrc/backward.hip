@@ -346,9 +346,9 @@ __device__ __forceinline__ float row_sum(float v) {
 
 template <typename T, int LPR>
 __global__ __launch_bounds__(256) void layer_norm_bwd_kernel(const T* __restrict__ x, const T* __restrict__ dy,
-                                                             const T* __restrict__ gamma, int64_t n, float eps,
-                                                             T* __restrict__ dx, float* __restrict__ dgamma,
-                                                             float* __restrict__ dbeta) {
+                                                             const T* __restrict__ gamma, const T* __restrict__ dres,
+                                                             int64_t n, float eps, T* __restrict__ dx,
+                                                             float* __restrict__ dgamma, float* __restrict__ dbeta) {
     constexpr int C = LPR * 8, RPW = PTV3_WAVE / LPR;
     __shared__ float part[2][4][C];
     const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
@@ -389,9 +389,12 @@ __global__ __launch_bounds__(256) void layer_norm_bwd_kernel(const T* __restrict
         s1 = row_sum<LPR>(s1) * (1.f / C);
         s2 = row_sum<LPR>(s2) * (1.f / C);
         if (valid) {
-            float o[8];
+            float o[8], extra[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) o[i] = rstd * (gv[i] - s1 - xv[i] * s2);
+            for (int i = 0; i < 8; ++i) extra[i] = 0.f;
+            if (dres) Row8<T>::load(dres + row * C + sub * 8, extra);   // gradient arriving at x by another path
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o[i] = rstd * (gv[i] - s1 - xv[i] * s2) + extra[i];
             Row8<T>::store(dx + row * C + sub * 8, o);
         }
     }
@@ -420,15 +423,15 @@ __global__ __launch_bounds__(256) void layer_norm_bwd_kernel(const T* __restrict
 }
 
 template <typename T>
-int launch_ln_bwd(const void* x, const void* dy, const void* gamma, int64_t n, int c, float eps, void* dx, float* dgamma,
-                  float* dbeta, hipStream_t stream) {
+int launch_ln_bwd(const void* x, const void* dy, const void* gamma, const void* dres, int64_t n, int c, float eps,
+                  void* dx, float* dgamma, float* dbeta, hipStream_t stream) {
     const int64_t rows_per_wg = 4 * (PTV3_WAVE / (c / 8));
     int64_t grid = ptv3_ceil_div(n, rows_per_wg);
     if (grid > 2048) grid = 2048;
 #define PTV3_LNB(L)                                                                                                   \
     if (c == 8 * L) {                                                                                                 \
         hipLaunchKernelGGL((layer_norm_bwd_kernel<T, L>), dim3((unsigned)grid), dim3(256), 0, stream, (const T*)x,    \
-                           (const T*)dy, (const T*)gamma, n, eps, (T*)dx, dgamma, dbeta);                             \
+                           (const T*)dy, (const T*)gamma, (const T*)dres, n, eps, (T*)dx, dgamma, dbeta);             \
         PTV3_RETURN_LAUNCH();                                                                                         \
     }
     PTV3_LNB(4) PTV3_LNB(8) PTV3_LNB(16) PTV3_LNB(32) PTV3_LNB(64)
@@ -597,17 +600,17 @@ extern "C" int ptv3_linear_wgrad(const void* x, const void* dout, int dtype, int
     return launch_outer<__bf16, false>(dout, x, n, nout, k, nullptr, 1, dweight, dbias, workspace, workspace_bytes, stream);
 }
 
-extern "C" int ptv3_layer_norm_bwd(const void* x, const void* dout, const void* gamma, int dtype, int64_t n, int c,
-                                   float eps, void* dx, float* dgamma, float* dbeta, void* stream_) {
+extern "C" int ptv3_layer_norm_bwd(const void* x, const void* dout, const void* gamma, const void* dres, int dtype,
+                                   int64_t n, int c, float eps, void* dx, float* dgamma, float* dbeta, void* stream_) {
     if (n < 0 || c < 1) return PTV3_EINVAL;
     if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
     if (c != 32 && c != 64 && c != 128 && c != 256 && c != 512) return PTV3_ESHAPE;
     if (n == 0) return PTV3_OK;
     if (!x || !dout || !gamma || !dx || !dgamma || !dbeta) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
-    if (dtype == PTV3_F16) return launch_ln_bwd<_Float16>(x, dout, gamma, n, c, eps, dx, dgamma, dbeta, stream);
-    if (dtype == PTV3_BF16) return launch_ln_bwd<__bf16>(x, dout, gamma, n, c, eps, dx, dgamma, dbeta, stream);
-    return launch_ln_bwd<float>(x, dout, gamma, n, c, eps, dx, dgamma, dbeta, stream);
+    if (dtype == PTV3_F16) return launch_ln_bwd<_Float16>(x, dout, gamma, dres, n, c, eps, dx, dgamma, dbeta, stream);
+    if (dtype == PTV3_BF16) return launch_ln_bwd<__bf16>(x, dout, gamma, dres, n, c, eps, dx, dgamma, dbeta, stream);
+    return launch_ln_bwd<float>(x, dout, gamma, dres, n, c, eps, dx, dgamma, dbeta, stream);
 }
 
 extern "C" int ptv3_segment_reduce_bwd(const void* src, const void* out, const void* dout, int dtype, int64_t n, int c,

@@ -11,7 +11,7 @@ import torch
 import torch.nn as nn
 
 from . import ops
-from .autograd import LayerNorm as LayerNormFn, SegmentReduce, UnpoolAdd
+from .autograd import AddLayerNorm, LayerNorm as LayerNormFn, SegmentReduce, UnpoolAdd
 from .point import AttrDict, Point, offset2bincount
 from .sparse import SparseConvTensor, SubMConv3d, is_spconv_module
 
@@ -23,14 +23,19 @@ class DropPath(nn.Module):
         super().__init__()
         self.drop_prob, self.scale_by_keep = drop_prob, scale_by_keep
 
-    def forward(self, x):
+    def mask(self, x):
+        """The per-row factor (0 or 1 / keep) forward multiplies x by, or None when it is the identity."""
         if self.drop_prob == 0.0 or not self.training:
-            return x
+            return None
         keep = 1.0 - self.drop_prob
         mask = x.new_empty((x.shape[0],) + (1,) * (x.ndim - 1)).bernoulli_(keep)
         if keep > 0.0 and self.scale_by_keep:
             mask.div_(keep)
-        return x * mask
+        return mask
+
+    def forward(self, x):
+        mask = self.mask(x)
+        return x if mask is None else x * mask
 
 
 class LayerNorm(nn.LayerNorm):
@@ -385,7 +390,30 @@ class Block(PointModule):
         point.sparse_conv_feat = point.sparse_conv_feat.replace_feature(feat)
         return point
 
+    def _forward_training(self, point):
+        """Pre-norm block with plain LayerNorms under autograd: as _forward_modular, with each residual add
+        (and its stochastic-depth factor) taken together with the LayerNorm that follows it."""
+        ln1, ln2 = self.norm1[0], self.norm2[0]
+        drop = self.drop_path[0]
+        path_mask = drop.mask if isinstance(drop, DropPath) else (lambda x: None)
+        skip = point.feat
+        point = self.cpe(point)
+        feat, point.feat = AddLayerNorm.apply(skip, point.feat, None, ln1.weight, ln1.bias, ln1.eps)
+        point = self.attn(point)
+        feat, point.feat = AddLayerNorm.apply(feat, point.feat, path_mask(point.feat), ln2.weight, ln2.bias, ln2.eps)
+        point = self.mlp(point)
+        mask = path_mask(point.feat)
+        point.feat = feat + point.feat if mask is None else torch.addcmul(feat, point.feat, mask)
+        point.sparse_conv_feat = point.sparse_conv_feat.replace_feature(point.feat)
+        return point
+
     def _forward_modular(self, point):
+        if (self.pre_norm and point.feat.is_cuda and self.channels in ops.LAYER_NORM_BWD_CHANNELS
+                and all(type(m[0]) is LayerNorm and m[0].weight is not None and m[0].bias is not None
+                        for m in (self.norm1, self.norm2))
+                and isinstance(self.drop_path[0], (DropPath, nn.Identity))
+                and ops.wants_grad(point.feat, *self.parameters())):
+            return self._forward_training(point)
         skip = point.feat
         point = self.cpe(point)
         point.feat = skip + point.feat

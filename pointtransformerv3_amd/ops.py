@@ -747,17 +747,19 @@ def layer_norm(x, weight, bias, eps=1e-5, residual=None, mode=0, weight2=None, b
 LAYER_NORM_BWD_CHANNELS = (32, 64, 128, 256, 512)
 
 
-def layer_norm_bwd(x, dout, weight, eps=1e-5):
-    """(dx, dweight, dbias) of LayerNorm over the rows of x; dweight and dbias in fp32."""
-    _dev(x, dout, weight)
+def layer_norm_bwd(x, dout, weight, eps=1e-5, dres=None):
+    """(dx, dweight, dbias) of LayerNorm over the rows of x; dweight and dbias in fp32. dres: a gradient that
+    reaches x by another path (a residual connection), added to dx in the same pass."""
+    _dev(x, dout, weight, dres)
     lib = _lib.load()
     x = x.contiguous()
     dout = dout.to(x.dtype).contiguous()
+    dres = None if dres is None else dres.to(x.dtype).contiguous()
     n, c = x.shape
     dx = torch.empty_like(x)
     dwb = torch.zeros((2, c), dtype=torch.float32, device=x.device)
-    _lib.check(lib.ptv3_layer_norm_bwd(_ptr(x), _ptr(dout), _ptr(weight.to(x.dtype).contiguous()), _dtype_code(x), n, c,
-                                       float(eps), _ptr(dx), _ptr(dwb[0]), _ptr(dwb[1]), _stream()),
+    _lib.check(lib.ptv3_layer_norm_bwd(_ptr(x), _ptr(dout), _ptr(weight.to(x.dtype).contiguous()), _ptr(dres),
+                                       _dtype_code(x), n, c, float(eps), _ptr(dx), _ptr(dwb[0]), _ptr(dwb[1]), _stream()),
                "ptv3_layer_norm_bwd")
     return dx, dwb[0], dwb[1]
 

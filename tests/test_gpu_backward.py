@@ -148,6 +148,37 @@ def test_layer_norm_backward_parity(dtype, n, c):
     assert rel_err(bg.grad, br.grad) < TOL[dtype]
 
 
+@pytest.mark.parametrize("with_mask", [False, True])
+@pytest.mark.parametrize("skip_dtype,branch_dtype", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
+                                                     (torch.float16, torch.float16)])
+def test_add_layer_norm_backward_parity(skip_dtype, branch_dtype, with_mask):
+    """Residual add (+ per-row stochastic-depth factor) and the following LayerNorm as one autograd node: both
+    results and all four gradients against torch CPU autograd, with a gradient arriving at the sum as well."""
+    from pointtransformerv3_amd.autograd import AddLayerNorm
+    n, c = 3001, 64
+    g = torch.Generator().manual_seed(4)
+    skip = torch.randn(n, c, generator=g).to(skip_dtype)
+    branch = torch.randn(n, c, generator=g).to(branch_dtype)
+    mask = ((torch.rand(n, 1, generator=g) < 0.7).float() / 0.7).to(branch_dtype) if with_mask else None
+    w = (torch.rand(c, generator=g) + 0.5)
+    b = torch.randn(c, generator=g)
+    ds = torch.randn(n, c, generator=g)
+    dy = torch.randn(n, c, generator=g)
+    sr, br, wr, bb = (t.float().clone().requires_grad_(True) for t in (skip, branch, w, b))
+    s_want = sr + br * (mask.float() if with_mask else 1.0)
+    y_want = torch.nn.functional.layer_norm(s_want, (c,), wr, bb, 1e-5)
+    torch.autograd.backward([s_want, y_want], [ds, dy])
+    sg, bg, wg, bg2 = (t.detach().to(DEV).requires_grad_(True) for t in (skip, branch, w, b))
+    s_got, y_got = AddLayerNorm.apply(sg, bg, None if mask is None else mask.to(DEV), wg, bg2, 1e-5)
+    torch.autograd.backward([s_got, y_got], [ds.to(DEV).to(s_got.dtype), dy.to(DEV).to(y_got.dtype)])
+    tol = TOL[torch.promote_types(skip_dtype, branch_dtype)]
+    assert rel_err(s_got, s_want) < tol and rel_err(y_got, y_want) < tol
+    assert rel_err(sg.grad, sr.grad) < tol
+    assert rel_err(bg.grad, br.grad) < TOL[branch_dtype]
+    assert rel_err(wg.grad, wr.grad) < tol
+    assert rel_err(bg2.grad, bb.grad) < tol
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("reduce", ["max", "min", "sum", "mean"])
 def test_segment_reduce_backward_parity(dtype, reduce):
