@@ -285,12 +285,25 @@ size_t ptv3_linear_wgrad_workspace_bytes(int64_t n, int k, int nout);
 int ptv3_linear_wgrad(const void *x, const void *dout, int dtype, int64_t n, int k, int nout, float *dweight,
                       float *dbias, void *workspace, size_t workspace_bytes, void *stream);
 
-/* Backward of nn.LayerNorm over rows (model.py:554, :557, :572 under autograd): x, dout, dx (n,c) and
- * gamma (c,) of dtype, c in {32, 64, 128, 256, 512}; mean and rstd are recomputed from x. dres (n,c) or
- * NULL is added to dx: the gradient that reaches x past the LayerNorm (the residual connection of
- * model.py:589-604). dgamma, dbeta (c,) fp32 are accumulated into (zero them first). */
-int ptv3_layer_norm_bwd(const void *x, const void *dout, const void *gamma, const void *dres, int dtype,
-                        int64_t n, int c, float eps, void *dx, float *dgamma, float *dbeta, void *stream);
+/* nn.LayerNorm for training (model.py:554, :557, :572), with the residual connection in front of it taken
+ * into the same pass where there is one (model.py:589-604):
+ * sum = skip + branch * row_scale, y = LayerNorm(sum). skip (n,c) and row_scale (n,) -- the stochastic-depth
+ * factor per row, model.py:583 -- may be NULL; sum may be NULL when only y is wanted (then this is a plain
+ * LayerNorm of branch). Every tensor has its own dtype code (0 fp32, 1 fp16, 2 bf16): under autocast the
+ * residual stream is float and the branches half precision. gamma, beta (c,) of param_dtype.
+ * c in {32, 64, 128, 256, 512}. The statistics are taken from sum as rounded to sum_dtype. */
+int ptv3_add_layer_norm_fwd(const void *skip, int skip_dtype, const void *branch, int branch_dtype,
+                            const void *row_scale, int row_scale_dtype, const void *gamma, const void *beta,
+                            int param_dtype, int64_t n, int c, float eps, void *sum, int sum_dtype, void *y,
+                            int y_dtype, void *stream);
+
+/* Its backward: g = LayerNorm'(sum; dy) + dsum (dsum: the gradient that reaches sum past the LayerNorm, or
+ * NULL); dskip = g and dbranch = g * row_scale, either may be NULL, each in its own dtype. dgamma, dbeta
+ * (c,) fp32 are accumulated into (zero them first). */
+int ptv3_add_layer_norm_bwd(const void *sum, int sum_dtype, const void *dy, int dy_dtype, const void *dsum,
+                            int dsum_dtype, const void *row_scale, int row_scale_dtype, const void *gamma,
+                            int param_dtype, int64_t n, int c, float eps, void *dskip, int dskip_dtype,
+                            void *dbranch, int dbranch_dtype, float *dgamma, float *dbeta, void *stream);
 
 /* Backward of ptv3_segment_reduce (torch_scatter.segment_csr's, model.py:684-689): dsrc (n,c).
  * max / min: the gradient of a cluster goes to the first member in list order whose value equals

@@ -99,31 +99,32 @@ class Linear(torch.autograd.Function):
 
 
 class LayerNorm(torch.autograd.Function):
-    """Row-wise LayerNorm in the dtype of x (statistics in fp32); mean and rstd are not kept, the backward
-    kernel recomputes them from x."""
+    """Row-wise LayerNorm, statistics in fp32, result in out_dtype (x's when None: autocast asks for float
+    where the result joins the residual stream, half precision where only a Linear reads it). Mean and rstd
+    are not kept: the backward kernel recomputes them from x."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, eps):
+    def forward(ctx, x, weight, bias, eps, out_dtype=None):
         ctx.save_for_backward(x, weight)
         ctx.eps, ctx.bias_dtype = eps, bias.dtype
-        return ops.layer_norm(x, weight.detach(), bias.detach(), eps)
+        return ops.add_layer_norm(None, x, None, weight.detach(), bias.detach(), eps, out_dtype=out_dtype)[1]
 
     @staticmethod
     def backward(ctx, dout):
         x, weight = ctx.saved_tensors
-        dx, dw, db = ops.layer_norm_bwd(x, dout, weight.detach(), ctx.eps)
-        return dx, dw.to(weight.dtype), db.to(ctx.bias_dtype), None
+        _, dx, dw, db = ops.add_layer_norm_bwd(x, dout, None, None, weight.detach(), ctx.eps, branch_dtype=x.dtype)
+        return dx, dw.to(weight.dtype), db.to(ctx.bias_dtype), None, None
 
 
 class AddLayerNorm(torch.autograd.Function):
     """s = skip + branch * mask, y = LayerNorm(s): a residual connection followed by the next pre-norm
-    (model.py:589-604; mask is the stochastic-depth factor per row, or None). Returns (s, y); the backward
-    kernel adds the gradient arriving at s to the LayerNorm's own, so autograd has nothing to accumulate."""
+    (model.py:589-604; mask is the stochastic-depth factor per row, or None), one kernel each way. Returns
+    (s, y), y in out_dtype; the backward kernel adds the gradient arriving at s to the LayerNorm's own, so
+    autograd has nothing to accumulate, and writes each input's gradient in that input's dtype."""
 
     @staticmethod
-    def forward(ctx, skip, branch, mask, weight, bias, eps):
-        s = skip + branch if mask is None else torch.addcmul(skip, branch, mask)   # promotes like skip + branch * mask
-        y = ops.layer_norm(s, weight.detach(), bias.detach(), eps)
+    def forward(ctx, skip, branch, mask, weight, bias, eps, out_dtype=None):
+        s, y = ops.add_layer_norm(skip, branch, mask, weight.detach(), bias.detach(), eps, out_dtype=out_dtype)
         ctx.save_for_backward(s, weight, mask)
         ctx.eps, ctx.dtypes = eps, (skip.dtype, branch.dtype, bias.dtype)
         return s, y
@@ -131,10 +132,11 @@ class AddLayerNorm(torch.autograd.Function):
     @staticmethod
     def backward(ctx, ds, dy):
         s, weight, mask = ctx.saved_tensors
-        g, dw, db = ops.layer_norm_bwd(s, dy, weight.detach(), ctx.eps, dres=ds)
         skip_dtype, branch_dtype, bias_dtype = ctx.dtypes
-        dbranch = g if mask is None else g * mask.to(g.dtype)
-        return g.to(skip_dtype), dbranch.to(branch_dtype), None, dw.to(weight.dtype), db.to(bias_dtype), None
+        dskip, dbranch, dw, db = ops.add_layer_norm_bwd(s, dy, ds, mask, weight.detach(), ctx.eps,
+                                                        skip_dtype=skip_dtype if ctx.needs_input_grad[0] else None,
+                                                        branch_dtype=branch_dtype if ctx.needs_input_grad[1] else None)
+        return dskip, dbranch, None, dw.to(weight.dtype), db.to(bias_dtype), None, None
 
 
 class SegmentReduce(torch.autograd.Function):

@@ -16,7 +16,9 @@
 //   dx = rstd * (g - mean(g) - xhat * mean(g * xhat)), dgamma = sum_rows dy * xhat, dbeta = sum_rows dy. Mean and
 //   rstd are recomputed from x (two passes over the registers, like the forward kernel); 8 channels per
 //   lane, a row per C / 8 lanes, column sums kept per lane over the rows and combined through LDS and
-//   one atomic per work-group and channel.
+//   one atomic per work-group and channel. The training forward and backward kernels also take the
+//   residual add in front of the LayerNorm (model.py:589-604) and its stochastic-depth factor, and read
+//   and write every tensor in its own dtype (float residual stream, half-precision branches under autocast).
 // * torch_scatter.segment_csr (model.py:684-689): max / min send the gradient of a cluster to the first
 //   member that attains the value, sum copies it to every member, mean divides it by the cluster size.
 #include <hip/hip_bf16.h>
@@ -344,29 +346,120 @@ __device__ __forceinline__ float row_sum(float v) {
     return v;
 }
 
-template <typename T, int LPR>
-__global__ __launch_bounds__(256) void layer_norm_bwd_kernel(const T* __restrict__ x, const T* __restrict__ dy,
-                                                             const T* __restrict__ gamma, const T* __restrict__ dres,
-                                                             int64_t n, float eps, T* __restrict__ dx,
-                                                             float* __restrict__ dgamma, float* __restrict__ dbeta) {
+// 8 consecutive values in any of the three dtypes, as floats
+__device__ __forceinline__ void load8_any(const void* p, int dtype, int64_t off, float* v) {
+    if (dtype == PTV3_F32) Row8<float>::load((const float*)p + off, v);
+    else if (dtype == PTV3_F16) Row8<_Float16>::load((const _Float16*)p + off, v);
+    else Row8<__bf16>::load((const __bf16*)p + off, v);
+}
+__device__ __forceinline__ void store8_any(void* p, int dtype, int64_t off, const float* v) {
+    if (dtype == PTV3_F32) Row8<float>::store((float*)p + off, v);
+    else if (dtype == PTV3_F16) Row8<_Float16>::store((_Float16*)p + off, v);
+    else Row8<__bf16>::store((__bf16*)p + off, v);
+}
+__device__ __forceinline__ float load1_any(const void* p, int dtype, int64_t off) {
+    if (dtype == PTV3_F32) return ((const float*)p)[off];
+    if (dtype == PTV3_F16) return (float)((const _Float16*)p)[off];
+    return (float)((const __bf16*)p)[off];
+}
+__device__ __forceinline__ float round_any(float v, int dtype) {
+    if (dtype == PTV3_F32) return v;
+    if (dtype == PTV3_F16) return (float)(_Float16)v;
+    return (float)(__bf16)v;
+}
+
+// Tensors of one call, each with its own dtype: autocast mixes a float residual stream with half-precision
+// branches, and the kernels read and write each in place instead of going through cast passes.
+struct AnyRows {
+    const void* p;
+    int dtype;
+};
+struct AnyRowsOut {
+    void* p;
+    int dtype;
+};
+
+// sum = skip + branch * row_scale (skip and row_scale optional), y = LayerNorm(sum): 8 channels per lane, a row
+// per LPR lanes; the statistics are taken from the sum as stored, so the backward kernel sees the same numbers.
+template <int LPR>
+__global__ __launch_bounds__(256) void add_layer_norm_fwd_kernel(AnyRows skip, AnyRows branch, AnyRows row_scale,
+                                                                 AnyRows gamma, AnyRows beta, int64_t n, float eps,
+                                                                 AnyRowsOut sum, AnyRowsOut y) {
+    constexpr int C = LPR * 8, RPW = PTV3_WAVE / LPR;
+    const int wave = threadIdx.x / PTV3_WAVE, lane = threadIdx.x % PTV3_WAVE;
+    const int sub = lane % LPR, rsub = lane / LPR;
+    float g[8], b[8];
+    load8_any(gamma.p, gamma.dtype, sub * 8, g);
+    load8_any(beta.p, beta.dtype, sub * 8, b);
+    const int64_t stride = (int64_t)gridDim.x * 4 * RPW;
+    for (int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * RPW; row0 < n; row0 += stride) {
+        const int64_t row = row0 + rsub;
+        const bool valid = row < n;
+        const int64_t off = row * C + sub * 8;
+        float xv[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) xv[i] = 0.f;
+        if (valid) {
+            load8_any(branch.p, branch.dtype, off, xv);
+            if (row_scale.p) {
+                const float m = load1_any(row_scale.p, row_scale.dtype, row);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) xv[i] *= m;
+            }
+            if (skip.p) {
+                float sv[8];
+                load8_any(skip.p, skip.dtype, off, sv);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) xv[i] += sv[i];
+            }
+            if (sum.p) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) xv[i] = round_any(xv[i], sum.dtype);
+                store8_any(sum.p, sum.dtype, off, xv);
+            }
+        }
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s += xv[i];
+        const float mean = row_sum<LPR>(s) * (1.f / C);
+        float q = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { xv[i] -= mean; q = fmaf(xv[i], xv[i], q); }
+        const float rstd = rsqrtf(row_sum<LPR>(q) * (1.f / C) + eps);
+        if (valid) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) xv[i] = fmaf(xv[i] * rstd, g[i], b[i]);
+            store8_any(y.p, y.dtype, off, xv);
+        }
+    }
+}
+
+// g = LayerNorm'(sum, dy) + dsum (dsum optional); dskip = g, dbranch = g * row_scale, each optional and in its
+// own dtype; dgamma / dbeta accumulated in fp32. Mean and rstd are recomputed from sum.
+template <int LPR>
+__global__ __launch_bounds__(256) void add_layer_norm_bwd_kernel(AnyRows sum, AnyRows dy, AnyRows dsum, AnyRows row_scale,
+                                                                 AnyRows gamma, int64_t n, float eps, AnyRowsOut dskip,
+                                                                 AnyRowsOut dbranch, float* __restrict__ dgamma,
+                                                                 float* __restrict__ dbeta) {
     constexpr int C = LPR * 8, RPW = PTV3_WAVE / LPR;
     __shared__ float part[2][4][C];
     const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
     const int sub = lane % LPR, rsub = lane / LPR;
     float g[8], ag[8], ab[8];
-    Row8<T>::load(gamma + sub * 8, g);
+    load8_any(gamma.p, gamma.dtype, sub * 8, g);
 #pragma unroll
     for (int i = 0; i < 8; ++i) { ag[i] = 0.f; ab[i] = 0.f; }
     const int64_t stride = (int64_t)gridDim.x * 4 * RPW;
     for (int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * RPW; row0 < n; row0 += stride) {
         const int64_t row = row0 + rsub;
         const bool valid = row < n;
+        const int64_t off = row * C + sub * 8;
         float xv[8], gv[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) { xv[i] = 0.f; gv[i] = 0.f; }
         if (valid) {
-            Row8<T>::load(x + row * C + sub * 8, xv);
-            Row8<T>::load(dy + row * C + sub * 8, gv);
+            load8_any(sum.p, sum.dtype, off, xv);
+            load8_any(dy.p, dy.dtype, off, gv);
         }
         float s = 0.f;
 #pragma unroll
@@ -392,10 +485,18 @@ __global__ __launch_bounds__(256) void layer_norm_bwd_kernel(const T* __restrict
             float o[8], extra[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) extra[i] = 0.f;
-            if (dres) Row8<T>::load(dres + row * C + sub * 8, extra);   // gradient arriving at x by another path
+            if (dsum.p) load8_any(dsum.p, dsum.dtype, off, extra);   // gradient arriving at the sum by another path
 #pragma unroll
             for (int i = 0; i < 8; ++i) o[i] = rstd * (gv[i] - s1 - xv[i] * s2) + extra[i];
-            Row8<T>::store(dx + row * C + sub * 8, o);
+            if (dskip.p) store8_any(dskip.p, dskip.dtype, off, o);
+            if (dbranch.p) {
+                if (row_scale.p) {
+                    const float m = load1_any(row_scale.p, row_scale.dtype, row);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) o[i] *= m;
+                }
+                store8_any(dbranch.p, dbranch.dtype, off, o);
+            }
         }
     }
     // column sums: over the rows a wave holds side by side, then over the waves, then one atomic per channel
@@ -422,22 +523,40 @@ __global__ __launch_bounds__(256) void layer_norm_bwd_kernel(const T* __restrict
     }
 }
 
-template <typename T>
-int launch_ln_bwd(const void* x, const void* dy, const void* gamma, const void* dres, int64_t n, int c, float eps,
-                  void* dx, float* dgamma, float* dbeta, hipStream_t stream) {
+int64_t ln_grid(int64_t n, int c) {
     const int64_t rows_per_wg = 4 * (PTV3_WAVE / (c / 8));
-    int64_t grid = ptv3_ceil_div(n, rows_per_wg);
-    if (grid > 2048) grid = 2048;
+    const int64_t grid = ptv3_ceil_div(n, rows_per_wg);
+    return grid > 2048 ? 2048 : grid;
+}
+
+int launch_add_ln_fwd(AnyRows skip, AnyRows branch, AnyRows row_scale, AnyRows gamma, AnyRows beta, int64_t n, int c,
+                      float eps, AnyRowsOut sum, AnyRowsOut y, hipStream_t stream) {
+#define PTV3_LNF(L)                                                                                                   \
+    if (c == 8 * L) {                                                                                                 \
+        hipLaunchKernelGGL((add_layer_norm_fwd_kernel<L>), dim3((unsigned)ln_grid(n, c)), dim3(256), 0, stream, skip, \
+                           branch, row_scale, gamma, beta, n, eps, sum, y);                                           \
+        PTV3_RETURN_LAUNCH();                                                                                         \
+    }
+    PTV3_LNF(4) PTV3_LNF(8) PTV3_LNF(16) PTV3_LNF(32) PTV3_LNF(64)
+#undef PTV3_LNF
+    return PTV3_ESHAPE;
+}
+
+int launch_add_ln_bwd(AnyRows sum, AnyRows dy, AnyRows dsum, AnyRows row_scale, AnyRows gamma, int64_t n, int c, float eps,
+                      AnyRowsOut dskip, AnyRowsOut dbranch, float* dgamma, float* dbeta, hipStream_t stream) {
 #define PTV3_LNB(L)                                                                                                   \
     if (c == 8 * L) {                                                                                                 \
-        hipLaunchKernelGGL((layer_norm_bwd_kernel<T, L>), dim3((unsigned)grid), dim3(256), 0, stream, (const T*)x,    \
-                           (const T*)dy, (const T*)gamma, (const T*)dres, n, eps, (T*)dx, dgamma, dbeta);             \
+        hipLaunchKernelGGL((add_layer_norm_bwd_kernel<L>), dim3((unsigned)ln_grid(n, c)), dim3(256), 0, stream, sum,  \
+                           dy, dsum, row_scale, gamma, n, eps, dskip, dbranch, dgamma, dbeta);                        \
         PTV3_RETURN_LAUNCH();                                                                                         \
     }
     PTV3_LNB(4) PTV3_LNB(8) PTV3_LNB(16) PTV3_LNB(32) PTV3_LNB(64)
 #undef PTV3_LNB
     return PTV3_ESHAPE;
 }
+
+bool ln_dtype_ok(int dtype) { return dtype >= PTV3_F32 && dtype <= PTV3_BF16; }
+bool ln_channels_ok(int c) { return c == 32 || c == 64 || c == 128 || c == 256 || c == 512; }
 
 // one thread per (cluster, channel): walks the members in list order
 template <typename T>
@@ -600,17 +719,36 @@ extern "C" int ptv3_linear_wgrad(const void* x, const void* dout, int dtype, int
     return launch_outer<__bf16, false>(dout, x, n, nout, k, nullptr, 1, dweight, dbias, workspace, workspace_bytes, stream);
 }
 
-extern "C" int ptv3_layer_norm_bwd(const void* x, const void* dout, const void* gamma, const void* dres, int dtype,
-                                   int64_t n, int c, float eps, void* dx, float* dgamma, float* dbeta, void* stream_) {
+extern "C" int ptv3_add_layer_norm_fwd(const void* skip, int skip_dtype, const void* branch, int branch_dtype,
+                                       const void* row_scale, int row_scale_dtype, const void* gamma, const void* beta,
+                                       int param_dtype, int64_t n, int c, float eps, void* sum, int sum_dtype, void* y,
+                                       int y_dtype, void* stream_) {
     if (n < 0 || c < 1) return PTV3_EINVAL;
-    if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
-    if (c != 32 && c != 64 && c != 128 && c != 256 && c != 512) return PTV3_ESHAPE;
+    if (!ln_dtype_ok(skip_dtype) || !ln_dtype_ok(branch_dtype) || !ln_dtype_ok(row_scale_dtype) ||
+        !ln_dtype_ok(param_dtype) || !ln_dtype_ok(sum_dtype) || !ln_dtype_ok(y_dtype))
+        return PTV3_EINVAL;
+    if (!ln_channels_ok(c)) return PTV3_ESHAPE;
     if (n == 0) return PTV3_OK;
-    if (!x || !dout || !gamma || !dx || !dgamma || !dbeta) return PTV3_EINVAL;
-    hipStream_t stream = (hipStream_t)stream_;
-    if (dtype == PTV3_F16) return launch_ln_bwd<_Float16>(x, dout, gamma, dres, n, c, eps, dx, dgamma, dbeta, stream);
-    if (dtype == PTV3_BF16) return launch_ln_bwd<__bf16>(x, dout, gamma, dres, n, c, eps, dx, dgamma, dbeta, stream);
-    return launch_ln_bwd<float>(x, dout, gamma, dres, n, c, eps, dx, dgamma, dbeta, stream);
+    if (!branch || !gamma || !beta || !y) return PTV3_EINVAL;
+    return launch_add_ln_fwd({skip, skip_dtype}, {branch, branch_dtype}, {row_scale, row_scale_dtype},
+                             {gamma, param_dtype}, {beta, param_dtype}, n, c, eps, {sum, sum_dtype}, {y, y_dtype},
+                             (hipStream_t)stream_);
+}
+
+extern "C" int ptv3_add_layer_norm_bwd(const void* sum, int sum_dtype, const void* dy, int dy_dtype, const void* dsum,
+                                       int dsum_dtype, const void* row_scale, int row_scale_dtype, const void* gamma,
+                                       int param_dtype, int64_t n, int c, float eps, void* dskip, int dskip_dtype,
+                                       void* dbranch, int dbranch_dtype, float* dgamma, float* dbeta, void* stream_) {
+    if (n < 0 || c < 1) return PTV3_EINVAL;
+    if (!ln_dtype_ok(sum_dtype) || !ln_dtype_ok(dy_dtype) || !ln_dtype_ok(dsum_dtype) || !ln_dtype_ok(row_scale_dtype) ||
+        !ln_dtype_ok(param_dtype) || !ln_dtype_ok(dskip_dtype) || !ln_dtype_ok(dbranch_dtype))
+        return PTV3_EINVAL;
+    if (!ln_channels_ok(c)) return PTV3_ESHAPE;
+    if (n == 0) return PTV3_OK;
+    if (!sum || !dy || !gamma || !dgamma || !dbeta) return PTV3_EINVAL;
+    return launch_add_ln_bwd({sum, sum_dtype}, {dy, dy_dtype}, {dsum, dsum_dtype}, {row_scale, row_scale_dtype},
+                             {gamma, param_dtype}, n, c, eps, {dskip, dskip_dtype}, {dbranch, dbranch_dtype}, dgamma,
+                             dbeta, (hipStream_t)stream_);
 }
 
 extern "C" int ptv3_segment_reduce_bwd(const void* src, const void* out, const void* dout, int dtype, int64_t n, int c,

@@ -46,9 +46,9 @@ class LayerNorm(nn.LayerNorm):
             return super().forward(x)
         if ops.wants_grad(x, self.weight, self.bias):
             if x.is_cuda and x.shape[1] in ops.LAYER_NORM_BWD_CHANNELS:
-                if torch.is_autocast_enabled():
-                    x = x.float()   # autocast runs layer_norm in float and hands out a float result
-                return LayerNormFn.apply(x, self.weight, self.bias, self.eps)
+                # autocast runs layer_norm in float and hands out a float result
+                out_dtype = torch.float32 if torch.is_autocast_enabled() else None
+                return LayerNormFn.apply(x, self.weight, self.bias, self.eps, out_dtype)
             return super().forward(x)
         return ops.layer_norm(x, self.weight, self.bias, self.eps)
 
@@ -396,11 +396,15 @@ class Block(PointModule):
         ln1, ln2 = self.norm1[0], self.norm2[0]
         drop = self.drop_path[0]
         path_mask = drop.mask if isinstance(drop, DropPath) else (lambda x: None)
+        # under autocast the normalised rows are only ever read by a Linear, which would cast them to half
+        # precision first: the kernel writes them in that dtype (the same single rounding), the sums stay float
+        normed_dtype = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else None
         skip = point.feat
         point = self.cpe(point)
-        feat, point.feat = AddLayerNorm.apply(skip, point.feat, None, ln1.weight, ln1.bias, ln1.eps)
+        feat, point.feat = AddLayerNorm.apply(skip, point.feat, None, ln1.weight, ln1.bias, ln1.eps, normed_dtype)
         point = self.attn(point)
-        feat, point.feat = AddLayerNorm.apply(feat, point.feat, path_mask(point.feat), ln2.weight, ln2.bias, ln2.eps)
+        feat, point.feat = AddLayerNorm.apply(feat, point.feat, path_mask(point.feat), ln2.weight, ln2.bias, ln2.eps,
+                                              normed_dtype)
         point = self.mlp(point)
         mask = path_mask(point.feat)
         point.feat = feat + point.feat if mask is None else torch.addcmul(feat, point.feat, mask)

@@ -747,21 +747,54 @@ def layer_norm(x, weight, bias, eps=1e-5, residual=None, mode=0, weight2=None, b
 LAYER_NORM_BWD_CHANNELS = (32, 64, 128, 256, 512)
 
 
-def layer_norm_bwd(x, dout, weight, eps=1e-5, dres=None):
-    """(dx, dweight, dbias) of LayerNorm over the rows of x; dweight and dbias in fp32. dres: a gradient that
-    reaches x by another path (a residual connection), added to dx in the same pass."""
-    _dev(x, dout, weight, dres)
+def _code(t, fallback=0):
+    return fallback if t is None else _DTYPE_CODE[t.dtype]
+
+
+def add_layer_norm(skip, branch, row_scale, weight, bias, eps, sum_dtype=None, out_dtype=None):
+    """(sum, y) with sum = skip + branch * row_scale and y = LayerNorm(sum), every tensor read and written in its
+    own dtype. skip and row_scale (N,) or (N, 1) may be None; sum is returned as None when skip is None (then
+    y = LayerNorm(branch * row_scale)). sum_dtype defaults to the promoted dtype of skip and branch, out_dtype to it."""
+    _dev(skip, branch, row_scale, weight, bias)
     lib = _lib.load()
-    x = x.contiguous()
-    dout = dout.to(x.dtype).contiguous()
-    dres = None if dres is None else dres.to(x.dtype).contiguous()
-    n, c = x.shape
-    dx = torch.empty_like(x)
-    dwb = torch.zeros((2, c), dtype=torch.float32, device=x.device)
-    _lib.check(lib.ptv3_layer_norm_bwd(_ptr(x), _ptr(dout), _ptr(weight.to(x.dtype).contiguous()), _ptr(dres),
-                                       _dtype_code(x), n, c, float(eps), _ptr(dx), _ptr(dwb[0]), _ptr(dwb[1]), _stream()),
-               "ptv3_layer_norm_bwd")
-    return dx, dwb[0], dwb[1]
+    branch = branch.contiguous()
+    n, c = branch.shape
+    skip = None if skip is None else skip.contiguous()
+    row_scale = None if row_scale is None else row_scale.reshape(-1).contiguous()
+    if sum_dtype is None:
+        sum_dtype = branch.dtype if skip is None else torch.promote_types(skip.dtype, branch.dtype)
+    out_dtype = out_dtype or sum_dtype
+    total = None if skip is None else torch.empty((n, c), dtype=sum_dtype, device=branch.device)
+    y = torch.empty((n, c), dtype=out_dtype, device=branch.device)
+    w = weight.contiguous()
+    b = bias.to(w.dtype).contiguous()
+    _lib.check(lib.ptv3_add_layer_norm_fwd(_ptr(skip), _code(skip), _ptr(branch), _code(branch), _ptr(row_scale),
+                                           _code(row_scale), _ptr(w), _ptr(b), _code(w), n, c, float(eps), _ptr(total),
+                                           _DTYPE_CODE[sum_dtype], _ptr(y), _DTYPE_CODE[out_dtype], _stream()),
+               "ptv3_add_layer_norm_fwd")
+    return total, y
+
+
+def add_layer_norm_bwd(total, dy, dsum, row_scale, weight, eps, skip_dtype=None, branch_dtype=None):
+    """Backward of add_layer_norm: (dskip, dbranch, dweight, dbias); total is the sum the forward normalised, dsum
+    the gradient reaching it past the LayerNorm (or None). dskip / dbranch are made in the given dtypes and are
+    None where the dtype is None; dweight, dbias in fp32."""
+    _dev(total, dy, dsum, row_scale, weight)
+    lib = _lib.load()
+    total, dy = total.contiguous(), dy.contiguous()
+    dsum = None if dsum is None else dsum.contiguous()
+    row_scale = None if row_scale is None else row_scale.reshape(-1).contiguous()
+    n, c = total.shape
+    dev = total.device
+    dskip = None if skip_dtype is None else torch.empty((n, c), dtype=skip_dtype, device=dev)
+    dbranch = None if branch_dtype is None else torch.empty((n, c), dtype=branch_dtype, device=dev)
+    dwb = torch.zeros((2, c), dtype=torch.float32, device=dev)
+    w = weight.contiguous()
+    _lib.check(lib.ptv3_add_layer_norm_bwd(_ptr(total), _code(total), _ptr(dy), _code(dy), _ptr(dsum), _code(dsum),
+                                           _ptr(row_scale), _code(row_scale), _ptr(w), _code(w), n, c, float(eps),
+                                           _ptr(dskip), _code(dskip), _ptr(dbranch), _code(dbranch), _ptr(dwb[0]),
+                                           _ptr(dwb[1]), _stream()), "ptv3_add_layer_norm_bwd")
+    return dskip, dbranch, dwb[0], dwb[1]
 
 
 LINEAR_LN_CHANNELS = (128, 256)   # square Linear + LayerNorm(s) + residual in one kernel
