@@ -192,9 +192,12 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
     float cs[8];
 #pragma unroll
     for (int c = 0; c < 8; ++c) cs[c] = 0.f;
-    for (int base = 0; base < count; base += 4 * 32) {   // the same trip count for every wave
+    // A wave's LDS tiles are its own and its LDS operations complete in order, so the loop needs no barrier:
+    // the waves drift apart and hide each other's load latency. The pieces of the next step are requested as
+    // soon as this step's have been written to LDS, and arrive while the MFMAs run.
+    u32x4 wa[4], wb[4];
+    auto fetch = [&](int base) {
         const int mine = base + wave * 32;
-        u32x4 wa[4], wb[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int idx = mine + 4 * rq + j;
@@ -207,6 +210,9 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
                 if (b_in) wb[j] = *(const u32x4*)(b + rb * k_total + k0 + 8 * g);
             }
         }
+    };
+    if (count > 0) fetch(0);
+    for (int base = 0; base < count; base += 4 * 32) {
         if (sum_cols) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -217,7 +223,7 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
         }
         put_transposed4(ta, g, rq, wa);
         put_transposed4(tb, g, rq, wb);
-        __syncthreads();
+        if (base + 4 * 32 < count) fetch(base + 4 * 32);
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             v8 fa[2], fb[2];
@@ -234,8 +240,8 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
                 for (int j = 0; j < 2; ++j)
                     if (i < tm && j < tk) acc[i][j] = Mfma16<T>::mfma(fa[i], fb[j], acc[i][j]);
         }
-        __syncthreads();
     }
+    __syncthreads();   // every wave is done with its tiles
     // the four waves hold sums over different rows: add them up in LDS (the operand tiles are free now), then
     // every thread stores 16 of the block's 64 x 64 values into this split's slab, without atomics.
     // acc[i][j][v]: m = 32 i + 8 (v / 4) + 4 hf + v % 4, k = 32 j + col
