@@ -283,6 +283,144 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
     }
 }
 
+// The same reduction for results of 128 channels or more a side: a work-group owns a 128 x 128 block, its
+// four waves a 64 x 64 quadrant each, and the 32 rows of a step are staged once for all of them (threads
+// 0..127 the pieces of a, 128..255 those of b) into one of two LDS buffers, a barrier per step. Per MFMA that
+// is half the operand traffic and half the staging work of the 64 x 64 form, which at 256 channels is bound by
+// the gathered 128-byte pieces coming out of L2.
+constexpr int OW_C = 128;
+
+template <typename T, bool GATHER>
+__global__ __launch_bounds__(256) void outer_rows_wide_kernel(const T* __restrict__ a, const T* __restrict__ b, int64_t n,
+                                                              int m_total, int k_total, const int32_t* __restrict__ nbr,
+                                                              int taps, int splits, int64_t rows_per_split,
+                                                              int64_t slab_stride, float* __restrict__ d,
+                                                              float* __restrict__ colsum) {
+    typedef typename Mfma16<T>::v8 v8;
+    __shared__ __align__(16) uint16_t tiles[2][2][OW_C * OR_S];
+    __shared__ int32_t list_a[GATHER ? OR_LIST : 1], list_b[GATHER ? OR_LIST : 1];
+    __shared__ int list_n;
+    __shared__ float wave_cols[2][OW_C];
+    const int tap = blockIdx.x / splits, split = blockIdx.x % splits;
+    const int m0 = blockIdx.y * OW_C, k0 = blockIdx.z * OW_C;
+    const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
+    const int64_t r0 = (int64_t)split * rows_per_split;
+    const int64_t r1 = min(n, r0 + rows_per_split);
+    int count = (int)(r1 - r0);
+    if (GATHER) {
+        if (tid == 0) list_n = 0;
+        __syncthreads();
+        const int32_t* nb = nbr + (int64_t)tap * n;
+        for (int64_t e = r0 + tid; e < r0 + ((r1 - r0 + 255) / 256) * 256; e += 256) {
+            const int32_t src = e < r1 ? nb[e] : -1;
+            const uint64_t mask = __ballot(src >= 0);
+            int base = 0;
+            if (lane == 0 && mask) base = atomicAdd(&list_n, __popcll(mask));
+            base = __shfl(base, 0, PTV3_WAVE);
+            if (src >= 0) {
+                const int pos = base + __popcll(mask & ((1ull << lane) - 1));
+                list_a[pos] = (int32_t)(e - r0);
+                list_b[pos] = src;
+            }
+        }
+        __syncthreads();
+        count = list_n;
+    }
+    // this wave's quadrant, 2 x 2 tiles
+    const int qm = (wave & 1) * 64, qk = (wave >> 1) * 64;
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    // staging role: operand, channel group, row quad
+    const bool is_b = tid >= 128;
+    const int st = tid & 127, g = st & 15, rq = st >> 4;
+    const T* src_ptr = is_b ? b : a;
+    const int width = is_b ? k_total : m_total, c0 = (is_b ? k0 : m0) + 8 * g;
+    const bool in_range = c0 < width;
+    const bool sum_cols = colsum != nullptr && blockIdx.z == 0 && (!GATHER || tap == taps / 2);
+    float cs[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) cs[c] = 0.f;
+    u32x4 w[4];
+    auto fetch = [&](int base) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int idx = base + 4 * rq + j;
+            w[j] = (u32x4){0, 0, 0, 0};
+            if (idx < count && in_range) {
+                const int64_t ra = r0 + (GATHER ? list_a[idx] : idx);
+                const int64_t row = is_b ? (GATHER ? (int64_t)list_b[idx] : ra) : ra;
+                w[j] = *(const u32x4*)(src_ptr + row * width + c0);
+            }
+        }
+    };
+    const int col = lane & 31, hf = lane >> 5;
+    if (count > 0) fetch(0);
+    int buf = 0;
+    for (int base = 0; base < count; base += 32, buf ^= 1) {
+        if (sum_cols && !is_b) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const v8 h = __builtin_bit_cast(v8, w[j]);
+#pragma unroll
+                for (int c = 0; c < 8; ++c) cs[c] += (float)h[c];
+            }
+        }
+        put_transposed4(tiles[buf][is_b], g, rq, w);
+        if (base + 32 < count) fetch(base + 32);
+        // One barrier per step: it also keeps a wave from overwriting this buffer two steps on while another
+        // still reads it, because nobody passes the next step's barrier before everyone has finished these reads.
+        __syncthreads();
+        const uint16_t* ta = tiles[buf][0];
+        const uint16_t* tb = tiles[buf][1];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            v8 fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int cha = qm + 32 * i + col, chb = qk + 32 * i + col;
+                fa[i] = __builtin_bit_cast(v8, *(const u32x4*)(ta + cha * OR_S + 8 * ((2 * ks + hf) ^ ((cha >> 3) & 3))));
+                fb[i] = __builtin_bit_cast(v8, *(const u32x4*)(tb + chb * OR_S + 8 * ((2 * ks + hf) ^ ((chb >> 3) & 3))));
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = Mfma16<T>::mfma(fa[i], fb[j], acc[i][j]);
+        }
+    }
+    // acc[i][j][v]: m = m0 + qm + 32 i + 8 (v / 4) + 4 hf + v % 4, k = k0 + qk + 32 j + col; the quadrant is this wave's alone
+    float* slab = d + (int64_t)split * slab_stride;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int k = k0 + qk + 32 * j + col;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + qm + 32 * i + 8 * (v >> 2) + 4 * hf + (v & 3);
+                if (m < m_total && k < k_total) slab[((int64_t)m * taps + tap) * k_total + k] = acc[i][j][v];
+            }
+        }
+    if (sum_cols) {   // the same for the whole work-group; waves 0 and 1 staged a
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            cs[c] += __shfl_xor(cs[c], 16, PTV3_WAVE);
+            cs[c] += __shfl_xor(cs[c], 32, PTV3_WAVE);
+        }
+        if (!is_b && lane < 16) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) wave_cols[wave][8 * g + c] = cs[c];
+        }
+        __syncthreads();
+        if (tid < OW_C && m0 + tid < m_total)
+            colsum[(int64_t)split * slab_stride + m0 + tid] = wave_cols[0][tid] + wave_cols[1][tid];
+    }
+}
+
 // out[i] = sum over the splits' slabs (of `stride` floats, the first `total` of them summed): a work-group takes 32 neighbouring values, its 8 thread rows share
 // out the splits (four loads in flight each) and meet in LDS
 __global__ __launch_bounds__(256) void slab_sum_kernel(const float* __restrict__ slabs, int64_t stride, int64_t total,
@@ -593,7 +731,7 @@ __global__ __launch_bounds__(256) void segment_reduce_bwd_kernel(const T* __rest
 }
 
 // Rows of the reduction per work-group: enough work-groups to fill the part, but at least 1024 rows each so
-// that the 64 x 64 block a work-group hands in is small next to what it read.
+// that the block a work-group hands in is small next to what it read.
 void outer_split(int64_t n, int64_t blocks_per_split, int64_t cap, int64_t* splits, int64_t* rows) {
     int64_t sp = ptv3_ceil_div(1024, blocks_per_split);
     const int64_t most = ptv3_ceil_div(n, 1024);
@@ -605,10 +743,14 @@ void outer_split(int64_t n, int64_t blocks_per_split, int64_t cap, int64_t* spli
     *splits = ptv3_ceil_div(n, r);
 }
 
+// block side: 128 when both sides of the result have that many channels, else 64
+int outer_side(int m_total, int k_total) { return (m_total >= OW_C && k_total >= OW_C) ? OW_C : OR_C; }
+
 template <bool GATHER>
 size_t outer_workspace(int64_t n, int m_total, int k_total, int taps) {
+    const int side = outer_side(m_total, k_total);
     int64_t splits, rows;
-    outer_split(n, (int64_t)taps * ptv3_ceil_div(m_total, OR_C) * ptv3_ceil_div(k_total, OR_C), GATHER ? OR_LIST : 0,
+    outer_split(n, (int64_t)taps * ptv3_ceil_div(m_total, side) * ptv3_ceil_div(k_total, side), GATHER ? OR_LIST : 0,
                 &splits, &rows);
     return splits > 1 ? ptv3_align256((size_t)splits * ((size_t)m_total * taps * k_total + m_total) * sizeof(float)) : 0;
 }
@@ -617,7 +759,8 @@ size_t outer_workspace(int64_t n, int m_total, int k_total, int taps) {
 template <typename T, bool GATHER>
 int launch_outer(const void* a, const void* b, int64_t n, int m_total, int k_total, const int32_t* nbr, int taps,
                  float* d, float* colsum, void* workspace, size_t workspace_bytes, hipStream_t stream) {
-    const int64_t bm = ptv3_ceil_div(m_total, OR_C), bk = ptv3_ceil_div(k_total, OR_C);
+    const int side = outer_side(m_total, k_total);
+    const int64_t bm = ptv3_ceil_div(m_total, side), bk = ptv3_ceil_div(k_total, side);
     int64_t splits, rows;
     outer_split(n, (int64_t)taps * bm * bk, GATHER ? OR_LIST : 0, &splits, &rows);
     if ((int64_t)taps * splits >= (1ll << 31)) return PTV3_EINVAL;
@@ -626,9 +769,13 @@ int launch_outer(const void* a, const void* b, int64_t n, int m_total, int k_tot
     if (splits > 1 && (!workspace || workspace_bytes < (size_t)splits * stride * sizeof(float))) return PTV3_EWORKSPACE;
     float* slabs = splits > 1 ? (float*)workspace : d;
     float* cols = !colsum ? nullptr : (splits > 1 ? slabs + count : colsum);
-    hipLaunchKernelGGL((outer_rows_kernel<T, GATHER>), dim3((unsigned)(taps * splits), (unsigned)bm, (unsigned)bk),
-                       dim3(256), 0, stream, (const T*)a, (const T*)b, n, m_total, k_total, nbr, taps, (int)splits, rows,
-                       stride, slabs, cols);
+    const dim3 grid((unsigned)(taps * splits), (unsigned)bm, (unsigned)bk);
+    if (side == OW_C)
+        hipLaunchKernelGGL((outer_rows_wide_kernel<T, GATHER>), grid, dim3(256), 0, stream, (const T*)a, (const T*)b, n,
+                           m_total, k_total, nbr, taps, (int)splits, rows, stride, slabs, cols);
+    else
+        hipLaunchKernelGGL((outer_rows_kernel<T, GATHER>), grid, dim3(256), 0, stream, (const T*)a, (const T*)b, n,
+                           m_total, k_total, nbr, taps, (int)splits, rows, stride, slabs, cols);
     if (splits > 1) {
         const int64_t total = colsum ? stride : count;
         hipLaunchKernelGGL(slab_sum_kernel, dim3((unsigned)ptv3_ceil_div(total, 32)), dim3(256), 0, stream,
