@@ -73,8 +73,8 @@ class Linear(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, weight, bias):
-        w = weight.detach().to(x.dtype)
-        b = None if bias is None else bias.detach().to(x.dtype)
+        w = ops.cast_cached(weight, x.dtype)
+        b = None if bias is None else ops.cast_cached(bias, x.dtype)
         if ops.linear_rows_pays(x, w):
             out = ops.linear_rows(x, w, b)
         else:
@@ -87,7 +87,13 @@ class Linear(torch.autograd.Function):
     def backward(ctx, dout):
         x, weight = ctx.saved_tensors
         dout = dout.contiguous()
-        dx = dout @ weight.detach().to(dout.dtype) if ctx.needs_input_grad[0] else None
+        dx = None
+        if ctx.needs_input_grad[0]:
+            wt = ops.cast_cached(weight, dout.dtype, transpose=True)   # (K, Nout): dx = dout wt^T
+            if ops.linear_rows_pays(dout, wt):
+                dx = ops.linear_rows(dout, wt)   # many rows, few channels: the row kernel again
+            else:
+                dx = dout @ ops.cast_cached(weight, dout.dtype)
         want_bias = ctx.bias_dtype is not None and ctx.needs_input_grad[2]
         dw = db = None
         if ctx.needs_input_grad[1]:

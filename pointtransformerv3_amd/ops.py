@@ -44,6 +44,27 @@ def wants_grad(*tensors):
     return torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors)
 
 
+_CAST_CACHE = {}
+
+
+def cast_cached(t, dtype, transpose=False):
+    """t.to(dtype) (transposed and made contiguous if asked) for a parameter, remembered until the parameter is
+    written to or moved: training casts every weight on every use, twice per step and layer otherwise."""
+    if t.dtype == dtype and not transpose:
+        return t
+    key = (id(t), dtype, transpose)
+    stamp = (t.data_ptr(), t._version)
+    hit = _CAST_CACHE.get(key)
+    if hit is not None and hit[0] == stamp and hit[2]() is t:
+        return hit[1]
+    with torch.no_grad():
+        out = (t.detach().t() if transpose else t.detach()).to(dtype).contiguous()
+    import weakref
+    ref = weakref.ref(t, lambda _r, k=key: _CAST_CACHE.pop(k, None))
+    _CAST_CACHE[key] = (stamp, out, ref)
+    return out
+
+
 class Readback:
     """Device -> host read of a small tensor that does not drain the stream.
 

@@ -101,3 +101,22 @@ def test_forward_on_cpu_tensors_fails_loudly():
     data = dict(feat=torch.zeros(10, 6), grid_coord=torch.arange(30).reshape(10, 3).int(), offset=torch.tensor([10]))
     with pytest.raises(Ptv3Error):
         m(data)
+
+
+def test_cast_cache_follows_in_place_updates_and_replacement():
+    """Weights are cast once per update, not once per use: the remembered copy must go stale when the
+    parameter is written in place (an optimizer step) or its storage is replaced."""
+    import torch
+    from pointtransformerv3_amd import ops
+    p = torch.nn.Parameter(torch.arange(6, dtype=torch.float32).reshape(2, 3))
+    a = ops.cast_cached(p, torch.bfloat16)
+    assert a.dtype == torch.bfloat16 and ops.cast_cached(p, torch.bfloat16) is a
+    t = ops.cast_cached(p, torch.bfloat16, transpose=True)
+    assert t.shape == (3, 2) and t.is_contiguous() and torch.equal(t, a.t())
+    with torch.no_grad():
+        p.add_(1.0)
+    b = ops.cast_cached(p, torch.bfloat16)
+    assert b is not a and torch.equal(b.float(), p.detach())
+    p.data = torch.zeros(2, 3)
+    assert torch.equal(ops.cast_cached(p, torch.bfloat16).float(), torch.zeros(2, 3))
+    assert ops.cast_cached(p, torch.float32) is p
