@@ -301,3 +301,40 @@ def test_training_step_under_autocast(dtype):
         losses.append(float(loss.detach()))
     assert not torch.equal(before, model.embedding.stem.norm.running_mean)
     assert losses[-1] < losses[0]
+
+
+@pytest.mark.parametrize("variant", ["pdnorm", "post_norm", "cls_mode", "no_flash_fp32", "input_gradient"])
+def test_training_step_of_model_variants(variant):
+    """One forward + backward of the model built other ways: every parameter that takes part gets a finite
+    gradient (PDNorm only trains the norms of the condition it is given)."""
+    kw, autocast, extra = {}, torch.bfloat16, {}
+    if variant == "pdnorm":
+        kw = dict(pdnorm_bn=True, pdnorm_ln=True)
+        extra = dict(condition="S3DIS")
+    elif variant == "post_norm":
+        kw = dict(pre_norm=False)
+    elif variant == "cls_mode":
+        kw = dict(cls_mode=True)
+    elif variant == "no_flash_fp32":
+        kw, autocast = dict(enable_flash=False), None
+    torch.manual_seed(3)
+    model, _ = _small_model(drop_path=0.2, shuffle_orders=True, **kw)
+    model = model.to(DEV).train()
+    d, feat = _scene(n=1200)
+    x = torch.from_numpy(feat).to(DEV).requires_grad_(variant == "input_gradient")
+    data = dict(feat=x, grid_coord=torch.from_numpy(d["grid_coord"]).to(DEV), offset=torch.from_numpy(d["offset"]).to(DEV),
+                **extra)
+    if autocast is None:
+        out = model(data).feat
+    else:
+        with torch.autocast("cuda", dtype=autocast):
+            out = model(data).feat
+    out.float().square().mean().backward()
+    missing = [n for n, p in model.named_parameters() if p.grad is None]
+    if variant == "pdnorm":
+        assert missing and all(".norm." in n and ".norm.1." not in n for n in missing), missing[:5]
+    else:
+        assert not missing, missing[:5]
+    assert all(torch.isfinite(p.grad).all() for p in model.parameters() if p.grad is not None)
+    if variant == "input_gradient":
+        assert x.grad is not None and torch.isfinite(x.grad).all() and x.grad.abs().max() > 0
