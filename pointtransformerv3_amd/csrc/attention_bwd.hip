@@ -20,28 +20,30 @@
 
 namespace {
 
-constexpr int BWD_THREADS = 512;
+constexpr int BWD_THREADS = 512;    // keys kernel: 8 waves, two key tiles each per sweep
 constexpr int BWD_WAVES = BWD_THREADS / PTV3_WAVE;
+constexpr int BWQ_THREADS = 1024;   // queries kernel: 16 waves, four per SIMD
+constexpr int BWQ_WAVES = BWQ_THREADS / PTV3_WAVE;
 constexpr float LN2 = 0.6931471805599453f;
 constexpr float LOG2E = 1.4426950408889634f;
 
 // Stages `count` slots of 16 channels into LDS: as rows of 32 B (ROWS) and / or transposed, 16
 // rows of t_stride bytes with the slot axis permuted inside 32-blocks to the order in which the
 // MFMA result registers hold them (TRANS). fetch(slot, half) returns channels [8 half, 8 half + 8).
-template <bool ROWS, bool TRANS, typename F>
+template <bool ROWS, bool TRANS, int THREADS, typename F>
 __device__ __forceinline__ void stage16(int tid, int count, F fetch, unsigned char* rows_lds, unsigned char* t_lds,
                                         int t_stride) {
-    for (int e0 = tid; e0 < count * 2; e0 += 4 * BWD_THREADS) {
+    for (int e0 = tid; e0 < count * 2; e0 += 4 * THREADS) {
         u32x4 w[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int e = e0 + j * BWD_THREADS;
+            const int e = e0 + j * THREADS;
             w[j] = (u32x4){0, 0, 0, 0};
             if (e < count * 2) w[j] = fetch(e >> 1, e & 1);
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int e = e0 + j * BWD_THREADS;
+            const int e = e0 + j * THREADS;
             if (e >= count * 2) break;
             const int key = e >> 1, half8 = e & 1;
             if (ROWS) *(u32x4*)(rows_lds + key * 32 + half8 * 16) = w[j];
@@ -84,7 +86,7 @@ __device__ __forceinline__ f32x16 splat16(float x) {
 
 // ---- kernel 1: one work-group per (sequence, head), a wave per 32-query tile
 template <typename T, bool HAVE_LSE>
-__global__ __launch_bounds__(BWD_THREADS) void attn_bwd_q_kernel(
+__global__ __launch_bounds__(BWQ_THREADS) void attn_bwd_q_kernel(
     const T* __restrict__ qkv, const T* __restrict__ out, const T* __restrict__ dout, int channels, int heads,
     const int32_t* __restrict__ slot_src, const int32_t* __restrict__ slot_dst,
     const int32_t* __restrict__ cu_seqlens, int lds_keys, float scale, int64_t n_pad, T* __restrict__ dqkv,
@@ -108,12 +110,12 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_q_kernel(
     const int64_t row_stride = 3 * (int64_t)channels;
 
     if (tid < 24) ((uint32_t*)zero_lds)[tid] = 0u;
-    stage16<true, true>(tid, len64, [&](int key, int half8) {
+    stage16<true, true, BWQ_THREADS>(tid, len64, [&](int key, int half8) {
         u32x4 w = {0, 0, 0, 0};
         if (key < len) w = *(const u32x4*)(qkv + (int64_t)slot_src[s0 + key] * row_stride + channels + head * HD + half8 * 8);
         return w;
     }, k_lds, kt_lds, kt_stride);
-    stage16<true, false>(tid, len64, [&](int key, int half8) {
+    stage16<true, false, BWQ_THREADS>(tid, len64, [&](int key, int half8) {
         u32x4 w = {0, 0, 0, 0};
         if (key < len) w = *(const u32x4*)(qkv + (int64_t)slot_src[s0 + key] * row_stride + 2 * channels + head * HD + half8 * 8);
         return w;
@@ -131,7 +133,7 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_q_kernel(
     const unsigned char* kt_base = col < HD ? kt_lds + (size_t)col * kt_stride + hf * 32 : zero_lds;
     const int kt_step = col < HD ? 128 : 0;
 
-    for (int qt = wave; qt < n_qtiles; qt += BWD_WAVES) {
+    for (int qt = wave; qt < n_qtiles; qt += BWQ_WAVES) {
         const int qi = qt * 32 + col;
         int dst = -1;
         u32x4 qreg = {0, 0, 0, 0}, doreg = {0, 0, 0, 0}, oreg = {0, 0, 0, 0};
@@ -196,37 +198,27 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_q_kernel(
         f32x16 acc = zero;
         const unsigned char* kt_ptr = kt_base;
         for (int kp = 0; kp < n_pairs; ++kp) {
-            const v8 k0 = __builtin_bit_cast(v8, *(const u32x4*)(k_base + (size_t)kp * 64 * 32));
-            const v8 k1 = __builtin_bit_cast(v8, *(const u32x4*)(k_base + (size_t)kp * 64 * 32 + 32 * 32));
-            const v8 v0 = __builtin_bit_cast(v8, *(const u32x4*)(v_base + (size_t)kp * 64 * 32));
-            const v8 v1 = __builtin_bit_cast(v8, *(const u32x4*)(v_base + (size_t)kp * 64 * 32 + 32 * 32));
-            f32x16 sa = Half<T>::mfma(k0, qfrag, c_lse);    // S - lse
-            f32x16 sb = Half<T>::mfma(k1, qfrag, c_lse);
-            const f32x16 da = Half<T>::mfma(v0, dofrag, c_d);   // dP - D
-            const f32x16 db = Half<T>::mfma(v1, dofrag, c_d);
-            const u32x4 ka0 = *(const u32x4*)kt_ptr;
-            const u32x4 ka1 = *(const u32x4*)(kt_ptr + 16);
-            const u32x4 kb0 = *(const u32x4*)(kt_ptr + 64);
-            const u32x4 kb1 = *(const u32x4*)(kt_ptr + 80);
-            kt_ptr += kt_step;
-            if (ragged && kp == n_pairs - 1) {
+            // the two 32-key halves of the step one after the other: fewer values alive at a time
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int key = kp * 64 + 8 * (v >> 2) + 4 * hf + (v & 3);
-                    if (key >= len) sa[v] = -INFINITY;
-                    if (key + 32 >= len) sb[v] = -INFINITY;
+            for (int h = 0; h < 2; ++h) {
+                const v8 kf = __builtin_bit_cast(v8, *(const u32x4*)(k_base + (size_t)kp * 64 * 32 + h * 32 * 32));
+                const v8 vf = __builtin_bit_cast(v8, *(const u32x4*)(v_base + (size_t)kp * 64 * 32 + h * 32 * 32));
+                f32x16 sc = Half<T>::mfma(kf, qfrag, c_lse);        // S - lse
+                const f32x16 dp = Half<T>::mfma(vf, dofrag, c_d);   // dP - D
+                const u32x4 kt0 = *(const u32x4*)(kt_ptr + 64 * h);
+                const u32x4 kt1 = *(const u32x4*)(kt_ptr + 64 * h + 16);
+                if (ragged && kp == n_pairs - 1) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        if (kp * 64 + 32 * h + 8 * (v >> 2) + 4 * hf + (v & 3) >= len) sc[v] = -INFINITY;
                 }
-            }
-            float dsa[16], dsb[16];
+                float ds[16];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                dsa[v] = __builtin_amdgcn_exp2f(sa[v]) * da[v];
-                dsb[v] = __builtin_amdgcn_exp2f(sb[v]) * db[v];
+                for (int v = 0; v < 16; ++v) ds[v] = __builtin_amdgcn_exp2f(sc[v]) * dp[v];
+                acc = Half<T>::mfma(__builtin_bit_cast(v8, kt0), pack8<T>(ds), acc);
+                acc = Half<T>::mfma(__builtin_bit_cast(v8, kt1), pack8<T>(ds + 8), acc);
             }
-            acc = Half<T>::mfma(__builtin_bit_cast(v8, ka0), pack8<T>(dsa), acc);
-            acc = Half<T>::mfma(__builtin_bit_cast(v8, ka1), pack8<T>(dsa + 8), acc);
-            acc = Half<T>::mfma(__builtin_bit_cast(v8, kb0), pack8<T>(dsb), acc);
-            acc = Half<T>::mfma(__builtin_bit_cast(v8, kb1), pack8<T>(dsb + 8), acc);
+            kt_ptr += kt_step;
         }
         if (dst >= 0) {
             // acc[v], v < 8: channel d = 8 (v / 4) + 4 hf + v % 4 of this lane's query
@@ -273,13 +265,13 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_kv_kernel(
     const float scale_log2e = scale * LOG2E;
 
     if (tid < 24) ((uint32_t*)zero_lds)[tid] = 0u;
-    stage16<true, true>(tid, len64, [&](int key, int half8) {
+    stage16<true, true, BWD_THREADS>(tid, len64, [&](int key, int half8) {
         u32x4 w = {0, 0, 0, 0};
         if (key < len)
             w = scale8<T>(*(const u32x4*)(qkv + (int64_t)slot_src[s0 + key] * row_stride + head * HD + half8 * 8), scale_log2e);
         return w;
     }, q_lds, qt_lds, t_stride);
-    stage16<true, true>(tid, len64, [&](int key, int half8) {
+    stage16<true, true, BWD_THREADS>(tid, len64, [&](int key, int half8) {
         u32x4 w = {0, 0, 0, 0};
         if (key < len) {
             const int dst = slot_dst[s0 + key];
@@ -643,7 +635,7 @@ int launch_half_bwd(const void* qkv, const void* out, const void* dout, int chan
         allowed_kv = lds_kv;
     }
     const unsigned grid = (unsigned)(n_seq * heads);
-    hipLaunchKernelGGL(kq, dim3(grid), dim3(BWD_THREADS), lds_q, stream, (const T*)qkv, (const T*)out, (const T*)dout,
+    hipLaunchKernelGGL(kq, dim3(grid), dim3(BWQ_THREADS), lds_q, stream, (const T*)qkv, (const T*)out, (const T*)dout,
                        channels, heads, slot_src, slot_dst, cu_seqlens, lds_keys, scale, n_pad, (T*)dqkv, lse_buf, ws.d);
     hipLaunchKernelGGL(kkv, dim3(grid), dim3(BWD_THREADS), lds_kv, stream, (const T*)qkv, (const T*)dout, channels,
                        heads, slot_src, slot_dst, cu_seqlens, lds_keys, scale, n_pad, lse_buf, ws.d, (T*)dqkv,
