@@ -512,6 +512,42 @@ __device__ __forceinline__ float round_any(float v, int dtype) {
     return (float)(__bf16)v;
 }
 
+// The bits of 8 consecutive values, fetched without looking at them, and their conversion afterwards: a kernel
+// issues the loads of all its operands back to back and converts once they have arrived (a conversion inside
+// the dtype branch would make every load wait for the one before).
+struct Raw8 {
+    u32x4 lo, hi;
+};
+__device__ __forceinline__ Raw8 raw8_load(const void* p, int dtype, int64_t off) {
+    Raw8 r;
+    const char* b = (const char*)p + off * (dtype == PTV3_F32 ? 4 : 2);
+    r.lo = *(const u32x4*)b;
+    r.hi = (u32x4){0, 0, 0, 0};
+    if (dtype == PTV3_F32) r.hi = *(const u32x4*)(b + 16);
+    return r;
+}
+__device__ __forceinline__ void raw8_floats(const Raw8& r, int dtype, float* v) {
+    if (dtype == PTV3_F32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t a = r.lo[i], b = r.hi[i];   // through scalars: a bit_cast of the subscript itself reads element 0
+            v[i] = __builtin_bit_cast(float, a);
+            v[4 + i] = __builtin_bit_cast(float, b);
+        }
+    } else if (dtype == PTV3_F16) {
+        typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+        const h8 h = __builtin_bit_cast(h8, r.lo);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (float)h[i];
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = __builtin_bit_cast(float, r.lo[i] << 16);
+            v[2 * i + 1] = __builtin_bit_cast(float, r.lo[i] & 0xffff0000u);
+        }
+    }
+}
+
 // Tensors of one call, each with its own dtype: autocast mixes a float residual stream with half-precision
 // branches, and the kernels read and write each in place instead of going through cast passes.
 struct AnyRows {
@@ -544,15 +580,16 @@ __global__ __launch_bounds__(256) void add_layer_norm_fwd_kernel(AnyRows skip, A
 #pragma unroll
         for (int i = 0; i < 8; ++i) xv[i] = 0.f;
         if (valid) {
-            load8_any(branch.p, branch.dtype, off, xv);
-            if (row_scale.p) {
-                const float m = load1_any(row_scale.p, row_scale.dtype, row);
+            const Raw8 rb = raw8_load(branch.p, branch.dtype, off);
+            Raw8 rs = rb;
+            if (skip.p) rs = raw8_load(skip.p, skip.dtype, off);
+            const float m = row_scale.p ? load1_any(row_scale.p, row_scale.dtype, row) : 1.f;
+            raw8_floats(rb, branch.dtype, xv);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) xv[i] *= m;
-            }
+            for (int i = 0; i < 8; ++i) xv[i] *= m;
             if (skip.p) {
                 float sv[8];
-                load8_any(skip.p, skip.dtype, off, sv);
+                raw8_floats(rs, skip.dtype, sv);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) xv[i] += sv[i];
             }
@@ -601,9 +638,18 @@ __global__ __launch_bounds__(256) void add_layer_norm_bwd_kernel(AnyRows sum, An
         float xv[8], gv[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) { xv[i] = 0.f; gv[i] = 0.f; }
+        float extra[8], scale = 1.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) extra[i] = 0.f;
         if (valid) {
-            load8_any(sum.p, sum.dtype, off, xv);
-            load8_any(dy.p, dy.dtype, off, gv);
+            const Raw8 rx = raw8_load(sum.p, sum.dtype, off);
+            const Raw8 rg = raw8_load(dy.p, dy.dtype, off);
+            Raw8 re = rx;
+            if (dsum.p) re = raw8_load(dsum.p, dsum.dtype, off);   // gradient arriving at the sum by another path
+            if (row_scale.p && dbranch.p) scale = load1_any(row_scale.p, row_scale.dtype, row);
+            raw8_floats(rx, sum.dtype, xv);
+            raw8_floats(rg, dy.dtype, gv);
+            if (dsum.p) raw8_floats(re, dsum.dtype, extra);
         }
         float s = 0.f;
 #pragma unroll
@@ -626,19 +672,13 @@ __global__ __launch_bounds__(256) void add_layer_norm_bwd_kernel(AnyRows sum, An
         s1 = row_sum<LPR>(s1) * (1.f / C);
         s2 = row_sum<LPR>(s2) * (1.f / C);
         if (valid) {
-            float o[8], extra[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) extra[i] = 0.f;
-            if (dsum.p) load8_any(dsum.p, dsum.dtype, off, extra);   // gradient arriving at the sum by another path
+            float o[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) o[i] = rstd * (gv[i] - s1 - xv[i] * s2) + extra[i];
             if (dskip.p) store8_any(dskip.p, dskip.dtype, off, o);
             if (dbranch.p) {
-                if (row_scale.p) {
-                    const float m = load1_any(row_scale.p, row_scale.dtype, row);
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) o[i] *= m;
-                }
+                for (int i = 0; i < 8; ++i) o[i] *= scale;
                 store8_any(dbranch.p, dbranch.dtype, off, o);
             }
         }
@@ -668,9 +708,10 @@ __global__ __launch_bounds__(256) void add_layer_norm_bwd_kernel(AnyRows sum, An
 }
 
 int64_t ln_grid(int64_t n, int c) {
+    const int64_t cap = 512;   // two work-groups per CU: more only add atomics on the column sums (measured)
     const int64_t rows_per_wg = 4 * (PTV3_WAVE / (c / 8));
     const int64_t grid = ptv3_ceil_div(n, rows_per_wg);
-    return grid > 2048 ? 2048 : grid;
+    return grid > cap ? cap : grid;
 }
 
 int launch_add_ln_fwd(AnyRows skip, AnyRows branch, AnyRows row_scale, AnyRows gamma, AnyRows beta, int64_t n, int c,
