@@ -305,6 +305,23 @@ int ptv3_add_layer_norm_bwd(const void *sum, int sum_dtype, const void *dy, int 
                             int param_dtype, int64_t n, int c, float eps, void *dskip, int dskip_dtype,
                             void *dbranch, int dbranch_dtype, float *dgamma, float *dbeta, void *stream);
 
+/* nn.BatchNorm1d in training mode (model.py:848; call sites :776-779, :707-710, :729-735), first half: the
+ * batch statistics of x (n,c), c in {32, 64, 128, 256, 512}. stats (3,c) fp32 receives mean, rsqrt(var + eps)
+ * and the biased variance; running_mean / running_var (c,) fp32, when given, are updated in place with
+ * `momentum` and the unbiased variance, as torch does. workspace: 2*c floats. The normalisation itself is
+ * ptv3_bn_act with mean = stats[0], var = stats[2]. */
+int ptv3_batch_norm_stats(const void *x, int dtype, int64_t n, int c, float eps, float momentum,
+                          float *running_mean, float *running_var, float *stats, float *workspace,
+                          void *stream);
+
+/* Backward of BatchNorm1d, optionally through the exact GELU behind it (gelu != 0: dout is the gradient of
+ * gelu(bn(x))). stats as written by ptv3_batch_norm_stats, or (running_mean, rsqrt(running_var + eps)) with
+ * batch_stats = 0 for a module in evaluation mode. gamma, beta (c,) of param_dtype or NULL. dx (n,c) of
+ * dx_dtype; dgamma_dbeta (2,c) fp32 receives the parameter gradients (every element written). */
+int ptv3_batch_norm_bwd(const void *x, int x_dtype, const void *dout, int dout_dtype, const float *stats,
+                        const void *gamma, const void *beta, int param_dtype, int64_t n, int c, int gelu,
+                        int batch_stats, void *dx, int dx_dtype, float *dgamma_dbeta, void *stream);
+
 /* Backward of ptv3_segment_reduce (torch_scatter.segment_csr's, model.py:684-689): dsrc (n,c).
  * max / min: the gradient of a cluster goes to the first member in list order whose value equals
  * out; sum: to every member; mean: divided by the cluster size. Every row of src must belong to

@@ -145,6 +145,42 @@ class AddLayerNorm(torch.autograd.Function):
         return dskip, dbranch, None, dw.to(weight.dtype), db.to(bias_dtype), None, None
 
 
+class BatchNormAct(torch.autograd.Function):
+    """nn.BatchNorm1d (batch statistics and running-average update in training mode, the running statistics
+    otherwise), optionally followed by exact GELU (model.py:776-779, :707-710, :729-735), as one node: the
+    pre-activation is not kept, the backward kernels recompute it from x."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, bn, gelu):
+        batch = bn.training or bn.running_mean is None
+        if batch:
+            track = bn.track_running_stats and bn.running_mean is not None and bn.running_mean.dtype == torch.float32
+            momentum = bn.momentum
+            if track and bn.num_batches_tracked is not None:
+                bn.num_batches_tracked += 1
+                if momentum is None:
+                    momentum = 1.0 / float(bn.num_batches_tracked)
+            stats = ops.batch_norm_stats(x, bn.eps, momentum or 0.0, bn.running_mean if track else None,
+                                         bn.running_var if track else None)
+            mean, var = stats[0], stats[2]
+        else:
+            mean, var = bn.running_mean.float(), bn.running_var.float()
+            stats = torch.stack([mean, torch.rsqrt(var + bn.eps)])
+        out = ops.bn_act(x, mean, var, None if weight is None else weight.detach(),
+                         None if bias is None else bias.detach(), bn.eps, gelu)
+        ctx.save_for_backward(x, weight, bias, stats)
+        ctx.gelu, ctx.batch = gelu, batch
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        x, weight, bias, stats = ctx.saved_tensors
+        dx, dw, db = ops.batch_norm_bwd(x, dout, stats, None if weight is None else weight.detach(),
+                                        None if bias is None else bias.detach(), ctx.gelu, ctx.batch)
+        return (dx, None if weight is None else dw.to(weight.dtype), None if bias is None else db.to(bias.dtype),
+                None, None)
+
+
 class SegmentReduce(torch.autograd.Function):
     @staticmethod
     def forward(ctx, src, indices, idx_ptr, reduce):

@@ -19,6 +19,12 @@
 //   one atomic per work-group and channel. The training forward and backward kernels also take the
 //   residual add in front of the LayerNorm (model.py:589-604) and its stochastic-depth factor, and read
 //   and write every tensor in its own dtype (float residual stream, half-precision branches under autocast).
+// * nn.BatchNorm1d in training mode, with the nn.GELU behind it (model.py:776-779, :707-710, :729-735): column
+//   statistics over all rows (sums of x - pivot and of its square per lane, pivot = the first row, so that
+//   a large mean does not cancel the variance), a one-work-group kernel that turns them into mean / rstd and
+//   updates the running averages, the normalisation itself by the inference kernel with the batch
+//   statistics; backward in two passes over x and dy: the column sums of dz and dz * xhat (dz = dy *
+//   gelu'(z), z recomputed), then dx = gamma * rstd * (dz - mean(dz) - xhat * mean(dz * xhat)).
 // * torch_scatter.segment_csr (model.py:684-689): max / min send the gradient of a cluster to the first
 //   member that attains the value, sum copies it to every member, mean divides it by the cluster size.
 #include <hip/hip_bf16.h>
@@ -740,6 +746,168 @@ int launch_add_ln_bwd(AnyRows sum, AnyRows dy, AnyRows dsum, AnyRows row_scale, 
     return PTV3_ESHAPE;
 }
 
+// ---- BatchNorm1d in training mode (+ exact GELU)
+__device__ __forceinline__ float gelu_grad(float z) {
+    const float cdf = 0.5f * (1.f + erff(z * 0.70710678118654752f));
+    return cdf + z * 0.3989422804014327f * __expf(-0.5f * z * z);
+}
+
+// adds every lane's eight column values up over the rows a wave holds side by side, the waves and, with one
+// atomic per channel, the work-groups: out[ch] += ..., out2[ch] += ...
+template <int LPR>
+__device__ __forceinline__ void column_sums_out(float* a, float* b, float (*part)[4][LPR * 8], float* out, float* out2) {
+    constexpr int C = LPR * 8;
+    const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
+    const int sub = lane % LPR, rsub = lane / LPR;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+#pragma unroll
+        for (int off = LPR; off < PTV3_WAVE; off <<= 1) {
+            a[i] += __shfl_xor(a[i], off, PTV3_WAVE);
+            b[i] += __shfl_xor(b[i], off, PTV3_WAVE);
+        }
+    }
+    if (rsub == 0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            part[0][wave][sub * 8 + i] = a[i];
+            part[1][wave][sub * 8 + i] = b[i];
+        }
+    }
+    __syncthreads();
+    for (int c = tid; c < 2 * C; c += 256) {
+        const int which = c / C, ch = c % C;
+        const float v = part[which][0][ch] + part[which][1][ch] + part[which][2][ch] + part[which][3][ch];
+        atomicAdd((which ? out2 : out) + ch, v);
+    }
+}
+
+// sums[0][ch] += sum_rows (x - x[0][ch]), sums[1][ch] += sum_rows (x - x[0][ch])^2
+template <int LPR>
+__global__ __launch_bounds__(256) void bn_stats_kernel(AnyRows x, int64_t n, float* __restrict__ sums) {
+    constexpr int C = LPR * 8, RPW = PTV3_WAVE / LPR;
+    __shared__ float part[2][4][C];
+    const int wave = threadIdx.x / PTV3_WAVE, lane = threadIdx.x % PTV3_WAVE;
+    const int sub = lane % LPR, rsub = lane / LPR;
+    float pivot[8], s1[8], s2[8];
+    load8_any(x.p, x.dtype, sub * 8, pivot);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { s1[i] = 0.f; s2[i] = 0.f; }
+    const int64_t stride = (int64_t)gridDim.x * 4 * RPW;
+    for (int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * RPW; row0 < n; row0 += stride) {
+        const int64_t row = row0 + rsub;
+        if (row < n) {
+            float v[8];
+            raw8_floats(raw8_load(x.p, x.dtype, row * C + sub * 8), x.dtype, v);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float d = v[i] - pivot[i];
+                s1[i] += d;
+                s2[i] = fmaf(d, d, s2[i]);
+            }
+        }
+    }
+    column_sums_out<LPR>(s1, s2, part, sums, sums + C);
+}
+
+// one work-group: stats[0] = mean, stats[1] = rstd from the sums above; running averages updated in place
+// (unbiased variance, as torch does), when given
+__global__ __launch_bounds__(256) void bn_finalize_kernel(AnyRows x, const float* __restrict__ sums, int64_t n, int c,
+                                                          float eps, float momentum, float* __restrict__ running_mean,
+                                                          float* __restrict__ running_var, float* __restrict__ stats) {
+    for (int ch = threadIdx.x; ch < c; ch += 256) {
+        const float pivot = load1_any(x.p, x.dtype, ch);
+        const float m1 = sums[ch] / (float)n;
+        const float var = fmaxf(sums[c + ch] / (float)n - m1 * m1, 0.f);
+        const float mean = pivot + m1;
+        stats[ch] = mean;
+        stats[c + ch] = rsqrtf(var + eps);
+        stats[2 * c + ch] = var;
+        if (running_mean) {
+            running_mean[ch] = (1.f - momentum) * running_mean[ch] + momentum * mean;
+            const float unbiased = n > 1 ? var * ((float)n / (float)(n - 1)) : var;
+            running_var[ch] = (1.f - momentum) * running_var[ch] + momentum * unbiased;
+        }
+    }
+}
+
+// PASS 0: sums[0][ch] += sum_rows dz * xhat, sums[1][ch] += sum_rows dz.
+// PASS 1: dx = gamma * rstd * (dz - sums[1] / n - xhat * sums[0] / n), or gamma * rstd * dz when the statistics
+// were not the batch's own (evaluation mode). dz = dy * gelu'(gamma * xhat + beta) with GELU, else dy.
+template <int LPR, int PASS>
+__global__ __launch_bounds__(256) void bn_bwd_kernel(AnyRows x, AnyRows dy, const float* __restrict__ stats,
+                                                     AnyRows gamma, AnyRows beta, int64_t n, int gelu, int batch_stats,
+                                                     float* __restrict__ sums, AnyRowsOut dx) {
+    constexpr int C = LPR * 8, RPW = PTV3_WAVE / LPR;
+    __shared__ float part[2][4][C];
+    const int wave = threadIdx.x / PTV3_WAVE, lane = threadIdx.x % PTV3_WAVE;
+    const int sub = lane % LPR, rsub = lane / LPR;
+    float mean[8], rstd[8], g[8], b[8], a1[8], a2[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        mean[i] = stats[sub * 8 + i];
+        rstd[i] = stats[C + sub * 8 + i];
+        g[i] = 1.f;
+        b[i] = 0.f;
+        a1[i] = 0.f;
+        a2[i] = 0.f;
+    }
+    if (gamma.p) load8_any(gamma.p, gamma.dtype, sub * 8, g);
+    if (beta.p) load8_any(beta.p, beta.dtype, sub * 8, b);
+    if (PASS == 1) {
+        const float inv_n = batch_stats ? 1.f / (float)n : 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            a1[i] = sums[sub * 8 + i] * inv_n;       // mean of dz * xhat
+            a2[i] = sums[C + sub * 8 + i] * inv_n;   // mean of dz
+        }
+    }
+    const int64_t stride = (int64_t)gridDim.x * 4 * RPW;
+    for (int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * RPW; row0 < n; row0 += stride) {
+        const int64_t row = row0 + rsub;
+        if (row < n) {
+            const int64_t off = row * C + sub * 8;
+            const Raw8 rx = raw8_load(x.p, x.dtype, off);
+            const Raw8 rg = raw8_load(dy.p, dy.dtype, off);
+            float xv[8], dz[8];
+            raw8_floats(rx, x.dtype, xv);
+            raw8_floats(rg, dy.dtype, dz);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                xv[i] = (xv[i] - mean[i]) * rstd[i];   // xhat
+                if (gelu) dz[i] *= gelu_grad(fmaf(g[i], xv[i], b[i]));
+            }
+            if (PASS == 0) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    a1[i] = fmaf(dz[i], xv[i], a1[i]);
+                    a2[i] += dz[i];
+                }
+            } else {
+                float o[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) o[i] = g[i] * rstd[i] * (dz[i] - a2[i] - xv[i] * a1[i]);
+                store8_any(dx.p, dx.dtype, off, o);
+            }
+        }
+    }
+    if (PASS == 0) column_sums_out<LPR>(a1, a2, part, sums, sums + C);
+}
+
+template <int PASS>
+int launch_bn_bwd(AnyRows x, AnyRows dy, const float* stats, AnyRows gamma, AnyRows beta, int64_t n, int c, int gelu,
+                  int batch_stats, float* sums, AnyRowsOut dx, hipStream_t stream) {
+#define PTV3_BNB(L)                                                                                                   \
+    if (c == 8 * L) {                                                                                                 \
+        hipLaunchKernelGGL((bn_bwd_kernel<L, PASS>), dim3((unsigned)ln_grid(n, c)), dim3(256), 0, stream, x, dy,      \
+                           stats, gamma, beta, n, gelu, batch_stats, sums, dx);                                       \
+        PTV3_RETURN_LAUNCH();                                                                                         \
+    }
+    PTV3_BNB(4) PTV3_BNB(8) PTV3_BNB(16) PTV3_BNB(32) PTV3_BNB(64)
+#undef PTV3_BNB
+    return PTV3_ESHAPE;
+}
+
 bool ln_dtype_ok(int dtype) { return dtype >= PTV3_F32 && dtype <= PTV3_BF16; }
 bool ln_channels_ok(int c) { return c == 32 || c == 64 || c == 128 || c == 256 || c == 512; }
 
@@ -943,6 +1111,45 @@ extern "C" int ptv3_add_layer_norm_bwd(const void* sum, int sum_dtype, const voi
     return launch_add_ln_bwd({sum, sum_dtype}, {dy, dy_dtype}, {dsum, dsum_dtype}, {row_scale, row_scale_dtype},
                              {gamma, param_dtype}, n, c, eps, {dskip, dskip_dtype}, {dbranch, dbranch_dtype}, dgamma,
                              dbeta, (hipStream_t)stream_);
+}
+
+extern "C" int ptv3_batch_norm_stats(const void* x, int dtype, int64_t n, int c, float eps, float momentum,
+                                     float* running_mean, float* running_var, float* stats, float* workspace,
+                                     void* stream_) {
+    if (n < 1 || c < 1) return PTV3_EINVAL;
+    if (!ln_dtype_ok(dtype)) return PTV3_EINVAL;
+    if (!ln_channels_ok(c)) return PTV3_ESHAPE;
+    if (!x || !stats || !workspace || ((running_mean == nullptr) != (running_var == nullptr))) return PTV3_EINVAL;
+    hipStream_t stream = (hipStream_t)stream_;
+    const AnyRows xr = {x, dtype};
+    hipLaunchKernelGGL(zero_kernel, dim3((unsigned)ptv3_ceil_div(2 * c, 256)), dim3(256), 0, stream, workspace, (int64_t)2 * c);
+#define PTV3_BNS(L)                                                                                                   \
+    if (c == 8 * L)                                                                                                   \
+        hipLaunchKernelGGL((bn_stats_kernel<L>), dim3((unsigned)ln_grid(n, c)), dim3(256), 0, stream, xr, n, workspace);
+    PTV3_BNS(4) PTV3_BNS(8) PTV3_BNS(16) PTV3_BNS(32) PTV3_BNS(64)
+#undef PTV3_BNS
+    hipLaunchKernelGGL(bn_finalize_kernel, dim3(1), dim3(256), 0, stream, xr, (const float*)workspace, n, c, eps, momentum,
+                       running_mean, running_var, stats);
+    PTV3_RETURN_LAUNCH();
+}
+
+extern "C" int ptv3_batch_norm_bwd(const void* x, int x_dtype, const void* dout, int dout_dtype, const float* stats,
+                                   const void* gamma, const void* beta, int param_dtype, int64_t n, int c, int gelu,
+                                   int batch_stats, void* dx, int dx_dtype, float* dgamma_dbeta, void* stream_) {
+    if (n < 0 || c < 1) return PTV3_EINVAL;
+    if (!ln_dtype_ok(x_dtype) || !ln_dtype_ok(dout_dtype) || !ln_dtype_ok(param_dtype) || !ln_dtype_ok(dx_dtype))
+        return PTV3_EINVAL;
+    if (!ln_channels_ok(c)) return PTV3_ESHAPE;
+    if (!dgamma_dbeta) return PTV3_EINVAL;
+    hipStream_t stream = (hipStream_t)stream_;
+    hipLaunchKernelGGL(zero_kernel, dim3((unsigned)ptv3_ceil_div(2 * c, 256)), dim3(256), 0, stream, dgamma_dbeta, (int64_t)2 * c);
+    if (n == 0) PTV3_RETURN_LAUNCH();
+    if (!x || !dout || !stats || !dx) return PTV3_EINVAL;
+    const AnyRows xr = {x, x_dtype}, gr = {dout, dout_dtype}, ga = {gamma, param_dtype}, be = {beta, param_dtype};
+    const AnyRowsOut out = {dx, dx_dtype};
+    int rc = launch_bn_bwd<0>(xr, gr, stats, ga, be, n, c, gelu, batch_stats, dgamma_dbeta, out, stream);
+    if (rc != PTV3_OK) return rc;
+    return launch_bn_bwd<1>(xr, gr, stats, ga, be, n, c, gelu, batch_stats, dgamma_dbeta, out, stream);
 }
 
 extern "C" int ptv3_segment_reduce_bwd(const void* src, const void* out, const void* dout, int dtype, int64_t n, int c,

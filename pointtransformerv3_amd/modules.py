@@ -11,7 +11,7 @@ import torch
 import torch.nn as nn
 
 from . import ops
-from .autograd import AddLayerNorm, LayerNorm as LayerNormFn, SegmentReduce, UnpoolAdd
+from .autograd import AddLayerNorm, BatchNormAct, LayerNorm as LayerNormFn, SegmentReduce, UnpoolAdd
 from .point import AttrDict, Point, offset2bincount
 from .sparse import SparseConvTensor, SubMConv3d, is_spconv_module
 
@@ -58,6 +58,15 @@ def _fusable_bn(module, feat):
     return (type(module) is nn.BatchNorm1d and not module.training and module.track_running_stats
             and module.running_mean is not None and feat.is_cuda and feat.dim() == 2 and feat.shape[1] % 8 == 0
             and not ops.wants_grad(feat, module.weight, module.bias))
+
+
+def _trainable_bn(module, feat):
+    """BatchNorm1d over (N, C) GPU features under autograd that the training kernels cover."""
+    return (type(module) is nn.BatchNorm1d and feat.is_cuda and feat.dim() == 2
+            and feat.shape[1] in ops.BATCH_NORM_TRAIN_CHANNELS and feat.shape[0] > 1
+            and (module.running_mean is None or module.running_mean.dtype == torch.float32)
+            and (module.weight is None) == (module.bias is None)
+            and ops.wants_grad(feat, module.weight, module.bias))
 
 
 def _exact_gelu(module):
@@ -117,6 +126,14 @@ class PointSequential(PointModule):
                 if "sparse_conv_feat" in input:
                     input.sparse_conv_feat = input.sparse_conv_feat.replace_feature(input.feat)
                 skip = 2 if with_act else 1
+                continue
+            if isinstance(input, Point) and _trainable_bn(module, input.feat):
+                # training: batch statistics, the GELU behind it and their backward as one autograd node
+                with_act = _exact_gelu(nxt)
+                input.feat = BatchNormAct.apply(input.feat, module.weight, module.bias, module, with_act)
+                if "sparse_conv_feat" in input:
+                    input.sparse_conv_feat = input.sparse_conv_feat.replace_feature(input.feat)
+                skip = int(with_act)
                 continue
             if isinstance(input, Point) and _fusable_bn(module, input.feat):
                 with_act = _exact_gelu(nxt)
@@ -524,7 +541,9 @@ class SerializedPooling(PointModule):
         pooled = Point(fields)
         norm = self.norm[0] if self.norm is not None and len(self.norm) == 1 else None
         act = self.act[0] if self.act is not None and len(self.act) == 1 else None
-        if norm is not None and _fusable_bn(norm, pooled.feat) and _exact_gelu(act):
+        if norm is not None and _trainable_bn(norm, pooled.feat) and _exact_gelu(act):
+            pooled.feat = BatchNormAct.apply(pooled.feat, norm.weight, norm.bias, norm, True)
+        elif norm is not None and _fusable_bn(norm, pooled.feat) and _exact_gelu(act):
             pooled.feat = ops.bn_act(pooled.feat, norm.running_mean, norm.running_var, norm.weight, norm.bias,
                                      norm.eps, True)
         else:

@@ -1007,6 +1007,40 @@ def block_tail_fused(attn, shortcut, proj, ln2, fc1, fc2):
     return out
 
 
+BATCH_NORM_TRAIN_CHANNELS = (32, 64, 128, 256, 512)
+
+
+def batch_norm_stats(x, eps, momentum=0.0, running_mean=None, running_var=None):
+    """(3, C) fp32: mean, rsqrt(var + eps) and biased variance of the rows of x; float32 running averages, when
+    given, are updated in place as a BatchNorm1d in training mode does."""
+    _dev(x, running_mean, running_var)
+    lib = _lib.load()
+    x = x.contiguous()
+    n, c = x.shape
+    stats = torch.empty((3, c), dtype=torch.float32, device=x.device)
+    ws = torch.empty(2 * c, dtype=torch.float32, device=x.device)
+    _lib.check(lib.ptv3_batch_norm_stats(_ptr(x), _dtype_code(x), n, c, float(eps), float(momentum), _ptr(running_mean),
+                                         _ptr(running_var), _ptr(stats), _ptr(ws), _stream()), "ptv3_batch_norm_stats")
+    return stats
+
+
+def batch_norm_bwd(x, dout, stats, weight, bias, gelu, batch_stats):
+    """(dx, dweight, dbias) of [GELU of] BatchNorm1d over the rows of x; stats[0] = mean, stats[1] = rstd; the
+    parameter gradients in fp32."""
+    _dev(x, dout, stats, weight, bias)
+    lib = _lib.load()
+    x, dout = x.contiguous(), dout.contiguous()
+    n, c = x.shape
+    dx = torch.empty_like(x)
+    dwb = torch.empty((2, c), dtype=torch.float32, device=x.device)
+    w = None if weight is None else weight.contiguous()
+    b = None if bias is None else bias.to(w.dtype if w is not None else bias.dtype).contiguous()
+    _lib.check(lib.ptv3_batch_norm_bwd(_ptr(x), _dtype_code(x), _ptr(dout), _dtype_code(dout), _ptr(stats), _ptr(w), _ptr(b),
+                                       _code(w if w is not None else b), n, c, int(bool(gelu)), int(bool(batch_stats)),
+                                       _ptr(dx), _dtype_code(dx), _ptr(dwb), _stream()), "ptv3_batch_norm_bwd")
+    return dx, dwb[0], dwb[1]
+
+
 def bn_act(x, running_mean, running_var, weight, bias, eps, gelu):
     """Inference-mode BatchNorm1d, optionally followed by exact GELU, in one pass. The running
     statistics may be float32 or of x's dtype."""

@@ -148,6 +148,42 @@ def test_layer_norm_backward_parity(dtype, n, c):
     assert rel_err(bg.grad, br.grad) < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n,c,gelu,training", [(5000, 32, True, True), (777, 64, False, True), (2, 128, True, True),
+                                               (3001, 256, True, False), (900, 512, True, True)])
+def test_batch_norm_act_parity(dtype, n, c, gelu, training):
+    """BatchNorm1d (+ GELU) as one autograd node: result, running averages and all gradients against torch CPU in
+    fp32 on the same rounded inputs; a mean far from zero checks that the variance does not cancel."""
+    from pointtransformerv3_amd.autograd import BatchNormAct
+    g = torch.Generator().manual_seed(n + c)
+    x = (torch.randn(n, c, generator=g) * 1.5 + 6.0).to(dtype)
+    dout = torch.randn(n, c, generator=g).to(dtype)
+    ref = torch.nn.BatchNorm1d(c, eps=1e-3, momentum=0.01)
+    with torch.no_grad():
+        ref.weight.copy_(torch.rand(c, generator=g) + 0.5)
+        ref.bias.copy_(torch.randn(c, generator=g))
+        ref.running_mean.copy_(torch.randn(c, generator=g) + 6.0)
+        ref.running_var.copy_(torch.rand(c, generator=g) + 1.5)
+    import copy
+    mod = copy.deepcopy(ref).to(DEV)
+    ref.train(training)
+    mod.train(training)
+    xr = x.float().clone().requires_grad_(True)
+    want = ref(xr)
+    want = torch.nn.functional.gelu(want) if gelu else want
+    want.backward(dout.float())
+    xg = x.detach().to(DEV).requires_grad_(True)
+    out = BatchNormAct.apply(xg, mod.weight, mod.bias, mod, gelu)
+    out.backward(dout.to(DEV))
+    tol = TOL[dtype] if dtype != torch.float32 else 2e-4   # sums over thousands of rows in another order
+    assert out.dtype == dtype and rel_err(out, want) < tol
+    assert rel_err(xg.grad, xr.grad) < tol
+    assert rel_err(mod.weight.grad, ref.weight.grad) < tol
+    assert rel_err(mod.bias.grad, ref.bias.grad) < tol
+    assert rel_err(mod.running_mean, ref.running_mean) < 1e-4 and rel_err(mod.running_var, ref.running_var) < 1e-3
+    assert int(mod.num_batches_tracked) == int(ref.num_batches_tracked)
+
+
 @pytest.mark.parametrize("with_mask", [False, True])
 @pytest.mark.parametrize("skip_dtype,branch_dtype", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
                                                      (torch.float16, torch.float16)])
