@@ -32,8 +32,9 @@ class SubMConv(torch.autograd.Function):
     @staticmethod
     def forward(ctx, feat, weight, bias, sparse, module):
         cout, cin = weight.shape[0], weight.shape[-1]
-        w = weight.detach().reshape(cout, -1, cin)
-        out = module.convolve(sparse, feat.detach(), w, None if bias is None else bias.detach())
+        w = ops.cast_cached(weight, feat.dtype).detach().reshape(cout, -1, cin)
+        b = None if bias is None else ops.cast_cached(bias, feat.dtype).detach()
+        out = module.convolve(sparse, feat.detach(), w, b)
         ctx.save_for_backward(feat, weight)
         ctx.sparse, ctx.module, ctx.has_bias = sparse, module, bias is not None
         ctx.bias_dtype = None if bias is None else bias.dtype

@@ -47,16 +47,43 @@ def wants_grad(*tensors):
 _CAST_CACHE = {}
 
 
+def _refresh_stale_casts(dtype):
+    """Every remembered plain cast to dtype whose parameter has been written since (an optimizer step touches all
+    of them at once) is redone in place, in one multi-tensor copy instead of one small launch per parameter."""
+    dsts, srcs, entries = [], [], []
+    for key, (stamp, out, ref) in _CAST_CACHE.items():
+        if key[1] != dtype or key[2]:
+            continue
+        t = ref()
+        if t is None:
+            continue
+        now = (t.data_ptr(), t._version)
+        if now != stamp and out.shape == t.shape and out.device == t.device:
+            dsts.append(out)
+            srcs.append(t.detach())
+            entries.append((key, now, ref))
+    if dsts:
+        with torch.no_grad():
+            torch._foreach_copy_(dsts, srcs)
+        for (key, now, ref), out in zip(entries, dsts):
+            _CAST_CACHE[key] = (now, out, ref)
+
+
 def cast_cached(t, dtype, transpose=False):
     """t.to(dtype) (transposed and made contiguous if asked) for a parameter, remembered until the parameter is
-    written to or moved: training casts every weight on every use, twice per step and layer otherwise."""
+    written to or moved: training casts every weight on every use, twice per step and layer otherwise. The
+    result must not be kept across optimizer steps: it is overwritten when the parameter changes."""
     if t.dtype == dtype and not transpose:
         return t
     key = (id(t), dtype, transpose)
     stamp = (t.data_ptr(), t._version)
     hit = _CAST_CACHE.get(key)
-    if hit is not None and hit[0] == stamp and hit[2]() is t:
-        return hit[1]
+    if hit is not None and hit[2]() is t:
+        if hit[0] != stamp and not transpose:
+            _refresh_stale_casts(dtype)
+            hit = _CAST_CACHE.get(key)
+        if hit[0] == stamp:
+            return hit[1]
     with torch.no_grad():
         out = (t.detach().t() if transpose else t.detach()).to(dtype).contiguous()
     import weakref

@@ -104,8 +104,8 @@ def test_forward_on_cpu_tensors_fails_loudly():
 
 
 def test_cast_cache_follows_in_place_updates_and_replacement():
-    """Weights are cast once per update, not once per use: the remembered copy must go stale when the
-    parameter is written in place (an optimizer step) or its storage is replaced."""
+    """Weights are cast once per update, not once per use: the remembered copy must follow the parameter when
+    it is written in place (an optimizer step: all stale copies are redone together) or its storage is replaced."""
     import torch
     from pointtransformerv3_amd import ops
     p = torch.nn.Parameter(torch.arange(6, dtype=torch.float32).reshape(2, 3))
@@ -115,8 +115,14 @@ def test_cast_cache_follows_in_place_updates_and_replacement():
     assert t.shape == (3, 2) and t.is_contiguous() and torch.equal(t, a.t())
     with torch.no_grad():
         p.add_(1.0)
+    q = torch.nn.Parameter(torch.ones(4))
+    qa = ops.cast_cached(q, torch.bfloat16)
+    with torch.no_grad():
+        q.mul_(3.0)
     b = ops.cast_cached(p, torch.bfloat16)
-    assert b is not a and torch.equal(b.float(), p.detach())
+    assert torch.equal(b.float(), p.detach())
+    assert torch.equal(qa.float(), q.detach())          # redone in the same sweep, in place
+    assert torch.equal(ops.cast_cached(p, torch.bfloat16, transpose=True).float(), p.detach().t())
     p.data = torch.zeros(2, 3)
     assert torch.equal(ops.cast_cached(p, torch.bfloat16).float(), torch.zeros(2, 3))
     assert ops.cast_cached(p, torch.float32) is p
