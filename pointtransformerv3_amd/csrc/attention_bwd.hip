@@ -84,13 +84,29 @@ __device__ __forceinline__ f32x16 splat16(float x) {
     return r;
 }
 
+// Work-group id -> (item, part of parts): the first full_items work-groups take one (sequence, head) item each;
+// the items of the last, partly filled round of resident work-groups are cut into `split` ranges of tiles, one
+// work-group each, so that the round is short (every range stages the sequence again).
+__device__ __forceinline__ void item_of_block(int full_items, int split, int* item, int* part, int* parts) {
+    if ((int)blockIdx.x < full_items) {
+        *item = blockIdx.x;
+        *part = 0;
+        *parts = 1;
+    } else {
+        const int r = blockIdx.x - full_items;
+        *item = full_items + r / split;
+        *part = r % split;
+        *parts = split;
+    }
+}
+
 // ---- kernel 1: one work-group per (sequence, head), a wave per 32-query tile
 template <typename T, bool HAVE_LSE>
 __global__ __launch_bounds__(BWQ_THREADS) void attn_bwd_q_kernel(
     const T* __restrict__ qkv, const T* __restrict__ out, const T* __restrict__ dout, int channels, int heads,
     const int32_t* __restrict__ slot_src, const int32_t* __restrict__ slot_dst,
     const int32_t* __restrict__ cu_seqlens, int lds_keys, float scale, int64_t n_pad, T* __restrict__ dqkv,
-    float* lse_ws, float* __restrict__ d_ws) {
+    float* lse_ws, float* __restrict__ d_ws, int full_items, int split) {
     typedef typename Half<T>::v8 v8;
     extern __shared__ __align__(16) unsigned char smem[];
     // K rows, V rows, K^T, 96 B of zeros
@@ -100,7 +116,9 @@ __global__ __launch_bounds__(BWQ_THREADS) void attn_bwd_q_kernel(
     unsigned char* kt_lds = v_lds + (size_t)lds_keys * 32;
     unsigned char* zero_lds = kt_lds + (size_t)HD * kt_stride;
 
-    const int seq = blockIdx.x / heads, head = blockIdx.x % heads;
+    int item, part, parts;
+    item_of_block(full_items, split, &item, &part, &parts);
+    const int seq = item / heads, head = item % heads;
     const int s0 = cu_seqlens[seq];
     const int len = cu_seqlens[seq + 1] - s0;
     if (len <= 0) return;
@@ -133,7 +151,8 @@ __global__ __launch_bounds__(BWQ_THREADS) void attn_bwd_q_kernel(
     const unsigned char* kt_base = col < HD ? kt_lds + (size_t)col * kt_stride + hf * 32 : zero_lds;
     const int kt_step = col < HD ? 128 : 0;
 
-    for (int qt = wave; qt < n_qtiles; qt += BWQ_WAVES) {
+    const int qt_lo = (int)((int64_t)part * n_qtiles / parts), qt_hi = (int)((int64_t)(part + 1) * n_qtiles / parts);
+    for (int qt = qt_lo + wave; qt < qt_hi; qt += BWQ_WAVES) {
         const int qi = qt * 32 + col;
         int dst = -1;
         u32x4 qreg = {0, 0, 0, 0}, doreg = {0, 0, 0, 0}, oreg = {0, 0, 0, 0};
@@ -241,7 +260,8 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_kv_kernel(
     const T* __restrict__ qkv, const T* __restrict__ dout, int channels, int heads,
     const int32_t* __restrict__ slot_src, const int32_t* __restrict__ slot_dst,
     const int32_t* __restrict__ cu_seqlens, int lds_keys, float scale, int64_t n_pad,
-    const float* __restrict__ lse_ws, const float* __restrict__ d_ws, T* __restrict__ dqkv, T* __restrict__ fill) {
+    const float* __restrict__ lse_ws, const float* __restrict__ d_ws, T* __restrict__ dqkv, T* __restrict__ fill,
+    int full_items, int split) {
     typedef typename Half<T>::v8 v8;
     typedef float f32x4 __attribute__((ext_vector_type(4)));
     extern __shared__ __align__(16) unsigned char smem[];
@@ -254,7 +274,9 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_kv_kernel(
     float* nd_lds = nlse_lds + lds_keys;
     unsigned char* zero_lds = (unsigned char*)(nd_lds + lds_keys);
 
-    const int seq = blockIdx.x / heads, head = blockIdx.x % heads;
+    int item, part, parts;
+    item_of_block(full_items, split, &item, &part, &parts);
+    const int seq = item / heads, head = item % heads;
     const int s0 = cu_seqlens[seq];
     const int len = cu_seqlens[seq + 1] - s0;
     if (len <= 0) return;
@@ -299,7 +321,8 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_kv_kernel(
     // Two key tiles per sweep over the queries: the query-side operands of a step (Q and dO rows, their
     // transposes, -lse and -D: 28 16-byte LDS reads) are fetched once and used for both, which halves the
     // LDS traffic per MFMA -- with one tile the kernel is bound by LDS bandwidth.
-    for (int kt = wave; kt < n_ktiles; kt += 2 * BWD_WAVES) {
+    const int kt_lo = (int)((int64_t)part * n_ktiles / parts), kt_hi = (int)((int64_t)(part + 1) * n_ktiles / parts);
+    for (int kt = kt_lo + wave; kt < kt_hi; kt += 2 * BWD_WAVES) {
         int key[2], kdst[2];
         int64_t row[2];
         bool valid[2];
@@ -308,7 +331,7 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_kv_kernel(
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             key[t] = (kt + t * BWD_WAVES) * 32 + col;
-            valid[t] = key[t] < len;
+            valid[t] = key[t] < len && kt + t * BWD_WAVES < kt_hi;
             row[t] = 0;
             kdst[t] = -1;
             u32x4 kreg = {0, 0, 0, 0}, vreg = {0, 0, 0, 0};
@@ -323,7 +346,7 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_kv_kernel(
             acc_v[t] = splat16(0.f);
             acc_k[t] = splat16(0.f);
         }
-        const bool two = kt + BWD_WAVES < n_ktiles;   // the same for every lane of the wave
+        const bool two = kt + BWD_WAVES < kt_hi;   // the same for every lane of the wave
         const unsigned char* qt_ptr = qt_base;
         const unsigned char* dot_ptr = dot_base;
         for (int st = 0; st < n_pairs; ++st) {
@@ -634,12 +657,34 @@ int launch_half_bwd(const void* qkv, const void* out, const void* dout, int chan
         if (e != hipSuccess) return (int)e;
         allowed_kv = lds_kv;
     }
-    const unsigned grid = (unsigned)(n_seq * heads);
+    // one work-group per CU is resident (LDS): the items beyond the last full round are cut into ranges of
+    // tiles when that shortens the round (each range stages the sequence again, about 0.15 of an item)
+    static int slots = 0;
+    if (slots == 0) {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        slots = cus;
+    }
+    const int64_t total = n_seq * heads;
+    const int64_t rem = total % slots;
+    int64_t full = total - rem, split = 1;
+    if (rem != 0) {
+        double best = 1.0;
+        for (int64_t sp = 2; sp <= 4; ++sp) {
+            const double cost = (double)((rem * sp + slots - 1) / slots) * (1.0 / (double)sp + 0.15);
+            if (cost < best - 1e-9) { best = cost; split = sp; }
+        }
+    }
+    if (split == 1) full = total;
+    const unsigned grid = (unsigned)(full + (total - full) * split);
     hipLaunchKernelGGL(kq, dim3(grid), dim3(BWQ_THREADS), lds_q, stream, (const T*)qkv, (const T*)out, (const T*)dout,
-                       channels, heads, slot_src, slot_dst, cu_seqlens, lds_keys, scale, n_pad, (T*)dqkv, lse_buf, ws.d);
+                       channels, heads, slot_src, slot_dst, cu_seqlens, lds_keys, scale, n_pad, (T*)dqkv, lse_buf, ws.d,
+                       (int)full, (int)split);
     hipLaunchKernelGGL(kkv, dim3(grid), dim3(BWD_THREADS), lds_kv, stream, (const T*)qkv, (const T*)dout, channels,
                        heads, slot_src, slot_dst, cu_seqlens, lds_keys, scale, n_pad, lse_buf, ws.d, (T*)dqkv,
-                       (T*)ws.fill);
+                       (T*)ws.fill, (int)full, (int)split);
     const int64_t items = n_pad * (2 * channels / 8);
     hipLaunchKernelGGL(attn_bwd_fill_kernel<T>, dim3((unsigned)ptv3_ceil_div(items, 256)), dim3(256), 0, stream,
                        (const T*)ws.fill, channels, slot_src, slot_dst, n_pad, (T*)dqkv);
