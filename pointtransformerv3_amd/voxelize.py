@@ -9,7 +9,7 @@ import torch
 from . import ops
 
 
-@torch.inference_mode()
+@torch.no_grad()   # not inference_mode: the returned features may enter a training step
 def grid_sample(coord, offset, grid_size, feat=None, keys=()):
     """coord (N,3) float, offset (B,) cumulative scene ends, both on the GPU.
 

@@ -374,3 +374,20 @@ def test_training_step_of_model_variants(variant):
     assert all(torch.isfinite(p.grad).all() for p in model.parameters() if p.grad is not None)
     if variant == "input_gradient":
         assert x.grad is not None and torch.isfinite(x.grad).all() and x.grad.abs().max() > 0
+
+
+def test_training_on_the_output_of_grid_sample():
+    """Raw points -> device voxelisation -> a training step: the batch must be usable under autograd."""
+    from pointtransformerv3_amd import synthetic, voxelize
+    raw = [synthetic.room_points(6000, 70 + i).astype(np.float32) for i in range(2)]
+    coord = torch.from_numpy(np.concatenate(raw)).to(DEV)
+    offset = torch.from_numpy(np.cumsum([len(r) for r in raw])).to(DEV)
+    feat = torch.rand(len(coord), 6, generator=torch.Generator().manual_seed(1)).to(DEV)
+    batch = voxelize.grid_sample(coord, offset, 0.05, feat=feat)
+    torch.manual_seed(2)
+    model, _ = _small_model()
+    model = model.to(DEV).train()
+    with torch.autocast("cuda", dtype=torch.float16):
+        out = model({k: batch[k] for k in ("feat", "grid_coord", "coord", "offset")}).feat
+    out.float().square().mean().backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in model.parameters())
