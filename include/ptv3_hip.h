@@ -60,11 +60,13 @@ int ptv3_grid_max(const int32_t *grid_coord, int64_t n, int32_t *out3, void *str
  * of every input point's voxel among the kept ones (or NULL), offset_out (n_scenes,) int64 = scene
  * ends of the kept points, counts (2,) int64 on the device = {m, status}; status 1 means a grid
  * coordinate needs more than 16 bits (the serialization's limit, model.py:108) and the rest is
- * meaningless. n < 2^30. */
+ * meaningless. n < 2^30. pick_seed 0 keeps the first point in input order (GridSample's test mode); any other
+ * value keeps a member of every voxel drawn uniformly, a different draw per seed (its train mode; the
+ * random stream is this library's own, not numpy's). */
 size_t ptv3_voxelize_workspace_bytes(int64_t n, int n_scenes);
 int ptv3_voxelize(const float *coord, int64_t n, const int64_t *offset, int n_scenes, float grid_size,
                   int32_t *grid_coord, int64_t *index, int64_t *inverse, int64_t *offset_out,
-                  int64_t *counts, void *workspace, size_t workspace_bytes, void *stream);
+                  int64_t *counts, uint32_t pick_seed, void *workspace, size_t workspace_bytes, void *stream);
 
 /* model.py:35-40 (offset2batch): scene id of each of the n points from the cumulative scene ends
  * offset (n_scenes,) int64 on the device, n = offset[n_scenes - 1] known to the caller. */

@@ -20,7 +20,7 @@ constexpr uint64_t VX_EMPTY = ~0ull;
 
 struct VoxWs {
     uint64_t* keys;       // [cap]
-    int32_t* first;       // [cap] lowest point index of the voxel
+    int32_t* first;       // [cap] lowest rank among the voxel's points (seed 0: lowest point index)
     int32_t* voxel;       // [cap] position of the voxel among the kept points
     int32_t* slot_of;     // [n]
     uint32_t* block_cnt;  // [blocks]
@@ -145,9 +145,29 @@ __device__ __forceinline__ void vx_grid(const float* __restrict__ coord, int64_t
     for (int a = 0; a < 3; ++a) g[a] = (int32_t)floorf((coord[3 * i + a] - ord2f(w.scene_min[3 * s + a])) / grid_size);
 }
 
+// Rank of point i among the points of its voxel: the point with the lowest rank is kept. Seed 0: the
+// index itself (the first point in input order, GridSample's test mode). Otherwise a bijection of the
+// 32-bit index keyed by the seed (odd multiplications and xor-shifts, each invertible), so ranks never tie
+// and the lowest belongs to a member drawn uniformly -- GridSample's train mode, which takes a random
+// member of every voxel.
+__device__ __forceinline__ int32_t vx_rank(int64_t i, uint32_t seed) {
+    uint32_t x = (uint32_t)i;
+    if (seed != 0u) {
+        x ^= seed;
+        x *= 0x9E3779B1u;
+        x ^= x >> 15;
+        x *= 0x85EBCA77u;
+        x ^= x >> 13;
+        x *= 0xC2B2AE3Du;
+        x ^= x >> 16;
+        x += seed * 0x27D4EB2Fu;
+    }
+    return (int32_t)x;
+}
+
 __global__ __launch_bounds__(VX_THREADS) void vx_insert_kernel(const float* __restrict__ coord, int64_t n,
                                                                const int64_t* __restrict__ offset, int nb,
-                                                               float grid_size, VoxWs w) {
+                                                               float grid_size, VoxWs w, uint32_t seed) {
     const int64_t i = (int64_t)blockIdx.x * VX_THREADS + threadIdx.x;
     if (i >= n) return;
     const int s = scene_of(offset, nb, i);
@@ -161,7 +181,7 @@ __global__ __launch_bounds__(VX_THREADS) void vx_insert_kernel(const float* __re
         const uint64_t prev = atomicCAS((unsigned long long*)&w.keys[slot], (unsigned long long)VX_EMPTY,
                                         (unsigned long long)key);
         if (prev == VX_EMPTY || prev == key) {
-            atomicMin(&w.first[slot], (int32_t)i);
+            atomicMin(&w.first[slot], vx_rank(i, seed));
             w.slot_of[i] = (int32_t)slot;
             return;
         }
@@ -192,9 +212,9 @@ __device__ __forceinline__ uint32_t vx_block_scan(uint32_t v, uint32_t* total) {
     return x + base;
 }
 
-__global__ __launch_bounds__(VX_THREADS) void vx_count_kernel(int64_t n, VoxWs w) {
+__global__ __launch_bounds__(VX_THREADS) void vx_count_kernel(int64_t n, VoxWs w, uint32_t seed) {
     const int64_t i = (int64_t)blockIdx.x * VX_THREADS + threadIdx.x;
-    const uint32_t keep = (i < n && w.first[w.slot_of[i]] == (int32_t)i) ? 1u : 0u;
+    const uint32_t keep = (i < n && w.first[w.slot_of[i]] == vx_rank(i, seed)) ? 1u : 0u;
     uint32_t total;
     vx_block_scan(keep, &total);
     if (threadIdx.x == 0) w.block_cnt[blockIdx.x] = total;
@@ -221,11 +241,11 @@ __global__ __launch_bounds__(VX_THREADS) void vx_assign_kernel(const float* __re
                                                                const int64_t* __restrict__ offset, int nb,
                                                                float grid_size, VoxWs w, int32_t* __restrict__ grid_out,
                                                                int64_t* __restrict__ index_out,
-                                                               int64_t* __restrict__ offset_out) {
+                                                               int64_t* __restrict__ offset_out, uint32_t seed) {
     const int64_t i = (int64_t)blockIdx.x * VX_THREADS + threadIdx.x;
     const bool live = i < n;
     const int32_t slot = live ? w.slot_of[i] : 0;
-    const bool keep = live && w.first[slot] == (int32_t)i;
+    const bool keep = live && w.first[slot] == vx_rank(i, seed);
     uint32_t total;
     const uint32_t inc = vx_block_scan(keep ? 1u : 0u, &total);
     if (!live) return;
@@ -259,7 +279,8 @@ extern "C" size_t ptv3_voxelize_workspace_bytes(int64_t n, int n_scenes) {
 
 extern "C" int ptv3_voxelize(const float* coord, int64_t n, const int64_t* offset, int n_scenes, float grid_size,
                              int32_t* grid_coord, int64_t* index, int64_t* inverse, int64_t* offset_out,
-                             int64_t* counts, void* workspace, size_t workspace_bytes, void* stream_) {
+                             int64_t* counts, uint32_t pick_seed, void* workspace, size_t workspace_bytes,
+                             void* stream_) {
     if (n < 1 || n >= (1ll << 30) || n_scenes < 1 || n_scenes > 65535 || !(grid_size > 0.f)) return PTV3_EINVAL;
     if (!coord || !offset || !grid_coord || !index || !offset_out || !counts || !workspace) return PTV3_EINVAL;
     VoxWs w = vx_carve(workspace, n, n_scenes);
@@ -272,11 +293,11 @@ extern "C" int ptv3_voxelize(const float* coord, int64_t n, const int64_t* offse
     hipLaunchKernelGGL(vx_scene_min_kernel, dim3((unsigned)ptv3_ceil_div(n, VX_THREADS * VX_MIN_ITERS)), dim3(VX_THREADS),
                        0, stream, coord, n, offset, n_scenes, w);
     hipLaunchKernelGGL(vx_insert_kernel, dim3((unsigned)blocks), dim3(VX_THREADS), 0, stream, coord, n, offset,
-                       n_scenes, grid_size, w);
-    hipLaunchKernelGGL(vx_count_kernel, dim3((unsigned)blocks), dim3(VX_THREADS), 0, stream, n, w);
+                       n_scenes, grid_size, w, pick_seed);
+    hipLaunchKernelGGL(vx_count_kernel, dim3((unsigned)blocks), dim3(VX_THREADS), 0, stream, n, w, pick_seed);
     hipLaunchKernelGGL(vx_scan_kernel, dim3(1), dim3(VX_THREADS), 0, stream, w, blocks, counts);
     hipLaunchKernelGGL(vx_assign_kernel, dim3((unsigned)blocks), dim3(VX_THREADS), 0, stream, coord, n, offset,
-                       n_scenes, grid_size, w, grid_coord, index, offset_out);
+                       n_scenes, grid_size, w, grid_coord, index, offset_out, pick_seed);
     if (inverse)
         hipLaunchKernelGGL(vx_inverse_kernel, dim3((unsigned)blocks), dim3(VX_THREADS), 0, stream, n, w, inverse);
     PTV3_RETURN_LAUNCH();

@@ -154,8 +154,9 @@ def grid_max(grid_coord):
     return out
 
 
-def voxelize(coord, offset, grid_size, with_inverse=True):
-    """Per scene grid_coord = floor((coord - scene minimum) / grid_size), first point of every voxel kept.
+def voxelize(coord, offset, grid_size, with_inverse=True, seed=0):
+    """Per scene grid_coord = floor((coord - scene minimum) / grid_size), one point of every voxel kept: the first
+    in input order when seed is 0, else a member drawn uniformly (another draw for another 32-bit seed).
 
     coord (N,3) float32 and offset (B,) cumulative scene ends on the device. Returns a dict:
     grid_coord (M,3) int32 and index (M,) int64 of the kept points in input order, offset (B,) int64
@@ -174,7 +175,8 @@ def voxelize(coord, offset, grid_size, with_inverse=True):
     nbytes = lib.ptv3_voxelize_workspace_bytes(n, nb)
     ws = _ws(nbytes, dev)
     _lib.check(lib.ptv3_voxelize(_ptr(coord), n, _ptr(off), nb, float(grid_size), _ptr(grid), _ptr(index), _ptr(inverse),
-                                 _ptr(off_out), _ptr(counts), _ptr(ws), nbytes, _stream()), "ptv3_voxelize")
+                                 _ptr(off_out), _ptr(counts), int(seed) & 0xFFFFFFFF, _ptr(ws), nbytes, _stream()),
+               "ptv3_voxelize")
     m, status = Readback(counts).get()
     if status:
         raise RuntimeError("voxelize: a grid coordinate does not fit 16 bits (grid_size too small for the scene extent)")

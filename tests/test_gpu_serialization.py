@@ -155,3 +155,46 @@ def test_voxelize_rejects_extents_beyond_16_bits():
     coord = torch.tensor([[0.0, 0.0, 0.0], [700.0, 0.0, 0.0]], device=DEV)
     with pytest.raises(RuntimeError, match="16 bits"):
         ops.voxelize(coord, torch.tensor([2], device=DEV), 0.01)
+
+
+def test_voxelize_train_mode_draws_a_uniform_member_of_every_voxel():
+    """GridSample's train mode: one random member per voxel. Checked by what any correct draw satisfies: the same
+    voxels as the first-point mode, every kept point inside its voxel, `inverse` consistent, another seed another
+    draw, and over many two-point voxels each member kept about half of the time."""
+    from pointtransformerv3_amd import ops, voxelize
+    rng = np.random.default_rng(5)
+    sizes = [60_000, 45_000]
+    coord = np.concatenate([rng.random((n, 3)) * np.array([4.0, 4.0, 0.2]) + rng.normal(0, 20, 3) for n in sizes]).astype(np.float32)
+    offset = np.cumsum(sizes).astype(np.int64)
+    grid = 0.05
+    wg, wi, winv, wends = OI.voxelize(coord, offset, grid)
+    c, o = torch.from_numpy(coord).to(DEV), torch.from_numpy(offset).to(DEV)
+    draws = [ops.voxelize(c, o, grid, seed=s) for s in (1, 2, 12345)]
+    scene = np.searchsorted(offset, np.arange(len(coord)), side="right")
+    first_voxel = winv                                            # voxel id (first-point numbering) of every input point
+    for d in draws:
+        idx = d["index"].cpu().numpy()
+        assert len(idx) == len(wi) and np.all(np.diff(idx) > 0)   # kept points in input order, one per voxel
+        assert np.array_equal(np.sort(first_voxel[idx]), np.arange(len(wi)))   # exactly one from every voxel
+        assert np.array_equal(d["offset"].cpu().numpy(), wends)
+        g = d["grid_coord"].cpu().numpy()
+        assert np.array_equal(g, wg[first_voxel[idx]])            # its grid coordinate is its voxel's
+        inv = d["inverse"].cpu().numpy()
+        assert np.array_equal(first_voxel[idx[inv]], first_voxel) and np.array_equal(scene[idx[inv]], scene)
+    a, b = draws[0]["index"].cpu().numpy(), draws[1]["index"].cpu().numpy()
+    assert (a != b).mean() > 0.2
+    # two-member voxels: the first member is kept in about half of them, for every seed
+    counts = np.bincount(first_voxel, minlength=len(wi))
+    pairs = np.nonzero(counts == 2)[0]
+    assert len(pairs) > 3000
+    for d in draws:
+        idx = d["index"].cpu().numpy()
+        kept_of = np.empty(len(wi), np.int64)
+        kept_of[first_voxel[idx]] = idx
+        frac = (kept_of[pairs] == wi[pairs]).mean()
+        assert abs(frac - 0.5) < 4 * 0.5 / np.sqrt(len(pairs)), frac
+    # seed 0 is the first-point mode; grid_sample's train mode keeps features and coordinates of the drawn points
+    assert np.array_equal(ops.voxelize(c, o, grid, seed=0)["index"].cpu().numpy(), wi)
+    feat = torch.from_numpy(rng.random((len(coord), 3)).astype(np.float32)).to(DEV)
+    batch = voxelize.grid_sample(c, o, grid, feat=feat, mode="train", seed=7)
+    assert torch.equal(batch["feat"], feat[batch["index"]]) and not np.array_equal(batch["index"].cpu().numpy(), wi)
