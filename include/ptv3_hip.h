@@ -140,6 +140,17 @@ int ptv3_patch_attn_bwd(const void *qkv, const void *out, const void *dout, int 
                         float scale, const float *lse, void *dqkv, void *workspace, size_t workspace_bytes,
                         void *stream);
 
+/* Backward of ptv3_patch_attn_rpe_fwd (fp32): as ptv3_patch_attn_bwd, with the relative position bias of
+ * model.py:297-316 in the scores; drpe_table (3 * R, heads) fp32 is accumulated into (zero it first):
+ * entry [a * R + c][h] += sum of dS(h, i, j) over the pairs (i, j) whose clamped offset along axis a is c.
+ * grid_coord == NULL: exactly ptv3_patch_attn_bwd. */
+int ptv3_patch_attn_rpe_bwd(const void *qkv, const void *out, const void *dout, int dtype, int64_t n_rows,
+                            int channels, int heads, const int32_t *slot_src, const int32_t *slot_dst,
+                            const int32_t *cu_seqlens, int64_t n_seq, int64_t max_seqlen, int64_t n_pad,
+                            float scale, const float *lse, const int32_t *grid_coord, const float *rpe_table,
+                            int pos_bnd, float *drpe_table, void *dqkv, void *workspace,
+                            size_t workspace_bytes, void *stream);
+
 /* spconv.SubMConv3d's index generation (call sites model.py:546-552, :767-774, tensor built
  * at :165-172). indices (n,4) int32 [batch,x,y,z], coordinates in [0, 65535];
  * nbr int32, entry (voxel i, tap t = (kx*ks+ky)*ks+kz) = row of the voxel at

@@ -25,6 +25,25 @@ class PatchAttention(torch.autograd.Function):
         return (ops.patch_attention_bwd(qkv, out, dout, *ctx.args, lse=ctx.lse),) + (None,) * 6
 
 
+class PatchAttentionRpe(torch.autograd.Function):
+    """Patch attention with the relative position bias (fp32, model.py:297-316, :463-471); the table takes a
+    gradient too."""
+
+    @staticmethod
+    def forward(ctx, qkv, rpe_table, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale, grid_coord, pos_bnd):
+        args = (num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale, grid_coord)
+        out = ops.patch_attention_rpe(qkv, *args, rpe_table.detach(), pos_bnd)
+        ctx.save_for_backward(qkv, out, rpe_table)
+        ctx.args, ctx.pos_bnd = args, pos_bnd
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        qkv, out, table = ctx.saved_tensors
+        dqkv, dtable = ops.patch_attention_rpe_bwd(qkv, out, dout, *ctx.args, table, ctx.pos_bnd)
+        return (dqkv, dtable.to(table.dtype)) + (None,) * 8
+
+
 class SubMConv(torch.autograd.Function):
     """module is the SubMConv3d whose forward dispatch (pair, tile or dense form) is reused for the
     input gradient; sparse is the SparseConvTensor that owns the neighbour maps."""

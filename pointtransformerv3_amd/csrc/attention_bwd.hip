@@ -428,13 +428,27 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_kv_kernel(
 constexpr int F32_B = 256;    // queries / keys per block
 constexpr int F32_C = 128;    // slots per chunk
 
+// Relative position bias of model.py:297-316, :468-469 on the fp32 path: score(query i, key j, head h) +=
+// sum over the axes a of table[a R + clamp(g_i[a] - g_j[a], -bnd, bnd) + bnd][h], R = 2 bnd + 1. grid == nullptr:
+// no bias. dtable (3 R, heads) receives the table's gradient (sum of dS over the pairs that read an entry).
+constexpr int RPE_MAX_BND = 128;
+struct Rpe {
+    const int32_t* grid;   // (n_rows, 3) grid coordinates in point order
+    const float* table;    // (3 R, heads)
+    float* dtable;         // (3 R, heads), accumulated into
+    int bnd;
+};
+__device__ __forceinline__ int rpe_index(int q, int k, int bnd) { return min(max(q - k, -bnd), bnd) + bnd; }
+
 __global__ __launch_bounds__(F32_B) void attn_bwd_q_f32_kernel(
     const float* __restrict__ qkv, const float* __restrict__ out, const float* __restrict__ dout, int channels,
     int heads, const int32_t* __restrict__ slot_src, const int32_t* __restrict__ slot_dst,
     const int32_t* __restrict__ cu_seqlens, int blocks, float scale, int64_t n_pad, float* __restrict__ dqkv,
-    float* __restrict__ lse_ws, float* __restrict__ d_ws) {
+    float* __restrict__ lse_ws, float* __restrict__ d_ws, Rpe rpe) {
     __shared__ float k_lds[F32_C][HD];
     __shared__ float v_lds[F32_C][HD];
+    __shared__ int32_t c_lds[F32_C][3];
+    __shared__ float t_lds[3 * (2 * RPE_MAX_BND + 1)], dt_lds[3 * (2 * RPE_MAX_BND + 1)];
     const int seq = blockIdx.x / (heads * blocks);
     const int rem = blockIdx.x % (heads * blocks);
     const int head = rem / blocks, qb = rem % blocks;
@@ -444,13 +458,25 @@ __global__ __launch_bounds__(F32_B) void attn_bwd_q_f32_kernel(
     const int tid = threadIdx.x;
     const int qi = qb * F32_B + tid;
     const int64_t row_stride = 3 * (int64_t)channels;
+    const int rnum = 2 * rpe.bnd + 1;
+    if (rpe.grid) {
+        for (int e = tid; e < 3 * rnum; e += F32_B) {
+            t_lds[e] = rpe.table[(int64_t)e * heads + head];
+            dt_lds[e] = 0.f;
+        }
+    }
 
     float q[HD], g[HD], dq[HD];
-    int dst = -1;
+    int dst = -1, qx = 0, qy = 0, qz = 0;
     float dsum = 0.f;
 #pragma unroll
     for (int d = 0; d < HD; ++d) { q[d] = 0.f; g[d] = 0.f; dq[d] = 0.f; }
     if (qi < len) dst = slot_dst[s0 + qi];
+    if (dst >= 0 && rpe.grid) {
+        qx = rpe.grid[3 * (int64_t)dst];
+        qy = rpe.grid[3 * (int64_t)dst + 1];
+        qz = rpe.grid[3 * (int64_t)dst + 2];
+    }
     if (dst >= 0) {
         const float* src = qkv + (int64_t)dst * row_stride + head * HD;
         const float* gs = dout + (int64_t)dst * channels + head * HD;
@@ -470,9 +496,11 @@ __global__ __launch_bounds__(F32_B) void attn_bwd_q_f32_kernel(
                 const int key = e / HD, d = e % HD;
                 float kv = 0.f, vv = 0.f;
                 if (c0 + key < len) {
-                    const float* src = qkv + (int64_t)slot_src[s0 + c0 + key] * row_stride + head * HD + d;
+                    const int64_t r = slot_src[s0 + c0 + key];
+                    const float* src = qkv + r * row_stride + head * HD + d;
                     kv = src[channels];
                     vv = src[2 * channels];
+                    if (rpe.grid && d < 3) c_lds[key][d] = rpe.grid[3 * r + d];
                 }
                 k_lds[key][d] = kv;
                 v_lds[key][d] = vv;
@@ -483,6 +511,13 @@ __global__ __launch_bounds__(F32_B) void attn_bwd_q_f32_kernel(
                 float s = 0.f;
 #pragma unroll
                 for (int d = 0; d < HD; ++d) s = fmaf(q[d], k_lds[key][d], s);
+                int bx = 0, by = 0, bz = 0;
+                if (rpe.grid) {
+                    bx = rpe_index(qx, c_lds[key][0], rpe.bnd);
+                    by = rnum + rpe_index(qy, c_lds[key][1], rpe.bnd);
+                    bz = 2 * rnum + rpe_index(qz, c_lds[key][2], rpe.bnd);
+                    s += t_lds[bx] + t_lds[by] + t_lds[bz];
+                }
                 if (sweep == 0) {
                     if (s > m) {
                         l *= __expf(m - s);
@@ -497,6 +532,11 @@ __global__ __launch_bounds__(F32_B) void attn_bwd_q_f32_kernel(
                     const float ds = p * (dp - dsum);
 #pragma unroll
                     for (int d = 0; d < HD; ++d) dq[d] = fmaf(ds, k_lds[key][d], dq[d]);
+                    if (rpe.grid && dst >= 0) {   // every (query, key) pair is seen exactly once, here
+                        atomicAdd(&dt_lds[bx], ds);
+                        atomicAdd(&dt_lds[by], ds);
+                        atomicAdd(&dt_lds[bz], ds);
+                    }
                 }
             }
         }
@@ -509,6 +549,11 @@ __global__ __launch_bounds__(F32_B) void attn_bwd_q_f32_kernel(
         lse_ws[(int64_t)head * n_pad + s0 + qi] = lse;   // natural-log units on this path
         d_ws[(int64_t)head * n_pad + s0 + qi] = dsum;
     }
+    if (rpe.grid) {
+        __syncthreads();
+        for (int e = tid; e < 3 * rnum; e += F32_B)
+            if (dt_lds[e] != 0.f) atomicAdd(rpe.dtable + (int64_t)e * heads + head, dt_lds[e]);
+    }
 }
 
 __global__ __launch_bounds__(F32_B) void attn_bwd_kv_f32_kernel(
@@ -516,11 +561,13 @@ __global__ __launch_bounds__(F32_B) void attn_bwd_kv_f32_kernel(
     const int32_t* __restrict__ slot_src, const int32_t* __restrict__ slot_dst,
     const int32_t* __restrict__ cu_seqlens, int blocks, float scale, int64_t n_pad,
     const float* __restrict__ lse_ws, const float* __restrict__ d_ws, float* __restrict__ dqkv,
-    float* __restrict__ fill) {
+    float* __restrict__ fill, Rpe rpe) {
     __shared__ float q_lds[F32_C][HD];    // q * scale
     __shared__ float g_lds[F32_C][HD];    // dO
     __shared__ float lse_lds[F32_C];
     __shared__ float d_lds[F32_C];
+    __shared__ int32_t c_lds[F32_C][3];
+    __shared__ float t_lds[3 * (2 * RPE_MAX_BND + 1)];
     const int seq = blockIdx.x / (heads * blocks);
     const int rem = blockIdx.x % (heads * blocks);
     const int head = rem / blocks, kb = rem % blocks;
@@ -531,10 +578,20 @@ __global__ __launch_bounds__(F32_B) void attn_bwd_kv_f32_kernel(
     const int ki = kb * F32_B + tid;
     const int64_t row_stride = 3 * (int64_t)channels;
 
+    const int rnum = 2 * rpe.bnd + 1;
+    if (rpe.grid)
+        for (int e = tid; e < 3 * rnum; e += F32_B) t_lds[e] = rpe.table[(int64_t)e * heads + head];
     float k[HD], v[HD], dk[HD], dv[HD];
     int64_t row = 0;
+    int kx = 0, ky = 0, kz = 0;
 #pragma unroll
     for (int d = 0; d < HD; ++d) { k[d] = 0.f; v[d] = 0.f; dk[d] = 0.f; dv[d] = 0.f; }
+    if (ki < len && rpe.grid) {
+        const int64_t r = slot_src[s0 + ki];
+        kx = rpe.grid[3 * r];
+        ky = rpe.grid[3 * r + 1];
+        kz = rpe.grid[3 * r + 2];
+    }
     if (ki < len) {
         row = slot_src[s0 + ki];
         const float* src = qkv + row * row_stride + head * HD;
@@ -554,6 +611,7 @@ __global__ __launch_bounds__(F32_B) void attn_bwd_kv_f32_kernel(
                 if (dst >= 0) {
                     qv = qkv[(int64_t)dst * row_stride + head * HD + d] * scale;
                     gv = dout[(int64_t)dst * channels + head * HD + d];
+                    if (rpe.grid && d < 3) c_lds[qi][d] = rpe.grid[3 * (int64_t)dst + d];
                 }
             }
             q_lds[qi][d] = qv;
@@ -573,6 +631,9 @@ __global__ __launch_bounds__(F32_B) void attn_bwd_kv_f32_kernel(
                 s = fmaf(q_lds[qi][d], k[d], s);
                 dp = fmaf(g_lds[qi][d], v[d], dp);
             }
+            if (rpe.grid && lse_lds[qi] != INFINITY)   // a real query: its coordinates are in c_lds
+                s += t_lds[rpe_index(c_lds[qi][0], kx, rpe.bnd)] + t_lds[rnum + rpe_index(c_lds[qi][1], ky, rpe.bnd)] +
+                     t_lds[2 * rnum + rpe_index(c_lds[qi][2], kz, rpe.bnd)];
             const float p = __expf(s - lse_lds[qi]);
             const float ds = p * (dp - d_lds[qi]);
 #pragma unroll
@@ -703,6 +764,20 @@ extern "C" int ptv3_patch_attn_bwd(const void* qkv, const void* out, const void*
                                    const int32_t* cu_seqlens, int64_t n_seq, int64_t max_seqlen, int64_t n_pad,
                                    float scale, const float* lse, void* dqkv, void* workspace, size_t workspace_bytes,
                                    void* stream_) {
+    return ptv3_patch_attn_rpe_bwd(qkv, out, dout, dtype, n_rows, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
+                                   max_seqlen, n_pad, scale, lse, nullptr, nullptr, 0, nullptr, dqkv, workspace,
+                                   workspace_bytes, stream_);
+}
+
+extern "C" int ptv3_patch_attn_rpe_bwd(const void* qkv, const void* out, const void* dout, int dtype, int64_t n_rows,
+                                       int channels, int heads, const int32_t* slot_src, const int32_t* slot_dst,
+                                       const int32_t* cu_seqlens, int64_t n_seq, int64_t max_seqlen, int64_t n_pad,
+                                       float scale, const float* lse, const int32_t* grid_coord, const float* rpe_table,
+                                       int pos_bnd, float* drpe_table, void* dqkv, void* workspace,
+                                       size_t workspace_bytes, void* stream_) {
+    if (grid_coord && (dtype != PTV3_F32 || !rpe_table || !drpe_table)) return PTV3_ESHAPE;   // the bias lives on the fp32 path
+    if (grid_coord && (pos_bnd < 0 || pos_bnd > RPE_MAX_BND)) return PTV3_ESHAPE;
+    const Rpe rpe = {grid_coord, rpe_table, drpe_table, grid_coord ? pos_bnd : 0};
     if (n_rows < 0 || n_seq < 0 || n_pad < 0 || channels < 1 || heads < 1 || max_seqlen < 1) return PTV3_EINVAL;
     if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
     if (channels % heads != 0 || channels / heads != HD) return PTV3_ESHAPE;
@@ -723,10 +798,10 @@ extern "C" int ptv3_patch_attn_bwd(const void* qkv, const void* out, const void*
     const unsigned grid = (unsigned)(n_seq * heads * blocks);
     hipLaunchKernelGGL(attn_bwd_q_f32_kernel, dim3(grid), dim3(F32_B), 0, stream, (const float*)qkv, (const float*)out,
                        (const float*)dout, channels, heads, slot_src, slot_dst, cu_seqlens, blocks, scale, n_pad,
-                       (float*)dqkv, ws.lse, ws.d);
+                       (float*)dqkv, ws.lse, ws.d, rpe);
     hipLaunchKernelGGL(attn_bwd_kv_f32_kernel, dim3(grid), dim3(F32_B), 0, stream, (const float*)qkv,
                        (const float*)dout, channels, heads, slot_src, slot_dst, cu_seqlens, blocks, scale, n_pad, ws.lse,
-                       ws.d, (float*)dqkv, (float*)ws.fill);
+                       ws.d, (float*)dqkv, (float*)ws.fill, rpe);
     const int64_t items = n_pad * (2 * channels / 8);
     hipLaunchKernelGGL(attn_bwd_fill_kernel<float>, dim3((unsigned)ptv3_ceil_div(items, 256)), dim3(256), 0, stream,
                        (const float*)ws.fill, channels, slot_src, slot_dst, n_pad, (float*)dqkv);

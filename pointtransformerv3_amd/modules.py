@@ -274,9 +274,12 @@ class SerializedAttention(PointModule):
             self.patch_size = min(int(sizes.min()), self.patch_size_max)
         _, _, cu_seqlens = self.get_padding_and_inverse(point)
         slot_src, slot_dst = self._slots(point)
-        grad = ops.wants_grad(qkv)
+        grad = ops.wants_grad(qkv, self.rpe.rpe_table if self.enable_rpe else None)
         if grad and self.enable_rpe:
-            raise NotImplementedError("the relative position bias has no backward kernel: train with enable_rpe=False")
+            from .autograd import PatchAttentionRpe
+            out = PatchAttentionRpe.apply(qkv.float(), self.rpe.rpe_table, self.num_heads, slot_src, slot_dst, cu_seqlens,
+                                          self.patch_size, self.scale, point.grid_coord, self.rpe.pos_bnd)
+            return out.to(qkv.dtype)
         if grad:
             from .autograd import PatchAttention
             half = qkv.half() if (self.enable_flash and qkv.dtype == torch.float32) else qkv

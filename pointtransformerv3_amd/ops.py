@@ -338,6 +338,29 @@ def patch_attention_rpe(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seql
     return out
 
 
+def patch_attention_rpe_bwd(qkv, out, dout, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale, grid_coord,
+                            rpe_table, pos_bnd):
+    """(dqkv, drpe_table) of patch_attention_rpe: fp32, the table's gradient (3 * (2 * pos_bnd + 1), H) in fp32."""
+    _dev(qkv, out, dout, slot_src, slot_dst, cu_seqlens, grid_coord, rpe_table)
+    lib = _lib.load()
+    qkv, out = qkv.contiguous(), out.contiguous()
+    dout = dout.to(qkv.dtype).contiguous()
+    n, c3 = qkv.shape
+    c = c3 // 3
+    n_pad = slot_src.shape[0]
+    g = grid_coord.to(torch.int32).contiguous()
+    t = rpe_table.detach().to(torch.float32).contiguous()
+    dqkv = torch.empty_like(qkv)
+    dtable = torch.zeros_like(t)
+    nbytes = lib.ptv3_patch_attn_bwd_workspace_bytes(0, n_pad, c, int(num_heads))
+    ws = _ws(nbytes, qkv.device)
+    _lib.check(lib.ptv3_patch_attn_rpe_bwd(_ptr(qkv), _ptr(out), _ptr(dout), 0, n, c, int(num_heads), _ptr(slot_src),
+                                           _ptr(slot_dst), _ptr(cu_seqlens), cu_seqlens.shape[0] - 1, int(max_seqlen),
+                                           n_pad, float(scale), None, _ptr(g), _ptr(t), int(pos_bnd), _ptr(dtable),
+                                           _ptr(dqkv), _ptr(ws), nbytes, _stream()), "ptv3_patch_attn_rpe_bwd")
+    return dqkv, dtable
+
+
 def kmap_build(indices, ks, tap_major=False):
     """int32 neighbour map of (N,4) int32 [batch,x,y,z] voxels: (N, ks^3), or (ks^3, N) when
     tap_major (the layout the convolution kernels read coalesced)."""

@@ -54,6 +54,39 @@ def test_attention_backward_parity(dtype, counts, patch):
         assert rel_err(x.grad[:, sl], want[:, sl]) < TOL[dtype], part
 
 
+@pytest.mark.parametrize("counts,patch", [([64], 64), ([700, 300], 256), ([1500], 512)])
+def test_attention_rpe_backward_parity_fp32(counts, patch):
+    """Relative position bias path: gradients of qkv and of the bias table vs autograd over the CPU oracle."""
+    from pointtransformerv3_amd.autograd import PatchAttentionRpe
+    heads, seed = 4, 33
+    rng = np.random.default_rng(seed)
+    g = torch.Generator().manual_seed(seed)
+    n, C = int(sum(counts)), heads * 16
+    offset = np.cumsum(counts).astype(np.int64)
+    starts = np.concatenate([[0], offset[:-1]])
+    order = np.concatenate([s + rng.permutation(c) for s, c in zip(starts, counts)]).astype(np.int64)
+    inverse = np.empty(n, np.int64)
+    inverse[order] = np.arange(n)
+    grid = rng.integers(0, 40, size=(n, 3)).astype(np.int32)
+    pos_bnd = int((4 * patch) ** (1 / 3) * 2)
+    table = (torch.randn(3 * (2 * pos_bnd + 1), heads, generator=g) * 0.3)
+    qkv = torch.randn(n, 3 * C, generator=g)
+    dout = torch.randn(n, C, generator=g)
+    pad, unpad, cu = OI.padding_tables(offset, patch)
+    xq = qkv.clone().requires_grad_(True)
+    tb = table.clone().requires_grad_(True)
+    OF.serialized_attention_core(xq, order, inverse, pad, unpad, cu, heads, rpe=(grid, tb, pos_bnd)).backward(dout)
+    o = ops()
+    gp, gu, gc = o.pad_index(to_dev(offset), offset.tolist(), patch)
+    src, dst = o.attn_slots(to_dev(order), to_dev(inverse), gp, gu)
+    x = qkv.to(DEV).requires_grad_(True)
+    t = table.to(DEV).requires_grad_(True)
+    out = PatchAttentionRpe.apply(x, t, heads, src, dst, gc, patch, 0.25, to_dev(grid), pos_bnd)
+    out.backward(dout.to(DEV))
+    assert rel_err(x.grad, xq.grad) < 1e-4
+    assert rel_err(t.grad, tb.grad) < 1e-4
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_attention_backward_recomputes_lse_when_not_kept(dtype):
     """The backward entry point without the forward's log-sum-exp rows: same result as with them."""
@@ -339,7 +372,7 @@ def test_training_step_under_autocast(dtype):
     assert losses[-1] < losses[0]
 
 
-@pytest.mark.parametrize("variant", ["pdnorm", "post_norm", "cls_mode", "no_flash_fp32", "input_gradient"])
+@pytest.mark.parametrize("variant", ["pdnorm", "post_norm", "cls_mode", "no_flash_fp32", "input_gradient", "rpe"])
 def test_training_step_of_model_variants(variant):
     """One forward + backward of the model built other ways: every parameter that takes part gets a finite
     gradient (PDNorm only trains the norms of the condition it is given)."""
@@ -353,6 +386,8 @@ def test_training_step_of_model_variants(variant):
         kw = dict(cls_mode=True)
     elif variant == "no_flash_fp32":
         kw, autocast = dict(enable_flash=False), None
+    elif variant == "rpe":
+        kw, autocast = dict(enable_flash=False, enable_rpe=True, upcast_attention=True, upcast_softmax=True), None
     torch.manual_seed(3)
     model, _ = _small_model(drop_path=0.2, shuffle_orders=True, **kw)
     model = model.to(DEV).train()
