@@ -119,37 +119,42 @@ int ptv3_patch_attn_rpe_fwd(const float *qkv, int64_t n_rows, int channels, int 
                             const int32_t *grid_coord, const float *rpe_table, int pos_bnd, float *out,
                             void *stream);
 
-/* ptv3_patch_attn_fwd (fp16 / bf16) that also keeps what the backward pass needs: lse (heads, n_pad) fp32,
- * lse[h][slot] = log2 of the sum over the slot's sequence of 2^(score * log2(e)) for every real slot
- * (filler slots are left unwritten). n_pad = cu_seqlens[n_seq]. */
+/* ptv3_patch_attn_fwd for training. fp16 / bf16: also keeps what the backward pass needs, lse (heads, n_pad)
+ * fp32, lse[h][slot] = log2 of the sum over the slot's sequence of 2^(score * log2(e)) for every real slot
+ * (filler slots are left unwritten); fp32: lse may be NULL (the backward recomputes it). n_pad =
+ * cu_seqlens[n_seq]. dropout_p in [0, 1): attention dropout (model.py:470, :480) -- probability (head, query
+ * slot, key slot) is zeroed when a hash of (dropout_seed, head, query slot, key slot) falls below
+ * dropout_p * 2^32, the others are divided by 1 - dropout_p; the backward entry points take the same two
+ * values and recompute the same bits. */
 int ptv3_patch_attn_fwd_lse(const void *qkv, int dtype, int64_t n_rows, int channels, int heads,
                             const int32_t *slot_src, const int32_t *slot_dst, const int32_t *cu_seqlens,
-                            int64_t n_seq, int64_t max_seqlen, int64_t n_pad, float scale, void *out,
-                            float *lse, void *stream);
+                            int64_t n_seq, int64_t max_seqlen, int64_t n_pad, float scale, float dropout_p,
+                            uint32_t dropout_seed, void *out, float *lse, void *stream);
 
 /* Backward of ptv3_patch_attn_fwd: what autograd derives for model.py:456-484 (the backward of the
  * flash_attn_varlen_qkvpacked_func call at :476-482 and of the row gathers around it). out is the
  * forward result, dout its gradient (n_rows, C); dqkv (n_rows, 3*C) receives [dq | dk | dv] per row,
  * every element written. Filler slots take no gradient as queries; as keys their share is added to
  * the row they repeat. n_pad = cu_seqlens[n_seq], the number of slots. lse: what ptv3_patch_attn_fwd_lse
- * wrote for the same inputs (fp16 / bf16 only), or NULL to have it recomputed. */
+ * wrote for the same inputs (fp16 / bf16 only), or NULL to have it recomputed. dropout_p, dropout_seed: as
+ * given to the forward call. */
 size_t ptv3_patch_attn_bwd_workspace_bytes(int dtype, int64_t n_pad, int channels, int heads);
 int ptv3_patch_attn_bwd(const void *qkv, const void *out, const void *dout, int dtype, int64_t n_rows,
                         int channels, int heads, const int32_t *slot_src, const int32_t *slot_dst,
                         const int32_t *cu_seqlens, int64_t n_seq, int64_t max_seqlen, int64_t n_pad,
-                        float scale, const float *lse, void *dqkv, void *workspace, size_t workspace_bytes,
-                        void *stream);
+                        float scale, const float *lse, float dropout_p, uint32_t dropout_seed, void *dqkv,
+                        void *workspace, size_t workspace_bytes, void *stream);
 
 /* Backward of ptv3_patch_attn_rpe_fwd (fp32): as ptv3_patch_attn_bwd, with the relative position bias of
  * model.py:297-316 in the scores; drpe_table (3 * R, heads) fp32 is accumulated into (zero it first):
  * entry [a * R + c][h] += sum of dS(h, i, j) over the pairs (i, j) whose clamped offset along axis a is c.
- * grid_coord == NULL: exactly ptv3_patch_attn_bwd. */
+ * grid_coord == NULL: exactly ptv3_patch_attn_bwd. (The relative-position forward has no dropout: pass 0.) */
 int ptv3_patch_attn_rpe_bwd(const void *qkv, const void *out, const void *dout, int dtype, int64_t n_rows,
                             int channels, int heads, const int32_t *slot_src, const int32_t *slot_dst,
                             const int32_t *cu_seqlens, int64_t n_seq, int64_t max_seqlen, int64_t n_pad,
-                            float scale, const float *lse, const int32_t *grid_coord, const float *rpe_table,
-                            int pos_bnd, float *drpe_table, void *dqkv, void *workspace,
-                            size_t workspace_bytes, void *stream);
+                            float scale, const float *lse, float dropout_p, uint32_t dropout_seed,
+                            const int32_t *grid_coord, const float *rpe_table, int pos_bnd, float *drpe_table,
+                            void *dqkv, void *workspace, size_t workspace_bytes, void *stream);
 
 /* spconv.SubMConv3d's index generation (call sites model.py:546-552, :767-774, tensor built
  * at :165-172). indices (n,4) int32 [batch,x,y,z], coordinates in [0, 65535];

@@ -29,10 +29,28 @@ def rpe_bias(coord, table, pos_bnd):
     return table[idx.reshape(-1)].reshape(idx.shape + (-1,)).sum(2).permute(2, 0, 1)
 
 
-def patch_attention(qkv, cu_seqlens, num_heads, scale=None, rpe=None):
+def dropout_keep_mask(seed, head, q_slots, k_slots, p):
+    """The attention-dropout mask of this build's kernels (flash_attn's own random stream, model.py:480, cannot
+    be reproduced): element (query slot, key slot) of a head is kept when a 32-bit hash of (seed, head, q, k)
+    is at least p * 2^32. q_slots (Lq,), k_slots (Lk,) are padded slot numbers. Returns (Lq, Lk) bool."""
+    m32 = np.uint64(0xFFFFFFFF)
+    q = np.asarray(q_slots, dtype=np.uint64)[:, None]
+    k = np.asarray(k_slots, dtype=np.uint64)[None, :]
+    x = ((q * np.uint64(0x9E3779B1)) & m32) ^ (((k + np.uint64(0x7F4A7C15)) * np.uint64(0x85EBCA77)) & m32)
+    x = x ^ ((np.uint64(head + 1) * np.uint64(0xC2B2AE3D)) & m32) ^ np.uint64(seed & 0xFFFFFFFF)
+    x ^= x >> np.uint64(16)
+    x = (x * np.uint64(0x7FEB352D)) & m32
+    x ^= x >> np.uint64(15)
+    x = (x * np.uint64(0x846CA68B)) & m32
+    x ^= x >> np.uint64(16)
+    return x >= np.uint64(min(int(p * 4294967296.0), 0xFFFFFFFF))
+
+
+def patch_attention(qkv, cu_seqlens, num_heads, scale=None, rpe=None, dropout=None):
     """qkv: (Npad, 3*C) fp32 rows already in padded serialized order, channel layout
     [3][H][D] (model.py:461,477). rpe = (coord (Npad, 3) in the same order, table, pos_bnd) adds the
-    relative position bias to the scores (model.py:468-469). Returns (Npad, C)."""
+    relative position bias to the scores (model.py:468-469). dropout = (p, seed): softmax probabilities are
+    zeroed where dropout_keep_mask says so and the rest divided by 1 - p (model.py:470, :480). Returns (Npad, C)."""
     qkv = torch.as_tensor(qkv, dtype=torch.float32)
     npad, c3 = qkv.shape
     C = c3 // 3
@@ -47,6 +65,10 @@ def patch_attention(qkv, cu_seqlens, num_heads, scale=None, rpe=None):
         if rpe is not None:
             score = score + rpe_bias(np.asarray(rpe[0])[s:e], rpe[1], rpe[2])
         attn = torch.softmax(score, dim=-1)
+        if dropout is not None and dropout[0] > 0:
+            slots = np.arange(s, e)
+            keep = np.stack([dropout_keep_mask(dropout[1], h, slots, slots, dropout[0]) for h in range(num_heads)])
+            attn = attn * torch.from_numpy(keep).to(attn.dtype) / (1.0 - dropout[0])
         out[s:e] = (attn @ v).transpose(0, 1).reshape(e - s, C)
     return out
 
@@ -73,7 +95,7 @@ def patch_attention_bruteforce(qkv, cu_seqlens, num_heads, scale=None):
 
 
 def serialized_attention_core(feat_qkv, order, inverse, pad, unpad, cu_seqlens, num_heads,
-                              scale=None, rpe=None):
+                              scale=None, rpe=None, dropout=None):
     """model.py:452-484: gather rows into padded serialized order, attend inside each
     patch, keep each point's primary slot. feat_qkv: (N, 3C); rpe = (grid_coord (N, 3) in point
     order, table, pos_bnd). Returns (N, C)."""
@@ -82,7 +104,7 @@ def serialized_attention_core(feat_qkv, order, inverse, pad, unpad, cu_seqlens, 
     back = torch.as_tensor(np.asarray(unpad)[np.asarray(inverse)])
     if rpe is not None:
         rpe = (np.asarray(rpe[0])[gidx.numpy()], rpe[1], rpe[2])
-    out = patch_attention(feat_qkv[gidx], cu_seqlens, num_heads, scale, rpe)
+    out = patch_attention(feat_qkv[gidx], cu_seqlens, num_heads, scale, rpe, dropout)
     return out[back]
 
 

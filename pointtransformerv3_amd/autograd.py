@@ -9,20 +9,18 @@ from . import ops
 
 class PatchAttention(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale):
+    def forward(ctx, qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale, dropout_p=0.0, seed=0):
         args = (num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale)
-        if qkv.dtype == torch.float32:
-            out, ctx.lse = ops.patch_attention(qkv, *args), None
-        else:
-            out, ctx.lse = ops.patch_attention_lse(qkv, *args)
+        out, ctx.lse = ops.patch_attention_lse(qkv, *args, dropout_p=dropout_p, seed=seed)
         ctx.save_for_backward(qkv, out)
-        ctx.args = args
+        ctx.args, ctx.dropout = args, (dropout_p, seed)
         return out
 
     @staticmethod
     def backward(ctx, dout):
         qkv, out = ctx.saved_tensors
-        return (ops.patch_attention_bwd(qkv, out, dout, *ctx.args, lse=ctx.lse),) + (None,) * 6
+        p, seed = ctx.dropout
+        return (ops.patch_attention_bwd(qkv, out, dout, *ctx.args, lse=ctx.lse, dropout_p=p, seed=seed),) + (None,) * 8
 
 
 class PatchAttentionRpe(torch.autograd.Function):

@@ -50,15 +50,19 @@ __device__ __forceinline__ int xcd_chunked_id(int bid, int total) {
 // SHIFT = true: scores arrive shifted by a running reference maximum that enters through the C
 // operand; the reference moves (and the accumulators are rescaled) only when a score exceeds it
 // by RESCALE_SLACK, which the per-step |q||k| bound rules out without looking at the scores.
-template <typename T, bool SHIFT, bool LSE>
+// DROP: attention dropout. The denominator is then summed on the VALU from the probabilities before the mask
+// (the ones row of the second product would add up the masked ones) and handed back in acc[8] like the other.
+template <typename T, bool SHIFT, bool LSE, bool DROP>
 __device__ __forceinline__ f32x16 attend_tile(typename Half<T>::v8 qfrag, float qnorm, float kn_reg,
                                               const unsigned char* k_ptr, const unsigned char* v_ptr,
-                                              int v_step, int n_pairs, int len, int hf) {
+                                              int v_step, int n_pairs, int len, int hf, Dropout drop, uint32_t hq,
+                                              uint32_t kslot0) {
     typedef typename Half<T>::v8 v8;
     f32x16 acc, cinit;
 #pragma unroll
     for (int v = 0; v < 16; ++v) { acc[v] = 0.f; cinit[v] = 0.f; }
     float m_ref = 0.f;   // reference maximum: the MFMA adds -m_ref to every score
+    float den = 0.f;     // DROP: sum of the probabilities this lane has seen
     const bool ragged = (len & 63) != 0;
     v8 k0 = __builtin_bit_cast(v8, *(const u32x4*)k_ptr);
     v8 k1 = __builtin_bit_cast(v8, *(const u32x4*)(k_ptr + 32 * 32));
@@ -106,14 +110,33 @@ __device__ __forceinline__ f32x16 attend_tile(typename Half<T>::v8 qfrag, float 
                     }
 #pragma unroll
                     for (int v = 0; v < 9; ++v) acc[v] *= alpha;   // rows 0..15 + denominator row
+                    if (DROP) den *= alpha;
                 }
             }
         }
         uint32_t pa[8], pb[8];
+        if (DROP) {
+            const uint32_t k0s = kslot0 + (uint32_t)kp * 64u + 4u * (uint32_t)hf;
 #pragma unroll
-        for (int v = 0; v < 8; ++v) {
-            pa[v] = Half<T>::pack2(__builtin_amdgcn_exp2f(sa[2 * v]), __builtin_amdgcn_exp2f(sa[2 * v + 1]));
-            pb[v] = Half<T>::pack2(__builtin_amdgcn_exp2f(sb[2 * v]), __builtin_amdgcn_exp2f(sb[2 * v + 1]));
+            for (int v = 0; v < 8; ++v) {
+                float e[4] = {__builtin_amdgcn_exp2f(sa[2 * v]), __builtin_amdgcn_exp2f(sa[2 * v + 1]),
+                              __builtin_amdgcn_exp2f(sb[2 * v]), __builtin_amdgcn_exp2f(sb[2 * v + 1])};
+                den += (e[0] + e[1]) + (e[2] + e[3]);
+                // register i of the first 32-block holds key 8 (i / 4) + 4 hf + i % 4; the second block is 32 on
+                const uint32_t ka = k0s + 8u * (uint32_t)((2 * v) >> 2) + (uint32_t)((2 * v) & 3);
+                if (!drop_keep(hq, ka, drop.threshold)) e[0] = 0.f;
+                if (!drop_keep(hq, ka + 1u, drop.threshold)) e[1] = 0.f;
+                if (!drop_keep(hq, ka + 32u, drop.threshold)) e[2] = 0.f;
+                if (!drop_keep(hq, ka + 33u, drop.threshold)) e[3] = 0.f;
+                pa[v] = Half<T>::pack2(e[0], e[1]);
+                pb[v] = Half<T>::pack2(e[2], e[3]);
+            }
+        } else {
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                pa[v] = Half<T>::pack2(__builtin_amdgcn_exp2f(sa[2 * v]), __builtin_amdgcn_exp2f(sa[2 * v + 1]));
+                pb[v] = Half<T>::pack2(__builtin_amdgcn_exp2f(sb[2 * v]), __builtin_amdgcn_exp2f(sb[2 * v + 1]));
+            }
         }
         acc = Half<T>::mfma(__builtin_bit_cast(v8, va0), __builtin_bit_cast(v8, (u32x4){pa[0], pa[1], pa[2], pa[3]}), acc);
         acc = Half<T>::mfma(__builtin_bit_cast(v8, va1), __builtin_bit_cast(v8, (u32x4){pa[4], pa[5], pa[6], pa[7]}), acc);
@@ -122,16 +145,18 @@ __device__ __forceinline__ f32x16 attend_tile(typename Half<T>::v8 qfrag, float 
     }
     // result row 17 / 21 multiplies zeros: its register carries the reference maximum to the caller
     if (SHIFT && LSE) acc[9] = m_ref;
+    if (DROP) acc[8] = den + __shfl_xor(den, 32, PTV3_WAVE);   // the other half-wave saw the other keys
     return acc;
 }
 
 // LSE: also write log2(sum_j 2^score_ij) of every real query, scores in log2 units (scale * log2(e) folded into
 // q), to lse[head * lse_stride + slot]: what the backward kernels need to rebuild the probabilities.
-template <typename T, bool LSE>
+template <typename T, bool LSE, bool DROP>
 __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
     const T* __restrict__ qkv, int channels, int heads, const int32_t* __restrict__ slot_src,
     const int32_t* __restrict__ slot_dst, const int32_t* __restrict__ cu_seqlens, int lds_keys,
-    float scale_log2e, T* __restrict__ out, int full_items, int split, float* __restrict__ lse, int64_t lse_stride) {
+    float scale_log2e, T* __restrict__ out, int full_items, int split, float* __restrict__ lse, int64_t lse_stride,
+    Dropout drop) {
     typedef typename Half<T>::v8 v8;
     extern __shared__ __align__(16) unsigned char smem[];
     // K tile: lds_keys + 64 rows of 32 B (the last 64 are only ever prefetched). V^T tile: 16 rows
@@ -242,13 +267,16 @@ __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
         const float qnorm = sqrtf(qn) * 1.0009765625f;
 
         f32x16 acc;
+        const uint32_t hq = DROP ? drop_hq(drop.seed, (uint32_t)head, (uint32_t)(s0 + qi)) : 0u;
         if (__ballot(qnorm * kn_all > Half<T>::plain_limit()) == 0)
-            acc = attend_tile<T, false, LSE>(qfrag, qnorm, kn_reg, k_base, v_base, v_step, n_pairs, len, hf);
+            acc = attend_tile<T, false, LSE, DROP>(qfrag, qnorm, kn_reg, k_base, v_base, v_step, n_pairs, len, hf, drop, hq,
+                                                   (uint32_t)s0);
         else
-            acc = attend_tile<T, true, LSE>(qfrag, qnorm, kn_reg, k_base, v_base, v_step, n_pairs, len, hf);
+            acc = attend_tile<T, true, LSE, DROP>(qfrag, qnorm, kn_reg, k_base, v_base, v_step, n_pairs, len, hf, drop, hq,
+                                                  (uint32_t)s0);
         // acc[v]: d = 8*(v/4) + 4*hf + v%4; acc[8] = sum of probabilities (row 16 / 20)
         if (dst >= 0) {
-            const float inv = 1.f / acc[8];
+            const float inv = (DROP ? drop.inv_keep : 1.f) / acc[8];
             T* o = out + (int64_t)dst * channels + head * HD + 4 * hf;
             u32x2 lo = {Half<T>::pack2(acc[0] * inv, acc[1] * inv), Half<T>::pack2(acc[2] * inv, acc[3] * inv)};
             u32x2 hi = {Half<T>::pack2(acc[4] * inv, acc[5] * inv), Half<T>::pack2(acc[6] * inv, acc[7] * inv)};
@@ -266,7 +294,7 @@ constexpr int F32_KC = 128;   // keys per chunk
 __global__ __launch_bounds__(F32_QB) void patch_attn_f32_kernel(
     const float* __restrict__ qkv, int channels, int heads, const int32_t* __restrict__ slot_src,
     const int32_t* __restrict__ slot_dst, const int32_t* __restrict__ cu_seqlens, int q_blocks,
-    float scale, float* __restrict__ out) {
+    float scale, float* __restrict__ out, Dropout drop) {
     __shared__ float k_lds[F32_KC][HD];
     __shared__ float v_lds[F32_KC][HD];
     const int seq = blockIdx.x / (heads * q_blocks);
@@ -289,6 +317,7 @@ __global__ __launch_bounds__(F32_QB) void patch_attn_f32_kernel(
 #pragma unroll
         for (int d = 0; d < HD; ++d) q[d] = src[d] * scale;
     }
+    const uint32_t hq = drop_hq(drop.seed, (uint32_t)head, (uint32_t)(s0 + qi));
     float m = -INFINITY, l = 0.f;
     for (int c0 = 0; c0 < len; c0 += F32_KC) {
         __syncthreads();
@@ -316,14 +345,15 @@ __global__ __launch_bounds__(F32_QB) void patch_attn_f32_kernel(
                 for (int d = 0; d < HD; ++d) o[d] *= a;
                 m = s;
             }
-            const float p = __expf(s - m);
+            float p = __expf(s - m);
             l += p;
+            if (drop.threshold && !drop_keep(hq, (uint32_t)(s0 + c0 + key), drop.threshold)) p = 0.f;
 #pragma unroll
             for (int d = 0; d < HD; ++d) o[d] = fmaf(p, v_lds[key][d], o[d]);
         }
     }
     if (dst >= 0) {
-        const float inv = 1.f / l;
+        const float inv = drop.inv_keep / l;
         float* dstp = out + (int64_t)dst * channels + head * HD;
 #pragma unroll
         for (int d = 0; d < HD; ++d) dstp[d] = o[d] * inv;
@@ -418,16 +448,17 @@ __global__ __launch_bounds__(F32_QB) void patch_attn_rpe_f32_kernel(
     }
 }
 
-template <typename T, bool LSE>
+template <typename T, bool LSE, bool DROP>
 int launch_half(const void* qkv, int channels, int heads, const int32_t* slot_src,
                 const int32_t* slot_dst, const int32_t* cu_seqlens, int64_t n_seq,
-                int64_t max_seqlen, float scale, void* out, float* lse, int64_t lse_stride, hipStream_t stream) {
+                int64_t max_seqlen, float scale, void* out, float* lse, int64_t lse_stride, Dropout drop,
+                hipStream_t stream) {
     const int lds_keys = (int)((max_seqlen + 63) & ~63ll);
     // K (+ one prefetch-only step), V^T, per-step key norms (padded to 16 B), ones and zeros
     const size_t lds = (size_t)(lds_keys + 64) * 32 + (size_t)HD * (lds_keys * 2 + VT_PAD_BYTES) +
                        (size_t)(lds_keys / 64) * sizeof(float) + 12 + 192;
     if (lds > 160 * 1024) return PTV3_ESHAPE;
-    auto kern = patch_attn_half_kernel<T, LSE>;
+    auto kern = patch_attn_half_kernel<T, LSE, DROP>;
     static size_t lds_allowed = 0;   // per instantiation; raised monotonically
     if (lds > lds_allowed) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -459,7 +490,7 @@ int launch_half(const void* qkv, int channels, int heads, const int32_t* slot_sr
     if (split == 1) full = total;
     hipLaunchKernelGGL(kern, dim3((unsigned)(full + (total - full) * split)), dim3(ATT_THREADS), lds, stream,
                        (const T*)qkv, channels, heads, slot_src, slot_dst, cu_seqlens, lds_keys,
-                       scale_log2e, (T*)out, (int)full, (int)split, lse, lse_stride);
+                       scale_log2e, (T*)out, (int)full, (int)split, lse, lse_stride, drop);
     PTV3_RETURN_LAUNCH();
 }
 
@@ -477,35 +508,49 @@ extern "C" int ptv3_patch_attn_fwd(const void* qkv, int dtype, int64_t n_rows, i
     if (!qkv || !slot_src || !slot_dst || !cu_seqlens || !out) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
     if (dtype == PTV3_F16)
-        return launch_half<_Float16, false>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
-                                            max_seqlen, scale, out, nullptr, 0, stream);
+        return launch_half<_Float16, false, false>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
+                                                   max_seqlen, scale, out, nullptr, 0, Dropout{0u, 0u, 1.f}, stream);
     if (dtype == PTV3_BF16)
-        return launch_half<__bf16, false>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
-                                          max_seqlen, scale, out, nullptr, 0, stream);
+        return launch_half<__bf16, false, false>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
+                                                 max_seqlen, scale, out, nullptr, 0, Dropout{0u, 0u, 1.f}, stream);
     const int q_blocks = (int)ptv3_ceil_div(max_seqlen, F32_QB);
     if (n_seq * heads * q_blocks >= (1ll << 31)) return PTV3_EINVAL;
     hipLaunchKernelGGL(patch_attn_f32_kernel, dim3((unsigned)(n_seq * heads * q_blocks)), dim3(F32_QB),
                        0, stream, (const float*)qkv, channels, heads, slot_src, slot_dst, cu_seqlens,
-                       q_blocks, scale, (float*)out);
+                       q_blocks, scale, (float*)out, Dropout{0u, 0u, 1.f});
     PTV3_RETURN_LAUNCH();
 }
 
 extern "C" int ptv3_patch_attn_fwd_lse(const void* qkv, int dtype, int64_t n_rows, int channels, int heads,
                                        const int32_t* slot_src, const int32_t* slot_dst, const int32_t* cu_seqlens,
-                                       int64_t n_seq, int64_t max_seqlen, int64_t n_pad, float scale, void* out,
-                                       float* lse, void* stream_) {
+                                       int64_t n_seq, int64_t max_seqlen, int64_t n_pad, float scale, float dropout_p,
+                                       uint32_t dropout_seed, void* out, float* lse, void* stream_) {
     if (n_rows < 0 || n_seq < 0 || n_pad < 0 || channels < 1 || heads < 1 || max_seqlen < 1) return PTV3_EINVAL;
-    if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
+    if (dtype < PTV3_F32 || dtype > PTV3_BF16 || !(dropout_p >= 0.f) || !(dropout_p < 1.f)) return PTV3_EINVAL;
     if (channels % heads != 0 || channels / heads != HD) return PTV3_ESHAPE;
     if (n_seq * heads >= (1ll << 31)) return PTV3_EINVAL;
     if (n_seq == 0 || n_rows == 0) return PTV3_OK;
-    if (!qkv || !slot_src || !slot_dst || !cu_seqlens || !out || !lse) return PTV3_EINVAL;
+    if (!qkv || !slot_src || !slot_dst || !cu_seqlens || !out || (dtype != PTV3_F32 && !lse)) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
-    if (dtype == PTV3_F16)
-        return launch_half<_Float16, true>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq, max_seqlen,
-                                           scale, out, lse, n_pad, stream);
-    return launch_half<__bf16, true>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq, max_seqlen, scale,
-                                     out, lse, n_pad, stream);
+    const Dropout drop = {dropout_seed, dropout_p > 0.f ? drop_threshold(dropout_p) : 0u, 1.f / (1.f - dropout_p)};
+    if (dtype == PTV3_F32) {   // the backward recomputes the log-sum-exp rows on this path
+        const int q_blocks = (int)ptv3_ceil_div(max_seqlen, F32_QB);
+        if (n_seq * heads * q_blocks >= (1ll << 31)) return PTV3_EINVAL;
+        hipLaunchKernelGGL(patch_attn_f32_kernel, dim3((unsigned)(n_seq * heads * q_blocks)), dim3(F32_QB), 0, stream,
+                           (const float*)qkv, channels, heads, slot_src, slot_dst, cu_seqlens, q_blocks, scale,
+                           (float*)out, drop);
+        PTV3_RETURN_LAUNCH();
+    }
+#define PTV3_ATT(T, D)                                                                                               \
+    return launch_half<T, true, D>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq, max_seqlen, scale, out, \
+                                   lse, n_pad, drop, stream)
+    if (dtype == PTV3_F16) {
+        if (drop.threshold) PTV3_ATT(_Float16, true);
+        PTV3_ATT(_Float16, false);
+    }
+    if (drop.threshold) PTV3_ATT(__bf16, true);
+    PTV3_ATT(__bf16, false);
+#undef PTV3_ATT
 }
 
 extern "C" int ptv3_patch_attn_rpe_fwd(const float* qkv, int64_t n_rows, int channels, int heads,

@@ -101,12 +101,12 @@ __device__ __forceinline__ void item_of_block(int full_items, int split, int* it
 }
 
 // ---- kernel 1: one work-group per (sequence, head), a wave per 32-query tile
-template <typename T, bool HAVE_LSE>
+template <typename T, bool HAVE_LSE, bool DROP>
 __global__ __launch_bounds__(BWQ_THREADS) void attn_bwd_q_kernel(
     const T* __restrict__ qkv, const T* __restrict__ out, const T* __restrict__ dout, int channels, int heads,
     const int32_t* __restrict__ slot_src, const int32_t* __restrict__ slot_dst,
     const int32_t* __restrict__ cu_seqlens, int lds_keys, float scale, int64_t n_pad, T* __restrict__ dqkv,
-    float* lse_ws, float* __restrict__ d_ws, int full_items, int split) {
+    float* lse_ws, float* __restrict__ d_ws, int full_items, int split, Dropout drop) {
     typedef typename Half<T>::v8 v8;
     extern __shared__ __align__(16) unsigned char smem[];
     // K rows, V rows, K^T, 96 B of zeros
@@ -169,6 +169,7 @@ __global__ __launch_bounds__(BWQ_THREADS) void attn_bwd_q_kernel(
         dsum += __shfl_xor(dsum, 32, PTV3_WAVE);
         const v8 qfrag = __builtin_bit_cast(v8, scale8<T>(qreg, scale_log2e));   // scores in log2 units
         const v8 dofrag = __builtin_bit_cast(v8, doreg);
+        const uint32_t hq = DROP ? drop_hq(drop.seed, (uint32_t)head, (uint32_t)(s0 + qi)) : 0u;
 
         // log-sum-exp of the query's score row: kept by the forward pass, or a first sweep over the keys
         // (this lane sees half of them)
@@ -223,7 +224,7 @@ __global__ __launch_bounds__(BWQ_THREADS) void attn_bwd_q_kernel(
                 const v8 kf = __builtin_bit_cast(v8, *(const u32x4*)(k_base + (size_t)kp * 64 * 32 + h * 32 * 32));
                 const v8 vf = __builtin_bit_cast(v8, *(const u32x4*)(v_base + (size_t)kp * 64 * 32 + h * 32 * 32));
                 f32x16 sc = Half<T>::mfma(kf, qfrag, c_lse);        // S - lse
-                const f32x16 dp = Half<T>::mfma(vf, dofrag, c_d);   // dP - D
+                const f32x16 dp = Half<T>::mfma(vf, dofrag, DROP ? zero : c_d);   // dP - D (dP alone with dropout)
                 const u32x4 kt0 = *(const u32x4*)(kt_ptr + 64 * h);
                 const u32x4 kt1 = *(const u32x4*)(kt_ptr + 64 * h + 16);
                 if (ragged && kp == n_pairs - 1) {
@@ -232,8 +233,18 @@ __global__ __launch_bounds__(BWQ_THREADS) void attn_bwd_q_kernel(
                         if (kp * 64 + 32 * h + 8 * (v >> 2) + 4 * hf + (v & 3) >= len) sc[v] = -INFINITY;
                 }
                 float ds[16];
+                if (DROP) {
+                    // the dropped probabilities pass no gradient on: dS = P o (mask o dP / (1 - p) - D)
+                    const uint32_t k0s = (uint32_t)s0 + (uint32_t)kp * 64u + 32u * (uint32_t)h + 4u * (uint32_t)hf;
 #pragma unroll
-                for (int v = 0; v < 16; ++v) ds[v] = __builtin_amdgcn_exp2f(sc[v]) * dp[v];
+                    for (int v = 0; v < 16; ++v) {
+                        const bool keep = drop_keep(hq, k0s + 8u * (uint32_t)(v >> 2) + (uint32_t)(v & 3), drop.threshold);
+                        ds[v] = __builtin_amdgcn_exp2f(sc[v]) * ((keep ? dp[v] * drop.inv_keep : 0.f) - dsum);
+                    }
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) ds[v] = __builtin_amdgcn_exp2f(sc[v]) * dp[v];
+                }
                 acc = Half<T>::mfma(__builtin_bit_cast(v8, kt0), pack8<T>(ds), acc);
                 acc = Half<T>::mfma(__builtin_bit_cast(v8, kt1), pack8<T>(ds + 8), acc);
             }
@@ -255,13 +266,13 @@ __global__ __launch_bounds__(BWQ_THREADS) void attn_bwd_q_kernel(
 }
 
 // ---- kernel 2: one work-group per (sequence, head), a wave per 32-key tile
-template <typename T>
+template <typename T, bool DROP>
 __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_kv_kernel(
     const T* __restrict__ qkv, const T* __restrict__ dout, int channels, int heads,
     const int32_t* __restrict__ slot_src, const int32_t* __restrict__ slot_dst,
     const int32_t* __restrict__ cu_seqlens, int lds_keys, float scale, int64_t n_pad,
     const float* __restrict__ lse_ws, const float* __restrict__ d_ws, T* __restrict__ dqkv, T* __restrict__ fill,
-    int full_items, int split) {
+    int full_items, int split, Dropout drop) {
     typedef typename Half<T>::v8 v8;
     typedef float f32x4 __attribute__((ext_vector_type(4)));
     extern __shared__ __align__(16) unsigned char smem[];
@@ -382,17 +393,36 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_kv_kernel(
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 if (t == 1 && !two) break;
+                const f32x16 zero = splat16(0.f);
                 const f32x16 sa = Half<T>::mfma(q0, kfrag[t], cla);    // S - lse, [query, this lane's key]
                 const f32x16 sb = Half<T>::mfma(q1, kfrag[t], clb);
-                const f32x16 da = Half<T>::mfma(g0, vfrag[t], cda);    // dP - D
-                const f32x16 db = Half<T>::mfma(g1, vfrag[t], cdb);
+                const f32x16 da = Half<T>::mfma(g0, vfrag[t], DROP ? zero : cda);    // dP - D (dP alone with dropout)
+                const f32x16 db = Half<T>::mfma(g1, vfrag[t], DROP ? zero : cdb);
                 float pa[16], pb[16], dsa[16], dsb[16];
+                if (DROP) {
+                    // the mask of (query, key): dV sees the kept, rescaled probabilities, dS = P o (mask o dP / (1 - p) - D)
+                    const uint32_t hconst = (((uint32_t)head + 1u) * 0xC2B2AE3Du) ^ drop.seed;
+                    const uint32_t kslot = (uint32_t)(s0 + key[t]);
+                    const uint32_t q0s = (uint32_t)s0 + (uint32_t)st * 64u + 4u * (uint32_t)hf;
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    pa[v] = __builtin_amdgcn_exp2f(sa[v]);
-                    pb[v] = __builtin_amdgcn_exp2f(sb[v]);
-                    dsa[v] = pa[v] * da[v];
-                    dsb[v] = pb[v] * db[v];
+                    for (int v = 0; v < 16; ++v) {
+                        const uint32_t qs = q0s + 8u * (uint32_t)(v >> 2) + (uint32_t)(v & 3);
+                        const bool ka = drop_keep((qs * 0x9E3779B1u) ^ hconst, kslot, drop.threshold);
+                        const bool kb = drop_keep(((qs + 32u) * 0x9E3779B1u) ^ hconst, kslot, drop.threshold);
+                        const float ea = __builtin_amdgcn_exp2f(sa[v]), eb = __builtin_amdgcn_exp2f(sb[v]);
+                        pa[v] = ka ? ea * drop.inv_keep : 0.f;
+                        pb[v] = kb ? eb * drop.inv_keep : 0.f;
+                        dsa[v] = ea * ((ka ? da[v] * drop.inv_keep : 0.f) + cda[v]);   // cda holds -D
+                        dsb[v] = eb * ((kb ? db[v] * drop.inv_keep : 0.f) + cdb[v]);
+                    }
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        pa[v] = __builtin_amdgcn_exp2f(sa[v]);
+                        pb[v] = __builtin_amdgcn_exp2f(sb[v]);
+                        dsa[v] = pa[v] * da[v];
+                        dsb[v] = pb[v] * db[v];
+                    }
                 }
                 acc_v[t] = Half<T>::mfma(ga0, pack8<T>(pa), acc_v[t]);
                 acc_v[t] = Half<T>::mfma(ga1, pack8<T>(pa + 8), acc_v[t]);
@@ -444,7 +474,7 @@ __global__ __launch_bounds__(F32_B) void attn_bwd_q_f32_kernel(
     const float* __restrict__ qkv, const float* __restrict__ out, const float* __restrict__ dout, int channels,
     int heads, const int32_t* __restrict__ slot_src, const int32_t* __restrict__ slot_dst,
     const int32_t* __restrict__ cu_seqlens, int blocks, float scale, int64_t n_pad, float* __restrict__ dqkv,
-    float* __restrict__ lse_ws, float* __restrict__ d_ws, Rpe rpe) {
+    float* __restrict__ lse_ws, float* __restrict__ d_ws, Rpe rpe, Dropout drop) {
     __shared__ float k_lds[F32_C][HD];
     __shared__ float v_lds[F32_C][HD];
     __shared__ int32_t c_lds[F32_C][3];
@@ -489,6 +519,7 @@ __global__ __launch_bounds__(F32_B) void attn_bwd_q_f32_kernel(
         }
     }
     float m = -INFINITY, l = 0.f, lse = 0.f;
+    const uint32_t hq = drop_hq(drop.seed, (uint32_t)head, (uint32_t)(s0 + qi));
     for (int sweep = 0; sweep < 2; ++sweep) {
         for (int c0 = 0; c0 < len; c0 += F32_C) {
             __syncthreads();
@@ -529,6 +560,8 @@ __global__ __launch_bounds__(F32_B) void attn_bwd_q_f32_kernel(
                     float dp = 0.f;
 #pragma unroll
                     for (int d = 0; d < HD; ++d) dp = fmaf(g[d], v_lds[key][d], dp);
+                    if (drop.threshold)
+                        dp = drop_keep(hq, (uint32_t)(s0 + c0 + key), drop.threshold) ? dp * drop.inv_keep : 0.f;
                     const float ds = p * (dp - dsum);
 #pragma unroll
                     for (int d = 0; d < HD; ++d) dq[d] = fmaf(ds, k_lds[key][d], dq[d]);
@@ -561,7 +594,7 @@ __global__ __launch_bounds__(F32_B) void attn_bwd_kv_f32_kernel(
     const int32_t* __restrict__ slot_src, const int32_t* __restrict__ slot_dst,
     const int32_t* __restrict__ cu_seqlens, int blocks, float scale, int64_t n_pad,
     const float* __restrict__ lse_ws, const float* __restrict__ d_ws, float* __restrict__ dqkv,
-    float* __restrict__ fill, Rpe rpe) {
+    float* __restrict__ fill, Rpe rpe, Dropout drop) {
     __shared__ float q_lds[F32_C][HD];    // q * scale
     __shared__ float g_lds[F32_C][HD];    // dO
     __shared__ float lse_lds[F32_C];
@@ -635,10 +668,17 @@ __global__ __launch_bounds__(F32_B) void attn_bwd_kv_f32_kernel(
                 s += t_lds[rpe_index(c_lds[qi][0], kx, rpe.bnd)] + t_lds[rnum + rpe_index(c_lds[qi][1], ky, rpe.bnd)] +
                      t_lds[2 * rnum + rpe_index(c_lds[qi][2], kz, rpe.bnd)];
             const float p = __expf(s - lse_lds[qi]);
+            float pv = p;   // what multiplied V in the forward pass
+            if (drop.threshold) {
+                const bool keep = drop_keep(drop_hq(drop.seed, (uint32_t)head, (uint32_t)(s0 + c0 + qi)), (uint32_t)(s0 + ki),
+                                            drop.threshold);
+                pv = keep ? p * drop.inv_keep : 0.f;
+                dp = keep ? dp * drop.inv_keep : 0.f;
+            }
             const float ds = p * (dp - d_lds[qi]);
 #pragma unroll
             for (int d = 0; d < HD; ++d) {
-                dv[d] = fmaf(p, g_lds[qi][d], dv[d]);
+                dv[d] = fmaf(pv, g_lds[qi][d], dv[d]);
                 dk[d] = fmaf(ds, q_lds[qi][d], dk[d]);   // q already carries the scale
             }
         }
@@ -697,21 +737,25 @@ BwdWs carve(void* base, int dtype, int64_t n_pad, int channels, int heads) {
 template <typename T>
 int launch_half_bwd(const void* qkv, const void* out, const void* dout, int channels, int heads,
                     const int32_t* slot_src, const int32_t* slot_dst, const int32_t* cu_seqlens, int64_t n_seq,
-                    int64_t max_seqlen, int64_t n_pad, float scale, void* dqkv, const BwdWs& ws, float* lse,
+                    int64_t max_seqlen, int64_t n_pad, float scale, void* dqkv, const BwdWs& ws, float* lse, Dropout drop,
                     hipStream_t stream) {
     const int lds_keys = (int)((max_seqlen + 63) & ~63ll);
     const size_t t_bytes = (size_t)HD * (lds_keys * 2 + VT_PAD_BYTES);
     const size_t lds_q = 2 * (size_t)lds_keys * 32 + t_bytes + 96;
     const size_t lds_kv = 2 * (size_t)lds_keys * 32 + 2 * t_bytes + 2 * (size_t)lds_keys * sizeof(float) + 96;
     if (lds_q > 160 * 1024 || lds_kv > 160 * 1024) return PTV3_ESHAPE;
-    auto kq = lse ? attn_bwd_q_kernel<T, true> : attn_bwd_q_kernel<T, false>;
+    const bool dropping = drop.threshold != 0u;
+    auto kq = dropping ? (lse ? attn_bwd_q_kernel<T, true, true> : attn_bwd_q_kernel<T, false, true>)
+                       : (lse ? attn_bwd_q_kernel<T, true, false> : attn_bwd_q_kernel<T, false, false>);
     float* lse_buf = lse ? lse : ws.lse;
-    auto kkv = attn_bwd_kv_kernel<T>;
-    static size_t allowed_q[2] = {0, 0}, allowed_kv = 0;
-    if (lds_q > allowed_q[lse != nullptr]) {
+    auto kkv = dropping ? attn_bwd_kv_kernel<T, true> : attn_bwd_kv_kernel<T, false>;
+    static size_t allowed_q[4] = {0, 0, 0, 0}, allowed_kvs[2] = {0, 0};
+    size_t& allowed_kv = allowed_kvs[dropping];
+    const int qi_ = (lse != nullptr) + 2 * dropping;
+    if (lds_q > allowed_q[qi_]) {
         hipError_t e = hipFuncSetAttribute((const void*)kq, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_q);
         if (e != hipSuccess) return (int)e;
-        allowed_q[lse != nullptr] = lds_q;
+        allowed_q[qi_] = lds_q;
     }
     if (lds_kv > allowed_kv) {
         hipError_t e = hipFuncSetAttribute((const void*)kkv, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_kv);
@@ -742,10 +786,10 @@ int launch_half_bwd(const void* qkv, const void* out, const void* dout, int chan
     const unsigned grid = (unsigned)(full + (total - full) * split);
     hipLaunchKernelGGL(kq, dim3(grid), dim3(BWQ_THREADS), lds_q, stream, (const T*)qkv, (const T*)out, (const T*)dout,
                        channels, heads, slot_src, slot_dst, cu_seqlens, lds_keys, scale, n_pad, (T*)dqkv, lse_buf, ws.d,
-                       (int)full, (int)split);
+                       (int)full, (int)split, drop);
     hipLaunchKernelGGL(kkv, dim3(grid), dim3(BWD_THREADS), lds_kv, stream, (const T*)qkv, (const T*)dout, channels,
                        heads, slot_src, slot_dst, cu_seqlens, lds_keys, scale, n_pad, lse_buf, ws.d, (T*)dqkv,
-                       (T*)ws.fill, (int)full, (int)split);
+                       (T*)ws.fill, (int)full, (int)split, drop);
     const int64_t items = n_pad * (2 * channels / 8);
     hipLaunchKernelGGL(attn_bwd_fill_kernel<T>, dim3((unsigned)ptv3_ceil_div(items, 256)), dim3(256), 0, stream,
                        (const T*)ws.fill, channels, slot_src, slot_dst, n_pad, (T*)dqkv);
@@ -762,22 +806,25 @@ extern "C" size_t ptv3_patch_attn_bwd_workspace_bytes(int dtype, int64_t n_pad, 
 extern "C" int ptv3_patch_attn_bwd(const void* qkv, const void* out, const void* dout, int dtype, int64_t n_rows,
                                    int channels, int heads, const int32_t* slot_src, const int32_t* slot_dst,
                                    const int32_t* cu_seqlens, int64_t n_seq, int64_t max_seqlen, int64_t n_pad,
-                                   float scale, const float* lse, void* dqkv, void* workspace, size_t workspace_bytes,
-                                   void* stream_) {
+                                   float scale, const float* lse, float dropout_p, uint32_t dropout_seed, void* dqkv,
+                                   void* workspace, size_t workspace_bytes, void* stream_) {
     return ptv3_patch_attn_rpe_bwd(qkv, out, dout, dtype, n_rows, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
-                                   max_seqlen, n_pad, scale, lse, nullptr, nullptr, 0, nullptr, dqkv, workspace,
-                                   workspace_bytes, stream_);
+                                   max_seqlen, n_pad, scale, lse, dropout_p, dropout_seed, nullptr, nullptr, 0, nullptr,
+                                   dqkv, workspace, workspace_bytes, stream_);
 }
 
 extern "C" int ptv3_patch_attn_rpe_bwd(const void* qkv, const void* out, const void* dout, int dtype, int64_t n_rows,
                                        int channels, int heads, const int32_t* slot_src, const int32_t* slot_dst,
                                        const int32_t* cu_seqlens, int64_t n_seq, int64_t max_seqlen, int64_t n_pad,
-                                       float scale, const float* lse, const int32_t* grid_coord, const float* rpe_table,
-                                       int pos_bnd, float* drpe_table, void* dqkv, void* workspace,
-                                       size_t workspace_bytes, void* stream_) {
+                                       float scale, const float* lse, float dropout_p, uint32_t dropout_seed,
+                                       const int32_t* grid_coord, const float* rpe_table, int pos_bnd,
+                                       float* drpe_table, void* dqkv, void* workspace, size_t workspace_bytes,
+                                       void* stream_) {
     if (grid_coord && (dtype != PTV3_F32 || !rpe_table || !drpe_table)) return PTV3_ESHAPE;   // the bias lives on the fp32 path
     if (grid_coord && (pos_bnd < 0 || pos_bnd > RPE_MAX_BND)) return PTV3_ESHAPE;
+    if (!(dropout_p >= 0.f) || !(dropout_p < 1.f)) return PTV3_EINVAL;
     const Rpe rpe = {grid_coord, rpe_table, drpe_table, grid_coord ? pos_bnd : 0};
+    const Dropout drop = {dropout_seed, dropout_p > 0.f ? drop_threshold(dropout_p) : 0u, 1.f / (1.f - dropout_p)};
     if (n_rows < 0 || n_seq < 0 || n_pad < 0 || channels < 1 || heads < 1 || max_seqlen < 1) return PTV3_EINVAL;
     if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
     if (channels % heads != 0 || channels / heads != HD) return PTV3_ESHAPE;
@@ -789,19 +836,19 @@ extern "C" int ptv3_patch_attn_rpe_bwd(const void* qkv, const void* out, const v
     hipStream_t stream = (hipStream_t)stream_;
     if (dtype == PTV3_F16)
         return launch_half_bwd<_Float16>(qkv, out, dout, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
-                                         max_seqlen, n_pad, scale, dqkv, ws, (float*)lse, stream);
+                                         max_seqlen, n_pad, scale, dqkv, ws, (float*)lse, drop, stream);
     if (dtype == PTV3_BF16)
         return launch_half_bwd<__bf16>(qkv, out, dout, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
-                                       max_seqlen, n_pad, scale, dqkv, ws, (float*)lse, stream);
+                                       max_seqlen, n_pad, scale, dqkv, ws, (float*)lse, drop, stream);
     const int blocks = (int)ptv3_ceil_div(max_seqlen, F32_B);
     if (n_seq * heads * blocks >= (1ll << 31)) return PTV3_EINVAL;
     const unsigned grid = (unsigned)(n_seq * heads * blocks);
     hipLaunchKernelGGL(attn_bwd_q_f32_kernel, dim3(grid), dim3(F32_B), 0, stream, (const float*)qkv, (const float*)out,
                        (const float*)dout, channels, heads, slot_src, slot_dst, cu_seqlens, blocks, scale, n_pad,
-                       (float*)dqkv, ws.lse, ws.d, rpe);
+                       (float*)dqkv, ws.lse, ws.d, rpe, drop);
     hipLaunchKernelGGL(attn_bwd_kv_f32_kernel, dim3(grid), dim3(F32_B), 0, stream, (const float*)qkv,
                        (const float*)dout, channels, heads, slot_src, slot_dst, cu_seqlens, blocks, scale, n_pad, ws.lse,
-                       ws.d, (float*)dqkv, (float*)ws.fill, rpe);
+                       ws.d, (float*)dqkv, (float*)ws.fill, rpe, drop);
     const int64_t items = n_pad * (2 * channels / 8);
     hipLaunchKernelGGL(attn_bwd_fill_kernel<float>, dim3((unsigned)ptv3_ceil_div(items, 256)), dim3(256), 0, stream,
                        (const float*)ws.fill, channels, slot_src, slot_dst, n_pad, (float*)dqkv);

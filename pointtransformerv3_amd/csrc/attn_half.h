@@ -22,6 +22,30 @@ constexpr int ATT_THREADS = 512;   // 8 waves, two work-groups per CU -> 4 waves
 constexpr int ATT_WAVES = ATT_THREADS / PTV3_WAVE;
 constexpr int VT_PAD_BYTES = 16;   // skews V^T rows across LDS banks
 
+// Attention dropout (model.py:470, :480): probability (head, query slot q, key slot k) is kept when a 32-bit
+// hash of (seed, head, q, k) reaches the threshold p * 2^32; forward and backward kernels recompute the same
+// bits instead of storing a mask. hq = the part that does not depend on the key.
+__device__ __forceinline__ uint32_t drop_hq(uint32_t seed, uint32_t head, uint32_t q) {
+    return (q * 0x9E3779B1u) ^ ((head + 1u) * 0xC2B2AE3Du) ^ seed;
+}
+__device__ __forceinline__ bool drop_keep(uint32_t hq, uint32_t k, uint32_t threshold) {
+    uint32_t x = hq ^ ((k + 0x7F4A7C15u) * 0x85EBCA77u);
+    x ^= x >> 16;
+    x *= 0x7FEB352Du;
+    x ^= x >> 15;
+    x *= 0x846CA68Bu;
+    x ^= x >> 16;
+    return x >= threshold;
+}
+static inline uint32_t drop_threshold(float p) {
+    const double t = (double)p * 4294967296.0;
+    return t >= 4294967295.0 ? 0xFFFFFFFFu : (uint32_t)t;
+}
+struct Dropout {
+    uint32_t seed, threshold;   // threshold 0: no dropout
+    float inv_keep;             // 1 / (1 - p)
+};
+
 template <typename T> struct Half;
 template <> struct Half<_Float16> {
     typedef f16x8 v8;

@@ -241,8 +241,8 @@ class SerializedAttention(PointModule):
             # that no padding is ever needed (model.py:359-363, :441-444)
             self.patch_size_max = patch_size
             self.patch_size = 0
-        assert attn_drop == 0.0, "attention dropout is a training feature outside this forward path"
-        self.attn_drop = attn_drop
+        assert 0.0 <= attn_drop < 1.0
+        self.attn_drop = attn_drop   # applied inside the attention kernels in training mode (model.py:470, :480)
         self.qkv = nn.Linear(channels, channels * 3, bias=qkv_bias)
         self.proj = nn.Linear(channels, channels)
         self.proj_drop = nn.Dropout(proj_drop)
@@ -275,6 +275,15 @@ class SerializedAttention(PointModule):
         _, _, cu_seqlens = self.get_padding_and_inverse(point)
         slot_src, slot_dst = self._slots(point)
         grad = ops.wants_grad(qkv, self.rpe.rpe_table if self.enable_rpe else None)
+        drop_p = self.attn_drop if self.training else 0.0
+        if drop_p > 0.0:
+            if self.enable_rpe:
+                raise NotImplementedError("attention dropout together with the relative position bias is not built")
+            from .autograd import PatchAttention
+            seed = int(torch.randint(0, 2 ** 31 - 1, (1,)).item())   # torch's CPU generator: follows torch.manual_seed
+            half = qkv.half() if (self.enable_flash and qkv.dtype == torch.float32) else qkv
+            return PatchAttention.apply(half, self.num_heads, slot_src, slot_dst, cu_seqlens, self.patch_size,
+                                        self.scale, drop_p, seed).to(qkv.dtype)
         if grad and self.enable_rpe:
             from .autograd import PatchAttentionRpe
             out = PatchAttentionRpe.apply(qkv.float(), self.rpe.rpe_table, self.num_heads, slot_src, slot_dst, cu_seqlens,

@@ -277,8 +277,10 @@ def patch_attention(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, 
     return out
 
 
-def patch_attention_lse(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale):
-    """patch_attention (fp16 / bf16) that also returns the (heads, n_pad) log-sum-exp rows the backward uses."""
+def patch_attention_lse(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale, dropout_p=0.0, seed=0):
+    """patch_attention for training: (out, lse) with lse the (heads, n_pad) log-sum-exp rows the half-precision
+    backward uses (None in fp32, where the backward recomputes them). dropout_p > 0: attention dropout, the kept
+    probabilities chosen by a hash of (seed, head, query slot, key slot) that the backward recomputes."""
     _dev(qkv, slot_src, slot_dst, cu_seqlens)
     lib = _lib.load()
     qkv = qkv.contiguous()
@@ -286,17 +288,20 @@ def patch_attention_lse(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seql
     c = c3 // 3
     n_pad = slot_src.shape[0]
     out = torch.empty((n, c), dtype=qkv.dtype, device=qkv.device)
-    lse = torch.empty((int(num_heads), n_pad), dtype=torch.float32, device=qkv.device)
+    lse = None
+    if qkv.dtype != torch.float32:
+        lse = torch.empty((int(num_heads), n_pad), dtype=torch.float32, device=qkv.device)
     _lib.check(lib.ptv3_patch_attn_fwd_lse(_ptr(qkv), _dtype_code(qkv), n, c, int(num_heads), _ptr(slot_src),
                                            _ptr(slot_dst), _ptr(cu_seqlens), cu_seqlens.shape[0] - 1, int(max_seqlen),
-                                           n_pad, float(scale), _ptr(out), _ptr(lse), _stream()),
-               "ptv3_patch_attn_fwd_lse")
+                                           n_pad, float(scale), float(dropout_p), int(seed) & 0xFFFFFFFF, _ptr(out),
+                                           _ptr(lse), _stream()), "ptv3_patch_attn_fwd_lse")
     return out, lse
 
 
-def patch_attention_bwd(qkv, out, dout, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale, lse=None):
+def patch_attention_bwd(qkv, out, dout, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale, lse=None,
+                        dropout_p=0.0, seed=0):
     """Gradient of patch_attention with respect to qkv, (N, 3C) laid out [dq | dk | dv]; lse from
-    patch_attention_lse saves the backward kernel a sweep over the keys."""
+    patch_attention_lse saves the backward kernel a sweep over the keys; dropout_p and seed as in the forward."""
     _dev(qkv, out, dout, slot_src, slot_dst, cu_seqlens)
     lib = _lib.load()
     qkv, out = qkv.contiguous(), out.contiguous()
@@ -310,8 +315,8 @@ def patch_attention_bwd(qkv, out, dout, num_heads, slot_src, slot_dst, cu_seqlen
     ws = _ws(nbytes, qkv.device)
     _lib.check(lib.ptv3_patch_attn_bwd(_ptr(qkv), _ptr(out), _ptr(dout), code, n, c, int(num_heads), _ptr(slot_src),
                                        _ptr(slot_dst), _ptr(cu_seqlens), cu_seqlens.shape[0] - 1, int(max_seqlen),
-                                       n_pad, float(scale), _ptr(lse), _ptr(dqkv), _ptr(ws), nbytes, _stream()),
-               "ptv3_patch_attn_bwd")
+                                       n_pad, float(scale), _ptr(lse), float(dropout_p), int(seed) & 0xFFFFFFFF,
+                                       _ptr(dqkv), _ptr(ws), nbytes, _stream()), "ptv3_patch_attn_bwd")
     return dqkv
 
 
@@ -356,7 +361,7 @@ def patch_attention_rpe_bwd(qkv, out, dout, num_heads, slot_src, slot_dst, cu_se
     ws = _ws(nbytes, qkv.device)
     _lib.check(lib.ptv3_patch_attn_rpe_bwd(_ptr(qkv), _ptr(out), _ptr(dout), 0, n, c, int(num_heads), _ptr(slot_src),
                                            _ptr(slot_dst), _ptr(cu_seqlens), cu_seqlens.shape[0] - 1, int(max_seqlen),
-                                           n_pad, float(scale), None, _ptr(g), _ptr(t), int(pos_bnd), _ptr(dtable),
+                                           n_pad, float(scale), None, 0.0, 0, _ptr(g), _ptr(t), int(pos_bnd), _ptr(dtable),
                                            _ptr(dqkv), _ptr(ws), nbytes, _stream()), "ptv3_patch_attn_rpe_bwd")
     return dqkv, dtable
 

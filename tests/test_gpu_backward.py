@@ -54,6 +54,45 @@ def test_attention_backward_parity(dtype, counts, patch):
         assert rel_err(x.grad[:, sl], want[:, sl]) < TOL[dtype], part
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("counts,patch,p", [([100], 32, 0.25), ([300, 17, 129], 128, 0.1), ([2500], 1024, 0.5)])
+def test_attention_dropout_forward_and_backward_parity(dtype, counts, patch, p):
+    """Attention dropout: the kernels' mask is a hash of (seed, head, query slot, key slot) that the oracle
+    restates, so result and gradient are compared exactly like without dropout; the kept fraction is 1 - p."""
+    from pointtransformerv3_amd.autograd import PatchAttention
+    heads, seed = 4, 1000 + patch
+    rng = np.random.default_rng(seed)
+    g = torch.Generator().manual_seed(seed)
+    n, C = int(sum(counts)), heads * 16
+    offset = np.cumsum(counts).astype(np.int64)
+    starts = np.concatenate([[0], offset[:-1]])
+    order = np.concatenate([s + rng.permutation(c) for s, c in zip(starts, counts)]).astype(np.int64)
+    inverse = np.empty(n, np.int64)
+    inverse[order] = np.arange(n)
+    qkv = torch.randn(n, 3 * C, generator=g).to(dtype)
+    dout = torch.randn(n, C, generator=g).to(dtype)
+    pad, unpad, cu = OI.padding_tables(offset, patch)
+    xr = qkv.float().clone().requires_grad_(True)
+    want = OF.serialized_attention_core(xr, order, inverse, pad, unpad, cu, heads, dropout=(p, seed))
+    want.backward(dout.float())
+    plain = OF.serialized_attention_core(qkv.float(), order, inverse, pad, unpad, cu, heads)
+    assert rel_err(want, plain) > 0.05                                   # the mask does something
+    keep = OF.dropout_keep_mask(seed, 1, np.arange(len(pad)), np.arange(min(len(pad), 512)), p)
+    assert abs(keep.mean() - (1 - p)) < 0.01
+    o = ops()
+    gp, gu, gc = o.pad_index(to_dev(offset), offset.tolist(), patch)
+    src, dst = o.attn_slots(to_dev(order), to_dev(inverse), gp, gu)
+    x = qkv.to(DEV).requires_grad_(True)
+    out = PatchAttention.apply(x, heads, src, dst, gc, patch, 16 ** -0.5, p, seed)
+    out.backward(dout.to(DEV))
+    assert rel_err(out, want) < TOL[dtype]
+    assert rel_err(x.grad, xr.grad) < TOL[dtype]
+    # another seed, another mask; the same seed, the same result
+    again = PatchAttention.apply(x.detach(), heads, src, dst, gc, patch, 16 ** -0.5, p, seed)
+    other = PatchAttention.apply(x.detach(), heads, src, dst, gc, patch, 16 ** -0.5, p, seed + 1)
+    assert torch.equal(again, out.detach()) and rel_err(other, want) > 0.05
+
+
 @pytest.mark.parametrize("counts,patch", [([64], 64), ([700, 300], 256), ([1500], 512)])
 def test_attention_rpe_backward_parity_fp32(counts, patch):
     """Relative position bias path: gradients of qkv and of the bias table vs autograd over the CPU oracle."""
@@ -372,7 +411,7 @@ def test_training_step_under_autocast(dtype):
     assert losses[-1] < losses[0]
 
 
-@pytest.mark.parametrize("variant", ["pdnorm", "post_norm", "cls_mode", "no_flash_fp32", "input_gradient", "rpe"])
+@pytest.mark.parametrize("variant", ["pdnorm", "post_norm", "cls_mode", "no_flash_fp32", "input_gradient", "rpe", "attn_drop"])
 def test_training_step_of_model_variants(variant):
     """One forward + backward of the model built other ways: every parameter that takes part gets a finite
     gradient (PDNorm only trains the norms of the condition it is given)."""
@@ -386,6 +425,8 @@ def test_training_step_of_model_variants(variant):
         kw = dict(cls_mode=True)
     elif variant == "no_flash_fp32":
         kw, autocast = dict(enable_flash=False), None
+    elif variant == "attn_drop":
+        kw = dict(attn_drop=0.1, proj_drop=0.1)
     elif variant == "rpe":
         kw, autocast = dict(enable_flash=False, enable_rpe=True, upcast_attention=True, upcast_softmax=True), None
     torch.manual_seed(3)
