@@ -130,3 +130,21 @@ def test_unpool_add_gradient():
     ch = torch.zeros(4, 3, requires_grad=True)
     OF.unpool_add(p, ch, cluster).backward(torch.tensor(dout))
     assert torch.allclose(dparent, p.grad) and torch.allclose(dchild, ch.grad, atol=1e-6)
+
+
+def test_dropout_mask_statistics():
+    """The attention-dropout mask both the kernels and the oracle use: kept fraction 1 - p, rows and columns
+    balanced, and no visible dependence between heads, seeds or neighbouring slots."""
+    q = np.arange(3000, 5048)
+    k = np.arange(100, 2148)
+    for p in (0.1, 0.3, 0.5):
+        m = OF.dropout_keep_mask(7, 0, q, k, p)
+        assert abs(m.mean() - (1 - p)) < 3e-3
+        assert np.abs(m.mean(0) - (1 - p)).max() < 0.06 and np.abs(m.mean(1) - (1 - p)).max() < 0.06
+    a = OF.dropout_keep_mask(7, 0, q, k, 0.5).astype(np.float64) - 0.5
+    for other in (OF.dropout_keep_mask(7, 1, q, k, 0.5), OF.dropout_keep_mask(8, 0, q, k, 0.5),
+                  OF.dropout_keep_mask(7, 0, q + 1, k, 0.5), OF.dropout_keep_mask(7, 0, q, k + 1, 0.5)):
+        b = other.astype(np.float64) - 0.5
+        assert abs((a * b).mean() / 0.25) < 5e-3          # correlation of two masks of four million bits
+    assert np.array_equal(OF.dropout_keep_mask(7, 0, q, k, 0.5), OF.dropout_keep_mask(7, 0, q, k, 0.5))
+    assert OF.dropout_keep_mask(1, 0, q, k, 0.0).all()
