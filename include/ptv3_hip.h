@@ -112,12 +112,12 @@ int ptv3_patch_attn_fwd(const void *qkv, int dtype, int64_t n_rows, int channels
  * applies it on its non-fused path, in float): score(query i, key j, head h) +=
  * sum over the axes a of rpe_table[a * R + clamp(g_i[a] - g_j[a], -pos_bnd, pos_bnd) + pos_bnd][h],
  * R = 2 * pos_bnd + 1; grid_coord (n_rows, 3) int32 in point order, rpe_table (3 * R, heads) fp32,
- * pos_bnd <= 128. */
+ * pos_bnd <= 128. dropout_p, dropout_seed: attention dropout as in ptv3_patch_attn_fwd_lse (0, 0 for none). */
 int ptv3_patch_attn_rpe_fwd(const float *qkv, int64_t n_rows, int channels, int heads,
                             const int32_t *slot_src, const int32_t *slot_dst,
                             const int32_t *cu_seqlens, int64_t n_seq, int64_t max_seqlen, float scale,
-                            const int32_t *grid_coord, const float *rpe_table, int pos_bnd, float *out,
-                            void *stream);
+                            const int32_t *grid_coord, const float *rpe_table, int pos_bnd, float dropout_p,
+                            uint32_t dropout_seed, float *out, void *stream);
 
 /* ptv3_patch_attn_fwd for training. fp16 / bf16: also keeps what the backward pass needs, lse (heads, n_pad)
  * fp32, lse[h][slot] = log2 of the sum over the slot's sequence of 2^(score * log2(e)) for every real slot
@@ -148,7 +148,7 @@ int ptv3_patch_attn_bwd(const void *qkv, const void *out, const void *dout, int 
 /* Backward of ptv3_patch_attn_rpe_fwd (fp32): as ptv3_patch_attn_bwd, with the relative position bias of
  * model.py:297-316 in the scores; drpe_table (3 * R, heads) fp32 is accumulated into (zero it first):
  * entry [a * R + c][h] += sum of dS(h, i, j) over the pairs (i, j) whose clamped offset along axis a is c.
- * grid_coord == NULL: exactly ptv3_patch_attn_bwd. (The relative-position forward has no dropout: pass 0.) */
+ * grid_coord == NULL: exactly ptv3_patch_attn_bwd. */
 int ptv3_patch_attn_rpe_bwd(const void *qkv, const void *out, const void *dout, int dtype, int64_t n_rows,
                             int channels, int heads, const int32_t *slot_src, const int32_t *slot_dst,
                             const int32_t *cu_seqlens, int64_t n_seq, int64_t max_seqlen, int64_t n_pad,

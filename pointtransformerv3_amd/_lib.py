@@ -28,7 +28,8 @@ SIGNATURES = {
     "ptv3_attn_slots": (_i32, [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp]),
     "ptv3_patch_attn_fwd": (_i32, [_vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _f32,
                                    _vp, _vp]),
-    "ptv3_patch_attn_rpe_fwd": (_i32, [_vp, _i64, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _f32, _vp, _vp, _i32, _vp, _vp]),
+    "ptv3_patch_attn_rpe_fwd": (_i32, [_vp, _i64, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _f32, _vp, _vp, _i32, _f32,
+                                       ctypes.c_uint32, _vp, _vp]),
     "ptv3_patch_attn_bwd_workspace_bytes": (_sz, [_i32, _i64, _i32, _i32]),
     "ptv3_patch_attn_fwd_lse": (_i32, [_vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _f32,
                                        ctypes.c_uint32, _vp, _vp, _vp]),

@@ -28,18 +28,19 @@ class PatchAttentionRpe(torch.autograd.Function):
     gradient too."""
 
     @staticmethod
-    def forward(ctx, qkv, rpe_table, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale, grid_coord, pos_bnd):
+    def forward(ctx, qkv, rpe_table, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale, grid_coord, pos_bnd,
+                dropout_p=0.0, seed=0):
         args = (num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale, grid_coord)
-        out = ops.patch_attention_rpe(qkv, *args, rpe_table.detach(), pos_bnd)
+        out = ops.patch_attention_rpe(qkv, *args, rpe_table.detach(), pos_bnd, dropout_p, seed)
         ctx.save_for_backward(qkv, out, rpe_table)
-        ctx.args, ctx.pos_bnd = args, pos_bnd
+        ctx.args, ctx.pos_bnd, ctx.dropout = args, pos_bnd, (dropout_p, seed)
         return out
 
     @staticmethod
     def backward(ctx, dout):
         qkv, out, table = ctx.saved_tensors
-        dqkv, dtable = ops.patch_attention_rpe_bwd(qkv, out, dout, *ctx.args, table, ctx.pos_bnd)
-        return (dqkv, dtable.to(table.dtype)) + (None,) * 8
+        dqkv, dtable = ops.patch_attention_rpe_bwd(qkv, out, dout, *ctx.args, table, ctx.pos_bnd, *ctx.dropout)
+        return (dqkv, dtable.to(table.dtype)) + (None,) * 10
 
 
 class SubMConv(torch.autograd.Function):

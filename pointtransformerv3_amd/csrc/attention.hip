@@ -370,7 +370,7 @@ __global__ __launch_bounds__(F32_QB) void patch_attn_rpe_f32_kernel(
     const float* __restrict__ qkv, int channels, int heads, const int32_t* __restrict__ slot_src,
     const int32_t* __restrict__ slot_dst, const int32_t* __restrict__ cu_seqlens, int q_blocks,
     float scale, const int32_t* __restrict__ grid_coord, const float* __restrict__ rpe_table, int pos_bnd,
-    float* __restrict__ out) {
+    float* __restrict__ out, Dropout drop) {
     __shared__ float k_lds[F32_KC][HD];
     __shared__ float v_lds[F32_KC][HD];
     __shared__ int32_t c_lds[F32_KC][3];
@@ -401,6 +401,7 @@ __global__ __launch_bounds__(F32_QB) void patch_attn_rpe_f32_kernel(
         qy = grid_coord[3 * r + 1];
         qz = grid_coord[3 * r + 2];
     }
+    const uint32_t hq = drop_hq(drop.seed, (uint32_t)head, (uint32_t)(s0 + qi));
     float m = -INFINITY, l = 0.f;
     for (int c0 = 0; c0 < len; c0 += F32_KC) {
         __syncthreads();
@@ -434,14 +435,15 @@ __global__ __launch_bounds__(F32_QB) void patch_attn_rpe_f32_kernel(
                 for (int d = 0; d < HD; ++d) o[d] *= a;
                 m = s;
             }
-            const float p = __expf(s - m);
+            float p = __expf(s - m);
             l += p;
+            if (drop.threshold && !drop_keep(hq, (uint32_t)(s0 + c0 + key), drop.threshold)) p = 0.f;
 #pragma unroll
             for (int d = 0; d < HD; ++d) o[d] = fmaf(p, v_lds[key][d], o[d]);
         }
     }
     if (dst >= 0) {
-        const float inv = 1.f / l;
+        const float inv = drop.inv_keep / l;
         float* dstp = out + (int64_t)dst * channels + head * HD;
 #pragma unroll
         for (int d = 0; d < HD; ++d) dstp[d] = o[d] * inv;
@@ -556,8 +558,10 @@ extern "C" int ptv3_patch_attn_fwd_lse(const void* qkv, int dtype, int64_t n_row
 extern "C" int ptv3_patch_attn_rpe_fwd(const float* qkv, int64_t n_rows, int channels, int heads,
                                        const int32_t* slot_src, const int32_t* slot_dst,
                                        const int32_t* cu_seqlens, int64_t n_seq, int64_t max_seqlen, float scale,
-                                       const int32_t* grid_coord, const float* rpe_table, int pos_bnd, float* out,
-                                       void* stream_) {
+                                       const int32_t* grid_coord, const float* rpe_table, int pos_bnd, float dropout_p,
+                                       uint32_t dropout_seed, float* out, void* stream_) {
+    if (!(dropout_p >= 0.f) || !(dropout_p < 1.f)) return PTV3_EINVAL;
+    const Dropout drop = {dropout_seed, dropout_p > 0.f ? drop_threshold(dropout_p) : 0u, 1.f / (1.f - dropout_p)};
     if (n_rows < 0 || n_seq < 0 || channels < 1 || heads < 1 || max_seqlen < 1) return PTV3_EINVAL;
     if (pos_bnd < 0 || pos_bnd > RPE_MAX_BND) return PTV3_ESHAPE;
     if (channels % heads != 0 || channels / heads != HD) return PTV3_ESHAPE;
@@ -567,6 +571,6 @@ extern "C" int ptv3_patch_attn_rpe_fwd(const float* qkv, int64_t n_rows, int cha
     if (n_seq * heads * q_blocks >= (1ll << 31)) return PTV3_EINVAL;
     hipLaunchKernelGGL(patch_attn_rpe_f32_kernel, dim3((unsigned)(n_seq * heads * q_blocks)), dim3(F32_QB), 0,
                        (hipStream_t)stream_, qkv, channels, heads, slot_src, slot_dst, cu_seqlens, q_blocks, scale,
-                       grid_coord, rpe_table, pos_bnd, out);
+                       grid_coord, rpe_table, pos_bnd, out, drop);
     PTV3_RETURN_LAUNCH();
 }

@@ -277,10 +277,13 @@ class SerializedAttention(PointModule):
         grad = ops.wants_grad(qkv, self.rpe.rpe_table if self.enable_rpe else None)
         drop_p = self.attn_drop if self.training else 0.0
         if drop_p > 0.0:
-            if self.enable_rpe:
-                raise NotImplementedError("attention dropout together with the relative position bias is not built")
-            from .autograd import PatchAttention
+            from .autograd import PatchAttention, PatchAttentionRpe
             seed = int(torch.randint(0, 2 ** 31 - 1, (1,)).item())   # torch's CPU generator: follows torch.manual_seed
+            if self.enable_rpe:
+                out = PatchAttentionRpe.apply(qkv.float(), self.rpe.rpe_table, self.num_heads, slot_src, slot_dst,
+                                              cu_seqlens, self.patch_size, self.scale, point.grid_coord,
+                                              self.rpe.pos_bnd, drop_p, seed)
+                return out.to(qkv.dtype)
             half = qkv.half() if (self.enable_flash and qkv.dtype == torch.float32) else qkv
             return PatchAttention.apply(half, self.num_heads, slot_src, slot_dst, cu_seqlens, self.patch_size,
                                         self.scale, drop_p, seed).to(qkv.dtype)

@@ -321,7 +321,7 @@ def patch_attention_bwd(qkv, out, dout, num_heads, slot_src, slot_dst, cu_seqlen
 
 
 def patch_attention_rpe(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale, grid_coord, rpe_table,
-                        pos_bnd):
+                        pos_bnd, dropout_p=0.0, seed=0):
     """patch_attention with the relative position bias of model.py:297-316 added to every score:
     fp32 qkv (N, 3C), grid_coord (N, 3) in point order, rpe_table (3 * (2 * pos_bnd + 1), H)."""
     _dev(qkv, slot_src, slot_dst, cu_seqlens, grid_coord, rpe_table)
@@ -338,13 +338,14 @@ def patch_attention_rpe(qkv, num_heads, slot_src, slot_dst, cu_seqlens, max_seql
     out = torch.empty((n, c), dtype=torch.float32, device=qkv.device)
     _lib.check(lib.ptv3_patch_attn_rpe_fwd(_ptr(qkv), n, c, int(num_heads), _ptr(slot_src), _ptr(slot_dst),
                                            _ptr(cu_seqlens), cu_seqlens.shape[0] - 1, int(max_seqlen), float(scale),
-                                           _ptr(g), _ptr(t), int(pos_bnd), _ptr(out), _stream()),
+                                           _ptr(g), _ptr(t), int(pos_bnd), float(dropout_p), int(seed) & 0xFFFFFFFF,
+                                           _ptr(out), _stream()),
                "ptv3_patch_attn_rpe_fwd")
     return out
 
 
 def patch_attention_rpe_bwd(qkv, out, dout, num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen, scale, grid_coord,
-                            rpe_table, pos_bnd):
+                            rpe_table, pos_bnd, dropout_p=0.0, seed=0):
     """(dqkv, drpe_table) of patch_attention_rpe: fp32, the table's gradient (3 * (2 * pos_bnd + 1), H) in fp32."""
     _dev(qkv, out, dout, slot_src, slot_dst, cu_seqlens, grid_coord, rpe_table)
     lib = _lib.load()
@@ -361,7 +362,8 @@ def patch_attention_rpe_bwd(qkv, out, dout, num_heads, slot_src, slot_dst, cu_se
     ws = _ws(nbytes, qkv.device)
     _lib.check(lib.ptv3_patch_attn_rpe_bwd(_ptr(qkv), _ptr(out), _ptr(dout), 0, n, c, int(num_heads), _ptr(slot_src),
                                            _ptr(slot_dst), _ptr(cu_seqlens), cu_seqlens.shape[0] - 1, int(max_seqlen),
-                                           n_pad, float(scale), None, 0.0, 0, _ptr(g), _ptr(t), int(pos_bnd), _ptr(dtable),
+                                           n_pad, float(scale), None, float(dropout_p), int(seed) & 0xFFFFFFFF, _ptr(g),
+                                           _ptr(t), int(pos_bnd), _ptr(dtable),
                                            _ptr(dqkv), _ptr(ws), nbytes, _stream()), "ptv3_patch_attn_rpe_bwd")
     return dqkv, dtable
 

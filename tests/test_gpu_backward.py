@@ -93,9 +93,11 @@ def test_attention_dropout_forward_and_backward_parity(dtype, counts, patch, p):
     assert torch.equal(again, out.detach()) and rel_err(other, want) > 0.05
 
 
+@pytest.mark.parametrize("drop_p", [0.0, 0.2])
 @pytest.mark.parametrize("counts,patch", [([64], 64), ([700, 300], 256), ([1500], 512)])
-def test_attention_rpe_backward_parity_fp32(counts, patch):
-    """Relative position bias path: gradients of qkv and of the bias table vs autograd over the CPU oracle."""
+def test_attention_rpe_backward_parity_fp32(counts, patch, drop_p):
+    """Relative position bias path (with and without attention dropout): result, gradients of qkv and of the bias
+    table vs autograd over the CPU oracle."""
     from pointtransformerv3_amd.autograd import PatchAttentionRpe
     heads, seed = 4, 33
     rng = np.random.default_rng(seed)
@@ -114,14 +116,17 @@ def test_attention_rpe_backward_parity_fp32(counts, patch):
     pad, unpad, cu = OI.padding_tables(offset, patch)
     xq = qkv.clone().requires_grad_(True)
     tb = table.clone().requires_grad_(True)
-    OF.serialized_attention_core(xq, order, inverse, pad, unpad, cu, heads, rpe=(grid, tb, pos_bnd)).backward(dout)
+    dropout = (drop_p, 77) if drop_p else None
+    want = OF.serialized_attention_core(xq, order, inverse, pad, unpad, cu, heads, rpe=(grid, tb, pos_bnd), dropout=dropout)
+    want.backward(dout)
     o = ops()
     gp, gu, gc = o.pad_index(to_dev(offset), offset.tolist(), patch)
     src, dst = o.attn_slots(to_dev(order), to_dev(inverse), gp, gu)
     x = qkv.to(DEV).requires_grad_(True)
     t = table.to(DEV).requires_grad_(True)
-    out = PatchAttentionRpe.apply(x, t, heads, src, dst, gc, patch, 0.25, to_dev(grid), pos_bnd)
+    out = PatchAttentionRpe.apply(x, t, heads, src, dst, gc, patch, 0.25, to_dev(grid), pos_bnd, drop_p, 77)
     out.backward(dout.to(DEV))
+    assert rel_err(out, want) < 1e-4
     assert rel_err(x.grad, xq.grad) < 1e-4
     assert rel_err(t.grad, tb.grad) < 1e-4
 
