@@ -303,6 +303,36 @@ size_t ptv3_linear_wgrad_workspace_bytes(int64_t n, int k, int nout);
 int ptv3_linear_wgrad(const void *x, const void *dout, int dtype, int64_t n, int k, int nout, float *dweight,
                       float *dbias, void *workspace, size_t workspace_bytes, void *stream);
 
+/* The first Linear of the MLP with its GELU, for training (model.py:505-507: fc1, act): pre = x w^T + bias and
+ * out = gelu(pre), both (n,nout) of dtype, from one pass; shapes as for ptv3_linear_fwd. */
+int ptv3_linear_gelu_fwd(const void *x, const void *w, const void *bias, int dtype, int64_t n, int k, int nout,
+                         void *pre, void *out, void *stream);
+
+/* Input gradient of the second Linear of the MLP taken back through the GELU in front of it (model.py:506-507):
+ * dpre = (dout wt^T) * gelu'(pre). dout (n,k) is the gradient of fc2's output, wt (nout,k) fc2's weight
+ * transposed (hidden x out channels), pre (n,nout) as written by ptv3_linear_gelu_fwd, dpre (n,nout). */
+int ptv3_linear_gelu_bwd(const void *dout, const void *wt, const void *pre, int dtype, int64_t n, int k, int nout,
+                         void *dpre, void *stream);
+
+/* Half-precision and transposed copies of fp32 master weights, many tensors per launch: what autocast does to the
+ * weight of every nn.Linear / spconv.SubMConv3d (model.py:366-367, :505-507, :546-553, :767-774) on each use, and
+ * the transposes their input gradients multiply by. One job per tensor; src is a contiguous fp32 (a, b, c) array.
+ *   mirror = 0: dst[i] = src[i] for all a*b*c elements;
+ *   mirror = 1: dst[(k*b + (b-1-j))*a + i] = src[(i*b + j)*c + k] -- (Cout, taps, Cin) to (Cin, mirrored taps, Cout);
+ *               with b = 1 the plain transpose of a matrix.
+ * first_block is the running sum of ptv3_cast_params_blocks(a, b, c, mirror) over the jobs before this one, and
+ * n_blocks the sum over all jobs. The table itself lies in device memory, dst are of dst_dtype and must not
+ * overlap any src. Shapes in the table are not checked: a wrong table writes out of bounds. */
+typedef struct {
+    const float *src;
+    void *dst;
+    int32_t a, b, c;
+    int32_t mirror;
+    int64_t first_block;
+} ptv3_cast_job;
+int64_t ptv3_cast_params_blocks(int a, int b, int c, int mirror);
+int ptv3_cast_params(const ptv3_cast_job *jobs, int n_jobs, int64_t n_blocks, int dst_dtype, void *stream);
+
 /* nn.LayerNorm for training (model.py:554, :557, :572), with the residual connection in front of it taken
  * into the same pass where there is one (model.py:589-604):
  * sum = skip + branch * row_scale, y = LayerNorm(sum). skip (n,c) and row_scale (n,) -- the stochastic-depth

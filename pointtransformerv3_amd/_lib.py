@@ -76,6 +76,10 @@ SIGNATURES = {
     "ptv3_batch_norm_stats": (_i32, [_vp, _i32, _i64, _i32, _f32, _f32, _vp, _vp, _vp, _vp, _vp]),
     "ptv3_batch_norm_bwd": (_i32, [_vp, _i32, _vp, _i32, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _i32, _vp,
                                    _vp]),
+    "ptv3_linear_gelu_fwd": (_i32, [_vp, _vp, _vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp]),
+    "ptv3_linear_gelu_bwd": (_i32, [_vp, _vp, _vp, _i32, _i64, _i32, _i32, _vp, _vp]),
+    "ptv3_cast_params_blocks": (_i64, [_i32, _i32, _i32, _i32]),
+    "ptv3_cast_params": (_i32, [_vp, _i32, _i64, _i32, _vp]),
     "ptv3_linear_wgrad_workspace_bytes": (_sz, [_i64, _i32, _i32]),
     "ptv3_linear_wgrad": (_i32, [_vp, _vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
     "ptv3_linear_ln_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _f32, _vp, _vp, _vp]),

@@ -67,10 +67,9 @@ class SubMConv(torch.autograd.Function):
         dfeat = dweight = dbias = None
         if ctx.needs_input_grad[0]:
             # the same convolution with mirrored taps and the weight transposed
-            wt = weight.detach().reshape(cout, -1, cin).flip(1).permute(2, 1, 0).contiguous()
-            pad = -cin % 16 if dout.dtype != torch.float32 else 0   # the half-precision forms write outputs in 16s
-            if pad:
-                wt = torch.nn.functional.pad(wt, (0, 0, 0, 0, 0, pad))
+            wt = ops.cast_cached(weight, dout.dtype, "mirror")
+            if dout.dtype != torch.float32 and cin % 16:   # the half-precision forms write outputs in 16s
+                wt = torch.nn.functional.pad(wt, (0, 0, 0, 0, 0, -cin % 16))
             dfeat = module.convolve(sparse, dout, wt, None)[:, :cin].to(feat.dtype)
         if ctx.needs_input_grad[1]:
             nbr = sparse.neighbour_map(module.kernel_size, module.indice_key)
@@ -108,7 +107,7 @@ class Linear(torch.autograd.Function):
         dout = dout.contiguous()
         dx = None
         if ctx.needs_input_grad[0]:
-            wt = ops.cast_cached(weight, dout.dtype, transpose=True)   # (K, Nout): dx = dout wt^T
+            wt = ops.cast_cached(weight, dout.dtype, "transpose")   # (K, Nout): dx = dout wt^T
             if ops.linear_rows_pays(dout, wt):
                 dx = ops.linear_rows(dout, wt)   # many rows, few channels: the row kernel again
             else:
@@ -121,6 +120,47 @@ class Linear(torch.autograd.Function):
         if want_bias:
             db = db.to(ctx.bias_dtype) if db is not None else dout.sum(0, dtype=torch.float32).to(ctx.bias_dtype)
         return dx, dw, db if want_bias else None
+
+
+class Mlp(torch.autograd.Function):
+    """fc2(gelu(fc1 x)) (model.py:493-516 without dropout) for half-precision rows; weights and biases may be
+    fp32 masters. The GELU's input and output are both kept, as autograd would keep them."""
+
+    @staticmethod
+    def forward(ctx, x, w1, b1, w2, b2):
+        dt = x.dtype
+        pre, act = ops.linear_gelu(x, ops.cast_cached(w1, dt), None if b1 is None else ops.cast_cached(b1, dt))
+        cw2, cb2 = ops.cast_cached(w2, dt), None if b2 is None else ops.cast_cached(b2, dt)
+        if ops.linear_rows_pays(act, cw2):
+            out = ops.linear_rows(act, cw2, cb2)
+        else:
+            out = torch.nn.functional.linear(act, cw2, cb2)
+        ctx.save_for_backward(x, pre, act, w1, w2)
+        ctx.bias_dtypes = tuple(None if b is None else b.dtype for b in (b1, b2))
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        x, pre, act, w1, w2 = ctx.saved_tensors
+        dout = dout.contiguous()
+        dt = dout.dtype
+        dpre = ops.linear_gelu_bwd(dout, ops.cast_cached(w2, dt, "transpose"), pre)
+        dx = None
+        if ctx.needs_input_grad[0]:
+            w1t = ops.cast_cached(w1, dt, "transpose")   # (in, hidden): dx = dpre w1t^T
+            dx = ops.linear_rows(dpre, w1t) if ops.linear_rows_pays(dpre, w1t) else dpre @ ops.cast_cached(w1, dt)
+        grads = []
+        for inp, dy, w, bias_dtype, wi in ((x, dpre, w1, ctx.bias_dtypes[0], 1), (act, dout, w2, ctx.bias_dtypes[1], 3)):
+            dw = db = None
+            if ctx.needs_input_grad[wi]:
+                dw, db = ops.linear_wgrad(inp, dy, with_bias=True)
+                dw = dw.to(w.dtype)
+            if bias_dtype is not None and ctx.needs_input_grad[wi + 1]:
+                db = db.to(bias_dtype) if db is not None else dy.sum(0, dtype=torch.float32).to(bias_dtype)
+            else:
+                db = None
+            grads += [dw, db]
+        return (dx, *grads)
 
 
 class LayerNorm(torch.autograd.Function):

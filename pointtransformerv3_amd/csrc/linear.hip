@@ -30,12 +30,17 @@ struct LinBn {
     int stats_f32;
 };
 
+// what follows the bias (and the BatchNorm): nothing, the exact GELU, the GELU with the value in front of it
+// kept in aux as well (training: its backward needs it), or a multiplication by gelu'(aux) -- the input
+// gradient of a Linear whose input came out of a GELU (model.py:505-507, fc2 back through act)
+enum { ACT_NONE = 0, ACT_GELU = 1, ACT_GELU_KEEP = 2, ACT_GELU_GRAD = 3 };
+
 // NW waves per work-group, rows staged SW channels at a time (64, or 32 where the weights leave LDS for
 // narrow tile buffers only and the work-group has 16 waves instead of 8)
-template <typename T, int K, bool GELU, bool BN, int NW, int SW>
+template <typename T, int K, int ACT, bool BN, int NW, int SW>
 __global__ __launch_bounds__(NW * PTV3_WAVE, (NW == 8 ? 2 : 1)) void linear_rows_kernel(
     const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ bias, LinBn bn, int64_t n, int nout,
-    int chunk, T* __restrict__ out) {
+    int chunk, T* __restrict__ out, T* __restrict__ aux) {
     typedef typename H16<T>::v8 v8;
     constexpr int KS = K / 16, WS = K + LIN_PAD, LIN_THREADS = NW * PTV3_WAVE, LIN_WAVES = NW, LIN_XSS = SW + LIN_PAD;
     extern __shared__ __align__(16) unsigned char lin_smem[];
@@ -105,6 +110,20 @@ __global__ __launch_bounds__(NW * PTV3_WAVE, (NW == 8 ? 2 : 1)) void linear_rows
         // ---- output channels SW at a time (two 32-tiles, or one)
         for (int o0 = 0; o0 < cn; o0 += SW) {
             const int nt = (cn - o0) >= SW ? SW / 32 : 1;
+            const int ppr_g = nt * 4;                        // 16-byte pieces per row of this group
+            const int its = 32 * ppr_g / PTV3_WAVE;          // 4 or 2
+            u32x4 pre[ACT == ACT_GELU_GRAD ? 4 : 1];         // the GELU's inputs at the places this lane writes
+            if (ACT == ACT_GELU_GRAD) {
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    if (it >= its) break;
+                    const int pidx = it * PTV3_WAVE + lane;
+                    const int64_t r = row0 + pidx / ppr_g;
+                    pre[it] = (u32x4){0, 0, 0, 0};
+                    if (r < n) pre[it] = *(const u32x4*)(aux + r * nout + c0 + o0 + (pidx % ppr_g) * 8);
+                }
+            }
+            u32x2 act[ACT == ACT_GELU_KEEP ? SW / 32 : 1][4];   // the activated values while the plain ones go out
 #pragma unroll
             for (int t = 0; t < SW / 32; ++t) {
                 if (t >= nt) break;
@@ -119,7 +138,7 @@ __global__ __launch_bounds__(NW * PTV3_WAVE, (NW == 8 ? 2 : 1)) void linear_rows
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     const f32x4 bb = *(const f32x4*)(b_lds + o0 + t * 32 + 8 * g + 4 * hf);
-                    float r[4];
+                    float r[4], a[4];
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         r[q] = d[4 * g + q] + bb[q];
@@ -127,32 +146,59 @@ __global__ __launch_bounds__(NW * PTV3_WAVE, (NW == 8 ? 2 : 1)) void linear_rows
                             const int c = o0 + t * 32 + 8 * g + 4 * hf + q;
                             r[q] = (H16<T>::round(r[q]) - mu_lds[c]) * sc_lds[c] + be_lds[c];
                         }
-                        if (GELU) r[q] = gelu_erf(H16<T>::round(r[q]));
+                        if (ACT == ACT_GELU) r[q] = gelu_erf(H16<T>::round(r[q]));
+                        if (ACT == ACT_GELU_KEEP) a[q] = gelu_erf(H16<T>::round(r[q]));
                     }
                     *(u32x2*)(xs + col * LIN_XSS + t * 32 + 8 * g + 4 * hf) =
                         (u32x2){H16<T>::pack2(r[0], r[1]), H16<T>::pack2(r[2], r[3])};
+                    if (ACT == ACT_GELU_KEEP) act[t][g] = (u32x2){H16<T>::pack2(a[0], a[1]), H16<T>::pack2(a[2], a[3])};
                 }
             }
             asm volatile("" ::: "memory");
-            const int ppr_g = nt * 4;                        // 16-byte pieces per row of this group
-            const int its = 32 * ppr_g / PTV3_WAVE;          // 4 or 2
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
                 if (it >= its) break;
                 const int pidx = it * PTV3_WAVE + lane;
                 const int rr = pidx / ppr_g, pc = pidx % ppr_g;
                 const int64_t r = row0 + rr;
-                const u32x4 o4 = *(const u32x4*)(xs + rr * LIN_XSS + pc * 8);
-                if (r < n) *(u32x4*)(out + r * nout + c0 + o0 + pc * 8) = o4;
+                u32x4 o4 = *(const u32x4*)(xs + rr * LIN_XSS + pc * 8);
+                if (ACT == ACT_GELU_GRAD) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const uint32_t hw = pre[it][q], dw = o4[q];
+                        o4[q] = H16<T>::pack2(H16<T>::lo(dw) * gelu_erf_grad(H16<T>::lo(hw)),
+                                              H16<T>::hi(dw) * gelu_erf_grad(H16<T>::hi(hw)));
+                    }
+                }
+                if (r < n) *(u32x4*)((ACT == ACT_GELU_KEEP ? aux : out) + r * nout + c0 + o0 + pc * 8) = o4;
             }
             asm volatile("" ::: "memory");
+            if (ACT == ACT_GELU_KEEP) {
+#pragma unroll
+                for (int t = 0; t < SW / 32; ++t) {
+                    if (t >= nt) break;
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) *(u32x2*)(xs + col * LIN_XSS + t * 32 + 8 * g + 4 * hf) = act[t][g];
+                }
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    if (it >= its) break;
+                    const int pidx = it * PTV3_WAVE + lane;
+                    const int rr = pidx / ppr_g, pc = pidx % ppr_g;
+                    const int64_t r = row0 + rr;
+                    const u32x4 o4 = *(const u32x4*)(xs + rr * LIN_XSS + pc * 8);
+                    if (r < n) *(u32x4*)(out + r * nout + c0 + o0 + pc * 8) = o4;
+                }
+                asm volatile("" ::: "memory");
+            }
         }
     }
 }
 
-template <typename T, int K, bool GELU, bool BN, int NW, int SW>
+template <typename T, int K, int ACT, bool BN, int NW, int SW>
 int launch_linear_shape(const void* x, const void* w, const void* bias, LinBn bn, int64_t n, int nout, void* out,
-                        hipStream_t stream) {
+                        void* aux, hipStream_t stream) {
     // output channels per work-group: as many 32-tiles as the LDS budget holds, spread evenly
     const int cap = (int)(lin_w_bytes(K) / ((K + LIN_PAD) * sizeof(T))) / 32 * 32;
     const int n_chunks = (nout + cap - 1) / cap;
@@ -160,7 +206,7 @@ int launch_linear_shape(const void* x, const void* w, const void* bias, LinBn bn
     constexpr int LIN_WAVES = NW, LIN_THREADS = NW * PTV3_WAVE, LIN_XSS = SW + LIN_PAD;
     const size_t lds = (size_t)chunk * (K + LIN_PAD) * sizeof(T) + (size_t)chunk * sizeof(float) * (BN ? 4 : 1) +
                        (size_t)LIN_WAVES * 32 * LIN_XSS * sizeof(T);
-    auto kern = linear_rows_kernel<T, K, GELU, BN, NW, SW>;
+    auto kern = linear_rows_kernel<T, K, ACT, BN, NW, SW>;
     static size_t lds_allowed = 0;
     if (lds > lds_allowed) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -174,31 +220,37 @@ int launch_linear_shape(const void* x, const void* w, const void* bias, LinBn bn
     const int64_t need = (tiles + LIN_WAVES - 1) / LIN_WAVES;
     if (per_chunk > need) per_chunk = need;
     hipLaunchKernelGGL(kern, dim3((unsigned)per_chunk, (unsigned)n_chunks), dim3(LIN_THREADS), lds, stream, (const T*)x,
-                       (const T*)w, (const T*)bias, bn, n, nout, chunk, (T*)out);
+                       (const T*)w, (const T*)bias, bn, n, nout, chunk, (T*)out, (T*)aux);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? PTV3_OK : (int)e;
 }
 
-template <typename T, int K, bool GELU, bool BN>
-int launch_linear(const void* x, const void* w, const void* bias, LinBn bn, int64_t n, int nout, void* out,
+template <typename T, int K, int ACT, bool BN>
+int launch_linear(const void* x, const void* w, const void* bias, LinBn bn, int64_t n, int nout, void* out, void* aux,
                   hipStream_t stream) {
     // 256 inputs with GELU: the weight chunk takes the LDS of the whole CU and the epilogue is VALU-heavy, so one
     // work-group of 16 waves with 32-channel tile buffers (four waves per SIMD) measured 13 % faster than 8 waves;
     // without GELU, and at 512 inputs where the x fragments alone need 128 registers, the 8-wave shape is faster
-    if constexpr (K == 256 && GELU)
-        return launch_linear_shape<T, K, GELU, BN, 16, 32>(x, w, bias, bn, n, nout, out, stream);
-    return launch_linear_shape<T, K, GELU, BN, 8, 64>(x, w, bias, bn, n, nout, out, stream);
+    if constexpr (K == 256 && ACT != ACT_NONE)
+        return launch_linear_shape<T, K, ACT, BN, 16, 32>(x, w, bias, bn, n, nout, out, aux, stream);
+    return launch_linear_shape<T, K, ACT, BN, 8, 64>(x, w, bias, bn, n, nout, out, aux, stream);
 }
 
+// act: one of ACT_*; the BatchNorm epilogue comes with ACT_NONE and ACT_GELU only
 int dispatch_linear(const void* x, const void* w, const void* bias, const LinBn* bn, int dtype, int64_t n, int k,
-                    int nout, int gelu, void* out, hipStream_t stream) {
+                    int nout, int act, void* out, void* aux, hipStream_t stream) {
     const LinBn none = {nullptr, nullptr, nullptr, nullptr, 0.f, 0};
-#define PTV3_LIN(T, K)                                                                                       \
-    if (k == K) {                                                                                            \
-        if (bn) return gelu ? launch_linear<T, K, true, true>(x, w, bias, *bn, n, nout, out, stream)         \
-                            : launch_linear<T, K, false, true>(x, w, bias, *bn, n, nout, out, stream);       \
-        return gelu ? launch_linear<T, K, true, false>(x, w, bias, none, n, nout, out, stream)               \
-                    : launch_linear<T, K, false, false>(x, w, bias, none, n, nout, out, stream);             \
+#define PTV3_LIN(T, K)                                                                                                \
+    if (k == K) {                                                                                                     \
+        if (bn) return act ? launch_linear<T, K, ACT_GELU, true>(x, w, bias, *bn, n, nout, out, aux, stream)          \
+                           : launch_linear<T, K, ACT_NONE, true>(x, w, bias, *bn, n, nout, out, aux, stream);         \
+        switch (act) {                                                                                                \
+            case ACT_NONE: return launch_linear<T, K, ACT_NONE, false>(x, w, bias, none, n, nout, out, aux, stream);  \
+            case ACT_GELU: return launch_linear<T, K, ACT_GELU, false>(x, w, bias, none, n, nout, out, aux, stream);  \
+            case ACT_GELU_KEEP:                                                                                       \
+                return launch_linear<T, K, ACT_GELU_KEEP, false>(x, w, bias, none, n, nout, out, aux, stream);        \
+            default: return launch_linear<T, K, ACT_GELU_GRAD, false>(x, w, bias, none, n, nout, out, aux, stream);   \
+        }                                                                                                             \
     }
     if (dtype == PTV3_F16) {
         PTV3_LIN(_Float16, 32) PTV3_LIN(_Float16, 64) PTV3_LIN(_Float16, 128) PTV3_LIN(_Float16, 256) PTV3_LIN(_Float16, 512)
@@ -224,7 +276,27 @@ extern "C" int ptv3_linear_fwd(const void* x, const void* w, const void* bias, i
     if (rc != PTV3_OK) return rc;
     if (n == 0) return PTV3_OK;
     if (!x || !w || !out) return PTV3_EINVAL;
-    return dispatch_linear(x, w, bias, nullptr, dtype, n, k, nout, gelu, out, (hipStream_t)stream_);
+    return dispatch_linear(x, w, bias, nullptr, dtype, n, k, nout, gelu ? ACT_GELU : ACT_NONE, out, nullptr,
+                           (hipStream_t)stream_);
+}
+
+extern "C" int ptv3_linear_gelu_fwd(const void* x, const void* w, const void* bias, int dtype, int64_t n, int k,
+                                    int nout, void* pre, void* out, void* stream_) {
+    const int rc = check_linear(dtype, n, k, nout);
+    if (rc != PTV3_OK) return rc;
+    if (n == 0) return PTV3_OK;
+    if (!x || !w || !pre || !out) return PTV3_EINVAL;
+    return dispatch_linear(x, w, bias, nullptr, dtype, n, k, nout, ACT_GELU_KEEP, out, pre, (hipStream_t)stream_);
+}
+
+extern "C" int ptv3_linear_gelu_bwd(const void* dout, const void* wt, const void* pre, int dtype, int64_t n, int k,
+                                    int nout, void* dpre, void* stream_) {
+    const int rc = check_linear(dtype, n, k, nout);
+    if (rc != PTV3_OK) return rc;
+    if (n == 0) return PTV3_OK;
+    if (!dout || !wt || !pre || !dpre) return PTV3_EINVAL;
+    return dispatch_linear(dout, wt, nullptr, nullptr, dtype, n, k, nout, ACT_GELU_GRAD, dpre, const_cast<void*>(pre),
+                           (hipStream_t)stream_);
 }
 
 extern "C" int ptv3_linear_bn_act_fwd(const void* x, const void* w, const void* bias, const void* running_mean,
@@ -236,5 +308,6 @@ extern "C" int ptv3_linear_bn_act_fwd(const void* x, const void* w, const void* 
     if (n == 0) return PTV3_OK;
     if (!x || !w || !running_mean || !running_var || !out) return PTV3_EINVAL;
     const LinBn bn = {running_mean, running_var, gamma, beta, eps, stats_f32};
-    return dispatch_linear(x, w, bias, &bn, dtype, n, k, nout, gelu, out, (hipStream_t)stream_);
+    return dispatch_linear(x, w, bias, &bn, dtype, n, k, nout, gelu ? ACT_GELU : ACT_NONE, out, nullptr,
+                           (hipStream_t)stream_);
 }

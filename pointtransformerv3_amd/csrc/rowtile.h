@@ -64,4 +64,17 @@ __device__ __forceinline__ float gelu_erf(float x) {
     return fmaf(copysignf(erf_abs, x), half_x, half_x);
 }
 
+// d/dx of gelu_erf: Phi(x) + x phi(x); the erf approximation's exponential is phi's as well
+__device__ __forceinline__ float gelu_erf_grad(float x) {
+    const float z = fabsf(x) * 0.70710678118654752f;
+    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
+    float p = fmaf(1.061405429f, t, -1.453152027f);
+    p = fmaf(p, t, 1.421413741f);
+    p = fmaf(p, t, -0.284496736f);
+    p = fmaf(p, t, 0.254829592f);
+    const float e = __builtin_amdgcn_exp2f(-z * z * 1.4426950408889634f);
+    const float erf_abs = fmaf(-p * t, e, 1.0f);
+    return fmaf(x * 0.3989422804014327f, e, fmaf(copysignf(erf_abs, x), 0.5f, 0.5f));
+}
+
 }  // namespace

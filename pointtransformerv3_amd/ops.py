@@ -5,6 +5,7 @@ the HIP kernels. All tensors must live on the GPU; CPU tensors are rejected.
 """
 import ctypes
 
+import numpy as np
 import torch
 
 from . import _lib
@@ -44,52 +45,83 @@ def wants_grad(*tensors):
     return torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors)
 
 
-_CAST_CACHE = {}
+_CAST_CACHE = {}     # (id(parameter), dtype, layout) -> _Cast
+_CAST_TABLES = {}    # (device, dtype) -> (table bytes, device table): optimizer steps ask for the same table again
+_CAST_JOB = np.dtype([("src", "<u8"), ("dst", "<u8"), ("a", "<i4"), ("b", "<i4"), ("c", "<i4"), ("mirror", "<i4"),
+                      ("first_block", "<i8")])   # ptv3_cast_job
 
 
-def _refresh_stale_casts(dtype):
-    """Every remembered plain cast to dtype whose parameter has been written since (an optimizer step touches all
-    of them at once) is redone in place, in one multi-tensor copy instead of one small launch per parameter."""
-    dsts, srcs, entries = [], [], []
-    for key, (stamp, out, ref) in _CAST_CACHE.items():
-        if key[1] != dtype or key[2]:
-            continue
-        t = ref()
-        if t is None:
+class _Cast:
+    __slots__ = ("stamp", "out", "ref", "shape", "mirror")
+
+
+def _cast_shape(t, layout):
+    """(a, b, c) of the parameter as the cast kernel sees it and the shape of the copy. layout "plain" keeps the
+    element order; "transpose" swaps the axes of a matrix; "mirror" turns a convolution weight (Cout, taps..., Cin)
+    into (Cin, mirrored taps, Cout), which is the weight of the input gradient."""
+    if layout == "plain":
+        return (1, 1, t.numel()), tuple(t.shape)
+    a, c = t.shape[0], t.shape[-1]
+    b = t.numel() // (a * c)
+    return (a, b, c), ((c, a) if layout == "transpose" else (c, b, a))
+
+
+def _refresh_stale_casts(dtype, device):
+    """Every remembered copy in dtype whose parameter has been written since (an optimizer step touches all of them
+    at once) is redone in place by one launch instead of a few small ones per parameter."""
+    stale, blocks = [], 0
+    for entry in _CAST_CACHE.values():
+        t = entry.ref()
+        if t is None or entry.out.dtype != dtype or t.device != device:
             continue
         now = (t.data_ptr(), t._version)
-        if now != stamp and out.shape == t.shape and out.device == t.device:
-            dsts.append(out)
-            srcs.append(t.detach())
-            entries.append((key, now, ref))
-    if dsts:
-        with torch.no_grad():
-            torch._foreach_copy_(dsts, srcs)
-        for (key, now, ref), out in zip(entries, dsts):
-            _CAST_CACHE[key] = (now, out, ref)
+        if now != entry.stamp:
+            a, b, c = entry.shape
+            stale.append((entry, now, (t.data_ptr(), entry.out.data_ptr(), a, b, c, entry.mirror, blocks)))
+            blocks += _lib.load().ptv3_cast_params_blocks(a, b, c, entry.mirror)
+    if not stale:
+        return
+    table = np.array([row for _, _, row in stale], dtype=_CAST_JOB).tobytes()
+    held = _CAST_TABLES.get((device, dtype))
+    if held is None or held[0] != table:
+        held = (table, torch.frombuffer(bytearray(table), dtype=torch.uint8).to(device))
+        _CAST_TABLES[(device, dtype)] = held
+    with torch.cuda.device(device):
+        _lib.check(_lib.load().ptv3_cast_params(held[1].data_ptr(), len(stale), blocks, _DTYPE_CODE[dtype],
+                                                _stream()), "ptv3_cast_params")
+    for entry, now, _ in stale:
+        entry.stamp = now
 
 
-def cast_cached(t, dtype, transpose=False):
-    """t.to(dtype) (transposed and made contiguous if asked) for a parameter, remembered until the parameter is
-    written to or moved: training casts every weight on every use, twice per step and layer otherwise. The
-    result must not be kept across optimizer steps: it is overwritten when the parameter changes."""
-    if t.dtype == dtype and not transpose:
+def cast_cached(t, dtype, layout="plain"):
+    """The parameter t in dtype -- as it is ("plain"), transposed, or as the mirrored convolution weight of the
+    input gradient (see _cast_shape) -- remembered until the parameter is written to or moved: training would
+    otherwise cast every weight on every use, twice per step and layer. fp32 masters on the GPU are converted by
+    ptv3_cast_params, all stale copies in one launch. The result must not be kept across optimizer steps: it is
+    overwritten in place when the parameter changes."""
+    if t.dtype == dtype and layout == "plain":
         return t
-    key = (id(t), dtype, transpose)
-    stamp = (t.data_ptr(), t._version)
-    hit = _CAST_CACHE.get(key)
-    if hit is not None and hit[2]() is t:
-        if hit[0] != stamp and not transpose:
-            _refresh_stale_casts(dtype)
-            hit = _CAST_CACHE.get(key)
-        if hit[0] == stamp:
-            return hit[1]
-    with torch.no_grad():
-        out = (t.detach().t() if transpose else t.detach()).to(dtype).contiguous()
-    import weakref
-    ref = weakref.ref(t, lambda _r, k=key: _CAST_CACHE.pop(k, None))
-    _CAST_CACHE[key] = (stamp, out, ref)
-    return out
+    if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and dtype in _DTYPE_CODE):
+        with torch.no_grad():   # half-precision masters, CPU tensors: not worth remembering
+            src = t.detach()
+            if layout == "transpose":
+                src = src.t()
+            elif layout == "mirror":
+                src = src.reshape(t.shape[0], -1, t.shape[-1]).flip(1).permute(2, 1, 0)
+            return src.to(dtype).contiguous()
+    key = (id(t), dtype, layout)
+    entry = _CAST_CACHE.get(key)
+    shape, out_shape = _cast_shape(t, layout)
+    if entry is None or entry.ref() is not t or entry.shape != shape or entry.out.device != t.device:
+        import weakref
+        entry = _Cast()
+        entry.stamp, entry.shape, entry.mirror = None, shape, int(layout != "plain")
+        entry.out = torch.empty(out_shape, dtype=dtype, device=t.device)
+        entry.ref = weakref.ref(t, lambda _r, k=key: _CAST_CACHE.pop(k, None))
+        _CAST_CACHE[key] = entry
+    if entry.stamp != (t.data_ptr(), t._version):
+        _refresh_stale_casts(dtype, t.device)
+    return entry.out
 
 
 class Readback:
@@ -945,6 +977,50 @@ def linear(x, mod, gelu=False):
         return linear_rows(x, mod.weight, mod.bias, gelu)
     y = torch.nn.functional.linear(x, mod.weight, mod.bias)
     return torch.nn.functional.gelu(y) if gelu else y
+
+
+def linear_gelu(x, weight, bias=None):
+    """(pre, gelu(pre)) with pre = x W^T + b from one pass over the rows (ptv3_linear_gelu_fwd): the training
+    form of fc1 + act, which keeps the GELU's input for the backward."""
+    _dev(x, weight, bias)
+    x = x.contiguous()
+    n, k = x.shape
+    w = weight.to(x.dtype).contiguous()
+    b = None if bias is None else bias.to(x.dtype).contiguous()
+    pre = torch.empty((n, w.shape[0]), dtype=x.dtype, device=x.device)
+    out = torch.empty_like(pre)
+    _lib.check(_lib.load().ptv3_linear_gelu_fwd(_ptr(x), _ptr(w), _ptr(b), _dtype_code(x), n, k, w.shape[0], _ptr(pre),
+                                                _ptr(out), _stream()), "ptv3_linear_gelu_fwd")
+    return pre, out
+
+
+def linear_gelu_bwd(dout, weight_t, pre):
+    """(dout weight_t^T) * gelu'(pre): the gradient of fc2's output taken back to the GELU's input in one pass
+    (ptv3_linear_gelu_bwd). weight_t (hidden, out) is fc2's weight transposed."""
+    _dev(dout, weight_t, pre)
+    dout, pre = dout.contiguous(), pre.contiguous()
+    n, k = dout.shape
+    w = weight_t.to(dout.dtype).contiguous()
+    if pre.shape != (n, w.shape[0]) or pre.dtype != dout.dtype:
+        raise _lib.Ptv3Error("linear_gelu_bwd: pre must be (rows, hidden) in dout's dtype")
+    dpre = torch.empty_like(pre)
+    _lib.check(_lib.load().ptv3_linear_gelu_bwd(_ptr(dout), _ptr(w), _ptr(pre), _dtype_code(dout), n, k, w.shape[0],
+                                                _ptr(dpre), _stream()), "ptv3_linear_gelu_bwd")
+    return dpre
+
+
+def mlp(x, fc1, fc2):
+    """fc2(gelu(fc1(x))) for two nn.Linear under autograd: the GELU rides on fc1's kernel going forward and on
+    fc2's input gradient going back. None where the fused form does not apply (the caller takes the modules
+    one by one)."""
+    xa = x.to(torch.get_autocast_dtype("cuda")) if (torch.is_autocast_enabled() and x.is_cuda) else x
+    if not (xa.is_cuda and xa.dim() == 2 and xa.dtype in (torch.float16, torch.bfloat16)
+            and fc1.weight.dtype in (torch.float32, xa.dtype) and fc2.weight.dtype == fc1.weight.dtype
+            and linear_rows_ok(xa, fc1.weight) and fc2.weight.shape[0] % 32 == 0
+            and fc2.weight.shape[0] in (32, 64, 128, 256, 512)):
+        return None
+    from .autograd import Mlp
+    return Mlp.apply(xa, fc1.weight, fc1.bias, fc2.weight, fc2.bias)
 
 
 def linear_rows(x, weight, bias=None, gelu=False):

@@ -472,3 +472,97 @@ def test_training_on_the_output_of_grid_sample():
         out = model({k: batch[k] for k in ("feat", "grid_coord", "coord", "offset")}).feat
     out.float().square().mean().backward()
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in model.parameters())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_parameter_casts_in_one_launch(dtype):
+    """ptv3_cast_params behind ops.cast_cached: plain, transposed and mirrored copies of fp32 masters equal
+    torch's own conversion bit for bit, follow in-place updates (all stale copies in one sweep, written in
+    place) and a replaced storage, for shapes that are not multiples of the tile or the vector width."""
+    o = ops()
+    g = torch.Generator().manual_seed(11)
+    shapes = [(96, 32), (13, 64), (64, 27, 64), (32, 5, 5, 5, 6), (70, 3, 130), (1, 7), (4099,)]
+    params = [torch.nn.Parameter(torch.randn(*s, generator=g).to(DEV)) for s in shapes]
+
+    def want(p, layout):
+        src = p.detach()
+        if layout == "transpose":
+            src = src.t()
+        elif layout == "mirror":
+            src = src.reshape(p.shape[0], -1, p.shape[-1]).flip(1).permute(2, 1, 0)
+        return src.to(dtype).contiguous()
+
+    def layouts(p):
+        return ["plain"] + (["transpose"] if p.dim() == 2 else []) + (["mirror"] if p.dim() >= 2 else [])
+
+    held = {}
+    for i, p in enumerate(params):
+        for layout in layouts(p):
+            got = o.cast_cached(p, dtype, layout)
+            if dtype == torch.float32 and layout == "plain":
+                assert got is p
+                continue
+            assert got.dtype == dtype and got.is_contiguous() and torch.equal(got, want(p, layout)), (i, layout)
+            assert o.cast_cached(p, dtype, layout) is got
+            held[(i, layout)] = got
+    with torch.no_grad():
+        for p in params:
+            p.mul_(1.5).add_(0.25)
+    first = next(iter(held))
+    o.cast_cached(params[first[0]], dtype, first[1])            # one call refreshes every stale copy ...
+    for (i, layout), got in held.items():
+        assert torch.equal(got, want(params[i], layout)), (i, layout)   # ... in place
+        assert o.cast_cached(params[i], dtype, layout) is got
+    params[2].data = torch.randn(64, 27, 64, generator=g).to(DEV)
+    assert torch.equal(o.cast_cached(params[2], dtype, "mirror"), want(params[2], "mirror"))
+    odd = torch.nn.Parameter(torch.randn(1001, generator=g).to(DEV)[1:])   # storage offset: 4-byte alignment only
+    if dtype != torch.float32:
+        assert torch.equal(o.cast_cached(odd, dtype), odd.detach().to(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n,c", [(1000, 32), (777, 64), (2048, 128), (300, 256), (129, 512), (1, 64)])
+def test_mlp_function_parity(dtype, n, c):
+    """The MLP under autograd with the GELU taken into fc1's kernel (forward) and into fc2's input gradient
+    (backward), model.py:493-516: output, input gradient and the four parameter gradients vs torch autograd over
+    the same fp32 masters in float64."""
+    from pointtransformerv3_amd.modules import MLP
+    torch.manual_seed(n + c)
+    mlp = MLP(c, 4 * c, c).to(DEV)
+    x = torch.randn(n, c, device=DEV, dtype=dtype, requires_grad=True)
+    dy = torch.randn(n, c, device=DEV, dtype=dtype)
+    with torch.autocast("cuda", dtype=dtype):
+        y = mlp(x)
+    assert y.dtype == dtype and "Mlp" in type(y.grad_fn).__name__
+    y.backward(dy)
+
+    ref = MLP(c, 4 * c, c).double()
+    ref.load_state_dict({k: v.double().cpu() for k, v in mlp.state_dict().items()})
+    xr = x.detach().double().cpu().requires_grad_(True)
+    h = torch.nn.functional.linear(xr, ref.fc1.weight, ref.fc1.bias)
+    yr = torch.nn.functional.linear(torch.nn.functional.gelu(h), ref.fc2.weight, ref.fc2.bias)
+    yr.backward(dy.double().cpu())
+    assert rel_err(y, yr) < TOL[dtype]
+    assert rel_err(x.grad, xr.grad) < TOL[dtype]
+    for name, p in mlp.named_parameters():
+        assert rel_err(p.grad, dict(ref.named_parameters())[name].grad) < TOL[dtype], name
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_linear_gelu_kernels_against_their_parts(dtype):
+    """ptv3_linear_gelu_fwd writes the same rows as the plain kernel followed by torch's GELU of them, and
+    ptv3_linear_gelu_bwd the product of the plain kernel's rows with gelu'(pre), to one rounding."""
+    o = ops()
+    torch.manual_seed(5)
+    for n, k, nout in [(5000, 64, 256), (333, 256, 1024), (64, 512, 2048), (31, 32, 128)]:
+        x = torch.randn(n, k, device=DEV, dtype=dtype)
+        w = (torch.randn(nout, k, device=DEV) / k ** 0.5).to(dtype)
+        b = torch.randn(nout, device=DEV).to(dtype)
+        pre, act = o.linear_gelu(x, w, b)
+        plain = o.linear_rows(x, w, b)
+        assert torch.equal(pre, plain)
+        assert rel_err(act, torch.nn.functional.gelu(plain.float()).cpu()) < 4e-3
+        d = o.linear_gelu_bwd(x, w, pre)
+        z = pre.double().requires_grad_(True)
+        torch.nn.functional.gelu(z).backward(o.linear_rows(x, w).double())
+        assert rel_err(d, z.grad.cpu()) < 4e-3

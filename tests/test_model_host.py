@@ -103,26 +103,16 @@ def test_forward_on_cpu_tensors_fails_loudly():
         m(data)
 
 
-def test_cast_cache_follows_in_place_updates_and_replacement():
-    """Weights are cast once per update, not once per use: the remembered copy must follow the parameter when
-    it is written in place (an optimizer step: all stale copies are redone together) or its storage is replaced."""
+def test_cast_of_cpu_parameters_is_computed_not_remembered():
+    """Off the GPU a parameter is converted on every call (there is nothing to launch for it): the layouts are
+    the ones the GPU kernel writes."""
     import torch
     from pointtransformerv3_amd import ops
-    p = torch.nn.Parameter(torch.arange(6, dtype=torch.float32).reshape(2, 3))
-    a = ops.cast_cached(p, torch.bfloat16)
-    assert a.dtype == torch.bfloat16 and ops.cast_cached(p, torch.bfloat16) is a
-    t = ops.cast_cached(p, torch.bfloat16, transpose=True)
-    assert t.shape == (3, 2) and t.is_contiguous() and torch.equal(t, a.t())
-    with torch.no_grad():
-        p.add_(1.0)
-    q = torch.nn.Parameter(torch.ones(4))
-    qa = ops.cast_cached(q, torch.bfloat16)
-    with torch.no_grad():
-        q.mul_(3.0)
-    b = ops.cast_cached(p, torch.bfloat16)
-    assert torch.equal(b.float(), p.detach())
-    assert torch.equal(qa.float(), q.detach())          # redone in the same sweep, in place
-    assert torch.equal(ops.cast_cached(p, torch.bfloat16, transpose=True).float(), p.detach().t())
-    p.data = torch.zeros(2, 3)
-    assert torch.equal(ops.cast_cached(p, torch.bfloat16).float(), torch.zeros(2, 3))
+    p = torch.nn.Parameter(torch.arange(24, dtype=torch.float32).reshape(2, 4, 3))
     assert ops.cast_cached(p, torch.float32) is p
+    assert torch.equal(ops.cast_cached(p, torch.bfloat16).float(), p.detach())
+    m = ops.cast_cached(p, torch.bfloat16, "mirror")
+    assert m.shape == (3, 4, 2) and m.is_contiguous()
+    assert all(float(m[k, 3 - j, i]) == float(p[i, j, k]) for i in range(2) for j in range(4) for k in range(3))
+    w = torch.nn.Parameter(torch.arange(6, dtype=torch.float32).reshape(2, 3))
+    assert torch.equal(ops.cast_cached(w, torch.float16, "transpose").float(), w.detach().t())
