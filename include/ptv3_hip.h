@@ -353,6 +353,13 @@ int ptv3_add_layer_norm_bwd(const void *sum, int sum_dtype, const void *dy, int 
                             int param_dtype, int64_t n, int c, float eps, void *dskip, int dskip_dtype,
                             void *dbranch, int dbranch_dtype, float *dgamma, float *dbeta, void *stream);
 
+/* A residual connection with no LayerNorm behind it (model.py:602-604, the end of a Block, with the
+ * stochastic-depth factor of model.py:583): out = skip + branch * row_scale, rows (n,c), c a multiple of 8, each
+ * tensor in its own dtype. skip and row_scale (n,) may be NULL: with skip NULL this is the gradient of the
+ * branch, dbranch = dout * row_scale, or a plain conversion. */
+int ptv3_scaled_add(const void *skip, int skip_dtype, const void *branch, int branch_dtype, const void *row_scale,
+                    int row_scale_dtype, int64_t n, int c, void *out, int out_dtype, void *stream);
+
 /* nn.BatchNorm1d in training mode (model.py:848; call sites :776-779, :707-710, :729-735), first half: the
  * batch statistics of x (n,c), c in {32, 64, 128, 256, 512}. stats (3,c) fp32 receives mean, rsqrt(var + eps)
  * and the biased variance; running_mean / running_var (c,) fp32, when given, are updated in place with

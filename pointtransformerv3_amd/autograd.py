@@ -204,6 +204,24 @@ class AddLayerNorm(torch.autograd.Function):
         return dskip, dbranch, None, dw.to(weight.dtype), db.to(bias_dtype), None, None
 
 
+class ResidualAdd(torch.autograd.Function):
+    """skip + branch * mask (model.py:602-604 with the stochastic-depth factor per row) in skip's dtype, the
+    branch read in its own; going back skip's gradient is the incoming one as it is and the branch's one
+    kernel, instead of autocast's conversions around an addcmul."""
+
+    @staticmethod
+    def forward(ctx, skip, branch, mask):
+        ctx.save_for_backward(mask)
+        ctx.branch_dtype = branch.dtype
+        return ops.scaled_add(skip, branch, mask, skip.dtype)
+
+    @staticmethod
+    def backward(ctx, dout):
+        (mask,) = ctx.saved_tensors
+        dbranch = ops.scaled_add(None, dout, mask, ctx.branch_dtype) if ctx.needs_input_grad[1] else None
+        return (dout if ctx.needs_input_grad[0] else None), dbranch, None
+
+
 class BatchNormAct(torch.autograd.Function):
     """nn.BatchNorm1d (batch statistics and running-average update in training mode, the running statistics
     otherwise), optionally followed by exact GELU (model.py:776-779, :707-710, :729-735), as one node: the

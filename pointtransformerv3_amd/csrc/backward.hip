@@ -746,6 +746,32 @@ int launch_add_ln_bwd(AnyRows sum, AnyRows dy, AnyRows dsum, AnyRows row_scale, 
     return PTV3_ESHAPE;
 }
 
+// out = skip + branch * row_scale without a LayerNorm behind it: the last residual connection of a Block
+// (model.py:602-604) going forward, and with skip absent the gradient of its branch going back
+// (dbranch = dout * row_scale), each tensor in its own dtype. 8 channels per thread; c is a multiple of 8.
+__global__ __launch_bounds__(256) void scaled_add_kernel(AnyRows skip, AnyRows branch, AnyRows row_scale, int64_t n, int c,
+                                                         AnyRowsOut out) {
+    const int64_t groups = n * (c / 8);
+    for (int64_t gi = (int64_t)blockIdx.x * 256 + threadIdx.x; gi < groups; gi += (int64_t)gridDim.x * 256) {
+        const int64_t off = gi * 8;
+        const Raw8 rb = raw8_load(branch.p, branch.dtype, off);
+        Raw8 rs = rb;
+        if (skip.p) rs = raw8_load(skip.p, skip.dtype, off);
+        const float m = row_scale.p ? load1_any(row_scale.p, row_scale.dtype, off / c) : 1.f;
+        float xv[8];
+        raw8_floats(rb, branch.dtype, xv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) xv[i] *= m;
+        if (skip.p) {
+            float sv[8];
+            raw8_floats(rs, skip.dtype, sv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) xv[i] += sv[i];
+        }
+        store8_any(out.p, out.dtype, off, xv);
+    }
+}
+
 // ---- BatchNorm1d in training mode (+ exact GELU)
 __device__ __forceinline__ float gelu_grad(float z) {
     const float cdf = 0.5f * (1.f + erff(z * 0.70710678118654752f));
@@ -1095,6 +1121,23 @@ extern "C" int ptv3_add_layer_norm_fwd(const void* skip, int skip_dtype, const v
     return launch_add_ln_fwd({skip, skip_dtype}, {branch, branch_dtype}, {row_scale, row_scale_dtype},
                              {gamma, param_dtype}, {beta, param_dtype}, n, c, eps, {sum, sum_dtype}, {y, y_dtype},
                              (hipStream_t)stream_);
+}
+
+extern "C" int ptv3_scaled_add(const void* skip, int skip_dtype, const void* branch, int branch_dtype,
+                               const void* row_scale, int row_scale_dtype, int64_t n, int c, void* out, int out_dtype,
+                               void* stream_) {
+    if (n < 0 || c < 1) return PTV3_EINVAL;
+    if (!ln_dtype_ok(skip_dtype) || !ln_dtype_ok(branch_dtype) || !ln_dtype_ok(row_scale_dtype) || !ln_dtype_ok(out_dtype))
+        return PTV3_EINVAL;
+    if (c % 8 != 0) return PTV3_ESHAPE;
+    if (n == 0) return PTV3_OK;
+    if (!branch || !out) return PTV3_EINVAL;
+    const int64_t groups = n * (c / 8);
+    const int64_t blocks = ptv3_ceil_div(groups, 256);
+    hipLaunchKernelGGL(scaled_add_kernel, dim3((unsigned)(blocks < 8192 ? blocks : 8192)), dim3(256), 0,
+                       (hipStream_t)stream_, AnyRows{skip, skip_dtype}, AnyRows{branch, branch_dtype},
+                       AnyRows{row_scale, row_scale_dtype}, n, c, AnyRowsOut{out, out_dtype});
+    PTV3_RETURN_LAUNCH();
 }
 
 extern "C" int ptv3_add_layer_norm_bwd(const void* sum, int sum_dtype, const void* dy, int dy_dtype, const void* dsum,

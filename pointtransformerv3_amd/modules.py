@@ -11,7 +11,7 @@ import torch
 import torch.nn as nn
 
 from . import ops
-from .autograd import AddLayerNorm, BatchNormAct, LayerNorm as LayerNormFn, SegmentReduce, UnpoolAdd
+from .autograd import AddLayerNorm, BatchNormAct, LayerNorm as LayerNormFn, ResidualAdd, SegmentReduce, UnpoolAdd
 from .point import AttrDict, Point, offset2bincount
 from .sparse import SparseConvTensor, SubMConv3d, is_spconv_module
 
@@ -444,7 +444,12 @@ class Block(PointModule):
                                               normed_dtype)
         point = self.mlp(point)
         mask = path_mask(point.feat)
-        point.feat = feat + point.feat if mask is None else torch.addcmul(feat, point.feat, mask)
+        if mask is None:
+            point.feat = feat + point.feat
+        elif self.channels % 8 == 0 and all(t.dtype in ops.DTYPE_CODES for t in (feat, point.feat, mask)):
+            point.feat = ResidualAdd.apply(feat, point.feat, mask)
+        else:
+            point.feat = torch.addcmul(feat, point.feat, mask)
         point.sparse_conv_feat = point.sparse_conv_feat.replace_feature(point.feat)
         return point
 

@@ -12,6 +12,7 @@ from . import _lib
 
 ORDER_IDS = {"z": 0, "z-trans": 1, "hilbert": 2, "hilbert-trans": 3}
 _DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+DTYPE_CODES = _DTYPE_CODE   # the dtypes the mixed-dtype row kernels read and write
 REDUCE_OPS = {"max": 0, "mean": 1, "sum": 2, "min": 3}
 
 
@@ -885,6 +886,21 @@ def add_layer_norm(skip, branch, row_scale, weight, bias, eps, sum_dtype=None, o
                                            _DTYPE_CODE[sum_dtype], _ptr(y), _DTYPE_CODE[out_dtype], _stream()),
                "ptv3_add_layer_norm_fwd")
     return total, y
+
+
+def scaled_add(skip, branch, row_scale, out_dtype):
+    """skip + branch * row_scale in out_dtype, each input read in its own dtype (ptv3_scaled_add); skip and
+    row_scale (N,) or (N, 1) may be None."""
+    _dev(skip, branch, row_scale)
+    branch = branch.contiguous()
+    n, c = branch.shape
+    skip = None if skip is None else skip.contiguous()
+    row_scale = None if row_scale is None else row_scale.reshape(-1).contiguous()
+    out = torch.empty((n, c), dtype=out_dtype, device=branch.device)
+    _lib.check(_lib.load().ptv3_scaled_add(_ptr(skip), _code(skip), _ptr(branch), _code(branch), _ptr(row_scale),
+                                           _code(row_scale), n, c, _ptr(out), _DTYPE_CODE[out_dtype], _stream()),
+               "ptv3_scaled_add")
+    return out
 
 
 def add_layer_norm_bwd(total, dy, dsum, row_scale, weight, eps, skip_dtype=None, branch_dtype=None):

@@ -566,3 +566,26 @@ def test_linear_gelu_kernels_against_their_parts(dtype):
         z = pre.double().requires_grad_(True)
         torch.nn.functional.gelu(z).backward(o.linear_rows(x, w).double())
         assert rel_err(d, z.grad.cpu()) < 4e-3
+
+
+@pytest.mark.parametrize("skip_dtype,branch_dtype", [(torch.float32, torch.bfloat16), (torch.float32, torch.float16),
+                                                     (torch.float32, torch.float32), (torch.float16, torch.float16)])
+@pytest.mark.parametrize("n,c", [(1000, 32), (77, 512), (1, 8), (4099, 64)])
+def test_residual_add_function(skip_dtype, branch_dtype, n, c):
+    """ptv3_scaled_add behind ResidualAdd: skip + branch * mask (model.py:602-604 with model.py:583's factor)
+    and its two gradients vs torch in float64."""
+    from pointtransformerv3_amd.autograd import ResidualAdd
+    g = torch.Generator().manual_seed(n * c)
+    skip = torch.randn(n, c, generator=g).to(skip_dtype).to(DEV).requires_grad_(True)
+    branch = torch.randn(n, c, generator=g).to(branch_dtype).to(DEV).requires_grad_(True)
+    mask = (torch.bernoulli(torch.full((n, 1), 0.7), generator=g) / 0.7).to(branch_dtype).to(DEV)
+    dout = torch.randn(n, c, generator=g).to(skip_dtype).to(DEV)
+    out = ResidualAdd.apply(skip, branch, mask)
+    out.backward(dout)
+    assert out.dtype == skip_dtype and skip.grad.dtype == skip_dtype and branch.grad.dtype == branch_dtype
+    want = skip.detach().double() + branch.detach().double() * mask.double()
+    tol = 1e-6 if skip_dtype == torch.float32 else 1e-3
+    assert rel_err(out, want.cpu()) < tol
+    assert torch.equal(skip.grad, dout)
+    tol = 1e-6 if branch_dtype == torch.float32 else (1e-3 if branch_dtype == torch.float16 else 4e-3)
+    assert rel_err(branch.grad, (dout.double() * mask.double()).cpu()) < tol
