@@ -112,6 +112,29 @@ __global__ __launch_bounds__(256) void conv_wgrad_kernel(const T* __restrict__ x
 // step: 16-byte pieces of the two operands are written transposed into the wave's LDS tiles (rows of
 // OR_S halves, 16-byte chunks swizzled by the channel group so that the writes spread over the banks),
 // then read back as MFMA operands.
+constexpr int XCDS = 8;   // work-groups of a launch go to the XCDs round-robin; each XCD has an L2 of its own
+
+// Which (tap, range of rows, block of the result) this work-group takes. All blocks of one range read the same
+// rows, so they should meet in one L2: item j of the order (tap, range, block) goes to XCD j / per_xcd, and within
+// it to the j % per_xcd-th work-group that lands there. Every XCD gets the same number of items, whatever the
+// number of ranges; the grid is per_xcd * XCDS work-groups and the ones past the last item leave.
+template <int SIDE>
+__device__ __forceinline__ bool outer_item(int taps, int splits, int m_total, int k_total, int* tap, int* split, int* m0,
+                                           int* k0) {
+    const int bm = (m_total + SIDE - 1) / SIDE, bk = (k_total + SIDE - 1) / SIDE;
+    const int64_t total = (int64_t)taps * splits * bm * bk;
+    const int64_t per_xcd = (total + XCDS - 1) / XCDS;
+    const int64_t j = (int64_t)(blockIdx.x % XCDS) * per_xcd + blockIdx.x / XCDS;
+    if (blockIdx.x / XCDS >= per_xcd || j >= total) return false;
+    const int64_t x = j / (bm * bk);
+    const int blk = (int)(j % (bm * bk));
+    *tap = (int)(x / splits);
+    *split = (int)(x % splits);
+    *m0 = (blk % bm) * SIDE;
+    *k0 = (blk / bm) * SIDE;
+    return true;
+}
+
 constexpr int OR_S = 40;      // halves per LDS row: 32 summed rows + padding that spreads the operand reads
 constexpr int OR_C = 64;      // channels per block side
 constexpr int OR_LIST = 4096; // most rows per work-group with GATHER (the compacted pair list lives in LDS)
@@ -152,8 +175,8 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
     __shared__ __align__(16) uint16_t tiles[4][2][OR_C * OR_S];
     __shared__ int32_t list_a[GATHER ? OR_LIST : 1], list_b[GATHER ? OR_LIST : 1];
     __shared__ int list_n;
-    const int tap = blockIdx.x / splits, split = blockIdx.x % splits;
-    const int m0 = blockIdx.y * OR_C, k0 = blockIdx.z * OR_C;
+    int tap, split, m0, k0;
+    if (!outer_item<OR_C>(taps, splits, m_total, k_total, &tap, &split, &m0, &k0)) return;
     const int tm = min(2, (m_total - m0 + 31) / 32), tk = min(2, (k_total - k0 + 31) / 32);
     const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
     const int64_t r0 = (int64_t)split * rows_per_split;
@@ -194,7 +217,7 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
     const int col = lane & 31, hf = lane >> 5;
     // column sums of a (the bias gradient) ride along in the blocks that read each of a's rows exactly once:
     // the first block along k, and with GATHER the centre tap, whose pairs are (i, i) for every voxel
-    const bool sum_cols = colsum != nullptr && blockIdx.z == 0 && (!GATHER || tap == taps / 2);
+    const bool sum_cols = colsum != nullptr && k0 == 0 && (!GATHER || tap == taps / 2);
     float cs[8];
 #pragma unroll
     for (int c = 0; c < 8; ++c) cs[c] = 0.f;
@@ -307,8 +330,8 @@ __global__ __launch_bounds__(256) void outer_rows_wide_kernel(const T* __restric
     __shared__ int32_t list_a[GATHER ? OR_LIST : 1], list_b[GATHER ? OR_LIST : 1];
     __shared__ int list_n;
     __shared__ float wave_cols[2][OW_C];
-    const int tap = blockIdx.x / splits, split = blockIdx.x % splits;
-    const int m0 = blockIdx.y * OW_C, k0 = blockIdx.z * OW_C;
+    int tap, split, m0, k0;
+    if (!outer_item<OW_C>(taps, splits, m_total, k_total, &tap, &split, &m0, &k0)) return;
     const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
     const int64_t r0 = (int64_t)split * rows_per_split;
     const int64_t r1 = min(n, r0 + rows_per_split);
@@ -347,7 +370,7 @@ __global__ __launch_bounds__(256) void outer_rows_wide_kernel(const T* __restric
     const T* src_ptr = is_b ? b : a;
     const int width = is_b ? k_total : m_total, c0 = (is_b ? k0 : m0) + 8 * g;
     const bool in_range = c0 < width;
-    const bool sum_cols = colsum != nullptr && blockIdx.z == 0 && (!GATHER || tap == taps / 2);
+    const bool sum_cols = colsum != nullptr && k0 == 0 && (!GATHER || tap == taps / 2);
     float cs[8];
 #pragma unroll
     for (int c = 0; c < 8; ++c) cs[c] = 0.f;
@@ -965,14 +988,37 @@ __global__ __launch_bounds__(256) void segment_reduce_bwd_kernel(const T* __rest
     }
 }
 
-// Rows of the reduction per work-group: enough work-groups to fill the part, but at least 1024 rows each so
-// that the block a work-group hands in is small next to what it read.
+int outer_cu_count() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v < 1)
+            v = 256;
+        cus = v;
+    }
+    return cus;
+}
+
+// Rows of the reduction per work-group. Two work-groups fit a CU, and they all start together: the launch takes
+// as long as the CU with the most of them, so a count just above a multiple of 2 x CUs costs a whole round more
+// (measured: 516 work-groups 55 us, 444 of the same layer 45 us). The number of ranges minimises
+// rounds x (rows per range + what a work-group costs apart from its rows: its block of the result written and
+// read again by the sum over ranges, about 384 rows' worth).
 void outer_split(int64_t n, int64_t blocks_per_split, int64_t cap, int64_t* splits, int64_t* rows) {
-    int64_t sp = ptv3_ceil_div(1024, blocks_per_split);
-    const int64_t most = ptv3_ceil_div(n, 1024);
-    if (sp > most) sp = most;
-    if (sp < 1) sp = 1;
-    int64_t r = ptv3_ceil_div(ptv3_ceil_div(n, sp), 128) * 128;
+    const int64_t slots = 2 * outer_cu_count(), fixed = 384;
+    int64_t lo = cap > 0 ? ptv3_ceil_div(n, cap) : 1;
+    if (lo < 1) lo = 1;
+    int64_t hi = 4 * slots / blocks_per_split;
+    const int64_t most = ptv3_ceil_div(n, 256);
+    if (hi > most) hi = most;
+    if (hi < lo) hi = lo;
+    int64_t best = lo, best_cost = INT64_MAX;
+    for (int64_t s = lo; s <= hi; ++s) {
+        const int64_t cost = ptv3_ceil_div(blocks_per_split * s, slots) * (ptv3_ceil_div(n, s) + fixed);
+        if (cost < best_cost) { best_cost = cost; best = s; }
+    }
+    int64_t r = ptv3_ceil_div(ptv3_ceil_div(n, best), 128) * 128;
     if (cap > 0 && r > cap) r = cap;
     *rows = r;
     *splits = ptv3_ceil_div(n, r);
@@ -1004,7 +1050,9 @@ int launch_outer(const void* a, const void* b, int64_t n, int m_total, int k_tot
     if (splits > 1 && (!workspace || workspace_bytes < (size_t)splits * stride * sizeof(float))) return PTV3_EWORKSPACE;
     float* slabs = splits > 1 ? (float*)workspace : d;
     float* cols = !colsum ? nullptr : (splits > 1 ? slabs + count : colsum);
-    const dim3 grid((unsigned)(taps * splits), (unsigned)bm, (unsigned)bk);
+    const int64_t items = (int64_t)taps * splits * bm * bk;
+    if (items >= (1ll << 31) - XCDS) return PTV3_EINVAL;
+    const dim3 grid((unsigned)(ptv3_ceil_div(items, XCDS) * XCDS));   // see outer_item
     if (side == OW_C)
         hipLaunchKernelGGL((outer_rows_wide_kernel<T, GATHER>), grid, dim3(256), 0, stream, (const T*)a, (const T*)b, n,
                            m_total, k_total, nbr, taps, (int)splits, rows, stride, slabs, cols);
