@@ -35,14 +35,6 @@ namespace {
 // accumulators are rescaled: probabilities then stay below 2^8, safe for fp16 operands.
 constexpr float RESCALE_SLACK = 8.f;
 
-// Work-group id -> (sequence, head) such that the heads of one sequence, which share cache
-// lines of the qkv rows, run on the same XCD (work-groups are dealt round-robin to 8 XCDs).
-__device__ __forceinline__ int xcd_chunked_id(int bid, int total) {
-    const int xcd = bid & 7, slot = bid >> 3;
-    const int per = total >> 3, rem = total & 7;
-    return xcd * per + min(xcd, rem) + slot;
-}
-
 // One 32-query tile of one wave against every key of the sequence in LDS.
 // SHIFT = false: the caller has checked that no score can leave [-limit, limit] (|q||k| bound),
 // so probabilities 2^score are representable as they are, the MFMA's C operand is the constant

@@ -89,7 +89,7 @@ __device__ __forceinline__ f32x16 splat16(float x) {
 // work-group each, so that the round is short (every range stages the sequence again).
 __device__ __forceinline__ void item_of_block(int full_items, int split, int* item, int* part, int* parts) {
     if ((int)blockIdx.x < full_items) {
-        *item = blockIdx.x;
+        *item = xcd_chunked_id(blockIdx.x, full_items);   // heads that share cache lines meet in one L2
         *part = 0;
         *parts = 1;
     } else {

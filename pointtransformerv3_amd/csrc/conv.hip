@@ -403,7 +403,10 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void pair_gemm_kernel(
         int32_t slot[MT][4];      // y rows of the pairs this lane stores in the epilogue, -1 past the end
         int cout0;
     };
-    auto setup = [&](int g, Tile& tl) {
+    auto setup = [&](int g_launch, Tile& tl) {
+        // the column tiles of one row tile gather the same rows: same XCD (the grid is a multiple of 8 or a
+        // single round), one after the other
+        const int g = xcd_chunked_id(g_launch, total);
         const int rid = g / col_tiles;
         tl.cout0 = (g % col_tiles) * COUT_TILE;
         int tap = 0, pstart = 0, pcount = 1;

@@ -40,7 +40,7 @@ enum { ACT_NONE = 0, ACT_GELU = 1, ACT_GELU_KEEP = 2, ACT_GELU_GRAD = 3 };
 template <typename T, int K, int ACT, bool BN, int NW, int SW>
 __global__ __launch_bounds__(NW * PTV3_WAVE, (NW == 8 ? 2 : 1)) void linear_rows_kernel(
     const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ bias, LinBn bn, int64_t n, int nout,
-    int chunk, T* __restrict__ out, T* __restrict__ aux) {
+    int chunk, int per_chunk, int n_chunks, T* __restrict__ out, T* __restrict__ aux) {
     typedef typename H16<T>::v8 v8;
     constexpr int KS = K / 16, WS = K + LIN_PAD, LIN_THREADS = NW * PTV3_WAVE, LIN_WAVES = NW, LIN_XSS = SW + LIN_PAD;
     extern __shared__ __align__(16) unsigned char lin_smem[];
@@ -51,10 +51,25 @@ __global__ __launch_bounds__(NW * PTV3_WAVE, (NW == 8 ? 2 : 1)) void linear_rows
     float* be_lds = sc_lds + (BN ? chunk : 0);
     T* xs_all = (T*)(be_lds + (BN ? chunk : 0));           // [waves][32][LIN_XSS]
 
+    // Work-groups go to the 8 XCDs round-robin and every XCD has its own L2: the n_chunks work-groups that walk
+    // the same rows (one per chunk of output channels) are dealt to one XCD, next to each other, so the rows
+    // leave HBM once. The walks themselves stay interleaved over the XCDs in launch order (with one chunk this
+    // is the plain order; handing each XCD a contiguous eighth of the rows measured 5-20 % slower).
+    // per_chunk < 0: the walks do not spread evenly over 8 XCDs that way; chunk-major launch order instead.
+    int row_group, chunk_id;
+    if (per_chunk > 0) {
+        const int slot = blockIdx.x >> 3;
+        row_group = (slot / n_chunks) * 8 + (blockIdx.x & 7);   // which of the per_chunk walks over the row tiles
+        chunk_id = slot % n_chunks;
+    } else {
+        per_chunk = -per_chunk;
+        row_group = blockIdx.x % per_chunk;
+        chunk_id = blockIdx.x / per_chunk;
+    }
     const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
     const int col = lane & 31, hf = lane >> 5;
     T* xs = xs_all + wave * (32 * LIN_XSS);
-    const int c0 = blockIdx.y * chunk;                     // first output channel of this work-group
+    const int c0 = chunk_id * chunk;                       // first output channel of this work-group
     const int cn = min(chunk, nout - c0);                  // its output channels (a multiple of 32)
 
     // ---- weight chunk and bias -> LDS (rows past cn are never read)
@@ -79,7 +94,7 @@ __global__ __launch_bounds__(NW * PTV3_WAVE, (NW == 8 ? 2 : 1)) void linear_rows
     __syncthreads();
 
     const int64_t n_tiles = (n + 31) / 32;
-    for (int64_t tile = (int64_t)blockIdx.x * LIN_WAVES + wave; tile < n_tiles; tile += (int64_t)gridDim.x * LIN_WAVES) {
+    for (int64_t tile = (int64_t)row_group * LIN_WAVES + wave; tile < n_tiles; tile += (int64_t)per_chunk * LIN_WAVES) {
         const int64_t row0 = tile * 32;
         // ---- 32 rows -> operand fragments, 64 channels at a time: lane (r, piece) moves 16 bytes
         v8 xf[KS];
@@ -219,8 +234,12 @@ int launch_linear_shape(const void* x, const void* w, const void* bias, LinBn bn
     if (per_chunk < 1) per_chunk = 1;
     const int64_t need = (tiles + LIN_WAVES - 1) / LIN_WAVES;
     if (per_chunk > need) per_chunk = need;
-    hipLaunchKernelGGL(kern, dim3((unsigned)per_chunk, (unsigned)n_chunks), dim3(LIN_THREADS), lds, stream, (const T*)x,
-                       (const T*)w, (const T*)bias, bn, n, nout, chunk, (T*)out, (T*)aux);
+    // several chunks and a number of walks that spreads evenly over the XCDs: chunks of a walk on one XCD (see
+    // the kernel); cutting the walks down to a multiple of 8 for the other shapes measured slower than it gained
+    const bool by_xcd = n_chunks > 1 && per_chunk % 8 == 0;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(per_chunk * n_chunks)), dim3(LIN_THREADS), lds, stream, (const T*)x,
+                       (const T*)w, (const T*)bias, bn, n, nout, chunk, (int)(by_xcd ? per_chunk : -per_chunk), n_chunks,
+                       (T*)out, (T*)aux);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? PTV3_OK : (int)e;
 }
