@@ -297,7 +297,7 @@ def training_step(args):
     torch.manual_seed(0)
     model = PointTransformerV3().to(dev).train()
     head = torch.nn.Linear(64, 13).to(dev)
-    opt = torch.optim.AdamW(list(model.parameters()) + list(head.parameters()), lr=1e-3)
+    opt = torch.optim.AdamW(list(model.parameters()) + list(head.parameters()), lr=1e-3, fused=True)
     d, feat = build_inputs(args.scenes, args.points, 4000)
     n_points = len(feat)
     data = dict(feat=torch.from_numpy(feat).to(dev), grid_coord=torch.from_numpy(d["grid_coord"]).to(dev),
@@ -327,7 +327,7 @@ def training_step(args):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": {"bfloat16": "bf16", "float16": "f16"}[args.train],
         "data": "synthetic",
-        "config": {"workload": f"forward + backward + AdamW, default architecture in training mode, autocast, "
+        "config": {"workload": f"forward + backward + fused AdamW, default architecture in training mode, autocast, "
                                f"{args.scenes} room scenes, {n_points} voxelised points, grid 0.02 m"},
         "peak_memory_gib": torch.cuda.max_memory_allocated() / 2 ** 30}))
 

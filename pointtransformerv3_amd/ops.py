@@ -47,6 +47,7 @@ def wants_grad(*tensors):
 
 
 _CAST_CACHE = {}     # (id(parameter), dtype, layout) -> _Cast
+_CAST_EPOCH = [0, False]   # bumped by invalidate_casts(); whether the optimizer hook is in place
 _CAST_TABLES = {}    # (device, dtype) -> (table bytes, device table): optimizer steps ask for the same table again
 _CAST_JOB = np.dtype([("src", "<u8"), ("dst", "<u8"), ("a", "<i4"), ("b", "<i4"), ("c", "<i4"), ("mirror", "<i4"),
                       ("first_block", "<i8")])   # ptv3_cast_job
@@ -67,6 +68,18 @@ def _cast_shape(t, layout):
     return (a, b, c), ((c, a) if layout == "transpose" else (c, b, a))
 
 
+def invalidate_casts():
+    """Declare every remembered parameter copy stale. In-place updates through torch show in the parameter's
+    version counter, which cast_cached checks by itself; fused optimizers (torch.optim.AdamW(fused=True)) write
+    the parameters without touching it, so every optimizer step calls this through a global post-step hook,
+    and so does the model at the start of a training forward. Call it after writing parameters some other way."""
+    _CAST_EPOCH[0] += 1
+
+
+def _cast_stamp(t):
+    return (t.data_ptr(), t._version, _CAST_EPOCH[0])
+
+
 def _refresh_stale_casts(dtype, device):
     """Every remembered copy in dtype whose parameter has been written since (an optimizer step touches all of them
     at once) is redone in place by one launch instead of a few small ones per parameter."""
@@ -75,7 +88,7 @@ def _refresh_stale_casts(dtype, device):
         t = entry.ref()
         if t is None or entry.out.dtype != dtype or t.device != device:
             continue
-        now = (t.data_ptr(), t._version)
+        now = _cast_stamp(t)
         if now != entry.stamp:
             a, b, c = entry.shape
             stale.append((entry, now, (t.data_ptr(), entry.out.data_ptr(), a, b, c, entry.mirror, blocks)))
@@ -110,6 +123,10 @@ def cast_cached(t, dtype, layout="plain"):
             elif layout == "mirror":
                 src = src.reshape(t.shape[0], -1, t.shape[-1]).flip(1).permute(2, 1, 0)
             return src.to(dtype).contiguous()
+    if not _CAST_EPOCH[1]:
+        from torch.optim.optimizer import register_optimizer_step_post_hook
+        register_optimizer_step_post_hook(lambda *_: invalidate_casts())
+        _CAST_EPOCH[1] = True
     key = (id(t), dtype, layout)
     entry = _CAST_CACHE.get(key)
     shape, out_shape = _cast_shape(t, layout)
@@ -120,7 +137,7 @@ def cast_cached(t, dtype, layout="plain"):
         entry.out = torch.empty(out_shape, dtype=dtype, device=t.device)
         entry.ref = weakref.ref(t, lambda _r, k=key: _CAST_CACHE.pop(k, None))
         _CAST_CACHE[key] = entry
-    if entry.stamp != (t.data_ptr(), t._version):
+    if entry.stamp != _cast_stamp(t):
         _refresh_stale_casts(dtype, t.device)
     return entry.out
 

@@ -589,3 +589,23 @@ def test_residual_add_function(skip_dtype, branch_dtype, n, c):
     assert torch.equal(skip.grad, dout)
     tol = 1e-6 if branch_dtype == torch.float32 else (1e-3 if branch_dtype == torch.float16 else 4e-3)
     assert rel_err(branch.grad, (dout.double() * mask.double()).cpu()) < tol
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_parameter_casts_follow_the_optimizer(fused):
+    """torch's fused optimizers write the parameters without touching their version counters: the remembered
+    half-precision copies are declared stale by a hook on every optimizer step (ops.invalidate_casts)."""
+    o = ops()
+    p = torch.nn.Parameter(torch.randn(64, 32, device=DEV))
+    opt = torch.optim.AdamW([p], lr=1e-1, fused=fused)
+    held = o.cast_cached(p, torch.bfloat16)
+    before = held.clone()
+    p.grad = torch.ones_like(p)
+    opt.step()
+    got = o.cast_cached(p, torch.bfloat16)
+    assert got is held and torch.equal(got, p.detach().to(torch.bfloat16)) and not torch.equal(got, before)
+    assert torch.equal(o.cast_cached(p, torch.bfloat16, "transpose"), p.detach().t().to(torch.bfloat16).contiguous())
+    with torch.no_grad():
+        p.data.mul_(2.0)          # behind autograd's back: only an explicit call can tell
+    o.invalidate_casts()
+    assert torch.equal(o.cast_cached(p, torch.bfloat16), p.detach().to(torch.bfloat16))
