@@ -7,6 +7,7 @@ import ctypes
 
 import numpy as np
 import torch
+from torch.optim.optimizer import register_optimizer_step_post_hook as _register_step_hook
 
 from . import _lib
 
@@ -47,7 +48,7 @@ def wants_grad(*tensors):
 
 
 _CAST_CACHE = {}     # (id(parameter), dtype, layout) -> _Cast
-_CAST_EPOCH = [0, False]   # bumped by invalidate_casts(); whether the optimizer hook is in place
+_CAST_EPOCH = [0]    # bumped by invalidate_casts()
 _CAST_TABLES = {}    # (device, dtype) -> (table bytes, device table): optimizer steps ask for the same table again
 _CAST_JOB = np.dtype([("src", "<u8"), ("dst", "<u8"), ("a", "<i4"), ("b", "<i4"), ("c", "<i4"), ("mirror", "<i4"),
                       ("first_block", "<i8")])   # ptv3_cast_job
@@ -76,8 +77,14 @@ def invalidate_casts():
     _CAST_EPOCH[0] += 1
 
 
-def _cast_stamp(t):
+def parameter_stamp(t):
+    """What a derived copy of parameter t remembers to know when it is stale: storage, version counter and the
+    count of invalidate_casts() calls."""
     return (t.data_ptr(), t._version, _CAST_EPOCH[0])
+
+
+_cast_stamp = parameter_stamp
+_register_step_hook(lambda *_: invalidate_casts())
 
 
 def _refresh_stale_casts(dtype, device):
@@ -123,10 +130,6 @@ def cast_cached(t, dtype, layout="plain"):
             elif layout == "mirror":
                 src = src.reshape(t.shape[0], -1, t.shape[-1]).flip(1).permute(2, 1, 0)
             return src.to(dtype).contiguous()
-    if not _CAST_EPOCH[1]:
-        from torch.optim.optimizer import register_optimizer_step_post_hook
-        register_optimizer_step_post_hook(lambda *_: invalidate_casts())
-        _CAST_EPOCH[1] = True
     key = (id(t), dtype, layout)
     entry = _CAST_CACHE.get(key)
     shape, out_shape = _cast_shape(t, layout)

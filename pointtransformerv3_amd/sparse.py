@@ -104,7 +104,7 @@ class SubMConv3d(nn.Module):
     def _packed_weight(self, dtype):
         """The weight in the tile kernel's fragment order, repacked when the parameter changes."""
         w = self.weight
-        key = (w.data_ptr(), w._version, dtype, w.device)
+        key = (ops.parameter_stamp(w), dtype, w.device)   # fused optimizers leave the version counter alone
         cached = getattr(self, "_packed", None)
         if cached is None or cached[0] != key:
             packed = ops.conv_pack_weight(w.detach().reshape(self.out_channels, -1, self.in_channels), 27, dtype)

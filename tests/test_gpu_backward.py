@@ -609,3 +609,19 @@ def test_parameter_casts_follow_the_optimizer(fused):
         p.data.mul_(2.0)          # behind autograd's back: only an explicit call can tell
     o.invalidate_casts()
     assert torch.equal(o.cast_cached(p, torch.bfloat16), p.detach().to(torch.bfloat16))
+
+
+def test_packed_convolution_weight_follows_a_fused_optimizer():
+    """The tile convolution's repacked weight (inference between training epochs) is redone after an optimizer
+    step that leaves the parameter's version counter alone."""
+    from pointtransformerv3_amd.sparse import SubMConv3d
+    o = ops()
+    conv = SubMConv3d(64, 64, kernel_size=3, bias=True, indice_key="k").to(DEV)
+    opt = torch.optim.AdamW(conv.parameters(), lr=1e-1, fused=True)
+    first = conv._packed_weight(torch.float16)
+    assert conv._packed_weight(torch.float16) is first
+    conv.weight.grad = torch.ones_like(conv.weight)
+    opt.step()
+    second = conv._packed_weight(torch.float16)
+    want = o.conv_pack_weight(conv.weight.detach().reshape(64, -1, 64), 27, torch.float16)
+    assert second is not first and torch.equal(second, want) and not torch.equal(second, first)
