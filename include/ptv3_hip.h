@@ -183,6 +183,18 @@ int ptv3_subm_conv_wgrad(const void *feat, const void *dout, int dtype, int64_t 
                          const int32_t *nbr, int taps, float *dweight, float *dbias, void *workspace,
                          size_t workspace_bytes, void *stream);
 
+/* The same weight gradient from the tap-major pair lists the forward pair kernels use (ptv3_conv_plan_*)
+ * instead of the neighbour map: work-groups take ranges of a tap's own pairs, so nothing is compacted and the
+ * ranges are equally long whatever the tap's density. pair_out[q] is the output voxel of pair q
+ * (ptv3_conv_plan_pair_out makes it from the plan's row_ptr and pair_slot); fp16 / bf16 with cin and cout
+ * multiples of 8 only; workspace as ptv3_subm_conv_wgrad_workspace_bytes says. The centre tap must pair every
+ * voxel with itself (true for a submanifold convolution): dbias is summed over its pairs. */
+int ptv3_conv_plan_pair_out(const int32_t *row_ptr, const int32_t *pair_slot, int64_t n, int64_t n_pairs,
+                            int32_t *pair_out, void *stream);
+int ptv3_subm_conv_wgrad_pairs(const void *feat, const void *dout, int dtype, int64_t n, int cin, int cout,
+                               const int32_t *tap_ptr, const int32_t *pair_in, const int32_t *pair_out, int taps,
+                               float *dweight, float *dbias, void *workspace, size_t workspace_bytes, void *stream);
+
 /* Sparse-pair form of the same convolution, for maps where most taps of most voxels are empty
  * (surface scans: 2-13 of 27 taps active). ptv3_conv_plan_count derives from nbr (n,taps) the
  * number of active (input, output) pairs per tap (tap_ptr, taps+1 int32, exclusive) and in total

@@ -79,6 +79,8 @@ SIGNATURES = {
     "ptv3_linear_gelu_fwd": (_i32, [_vp, _vp, _vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp]),
     "ptv3_linear_gelu_bwd": (_i32, [_vp, _vp, _vp, _i32, _i64, _i32, _i32, _vp, _vp]),
     "ptv3_scaled_add": (_i32, [_vp, _i32, _vp, _i32, _vp, _i32, _i64, _i32, _vp, _i32, _vp]),
+    "ptv3_conv_plan_pair_out": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp]),
+    "ptv3_subm_conv_wgrad_pairs": (_i32, [_vp, _vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _sz, _vp]),
     "ptv3_cast_params_blocks": (_i64, [_i32, _i32, _i32, _i32]),
     "ptv3_cast_params": (_i32, [_vp, _i32, _i64, _i32, _vp]),
     "ptv3_linear_wgrad_workspace_bytes": (_sz, [_i64, _i32, _i32]),

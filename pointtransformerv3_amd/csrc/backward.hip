@@ -166,6 +166,8 @@ __device__ __forceinline__ void put_transposed4(uint16_t* tile, int g, int q, co
 template <typename T, bool GATHER>
 __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a, const T* __restrict__ b, int64_t n,
                                                          int m_total, int k_total, const int32_t* __restrict__ nbr,
+                                                         const int32_t* __restrict__ tap_ptr,
+                                                         const int32_t* __restrict__ pair_in,
                                                          int taps, int splits, int64_t rows_per_split,
                                                          int64_t slab_stride, float* __restrict__ d,
                                                          float* __restrict__ colsum) {
@@ -178,10 +180,22 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
     if (!outer_item<OR_C>(taps, splits, m_total, k_total, &tap, &split, &m0, &k0)) return;
     const int tm = min(2, (m_total - m0 + 31) / 32), tk = min(2, (k_total - k0 + 31) / 32);
     const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
-    const int64_t r0 = (int64_t)split * rows_per_split;
+    int64_t r0 = (int64_t)split * rows_per_split;
     const int64_t r1 = min(n, r0 + rows_per_split);
     int count = (int)(r1 - r0);
-    if (GATHER) {
+    if (GATHER && tap_ptr) {
+        // the tap's own list of (output row, input row) pairs, rows_per_split of them per range: nbr holds the
+        // output rows here. Ranges past the end of a short tap's list have nothing to add and hand in zeros.
+        const int64_t p0 = tap_ptr[tap] + (int64_t)split * rows_per_split;
+        const int64_t left = (int64_t)tap_ptr[tap + 1] - p0;
+        count = left < 0 ? 0 : (int)min(left, rows_per_split);
+        for (int e = tid; e < count; e += 256) {
+            list_a[e] = nbr[p0 + e];
+            list_b[e] = pair_in[p0 + e];
+        }
+        r0 = 0;
+        __syncthreads();
+    } else if (GATHER) {
         // compact the voxels of the range that have this neighbour: (output row, input row) pairs
         if (tid == 0) list_n = 0;
         __syncthreads();
@@ -321,6 +335,8 @@ constexpr int OW_C = 128;
 template <typename T, bool GATHER>
 __global__ __launch_bounds__(256) void outer_rows_wide_kernel(const T* __restrict__ a, const T* __restrict__ b, int64_t n,
                                                               int m_total, int k_total, const int32_t* __restrict__ nbr,
+                                                              const int32_t* __restrict__ tap_ptr,
+                                                              const int32_t* __restrict__ pair_in,
                                                               int taps, int splits, int64_t rows_per_split,
                                                               int64_t slab_stride, float* __restrict__ d,
                                                               float* __restrict__ colsum) {
@@ -332,10 +348,22 @@ __global__ __launch_bounds__(256) void outer_rows_wide_kernel(const T* __restric
     int tap, split, m0, k0;
     if (!outer_item<OW_C>(taps, splits, m_total, k_total, &tap, &split, &m0, &k0)) return;
     const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
-    const int64_t r0 = (int64_t)split * rows_per_split;
+    int64_t r0 = (int64_t)split * rows_per_split;
     const int64_t r1 = min(n, r0 + rows_per_split);
     int count = (int)(r1 - r0);
-    if (GATHER) {
+    if (GATHER && tap_ptr) {
+        // the tap's own list of (output row, input row) pairs, rows_per_split of them per range: nbr holds the
+        // output rows here. Ranges past the end of a short tap's list have nothing to add and hand in zeros.
+        const int64_t p0 = tap_ptr[tap] + (int64_t)split * rows_per_split;
+        const int64_t left = (int64_t)tap_ptr[tap + 1] - p0;
+        count = left < 0 ? 0 : (int)min(left, rows_per_split);
+        for (int e = tid; e < count; e += 256) {
+            list_a[e] = nbr[p0 + e];
+            list_b[e] = pair_in[p0 + e];
+        }
+        r0 = 0;
+        __syncthreads();
+    } else if (GATHER) {
         if (tid == 0) list_n = 0;
         __syncthreads();
         const int32_t* nb = nbr + (int64_t)tap * n;
@@ -959,6 +987,23 @@ int launch_bn_bwd(AnyRows x, AnyRows dy, const float* stats, AnyRows gamma, AnyR
 bool ln_dtype_ok(int dtype) { return dtype >= PTV3_F32 && dtype <= PTV3_BF16; }
 bool ln_channels_ok(int c) { return c == 32 || c == 64 || c == 128 || c == 256 || c == 512; }
 
+// The output voxel of every pair of a tap-major pair list: pair q's product row has slot pair_slot[q], and the
+// slots of voxel i are [row_ptr[i], row_ptr[i + 1]).
+__global__ __launch_bounds__(256) void pair_out_kernel(const int32_t* __restrict__ row_ptr,
+                                                       const int32_t* __restrict__ pair_slot, int64_t n, int64_t n_pairs,
+                                                       int32_t* __restrict__ pair_out) {
+    const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (q >= n_pairs) return;
+    const int32_t slot = pair_slot[q];
+    int64_t lo = 0, hi = n - 1;   // the last voxel whose first slot is at or before this one
+    while (lo < hi) {
+        const int64_t mid = (lo + hi + 1) >> 1;
+        if (row_ptr[mid] <= slot) lo = mid;
+        else hi = mid - 1;
+    }
+    pair_out[q] = (int32_t)lo;
+}
+
 // one thread per (cluster, channel): walks the members in list order
 template <typename T>
 __global__ __launch_bounds__(256) void segment_reduce_bwd_kernel(const T* __restrict__ src, const T* __restrict__ out,
@@ -1042,7 +1087,8 @@ size_t outer_workspace(int64_t n, int m_total, int k_total, int taps) {
 // d (m_total, taps, k_total) fp32 is written in full; so is colsum (m_total,) when given: the column sums of a
 template <typename T, bool GATHER>
 int launch_outer(const void* a, const void* b, int64_t n, int m_total, int k_total, const int32_t* nbr, int taps,
-                 float* d, float* colsum, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                 float* d, float* colsum, void* workspace, size_t workspace_bytes, hipStream_t stream,
+                 const int32_t* tap_ptr = nullptr, const int32_t* pair_in = nullptr) {
     const int side = outer_side(m_total, k_total);
     const int64_t bm = ptv3_ceil_div(m_total, side), bk = ptv3_ceil_div(k_total, side);
     int64_t splits, rows;
@@ -1058,10 +1104,10 @@ int launch_outer(const void* a, const void* b, int64_t n, int m_total, int k_tot
     const dim3 grid((unsigned)items);
     if (side == OW_C)
         hipLaunchKernelGGL((outer_rows_wide_kernel<T, GATHER>), grid, dim3(256), 0, stream, (const T*)a, (const T*)b, n,
-                           m_total, k_total, nbr, taps, (int)splits, rows, stride, slabs, cols);
+                           m_total, k_total, nbr, tap_ptr, pair_in, taps, (int)splits, rows, stride, slabs, cols);
     else
         hipLaunchKernelGGL((outer_rows_kernel<T, GATHER>), grid, dim3(256), 0, stream, (const T*)a, (const T*)b, n,
-                           m_total, k_total, nbr, taps, (int)splits, rows, stride, slabs, cols);
+                           m_total, k_total, nbr, tap_ptr, pair_in, taps, (int)splits, rows, stride, slabs, cols);
     if (splits > 1) {
         const int64_t total = colsum ? stride : count;
         hipLaunchKernelGGL(slab_sum_kernel, dim3((unsigned)ptv3_ceil_div(total, 32)), dim3(256), 0, stream,
@@ -1132,6 +1178,32 @@ extern "C" int ptv3_subm_conv_wgrad(const void* feat, const void* dout, int dtyp
     if (dtype == PTV3_F16) return launch_wgrad<_Float16>(feat, dout, n, cin, cout, nbr, taps, dweight, stream);
     if (dtype == PTV3_BF16) return launch_wgrad<__bf16>(feat, dout, n, cin, cout, nbr, taps, dweight, stream);
     return launch_wgrad<float>(feat, dout, n, cin, cout, nbr, taps, dweight, stream);
+}
+
+extern "C" int ptv3_conv_plan_pair_out(const int32_t* row_ptr, const int32_t* pair_slot, int64_t n, int64_t n_pairs,
+                                       int32_t* pair_out, void* stream_) {
+    if (n < 0 || n_pairs < 0) return PTV3_EINVAL;
+    if (n == 0 || n_pairs == 0) return PTV3_OK;
+    if (!row_ptr || !pair_slot || !pair_out) return PTV3_EINVAL;
+    hipLaunchKernelGGL(pair_out_kernel, dim3((unsigned)ptv3_ceil_div(n_pairs, 256)), dim3(256), 0, (hipStream_t)stream_,
+                       row_ptr, pair_slot, n, n_pairs, pair_out);
+    PTV3_RETURN_LAUNCH();
+}
+
+extern "C" int ptv3_subm_conv_wgrad_pairs(const void* feat, const void* dout, int dtype, int64_t n, int cin, int cout,
+                                          const int32_t* tap_ptr, const int32_t* pair_in, const int32_t* pair_out,
+                                          int taps, float* dweight, float* dbias, void* workspace,
+                                          size_t workspace_bytes, void* stream_) {
+    if (n < 1 || cin < 1 || cout < 1 || taps < 1) return PTV3_EINVAL;
+    if (!wgrad_on_mfma(dtype, cin, cout)) return PTV3_ESHAPE;
+    if (!feat || !dout || !tap_ptr || !pair_in || !pair_out || !dweight) return PTV3_EINVAL;
+    if ((int64_t)taps * ptv3_ceil_div(n, 256) >= (1ll << 31)) return PTV3_EINVAL;
+    hipStream_t stream = (hipStream_t)stream_;
+    if (dtype == PTV3_F16)
+        return launch_outer<_Float16, true>(dout, feat, n, cout, cin, pair_out, taps, dweight, dbias, workspace,
+                                            workspace_bytes, stream, tap_ptr, pair_in);
+    return launch_outer<__bf16, true>(dout, feat, n, cout, cin, pair_out, taps, dweight, dbias, workspace,
+                                      workspace_bytes, stream, tap_ptr, pair_in);
 }
 
 extern "C" size_t ptv3_linear_wgrad_workspace_bytes(int64_t n, int k, int nout) {

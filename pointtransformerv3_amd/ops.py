@@ -477,10 +477,42 @@ def subm_conv_wgrad(feat, dout, nbr, with_bias=False):
     return (dw, db) if with_bias else dw
 
 
+OUTER_WIDE_CHANNELS = 128   # from here on both sides, the weight-gradient kernels work on 128 x 128 blocks
+
+
+def subm_conv_wgrad_pairs(feat, dout, plan, with_bias=False):
+    """The same weight gradient (and bias gradient) from a ConvPlan's pair lists instead of the neighbour map
+    (ptv3_subm_conv_wgrad_pairs): half precision, channels in 8s."""
+    _dev(feat, dout)
+    lib = _lib.load()
+    feat = feat.contiguous()
+    dout = dout.to(feat.dtype).contiguous()
+    n, cin = feat.shape
+    cout = dout.shape[1]
+    dw = torch.empty((cout, plan.taps, cin), dtype=torch.float32, device=feat.device)
+    db = torch.empty(cout, dtype=torch.float32, device=feat.device) if with_bias else None
+    nbytes = lib.ptv3_subm_conv_wgrad_workspace_bytes(_dtype_code(feat), n, cin, cout, plan.taps)
+    ws = _ws(nbytes, feat.device) if nbytes else None
+    _lib.check(lib.ptv3_subm_conv_wgrad_pairs(_ptr(feat), _ptr(dout), _dtype_code(feat), n, cin, cout, _ptr(plan.tap_ptr),
+                                              _ptr(plan.pair_in), _ptr(plan.pair_out()), plan.taps, _ptr(dw), _ptr(db),
+                                              _ptr(ws), nbytes, _stream()), "ptv3_subm_conv_wgrad_pairs")
+    return (dw, db) if with_bias else dw
+
+
 class ConvPlan:
     """Active (input, output) pairs of a neighbour map, tap-major, plus each voxel's slots."""
 
-    __slots__ = ("n", "taps", "_n_pairs", "tap_ptr", "row_ptr", "pair_in", "pair_slot", "_slot_pair", "_tiles")
+    __slots__ = ("n", "taps", "_n_pairs", "tap_ptr", "row_ptr", "pair_in", "pair_slot", "_slot_pair", "_tiles",
+                 "_pair_out")
+
+    def pair_out(self):
+        """The output voxel of every pair (the weight gradient's other index), made on first use."""
+        if getattr(self, "_pair_out", None) is None:
+            po = torch.empty(max(self.n_pairs, 1), dtype=torch.int32, device=self.pair_in.device)
+            _lib.check(_lib.load().ptv3_conv_plan_pair_out(_ptr(self.row_ptr), _ptr(self.pair_slot), self.n, self.n_pairs,
+                                                           _ptr(po), _stream()), "ptv3_conv_plan_pair_out")
+            self._pair_out = po
+        return self._pair_out
 
     @property
     def n_pairs(self):

@@ -625,3 +625,22 @@ def test_packed_convolution_weight_follows_a_fused_optimizer():
     second = conv._packed_weight(torch.float16)
     want = o.conv_pack_weight(conv.weight.detach().reshape(64, -1, 64), 27, torch.float16)
     assert second is not first and torch.equal(second, want) and not torch.equal(second, first)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("cin,cout,ks", [(64, 64, 3), (128, 128, 3), (8, 32, 5), (256, 128, 3)])
+def test_conv_weight_gradient_from_pair_lists(dtype, cin, cout, ks):
+    """ptv3_subm_conv_wgrad_pairs (ranges of each tap's own pair list) against ptv3_subm_conv_wgrad (compaction
+    of the neighbour map) on the same inputs: the same sums in another order, and the same bias gradient."""
+    o = ops()
+    rng = np.random.default_rng(cin + cout + ks)
+    grid, batch, _ = unique_voxels(rng, 6000, 24, nb=2)
+    indices = torch.cat([to_dev(batch).int()[:, None], to_dev(grid)], 1).contiguous()   # (N, 4) batch, x, y, z
+    nbr = o.kmap_build(indices, ks, tap_major=True)
+    plan = o.conv_plan(nbr, tap_major=True)
+    n = grid.shape[0]
+    x = torch.randn(n, cin, device=DEV).to(dtype)
+    dy = torch.randn(n, cout, device=DEV).to(dtype)
+    dw_a, db_a = o.subm_conv_wgrad(x, dy, nbr, with_bias=True)
+    dw_b, db_b = o.subm_conv_wgrad_pairs(x, dy, plan, with_bias=True)
+    assert rel_err(dw_b, dw_a.cpu()) < 1e-5 and rel_err(db_b, db_a.cpu()) < 1e-5
