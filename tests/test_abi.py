@@ -44,6 +44,37 @@ def test_argument_errors_without_a_device():
     assert b"workspace" in lib.ptv3_strerror(-3)
 
 
+def test_argument_errors_of_the_training_entry_points():
+    """Shape and pointer checks come before any launch, so they can be exercised without a GPU."""
+    from pointtransformerv3_amd import _lib
+    lib = _lib.load()
+    # Linear + GELU: fp16 / bf16 only, 32 ... 512 inputs, outputs in 32s; empty input is fine; null pointers
+    assert lib.ptv3_linear_gelu_fwd(None, None, None, 0, 10, 64, 256, None, None, None) == -4
+    assert lib.ptv3_linear_gelu_fwd(None, None, None, 1, 10, 48, 256, None, None, None) == -4
+    assert lib.ptv3_linear_gelu_fwd(None, None, None, 1, 10, 64, 250, None, None, None) == -4
+    assert lib.ptv3_linear_gelu_fwd(None, None, None, 1, 0, 64, 256, None, None, None) == 0
+    assert lib.ptv3_linear_gelu_fwd(None, None, None, 1, 10, 64, 256, None, None, None) == -1
+    assert lib.ptv3_linear_gelu_bwd(None, None, None, 2, 10, 64, 256, None, None) == -1
+    assert lib.ptv3_linear_gelu_bwd(None, None, None, 2, 10, 1024, 256, None, None) == -4
+    # mixed-dtype residual add: channels in 8s, known dtype codes
+    assert lib.ptv3_scaled_add(None, 0, None, 2, None, 0, 10, 12, None, 0, None) == -4
+    assert lib.ptv3_scaled_add(None, 0, None, 7, None, 0, 10, 16, None, 0, None) == -1
+    assert lib.ptv3_scaled_add(None, 0, None, 2, None, 0, 0, 16, None, 0, None) == 0
+    assert lib.ptv3_scaled_add(None, 0, None, 2, None, 0, 10, 16, None, 0, None) == -1
+    # parameter casts: block counts of the two job kinds, empty tables, unknown dtype
+    assert lib.ptv3_cast_params_blocks(1, 1, 4096, 0) == 1 and lib.ptv3_cast_params_blocks(1, 1, 4097, 0) == 2
+    assert lib.ptv3_cast_params_blocks(65, 27, 64, 1) == 27 * 2 * 1 and lib.ptv3_cast_params_blocks(0, 3, 3, 1) == 0
+    assert lib.ptv3_cast_params(None, 0, 0, 1, None) == 0
+    assert lib.ptv3_cast_params(None, 3, 5, 1, None) == -1
+    assert lib.ptv3_cast_params(None, -1, 5, 1, None) == -1
+    # weight gradient from pair lists: matrix-core shapes only, every list needed
+    assert lib.ptv3_subm_conv_wgrad_pairs(None, None, 0, 10, 64, 64, None, None, None, 27, None, None, None, 0, None) == -4
+    assert lib.ptv3_subm_conv_wgrad_pairs(None, None, 1, 10, 60, 64, None, None, None, 27, None, None, None, 0, None) == -4
+    assert lib.ptv3_subm_conv_wgrad_pairs(None, None, 1, 10, 64, 64, None, None, None, 27, None, None, None, 0, None) == -1
+    assert lib.ptv3_conv_plan_pair_out(None, None, 0, 0, None, None) == 0
+    assert lib.ptv3_conv_plan_pair_out(None, None, 5, 9, None, None) == -1
+
+
 def test_pad_sizes_host_arithmetic():
     from pointtransformerv3_amd import ops
     assert ops.pad_sizes([2500], 1024) == (3072, 3)
