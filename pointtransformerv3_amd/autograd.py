@@ -78,8 +78,8 @@ class SubMConv(torch.autograd.Function):
             want_bias = ctx.has_bias and ctx.needs_input_grad[2]
             if x.dtype != torch.float32 and cout % 8 == 0 and min(x.shape[1], cout) < ops.OUTER_WIDE_CHANNELS:
                 # the forward's pair lists: no neighbour map to build, no compaction, ranges of equal length
-                # (24 % faster on the 64 x 64 block kernel; the 128 x 128 one measured 14 % slower that way:
-                # its short taps hand in blocks of zeros four times the size)
+                # (half the time on the 64 x 64 block kernel; the 128 x 128 one measured 10 % slower that way:
+                # it wants more and shorter work-groups than full ranges give it)
                 dw, db = ops.subm_conv_wgrad_pairs(x, dout, sparse.conv_plan(module.kernel_size, module.indice_key),
                                                    with_bias=True)
             else:

@@ -185,10 +185,12 @@ __global__ __launch_bounds__(256) void outer_rows_kernel(const T* __restrict__ a
     int count = (int)(r1 - r0);
     if (GATHER && tap_ptr) {
         // the tap's own list of (output row, input row) pairs, rows_per_split of them per range: nbr holds the
-        // output rows here. Ranges past the end of a short tap's list have nothing to add and hand in zeros.
+        // output rows here.
         const int64_t p0 = tap_ptr[tap] + (int64_t)split * rows_per_split;
         const int64_t left = (int64_t)tap_ptr[tap + 1] - p0;
         count = left < 0 ? 0 : (int)min(left, rows_per_split);
+        // past the end of a short tap's list: the sum over ranges skips this one (a single range is the result itself)
+        if (count == 0 && splits > 1) return;
         for (int e = tid; e < count; e += 256) {
             list_a[e] = nbr[p0 + e];
             list_b[e] = pair_in[p0 + e];
@@ -353,10 +355,12 @@ __global__ __launch_bounds__(256) void outer_rows_wide_kernel(const T* __restric
     int count = (int)(r1 - r0);
     if (GATHER && tap_ptr) {
         // the tap's own list of (output row, input row) pairs, rows_per_split of them per range: nbr holds the
-        // output rows here. Ranges past the end of a short tap's list have nothing to add and hand in zeros.
+        // output rows here.
         const int64_t p0 = tap_ptr[tap] + (int64_t)split * rows_per_split;
         const int64_t left = (int64_t)tap_ptr[tap + 1] - p0;
         count = left < 0 ? 0 : (int)min(left, rows_per_split);
+        // past the end of a short tap's list: the sum over ranges skips this one (a single range is the result itself)
+        if (count == 0 && splits > 1) return;
         for (int e = tid; e < count; e += 256) {
             list_a[e] = nbr[p0 + e];
             list_b[e] = pair_in[p0 + e];
@@ -479,14 +483,22 @@ __global__ __launch_bounds__(256) void outer_rows_wide_kernel(const T* __restric
 
 // out[i] = sum over the splits' slabs (of `stride` floats, the first `total` of them summed): a work-group takes 32 neighbouring values, its 8 thread rows share
 // out the splits (four loads in flight each) and meet in LDS
+// With tap_ptr (pair-list ranges) the value i = (m * taps + tap) * k_total + k of the first result only has the
+// ranges its tap's list reaches: ceil(pairs of the tap / rows_per_split) of them; the others were never written.
 __global__ __launch_bounds__(256) void slab_sum_kernel(const float* __restrict__ slabs, int64_t stride, int64_t total,
                                                        int splits, float* __restrict__ out, int64_t first,
-                                                       float* __restrict__ out2) {
+                                                       float* __restrict__ out2, const int32_t* __restrict__ tap_ptr,
+                                                       int taps, int k_total, int64_t rows_per_split) {
     __shared__ float part[8][32];
     const int e = threadIdx.x % 32, lane_s = threadIdx.x / 32;
     const int64_t i = (int64_t)blockIdx.x * 32 + e;
     float v0 = 0.f, v1 = 0.f, v2 = 0.f, v3 = 0.f;
     if (i < total) {
+        if (tap_ptr && i < first) {
+            const int t = (int)(((uint32_t)i / (uint32_t)k_total) % (uint32_t)taps);   // first < 2^31: checked at launch
+            const int64_t have = ((int64_t)tap_ptr[t + 1] - tap_ptr[t] + rows_per_split - 1) / rows_per_split;
+            if (have < splits) splits = (int)have;
+        }
         int s = lane_s;
         for (; s + 24 < splits; s += 32) {
             v0 += slabs[(int64_t)s * stride + i];
@@ -1109,9 +1121,10 @@ int launch_outer(const void* a, const void* b, int64_t n, int m_total, int k_tot
         hipLaunchKernelGGL((outer_rows_kernel<T, GATHER>), grid, dim3(256), 0, stream, (const T*)a, (const T*)b, n,
                            m_total, k_total, nbr, tap_ptr, pair_in, taps, (int)splits, rows, stride, slabs, cols);
     if (splits > 1) {
+        if (tap_ptr && count >= (1ll << 31)) return PTV3_EINVAL;
         const int64_t total = colsum ? stride : count;
         hipLaunchKernelGGL(slab_sum_kernel, dim3((unsigned)ptv3_ceil_div(total, 32)), dim3(256), 0, stream,
-                           (const float*)slabs, stride, total, (int)splits, d, count, colsum);
+                           (const float*)slabs, stride, total, (int)splits, d, count, colsum, tap_ptr, taps, k_total, rows);
     }
     PTV3_RETURN_LAUNCH();
 }
