@@ -351,19 +351,26 @@ int ptv3_cast_params(const ptv3_cast_job *jobs, int n_jobs, int64_t n_blocks, in
  * factor per row, model.py:583 -- may be NULL; sum may be NULL when only y is wanted (then this is a plain
  * LayerNorm of branch). Every tensor has its own dtype code (0 fp32, 1 fp16, 2 bf16): under autocast the
  * residual stream is float and the branches half precision. gamma, beta (c,) of param_dtype.
- * c in {32, 64, 128, 256, 512}. The statistics are taken from sum as rounded to sum_dtype. */
+ * c in {32, 64, 128, 256, 512}. The statistics are taken from sum as rounded to sum_dtype.
+ * pre_gamma, pre_beta (c,) of param_dtype, both or neither NULL: the branch first goes through a LayerNorm of
+ * its own (the xCPE's norm in front of a Block's first residual connection, model.py:546-554, :589-592),
+ * sum = skip + LayerNorm_pre(branch) * row_scale, in the same pass and without rounding in between. */
 int ptv3_add_layer_norm_fwd(const void *skip, int skip_dtype, const void *branch, int branch_dtype,
                             const void *row_scale, int row_scale_dtype, const void *gamma, const void *beta,
                             int param_dtype, int64_t n, int c, float eps, void *sum, int sum_dtype, void *y,
-                            int y_dtype, void *stream);
+                            int y_dtype, const void *pre_gamma, const void *pre_beta, float pre_eps, void *stream);
 
 /* Its backward: g = LayerNorm'(sum; dy) + dsum (dsum: the gradient that reaches sum past the LayerNorm, or
  * NULL); dskip = g and dbranch = g * row_scale, either may be NULL, each in its own dtype. dgamma, dbeta
- * (c,) fp32 are accumulated into (zero them first). */
+ * (c,) fp32 are accumulated into (zero them first). With pre_x (the branch as the forward read it, n x c of
+ * pre_x_dtype) the branch's own LayerNorm is taken back as well: dbranch is then the gradient of pre_x, and
+ * dpre_gamma, dpre_beta (c,) fp32 are accumulated into like dgamma, dbeta. */
 int ptv3_add_layer_norm_bwd(const void *sum, int sum_dtype, const void *dy, int dy_dtype, const void *dsum,
                             int dsum_dtype, const void *row_scale, int row_scale_dtype, const void *gamma,
                             int param_dtype, int64_t n, int c, float eps, void *dskip, int dskip_dtype,
-                            void *dbranch, int dbranch_dtype, float *dgamma, float *dbeta, void *stream);
+                            void *dbranch, int dbranch_dtype, float *dgamma, float *dbeta, const void *pre_x,
+                            int pre_x_dtype, const void *pre_gamma, float pre_eps, float *dpre_gamma,
+                            float *dpre_beta, void *stream);
 
 /* A residual connection with no LayerNorm behind it (model.py:602-604, the end of a Block, with the
  * stochastic-depth factor of model.py:583): out = skip + branch * row_scale, rows (n,c), c a multiple of 8, each

@@ -70,9 +70,9 @@ SIGNATURES = {
     "ptv3_linear_fwd": (_i32, [_vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp]),
     "ptv3_linear_bn_act_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _f32, _i32, _i64, _i32, _i32, _i32, _vp, _vp]),
     "ptv3_add_layer_norm_fwd": (_i32, [_vp, _i32, _vp, _i32, _vp, _i32, _vp, _vp, _i32, _i64, _i32, _f32, _vp, _i32,
-                                       _vp, _i32, _vp]),
+                                       _vp, _i32, _vp, _vp, _f32, _vp]),
     "ptv3_add_layer_norm_bwd": (_i32, [_vp, _i32, _vp, _i32, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i32, _f32, _vp,
-                                       _i32, _vp, _i32, _vp, _vp, _vp]),
+                                       _i32, _vp, _i32, _vp, _vp, _vp, _i32, _vp, _f32, _vp, _vp, _vp]),
     "ptv3_batch_norm_stats": (_i32, [_vp, _i32, _i64, _i32, _f32, _f32, _vp, _vp, _vp, _vp, _vp]),
     "ptv3_batch_norm_bwd": (_i32, [_vp, _i32, _vp, _i32, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _i32, _vp,
                                    _vp]),

@@ -192,23 +192,32 @@ class AddLayerNorm(torch.autograd.Function):
     """s = skip + branch * mask, y = LayerNorm(s): a residual connection followed by the next pre-norm
     (model.py:589-604; mask is the stochastic-depth factor per row, or None), one kernel each way. Returns
     (s, y), y in out_dtype; the backward kernel adds the gradient arriving at s to the LayerNorm's own, so
-    autograd has nothing to accumulate, and writes each input's gradient in that input's dtype."""
+    autograd has nothing to accumulate, and writes each input's gradient in that input's dtype.
+    With pre_weight, pre_bias, pre_eps the branch first goes through a LayerNorm of its own in the same pass
+    (s = skip + LayerNorm_pre(branch) * mask: the xCPE's norm, model.py:546-554)."""
 
     @staticmethod
-    def forward(ctx, skip, branch, mask, weight, bias, eps, out_dtype=None):
-        s, y = ops.add_layer_norm(skip, branch, mask, weight.detach(), bias.detach(), eps, out_dtype=out_dtype)
-        ctx.save_for_backward(s, weight, mask)
-        ctx.eps, ctx.dtypes = eps, (skip.dtype, branch.dtype, bias.dtype)
+    def forward(ctx, skip, branch, mask, weight, bias, eps, out_dtype=None, pre_weight=None, pre_bias=None, pre_eps=0.0):
+        pre = None if pre_weight is None else (pre_weight.detach(), pre_bias.detach(), pre_eps)
+        s, y = ops.add_layer_norm(skip, branch, mask, weight.detach(), bias.detach(), eps, out_dtype=out_dtype, pre=pre)
+        ctx.save_for_backward(s, weight, mask, *(() if pre is None else (branch, pre_weight)))
+        ctx.eps, ctx.pre_eps, ctx.dtypes = eps, pre_eps, (skip.dtype, branch.dtype, bias.dtype)
+        ctx.pre_bias_dtype = None if pre is None else pre_bias.dtype
         return s, y
 
     @staticmethod
     def backward(ctx, ds, dy):
-        s, weight, mask = ctx.saved_tensors
+        s, weight, mask, *rest = ctx.saved_tensors
         skip_dtype, branch_dtype, bias_dtype = ctx.dtypes
-        dskip, dbranch, dw, db = ops.add_layer_norm_bwd(s, dy, ds, mask, weight.detach(), ctx.eps,
-                                                        skip_dtype=skip_dtype if ctx.needs_input_grad[0] else None,
-                                                        branch_dtype=branch_dtype if ctx.needs_input_grad[1] else None)
-        return dskip, dbranch, None, dw.to(weight.dtype), db.to(bias_dtype), None, None
+        pre = (rest[0], rest[1].detach(), ctx.pre_eps) if rest else None
+        out = ops.add_layer_norm_bwd(s, dy, ds, mask, weight.detach(), ctx.eps,
+                                     skip_dtype=skip_dtype if ctx.needs_input_grad[0] else None,
+                                     branch_dtype=branch_dtype if ctx.needs_input_grad[1] else None, pre=pre)
+        dskip, dbranch, dw, db = out[:4]
+        dpw = dpb = None
+        if pre is not None:
+            dpw, dpb = out[4].to(rest[1].dtype), out[5].to(ctx.pre_bias_dtype)
+        return dskip, dbranch, None, dw.to(weight.dtype), db.to(bias_dtype), None, None, dpw, dpb, None
 
 
 class ResidualAdd(torch.autograd.Function):

@@ -629,38 +629,55 @@ struct AnyRowsOut {
 
 // sum = skip + branch * row_scale (skip and row_scale optional), y = LayerNorm(sum): 8 channels per lane, a row
 // per LPR lanes; the statistics are taken from the sum as stored, so the backward kernel sees the same numbers.
-template <int LPR>
+// PRE: the branch goes through a LayerNorm of its own first (pre_gamma, pre_beta, pre_eps): the xCPE's norm in front
+// of the first residual connection of a Block (model.py:546-554, :589-592).
+template <int LPR, bool PRE>
 __global__ __launch_bounds__(256) void add_layer_norm_fwd_kernel(AnyRows skip, AnyRows branch, AnyRows row_scale,
                                                                  AnyRows gamma, AnyRows beta, int64_t n, float eps,
-                                                                 AnyRowsOut sum, AnyRowsOut y) {
+                                                                 AnyRowsOut sum, AnyRowsOut y, AnyRows pre_gamma,
+                                                                 AnyRows pre_beta, float pre_eps) {
     constexpr int C = LPR * 8, RPW = PTV3_WAVE / LPR;
     const int wave = threadIdx.x / PTV3_WAVE, lane = threadIdx.x % PTV3_WAVE;
     const int sub = lane % LPR, rsub = lane / LPR;
-    float g[8], b[8];
+    float g[8], b[8], pg[8], pb[8];
     load8_any(gamma.p, gamma.dtype, sub * 8, g);
     load8_any(beta.p, beta.dtype, sub * 8, b);
+    if (PRE) {
+        load8_any(pre_gamma.p, pre_gamma.dtype, sub * 8, pg);
+        load8_any(pre_beta.p, pre_beta.dtype, sub * 8, pb);
+    }
     const int64_t stride = (int64_t)gridDim.x * 4 * RPW;
     for (int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * RPW; row0 < n; row0 += stride) {
         const int64_t row = row0 + rsub;
         const bool valid = row < n;
         const int64_t off = row * C + sub * 8;
-        float xv[8];
+        float xv[8], sv[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) xv[i] = 0.f;
+        for (int i = 0; i < 8; ++i) { xv[i] = 0.f; sv[i] = 0.f; }
+        float m = 1.f;
         if (valid) {
             const Raw8 rb = raw8_load(branch.p, branch.dtype, off);
             Raw8 rs = rb;
             if (skip.p) rs = raw8_load(skip.p, skip.dtype, off);
-            const float m = row_scale.p ? load1_any(row_scale.p, row_scale.dtype, row) : 1.f;
+            if (row_scale.p) m = load1_any(row_scale.p, row_scale.dtype, row);
             raw8_floats(rb, branch.dtype, xv);
+            if (skip.p) raw8_floats(rs, skip.dtype, sv);
+        }
+        if (PRE) {   // every lane takes part in the row sums, rows past the end with zeros
+            float ps = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) xv[i] *= m;
-            if (skip.p) {
-                float sv[8];
-                raw8_floats(rs, skip.dtype, sv);
+            for (int i = 0; i < 8; ++i) ps += xv[i];
+            const float pmean = row_sum<LPR>(ps) * (1.f / C);
+            float pq = 0.f;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) xv[i] += sv[i];
-            }
+            for (int i = 0; i < 8; ++i) { xv[i] -= pmean; pq = fmaf(xv[i], xv[i], pq); }
+            const float prstd = rsqrtf(row_sum<LPR>(pq) * (1.f / C) + pre_eps);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) xv[i] = fmaf(xv[i] * prstd, pg[i], pb[i]);
+        }
+        if (valid) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) xv[i] = fmaf(xv[i], m, sv[i]);
             if (sum.p) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) xv[i] = round_any(xv[i], sum.dtype);
@@ -685,19 +702,25 @@ __global__ __launch_bounds__(256) void add_layer_norm_fwd_kernel(AnyRows skip, A
 
 // g = LayerNorm'(sum, dy) + dsum (dsum optional); dskip = g, dbranch = g * row_scale, each optional and in its
 // own dtype; dgamma / dbeta accumulated in fp32. Mean and rstd are recomputed from sum.
-template <int LPR>
+// PRE: the branch came out of a LayerNorm of its own (see the forward kernel): pre_x is that norm's input,
+// dbranch its gradient, dpre_gamma / dpre_beta the norm's parameter gradients.
+template <int LPR, bool PRE>
 __global__ __launch_bounds__(256) void add_layer_norm_bwd_kernel(AnyRows sum, AnyRows dy, AnyRows dsum, AnyRows row_scale,
                                                                  AnyRows gamma, int64_t n, float eps, AnyRowsOut dskip,
                                                                  AnyRowsOut dbranch, float* __restrict__ dgamma,
-                                                                 float* __restrict__ dbeta) {
+                                                                 float* __restrict__ dbeta, AnyRows pre_x,
+                                                                 AnyRows pre_gamma, float pre_eps,
+                                                                 float* __restrict__ dpre_gamma,
+                                                                 float* __restrict__ dpre_beta) {
     constexpr int C = LPR * 8, RPW = PTV3_WAVE / LPR;
-    __shared__ float part[2][4][C];
+    __shared__ float part[PRE ? 4 : 2][4][C];
     const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
     const int sub = lane % LPR, rsub = lane / LPR;
-    float g[8], ag[8], ab[8];
+    float g[8], ag[8], ab[8], pg[8], pag[8], pab[8];
     load8_any(gamma.p, gamma.dtype, sub * 8, g);
+    if (PRE) load8_any(pre_gamma.p, pre_gamma.dtype, sub * 8, pg);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { ag[i] = 0.f; ab[i] = 0.f; }
+    for (int i = 0; i < 8; ++i) { ag[i] = 0.f; ab[i] = 0.f; pag[i] = 0.f; pab[i] = 0.f; }
     const int64_t stride = (int64_t)gridDim.x * 4 * RPW;
     for (int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * RPW; row0 < n; row0 += stride) {
         const int64_t row = row0 + rsub;
@@ -719,6 +742,13 @@ __global__ __launch_bounds__(256) void add_layer_norm_bwd_kernel(AnyRows sum, An
             raw8_floats(rg, dy.dtype, gv);
             if (dsum.p) raw8_floats(re, dsum.dtype, extra);
         }
+        float cv[8];   // PRE: the input of the branch's own norm
+#pragma unroll
+        for (int i = 0; i < 8; ++i) cv[i] = 0.f;
+        if (PRE && valid) {
+            const Raw8 rc = raw8_load(pre_x.p, pre_x.dtype, off);
+            raw8_floats(rc, pre_x.dtype, cv);
+        }
         float s = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) s += xv[i];
@@ -739,17 +769,38 @@ __global__ __launch_bounds__(256) void add_layer_norm_bwd_kernel(AnyRows sum, An
         }
         s1 = row_sum<LPR>(s1) * (1.f / C);
         s2 = row_sum<LPR>(s2) * (1.f / C);
-        if (valid) {
-            float o[8];
+        float o[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) o[i] = rstd * (gv[i] - s1 - xv[i] * s2) + extra[i];
-            if (dskip.p) store8_any(dskip.p, dskip.dtype, off, o);
-            if (dbranch.p) {
+        for (int i = 0; i < 8; ++i) o[i] = valid ? rstd * (gv[i] - s1 - xv[i] * s2) + extra[i] : 0.f;
+        if (valid && dskip.p) store8_any(dskip.p, dskip.dtype, off, o);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) o[i] *= scale;
-                store8_any(dbranch.p, dbranch.dtype, off, o);
+        for (int i = 0; i < 8; ++i) o[i] *= scale;   // the gradient of the branch as it was added
+        if (PRE) {
+            // back through the branch's own norm: statistics again from its input, rows past the end carry zeros
+            float cs = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) cs += cv[i];
+            const float cmean = row_sum<LPR>(cs) * (1.f / C);
+            float cq = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { cv[i] -= cmean; cq = fmaf(cv[i], cv[i], cq); }
+            const float crstd = rsqrtf(row_sum<LPR>(cq) * (1.f / C) + pre_eps);
+            float t1 = 0.f, t2 = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                cv[i] *= crstd;                        // xhat of the branch's norm
+                pag[i] = fmaf(o[i], cv[i], pag[i]);
+                pab[i] += o[i];
+                o[i] *= pg[i];
+                t1 += o[i];
+                t2 = fmaf(o[i], cv[i], t2);
             }
+            t1 = row_sum<LPR>(t1) * (1.f / C);
+            t2 = row_sum<LPR>(t2) * (1.f / C);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o[i] = crstd * (o[i] - t1 - cv[i] * t2);
         }
+        if (valid && dbranch.p) store8_any(dbranch.p, dbranch.dtype, off, o);
     }
     // column sums: over the rows a wave holds side by side, then over the waves, then one atomic per channel
 #pragma unroll
@@ -760,18 +811,33 @@ __global__ __launch_bounds__(256) void add_layer_norm_bwd_kernel(AnyRows sum, An
             ab[i] += __shfl_xor(ab[i], off, PTV3_WAVE);
         }
     }
+    if (PRE) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int off = LPR; off < PTV3_WAVE; off <<= 1) {
+                pag[i] += __shfl_xor(pag[i], off, PTV3_WAVE);
+                pab[i] += __shfl_xor(pab[i], off, PTV3_WAVE);
+            }
+        }
+    }
     if (rsub == 0) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             part[0][wave][sub * 8 + i] = ag[i];
             part[1][wave][sub * 8 + i] = ab[i];
+            if (PRE) {
+                part[2][wave][sub * 8 + i] = pag[i];
+                part[3][wave][sub * 8 + i] = pab[i];
+            }
         }
     }
     __syncthreads();
-    for (int c = tid; c < 2 * C; c += 256) {
+    for (int c = tid; c < (PRE ? 4 : 2) * C; c += 256) {
         const int which = c / C, ch = c % C;
         const float v = part[which][0][ch] + part[which][1][ch] + part[which][2][ch] + part[which][3][ch];
-        atomicAdd((which ? dbeta : dgamma) + ch, v);
+        float* dst = which == 0 ? dgamma : which == 1 ? dbeta : which == 2 ? dpre_gamma : dpre_beta;
+        atomicAdd(dst + ch, v);
     }
 }
 
@@ -783,11 +849,18 @@ int64_t ln_grid(int64_t n, int c) {
 }
 
 int launch_add_ln_fwd(AnyRows skip, AnyRows branch, AnyRows row_scale, AnyRows gamma, AnyRows beta, int64_t n, int c,
-                      float eps, AnyRowsOut sum, AnyRowsOut y, hipStream_t stream) {
+                      float eps, AnyRowsOut sum, AnyRowsOut y, AnyRows pre_gamma, AnyRows pre_beta, float pre_eps,
+                      hipStream_t stream) {
 #define PTV3_LNF(L)                                                                                                   \
     if (c == 8 * L) {                                                                                                 \
-        hipLaunchKernelGGL((add_layer_norm_fwd_kernel<L>), dim3((unsigned)ln_grid(n, c)), dim3(256), 0, stream, skip, \
-                           branch, row_scale, gamma, beta, n, eps, sum, y);                                           \
+        if (pre_gamma.p)                                                                                              \
+            hipLaunchKernelGGL((add_layer_norm_fwd_kernel<L, true>), dim3((unsigned)ln_grid(n, c)), dim3(256), 0,     \
+                               stream, skip, branch, row_scale, gamma, beta, n, eps, sum, y, pre_gamma, pre_beta,     \
+                               pre_eps);                                                                              \
+        else                                                                                                          \
+            hipLaunchKernelGGL((add_layer_norm_fwd_kernel<L, false>), dim3((unsigned)ln_grid(n, c)), dim3(256), 0,    \
+                               stream, skip, branch, row_scale, gamma, beta, n, eps, sum, y, pre_gamma, pre_beta,     \
+                               pre_eps);                                                                              \
         PTV3_RETURN_LAUNCH();                                                                                         \
     }
     PTV3_LNF(4) PTV3_LNF(8) PTV3_LNF(16) PTV3_LNF(32) PTV3_LNF(64)
@@ -796,11 +869,18 @@ int launch_add_ln_fwd(AnyRows skip, AnyRows branch, AnyRows row_scale, AnyRows g
 }
 
 int launch_add_ln_bwd(AnyRows sum, AnyRows dy, AnyRows dsum, AnyRows row_scale, AnyRows gamma, int64_t n, int c, float eps,
-                      AnyRowsOut dskip, AnyRowsOut dbranch, float* dgamma, float* dbeta, hipStream_t stream) {
+                      AnyRowsOut dskip, AnyRowsOut dbranch, float* dgamma, float* dbeta, AnyRows pre_x, AnyRows pre_gamma,
+                      float pre_eps, float* dpre_gamma, float* dpre_beta, hipStream_t stream) {
 #define PTV3_LNB(L)                                                                                                   \
     if (c == 8 * L) {                                                                                                 \
-        hipLaunchKernelGGL((add_layer_norm_bwd_kernel<L>), dim3((unsigned)ln_grid(n, c)), dim3(256), 0, stream, sum,  \
-                           dy, dsum, row_scale, gamma, n, eps, dskip, dbranch, dgamma, dbeta);                        \
+        if (pre_x.p)                                                                                                  \
+            hipLaunchKernelGGL((add_layer_norm_bwd_kernel<L, true>), dim3((unsigned)ln_grid(n, c)), dim3(256), 0,     \
+                               stream, sum, dy, dsum, row_scale, gamma, n, eps, dskip, dbranch, dgamma, dbeta, pre_x, \
+                               pre_gamma, pre_eps, dpre_gamma, dpre_beta);                                            \
+        else                                                                                                          \
+            hipLaunchKernelGGL((add_layer_norm_bwd_kernel<L, false>), dim3((unsigned)ln_grid(n, c)), dim3(256), 0,    \
+                               stream, sum, dy, dsum, row_scale, gamma, n, eps, dskip, dbranch, dgamma, dbeta, pre_x, \
+                               pre_gamma, pre_eps, dpre_gamma, dpre_beta);                                            \
         PTV3_RETURN_LAUNCH();                                                                                         \
     }
     PTV3_LNB(4) PTV3_LNB(8) PTV3_LNB(16) PTV3_LNB(32) PTV3_LNB(64)
@@ -1246,17 +1326,18 @@ extern "C" int ptv3_linear_wgrad(const void* x, const void* dout, int dtype, int
 extern "C" int ptv3_add_layer_norm_fwd(const void* skip, int skip_dtype, const void* branch, int branch_dtype,
                                        const void* row_scale, int row_scale_dtype, const void* gamma, const void* beta,
                                        int param_dtype, int64_t n, int c, float eps, void* sum, int sum_dtype, void* y,
-                                       int y_dtype, void* stream_) {
+                                       int y_dtype, const void* pre_gamma, const void* pre_beta, float pre_eps,
+                                       void* stream_) {
     if (n < 0 || c < 1) return PTV3_EINVAL;
     if (!ln_dtype_ok(skip_dtype) || !ln_dtype_ok(branch_dtype) || !ln_dtype_ok(row_scale_dtype) ||
         !ln_dtype_ok(param_dtype) || !ln_dtype_ok(sum_dtype) || !ln_dtype_ok(y_dtype))
         return PTV3_EINVAL;
     if (!ln_channels_ok(c)) return PTV3_ESHAPE;
     if (n == 0) return PTV3_OK;
-    if (!branch || !gamma || !beta || !y) return PTV3_EINVAL;
+    if (!branch || !gamma || !beta || !y || (pre_gamma == nullptr) != (pre_beta == nullptr)) return PTV3_EINVAL;
     return launch_add_ln_fwd({skip, skip_dtype}, {branch, branch_dtype}, {row_scale, row_scale_dtype},
                              {gamma, param_dtype}, {beta, param_dtype}, n, c, eps, {sum, sum_dtype}, {y, y_dtype},
-                             (hipStream_t)stream_);
+                             {pre_gamma, param_dtype}, {pre_beta, param_dtype}, pre_eps, (hipStream_t)stream_);
 }
 
 extern "C" int ptv3_scaled_add(const void* skip, int skip_dtype, const void* branch, int branch_dtype,
@@ -1279,17 +1360,21 @@ extern "C" int ptv3_scaled_add(const void* skip, int skip_dtype, const void* bra
 extern "C" int ptv3_add_layer_norm_bwd(const void* sum, int sum_dtype, const void* dy, int dy_dtype, const void* dsum,
                                        int dsum_dtype, const void* row_scale, int row_scale_dtype, const void* gamma,
                                        int param_dtype, int64_t n, int c, float eps, void* dskip, int dskip_dtype,
-                                       void* dbranch, int dbranch_dtype, float* dgamma, float* dbeta, void* stream_) {
+                                       void* dbranch, int dbranch_dtype, float* dgamma, float* dbeta, const void* pre_x,
+                                       int pre_x_dtype, const void* pre_gamma, float pre_eps, float* dpre_gamma,
+                                       float* dpre_beta, void* stream_) {
     if (n < 0 || c < 1) return PTV3_EINVAL;
     if (!ln_dtype_ok(sum_dtype) || !ln_dtype_ok(dy_dtype) || !ln_dtype_ok(dsum_dtype) || !ln_dtype_ok(row_scale_dtype) ||
-        !ln_dtype_ok(param_dtype) || !ln_dtype_ok(dskip_dtype) || !ln_dtype_ok(dbranch_dtype))
+        !ln_dtype_ok(param_dtype) || !ln_dtype_ok(dskip_dtype) || !ln_dtype_ok(dbranch_dtype) || !ln_dtype_ok(pre_x_dtype))
         return PTV3_EINVAL;
     if (!ln_channels_ok(c)) return PTV3_ESHAPE;
     if (n == 0) return PTV3_OK;
     if (!sum || !dy || !gamma || !dgamma || !dbeta) return PTV3_EINVAL;
+    if (pre_x && (!pre_gamma || !dpre_gamma || !dpre_beta)) return PTV3_EINVAL;
     return launch_add_ln_bwd({sum, sum_dtype}, {dy, dy_dtype}, {dsum, dsum_dtype}, {row_scale, row_scale_dtype},
                              {gamma, param_dtype}, n, c, eps, {dskip, dskip_dtype}, {dbranch, dbranch_dtype}, dgamma,
-                             dbeta, (hipStream_t)stream_);
+                             dbeta, {pre_x, pre_x_dtype}, {pre_gamma, param_dtype}, pre_eps, dpre_gamma, dpre_beta,
+                             (hipStream_t)stream_);
 }
 
 extern "C" int ptv3_batch_norm_stats(const void* x, int dtype, int64_t n, int c, float eps, float momentum,

@@ -437,8 +437,16 @@ class Block(PointModule):
         # precision first: the kernel writes them in that dtype (the same single rounding), the sums stay float
         normed_dtype = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else None
         skip = point.feat
-        point = self.cpe(point)
-        feat, point.feat = AddLayerNorm.apply(skip, point.feat, None, ln1.weight, ln1.bias, ln1.eps, normed_dtype)
+        conv, lin, ln_cpe = self.cpe[0], self.cpe[1], self.cpe[2]
+        if (type(lin) is nn.Linear and type(ln_cpe) is LayerNorm and ln_cpe.weight is not None
+                and ln_cpe.bias is not None and "sparse_conv_feat" in point):
+            # the xCPE's own norm rides on the kernel of the residual add and norm1 behind it
+            branch = ops.linear(conv(point.sparse_conv_feat).features, lin)
+            feat, point.feat = AddLayerNorm.apply(skip, branch, None, ln1.weight, ln1.bias, ln1.eps, normed_dtype,
+                                                  ln_cpe.weight, ln_cpe.bias, ln_cpe.eps)
+        else:
+            point = self.cpe(point)
+            feat, point.feat = AddLayerNorm.apply(skip, point.feat, None, ln1.weight, ln1.bias, ln1.eps, normed_dtype)
         point = self.attn(point)
         feat, point.feat = AddLayerNorm.apply(feat, point.feat, path_mask(point.feat), ln2.weight, ln2.bias, ln2.eps,
                                               normed_dtype)

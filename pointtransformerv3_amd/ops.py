@@ -916,10 +916,11 @@ def _code(t, fallback=0):
     return fallback if t is None else _DTYPE_CODE[t.dtype]
 
 
-def add_layer_norm(skip, branch, row_scale, weight, bias, eps, sum_dtype=None, out_dtype=None):
+def add_layer_norm(skip, branch, row_scale, weight, bias, eps, sum_dtype=None, out_dtype=None, pre=None):
     """(sum, y) with sum = skip + branch * row_scale and y = LayerNorm(sum), every tensor read and written in its
     own dtype. skip and row_scale (N,) or (N, 1) may be None; sum is returned as None when skip is None (then
-    y = LayerNorm(branch * row_scale)). sum_dtype defaults to the promoted dtype of skip and branch, out_dtype to it."""
+    y = LayerNorm(branch * row_scale)). sum_dtype defaults to the promoted dtype of skip and branch, out_dtype to it.
+    pre = (weight, bias, eps) of a LayerNorm the branch goes through first, in the same pass."""
     _dev(skip, branch, row_scale, weight, bias)
     lib = _lib.load()
     branch = branch.contiguous()
@@ -933,11 +934,47 @@ def add_layer_norm(skip, branch, row_scale, weight, bias, eps, sum_dtype=None, o
     y = torch.empty((n, c), dtype=out_dtype, device=branch.device)
     w = weight.contiguous()
     b = bias.to(w.dtype).contiguous()
+    pw = pb = None
+    if pre is not None:
+        pw, pb = pre[0].to(w.dtype).contiguous(), pre[1].to(w.dtype).contiguous()
     _lib.check(lib.ptv3_add_layer_norm_fwd(_ptr(skip), _code(skip), _ptr(branch), _code(branch), _ptr(row_scale),
                                            _code(row_scale), _ptr(w), _ptr(b), _code(w), n, c, float(eps), _ptr(total),
-                                           _DTYPE_CODE[sum_dtype], _ptr(y), _DTYPE_CODE[out_dtype], _stream()),
+                                           _DTYPE_CODE[sum_dtype], _ptr(y), _DTYPE_CODE[out_dtype], _ptr(pw), _ptr(pb),
+                                           float(pre[2]) if pre is not None else 0.0, _stream()),
                "ptv3_add_layer_norm_fwd")
     return total, y
+
+
+def add_layer_norm_bwd(total, dy, dsum, row_scale, weight, eps, skip_dtype=None, branch_dtype=None, pre=None):
+    """Backward of add_layer_norm: (dskip, dbranch, dweight, dbias); total is the sum the forward normalised, dsum
+    the gradient reaching it past the LayerNorm (or None). dskip / dbranch are made in the given dtypes and are
+    None where the dtype is None; dweight, dbias in fp32. pre = (x, weight, eps) of the LayerNorm the branch went
+    through first (x its input): dbranch is then x's gradient, and that norm's (dweight, dbias) are returned too."""
+    _dev(total, dy, dsum, row_scale, weight)
+    lib = _lib.load()
+    total, dy = total.contiguous(), dy.contiguous()
+    dsum = None if dsum is None else dsum.contiguous()
+    row_scale = None if row_scale is None else row_scale.reshape(-1).contiguous()
+    n, c = total.shape
+    dev = total.device
+    dskip = None if skip_dtype is None else torch.empty((n, c), dtype=skip_dtype, device=dev)
+    dbranch = None if branch_dtype is None else torch.empty((n, c), dtype=branch_dtype, device=dev)
+    dwb = torch.zeros((4 if pre is not None else 2, c), dtype=torch.float32, device=dev)
+    w = weight.contiguous()
+    px = pw = None
+    if pre is not None:
+        px, pw = pre[0].contiguous(), pre[1].to(w.dtype).contiguous()
+    _lib.check(lib.ptv3_add_layer_norm_bwd(_ptr(total), _code(total), _ptr(dy), _code(dy), _ptr(dsum), _code(dsum),
+                                           _ptr(row_scale), _code(row_scale), _ptr(w), _code(w), n, c, float(eps),
+                                           _ptr(dskip), _code(dskip), _ptr(dbranch), _code(dbranch), _ptr(dwb[0]),
+                                           _ptr(dwb[1]), _ptr(px), _code(px), _ptr(pw),
+                                           float(pre[2]) if pre is not None else 0.0,
+                                           _ptr(dwb[2]) if pre is not None else None,
+                                           _ptr(dwb[3]) if pre is not None else None, _stream()),
+               "ptv3_add_layer_norm_bwd")
+    if pre is not None:
+        return dskip, dbranch, dwb[0], dwb[1], dwb[2], dwb[3]
+    return dskip, dbranch, dwb[0], dwb[1]
 
 
 def scaled_add(skip, branch, row_scale, out_dtype):
@@ -953,28 +990,6 @@ def scaled_add(skip, branch, row_scale, out_dtype):
                                            _code(row_scale), n, c, _ptr(out), _DTYPE_CODE[out_dtype], _stream()),
                "ptv3_scaled_add")
     return out
-
-
-def add_layer_norm_bwd(total, dy, dsum, row_scale, weight, eps, skip_dtype=None, branch_dtype=None):
-    """Backward of add_layer_norm: (dskip, dbranch, dweight, dbias); total is the sum the forward normalised, dsum
-    the gradient reaching it past the LayerNorm (or None). dskip / dbranch are made in the given dtypes and are
-    None where the dtype is None; dweight, dbias in fp32."""
-    _dev(total, dy, dsum, row_scale, weight)
-    lib = _lib.load()
-    total, dy = total.contiguous(), dy.contiguous()
-    dsum = None if dsum is None else dsum.contiguous()
-    row_scale = None if row_scale is None else row_scale.reshape(-1).contiguous()
-    n, c = total.shape
-    dev = total.device
-    dskip = None if skip_dtype is None else torch.empty((n, c), dtype=skip_dtype, device=dev)
-    dbranch = None if branch_dtype is None else torch.empty((n, c), dtype=branch_dtype, device=dev)
-    dwb = torch.zeros((2, c), dtype=torch.float32, device=dev)
-    w = weight.contiguous()
-    _lib.check(lib.ptv3_add_layer_norm_bwd(_ptr(total), _code(total), _ptr(dy), _code(dy), _ptr(dsum), _code(dsum),
-                                           _ptr(row_scale), _code(row_scale), _ptr(w), _code(w), n, c, float(eps),
-                                           _ptr(dskip), _code(dskip), _ptr(dbranch), _code(dbranch), _ptr(dwb[0]),
-                                           _ptr(dwb[1]), _stream()), "ptv3_add_layer_norm_bwd")
-    return dskip, dbranch, dwb[0], dwb[1]
 
 
 LINEAR_LN_CHANNELS = (128, 256)   # square Linear + LayerNorm(s) + residual in one kernel

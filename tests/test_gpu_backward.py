@@ -644,3 +644,35 @@ def test_conv_weight_gradient_from_pair_lists(dtype, cin, cout, ks):
     dw_a, db_a = o.subm_conv_wgrad(x, dy, nbr, with_bias=True)
     dw_b, db_b = o.subm_conv_wgrad_pairs(x, dy, plan, with_bias=True)
     assert rel_err(dw_b, dw_a.cpu()) < 1e-5 and rel_err(db_b, db_a.cpu()) < 1e-5
+
+
+@pytest.mark.parametrize("with_mask", [False, True])
+@pytest.mark.parametrize("c", [32, 64, 128, 256, 512])
+@pytest.mark.parametrize("skip_dtype,branch_dtype", [(torch.float32, torch.bfloat16), (torch.float32, torch.float32),
+                                                     (torch.float16, torch.float16)])
+def test_add_layer_norm_with_the_branch_norm_in_front(skip_dtype, branch_dtype, with_mask, c):
+    """s = skip + LayerNorm_pre(branch) * mask, y = LayerNorm(s) as one node (the xCPE's norm, the first residual
+    connection of a Block and norm1, model.py:546-554, :589-592): both results and all six gradients against
+    torch CPU autograd in float32, with a gradient arriving at the sum as well."""
+    from pointtransformerv3_amd.autograd import AddLayerNorm
+    n = 1501 if c >= 256 else 3001
+    g = torch.Generator().manual_seed(c)
+    skip = torch.randn(n, c, generator=g).to(skip_dtype)
+    branch = (torch.randn(n, c, generator=g) * 2 + 0.5).to(branch_dtype)
+    mask = ((torch.rand(n, 1, generator=g) < 0.7).float() / 0.7).to(branch_dtype) if with_mask else None
+    w, pw = torch.rand(c, generator=g) + 0.5, torch.rand(c, generator=g) + 0.5
+    b, pb = torch.randn(c, generator=g), torch.randn(c, generator=g)
+    ds, dy = torch.randn(n, c, generator=g), torch.randn(n, c, generator=g)
+    ref = [t.float().clone().requires_grad_(True) for t in (skip, branch, w, b, pw, pb)]
+    pre = torch.nn.functional.layer_norm(ref[1], (c,), ref[4], ref[5], 1e-6)
+    s_want = ref[0] + pre * (mask.float() if with_mask else 1.0)
+    y_want = torch.nn.functional.layer_norm(s_want, (c,), ref[2], ref[3], 1e-5)
+    torch.autograd.backward([s_want, y_want], [ds, dy])
+    got = [t.detach().to(DEV).requires_grad_(True) for t in (skip, branch, w, b, pw, pb)]
+    s_got, y_got = AddLayerNorm.apply(got[0], got[1], None if mask is None else mask.to(DEV), got[2], got[3], 1e-5, None,
+                                      got[4], got[5], 1e-6)
+    torch.autograd.backward([s_got, y_got], [ds.to(DEV).to(s_got.dtype), dy.to(DEV).to(y_got.dtype)])
+    tol = TOL[torch.promote_types(skip_dtype, branch_dtype)]
+    assert rel_err(s_got, s_want) < tol and rel_err(y_got, y_want) < tol
+    for i, name in enumerate(["skip", "branch", "weight", "bias", "pre_weight", "pre_bias"]):
+        assert rel_err(got[i].grad, ref[i].grad) < (TOL[branch_dtype] if i == 1 else tol), name
