@@ -220,6 +220,23 @@ class AddLayerNorm(torch.autograd.Function):
         return dskip, dbranch, None, dw.to(weight.dtype), db.to(bias_dtype), None, None, dpw, dpb, None
 
 
+class SplitCast(torch.autograd.Function):
+    """(x, x in half precision) for a float x with two readers, one of which reads halves (the residual stream at
+    the head of a Block: the skip connection and the xCPE convolution under autocast, model.py:589-592). Going
+    back, the float and the half-precision gradient are added by one kernel instead of a conversion followed
+    by autograd's accumulation."""
+
+    @staticmethod
+    def forward(ctx, x, dtype):
+        return x.view_as(x), x.to(dtype)
+
+    @staticmethod
+    def backward(ctx, dx, dhalf):
+        if dx is None or dhalf is None:
+            return (dx if dhalf is None else dhalf.to(torch.float32)), None
+        return ops.scaled_add(dx, dhalf, None, dx.dtype), None
+
+
 class ResidualAdd(torch.autograd.Function):
     """skip + branch * mask (model.py:602-604 with the stochastic-depth factor per row) in skip's dtype, the
     branch read in its own; going back skip's gradient is the incoming one as it is and the branch's one

@@ -11,7 +11,8 @@ import torch
 import torch.nn as nn
 
 from . import ops
-from .autograd import AddLayerNorm, BatchNormAct, LayerNorm as LayerNormFn, ResidualAdd, SegmentReduce, UnpoolAdd
+from .autograd import (AddLayerNorm, BatchNormAct, LayerNorm as LayerNormFn, ResidualAdd, SegmentReduce, SplitCast,
+                       UnpoolAdd)
 from .point import AttrDict, Point, offset2bincount
 from .sparse import SparseConvTensor, SubMConv3d, is_spconv_module
 
@@ -441,7 +442,12 @@ class Block(PointModule):
         if (type(lin) is nn.Linear and type(ln_cpe) is LayerNorm and ln_cpe.weight is not None
                 and ln_cpe.bias is not None and "sparse_conv_feat" in point):
             # the xCPE's own norm rides on the kernel of the residual add and norm1 behind it
-            branch = ops.linear(conv(point.sparse_conv_feat).features, lin)
+            sparse = point.sparse_conv_feat
+            if (normed_dtype is not None and skip.dtype == torch.float32 and skip.requires_grad
+                    and self.channels % 8 == 0 and sparse.features is skip):
+                skip, half = SplitCast.apply(skip, normed_dtype)   # one kernel adds the two gradients going back
+                sparse = sparse.replace_feature(half)
+            branch = ops.linear(conv(sparse).features, lin)
             feat, point.feat = AddLayerNorm.apply(skip, branch, None, ln1.weight, ln1.bias, ln1.eps, normed_dtype,
                                                   ln_cpe.weight, ln_cpe.bias, ln_cpe.eps)
         else:
