@@ -194,12 +194,15 @@ class AddLayerNorm(torch.autograd.Function):
     (s, y), y in out_dtype; the backward kernel adds the gradient arriving at s to the LayerNorm's own, so
     autograd has nothing to accumulate, and writes each input's gradient in that input's dtype.
     With pre_weight, pre_bias, pre_eps the branch first goes through a LayerNorm of its own in the same pass
-    (s = skip + LayerNorm_pre(branch) * mask: the xCPE's norm, model.py:546-554)."""
+    (s = skip + LayerNorm_pre(branch) * mask: the xCPE's norm, model.py:546-554); sum_dtype then says what that
+    norm's result would have been added in (float under autocast, which runs layer_norm in float)."""
 
     @staticmethod
-    def forward(ctx, skip, branch, mask, weight, bias, eps, out_dtype=None, pre_weight=None, pre_bias=None, pre_eps=0.0):
+    def forward(ctx, skip, branch, mask, weight, bias, eps, out_dtype=None, pre_weight=None, pre_bias=None, pre_eps=0.0,
+                sum_dtype=None):
         pre = None if pre_weight is None else (pre_weight.detach(), pre_bias.detach(), pre_eps)
-        s, y = ops.add_layer_norm(skip, branch, mask, weight.detach(), bias.detach(), eps, out_dtype=out_dtype, pre=pre)
+        s, y = ops.add_layer_norm(skip, branch, mask, weight.detach(), bias.detach(), eps, sum_dtype=sum_dtype,
+                                  out_dtype=out_dtype, pre=pre)
         ctx.save_for_backward(s, weight, mask, *(() if pre is None else (branch, pre_weight)))
         ctx.eps, ctx.pre_eps, ctx.dtypes = eps, pre_eps, (skip.dtype, branch.dtype, bias.dtype)
         ctx.pre_bias_dtype = None if pre is None else pre_bias.dtype
@@ -217,7 +220,7 @@ class AddLayerNorm(torch.autograd.Function):
         dpw = dpb = None
         if pre is not None:
             dpw, dpb = out[4].to(rest[1].dtype), out[5].to(ctx.pre_bias_dtype)
-        return dskip, dbranch, None, dw.to(weight.dtype), db.to(bias_dtype), None, None, dpw, dpb, None
+        return dskip, dbranch, None, dw.to(weight.dtype), db.to(bias_dtype), None, None, dpw, dpb, None, None
 
 
 class SplitCast(torch.autograd.Function):

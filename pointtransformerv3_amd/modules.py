@@ -448,8 +448,10 @@ class Block(PointModule):
                 skip, half = SplitCast.apply(skip, normed_dtype)   # one kernel adds the two gradients going back
                 sparse = sparse.replace_feature(half)
             branch = ops.linear(conv(sparse).features, lin)
+            # autocast's layer_norm hands out float, so the sum (the residual stream from here on) is float
             feat, point.feat = AddLayerNorm.apply(skip, branch, None, ln1.weight, ln1.bias, ln1.eps, normed_dtype,
-                                                  ln_cpe.weight, ln_cpe.bias, ln_cpe.eps)
+                                                  ln_cpe.weight, ln_cpe.bias, ln_cpe.eps,
+                                                  torch.float32 if normed_dtype is not None else None)
         else:
             point = self.cpe(point)
             feat, point.feat = AddLayerNorm.apply(skip, point.feat, None, ln1.weight, ln1.bias, ln1.eps, normed_dtype)
