@@ -24,7 +24,11 @@ DEFAULTS = dict(
     order=("z", "z-trans", "hilbert", "hilbert-trans"), stride=(2, 2, 2, 2),
     enc_depths=(2, 2, 2, 6, 2), enc_channels=(32, 64, 128, 256, 512), enc_num_head=(2, 4, 8, 16, 32),
     enc_patch_size=(1024,) * 5, dec_depths=(2, 2, 2, 2), dec_channels=(64, 64, 128, 256),
-    dec_num_head=(4, 4, 8, 16), dec_patch_size=(1024,) * 4, cls_mode=False, enable_flash=True)
+    dec_num_head=(4, 4, 8, 16), dec_patch_size=(1024,) * 4, cls_mode=False, enable_flash=True,
+    # model.py:477 hands flash_attn qkv.half() and gets fp16 back whatever the model's dtype: True restates that
+    # rounding (what the reference computes in a float model); False keeps float throughout (what a float
+    # model computes here, and what half-precision runs are compared with)
+    flash_half=False)
 
 
 def _linear(sd, name, x):
@@ -57,13 +61,24 @@ def _attention(sd, name, level, x, heads, patch, order_index):
     if not level["flash"]:
         # without the fused path the patch shrinks to the smallest scene (model.py:441-444)
         patch = min(int(OI.offset2bincount(level["offset"]).min()), patch)
-    key = ("pad", patch)
-    if key not in level:
-        level[key] = OI.padding_tables(level["offset"], patch)
-    pad, unpad, cu = level[key]
+    # the tables are made by the first block that reaches this Point and kept under fixed keys (model.py:384-391):
+    # decoder blocks of a stage run on the tables its encoder blocks made, whatever their own patch size
+    if "pad" not in level:
+        level["pad"] = (patch, OI.padding_tables(level["offset"], patch))
+    built_for, (pad, unpad, cu) = level["pad"]
+    if level["flash"]:
+        # flash_attn takes the patch as max_seqlen (model.py:479): sequences longer than that are outside its contract
+        assert built_for <= patch, f"cached patches of {built_for} points exceed this block's patch size {patch}"
+    else:
+        # model.py:461 reshapes the cached padded rows into patches of the current size
+        assert built_for == patch, "patch sizes that differ within a stage are not restated for the non-fused path"
     qkv = _linear(sd, name + ".qkv", x)
+    if level["flash"] and level["flash_half"]:
+        qkv = qkv.half().float()                                                  # model.py:477
     out = OF.serialized_attention_core(qkv, level["order"][order_index], level["inverse"][order_index],
                                        pad, unpad, cu, heads, rpe=rpe)
+    if level["flash"] and level["flash_half"]:
+        out = out.half().float()                    # flash_attn returns fp16, model.py:483 casts it back
     return _linear(sd, name + ".proj", out)
 
 
@@ -95,7 +110,7 @@ def _pool(sd, name, parent, perm, stride=2):
     return dict(feat=feat, sparse_feat=feat, grid_coord=pc["grid_coord"], batch=pc["batch"],
                 offset=OI.batch2offset(pc["batch"]), code=code, order=order, inverse=inverse,
                 depth=parent["depth"] - pooling_depth, kmaps={}, cluster=pc["cluster"], parent=parent,
-                flash=parent["flash"])
+                flash=parent["flash"], flash_half=parent["flash_half"])
 
 
 def _unpool(sd, name, child):
@@ -129,7 +144,8 @@ def ptv3_forward(state_dict, grid_coord, feat, offset, perms=None, trace=None, *
         code, order, inverse = code[perms[0]], order[perms[0]], inverse[perms[0]]
     x = torch.as_tensor(feat).float()
     level = dict(feat=x, sparse_feat=x, grid_coord=grid_coord, batch=batch, offset=offset, code=code,
-                 order=order, inverse=inverse, depth=depth, kmaps={}, flash=bool(cfg["enable_flash"]))
+                 order=order, inverse=inverse, depth=depth, kmaps={}, flash=bool(cfg["enable_flash"]),
+                 flash_half=bool(cfg["flash_half"]))
 
     # stem (model.py:766-779): 5x5x5 conv without bias, BN, GELU
     y = OF.subm_conv(x, _kmap(level, 5), sd["embedding.stem.conv.weight"], None)

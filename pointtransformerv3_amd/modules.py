@@ -11,6 +11,7 @@ import torch
 import torch.nn as nn
 
 from . import ops
+from ._lib import Ptv3Error
 from .autograd import (AddLayerNorm, BatchNormAct, LayerNorm as LayerNormFn, ResidualAdd, SegmentReduce, SplitCast,
                        UnpoolAdd)
 from .point import AttrDict, Point, offset2bincount
@@ -256,7 +257,29 @@ class SerializedAttention(PointModule):
         if not {"pad", "unpad", "cu_seqlens_key"}.issubset(point.keys()):
             pad, unpad, cu = ops.pad_index(point.offset, point.offset_host(), self.patch_size)
             point["pad"], point["unpad"], point["cu_seqlens_key"] = pad, unpad, cu
+            point["_pad_patch"] = self.patch_size
         return point["pad"], point["unpad"], point["cu_seqlens_key"]
+
+    def _cached_patch(self, point):
+        """Longest sequence of the padding tables cached on the Point. The first attention layer that
+        reaches a Point makes them and every later one reuses them under the same keys (model.py:384-391),
+        so the decoder blocks of a stage attend over the patches its encoder blocks defined. The kernels size
+        their staging from this value, never from the layer's own patch size."""
+        built_for = point.get("_pad_patch")
+        if built_for is None:   # tables put on the Point by the caller: measure them
+            cu = point["cu_seqlens_key"]
+            built_for = int((cu[1:] - cu[:-1]).max()) if cu.numel() > 1 else 0
+            point["_pad_patch"] = built_for
+        if self.enable_flash and built_for > self.patch_size:
+            # the reference would hand flash_attn sequences longer than its max_seqlen (model.py:479)
+            raise Ptv3Error(f"the padding tables cached on this Point hold patches of {built_for} points, more than "
+                            f"this layer's patch_size {self.patch_size}: undefined in the reference; use patch "
+                            f"sizes that do not shrink from the encoder to the decoder of a stage")
+        if not self.enable_flash and built_for != self.patch_size:
+            # model.py:461 would reshape rows padded for one patch size into patches of another
+            raise Ptv3Error(f"the padding tables cached on this Point were made for patches of {built_for} points, "
+                            f"this layer wants {self.patch_size}: not supported without the fused path")
+        return built_for
 
     @torch.no_grad()
     def _slots(self, point):
@@ -274,6 +297,7 @@ class SerializedAttention(PointModule):
             sizes = offset2bincount(torch.as_tensor(point.offset_host()))
             self.patch_size = min(int(sizes.min()), self.patch_size_max)
         _, _, cu_seqlens = self.get_padding_and_inverse(point)
+        max_seqlen = self._cached_patch(point)
         slot_src, slot_dst = self._slots(point)
         grad = ops.wants_grad(qkv, self.rpe.rpe_table if self.enable_rpe else None)
         drop_p = self.attn_drop if self.training else 0.0
@@ -282,34 +306,34 @@ class SerializedAttention(PointModule):
             seed = int(torch.randint(0, 2 ** 31 - 1, (1,)).item())   # torch's CPU generator: follows torch.manual_seed
             if self.enable_rpe:
                 out = PatchAttentionRpe.apply(qkv.float(), self.rpe.rpe_table, self.num_heads, slot_src, slot_dst,
-                                              cu_seqlens, self.patch_size, self.scale, point.grid_coord,
+                                              cu_seqlens, max_seqlen, self.scale, point.grid_coord,
                                               self.rpe.pos_bnd, drop_p, seed)
                 return out.to(qkv.dtype)
             half = qkv.half() if (self.enable_flash and qkv.dtype == torch.float32) else qkv
-            return PatchAttention.apply(half, self.num_heads, slot_src, slot_dst, cu_seqlens, self.patch_size,
+            return PatchAttention.apply(half, self.num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen,
                                         self.scale, drop_p, seed).to(qkv.dtype)
         if grad and self.enable_rpe:
             from .autograd import PatchAttentionRpe
             out = PatchAttentionRpe.apply(qkv.float(), self.rpe.rpe_table, self.num_heads, slot_src, slot_dst, cu_seqlens,
-                                          self.patch_size, self.scale, point.grid_coord, self.rpe.pos_bnd)
+                                          max_seqlen, self.scale, point.grid_coord, self.rpe.pos_bnd)
             return out.to(qkv.dtype)
         if grad:
             from .autograd import PatchAttention
             half = qkv.half() if (self.enable_flash and qkv.dtype == torch.float32) else qkv
-            return PatchAttention.apply(half, self.num_heads, slot_src, slot_dst, cu_seqlens, self.patch_size,
+            return PatchAttention.apply(half, self.num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen,
                                         self.scale).to(qkv.dtype)
         if self.enable_rpe:
             # bias from the grid offsets of (query, key) inside the patch, added before the softmax; the
             # reference takes this path in float (upcast_attention / upcast_softmax, model.py:463-471)
-            out = ops.patch_attention_rpe(qkv.float(), self.num_heads, slot_src, slot_dst, cu_seqlens, self.patch_size,
+            out = ops.patch_attention_rpe(qkv.float(), self.num_heads, slot_src, slot_dst, cu_seqlens, max_seqlen,
                                           self.scale, point.grid_coord, self.rpe.rpe_table, self.rpe.pos_bnd)
             return out.to(qkv.dtype)
         if self.enable_flash and qkv.dtype == torch.float32:
             # the fused path of the reference always computes in half precision (model.py:477,483)
             return ops.patch_attention(qkv.half(), self.num_heads, slot_src, slot_dst, cu_seqlens,
-                                       self.patch_size, self.scale).to(qkv.dtype)
+                                       max_seqlen, self.scale).to(qkv.dtype)
         return ops.patch_attention(qkv, self.num_heads, slot_src, slot_dst, cu_seqlens,
-                                   self.patch_size, self.scale)
+                                   max_seqlen, self.scale)
 
     def forward(self, point):
         feat = self.attend(point, ops.linear(point.feat, self.qkv))
