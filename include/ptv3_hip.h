@@ -28,6 +28,7 @@ extern "C" {
 #define PTV3_EDEPTH (-2)    /* depth outside 1..16 or code wider than 63 bits (model.py:103,108) */
 #define PTV3_EWORKSPACE (-3) /* workspace smaller than *_workspace_bytes says */
 #define PTV3_ESHAPE (-4)    /* channel / head / patch shape the kernels do not cover */
+#define PTV3_ESTATIC (-5)   /* input larger than the fixed on-device buffer of a *_static entry point */
 
 #define PTV3_F32 0
 #define PTV3_F16 1
@@ -278,6 +279,19 @@ int ptv3_pool_clusters(const int64_t *code0, const int64_t *order0, int64_t n, i
                        const int64_t *offset, int n_scenes, int64_t *cluster, int64_t *idx_ptr,
                        int64_t *head, int64_t *n_clusters, void *workspace, size_t workspace_bytes,
                        void *stream);
+
+/* ptv3_pool_clusters for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. Same outputs as
+ * ptv3_pool_clusters, bit for bit, and no workspace argument: the per-block cluster counts live in a fixed
+ * 256 KiB array inside the library's device code, one copy per GPU, held until the process ends. Nothing is
+ * allocated or freed, here or in a library underneath; the first call on a GPU looks the array's device
+ * address up once. n <= ptv3_pool_clusters_static_max_points() = 16,777,216, else PTV3_ESTATIC. The stream
+ * must belong to the current device. All calls on one GPU share the array: calls that overlap on one GPU
+ * (different streams, or different threads) race on it -- serialise them; calls on one stream are ordered. */
+int64_t ptv3_pool_clusters_static_max_points(void);
+int ptv3_pool_clusters_static(const int64_t *code0, const int64_t *order0, int64_t n, int shift,
+                              const int64_t *offset, int n_scenes, int64_t *cluster, int64_t *idx_ptr,
+                              int64_t *head, int64_t *n_clusters, void *stream);
 
 /* model.py:666-674,690,695 once the cluster count m is known on the host: pooled codes
  * (k,m) = code[:, head] >> shift, pooled grid_coord (m,3) = grid_coord[head] >> pool_depth,

@@ -59,6 +59,8 @@ SIGNATURES = {
                                         _i32, _vp, _vp, _vp]),
     "ptv3_pool_clusters_workspace_bytes": (_sz, [_i64]),
     "ptv3_pool_clusters": (_i32, [_vp, _vp, _i64, _i32, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "ptv3_pool_clusters_static_max_points": (_i64, []),
+    "ptv3_pool_clusters_static": (_i32, [_vp, _vp, _i64, _i32, _vp, _i32, _vp, _vp, _vp, _vp, _vp]),
     "ptv3_pool_gather": (_i32, [_vp, _i64, _i32, _i32, _vp, _i32, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp,
                                 _vp]),
     "ptv3_pool_orders_workspace_bytes": (_sz, [_i64, _i32]),

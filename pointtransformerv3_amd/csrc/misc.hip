@@ -10,6 +10,7 @@ extern "C" const char* ptv3_strerror(int rc) {
         case PTV3_EDEPTH: return "depth outside 1..16 or code wider than 63 bits";
         case PTV3_EWORKSPACE: return "workspace too small";
         case PTV3_ESHAPE: return "shape not covered by the kernels";
+        case PTV3_ESTATIC: return "input larger than the fixed on-device buffer of this entry point";
         default: return rc > 0 ? hipGetErrorString((hipError_t)rc) : "unknown error";
     }
 }

@@ -7,6 +7,8 @@
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 
+#include <mutex>
+
 #include "common.h"
 
 namespace {
@@ -292,17 +294,21 @@ extern "C" size_t ptv3_pool_clusters_workspace_bytes(int64_t n) {
     return ptv3_align256((size_t)(ptv3_ceil_div(n > 0 ? n : 1, PB)) * sizeof(uint32_t));
 }
 
-extern "C" int ptv3_pool_clusters(const int64_t* code0, const int64_t* order0, int64_t n, int shift,
-                                  const int64_t* offset, int n_scenes, int64_t* cluster, int64_t* idx_ptr,
-                                  int64_t* head, int64_t* n_clusters, void* workspace, size_t workspace_bytes,
-                                  void* stream_) {
-    if (n < 1 || n >= (1ll << 31) || shift < 0 || shift > 62 || n_scenes < 0) return PTV3_EINVAL;
-    if (n_scenes > 0 && !offset) return PTV3_EINVAL;
-    if (!code0 || !order0 || !cluster || !idx_ptr || !head || !n_clusters || !workspace) return PTV3_EINVAL;
-    if (workspace_bytes < ptv3_pool_clusters_workspace_bytes(n)) return PTV3_EWORKSPACE;
-    hipStream_t stream = (hipStream_t)stream_;
+// Per-block cluster counts of ptv3_pool_clusters_static: device memory that belongs to the library's code
+// object, one copy per GPU, held until the process ends. 65,536 blocks of 256 points = 256 KiB.
+static constexpr int64_t STATIC_MAX_POINTS = (int64_t)1 << 24;
+static __device__ __align__(256) uint32_t scratch[STATIC_MAX_POINTS / 256];
+
+namespace {
+
+static_assert(PB == 256, "scratch is sized for 256-point blocks");
+
+int launch_pool_clusters(const int64_t* code0, const int64_t* order0, int64_t n, int shift, const int64_t* offset,
+                         int n_scenes, int64_t* cluster, int64_t* idx_ptr, int64_t* head, int64_t* n_clusters,
+                         uint32_t* block_cnt, hipStream_t stream) {
     const int64_t blocks = ptv3_ceil_div(n, PB);
-    uint32_t* block_cnt = (uint32_t*)workspace;
+    // every one of the `blocks` counts is written by the first kernel before the second reads it: the buffer
+    // needs no clearing, whatever an earlier call left in it
     hipLaunchKernelGGL(cluster_count_kernel, dim3((unsigned)blocks), dim3(PB), 0, stream, code0, order0, n,
                        shift, block_cnt);
     hipLaunchKernelGGL(cluster_scan_kernel, dim3(1), dim3(PB), 0, stream, block_cnt, blocks, n_clusters);
@@ -312,6 +318,59 @@ extern "C" int ptv3_pool_clusters(const int64_t* code0, const int64_t* order0, i
         hipLaunchKernelGGL(pool_offsets_kernel, dim3((unsigned)ptv3_ceil_div(n_scenes, 256)), dim3(256), 0, stream,
                            offset, n_scenes, order0, (const int64_t*)cluster, n_clusters + 1);
     PTV3_RETURN_LAUNCH();
+}
+
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mutex;
+uint32_t* scratch_ptr[MAX_DEVICES];   // device address of `scratch` on each GPU, looked up on first use
+
+// The array's name is a host-side handle, not an address a kernel can use: its address on the current device
+// comes from the runtime, once per device.
+int static_scratch(uint32_t** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= MAX_DEVICES) return PTV3_EINVAL;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return PTV3_EINVAL;
+        scratch_ptr[dev] = (uint32_t*)p;
+    }
+    *out = scratch_ptr[dev];
+    return PTV3_OK;
+}
+
+}  // namespace
+
+extern "C" int ptv3_pool_clusters(const int64_t* code0, const int64_t* order0, int64_t n, int shift,
+                                  const int64_t* offset, int n_scenes, int64_t* cluster, int64_t* idx_ptr,
+                                  int64_t* head, int64_t* n_clusters, void* workspace, size_t workspace_bytes,
+                                  void* stream_) {
+    if (n < 1 || n >= (1ll << 31) || shift < 0 || shift > 62 || n_scenes < 0) return PTV3_EINVAL;
+    if (n_scenes > 0 && !offset) return PTV3_EINVAL;
+    if (!code0 || !order0 || !cluster || !idx_ptr || !head || !n_clusters || !workspace) return PTV3_EINVAL;
+    if (workspace_bytes < ptv3_pool_clusters_workspace_bytes(n)) return PTV3_EWORKSPACE;
+    return launch_pool_clusters(code0, order0, n, shift, offset, n_scenes, cluster, idx_ptr, head, n_clusters,
+                                (uint32_t*)workspace, (hipStream_t)stream_);
+}
+
+extern "C" int64_t ptv3_pool_clusters_static_max_points(void) { return STATIC_MAX_POINTS; }
+
+extern "C" int ptv3_pool_clusters_static(const int64_t* code0, const int64_t* order0, int64_t n, int shift,
+                                         const int64_t* offset, int n_scenes, int64_t* cluster, int64_t* idx_ptr,
+                                         int64_t* head, int64_t* n_clusters, void* stream_) {
+    if (n < 1 || shift < 0 || shift > 62 || n_scenes < 0) return PTV3_EINVAL;
+    if (n > STATIC_MAX_POINTS) return PTV3_ESTATIC;
+    if (n_scenes > 0 && !offset) return PTV3_EINVAL;
+    if (!code0 || !order0 || !cluster || !idx_ptr || !head || !n_clusters) return PTV3_EINVAL;
+    uint32_t* block_cnt = nullptr;
+    const int rc = static_scratch(&block_cnt);
+    if (rc != PTV3_OK) return rc;
+    return launch_pool_clusters(code0, order0, n, shift, offset, n_scenes, cluster, idx_ptr, head, n_clusters,
+                                block_cnt, (hipStream_t)stream_);
 }
 
 extern "C" int ptv3_pool_gather(const int64_t* code, int64_t n, int k, int shift,

@@ -98,3 +98,13 @@ def test_ops_reject_cpu_tensors():
         ops.encode_orders(torch.zeros(4, 3, dtype=torch.int32), None, 8, ["z"])
     with pytest.raises(_lib.Ptv3Error):
         ops.kmap_build(torch.zeros(4, 4, dtype=torch.int32), 3)
+
+
+def test_static_entry_point_refuses_more_points_than_its_buffer_holds():
+    """The size check comes before anything touches a device."""
+    from pointtransformerv3_amd import _lib
+    lib = _lib.load()
+    limit = lib.ptv3_pool_clusters_static_max_points()
+    assert limit == 1 << 24
+    rc = lib.ptv3_pool_clusters_static(None, None, limit + 1, 3, None, 0, None, None, None, None, None)
+    assert rc == -5 and b"fixed" in lib.ptv3_strerror(rc)
