@@ -69,6 +69,18 @@ def room_voxels(n_voxels, seed, grid_size=0.02):
         n_draw = int(n_draw * 1.3)
 
 
+def cube_scene(n_voxels, seed, grid_size=0.02, side=5.0):
+    """Exactly `n_voxels` unique voxels of points uniform in a cube of `side` metres (a volume, not a
+    surface: the plumbing case of the CPU-runnable baseline configuration)."""
+    rng = np.random.default_rng(seed)
+    pts = rng.random((int(n_voxels * 1.05) + 64, 3)) * side
+    while True:
+        g, keep = voxelize_unique(pts, grid_size)
+        if len(g) >= n_voxels:
+            return dict(coord=pts[keep][:n_voxels].astype(np.float32), grid_coord=g[:n_voxels])
+        pts = np.concatenate([pts, rng.random((n_voxels, 3)) * side])
+
+
 def lidar_scene(seed, grid_size=0.05, beams=64, az_step_deg=0.2, max_range=75.0, n_boxes=30):
     """One spinning-LiDAR sweep: `beams` elevations in [-25,+3] deg, azimuth step 0.2 deg
     (115,200 rays), cast against the ground plane z=-1.8 m, random boxes (vehicles, buildings) and

@@ -71,30 +71,78 @@ def test_attention_config1_shape_fp32():
     assert rel_err(got, want) < 1e-4
 
 
-def test_attention_config2_shape_bf16_sampled():
-    # one 100k-point scene, C=512, 32 heads, bf16, q/k/v ~ N(0,1)/4; the oracle checks a
-    # sample of patches (first, middle, last-with-fillers), every head
-    n, patch, heads, C = 100_000, 1024, 32, 512
-    rng = np.random.default_rng(2)
-    g = torch.Generator().manual_seed(2)
-    order = rng.permutation(n).astype(np.int64)
-    inverse = np.empty(n, np.int64)
-    inverse[order] = np.arange(n)
-    qkv = (torch.randn(n, 3 * C, generator=g) / 4).to(torch.bfloat16)
-    pad, unpad, cu = OI.padding_tables([n], patch)
+def test_baseline_config1_serialization_then_one_attention_block_fp32():
+    """Baseline configuration 1 as written: 16,384 points uniform in a 5 m cube at grid 0.02 m; z-order and
+    Hilbert codes and orders at the adaptive depth (8) and at depth 16, bit-exact; then one SerializedAttention
+    (patch 1024, C = 64, 4 heads, seeded weights) on the CPU reference path -- no fused attention, fp32."""
+    from oracle import serialization as OS
+    from pointtransformerv3_amd import Point, synthetic
+    from pointtransformerv3_amd.modules import SerializedAttention
+    sc = synthetic.cube_scene(16_384, 1000, 0.02)
+    grid = sc["grid_coord"]
+    n = len(grid)
+    assert n == 16_384 and int(grid.max()).bit_length() == 8
+    offset = np.array([n], np.int64)
+    batch = np.zeros(n, np.int64)
+    orders = ["z", "hilbert"]
+    points = {}
+    for depth in (None, 16):
+        p = Point(grid_coord=torch.from_numpy(grid).to(DEV), offset=torch.from_numpy(offset).to(DEV),
+                  feat=torch.zeros(n, 1, device=DEV))
+        p.serialization(order=orders, depth=depth)
+        want_depth, code, order, inverse = OS.serialize(grid, batch, orders, depth=depth)
+        assert p.serialized_depth == want_depth == (8 if depth is None else 16)
+        assert np.array_equal(p.serialized_code.cpu().numpy(), code)
+        assert np.array_equal(p.serialized_order.cpu().numpy(), order)
+        assert np.array_equal(p.serialized_inverse.cpu().numpy(), inverse)
+        points[depth] = (p, order, inverse)
+    # the block: Linear -> patch attention along the Hilbert order -> Linear
+    C, heads, patch = 64, 4, 1024
+    torch.manual_seed(1001)
+    attn = SerializedAttention(C, heads, patch_size=patch, order_index=1, enable_flash=False).eval()
+    sd = {k: v.clone() for k, v in attn.state_dict().items()}
+    feat = torch.randn(n, C, generator=torch.Generator().manual_seed(1002))
+    p, order, inverse = points[16]
+    p.feat = feat.to(DEV)
+    with torch.inference_mode():
+        got = attn.to(DEV)(p).feat
+    assert attn.patch_size == patch and got.dtype == torch.float32
+    pad, unpad, cu = OI.padding_tables(offset, patch)
+    assert len(cu) == 17
+    qkv = torch.nn.functional.linear(feat, sd["qkv.weight"], sd["qkv.bias"])
+    core = OF.serialized_attention_core(qkv, order[1], inverse[1], pad, unpad, cu, heads)
+    want = torch.nn.functional.linear(core, sd["proj.weight"], sd["proj.bias"])
+    assert rel_err(got, want) < 1e-4
+
+
+def test_baseline_config2_attention_bf16_every_patch():
+    """Baseline configuration 2 as written: one room scene of ~100k voxelised points at 2 cm, its Hilbert order
+    (adaptive depth), patch 1024, C = 512, 32 heads, q/k/v ~ N(0,1)/4 in bf16. Every patch and head is checked,
+    the borrowed tail patch included."""
+    from pointtransformerv3_amd import synthetic
+    sc = synthetic.room_scene(106_000, 2000, 0.02)
+    grid = sc["grid_coord"]
+    n, patch, heads, C = len(grid), 1024, 32, 512
+    assert 95_000 < n < 106_000 and n % patch != 0
     o = ops()
+    depth = int(grid.max()).bit_length()
+    code = o.encode_orders(to_dev(grid), torch.zeros(n, dtype=torch.int64, device=DEV), depth, ["hilbert"])
+    order_d, inverse_d = o.argsort_rows(code, 3 * depth + 1)
+    order, inverse = order_d[0].cpu().numpy(), inverse_d[0].cpu().numpy()
+    from oracle import serialization as OS
+    assert np.array_equal(order, OS.serialize(grid, np.zeros(n, np.int64), ["hilbert"])[2][0])
+    qkv = (torch.randn(n, 3 * C, generator=torch.Generator().manual_seed(2)) / 4).to(torch.bfloat16)
+    pad, unpad, cu = OI.padding_tables([n], patch)
+    assert len(cu) - 1 == -(-n // patch) and len(pad) == (len(cu) - 1) * patch
     gp, gu, gc = o.pad_index(to_dev(np.array([n])), [n], patch)
-    src, dst = o.attn_slots(to_dev(order), to_dev(inverse), gp, gu)
-    got = o.patch_attention(qkv.to(DEV), heads, src, dst, gc, patch, 0.25).float().cpu()
-    assert torch.isfinite(got).all()
-    rows = order[pad]
-    for p in (0, 48, 96, 97):
-        s, e = int(cu[p]), int(cu[p + 1])
-        want = OF.patch_attention(qkv[rows[s:e]].float(), [0, e - s], heads)
-        primary = unpad[inverse[rows[s:e]]] == np.arange(s, e)
-        sel = torch.as_tensor(rows[s:e][primary])
-        err = (got[sel] - want[torch.as_tensor(primary)]).abs().max() / want.abs().max()
-        assert err < 2e-2, (p, float(err))
+    src, dst = o.attn_slots(order_d[0], inverse_d[0], gp, gu)
+    got = o.patch_attention(qkv.to(DEV), heads, src, dst, gc, patch, 0.25)
+    assert torch.isfinite(got.float()).all()
+    want = OF.serialized_attention_core(qkv.float(), order, inverse, pad, unpad, cu, heads)
+    assert rel_err(got, want) < 2e-2
+    # the tail: the last r points sit in a patch completed with the K - r points in front of them
+    last = order[n - (n % patch):]
+    assert rel_err(got[torch.as_tensor(last, device=DEV)], want[torch.as_tensor(last)]) < 2e-2
 
 
 @pytest.mark.parametrize("counts,patch", [([64], 64), ([700, 300], 256), ([2500], 1024)])
