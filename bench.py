@@ -125,10 +125,49 @@ def attention_config2(reps):
                       "us": us, "flops": fl, "tflops": fl / us / 1e6, "frac_mfma_peak": fl / us / 1e6 / MFMA_PEAK_TFLOPS}))
 
 
+ENC_CHANNELS = (32, 64, 128, 256, 512)
+
+
+def conv_case(which, reps):
+    """The xCPE convolution alone, through the module's own dispatch (pair, tile or dense form), fp16:
+    `config3` = baseline config 3 (200,000 room voxels at 2 cm, 64 -> 64); `level0` .. `level4` = the voxel set
+    of that encoder level of the benchmark batch (4 rooms pooled with stride 2 per level) at that level's width.
+    Prints one JSON line with the time per call against both rooflines; the command to put under rocprofv3."""
+    from pointtransformerv3_amd import synthetic
+    from pointtransformerv3_amd.sparse import SparseConvTensor, SubMConv3d
+    dev = "cuda:0"
+    if which == "config3":
+        vox = synthetic.room_voxels(200_000, 3000)["grid_coord"]
+        idx = torch.from_numpy(np.concatenate([np.zeros((len(vox), 1), np.int32), vox], 1)).to(dev)
+        channels, label = 64, "baseline config 3: 200,000 room voxels at 2 cm"
+    else:
+        level = int(which[len("level"):])
+        d, _ = build_inputs(4, 106_000, 4000)
+        full = torch.from_numpy(np.concatenate([d["batch"][:, None].astype(np.int32), d["grid_coord"]], 1)).to(dev)
+        full[:, 1:] >>= level
+        idx = torch.unique(full, dim=0).contiguous() if level else full.contiguous()
+        channels = ENC_CHANNELS[level]
+        label = f"encoder level {level} of the benchmark batch ({2 << level} cm voxels)"
+    n = len(idx)
+    gen = torch.Generator(device="cpu").manual_seed(3)
+    conv = SubMConv3d(channels, channels, 3, bias=True, indice_key="bench").to(dev).half()
+    x = SparseConvTensor(torch.randn(n, channels, generator=gen).half().to(dev), idx, [1, 1, 1], 4)
+    with torch.inference_mode():
+        plan = x.conv_plan(3, "bench")
+        per_voxel = plan.n_pairs / n
+        form = ("tile" if channels in (64, 128) and per_voxel >= SubMConv3d.TILE_MODE_MIN_PAIRS_PER_VOXEL else "pair")
+        us = _time_us(lambda: conv(x), iters=reps, warmup=2)
+    flops = 2.0 * plan.n_pairs * channels * channels
+    min_bytes = 2.0 * n * channels * 2 + 27.0 * channels * channels * 2 + 4.0 * plan.n_pairs
+    print(json.dumps({"workload": label, "voxels": n, "channels": channels, "pairs": plan.n_pairs,
+                      "pairs_per_voxel": per_voxel, "form": form, "us": us, "flops": flops, "tflops": flops / us / 1e6,
+                      "frac_mfma_peak": flops / us / 1e6 / MFMA_PEAK_TFLOPS, "min_bytes": min_bytes,
+                      "gbs": min_bytes / us / 1e3, "frac_hbm_peak": min_bytes / us / 1e3 / HBM_PEAK_GBS}))
+
+
 def kernel_rooflines(path):
     """Per-kernel measurements at the sizes the baseline configs name, each against the roofline
     that bounds it (algorithmic bytes or flops / measured time). Written to `path` as JSON."""
-    from oracle import indexing as OI
     from pointtransformerv3_amd import ops, synthetic
     dev = "cuda:0"
     rows = []
@@ -346,6 +385,12 @@ def main():
     ap.add_argument("--attention-config2", metavar="REPS", type=int, default=0,
                     help="only run the patch attention kernel at baseline config 2 (one 100k-point scene, C=512, 32 "
                          "heads, fp16) REPS times and print its rate: the command to put under rocprofv3 --pmc")
+    ap.add_argument("--conv", metavar="CASE", default=None,
+                    choices=["config3", "level0", "level1", "level2", "level3", "level4"],
+                    help="only run the 3x3x3 submanifold convolution of one workload (baseline config 3, or one encoder "
+                         "level of the benchmark batch at its width) --reps times and print its rate: the command to "
+                         "put under rocprofv3 --pmc")
+    ap.add_argument("--reps", type=int, default=20, help="timed calls of --conv")
     ap.add_argument("--train", metavar="DTYPE", default=None, choices=["bfloat16", "float16"],
                     help="instead of the forward benchmark, time a training step (forward, backward, AdamW) of the "
                          "same model and input under autocast to DTYPE and print its own JSON line")
@@ -361,6 +406,9 @@ def main():
 
     if args.attention_config2 > 0:
         attention_config2(args.attention_config2)
+        return
+    if args.conv:
+        conv_case(args.conv, args.reps)
         return
     if args.train:
         training_step(args)

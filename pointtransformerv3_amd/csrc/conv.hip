@@ -544,6 +544,192 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void pair_gemm_kernel(
     }
 }
 
+// Pair mode for 256-channel layers, weight-stationary in REGISTERS.
+// A work-group takes one tap and a range of that tap's pairs. Its 8 waves are 2 row halves x 4 output-channel
+// quarters; a wave keeps W[its 64 output channels, tap, all 256 input channels] as MFMA operand fragments in
+// 128 registers for its whole life (staged once through LDS so that the global reads are whole rows), and the
+// range streams through 64 pairs at a time. Inside the loop the only LDS traffic is the gathered input rows
+// (0.5 KB per MFMA: every row fragment meets two weight fragments that are already in registers) and the only
+// stream from memory is those rows; the weights leave L2 once per work-group instead of once per tile.
+// The input rows of a tile go through LDS in 64-channel steps (64 rows x 128 B), double-buffered, one barrier per
+// step, software-pipelined by hand: right after the barrier that publishes step s+1 a wave asks for its
+// fragments of step s+1 and then issues the eight MFMAs of step s, so the LDS reads run under the matrix work
+// instead of in front of it. The rows of the next four steps (a whole tile) are in flight in a ring of registers
+// that runs on across tile boundaries; pair indices and result slots are fetched two and one tiles ahead.
+// Product rows go to y[pair_slot] for the segment sum, as in the other pair kernels.
+constexpr int WS_THREADS = 512;
+constexpr int WS_ROWS = 64;
+constexpr int WS_KC = 64;
+constexpr int WS_XSTRIDE = WS_KC + 8;   // halfs per staged row
+constexpr int WS_DEPTH = 4;
+constexpr int WS_CIN = 256, WS_COUT = 256;
+
+template <typename T>
+__global__ __launch_bounds__(WS_THREADS, 2) void pair_wstat_kernel(
+    const T* __restrict__ feat, int taps, const T* __restrict__ weight, int cout, T* __restrict__ y,
+    const int32_t* __restrict__ pair_in, const int32_t* __restrict__ pair_slot, const int32_t* __restrict__ tap_ptr,
+    int range_rows) {
+    typedef typename HalfOps<T>::v8 v8;
+    constexpr int CIN = WS_CIN, COUT_T = WS_COUT;
+    constexpr int KSTEPS = CIN / WS_KC;        // 4
+    constexpr int KS = WS_KC / 16;             // MFMA contraction steps per staged step
+    constexpr int WSTRIDE = CIN + W_PAD;
+    constexpr int NT = 2;
+    constexpr int XBUF = WS_ROWS * WS_XSTRIDE;
+    static_assert(KSTEPS % 2 == 0 && KSTEPS == WS_DEPTH, "buffer parity and ring position carry over from tile to tile");
+    static_assert(WS_THREADS == WS_ROWS * (WS_KC / 8), "one 16-byte piece per thread and step");
+    extern __shared__ __align__(16) unsigned char ws_smem[];
+    T* w_lds = (T*)ws_smem;                       // [COUT_T][WSTRIDE], only while the fragments are taken
+    T* x_lds = w_lds + COUT_T * WSTRIDE;          // [2][WS_ROWS][WS_XSTRIDE]
+
+    // which (tap, range) is mine: ranges of range_rows pairs, tap after tap
+    int g = blockIdx.x, tap = -1, p0 = 0, p1 = 0;
+    for (int t = 0; t < taps; ++t) {
+        const int first = tap_ptr[t], cnt = tap_ptr[t + 1] - first;
+        const int nr = (cnt + range_rows - 1) / range_rows;
+        if (g < nr) {
+            tap = t;
+            p0 = first + g * range_rows;
+            p1 = min(first + cnt, p0 + range_rows);
+            break;
+        }
+        g -= nr;
+    }
+    if (tap < 0) return;
+    const int cout0 = blockIdx.y * COUT_T;
+    const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
+    const int col = lane & 31, hf = lane >> 5;
+    const int row0 = (wave >> 2) * 32;                 // the wave's first row inside a tile
+    const int c0 = (wave & 3) * (NT * 32);             // its first output channel inside the tile
+    const int grow = tid >> 3, gpc = tid & 7;          // the row and 16-byte piece this thread gathers
+
+    const int n_tiles = (p1 - p0 + WS_ROWS - 1) / WS_ROWS;
+    auto gather_ptr = [&](int tile) {
+        const int v = p0 + min(tile, n_tiles - 1) * WS_ROWS + grow;
+        return feat + (int64_t)pair_in[min(v, p1 - 1)] * CIN + gpc * 8;
+    };
+    const T* ptr_cur = gather_ptr(0);
+    const T* ptr_nxt = gather_ptr(1);
+    const T* ptr_nn = gather_ptr(2);
+    u32x4 ring[WS_DEPTH];   // ring[r]: the earliest step not yet in LDS whose number is r modulo WS_DEPTH
+#pragma unroll
+    for (int j = 0; j < WS_DEPTH; ++j) ring[j] = *(const u32x4*)(ptr_cur + j * WS_KC);
+
+    // ---- the tap's weights: whole rows into LDS, then this wave's fragments into registers
+    {
+        constexpr int PIECES = COUT_T * (CIN / 8) / WS_THREADS;   // 16 per thread, 8 in flight together
+#pragma unroll
+        for (int i0 = 0; i0 < PIECES; i0 += 8) {
+            u32x4 piece[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int e = tid + (i0 + i) * WS_THREADS, co = e / (CIN / 8), pc = e % (CIN / 8);
+                piece[i] = *(const u32x4*)(weight + ((int64_t)(cout0 + co) * taps + tap) * CIN + pc * 8);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int e = tid + (i0 + i) * WS_THREADS, co = e / (CIN / 8), pc = e % (CIN / 8);
+                *(u32x4*)(w_lds + co * WSTRIDE + pc * 8) = piece[i];
+            }
+        }
+    }
+    __syncthreads();
+    u32x4 wreg[NT][CIN / 16];
+#pragma unroll
+    for (int b = 0; b < NT; ++b)
+#pragma unroll
+        for (int k = 0; k < CIN / 16; ++k)
+            wreg[b][k] = *(const u32x4*)(w_lds + (c0 + b * 32 + col) * WSTRIDE + k * 16 + hf * 8);
+
+    const T* xa = x_lds + (row0 + col) * WS_XSTRIDE + hf * 8;
+    T* xw = x_lds + grow * WS_XSTRIDE + gpc * 8;
+    // where the product rows go: lane l holds the slot of the wave's row l % 32 (its 32 rows, in store order)
+    int32_t slot_nxt = pair_slot[min(p0 + row0 + col, p1 - 1)];
+    // nothing but the ring may be in flight when the loop is entered: the wait-count bookkeeping of a loop is
+    // the union of its entry and its back edge, and a value still pending at entry would be waited for in every
+    // iteration -- in issue order, i.e. together with the whole ring
+    asm volatile("" ::"v"(slot_nxt));
+    asm volatile("" ::"v"(ptr_nn));
+    // the weight rows in LDS are dead once every wave holds its fragments (the first barrier below): each wave
+    // turns its product tiles into row segments there
+    T* stage = w_lds + wave * (32 * XS_STRIDE);
+
+    // step 0 of the first tile: into buffer 0, its fragments into registers
+    *(u32x4*)xw = ring[0];
+    ring[0] = *(const u32x4*)ptr_nxt;   // step WS_DEPTH = step 0 of the second tile
+    __syncthreads();
+    u32x4 xf[2][KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) xf[0][ks] = *(const u32x4*)(xa + ks * 16);
+
+    for (int tile = 0; tile < n_tiles; ++tile) {
+        // the rows three tiles on (the ring already asks for the first step of the tile after next while this one
+        // is multiplied), and where the next tile's product rows go
+        // (asked for a tile ahead: a value used right after its load would make the wave wait for every older
+        // load as well, the whole ring of gathered rows included)
+        const int v3 = p0 + min(tile + 3, n_tiles - 1) * WS_ROWS + grow;
+        int32_t idx3 = pair_in[min(v3, p1 - 1)];
+        const int32_t slot = slot_nxt;
+        const int32_t slot_ahead = pair_slot[min(p0 + min(tile + 1, n_tiles - 1) * WS_ROWS + row0 + col, p1 - 1)];
+        f32x16 acc[NT];
+#pragma unroll
+        for (int b = 0; b < NT; ++b)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[b][v] = 0.f;
+#pragma unroll
+        for (int kc = 0; kc < KSTEPS; ++kc) {
+            // publish step kc + 1 (of the next tile when this is the tile's last step) ...
+            const int nb = (kc + 1) & 1;
+            *(u32x4*)(xw + nb * XBUF) = ring[(kc + 1) % WS_DEPTH];
+            // ... and ask for the step that takes its place in the ring: step kc + 1 of the next tile
+            if (kc + 1 < KSTEPS) ring[(kc + 1) % WS_DEPTH] = *(const u32x4*)(ptr_nxt + (kc + 1) * WS_KC);
+            else ring[0] = *(const u32x4*)ptr_nn;
+            __syncthreads();
+            // fragments of step kc + 1 first, then the products of step kc
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) xf[nb][ks] = *(const u32x4*)(xa + nb * XBUF + ks * 16);
+            __builtin_amdgcn_sched_barrier(0);   // the scheduler would put the reads behind the matrix work
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int b = 0; b < NT; ++b)
+                    acc[b] = HalfOps<T>::mfma(__builtin_bit_cast(v8, wreg[b][kc * KS + ks]),
+                                              __builtin_bit_cast(v8, xf[kc & 1][ks]), acc[b]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // acc[b][v]: output channel cout0 + c0 + b*32 + 8*(v/4) + 4*hf + v%4 of pair row0 + col.
+        // Through the wave's own LDS rows into row-segment shape: a store instruction then writes 8 rows x 128 B
+        // (8 lanes x 16 B per row) instead of 32 rows x 16 B.
+        // Rows past the end of the range repeat its last pair (same input row, same slot): they store the same
+        // values to the same place, so neither the loads nor the stores of the loop are conditional -- with a
+        // branch around them the wait counts in front of the ring would be those of the path that skips them.
+#pragma unroll
+        for (int b = 0; b < NT; ++b)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                u32x2 pk = {HalfOps<T>::pack2(acc[b][4 * q], acc[b][4 * q + 1]),
+                            HalfOps<T>::pack2(acc[b][4 * q + 2], acc[b][4 * q + 3])};
+                *(u32x2*)(stage + col * XS_STRIDE + b * 32 + 8 * q + 4 * hf) = pk;
+            }
+        lds_fence();
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int orow = it * 8 + (lane >> 3), opc = lane & 7;
+            const u32x4 val = *(const u32x4*)(stage + orow * XS_STRIDE + opc * 8);
+            const int32_t dst = __shfl(slot, orow, PTV3_WAVE);
+            *(u32x4*)(y + (int64_t)dst * cout + cout0 + c0 + opc * 8) = val;
+        }
+        lds_fence();
+        ptr_cur = ptr_nxt;
+        ptr_nxt = ptr_nn;
+        // tied to the last product so that the index is not turned into a pointer (and waited for, with every
+        // older load) at the top of the tile
+        asm volatile("" : "+v"(idx3) : "v"(acc[NT - 1][15]));
+        ptr_nn = feat + (int64_t)idx3 * CIN + gpc * 8;
+        slot_nxt = slot_ahead;
+    }
+}
+
 // Pair mode, weight-stationary. A work-group takes one tap and a range of up to `range_rows`
 // of that tap's pairs (tap-major list), keeps W[couts, tap, all input channels] in LDS for its
 // whole life and streams the range through it in tiles of ROWS pairs. Steps (tile, 64-channel
@@ -888,9 +1074,35 @@ int launch_pair_gemm(const void* feat, int cin, int taps, int64_t n_pairs, const
     return PTV3_OK;
 }
 template <typename T>
+int launch_pair_wstat(const void* feat, int taps, int64_t n_pairs, const int32_t* tap_ptr, const int32_t* pair_in,
+                      const int32_t* pair_slot, const void* weight, int cout, void* y, hipStream_t stream) {
+    const size_t lds = ((size_t)WS_COUT * (WS_CIN + W_PAD) + 2 * (size_t)WS_ROWS * WS_XSTRIDE) * sizeof(T);
+    static_assert(8 * 32 * XS_STRIDE <= WS_COUT * (WS_CIN + W_PAD), "the waves' staging rows fit where the weights were");
+    auto kern = pair_wstat_kernel<T>;
+    static bool allowed = false;   // per instantiation
+    if (!allowed) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        allowed = true;
+    }
+    // One work-group per CU (its registers hold the weights). Ranges in whole tiles: one round of work-groups
+    // over the machine, long enough to pay for staging one tap's weights.
+    const int64_t col_tiles = cout / WS_COUT;
+    int64_t range_rows = ptv3_ceil_div(ptv3_ceil_div(n_pairs * col_tiles, 256 - taps), WS_ROWS) * WS_ROWS;
+    if (range_rows < 8 * WS_ROWS) range_rows = 8 * WS_ROWS;
+    dim3 grid((unsigned)(n_pairs / range_rows + taps), (unsigned)col_tiles);   // every tap may end with a partial range
+    hipLaunchKernelGGL(kern, grid, dim3(WS_THREADS), lds, stream, (const T*)feat, taps, (const T*)weight, cout, (T*)y,
+                       pair_in, pair_slot, tap_ptr, (int)range_rows);
+    return PTV3_OK;
+}
+
+template <typename T>
 int launch_pairs_chunked(const void* feat, int cin, int taps, int64_t n_pairs, const int32_t* tap_ptr,
                          const int32_t* pair_in, const int32_t* pair_slot, const void* weight, int cout, void* y,
                          hipStream_t stream) {
+    // wide square-ish layers: one tap's weights stay in LDS
+    if (cin == WS_CIN && cout % WS_COUT == 0 && taps <= 128)
+        return launch_pair_wstat<T>(feat, taps, n_pairs, tap_ptr, pair_in, pair_slot, weight, cout, y, stream);
     // the ring of the persistent kernel is four 32-channel steps deep
     if (cin % 128 == 0 && taps <= 128)
         return launch_pair_gemm<T, 1, 4, 4>(feat, cin, taps, n_pairs, tap_ptr, pair_in, pair_slot, weight, cout, y, stream);

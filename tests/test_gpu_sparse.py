@@ -197,7 +197,8 @@ def test_conv_plan_direct_equals_plan_of_map(ks, n, extent, nb):
 @pytest.mark.parametrize("ks,cin,cout,n,extent", [(3, 32, 32, 3000, 20), (3, 64, 64, 50_000, 60), (3, 128, 128, 9000, 24),
                                                   (3, 256, 256, 2000, 12), (3, 512, 512, 600, 8), (5, 16, 32, 20_000, 40),
                                                   (3, 192, 192, 1500, 12), (3, 256, 160, 1500, 12), (3, 128, 256, 4000, 16),
-                                                  (3, 384, 72, 900, 10), (3, 128, 128, 2, 4)])
+                                                  (3, 384, 72, 900, 10), (3, 128, 128, 2, 4), (3, 256, 256, 20_000, 30), (3, 512, 512, 7000, 16),
+                                                  (3, 256, 512, 3000, 14), (3, 256, 256, 2, 2)])
 def test_subm_conv_pairs_parity(dtype, ks, cin, cout, n, extent):
     rng = np.random.default_rng(cin + n)
     g = torch.Generator().manual_seed(cin + n)
