@@ -449,6 +449,18 @@ int ptv3_bn_act(const void *x, const void *running_mean, const void *running_var
  * over memory along k. */
 int ptv3_linear_fwd(const void *x, const void *w, const void *bias, int dtype, int64_t n, int k, int nout,
                     int gelu, void *out, void *stream);
+/* The same layers at 256 inputs (the 16 cm level of the default model: cpe.1, qkv, proj, fc1 + GELU) with the
+ * weights resident in registers instead of LDS: k == 256, nout a multiple of 256 (PTV3_ESHAPE otherwise: use
+ * ptv3_linear_fwd). Same result as ptv3_linear_fwd: fp32 accumulation over the 256 inputs, one rounding. */
+int ptv3_linear_wide_fwd(const void *x, const void *w, const void *bias, int dtype, int64_t n, int k, int nout,
+                         int gelu, void *out, void *stream);
+/* nn.Linear with a long contraction (model.py:514 fc2 of the wide blocks, 1024 -> 256 and 2048 -> 512, with the
+ * residual addition of :602 taken in; :450 the 512 -> 1536 qkv): out = resid + x w^T + bias, a tiled GEMM.
+ * x (n, k), w (nout, k), bias (nout,) or NULL, resid (n, nout) or NULL (it may be `out` itself: every element is
+ * read before it is written, by the same thread), fp16 / bf16, k a multiple of 128, nout a multiple of 128
+ * (PTV3_ESHAPE otherwise). Sums and the residual are added in fp32 and rounded once. */
+int ptv3_linear_gemm_fwd(const void *x, const void *w, const void *bias, const void *resid, int dtype, int64_t n,
+                         int k, int nout, void *out, void *stream);
 /* The same followed by an inference-mode nn.BatchNorm1d and optionally the GELU, the projections of
  * model.py:726-735 (Linear -> BatchNorm1d -> GELU) in one kernel; statistics and affine parameters as
  * for ptv3_bn_act. The Linear's result is rounded to dtype before the normalisation, as when stored. */

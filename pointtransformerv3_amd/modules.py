@@ -445,7 +445,11 @@ class Block(PointModule):
             feat = ops.mlp_fused(normed, feat, mlp.fc1.weight, mlp.fc1.bias, mlp.fc2.weight, mlp.fc2.bias)
         elif plain_mlp:
             hidden = ops.linear(normed, mlp.fc1, gelu=True) if exact_gelu else mlp.act(mlp.fc1(normed))
-            feat = feat.addmm_(hidden, mlp.fc2.weight.to(hidden.dtype).t())   # onto the stored sum, no copy of it
+            if (not ops.LIBRARY_GEMM and ops.linear_gemm_ok(hidden, mlp.fc2.weight) and feat.is_contiguous()
+                    and feat.dtype == hidden.dtype):
+                feat = ops.linear_gemm(hidden, mlp.fc2.weight, None, resid=feat)   # onto the stored sum, in place
+            else:
+                feat = feat.addmm_(hidden, mlp.fc2.weight.to(hidden.dtype).t())
         else:
             feat = feat + mlp(normed)
         point.feat = feat

@@ -1058,6 +1058,8 @@ def linear(x, mod, gelu=False):
         return torch.nn.functional.gelu(y) if gelu else y
     if linear_rows_pays(x, mod.weight, gelu):
         return linear_rows(x, mod.weight, mod.bias, gelu)
+    if not LIBRARY_GEMM and not gelu and linear_gemm_ok(x, mod.weight):
+        return linear_gemm(x, mod.weight, mod.bias)
     y = torch.nn.functional.linear(x, mod.weight, mod.bias)
     return torch.nn.functional.gelu(y) if gelu else y
 
@@ -1106,6 +1108,37 @@ def mlp(x, fc1, fc2):
     return Mlp.apply(xa, fc1.weight, fc1.bias, fc2.weight, fc2.bias)
 
 
+def linear_gemm(x, weight, bias=None, resid=None):
+    """resid + x W^T + b through the tiled GEMM kernel (ptv3_linear_gemm_fwd): any number of inputs in 128s, outputs
+    in 128s, fp16 / bf16. With resid the result is written over it (fc2 accumulating onto the stored sum)."""
+    _dev(x, weight, bias, resid)
+    x = x.contiguous()
+    n, k = x.shape
+    w = weight.to(x.dtype).contiguous()
+    b = None if bias is None else bias.to(x.dtype).contiguous()
+    if resid is not None and not (resid.is_contiguous() and resid.dtype == x.dtype and resid.shape == (n, w.shape[0])):
+        raise _lib.Ptv3Error("linear_gemm: resid must be a contiguous (rows, outputs) tensor of x's dtype")
+    out = resid if resid is not None else torch.empty((n, w.shape[0]), dtype=x.dtype, device=x.device)
+    _lib.check(_lib.load().ptv3_linear_gemm_fwd(_ptr(x), _ptr(w), _ptr(b), _ptr(resid), _dtype_code(x), n, k, w.shape[0],
+                                                _ptr(out), _stream()), "ptv3_linear_gemm_fwd")
+    return out
+
+
+# The three long-contraction layers of the default model (fc2 at 256 and 512 channels, the 512 -> 1536 qkv) are
+# plain GEMMs on which the library's 256 x 160 tiles measured 26-29 us against 43-48 us for this package's
+# 128 x 128-tile kernel (both bound by what the L2s deliver per tile, see csrc/linearw.hip). True: the library GEMM
+# takes them; False: no library call anywhere in the forward.
+LIBRARY_GEMM = True
+
+
+def linear_gemm_ok(x, weight):
+    return (x.is_cuda and x.dim() == 2 and x.dtype in (torch.float16, torch.bfloat16) and weight.shape[1] % 128 == 0
+            and weight.shape[0] % 128 == 0)
+
+
+LINEAR_WIDE = True   # 256 inputs, outputs in 256s: the kernel with the weights resident in registers
+
+
 def linear_rows(x, weight, bias=None, gelu=False):
     """act(x W^T + b) for many rows and few channels (see ptv3_linear_fwd); act = exact GELU if gelu."""
     _dev(x, weight, bias)
@@ -1115,6 +1148,10 @@ def linear_rows(x, weight, bias=None, gelu=False):
     w = weight.to(x.dtype).contiguous()
     b = None if bias is None else bias.to(x.dtype).contiguous()
     out = torch.empty((n, w.shape[0]), dtype=x.dtype, device=x.device)
+    if LINEAR_WIDE and k == 256 and w.shape[0] % 256 == 0 and n >= 4096:
+        _lib.check(lib.ptv3_linear_wide_fwd(_ptr(x), _ptr(w), _ptr(b), _dtype_code(x), n, k, w.shape[0], int(bool(gelu)),
+                                            _ptr(out), _stream()), "ptv3_linear_wide_fwd")
+        return out
     _lib.check(lib.ptv3_linear_fwd(_ptr(x), _ptr(w), _ptr(b), _dtype_code(x), n, k, w.shape[0], int(bool(gelu)),
                                    _ptr(out), _stream()), "ptv3_linear_fwd")
     return out

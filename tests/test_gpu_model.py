@@ -314,3 +314,22 @@ def test_forward_tiny_and_ragged_scenes_fp32(sizes):
     want = ptv3_forward(model.state_dict(), d["grid_coord"], feat, d["offset"], enable_flash=False, perms=perms, **kw)
     point = _run(model.to(DEV), d, feat, torch.float32)
     assert rel_err(point.feat, want) < 1e-4
+
+
+def test_forward_fp16_without_any_library_gemm():
+    """ops.LIBRARY_GEMM = False: fc2 of the 256- and 512-channel blocks and the 512 -> 1536 qkv run on this package's
+    tiled GEMM instead of the library's; the forward is then library-free end to end. Same bar."""
+    from pointtransformerv3_amd import PointTransformerV3, ops
+    torch.manual_seed(1)
+    model = PointTransformerV3(shuffle_orders=False).eval().half()
+    d, feat = _data(20000, 2, grid=0.02)
+    perms = _draw_perms(78, False)
+    sd = {k: v.float() for k, v in model.state_dict().items()}
+    x = feat.astype(np.float16).astype(np.float32)
+    ops.LIBRARY_GEMM = False
+    try:
+        point = _run(model.to(DEV), d, x, torch.float16)
+    finally:
+        ops.LIBRARY_GEMM = True
+    want = ptv3_forward(sd, d["grid_coord"], x, d["offset"], perms=perms)
+    assert rel_err(point.feat, want) < 2e-2

@@ -424,7 +424,9 @@ def test_voxel_hash_edge_coordinates(ks):
 @pytest.mark.parametrize("k,nout,n,gelu,bias", [(32, 64, 50_001, False, True), (64, 64, 31, False, True), (64, 128, 4000, True, False),
                                                 (128, 128, 1, False, True), (128, 384, 40_001, False, True), (128, 512, 777, True, True),
                                                 (256, 768, 9000, False, True), (256, 1024, 5000, True, True), (256, 96, 33, False, False),
-                                                (512, 512, 2500, False, True), (512, 2048, 1000, True, True), (512, 1536, 64, False, True)])
+                                                (512, 512, 2500, False, True), (512, 2048, 1000, True, True), (512, 1536, 64, False, True),
+                                                (256, 256, 37_681, False, True), (256, 1024, 37_681, True, True), (256, 256, 4097, False, False),
+                                                (256, 768, 16_384, False, True)])
 def test_linear_rows_parity(dtype, k, nout, n, gelu, bias):
     import torch.nn.functional as F
     g = torch.Generator().manual_seed(k + nout + n)
@@ -436,6 +438,29 @@ def test_linear_rows_parity(dtype, k, nout, n, gelu, bias):
         want = F.gelu(want)
     got = ops().linear_rows(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), gelu)
     assert got.dtype == dtype and got.shape == (n, nout)
+    assert rel_err(got, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("k,nout,n,resid,bias", [(1024, 256, 37_681, True, False), (2048, 512, 8617, True, False),
+                                                 (512, 1536, 8617, False, True), (128, 128, 1, False, True),
+                                                 (384, 128, 129, True, True), (1024, 256, 127, True, True)])
+def test_linear_gemm_parity(dtype, k, nout, n, resid, bias):
+    """The tiled GEMM of the long contractions: resid + x W^T + b, added in fp32, rounded once, written over resid."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(k + nout + n)
+    x = torch.randn(n, k, generator=g).to(dtype)
+    w = (torch.randn(nout, k, generator=g) / k ** 0.5).to(dtype)
+    b = (torch.randn(nout, generator=g) * 0.5).to(dtype) if bias else None
+    r = torch.randn(n, nout, generator=g).to(dtype) if resid else None
+    want = F.linear(x.float(), w.float(), None if b is None else b.float())
+    if resid:
+        want = want + r.float()
+    r_dev = None if r is None else r.to(DEV)
+    got = ops().linear_gemm(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), r_dev)
+    assert got.dtype == dtype and got.shape == (n, nout)
+    if resid:
+        assert got.data_ptr() == r_dev.data_ptr()
     assert rel_err(got, want) < TOL[dtype]
 
 
