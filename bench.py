@@ -5,8 +5,10 @@
 A step is one full PointTransformerV3 forward (default architecture, fp16, eval) over a batch
 of 4 synthetic room scenes of ~100k voxelised points each, inputs resident in HBM. Prints one
 JSON line: throughput in points/s, the roofline of the dominant kernel (patch attention,
-MFMA-bound) measured with HIP events around every launch inside the timed region, and the
-CPU oracle timed on this machine's host cores on one of the four scenes.
+MFMA-bound nominally, VALU-bound in fact: both fractions are given) and of the sparse convolutions,
+measured with HIP events around every launch inside the timed region, the CPU oracle timed on
+this machine's host cores (one of the four scenes, and baseline config 1 in full), and short
+runs of the other baseline configurations (5, 2, 3) after the timed region.
 """
 import argparse
 import json
@@ -52,6 +54,25 @@ def attention_flops(work):
     return float(4.0 * (lens * lens).sum().item() * channels)
 
 
+def conv_flops(work):
+    """2 * active pairs * Cin * Cout for one convolution launch (pair or tile form)."""
+    n_pairs, n, cin, cout, taps, form = work
+    return 2.0 * n_pairs * cin * cout
+
+
+def conv_min_bytes(work):
+    """Rows in and out once, the weights once, one index per pair."""
+    n_pairs, n, cin, cout, taps, form = work
+    return 2.0 * n * (cin + cout) + 2.0 * taps * cin * cout + 4.0 * n_pairs
+
+
+# per 64 keys x 32 queries a wave has to issue 32 v_exp_f32 (8 cycles each on this part) and 16 packed conversions
+# (4 each) whatever else it does: 320 VALU cycles per 2048 scores and SIMD
+VALU_CYCLES_PER_SCORE = 320.0 / 2048.0
+NOMINAL_CLOCK_HZ = 2.4e9
+N_SIMDS = 1024
+
+
 def recorded_traffic(n_points):
     """HBM bytes per attention launch from the committed rocprofv3 --pmc summary of this same
     workload (FETCH_SIZE and WRITE_SIZE runs, each scaled by a 1 GiB copy in the same process);
@@ -85,7 +106,40 @@ def cpu_baseline(model, d, feat):
     ptv3_forward(sd, d["grid_coord"][:n0], feat[:n0], d["offset"][:1])
     dt = time.perf_counter() - t0
     return {"value": n0 / dt, "unit": "points/s", "cores": cores, "kind": "port",
-            "sample": f"one forward of the CPU oracle over scene 0 of the batch ({n0} points), {dt:.1f} s"}
+            "sample": f"one forward of the CPU oracle over scene 0 of the batch ({n0} points), {dt:.1f} s",
+            "config1": cpu_baseline_config1(cores)}
+
+
+def cpu_baseline_config1(cores):
+    """Baseline configuration 1 on the host cores: z-order + Hilbert serialization (adaptive depth and depth 16) of
+    16,384 points uniform in a 5 m cube, then one attention block (patch 1024, C = 64, 4 heads) in fp32 through
+    the CPU oracle. Median of 3."""
+    from oracle import functional as OF
+    from oracle import indexing as OI
+    from oracle import serialization as OS
+    from pointtransformerv3_amd import synthetic
+    sc = synthetic.cube_scene(16_384, 1000, 0.02)
+    grid = sc["grid_coord"]
+    n = len(grid)
+    batch = np.zeros(n, np.int64)
+    gen = torch.Generator().manual_seed(1001)
+    feat = torch.randn(n, 64, generator=gen)
+    wq, bq = torch.randn(192, 64, generator=gen) / 8, torch.zeros(192)
+    wp, bp = torch.randn(64, 64, generator=gen) / 8, torch.zeros(64)
+    pad, unpad, cu = OI.padding_tables(np.array([n], np.int64), 1024)
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        OS.serialize(grid, batch, ["z", "hilbert"])
+        _, _, order, inverse = OS.serialize(grid, batch, ["z", "hilbert"], depth=16)
+        qkv = torch.nn.functional.linear(feat, wq, bq)
+        core = OF.serialized_attention_core(qkv, order[1], inverse[1], pad, unpad, cu, 4)
+        torch.nn.functional.linear(core, wp, bp)
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[1]
+    return {"value": n / med, "unit": "points/s", "cores": cores, "kind": "port",
+            "sample": f"baseline config 1 in full (16,384 points: z + Hilbert serialization at depth 8 and 16, one "
+                      f"attention block, fp32), median of 3: {med * 1e3:.0f} ms"}
 
 
 HBM_PEAK_GBS = 8000.0
@@ -105,8 +159,8 @@ def _time_us(fn, iters=20, warmup=3):
     return s.elapsed_time(e) * 1e3 / iters
 
 
-def attention_config2(reps):
-    """Baseline config 2 alone: Hilbert order of one room scene, patch 1024, C=512, 32 heads, fp16."""
+def attention_config2(reps, dtype=torch.float16):
+    """Baseline config 2 alone: Hilbert order of one room scene, patch 1024, C=512, 32 heads."""
     from pointtransformerv3_amd import ops, synthetic
     dev = "cuda:0"
     sc = synthetic.room_scene(106_000, 2000, 0.02)
@@ -117,12 +171,13 @@ def attention_config2(reps):
     pad2, unpad2, cu2 = ops.pad_index(torch.tensor([n2], device=dev), [n2], 1024)
     src2, dst2 = ops.attn_slots(order2[0], inv2[0], pad2, unpad2)
     gen = torch.Generator(device="cpu").manual_seed(2)
-    qkv = (torch.randn(n2, 3 * 512, generator=gen) / 4).half().to(dev)
+    qkv = (torch.randn(n2, 3 * 512, generator=gen) / 4).to(dtype).to(dev)
     us = _time_us(lambda: ops.patch_attention(qkv, 32, src2, dst2, cu2, 1024, 0.25), iters=reps, warmup=1)
     lens = torch.diff(cu2.long()).double()
     fl = float(4.0 * (lens * lens).sum().item() * 512)
-    print(json.dumps({"kernel": "patch_attn_half_kernel<f16>", "points": n2, "sequences": int(len(cu2) - 1), "heads": 32,
-                      "us": us, "flops": fl, "tflops": fl / us / 1e6, "frac_mfma_peak": fl / us / 1e6 / MFMA_PEAK_TFLOPS}))
+    name = {torch.float16: "f16", torch.bfloat16: "bf16"}[dtype]
+    return {"kernel": f"patch_attn_half_kernel<{name}>", "points": n2, "sequences": int(len(cu2) - 1), "heads": 32,
+            "us": us, "flops": fl, "tflops": fl / us / 1e6, "frac_mfma_peak": fl / us / 1e6 / MFMA_PEAK_TFLOPS}
 
 
 ENC_CHANNELS = (32, 64, 128, 256, 512)
@@ -132,7 +187,8 @@ def conv_case(which, reps):
     """The xCPE convolution alone, through the module's own dispatch (pair, tile or dense form), fp16:
     `config3` = baseline config 3 (200,000 room voxels at 2 cm, 64 -> 64); `level0` .. `level4` = the voxel set
     of that encoder level of the benchmark batch (4 rooms pooled with stride 2 per level) at that level's width.
-    Prints one JSON line with the time per call against both rooflines; the command to put under rocprofv3."""
+    Returns the time per call against both rooflines (printed as one JSON line by --conv: the command to put under
+    rocprofv3)."""
     from pointtransformerv3_amd import synthetic
     from pointtransformerv3_amd.sparse import SparseConvTensor, SubMConv3d
     dev = "cuda:0"
@@ -159,10 +215,52 @@ def conv_case(which, reps):
         us = _time_us(lambda: conv(x), iters=reps, warmup=2)
     flops = 2.0 * plan.n_pairs * channels * channels
     min_bytes = 2.0 * n * channels * 2 + 27.0 * channels * channels * 2 + 4.0 * plan.n_pairs
-    print(json.dumps({"workload": label, "voxels": n, "channels": channels, "pairs": plan.n_pairs,
-                      "pairs_per_voxel": per_voxel, "form": form, "us": us, "flops": flops, "tflops": flops / us / 1e6,
-                      "frac_mfma_peak": flops / us / 1e6 / MFMA_PEAK_TFLOPS, "min_bytes": min_bytes,
-                      "gbs": min_bytes / us / 1e3, "frac_hbm_peak": min_bytes / us / 1e3 / HBM_PEAK_GBS}))
+    return {"workload": label, "voxels": n, "channels": channels, "pairs": plan.n_pairs,
+            "pairs_per_voxel": per_voxel, "form": form, "us": us, "flops": flops, "tflops": flops / us / 1e6,
+            "frac_mfma_peak": flops / us / 1e6 / MFMA_PEAK_TFLOPS, "min_bytes": min_bytes,
+            "gbs": min_bytes / us / 1e3, "frac_hbm_peak": min_bytes / us / 1e3 / HBM_PEAK_GBS}
+
+
+def other_configs():
+    """The baseline configurations that are not the headline, a few iterations each: config 5 (two LiDAR-like sweeps,
+    full forward, fp16), config 2 (patch attention alone, bf16), config 3 (pair lists + 3x3x3 convolution alone, fp16)."""
+    from pointtransformerv3_amd import PointTransformerV3, ops, synthetic
+    dev = "cuda:0"
+    res = {}
+    # ---- config 5
+    scenes = [synthetic.lidar_scene(5000 + i, 0.05) for i in range(2)]
+    d = synthetic.collate(scenes)
+    feat = synthetic.lidar_features(d["coord"], 5000)
+    torch.manual_seed(5)
+    model = PointTransformerV3(in_channels=4).eval().half().to(dev)
+    data = dict(feat=torch.from_numpy(feat).to(dev).half(), grid_coord=torch.from_numpy(d["grid_coord"]).to(dev),
+                offset=torch.from_numpy(d["offset"]).to(dev))
+    with torch.inference_mode():
+        for _ in range(3):
+            out = model(dict(data))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            out = model(dict(data))
+        torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / 10 * 1e3
+    assert torch.isfinite(out.feat.float()).all()
+    res["config5_lidar_forward_fp16"] = {"points": len(feat), "scenes": 2, "ms": ms, "points_per_s": len(feat) / ms * 1e3}
+    del model, data, out
+    # ---- config 2
+    a = attention_config2(10, torch.bfloat16)
+    res["config2_attention_bf16"] = {"points": a["points"], "ms": a["us"] / 1e3, "points_per_s": a["points"] / a["us"] * 1e6,
+                                     "tflops": a["tflops"], "frac_mfma_peak": a["frac_mfma_peak"]}
+    # ---- config 3
+    c = conv_case("config3", 10)
+    vox = synthetic.room_voxels(200_000, 3000)["grid_coord"]
+    idx = torch.from_numpy(np.concatenate([np.zeros((len(vox), 1), np.int32), vox], 1)).to(dev)
+    kmap_us = _time_us(lambda: ops.conv_plan_direct(idx, 3), iters=10)
+    res["config3_kmap_conv_fp16"] = {"voxels": c["voxels"], "pairs": c["pairs"], "kmap_us": kmap_us, "conv_us": c["us"],
+                                     "ms": (kmap_us + c["us"]) / 1e3, "voxels_per_s": c["voxels"] / (kmap_us + c["us"]) * 1e6,
+                                     "conv_tflops": c["tflops"], "conv_frac_mfma_peak": c["frac_mfma_peak"],
+                                     "conv_frac_hbm_peak": c["frac_hbm_peak"]}
+    return res
 
 
 def kernel_rooflines(path):
@@ -379,6 +477,8 @@ def main():
     ap.add_argument("--scenes", type=int, default=4)
     ap.add_argument("--points", type=int, default=106_000, help="points drawn per scene before voxel dedup")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the short runs of baseline configs 5, 2 and 3 after the timed region")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device copy (a kernel of known traffic) so that rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings of this process can be scaled to bytes")
@@ -405,10 +505,10 @@ def main():
     from pointtransformerv3_amd import PointTransformerV3, ops
 
     if args.attention_config2 > 0:
-        attention_config2(args.attention_config2)
+        print(json.dumps(attention_config2(args.attention_config2)))
         return
     if args.conv:
-        conv_case(args.conv, args.reps)
+        print(json.dumps(conv_case(args.conv, args.reps)))
         return
     if args.train:
         training_step(args)
@@ -443,6 +543,12 @@ def main():
     ms_per_step = wall / args.steps * 1e3
     launches, attn_ms, attn_flops = timer.summary("patch_attn", attention_flops)
     achieved = attn_flops / (attn_ms * 1e-3) / 1e12 if attn_ms > 0 else 0.0
+    # the bound that actually applies at head_dim 16: one exponential and half a conversion per score on the VALU
+    scores = attn_flops / 64.0                       # flops = 4 * sum len^2 * C, scores = sum len^2 * C / 16
+    exp_floor_ms = scores * VALU_CYCLES_PER_SCORE / N_SIMDS / NOMINAL_CLOCK_HZ * 1e3
+    conv_launches, conv_ms, conv_fl = timer.summary("subm_conv", conv_flops)
+    _, _, conv_by = timer.summary("subm_conv", conv_min_bytes)
+    conv_tf = conv_fl / (conv_ms * 1e-3) / 1e12 if conv_ms > 0 else 0.0
     result = {
         "metric": "PTv3 fwd points/sec (4x100k-pt scenes)",
         "value": n_points / (ms_per_step * 1e-3),
@@ -463,9 +569,19 @@ def main():
                      "traffic": recorded_traffic(n_points), "launches": launches,
                      "avg_launch_us": attn_ms * 1e3 / max(launches, 1),
                      "flops_per_launch": attn_flops / max(launches, 1),
-                     "attn_ms_per_step": attn_ms / args.steps},
+                     "attn_ms_per_step": attn_ms / args.steps,
+                     "valu_exp_floor_ms_per_step": exp_floor_ms / args.steps,
+                     "valu_exp_frac": exp_floor_ms / attn_ms if attn_ms > 0 else 0.0,
+                     "conv": {"kernels": "pair_wstat / pair_gemm / subm_conv_pairs + pair_segment_sum, conv_tile",
+                              "bound": "mfma", "launches": conv_launches, "ms_per_step": conv_ms / args.steps,
+                              "achieved": conv_tf, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                              "frac": conv_tf / MFMA_PEAK_TFLOPS,
+                              "hbm_frac": (conv_by / (conv_ms * 1e-3) / 1e9 / HBM_PEAK_GBS) if conv_ms > 0 else 0.0}},
         "cpu_baseline": cpu,
     }
+    if not args.no_other_configs:
+        del model, data, out
+        result["other_configs"] = other_configs()
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)

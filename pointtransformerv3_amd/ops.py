@@ -704,10 +704,17 @@ def subm_conv_pairs(feat, plan, weight, bias=None):
     b = None if bias is None else bias.to(feat.dtype).contiguous()
     y = torch.empty((max(plan.n_pairs, 1), cout), dtype=feat.dtype, device=feat.device)
     out = torch.empty((n, cout), dtype=feat.dtype, device=feat.device)
-    _lib.check(lib.ptv3_subm_conv_pairs_fwd(_ptr(feat), _dtype_code(feat), n, cin, plan.taps, plan.n_pairs,
-                                            _ptr(plan.tap_ptr), _ptr(plan.row_ptr), _ptr(plan.pair_in),
-                                            _ptr(plan.pair_slot), _ptr(w), _ptr(b), cout, _ptr(y), _ptr(out),
-                                            _stream()), "ptv3_subm_conv_pairs_fwd")
+
+    def call():
+        _lib.check(lib.ptv3_subm_conv_pairs_fwd(_ptr(feat), _dtype_code(feat), n, cin, plan.taps, plan.n_pairs,
+                                                _ptr(plan.tap_ptr), _ptr(plan.row_ptr), _ptr(plan.pair_in),
+                                                _ptr(plan.pair_slot), _ptr(w), _ptr(b), cout, _ptr(y), _ptr(out),
+                                                _stream()), "ptv3_subm_conv_pairs_fwd")
+
+    if _LAUNCH_TIMER is not None:
+        _LAUNCH_TIMER.launch("subm_conv", (plan.n_pairs, n, cin, cout, plan.taps, "pair"), call)
+    else:
+        call()
     return out
 
 
@@ -736,9 +743,16 @@ def subm_conv_tiles(feat, plan, packed_weight, bias=None):
     b = None if bias is None else bias.to(feat.dtype).contiguous()
     out = torch.empty((n, c), dtype=feat.dtype, device=feat.device)
     tile_tap, tile_pair, vox_taps = plan.tiles()
-    _lib.check(lib.ptv3_subm_conv_tiles_fwd(_ptr(feat), _dtype_code(feat), n, c, plan.taps, _ptr(packed_weight), _ptr(b),
-                                            _ptr(tile_tap), _ptr(tile_pair), _ptr(vox_taps), _ptr(out), _stream()),
-               "ptv3_subm_conv_tiles_fwd")
+
+    def call():
+        _lib.check(lib.ptv3_subm_conv_tiles_fwd(_ptr(feat), _dtype_code(feat), n, c, plan.taps, _ptr(packed_weight),
+                                                _ptr(b), _ptr(tile_tap), _ptr(tile_pair), _ptr(vox_taps), _ptr(out),
+                                                _stream()), "ptv3_subm_conv_tiles_fwd")
+
+    if _LAUNCH_TIMER is not None:
+        _LAUNCH_TIMER.launch("subm_conv", (plan.n_pairs, n, c, c, plan.taps, "tile"), call)
+    else:
+        call()
     return out
 
 
