@@ -48,6 +48,12 @@ const char *ptv3_strerror(int rc);
 int ptv3_encode(const int32_t *grid_coord, const int64_t *batch, int64_t n, int depth,
                 const int32_t *order_ids_host, int k, int64_t *code, void *stream);
 
+/* serialization/default.py:27-39 -> z_order.py:104-126, hilbert.py:201-303 (the inverse of ptv3_encode for one
+ * order). code (n,) int64; grid_coord (n,3) int64 out (the reference returns int64 coordinates);
+ * batch (n,) int64 out or NULL: code >> 3*depth. */
+int ptv3_decode(const int64_t *code, int64_t n, int depth, int order_id, int64_t *grid_coord,
+                int64_t *batch, void *stream);
+
 /* model.py:100 (depth = bit length of the largest coordinate) and :162-164 (sparse_shape):
  * per-axis maximum of grid_coord (n,3) int32 into out3 (3 int32, device). n >= 1. */
 int ptv3_grid_max(const int32_t *grid_coord, int64_t n, int32_t *out3, void *stream);

@@ -16,6 +16,7 @@ SIGNATURES = {
     "ptv3_version": (_i32, []),
     "ptv3_strerror": (ctypes.c_char_p, [_i32]),
     "ptv3_encode": (_i32, [_vp, _vp, _i64, _i32, _vp, _i32, _vp, _vp]),
+    "ptv3_decode": (_i32, [_vp, _i64, _i32, _i32, _vp, _vp, _vp]),
     "ptv3_grid_max": (_i32, [_vp, _i64, _vp, _vp]),
     "ptv3_voxelize_workspace_bytes": (_sz, [_i64, _i32]),
     "ptv3_voxelize": (_i32, [_vp, _i64, _vp, _i32, _f32, _vp, _vp, _vp, _vp, _vp, ctypes.c_uint32, _vp, _sz, _vp]),

@@ -1,4 +1,4 @@
-// Space-filling-curve codes for all requested orders in one pass over the points.
+// Space-filling-curve codes for all requested orders in one pass over the points, and their inverse.
 //
 // Replaces serialization/default.py:8-24 with z_order.py:66-101 and hilbert.py:91-198 of the
 // reference: one thread per point, coordinates stay in registers, the k codes are written
@@ -29,7 +29,33 @@ __global__ __launch_bounds__(256) void encode_kernel(const int32_t* __restrict__
     }
 }
 
+// serialization/default.py:27-39: the batch index is what sits above the 3 depth curve bits
+__global__ __launch_bounds__(256) void decode_kernel(const int64_t* __restrict__ code, int64_t n, int depth, int id,
+                                                     int64_t* __restrict__ grid_coord, int64_t* __restrict__ batch) {
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= n) return;
+    const int64_t c = code[p];
+    const uint64_t low = (uint64_t)c & ((1ull << (3 * depth)) - 1ull);   // depth <= 16: at most 48 bits
+    uint32_t x, y, z;
+    ptv3::curve_point(id, low, depth, x, y, z);
+    grid_coord[3 * p + 0] = x;
+    grid_coord[3 * p + 1] = y;
+    grid_coord[3 * p + 2] = z;
+    if (batch) batch[p] = c >> (3 * depth);   // arithmetic shift, as torch's >> on int64
+}
+
 }  // namespace
+
+extern "C" int ptv3_decode(const int64_t* code, int64_t n, int depth, int order_id, int64_t* grid_coord,
+                           int64_t* batch, void* stream) {
+    if (n < 0 || order_id < 0 || order_id > 3) return PTV3_EINVAL;
+    if (depth < 1 || depth > 16) return PTV3_EDEPTH;
+    if (n == 0) return PTV3_OK;
+    if (!code || !grid_coord) return PTV3_EINVAL;
+    hipLaunchKernelGGL(decode_kernel, dim3((unsigned)ptv3_ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream,
+                       code, n, depth, order_id, grid_coord, batch);
+    PTV3_RETURN_LAUNCH();
+}
 
 extern "C" int ptv3_encode(const int32_t* grid_coord, const int64_t* batch, int64_t n, int depth,
                            const int32_t* order_ids_host, int k, int64_t* code, void* stream) {

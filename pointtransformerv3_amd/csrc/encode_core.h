@@ -58,11 +58,60 @@ PTV3_HD uint64_t hilbert3(uint32_t x0, uint32_t x1, uint32_t x2, int depth) {
 }
 
 
+// Inverse of spread3: gather bits 0, 3, 6, ... of x into the low 16 bits.
+PTV3_HD uint32_t compact3(uint64_t x) {
+    x &= 0x1249249249249249ull;
+    x = (x | (x >> 2)) & 0x10c30c30c30c30c3ull;
+    x = (x | (x >> 4)) & 0x100f00f00f00f00full;
+    x = (x | (x >> 8)) & 0x001f0000ff0000ffull;
+    x = (x | (x >> 16)) & 0x001f00000000ffffull;
+    x = (x | (x >> 32)) & 0xffffull;
+    return (uint32_t)x;
+}
+
+// Inverse of hilbert3: Gray encode, de-interleave, then undo Skilling's edits from the lowest level up.
+PTV3_HD void hilbert3_inverse(uint64_t h, int depth, uint32_t& x0, uint32_t& x1, uint32_t& x2) {
+    const uint64_t g = h ^ (h >> 1);
+    x0 = compact3(g >> 2);
+    x1 = compact3(g >> 1);
+    x2 = compact3(g);
+    for (int q = 1; q < depth; ++q) {
+        const uint32_t Q = 1u << q, P = Q - 1u;
+        {
+            const uint32_t t = (x0 ^ x2) & P;
+            const bool on = x2 & Q;
+            x0 ^= on ? P : t;
+            x2 ^= on ? 0u : t;
+        }
+        {
+            const uint32_t t = (x0 ^ x1) & P;
+            const bool on = x1 & Q;
+            x0 ^= on ? P : t;
+            x1 ^= on ? 0u : t;
+        }
+        x0 ^= (x0 & Q) ? P : 0u;
+    }
+}
+
 // order id: bit 0 = swap x/y ("-trans"), ids 2..3 = Hilbert.
 PTV3_HD uint64_t curve_code(int id, uint32_t x, uint32_t y, uint32_t z, int depth) {
     const uint32_t a = (id & 1) ? y : x;
     const uint32_t b = (id & 1) ? x : y;
     return (id < 2) ? interleave(a, b, z) : hilbert3(a, b, z, depth);
+}
+
+// Inverse of curve_code on a code below 2^(3 depth).
+PTV3_HD void curve_point(int id, uint64_t c, int depth, uint32_t& x, uint32_t& y, uint32_t& z) {
+    uint32_t a, b;
+    if (id < 2) {
+        a = compact3(c >> 2);
+        b = compact3(c >> 1);
+        z = compact3(c);
+    } else {
+        hilbert3_inverse(c, depth, a, b, z);
+    }
+    x = (id & 1) ? b : a;
+    y = (id & 1) ? a : b;
 }
 
 }  // namespace ptv3

@@ -197,6 +197,19 @@ def encode_orders(grid_coord, batch, depth, orders):
     return code
 
 
+def decode_order(code, depth, order, with_batch=True):
+    """Inverse of one row of encode_orders: (grid_coord (N,3) int64, batch (N,) int64 or None)."""
+    _dev(code)
+    lib = _lib.load()
+    c = code.to(torch.int64).contiguous().reshape(-1)
+    n = c.shape[0]
+    grid = torch.empty((n, 3), dtype=torch.int64, device=c.device)
+    batch = torch.empty((n,), dtype=torch.int64, device=c.device) if with_batch else None
+    _lib.check(lib.ptv3_decode(_ptr(c), n, int(depth), ORDER_IDS[order], _ptr(grid), _ptr(batch), _stream()),
+               "ptv3_decode")
+    return grid, batch
+
+
 def grid_max(grid_coord):
     """Per-axis maximum of (N,3) int32 coordinates as a (3,) int32 device tensor."""
     _dev(grid_coord)

@@ -36,6 +36,10 @@ def test_argument_errors_without_a_device():
     assert lib.ptv3_encode(None, None, 0, 8, ids, 1, None, None) == 0         # empty input is fine
     bad = (ctypes.c_int32 * 1)(7)
     assert lib.ptv3_encode(None, None, 0, 8, bad, 1, None, None) == -1        # unknown order
+    assert lib.ptv3_decode(None, 10, 17, 0, None, None, None) == -2
+    assert lib.ptv3_decode(None, 10, 8, 4, None, None, None) == -1            # unknown order
+    assert lib.ptv3_decode(None, 10, 8, 0, None, None, None) == -1            # null pointers
+    assert lib.ptv3_decode(None, 0, 8, 2, None, None, None) == 0
     assert lib.ptv3_argsort(None, 10, 4, 64, None, None, None, 0, None) == -2  # > 63 bits (model.py:103)
     assert lib.ptv3_argsort(None, 0, 4, 30, None, None, None, 0, None) == 0
     assert lib.ptv3_patch_attn_fwd(None, 1, 10, 64, 2, None, None, None, 1, 1024, 0.25, None, None) == -4

@@ -48,6 +48,64 @@ def test_encode_mirror_of_reference_signature():
     assert encode(to_dev(g), b, 16, "z").tolist() == [(3 << 48) | 4, (3 << 48) | 36, (3 << 48) | (1 << 26)]
 
 
+@pytest.mark.parametrize("name", sorted(k[:-3] for k in GOLD.files if k.endswith("_in")))
+def test_hilbert_decode_kernel_inverts_reference_golden(name):
+    """The codes the reference's hilbert.py encode wrote for these points decode back to the points."""
+    from pointtransformerv3_amd.serialization import hilbert_decode
+    depth = int(name.split("_d")[1])
+    got = hilbert_decode(to_dev(GOLD[name + "_out"]), depth)
+    # ("trunc" holds coordinates past the depth: encode keeps their low bits, decode returns those)
+    assert got.dtype == torch.int64 and np.array_equal(got.cpu().numpy(), GOLD[name + "_in"] & ((1 << depth) - 1))
+
+
+@pytest.mark.parametrize("depth", [1, 4, 8, 9, 12, 16])
+@pytest.mark.parametrize("n", [1, 63, 100_003])
+def test_decode_matches_oracle(depth, n):
+    """Random codes (not only images of encode), with a batch index above the curve bits."""
+    from pointtransformerv3_amd import serialization as PS
+    rng = np.random.default_rng(100 * depth + n % 97)
+    low = rng.integers(0, 1 << (3 * depth), size=n, dtype=np.int64)
+    b = rng.integers(0, 1 << min(15, 63 - 3 * depth), size=n, dtype=np.int64)
+    code = (b << np.int64(3 * depth)) | low
+    for order, ref in (("z", OS.z_order_decode), ("hilbert", OS.hilbert_decode)):
+        grid, batch = PS.decode(to_dev(code), depth, order)
+        assert np.array_equal(grid.cpu().numpy(), ref(low, depth)), order
+        assert np.array_equal(batch.cpu().numpy(), b), order
+    assert np.array_equal(PS.z_order_decode(to_dev(low), depth).cpu().numpy(), OS.z_order_decode(low, depth))
+    assert np.array_equal(PS.hilbert_decode(to_dev(low), depth).cpu().numpy(), OS.hilbert_decode(low, depth))
+    # the transposed orders through the operator layer: decode of encode is the identity for all four
+    g = rng.integers(0, 1 << depth, size=(n, 3)).astype(np.int32)
+    codes = ops().encode_orders(to_dev(g), to_dev(b), depth, list(OS.ORDERS))
+    for r, order in enumerate(OS.ORDERS):
+        grid, batch = ops().decode_order(codes[r], depth, order)
+        assert np.array_equal(grid.cpu().numpy(), g) and np.array_equal(batch.cpu().numpy(), b), order
+
+
+def test_decode_round_trip_full_size():
+    from pointtransformerv3_amd import serialization as PS
+    rng = np.random.default_rng(5)
+    g = to_dev(rng.integers(0, 1 << 16, size=(6_400_000, 3)).astype(np.int32))
+    b = to_dev(np.sort(rng.integers(0, 4, size=6_400_000)).astype(np.int64))
+    for order in ("z", "hilbert"):
+        grid, batch = PS.decode(PS.encode(g, b, 16, order), 16, order)
+        assert torch.equal(grid, g.long()) and torch.equal(batch, b)
+    assert torch.equal(PS.z_order_decode(PS.z_order_encode(g, 16), 16), g.long())
+    assert torch.equal(PS.hilbert_decode(PS.hilbert_encode(g, 16), 16), g.long())
+
+
+def test_decode_mirror_of_reference_signature():
+    from pointtransformerv3_amd.serialization import decode, z_order_decode
+    from pointtransformerv3_amd._lib import Ptv3Error
+    code = to_dev(np.array([4, 36, 1 << 26, (3 << 48) | 7], np.int64))
+    grid, batch = decode(code, 16, "z")
+    assert grid.tolist() == [[1, 0, 0], [3, 0, 0], [256, 0, 0], [1, 1, 1]] and batch.tolist() == [0, 0, 0, 3]
+    assert z_order_decode(code[:0], 16).shape == (0, 3)
+    with pytest.raises(AssertionError):
+        decode(code, 16, "z-trans")             # default.py:29 takes "z" and "hilbert" only
+    with pytest.raises(Ptv3Error):
+        decode(code, 17, "z")
+
+
 def test_encode_rejects_bad_depth_and_cpu_tensors():
     from pointtransformerv3_amd._lib import Ptv3Error
     g = to_dev(np.zeros((4, 3), np.int32))

@@ -86,6 +86,25 @@ def test_z_order_matches_byte_lut_form():
         assert np.array_equal(S.z_order_code(p.astype(np.int32), depth), key)
 
 
+def test_hilbert_decode_inverts_reference_golden():
+    """hilbert_decode on the codes the reference's own hilbert.py wrote for the fixture's points."""
+    import os
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "hilbert_golden.npz"))
+    names = sorted(k[:-3] for k in gold.files if k.endswith("_in"))
+    assert names
+    for name in names:
+        depth = int(name.split("_d")[1])
+        # ("trunc" holds coordinates past the depth: encode keeps their low bits, decode returns those)
+        assert np.array_equal(S.hilbert_decode(gold[name + "_out"], depth), gold[name + "_in"] & ((1 << depth) - 1)), name
+
+
+def test_z_order_decode_hand_cases():
+    """Bit 3i+2 is x's bit i, 3i+1 y's, 3i z's (z_order.py:66-101 read backwards)."""
+    code = np.array([0b100, 0b010, 0b001, 0b100100, 1 << 26, (1 << 48) - 1], np.int64)
+    want = [[1, 0, 0], [0, 1, 0], [0, 0, 1], [3, 0, 0], [256, 0, 0], [65535, 65535, 65535]]
+    assert S.z_order_decode(code, 16).tolist() == want
+
+
 @pytest.mark.parametrize("depth", [1, 5, 8, 9, 12, 16])
 def test_roundtrip_and_c_agreement(depth):
     rng = np.random.default_rng(depth)
