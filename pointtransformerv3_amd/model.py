@@ -119,10 +119,10 @@ class PointTransformerV3(PointModule):
     def forward(self, data_dict):
         """data_dict: feat, grid_coord (or coord + grid_size), offset or batch. Returns the Point
         whose feat is (N, dec_channels[0]) in the original point order."""
-        if torch.is_grad_enabled():
-            # an optimizer that writes the parameters behind autograd's back (fused kernels, .data) leaves no
-            # trace on them: the half-precision copies of the masters are redone once per training forward
-            ops.invalidate_casts()
+        # whoever writes the parameters behind autograd's back (fused optimizer kernels, .data, weight surgery
+        # under no_grad) leaves no trace on them: the derived copies (half-precision casts of float masters,
+        # the tile convolutions' packed weights) are redone once per forward, in evaluation as well
+        ops.invalidate_casts()
         point = Point(data_dict)
         # the pair lists of the stem and of the first stage's xCPE depend on the coordinates only:
         # their first halves are queued behind the first host read-back and run while the host waits

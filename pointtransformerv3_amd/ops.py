@@ -72,8 +72,9 @@ def _cast_shape(t, layout):
 def invalidate_casts():
     """Declare every remembered parameter copy stale. In-place updates through torch show in the parameter's
     version counter, which cast_cached checks by itself; fused optimizers (torch.optim.AdamW(fused=True)) write
-    the parameters without touching it, so every optimizer step calls this through a global post-step hook,
-    and so does the model at the start of a training forward. Call it after writing parameters some other way."""
+    the parameters without touching it, and so does a write through .data: every optimizer step calls this through
+    a global post-step hook, and so does the model at the start of every forward. Code that calls the operators
+    without the model calls it after writing parameters some other way."""
     _CAST_EPOCH[0] += 1
 
 

@@ -1,9 +1,12 @@
 """Device-side voxelisation and collation in front of PointTransformerV3.forward.
 
-Pointcept prepares a batch on the host (GridSample: grid coordinates relative to the scene minimum,
-one point kept per voxel; then the scenes are concatenated with cumulative `offset`); the model
-itself only has a fallback that derives grid_coord (model.py:88-96). grid_sample does that step
-on the GPU for a whole batch at once and returns the dictionary the model's forward takes."""
+This is this package's own contract, not a mirror of anything in the reference: the reference tree holds the
+model only, whose sole voxelisation is the fallback that derives grid_coord from coord with the batch-wide minimum
+and truncation (model.py:88-96; Point does the same when grid_coord is missing). The transform a training
+pipeline runs on the host before the model is not part of that tree, so which points survive here (voxel
+boundaries, the point kept per voxel) is pinned only by this repository's brute-force check, not by parity
+with such a pipeline. grid_sample computes floor((coord - minimum of the point's own scene) / grid_size), keeps
+one point per voxel, and returns the dictionary the model's forward takes, for a whole batch at once."""
 import torch
 
 from . import ops
@@ -14,8 +17,8 @@ def grid_sample(coord, offset, grid_size, feat=None, keys=(), mode="test", seed=
     """coord (N,3) float, offset (B,) cumulative scene ends, both on the GPU.
 
     Keeps one point of every grid_size voxel of every scene: the first in input order with mode "test", a
-    member drawn uniformly with mode "train" (GridSample's two modes; the draw follows `seed`, or torch's CPU
-    generator when seed is None -- not numpy's stream, which the reference's pipeline uses). Returns a dict
+    member drawn uniformly with mode "train" (the draw follows `seed`, or torch's CPU generator when seed is
+    None; it reproduces no other library's random stream). Returns a dict
     ready for PointTransformerV3.forward: coord, grid_coord, offset, grid_size, feat (if given,
     rows of the kept points), plus index (kept input rows) and inverse (voxel of every input point),
     and any extra per-point tensors passed in `keys` as (name, tensor) pairs, gathered alike."""

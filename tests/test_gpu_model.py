@@ -333,3 +333,40 @@ def test_forward_fp16_without_any_library_gemm():
         ops.LIBRARY_GEMM = True
     want = ptv3_forward(sd, d["grid_coord"], x, d["offset"], perms=perms)
     assert rel_err(point.feat, want) < 2e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_eval_forward_follows_parameters_written_through_data(dtype):
+    """A write through .data leaves no trace on a parameter's version counter; the derived copies (packed weights of
+    the tile convolutions in a half model, half copies of float masters under autocast) are redone at every forward,
+    so an evaluation forward after such a write computes with the new values."""
+    from pointtransformerv3_amd import PointTransformerV3
+    torch.manual_seed(3)
+    model = PointTransformerV3(shuffle_orders=False).eval().to(DEV)
+    if dtype == torch.float16:
+        model = model.half()
+    d, feat = _data(20000, 1, grid=0.02)
+    x = feat.astype(np.float16).astype(np.float32)
+
+    def run():
+        torch.manual_seed(11)   # the pooling layers draw their order permutations from torch's CPU generator
+        with torch.autocast("cuda", dtype=torch.float16, enabled=dtype == torch.float32):
+            return _run(model, d, x, dtype).feat.float().clone()
+
+    first = run()
+    assert torch.equal(run(), first)
+    # a 64-channel xCPE convolution (tile form in half precision) and a Linear weight
+    conv = model.enc.enc1.block0.cpe[0]
+    assert conv.in_channels == 64
+    saved = conv.weight.data.clone()
+    with torch.no_grad():
+        version = conv.weight._version
+        conv.weight.data.mul_(2.0)
+        assert conv.weight._version == version          # nothing for a version check to see
+        changed = run()
+        assert not torch.equal(changed, first)
+        conv.weight.data.copy_(saved)
+        assert torch.equal(run(), first)
+        fc = model.enc.enc2.block1.mlp[0].fc1
+        fc.weight.data.mul_(0.5)
+        assert not torch.equal(run(), first)
