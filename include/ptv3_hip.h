@@ -274,6 +274,14 @@ int ptv3_subm_conv_tiles_fwd(const void *feat, int dtype, int64_t n, int channel
                              const void *packed_weight, const void *bias, const int32_t *tile_tap,
                              const int32_t *tile_pair, const int32_t *vox_taps, void *out, void *stream);
 
+/* model.py:546-552 (spconv.SubMConv3d, 3x3x3, in == out channels) where a voxel has few neighbours: the same
+ * tiles and packed weight as ptv3_subm_conv_tiles_fwd, but the work is in proportion to the pairs (an MFMA row
+ * is a pair, not an output voxel with or without the tap) and nothing but feat, the lists and out touches
+ * memory. channels 32 or 64; f16 / bf16. */
+int ptv3_subm_conv_sparse_fwd(const void *feat, int dtype, int64_t n, int channels, int taps,
+                              const void *packed_weight, const void *bias, const int32_t *tile_tap,
+                              const int32_t *tile_pair, void *out, void *stream);
+
 /* model.py:652-664,690-695: clusters of code0 >> shift walked in sorted order (order0 sorts
  * code0, so no further sort is needed). Outputs: cluster (n,) int64 [pooling_inverse],
  * indices (n,) int64 (= order0: points grouped by cluster), idx_ptr (n+1 allocated, m+1 used),

@@ -770,6 +770,33 @@ def subm_conv_tiles(feat, plan, packed_weight, bias=None):
     return out
 
 
+CONV_SPARSE_CHANNELS = (32, 64)   # cin == cout widths of the sparse tile form
+
+
+def subm_conv_sparse(feat, plan, packed_weight, bias=None):
+    """3x3x3 submanifold convolution with cin == cout where voxels have few neighbours: the tiles and packed
+    weight of subm_conv_tiles, work in proportion to the pairs (fp16 / bf16)."""
+    _dev(feat, packed_weight, bias)
+    lib = _lib.load()
+    feat = feat.contiguous()
+    n, c = feat.shape
+    assert packed_weight.dtype == feat.dtype and packed_weight.numel() == plan.taps * c * c
+    b = None if bias is None else bias.to(feat.dtype).contiguous()
+    out = torch.empty((n, c), dtype=feat.dtype, device=feat.device)
+    tile_tap, tile_pair, _ = plan.tiles()
+
+    def call():
+        _lib.check(lib.ptv3_subm_conv_sparse_fwd(_ptr(feat), _dtype_code(feat), n, c, plan.taps, _ptr(packed_weight),
+                                                 _ptr(b), _ptr(tile_tap), _ptr(tile_pair), _ptr(out), _stream()),
+                   "ptv3_subm_conv_sparse_fwd")
+
+    if _LAUNCH_TIMER is not None:
+        _LAUNCH_TIMER.launch("subm_conv", (plan.n_pairs, n, c, c, plan.taps, "sparse"), call)
+    else:
+        call()
+    return out
+
+
 class PendingClusters:
     __slots__ = ("cluster", "idx_ptr", "head", "count", "read", "with_offset")
 

@@ -81,6 +81,9 @@ class SubMConv3d(nn.Module):
     # from this many pairs per voxel on, the tile form (sums kept on chip, no pair matrix through memory)
     # measured faster than the pair form at 64 and 128 channels; sparser levels stay on the pair form
     TILE_MODE_MIN_PAIRS_PER_VOXEL = 4.0
+    # 32 and 64 channels: the sparse tile form (work in proportion to the pairs) up to this many pairs per voxel;
+    # measured faster than both other forms from 2.5 to 10 pairs per voxel, a full grid (27) is the tile form's case
+    SPARSE_MODE_MAX_PAIRS_PER_VOXEL = 14.0
 
     def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
                  groups=1, bias=True, indice_key=None):
@@ -113,8 +116,8 @@ class SubMConv3d(nn.Module):
 
     def convolve(self, x, feat, weight, bias, packed=None):
         """The convolution of feat (N, Cin) over x's neighbourhoods with weight (Cout, V, Cin), on whichever
-        form fits: dense output-stationary (fp32, or many active taps), pair lists, or tiles. packed() hands
-        out the weight in the tile kernel's order when the caller has it cached."""
+        form fits: dense output-stationary (fp32, or many active taps), pair lists, tiles, or sparse tiles.
+        packed() hands out the weight in the tile kernels' order when the caller has it cached."""
         cout, _, cin = weight.shape
         if feat.dtype == torch.float32:
             nbr = x.neighbour_map(self.kernel_size, self.indice_key)
@@ -125,6 +128,10 @@ class SubMConv3d(nn.Module):
             feat = nn.functional.pad(feat, (0, pad))
             weight = nn.functional.pad(weight, (0, pad))
         plan = x.conv_plan(self.kernel_size, self.indice_key)
+        if (self.kernel_size == 3 and cin == cout and cin in ops.CONV_SPARSE_CHANNELS and plan.n < (1 << 24)
+                and plan.n_pairs <= self.SPARSE_MODE_MAX_PAIRS_PER_VOXEL * plan.n):
+            tiles = packed() if packed is not None else ops.conv_pack_weight(weight, 27, feat.dtype)
+            return ops.subm_conv_sparse(feat, plan, tiles, bias)
         if (self.kernel_size == 3 and cin == cout and cin in ops.CONV_TILE_CHANNELS
                 and plan.n < (1 << 24) and plan.n_pairs >= self.TILE_MODE_MIN_PAIRS_PER_VOXEL * plan.n):
             tiles = packed() if packed is not None else ops.conv_pack_weight(weight, 27, feat.dtype)

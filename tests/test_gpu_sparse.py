@@ -529,6 +529,37 @@ def test_subm_conv_tiles_parity(dtype, c, n, extent):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("c,n,extent", [(64, 3000, 20), (64, 50_000, 60), (32, 9000, 24), (32, 2000, 12), (64, 2, 4),
+                                        (32, 900, 8), (64, 40_001, 90), (32, 60_000, 120), (64, 400, 6), (32, 2, 3),
+                                        (64, 2400, 11), (32, 1900, 10)])
+def test_subm_conv_sparse_parity(dtype, c, n, extent):
+    """Sparse tile form of the xCPE convolution (an MFMA row is a pair, sums in LDS) against the oracle, from
+    scans with a neighbour or two per voxel to full grids (all 27 taps, several blocks per tap), the same bits
+    on every run, and the same result as the other two forms up to the rounding of their sums."""
+    rng = np.random.default_rng(c + n)
+    g = torch.Generator().manual_seed(c + n)
+    idx, *_ = _indices(rng, n // 2, extent, 2)
+    nbr = OI.subm_kmap(idx, 3)
+    feat = torch.randn(len(idx), c, generator=g).to(dtype)
+    bound = 1.0 / np.sqrt(27 * c)
+    w = ((torch.rand(c, 3, 3, 3, c, generator=g) * 2 - 1) * bound * 3).to(dtype)
+    b = ((torch.rand(c, generator=g) * 2 - 1) * 0.2).to(dtype)
+    want = OF.subm_conv(feat.float(), nbr, w.float(), b.float())
+    o = ops()
+    plan = o.conv_plan_direct(to_dev(idx), 3)
+    packed = o.conv_pack_weight(w.to(DEV), 27, dtype)
+    got = o.subm_conv_sparse(feat.to(DEV), plan, packed, b.to(DEV))
+    assert got.dtype == dtype and got.shape == (len(idx), c)
+    assert rel_err(got, want) < TOL[dtype]
+    again = o.subm_conv_sparse(feat.to(DEV), plan, packed, b.to(DEV))
+    assert torch.equal(got, again)
+    nob = o.subm_conv_sparse(feat.to(DEV), plan, packed, None)
+    assert rel_err(nob, OF.subm_conv(feat.float(), nbr, w.float(), None)) < TOL[dtype]
+    pairs = o.subm_conv_pairs(feat.to(DEV), plan, w.reshape(c, 27, c).to(DEV), b.to(DEV))
+    assert rel_err(got, pairs.float().cpu()) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("c,n,mode", [(128, 5001, 3), (128, 77, 2), (256, 3000, 3), (256, 40_001, 2), (256, 1, 3), (128, 33, 3)])
 def test_linear_ln_parity(dtype, c, n, mode):
     """Square Linear + LayerNorm(s) + residual in one kernel (model.py:541-545,587-597) against torch in
