@@ -183,13 +183,23 @@ def attention_config2(reps, dtype=torch.float16):
 ENC_CHANNELS = (32, 64, 128, 256, 512)
 
 
+class _FormProbe:
+    """Stands in for the launch timer for one call: remembers the form of the convolution that was launched."""
+    form = "dense"
+
+    def launch(self, kind, work, call):
+        if kind == "subm_conv":
+            self.form = work[-1]
+        call()
+
+
 def conv_case(which, reps):
-    """The xCPE convolution alone, through the module's own dispatch (pair, tile or dense form), fp16:
+    """The xCPE convolution alone, through the module's own dispatch (pair, tile, sparse tile or dense form), fp16:
     `config3` = baseline config 3 (200,000 room voxels at 2 cm, 64 -> 64); `level0` .. `level4` = the voxel set
     of that encoder level of the benchmark batch (4 rooms pooled with stride 2 per level) at that level's width.
     Returns the time per call against both rooflines (printed as one JSON line by --conv: the command to put under
     rocprofv3)."""
-    from pointtransformerv3_amd import synthetic
+    from pointtransformerv3_amd import ops, synthetic
     from pointtransformerv3_amd.sparse import SparseConvTensor, SubMConv3d
     dev = "cuda:0"
     if which == "config3":
@@ -211,7 +221,11 @@ def conv_case(which, reps):
     with torch.inference_mode():
         plan = x.conv_plan(3, "bench")
         per_voxel = plan.n_pairs / n
-        form = ("tile" if channels in (64, 128) and per_voxel >= SubMConv3d.TILE_MODE_MIN_PAIRS_PER_VOXEL else "pair")
+        probe = _FormProbe()          # which form the module's dispatch picks: what the operator layer reports
+        ops.set_launch_timer(probe)
+        conv(x)
+        ops.set_launch_timer(None)
+        form = probe.form
         us = _time_us(lambda: conv(x), iters=reps, warmup=2)
     flops = 2.0 * plan.n_pairs * channels * channels
     min_bytes = 2.0 * n * channels * 2 + 27.0 * channels * channels * 2 + 4.0 * plan.n_pairs
@@ -572,7 +586,7 @@ def main():
                      "attn_ms_per_step": attn_ms / args.steps,
                      "valu_exp_floor_ms_per_step": exp_floor_ms / args.steps,
                      "valu_exp_frac": exp_floor_ms / attn_ms if attn_ms > 0 else 0.0,
-                     "conv": {"kernels": "pair_wstat / pair_gemm / subm_conv_pairs + pair_segment_sum, conv_tile",
+                     "conv": {"kernels": "conv_sparse, conv_tile, pair_wstat / pair_gemm + pair_segment_sum",
                               "bound": "mfma", "launches": conv_launches, "ms_per_step": conv_ms / args.steps,
                               "achieved": conv_tf, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                               "frac": conv_tf / MFMA_PEAK_TFLOPS,
