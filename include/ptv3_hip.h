@@ -270,6 +270,18 @@ int64_t ptv3_conv_plan_tile_count(int64_t n);
 int ptv3_conv_plan_tiles(const int32_t *row_ptr, const int32_t *slot_pair, int64_t n, int taps,
                          int32_t *tile_tap, int32_t *tile_pair, int32_t *vox_taps, void *stream);
 int ptv3_subm_conv_pack_weight(const void *weight, int dtype, int channels, int taps, void *packed, void *stream);
+/* ptv3_subm_conv_pack_weight for several weights in one launch (a model repacks all of them when its parameters
+ * may have changed). The table lies in device memory; first_block is the running sum of
+ * ptv3_subm_conv_pack_weight_blocks(channels, taps) over the jobs before this one, n_blocks the sum over all.
+ * Shapes in the table are not checked: a wrong table writes out of bounds. */
+typedef struct {
+    const void *weight;   /* (channels, taps, channels), f16 or bf16 */
+    void *packed;         /* same size and type */
+    int32_t channels, taps;
+    int64_t first_block;
+} ptv3_pack_job;
+int64_t ptv3_subm_conv_pack_weight_blocks(int channels, int taps);
+int ptv3_subm_conv_pack_weight_batch(const ptv3_pack_job *jobs, int n_jobs, int64_t n_blocks, void *stream);
 int ptv3_subm_conv_tiles_fwd(const void *feat, int dtype, int64_t n, int channels, int taps,
                              const void *packed_weight, const void *bias, const int32_t *tile_tap,
                              const int32_t *tile_pair, const int32_t *vox_taps, void *out, void *stream);

@@ -80,6 +80,28 @@ __global__ __launch_bounds__(CT_THREADS) void pack_weight_kernel(const T* __rest
     *(u32x4*)(packed + idx * 8) = *(const u32x4*)(w + ((int64_t)co * taps + t) * c + k);
 }
 
+// the same for several weights in one launch: job j owns blocks first_block[j] .. first_block[j + 1]
+__global__ __launch_bounds__(CT_THREADS) void pack_weight_batch_kernel(const ptv3_pack_job* __restrict__ jobs, int n_jobs) {
+    int j = 0;
+    for (int i = 1; i < n_jobs; ++i)
+        if (jobs[i].first_block <= (int64_t)blockIdx.x) j = i;   // uniform: a handful of jobs, first_block ascending
+    const ptv3_pack_job job = jobs[j];
+    const int c = job.channels, taps = job.taps;
+    const int64_t total = (int64_t)taps * c * c / 8;
+    const int64_t idx = ((int64_t)blockIdx.x - job.first_block) * CT_THREADS + threadIdx.x;
+    if (idx >= total) return;
+    const int lane = (int)(idx % 64);
+    int64_t r = idx / 64;
+    const int steps = c / 16, slices = c / 32;
+    const int st = (int)(r % steps);
+    r /= steps;
+    const int sl = (int)(r % slices);
+    const int t = (int)(r / slices);
+    const int co = 32 * sl + lane % 32, k = 16 * st + 8 * (lane / 32);
+    const uint16_t* w = (const uint16_t*)job.weight;   // both half types are 16-bit patterns here
+    *(u32x4*)((uint16_t*)job.packed + idx * 8) = *(const u32x4*)(w + ((int64_t)co * taps + t) * c + k);
+}
+
 // output-major pair words from the tap-major lists: slot_pair[pair_slot[q]] = tap(q) << 24 | pair_in[q]
 __global__ __launch_bounds__(CT_THREADS) void plan_slots_kernel(const int32_t* __restrict__ tap_ptr, int taps,
                                                                 const int32_t* __restrict__ pair_in,
@@ -407,6 +429,20 @@ extern "C" int ptv3_subm_conv_pack_weight(const void* weight, int dtype, int cha
     // both half types are 16-bit patterns here: one instantiation moves either
     hipLaunchKernelGGL(pack_weight_kernel<_Float16>, grid, dim3(CT_THREADS), 0, (hipStream_t)stream_,
                        (const _Float16*)weight, channels, taps, (_Float16*)packed);
+    PTV3_RETURN_LAUNCH();
+}
+
+extern "C" int64_t ptv3_subm_conv_pack_weight_blocks(int channels, int taps) {
+    if (channels < 32 || channels % 32 != 0 || taps < 1) return 0;
+    return ptv3_ceil_div((int64_t)taps * channels * channels / 8, CT_THREADS);
+}
+
+extern "C" int ptv3_subm_conv_pack_weight_batch(const ptv3_pack_job* jobs, int n_jobs, int64_t n_blocks, void* stream_) {
+    if (n_jobs < 0 || n_blocks < 0 || n_blocks > 0x7fffffffLL) return PTV3_EINVAL;
+    if (n_jobs == 0 || n_blocks == 0) return PTV3_OK;
+    if (!jobs) return PTV3_EINVAL;
+    hipLaunchKernelGGL(pack_weight_batch_kernel, dim3((unsigned)n_blocks), dim3(CT_THREADS), 0, (hipStream_t)stream_, jobs,
+                       n_jobs);
     PTV3_RETURN_LAUNCH();
 }
 

@@ -770,6 +770,49 @@ def subm_conv_tiles(feat, plan, packed_weight, bias=None):
     return out
 
 
+_PACK_JOB = np.dtype([("weight", "<u8"), ("packed", "<u8"), ("channels", "<i4"), ("taps", "<i4"),
+                      ("first_block", "<i8")])   # ptv3_pack_job
+_PACK_TABLES = {}
+
+
+def repack_conv_weights(modules, dtype, device):
+    """Packed (fragment-order) copies, in dtype, of the weights of every 3x3x3 cin == cout convolution in `modules`
+    whose copy is missing or older than its parameter (parameter_stamp): one launch for all of them. A module keeps
+    its copies in module._packed[dtype] = ((stamp, device), tensor); float masters go through cast_cached first."""
+    lib = _lib.load()
+    jobs, blocks, done = [], 0, []
+    for m in list(modules):
+        w = m.weight
+        if w.device != device or m.kernel_size != 3 or m.in_channels != m.out_channels or m.in_channels % 32:
+            continue
+        if not isinstance(getattr(m, "_packed", None), dict):
+            m._packed = {}
+        now = (parameter_stamp(w), w.device)
+        held = m._packed.get(dtype)
+        if held is not None and held[0] == now:
+            continue
+        src = cast_cached(w, dtype).detach()
+        if not src.is_contiguous():
+            src = src.contiguous()
+        packed = held[1] if held is not None and held[1].device == device else torch.empty(
+            (m.out_channels, 27, m.in_channels), dtype=dtype, device=device)
+        jobs.append((src.data_ptr(), packed.data_ptr(), m.in_channels, 27, blocks))
+        blocks += lib.ptv3_subm_conv_pack_weight_blocks(m.in_channels, 27)
+        done.append((m, now, packed, src))
+    if not jobs:
+        return
+    table = np.array(jobs, dtype=_PACK_JOB).tobytes()
+    held = _PACK_TABLES.get((device, dtype))
+    if held is None or held[0] != table:
+        held = (table, torch.frombuffer(bytearray(table), dtype=torch.uint8).to(device))
+        _PACK_TABLES[(device, dtype)] = held
+    with torch.cuda.device(device):
+        _lib.check(lib.ptv3_subm_conv_pack_weight_batch(held[1].data_ptr(), len(jobs), blocks, _stream()),
+                   "ptv3_subm_conv_pack_weight_batch")
+    for m, now, packed, _ in done:
+        m._packed[dtype] = (now, packed)
+
+
 CONV_SPARSE_CHANNELS = (32, 64)   # cin == cout widths of the sparse tile form
 
 

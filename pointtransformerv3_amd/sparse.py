@@ -105,14 +105,15 @@ class SubMConv3d(nn.Module):
             nn.init.uniform_(self.bias, -bound, bound)
 
     def _packed_weight(self, dtype):
-        """The weight in the tile kernel's fragment order, repacked when the parameter changes."""
+        """The weight in the tile kernels' fragment order, repacked when the parameter may have changed -- together
+        with every other convolution's that is stale, in one launch (ops.repack_conv_weights)."""
         w = self.weight
-        key = (ops.parameter_stamp(w), dtype, w.device)   # fused optimizers leave the version counter alone
-        cached = getattr(self, "_packed", None)
-        if cached is None or cached[0] != key:
-            packed = ops.conv_pack_weight(w.detach().reshape(self.out_channels, -1, self.in_channels), 27, dtype)
-            self._packed = cached = (key, packed)
-        return cached[1]
+        held = self._packed.get(dtype) if isinstance(getattr(self, "_packed", None), dict) else None
+        if held is None or held[0] != (ops.parameter_stamp(w), w.device):
+            _PACKED_USERS.add(self)
+            ops.repack_conv_weights(_PACKED_USERS, dtype, w.device)
+            held = self._packed[dtype]
+        return held[1]
 
     def convolve(self, x, feat, weight, bias, packed=None):
         """The convolution of feat (N, Cin) over x's neighbourhoods with weight (Cout, V, Cin), on whichever
@@ -150,6 +151,11 @@ class SubMConv3d(nn.Module):
             return x.replace_feature(SubMConv.apply(feat, self.weight, self.bias, x, self))
         weight = self.weight.reshape(self.out_channels, -1, self.in_channels)
         return x.replace_feature(self.convolve(x, feat, weight, self.bias, lambda: self._packed_weight(feat.dtype)))
+
+
+# the convolutions that have been asked for packed weights: one stale weight has all stale ones repacked together
+import weakref   # noqa: E402
+_PACKED_USERS = weakref.WeakSet()
 
 
 def is_spconv_module(module):

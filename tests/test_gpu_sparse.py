@@ -528,6 +528,37 @@ def test_subm_conv_tiles_parity(dtype, c, n, extent):
     assert rel_err(nob, OF.subm_conv(feat.float(), nbr, w.float(), None)) < TOL[dtype]
 
 
+def test_repack_conv_weights_batch_equals_single_packs():
+    """One launch repacks every stale convolution weight; each result equals the single-weight packing, float
+    masters included (their half copy is made first), and only stale copies are touched."""
+    from pointtransformerv3_amd.sparse import SubMConv3d
+    o = ops()
+    torch.manual_seed(4)
+    mods = [SubMConv3d(c, c, 3).to(DEV) for c in (32, 64, 128, 64)] + [SubMConv3d(6, 32, 5).to(DEV)]
+    mods[1].half()
+    for dtype in (torch.float16, torch.bfloat16):
+        o.repack_conv_weights(mods, dtype, torch.device(DEV))
+        assert not hasattr(mods[4], "_packed") or dtype not in mods[4]._packed     # 5x5x5, cin != cout: not packable
+        for m in mods[:4]:
+            c = m.in_channels
+            if m.weight.dtype == torch.float16 and dtype == torch.bfloat16:
+                want = o.conv_pack_weight(m.weight.detach().to(dtype).reshape(c, 27, c), 27, dtype)
+            else:
+                want = o.conv_pack_weight(m.weight.detach().reshape(c, 27, c), 27, dtype)
+            assert torch.equal(m._packed[dtype][1], want), (c, dtype)
+    # nothing stale: no launch, same tensors; one weight written through .data after invalidate: only that one changes
+    before = [m._packed[torch.float16][1].clone() for m in mods[:4]]
+    o.repack_conv_weights(mods, torch.float16, torch.device(DEV))
+    assert all(torch.equal(a, m._packed[torch.float16][1]) for a, m in zip(before, mods[:4]))
+    mods[2].weight.data.mul_(3.0)
+    o.invalidate_casts()
+    o.repack_conv_weights(mods, torch.float16, torch.device(DEV))
+    assert not torch.equal(before[2], mods[2]._packed[torch.float16][1])
+    assert torch.equal(before[0], mods[0]._packed[torch.float16][1])
+    assert torch.equal(mods[2]._packed[torch.float16][1],
+                       o.conv_pack_weight(mods[2].weight.detach().reshape(128, 27, 128), 27, torch.float16))
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("c,n,extent", [(64, 3000, 20), (64, 50_000, 60), (32, 9000, 24), (32, 2000, 12), (64, 2, 4),
                                         (32, 900, 8), (64, 40_001, 90), (32, 60_000, 120), (64, 400, 6), (32, 2, 3),
