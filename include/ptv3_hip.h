@@ -251,8 +251,8 @@ int ptv3_subm_conv_pairs_fwd(const void *feat, int dtype, int64_t n, int cin, in
                              const int32_t *pair_in, const int32_t *pair_slot, const void *weight,
                              const void *bias, int cout, void *y, void *out, void *stream);
 
-/* Tile form of the 3x3x3 convolution with cin == cout == channels in {32, 64, 128, 256} (the xCPE of
- * every block, model.py:546-552), fp16/bf16: a work-group keeps the fp32 sums of a tile of 128
+/* Tile form of the 3x3x3 convolution with cin == cout == channels in {64, 128} (the xCPE of
+ * every block, model.py:546-552; ptv3_subm_conv_pack_weight itself takes any multiple of 32), fp16/bf16: a work-group keeps the fp32 sums of a tile of 128
  * consecutive output voxels on chip and walks their pairs tap by tap, so no product row per pair
  * goes through memory; sums in tap order, nothing atomic, same result on every run.
  * Lists, made once per plan (n < 2^24, taps == 27):
