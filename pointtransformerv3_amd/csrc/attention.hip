@@ -147,8 +147,8 @@ template <typename T, bool LSE, bool DROP>
 __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
     const T* __restrict__ qkv, int channels, int heads, const int32_t* __restrict__ slot_src,
     const int32_t* __restrict__ slot_dst, const int32_t* __restrict__ cu_seqlens, int lds_keys,
-    float scale_log2e, T* __restrict__ out, int full_items, int split, float* __restrict__ lse, int64_t lse_stride,
-    Dropout drop) {
+    float scale_log2e, T* __restrict__ out, int full_items, int split, int total_items, float* __restrict__ lse,
+    int64_t lse_stride, Dropout drop) {
     typedef typename Half<T>::v8 v8;
     extern __shared__ __align__(16) unsigned char smem[];
     // K tile: lds_keys + 64 rows of 32 B (the last 64 are only ever prefetched). V^T tile: 16 rows
@@ -167,10 +167,15 @@ __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
     if ((int)blockIdx.x < full_items) {
         wg = xcd_chunked_id(blockIdx.x, full_items);
     } else {
+        // the ranges of one item take work-group ids 8 apart, one after the other: they run on the same XCD
+        // (ids go round the XCDs; full_items is a multiple of the resident work-groups) at about the same time,
+        // so the keys and values the later ranges stage are in that XCD's L2
         const int r = blockIdx.x - full_items;
-        wg = full_items + r / split;
-        part = r % split;
+        const int xcd = r & 7, j = r >> 3;
+        wg = full_items + (j / split) * 8 + xcd;
+        part = j % split;
         parts = split;
+        if (wg >= total_items) return;
     }
     const int seq = wg / heads, head = wg % heads;
     const int s0 = cu_seqlens[seq];
@@ -482,9 +487,10 @@ int launch_half(const void* qkv, int channels, int heads, const int32_t* slot_sr
         }
     }
     if (split == 1) full = total;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(full + (total - full) * split)), dim3(ATT_THREADS), lds, stream,
+    const int64_t tail = (total - full + 7) / 8 * 8;   // the tail's items in groups of 8, one per XCD
+    hipLaunchKernelGGL(kern, dim3((unsigned)(full + tail * split)), dim3(ATT_THREADS), lds, stream,
                        (const T*)qkv, channels, heads, slot_src, slot_dst, cu_seqlens, lds_keys,
-                       scale_log2e, (T*)out, (int)full, (int)split, lse, lse_stride, drop);
+                       scale_log2e, (T*)out, (int)full, (int)split, (int)total, lse, lse_stride, drop);
     PTV3_RETURN_LAUNCH();
 }
 
