@@ -167,15 +167,17 @@ __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
     if ((int)blockIdx.x < full_items) {
         wg = xcd_chunked_id(blockIdx.x, full_items);
     } else {
-        // the ranges of one item take work-group ids 8 apart, one after the other: they run on the same XCD
-        // (ids go round the XCDs; full_items is a multiple of the resident work-groups) at about the same time,
-        // so the keys and values the later ranges stage are in that XCD's L2
+        // Work-group ids go round the XCDs (full_items is a multiple of the resident work-groups). Every XCD takes a
+        // contiguous eighth of the tail's items, range after range of one item, then the next item: the ranges of
+        // an item meet in one L2 (the keys and values the later ranges stage are there), and so do the heads of a
+        // sequence, which read neighbouring pieces of the same cache lines.
         const int r = blockIdx.x - full_items;
         const int xcd = r & 7, j = r >> 3;
-        wg = full_items + (j / split) * 8 + xcd;
+        const int per = (total_items - full_items + 7) >> 3;
+        wg = full_items + xcd * per + j / split;
         part = j % split;
         parts = split;
-        if (wg >= total_items) return;
+        if (j / split >= per || wg >= total_items) return;
     }
     const int seq = wg / heads, head = wg % heads;
     const int s0 = cu_seqlens[seq];
