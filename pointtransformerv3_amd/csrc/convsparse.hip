@@ -89,7 +89,9 @@ __global__ __launch_bounds__(64) void conv_sparse_kernel(const T* __restrict__ f
     __shared__ uint32_t items[SP_MAX_ITEMS + 1];
 
     const int lane = threadIdx.x, col = lane & 31, hf = lane >> 5;
-    const int tile = blockIdx.x;
+    // work-group ids go round the XCDs: every XCD works through one contiguous eighth of the tiles, so that tiles
+    // which gather the same neighbour rows (voxels of a pooled level are in curve order) meet in one L2
+    const int tile = xcd_chunked_id(blockIdx.x, gridDim.x);
     const int cout0 = blockIdx.y * CW;
     const int64_t v0 = (int64_t)tile * SP_TV;
     const int nv = (int)min((int64_t)SP_TV, n - v0);

@@ -228,8 +228,9 @@ __global__ __launch_bounds__(TileShape<C>::THREADS, TileShape<C>::OCC) void conv
     const int col = lane & 31, hf = lane >> 5;
     const int cw = wave % CW, pw = wave / CW;
     const int cout0 = blockIdx.y * COUT_WG;             // first output channel of the work-group
-    // (giving each XCD one contiguous range of tiles instead of round-robin measured no faster)
-    const int tile = blockIdx.x;
+    // work-group ids go round the XCDs: every XCD works through one contiguous eighth of the tiles, so that tiles
+    // which gather the same neighbour rows meet in one L2 (no faster, but half the HBM reads)
+    const int tile = xcd_chunked_id(blockIdx.x, gridDim.x);
     const int64_t v0 = (int64_t)tile * TV;
     const int nv = (int)min((int64_t)TV, n - v0);
 
