@@ -321,6 +321,14 @@ def kernel_rooflines(path):
     add("argsort+inverse", f"4 x {nb} codes, {bits} significant bits, {passes} passes", "hbm",
         4.0 * nb * (passes * 24 + 16), us, f"B ({passes * 24 + 16} B per point and order)")
     del code_big
+    # ---- for scale: a device-to-device copy of as many bytes as the encode above moves (what a kernel that does
+    # nothing but move its algorithmic bytes reaches on this part)
+    half_bytes = nb * 52 // 2 // 8 * 8
+    src = torch.zeros(half_bytes // 8, dtype=torch.int64, device=dev)
+    dst = torch.empty_like(src)
+    us = _time_us(lambda: dst.copy_(src), iters=20)
+    add("device copy (reference)", f"{half_bytes / 1e6:.0f} MB read + {half_bytes / 1e6:.0f} MB written", "hbm", 2.0 * half_bytes, us, "B")
+    del src, dst
     # ---- padding tables + slot tables
     off_host = [int(v) for v in d["offset"]]
     off = torch.from_numpy(d["offset"]).to(dev)
