@@ -128,6 +128,19 @@ __global__ __launch_bounds__(64) void conv_sparse_kernel(const T* __restrict__ f
         for (int e = lane; e < SP_TV * Q; e += 64) *(f32x4*)(sums + (e / Q) * SS + (e % Q) * 4) = b4;
     }
     __builtin_amdgcn_wave_barrier();   // the block table is read next (LDS serves a wave's accesses in order)
+    if (n_items == 0) {   // no pairs at all (never for a submanifold map, whose voxels pair with themselves): bias rows
+        constexpr int E0 = CW / 8;
+        for (int e = lane; e < nv * E0; e += 64) {
+            const int r = e / E0, c8 = e % E0;
+            u32x4 o;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                o[j] = SpOps<T>::pack2(bias ? (float)bias[cout0 + c8 * 8 + 2 * j] : 0.f,
+                                       bias ? (float)bias[cout0 + c8 * 8 + 2 * j + 1] : 0.f);
+            *(u32x4*)(out + (v0 + r) * C + cout0 + c8 * 8) = o;
+        }
+        return;
+    }
 
     // descriptors of the blocks k0 .. k0 + 2D - 1 (da) and k0 + 2D .. k0 + 4D - 1 (db) as scalars: one LDS read per
     // 2D blocks; past the end the last block repeats (its loads are valid, its products go to the spare row)

@@ -2,6 +2,7 @@
 kernels. Stands in for the two spconv types the reference touches (model.py:165-172,
 :233-236, :546-552, :767-774): same constructor arguments and attribute names."""
 import math
+import weakref
 
 import torch
 import torch.nn as nn
@@ -154,7 +155,6 @@ class SubMConv3d(nn.Module):
 
 
 # the convolutions that have been asked for packed weights: one stale weight has all stale ones repacked together
-import weakref   # noqa: E402
 _PACKED_USERS = weakref.WeakSet()
 
 
