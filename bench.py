@@ -389,6 +389,9 @@ def kernel_rooflines(path):
     us = _time_us(lambda: ops.subm_conv_tiles(feat, plan, packed, bias))
     add("subm_conv tiles<f16>", f"{nv} voxels, {plan.n_pairs} pairs ({plan.n_pairs / nv:.2f}/voxel), 64->64", "mfma",
         2.0 * plan.n_pairs * 64 * 64, us, "FLOP (2 * P_act * Cin * Cout)")
+    us = _time_us(lambda: ops.subm_conv_sparse(feat, plan, packed, bias))
+    add("subm_conv sparse tiles<f16>", f"{nv} voxels, {plan.n_pairs} pairs ({plan.n_pairs / nv:.2f}/voxel), 64->64", "mfma",
+        2.0 * plan.n_pairs * 64 * 64, us, "FLOP (2 * P_act * Cin * Cout); the form the model's dispatch picks here")
     # the level the forward runs the tile form on: the 4-scene batch pooled twice (8 cm voxels), 128 channels
     lvl = torch.unique(torch.cat([b[:, None].int(), (g >> 2).int()], 1), dim=0).contiguous()
     nl = len(lvl)
