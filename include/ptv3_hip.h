@@ -513,6 +513,16 @@ int ptv3_mlp_fused(const void *x, const void *resid, const void *w1, const void 
                    const void *b2, int dtype, int64_t n, int channels, int hidden, void *out,
                    void *stream);
 
+/* The same MLP (model.py:510-516, :602) at 128, 256 or 512 channels with both weight matrices handed over in the
+ * order the kernel streams them, so that every MFMA operand fragment is one contiguous KB (the layers' own
+ * (out, in) layout costs the kernel 32 cache lines per load instruction). ptv3_mlp_pack_weights writes that
+ * copy: packed holds 8 * channels^2 elements of dtype, first w1 (4 * channels, channels) and w2 (channels,
+ * 4 * channels) interleaved chunk by chunk; redo it whenever the parameters change. Same results, bit for bit,
+ * as ptv3_mlp_fused. */
+int ptv3_mlp_pack_weights(const void *w1, const void *w2, int dtype, int channels, void *packed, void *stream);
+int ptv3_mlp_fused_packed(const void *x, const void *resid, const void *packed, const void *b1, const void *b2,
+                          int dtype, int64_t n, int channels, void *out, void *stream);
+
 /* Head of a block for thin channels, model.py:541-545, :587-589, :592-593 and :450 in one kernel:
  *   feat = shortcut + LayerNorm_cpe(conv @ w_cpe^T + b_cpe)
  *   qkv  = LayerNorm_1(feat) @ w_qkv^T + b_qkv

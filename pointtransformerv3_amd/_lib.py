@@ -95,6 +95,8 @@ SIGNATURES = {
     "ptv3_linear_wgrad": (_i32, [_vp, _vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
     "ptv3_linear_ln_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _f32, _vp, _vp, _vp]),
     "ptv3_mlp_fused": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _vp, _vp]),
+    "ptv3_mlp_pack_weights": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp]),
+    "ptv3_mlp_fused_packed": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _vp, _vp]),
     "ptv3_block_head_fused": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _vp, _f32, _vp, _vp, _i32, _i64, _i32,
                                      _vp, _vp, _vp]),
     "ptv3_block_tail_fused": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32,

@@ -14,6 +14,10 @@
 // is fetched into LDS twice, and the weight stream runs DEPTH steps ahead in a ring of registers
 // that is never drained: its addresses do not depend on the tile, so it runs on across stages,
 // chunks and tiles of the persistent work-group.
+// Read from the Linear layers' own (out, in) layout such a step touches 32 weight rows with 2 x 16 bytes each
+// per instruction, and the texture path spends a cycle per lane and line on that: three to four times what a
+// contiguous KB costs. ptv3_mlp_pack_weights therefore writes both matrices once in the order of the stream
+// (step, 32-unit block, piece, lane), and the PACKED kernel fetches every fragment as one contiguous KB.
 // Intermediates are rounded to the storage type where the separate layers would have stored them.
 #include "rowtile.h"
 
@@ -23,7 +27,25 @@ constexpr int MW_THREADS = 512;
 constexpr int MW_WAVES = MW_THREADS / PTV3_WAVE;
 constexpr int MW_PAD = 8;   // halfs of padding per LDS row
 
-template <typename T, int C, int WM, int WN, int MT, int DEPTH>
+// weight step u of the stream (UNITS = 8 C / 32 of them): chunk u / (2 KU), stage (u / KU) & 1 (fc1, fc2), 32-wide
+// contraction step kk = u % KU with KU = C / 32. Piece j of lane (col, hf) for the 32-unit block ub holds inputs
+// 32 kk + 16 hf + 8 j .. + 8 of unit 32 ub + col: row chunk C + unit of fc1, or row unit of fc2 from column chunk C on.
+// packed[((u * (C / 32) + ub) * 2 + j) * 512 + lane * 8 .. + 8]
+template <typename T>
+__global__ __launch_bounds__(256) void mlp_pack_kernel(const T* __restrict__ w1, const T* __restrict__ w2, int c,
+                                                        T* __restrict__ packed) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;   // one 16-byte piece each
+    if (idx >= (int64_t)c * c) return;                            // 8 C^2 elements in pieces of 8
+    const int lane = (int)(idx % 64), j = (int)(idx / 64 % 2), ub = (int)(idx / 128 % (c / 32));
+    const int u = (int)(idx / 128 / (c / 32)), ku = c / 32;
+    const int chunk = u / (2 * ku), st = (u / ku) & 1, kk = u % ku;
+    const int unit = ub * 32 + lane % 32, k = kk * 32 + (lane / 32) * 16 + j * 8;
+    const T* src = st == 0 ? w1 + (int64_t)(chunk * c + unit) * c + k : w2 + (int64_t)unit * 4 * c + chunk * c + k;
+    *(u32x4*)(packed + idx * 8) = *(const u32x4*)src;
+}
+
+// PACKED: w1 is the packed stream of both matrices and w2 is not read
+template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED>
 __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
     const T* __restrict__ x, const T* __restrict__ resid, const T* __restrict__ w1, const T* __restrict__ b1,
     const T* __restrict__ w2, const T* __restrict__ b2, int64_t n, T* __restrict__ out) {
@@ -51,6 +73,12 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
         const int chunk = u / (2 * KU), st = (u / KU) & 1, kk = u % KU;
 #pragma unroll
         for (int a = 0; a < MT; ++a) {
+            if (PACKED) {
+                const T* p = w1 + ((u * (C / 32) + wn * MT + a) * 2) * 512 + lane * 8;
+                r[a][0] = *(const u32x4*)p;
+                r[a][1] = *(const u32x4*)(p + 512);
+                continue;
+            }
             const int unit = ch0 + a * 32 + col;
             const T* p = st == 0 ? w1 + (int64_t)(chunk * C + unit) * C + kk * 32 + hf * 16
                                  : w2 + (int64_t)unit * H + chunk * C + kk * 32 + hf * 16;
@@ -181,12 +209,12 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
     }
 }
 
-template <typename T, int C, int WM, int WN, int MT, int DEPTH>
+template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED>
 int launch_mlp_wide(const void* x, const void* resid, const void* w1, const void* b1, const void* w2, const void* b2,
                     int64_t n, void* out, hipStream_t stream) {
     constexpr int R = 64 * WM;
     const size_t lds = (size_t)2 * R * (C + MW_PAD) * sizeof(T);
-    auto kern = mlp_wide_kernel<T, C, WM, WN, MT, DEPTH>;
+    auto kern = mlp_wide_kernel<T, C, WM, WN, MT, DEPTH, PACKED>;
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -202,19 +230,46 @@ int launch_mlp_wide(const void* x, const void* resid, const void* w1, const void
     return e == hipSuccess ? PTV3_OK : (int)e;
 }
 
-}  // namespace
-
-// called by ptv3_mlp_fused for channels 128, 256 and 512
-int mlp_wide_dispatch(const void* x, const void* resid, const void* w1, const void* b1, const void* w2, const void* b2,
-                  int dtype, int64_t n, int channels, void* out, hipStream_t stream) {
-#define PTV3_MW(T)                                                                                                  \
-    do {                                                                                                            \
-        if (channels == 128) return launch_mlp_wide<T, 128, 2, 4, 1, 4>(x, resid, w1, b1, w2, b2, n, out, stream);   \
-        if (channels == 256) return launch_mlp_wide<T, 256, 1, 8, 1, 4>(x, resid, w1, b1, w2, b2, n, out, stream);   \
-        if (channels == 512) return launch_mlp_wide<T, 512, 1, 8, 2, 2>(x, resid, w1, b1, w2, b2, n, out, stream);   \
+template <bool PACKED>
+int mlp_wide_any(const void* x, const void* resid, const void* w1, const void* b1, const void* w2, const void* b2,
+                 int dtype, int64_t n, int channels, void* out, hipStream_t stream) {
+#define PTV3_MW(T)                                                                                                          \
+    do {                                                                                                                    \
+        if (channels == 128) return launch_mlp_wide<T, 128, 2, 4, 1, 4, PACKED>(x, resid, w1, b1, w2, b2, n, out, stream);   \
+        if (channels == 256) return launch_mlp_wide<T, 256, 1, 8, 1, 4, PACKED>(x, resid, w1, b1, w2, b2, n, out, stream);   \
+        if (channels == 512) return launch_mlp_wide<T, 512, 1, 8, 2, 2, PACKED>(x, resid, w1, b1, w2, b2, n, out, stream);   \
     } while (0)
     if (dtype == PTV3_F16) PTV3_MW(_Float16);
     if (dtype == PTV3_BF16) PTV3_MW(__bf16);
 #undef PTV3_MW
     return PTV3_ESHAPE;
+}
+
+}  // namespace
+
+// called by ptv3_mlp_fused for channels 128, 256 and 512
+int mlp_wide_dispatch(const void* x, const void* resid, const void* w1, const void* b1, const void* w2, const void* b2,
+                      int dtype, int64_t n, int channels, void* out, hipStream_t stream) {
+    return mlp_wide_any<false>(x, resid, w1, b1, w2, b2, dtype, n, channels, out, stream);
+}
+
+extern "C" int ptv3_mlp_pack_weights(const void* w1, const void* w2, int dtype, int channels, void* packed, void* stream_) {
+    if (channels != 128 && channels != 256 && channels != 512) return PTV3_ESHAPE;
+    if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
+    if (!w1 || !w2 || !packed) return PTV3_EINVAL;
+    const int64_t pieces = (int64_t)channels * channels;
+    // both half types are 16-bit patterns here: one instantiation moves either
+    hipLaunchKernelGGL(mlp_pack_kernel<_Float16>, dim3((unsigned)ptv3_ceil_div(pieces, 256)), dim3(256), 0,
+                       (hipStream_t)stream_, (const _Float16*)w1, (const _Float16*)w2, channels, (_Float16*)packed);
+    PTV3_RETURN_LAUNCH();
+}
+
+extern "C" int ptv3_mlp_fused_packed(const void* x, const void* resid, const void* packed, const void* b1, const void* b2,
+                                     int dtype, int64_t n, int channels, void* out, void* stream_) {
+    if (n < 0) return PTV3_EINVAL;
+    if (channels != 128 && channels != 256 && channels != 512) return PTV3_ESHAPE;
+    if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
+    if (n == 0) return PTV3_OK;
+    if (!x || !resid || !packed || !b1 || !b2 || !out) return PTV3_EINVAL;
+    return mlp_wide_any<true>(x, resid, packed, b1, nullptr, b2, dtype, n, channels, out, (hipStream_t)stream_);
 }

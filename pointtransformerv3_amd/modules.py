@@ -442,7 +442,7 @@ class Block(PointModule):
             feat, normed = ops.layer_norm(branch, ln2.weight, ln2.bias, ln2.eps, residual=feat, mode=2, shift=shift)
         if fused_mlp:
             # fc1 + GELU + fc2 + residual in one kernel, the 4C-wide hidden tensor never leaves the CU
-            feat = ops.mlp_fused(normed, feat, mlp.fc1.weight, mlp.fc1.bias, mlp.fc2.weight, mlp.fc2.bias)
+            feat = ops.mlp_fused_module(normed, feat, mlp)
         elif plain_mlp:
             hidden = ops.linear(normed, mlp.fc1, gelu=True) if exact_gelu else mlp.act(mlp.fc1(normed))
             if (not ops.LIBRARY_GEMM and ops.linear_gemm_ok(hidden, mlp.fc2.weight) and feat.is_contiguous()

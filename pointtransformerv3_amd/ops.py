@@ -1316,6 +1316,57 @@ def mlp_fused(x, resid, w1, b1, w2, b2):
     return out
 
 
+MLP_PACKED_CHANNELS = (128, 256, 512)               # widths whose fused MLP streams its weights from a packed copy
+
+
+def mlp_pack_weights(w1, w2, dtype, out=None):
+    """fc1's (4C, C) and fc2's (C, 4C) weights in the order the wide fused MLP kernel streams them, as one
+    tensor of 8 C^2 elements of dtype (ptv3_mlp_pack_weights); written into `out` when given."""
+    _dev(w1, w2)
+    lib = _lib.load()
+    c = w2.shape[0]
+    assert c in MLP_PACKED_CHANNELS and tuple(w1.shape) == (4 * c, c) and tuple(w2.shape) == (c, 4 * c)
+    w1c, w2c = w1.detach().to(dtype).contiguous(), w2.detach().to(dtype).contiguous()
+    if out is None:
+        out = torch.empty(8 * c * c, dtype=dtype, device=w1.device)
+    assert out.dtype == dtype and out.numel() == 8 * c * c and out.is_contiguous()
+    _lib.check(lib.ptv3_mlp_pack_weights(_ptr(w1c), _ptr(w2c), _DTYPE_CODE[dtype], c, _ptr(out), _stream()),
+               "ptv3_mlp_pack_weights")
+    return out
+
+
+def mlp_fused_packed(x, resid, packed, b1, b2):
+    """mlp_fused with the weights as mlp_pack_weights leaves them (C in MLP_PACKED_CHANNELS): same results."""
+    _dev(x, resid, packed, b1, b2)
+    lib = _lib.load()
+    x = x.contiguous()
+    resid = resid.to(x.dtype).contiguous()
+    n, c = x.shape
+    dt = x.dtype
+    assert packed.dtype == dt and packed.numel() == 8 * c * c
+    b1c, b2c = b1.to(dt).contiguous(), b2.to(dt).contiguous()
+    out = torch.empty_like(x)
+    _lib.check(lib.ptv3_mlp_fused_packed(_ptr(x), _ptr(resid), _ptr(packed), _ptr(b1c), _ptr(b2c), _dtype_code(x),
+                                         n, c, _ptr(out), _stream()), "ptv3_mlp_fused_packed")
+    return out
+
+
+def mlp_fused_module(x, resid, mlp):
+    """resid + mlp(x) from the fused kernel for a module with fc1 and fc2. At MLP_PACKED_CHANNELS the weights go
+    through a packed copy that the module keeps per dtype and that is redone, in place, when a parameter may have
+    changed (parameter_stamp)."""
+    w1, w2 = mlp.fc1.weight, mlp.fc2.weight
+    if x.shape[1] not in MLP_PACKED_CHANNELS:
+        return mlp_fused(x, resid, w1, mlp.fc1.bias, w2, mlp.fc2.bias)
+    held = mlp.__dict__.setdefault("_packed_stream", {})
+    key = (parameter_stamp(w1), parameter_stamp(w2), w1.device)
+    entry = held.get(x.dtype)
+    if entry is None or entry[0] != key:
+        packed = mlp_pack_weights(w1, w2, x.dtype, out=None if entry is None or entry[0][2] != w1.device else entry[1])
+        held[x.dtype] = entry = (key, packed)
+    return mlp_fused_packed(x, resid, entry[1], mlp.fc1.bias, mlp.fc2.bias)
+
+
 def _opt(t, dt):
     return None if t is None else t.to(dt).contiguous()
 

@@ -254,6 +254,53 @@ def test_mlp_fused_parity(dtype, c, n):
     assert got.dtype == dtype and rel_err(got, want) < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("c,n", [(128, 1), (128, 40_001), (256, 64), (256, 20_001), (512, 9000)])
+def test_mlp_fused_packed_weights_give_the_same_bits(dtype, c, n):
+    """The packed weight stream only changes where the kernel finds its operands: against the torch fp32 layers
+    within the half-precision bar, and bit for bit what the kernel gives on the layers' own layout."""
+    import torch.nn.functional as F
+    o = ops()
+    g = torch.Generator().manual_seed(3 * c + n)
+    x = torch.randn(n, c, generator=g).to(dtype)
+    r = torch.randn(n, c, generator=g).to(dtype)
+    w1 = (torch.randn(4 * c, c, generator=g) / c ** 0.5).to(dtype)
+    b1 = (torch.randn(4 * c, generator=g) * 0.5).to(dtype)
+    w2 = (torch.randn(c, 4 * c, generator=g) / (4 * c) ** 0.5).to(dtype)
+    b2 = (torch.randn(c, generator=g) * 0.5).to(dtype)
+    want = r.float() + F.linear(F.gelu(F.linear(x.float(), w1.float(), b1.float())), w2.float(), b2.float())
+    dx, dr, dw1, db1, dw2, db2 = (t.to(DEV) for t in (x, r, w1, b1, w2, b2))
+    packed = o.mlp_pack_weights(dw1, dw2, dtype)
+    # the packed copy is a permutation of the two matrices' elements
+    assert torch.equal(packed.view(torch.int16).sort().values,
+                       torch.cat([dw1.flatten(), dw2.flatten()]).view(torch.int16).sort().values)
+    got = o.mlp_fused_packed(dx, dr, packed, db1, db2)
+    assert got.dtype == dtype and rel_err(got, want) < TOL[dtype]
+    assert torch.equal(got, o.mlp_fused(dx, dr, dw1, db1, dw2, db2))
+
+
+def test_mlp_fused_module_repacks_after_a_parameter_write():
+    from pointtransformerv3_amd.modules import MLP
+    o = ops()
+    torch.manual_seed(5)
+    mlp = MLP(128, 512).half().to(DEV)
+    x = torch.randn(500, 128, device=DEV).half()
+    r = torch.randn(500, 128, device=DEV).half()
+    plain = lambda: o.mlp_fused(x, r, mlp.fc1.weight, mlp.fc1.bias, mlp.fc2.weight, mlp.fc2.bias)
+    first = o.mlp_fused_module(x, r, mlp)
+    assert torch.equal(first, plain())
+    held = mlp._packed_stream[torch.float16][1]
+    with torch.no_grad():
+        mlp.fc2.weight.mul_(0.5)              # bumps the version counter
+    second = o.mlp_fused_module(x, r, mlp)
+    assert torch.equal(second, plain()) and not torch.equal(second, first)
+    assert mlp._packed_stream[torch.float16][1] is held     # redone in place
+    mlp.fc1.weight.data.mul_(2.0)             # no version bump: callers announce it
+    o.invalidate_casts()
+    assert torch.equal(o.mlp_fused_module(x, r, mlp), plain())
+    assert "_packed_stream" not in mlp.state_dict()
+
+
 def _lin(cin, cout, g, dtype, bias=True):
     m = torch.nn.Linear(cin, cout, bias=bias)
     with torch.no_grad():
