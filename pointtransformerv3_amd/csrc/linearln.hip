@@ -6,8 +6,8 @@
 //          accumulate onto out0 later, as in the LayerNorm kernel's mode 2)
 //   mode 3 (xCPE, model.py:587-593): s = res + LN(Linear(x)); out0 = s; out1 = LN2(s)
 //          (cpe.1 Linear, cpe.2 LayerNorm, the residual, then the attention's pre-norm)
-// for C = 128 and 256 channels in and out (64 and below are covered by the block head / tail
-// kernels). Every intermediate is rounded to the storage type exactly where the separate kernels
+// for C = 128 channels in and out (64 and below are covered by the block head / tail kernels; 256 by the
+// kernel that keeps the weights in registers, linear_wide_kernel with its LN modes). Every intermediate is rounded to the storage type exactly where the separate kernels
 // store it (Linear output, normalised value, sum), so fusing changes no value.
 //
 // Structure as the tall-and-skinny Linear kernel: a wave owns 32 rows as K/16 MFMA operand fragments,
@@ -25,9 +25,9 @@ constexpr int LL_PAD = 8;              // halfs of padding per LDS weight row
 constexpr int LL_XSS = 64 + LL_PAD;    // tile buffer row stride: 64 channels at a time
 
 template <int C> struct LlShape {
-    static constexpr int WAVES = C <= 128 ? 8 : 4;     // 256 channels: the weights leave LDS for 4 tile buffers only
+    static constexpr int WAVES = 8;
     static constexpr int THREADS = WAVES * PTV3_WAVE;
-    static constexpr int OCC = 1;                      // a row's C outputs stay in registers: 256 (C = 128) / 512 per lane
+    static constexpr int OCC = 1;                      // a row's C outputs stay in registers: 256 per lane
     static constexpr size_t LDS = (size_t)C * (C + LL_PAD) * 2 + (size_t)6 * C * 4 + (size_t)WAVES * 32 * LL_XSS * 2;
 };
 
@@ -257,12 +257,16 @@ int dispatch_linear_ln(const void* x, const void* w, const void* bias, const voi
 #define PTV3_LL(C, M)                                                                                           \
     if (c == C && mode == M)                                                                                    \
         return launch_linear_ln<T, C, M>(x, w, bias, res, gamma, beta, gamma2, beta2, shift, n, eps, out0, out1, stream);
-    PTV3_LL(128, 2) PTV3_LL(128, 3) PTV3_LL(256, 2) PTV3_LL(256, 3)
+    PTV3_LL(128, 2) PTV3_LL(128, 3)
 #undef PTV3_LL
     return PTV3_ESHAPE;
 }
 
 }  // namespace
+
+int linear_wide_ln_dispatch(const void* x, const void* w, const void* bias, const void* res, const void* gamma,
+                            const void* beta, const void* gamma2, const void* beta2, const void* shift, int dtype,
+                            int64_t n, int mode, float eps, void* out0, void* out1, hipStream_t stream);
 
 extern "C" int ptv3_linear_ln_fwd(const void* x, const void* w, const void* bias, const void* res, const void* gamma,
                                   const void* beta, const void* gamma2, const void* beta2, const void* shift, int dtype,
@@ -274,6 +278,10 @@ extern "C" int ptv3_linear_ln_fwd(const void* x, const void* w, const void* bias
     if (!x || !w || !res || !gamma || !beta || !out0 || !out1) return PTV3_EINVAL;
     if (mode == 3 && (!gamma2 || !beta2)) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
+    // 256 channels: the kernel that keeps the weights in registers (linearw.hip); below that they fit the LDS
+    if (channels == 256)
+        return linear_wide_ln_dispatch(x, w, bias, res, gamma, beta, gamma2, beta2, shift, dtype, n, mode, eps, out0, out1,
+                                       stream);
     if (dtype == PTV3_F16)
         return dispatch_linear_ln<_Float16>(x, w, bias, res, gamma, beta, gamma2, beta2, shift, n, channels, mode, eps,
                                             out0, out1, stream);

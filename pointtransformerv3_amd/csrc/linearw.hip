@@ -27,10 +27,22 @@ constexpr int LW_K = 256, LW_N = 256;
 constexpr int LW_WSTRIDE = LW_K + 8;
 constexpr int LW_OSTRIDE = 64 + 8;      // halfs per row of a wave's result staging
 
-template <typename T, bool GELU>
+// What follows the Linear when it is the cpe.1 or proj layer of a 256-channel block (LN = 3, 2; model.py:587-597),
+// as in ptv3_linear_ln_fwd: the residual, the LayerNorm(s) and the second output.
+template <typename T> struct LwNorm {
+    const T *res, *gamma, *beta, *gamma2, *beta2, *shift;
+    float eps;
+    T* out1;
+};
+
+// LN = 0: out = act(x W^T + b). LN = 2 / 3 (nout = 256, one tile of output channels, so a work-group holds whole
+// rows): modes 2 / 3 of the Linear + LayerNorm kernel on the accumulators, every intermediate rounded where the
+// separate kernels store it. A row's 256 channels are spread over the four waves of its row half: the sums of a
+// LayerNorm go through LDS (mean first, then the squared deviations), one barrier each.
+template <typename T, bool GELU, int LN>
 __global__ __launch_bounds__(LW_THREADS, 2) void linear_wide_kernel(
     const T* __restrict__ x, const T* __restrict__ weight, const T* __restrict__ bias, int64_t n, int nout,
-    T* __restrict__ out, int span_rows) {
+    T* __restrict__ out, int span_rows, LwNorm<T> ln) {
     typedef typename H16<T>::v8 v8;
     constexpr int KSTEPS = LW_K / LW_KC;       // 4 = depth of the ring
     constexpr int KS = LW_KC / 16;             // MFMA contraction steps per staged step
@@ -105,12 +117,31 @@ __global__ __launch_bounds__(LW_THREADS, 2) void linear_wide_kernel(
     *(u32x4*)xw = ring[0];
     ring[0] = *(const u32x4*)ptr_nxt;   // step KSTEPS = step 0 of the second tile
     __syncthreads();
+    // behind the staging rows, also where the weights were: the LayerNorm parameters and the waves' partial sums
+    float* p_lds = (float*)(w_lds + LW_THREADS / PTV3_WAVE * 32 * LW_OSTRIDE);   // [5][LW_N]
+    float* ex_lds = p_lds + 5 * LW_N;                                            // [4][LW_ROWS][4]
+    if (LN != 0 && tid < LW_N) {
+        p_lds[tid] = (float)ln.gamma[tid];
+        p_lds[LW_N + tid] = (float)ln.beta[tid];
+        p_lds[2 * LW_N + tid] = LN == 3 ? (float)ln.gamma2[tid] : 0.f;
+        p_lds[3 * LW_N + tid] = LN == 3 ? (float)ln.beta2[tid] : 0.f;
+        p_lds[4 * LW_N + tid] = (LN == 2 && ln.shift) ? (float)ln.shift[tid] : 0.f;
+    }   // published by the first barrier of the loop below
     u32x4 xf[2][KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) xf[0][ks] = *(const u32x4*)(xa + ks * 16);
 
     for (int tile = 0; tile < n_tiles; ++tile) {
         const T* ptr_3 = row_ptr(tile + 3);
+        u32x4 resv[LN != 0 ? 4 : 1];   // the residual rows of this wave's 32 x 64 block, whole row segments
+        if (LN != 0) {
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                int64_t r = r0 + (int64_t)tile * LW_ROWS + row0 + it * 8 + (lane >> 3);
+                r = r < n ? r : n - 1;
+                resv[it] = *(const u32x4*)(ln.res + r * LW_N + c0 + (lane & 7) * 8);
+            }
+        }
         f32x16 acc[NT];
 #pragma unroll
         for (int b = 0; b < NT; ++b)
@@ -138,42 +169,141 @@ __global__ __launch_bounds__(LW_THREADS, 2) void linear_wide_kernel(
             __builtin_amdgcn_sched_barrier(0);
         }
         // acc[b][v]: output channel cout0 + c0 + b*32 + 8*(v/4) + 4*hf + v%4 of row row0 + col of the tile
+        auto store_rows = [&](T* dst) {   // the wave's staged 32 x 64 block as whole row segments
+            asm volatile("" ::: "memory");
 #pragma unroll
-        for (int b = 0; b < NT; ++b)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const f32x4 bb = *(const f32x4*)(b_lds + c0 + b * 32 + 8 * q + 4 * hf);
-                float r[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    r[i] = acc[b][4 * q + i] + bb[i];
-                    if (GELU) r[i] = gelu_erf(H16<T>::round(r[i]));
-                }
-                *(u32x2*)(stage + col * LW_OSTRIDE + b * 32 + 8 * q + 4 * hf) =
-                    (u32x2){H16<T>::pack2(r[0], r[1]), H16<T>::pack2(r[2], r[3])};
+            for (int it = 0; it < 4; ++it) {
+                const int orow = it * 8 + (lane >> 3), opc = lane & 7;
+                const u32x4 val = *(const u32x4*)(stage + orow * LW_OSTRIDE + opc * 8);
+                int64_t r = r0 + (int64_t)tile * LW_ROWS + row0 + orow;
+                r = r < n ? r : n - 1;
+                *(u32x4*)(dst + r * nout + cout0 + c0 + opc * 8) = val;
             }
-        asm volatile("" ::: "memory");
+            asm volatile("" ::: "memory");
+        };
+        if constexpr (LN == 0) {
 #pragma unroll
-        for (int it = 0; it < 4; ++it) {
-            const int orow = it * 8 + (lane >> 3), opc = lane & 7;
-            const u32x4 val = *(const u32x4*)(stage + orow * LW_OSTRIDE + opc * 8);
-            int64_t r = r0 + (int64_t)tile * LW_ROWS + row0 + orow;
-            r = r < n ? r : n - 1;
-            *(u32x4*)(out + r * nout + cout0 + c0 + opc * 8) = val;
+            for (int b = 0; b < NT; ++b)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const f32x4 bb = *(const f32x4*)(b_lds + c0 + b * 32 + 8 * q + 4 * hf);
+                    float r[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        r[i] = acc[b][4 * q + i] + bb[i];
+                        if (GELU) r[i] = gelu_erf(H16<T>::round(r[i]));
+                    }
+                    *(u32x2*)(stage + col * LW_OSTRIDE + b * 32 + 8 * q + 4 * hf) =
+                        (u32x2){H16<T>::pack2(r[0], r[1]), H16<T>::pack2(r[2], r[3])};
+                }
+            store_rows(out);
+        } else {
+            // ---- the residual block through the staging rows into accumulator order
+#pragma unroll
+            for (int it = 0; it < 4; ++it)
+                *(u32x4*)(stage + (it * 8 + (lane >> 3)) * LW_OSTRIDE + (lane & 7) * 8) = resv[it];
+            asm volatile("" ::: "memory");
+            float val[NT][16];
+#pragma unroll
+            for (int b = 0; b < NT; ++b)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const f32x4 bb = *(const f32x4*)(b_lds + c0 + b * 32 + 8 * q + 4 * hf);
+                    const u32x2 rp = *(const u32x2*)(stage + col * LW_OSTRIDE + b * 32 + 8 * q + 4 * hf);
+                    const float rr[4] = {H16<T>::lo(rp[0]), H16<T>::hi(rp[0]), H16<T>::lo(rp[1]), H16<T>::hi(rp[1])};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float lin = H16<T>::round(acc[b][4 * q + i] + bb[i]);
+                        // mode 2: the sum is final here; mode 3: the residual waits in the upper half of the pair
+                        val[b][4 * q + i] = LN == 2 ? H16<T>::round(lin + rr[i]) : lin;
+                        if (LN == 3) acc[b][4 * q + i] = rr[i];
+                    }
+                }
+            asm volatile("" ::: "memory");
+            // mean and 1 / std of the wave's row over all 256 channels: slot, slot + 1 of the exchange buffer
+            auto row_stats = [&](int slot, float& mean, float& rstd) {
+                float sum = 0.f;
+#pragma unroll
+                for (int b = 0; b < NT; ++b)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) sum += val[b][v];
+                sum += __shfl_xor(sum, 32, PTV3_WAVE);
+                float* mine = ex_lds + (slot * LW_ROWS + row0 + col) * 4;
+                if (hf == 0) mine[wave & 3] = sum;
+                __syncthreads();
+                const f32x4 ps = *(const f32x4*)mine;
+                mean = (ps[0] + ps[1] + ps[2] + ps[3]) * (1.f / LW_N);
+                float dev = 0.f;
+#pragma unroll
+                for (int b = 0; b < NT; ++b)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) dev += (val[b][v] - mean) * (val[b][v] - mean);
+                dev += __shfl_xor(dev, 32, PTV3_WAVE);
+                if (hf == 0) mine[LW_ROWS * 4 + (wave & 3)] = dev;
+                __syncthreads();
+                const f32x4 pd = *(const f32x4*)(mine + LW_ROWS * 4);
+                rstd = rsqrtf((pd[0] + pd[1] + pd[2] + pd[3]) * (1.f / LW_N) + ln.eps);
+            };
+            float mean, rstd;
+            if (LN == 3) {   // s = res + LN(lin), every stage rounded
+                row_stats(0, mean, rstd);
+#pragma unroll
+                for (int b = 0; b < NT; ++b)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int c = c0 + b * 32 + 8 * q + 4 * hf;
+                        const f32x4 ga = *(const f32x4*)(p_lds + c), be = *(const f32x4*)(p_lds + LW_N + c);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const float y = (val[b][4 * q + i] - mean) * rstd * ga[i] + be[i];
+                            val[b][4 * q + i] = H16<T>::round(H16<T>::round(y) + acc[b][4 * q + i]);
+                        }
+                    }
+            }
+            // ---- out0 = s (+ shift), out1 = LN(s) with the second (mode 3) or only (mode 2) parameters
+#pragma unroll
+            for (int b = 0; b < NT; ++b)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int c = c0 + b * 32 + 8 * q + 4 * hf;
+                    f32x4 sh = {0.f, 0.f, 0.f, 0.f};
+                    if (LN == 2) sh = *(const f32x4*)(p_lds + 4 * LW_N + c);
+                    *(u32x2*)(stage + col * LW_OSTRIDE + b * 32 + 8 * q + 4 * hf) =
+                        (u32x2){H16<T>::pack2(val[b][4 * q] + sh[0], val[b][4 * q + 1] + sh[1]),
+                                H16<T>::pack2(val[b][4 * q + 2] + sh[2], val[b][4 * q + 3] + sh[3])};
+                }
+            store_rows(out);
+            row_stats(2, mean, rstd);
+            const float* ga_l = p_lds + (LN == 3 ? 2 * LW_N : 0);
+            const float* be_l = p_lds + (LN == 3 ? 3 * LW_N : LW_N);
+#pragma unroll
+            for (int b = 0; b < NT; ++b)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int c = c0 + b * 32 + 8 * q + 4 * hf;
+                    const f32x4 ga = *(const f32x4*)(ga_l + c), be = *(const f32x4*)(be_l + c);
+                    float o[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) o[i] = (val[b][4 * q + i] - mean) * rstd * ga[i] + be[i];
+                    *(u32x2*)(stage + col * LW_OSTRIDE + b * 32 + 8 * q + 4 * hf) =
+                        (u32x2){H16<T>::pack2(o[0], o[1]), H16<T>::pack2(o[2], o[3])};
+                }
+            store_rows(ln.out1);
         }
-        asm volatile("" ::: "memory");
         ptr_cur = ptr_nxt;
         ptr_nxt = ptr_nn;
         ptr_nn = ptr_3;
     }
 }
 
-template <typename T, bool GELU>
+template <typename T, bool GELU, int LN = 0>
 int launch_linear_wide(const void* x, const void* w, const void* bias, int64_t n, int nout, void* out,
-                       hipStream_t stream) {
+                       hipStream_t stream, LwNorm<T> ln = LwNorm<T>{}) {
     const size_t lds = ((size_t)LW_N * LW_WSTRIDE + 2 * (size_t)LW_ROWS * LW_XSTRIDE) * sizeof(T) + LW_N * sizeof(float);
     static_assert(8 * 32 * LW_OSTRIDE <= LW_N * LW_WSTRIDE, "the waves' staging rows fit where the weights were");
-    auto kern = linear_wide_kernel<T, GELU>;
+    static_assert((8 * 32 * LW_OSTRIDE) * 2 + (5 * LW_N + 4 * LW_ROWS * 4) * 4 <= LW_N * LW_WSTRIDE * 2,
+                  "staging rows, LayerNorm parameters and partial sums fit where the weights were");
+    auto kern = linear_wide_kernel<T, GELU, LN>;
     static bool allowed = false;   // per instantiation
     if (!allowed) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -188,7 +318,7 @@ int launch_linear_wide(const void* x, const void* w, const void* bias, int64_t n
     int64_t span_rows = ptv3_ceil_div(ptv3_ceil_div(n, spans), LW_ROWS) * LW_ROWS;
     spans = ptv3_ceil_div(n, span_rows);
     hipLaunchKernelGGL(kern, dim3((unsigned)spans, (unsigned)col_tiles), dim3(LW_THREADS), lds, stream, (const T*)x,
-                       (const T*)w, (const T*)bias, n, nout, (T*)out, (int)span_rows);
+                       (const T*)w, (const T*)bias, n, nout, (T*)out, (int)span_rows, ln);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? PTV3_OK : (int)e;
 }
@@ -383,6 +513,23 @@ int launch_linear_gemm(const void* x, const void* w, const void* bias, const voi
 }
 
 }  // namespace
+
+// called by ptv3_linear_ln_fwd for 256 channels (modes 2 and 3)
+int linear_wide_ln_dispatch(const void* x, const void* w, const void* bias, const void* res, const void* gamma,
+                            const void* beta, const void* gamma2, const void* beta2, const void* shift, int dtype,
+                            int64_t n, int mode, float eps, void* out0, void* out1, hipStream_t stream) {
+#define PTV3_LWLN(T, M)                                                                                         \
+    return launch_linear_wide<T, false, M>(x, w, bias, n, LW_N, out0, stream,                                   \
+                                           LwNorm<T>{(const T*)res, (const T*)gamma, (const T*)beta, (const T*)gamma2, \
+                                                     (const T*)beta2, (const T*)shift, eps, (T*)out1})
+    if (dtype == PTV3_F16) {
+        if (mode == 2) PTV3_LWLN(_Float16, 2);
+        PTV3_LWLN(_Float16, 3);
+    }
+    if (mode == 2) PTV3_LWLN(__bf16, 2);
+    PTV3_LWLN(__bf16, 3);
+#undef PTV3_LWLN
+}
 
 extern "C" int ptv3_linear_wide_fwd(const void* x, const void* w, const void* bias, int dtype, int64_t n, int k,
                                     int nout, int gelu, void* out, void* stream_) {

@@ -1091,10 +1091,10 @@ def scaled_add(skip, branch, row_scale, out_dtype):
 
 
 LINEAR_LN_CHANNELS = (128, 256)   # square Linear + LayerNorm(s) + residual in one kernel
-# where that kernel measured faster than Linear kernel + LayerNorm kernel on MI355X: at 128 channels
-# (146k rows: 35 us against 42-49); at 256 the C x C weights fill the LDS, four waves per CU remain
-# and the two kernels win (38k rows: 44-67 us against 33-35)
-LINEAR_LN_PAYS = (128,)
+# where that measured faster than Linear kernel + LayerNorm kernel on MI355X: at 128 channels (weights in LDS;
+# 146k rows: 35 us against 42-49) and at 256 (weights in registers, the LayerNorm sums exchanged between the four
+# waves of a row through LDS; 38k rows: 25-27 us against 37-41)
+LINEAR_LN_PAYS = (128, 256)
 
 
 def linear_ln_ok(x, lin):
