@@ -1222,11 +1222,12 @@ def linear_gemm(x, weight, bias=None, resid=None):
     return out
 
 
-# The three long-contraction layers of the default model (fc2 at 256 and 512 channels, the 512 -> 1536 qkv) are
-# plain GEMMs on which the library's 256 x 160 tiles measured 26-29 us against 43-48 us for this package's
-# 128 x 128-tile kernel (both bound by what the L2s deliver per tile, see csrc/linearw.hip). True: the library GEMM
-# takes them; False: no library call anywhere in the forward.
-LIBRARY_GEMM = True
+# The long-contraction layers of the default model are plain GEMMs: fc2 at 256 and 512 channels (inside the fused
+# MLP kernel by default, see MLP_ONLY_FUSED_PAYS) and the 512 -> 1536 qkv, on which the library's 256 x 160 tiles
+# measured 26-29 us against 43-48 us for this package's 128 x 128-tile kernel (both bound by what the L2s deliver
+# per tile, see csrc/linearw.hip). False: no library call anywhere in the forward (the default: every kernel of
+# the path is this package's own; 0.04 ms per forward slower). True: the library GEMM takes them.
+LIBRARY_GEMM = False
 
 
 def linear_gemm_ok(x, weight):
@@ -1297,7 +1298,10 @@ def linear_bn_act(x, lin, bn, gelu):
 
 MLP_FUSED_CHANNELS = (32, 64)             # widths of the fused block head / tail kernels
 MLP_ONLY_FUSED_CHANNELS = (32, 64, 128, 256, 512)   # widths the fused MLP kernel supports
-MLP_ONLY_FUSED_PAYS = (32, 64, 128)                 # widths at which it beats fc1, GELU and fc2 as three launches
+# widths at which the model uses it. At 32 ... 128 it beats fc1 + GELU and fc2 as separate launches by 1.8-2.4x; at
+# 256 and 512 it is on a par with Linear kernel + library GEMM inside the forward (0.02-0.04 ms per forward slower)
+# and keeps the hidden tensor and the library out of the path; (32, 64, 128) restores the separate layers there
+MLP_ONLY_FUSED_PAYS = (32, 64, 128, 256, 512)
 
 
 def mlp_fused(x, resid, w1, b1, w2, b2):

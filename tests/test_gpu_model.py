@@ -316,9 +316,11 @@ def test_forward_tiny_and_ragged_scenes_fp32(sizes):
     assert rel_err(point.feat, want) < 1e-4
 
 
-def test_forward_fp16_without_any_library_gemm():
-    """ops.LIBRARY_GEMM = False: fc2 of the 256- and 512-channel blocks and the 512 -> 1536 qkv run on this package's
-    tiled GEMM instead of the library's; the forward is then library-free end to end. Same bar."""
+@pytest.mark.parametrize("library", [False, True])
+def test_forward_fp16_with_and_without_the_library_gemm(library):
+    """The default forward makes no library call (ops.LIBRARY_GEMM = False, the fused MLP at every width). The other
+    setting -- fc1 + GELU and fc2 as separate layers from 256 channels on, fc2 and the 512 -> 1536 qkv on the
+    library's GEMM -- is held to the same bar."""
     from pointtransformerv3_amd import PointTransformerV3, ops
     torch.manual_seed(1)
     model = PointTransformerV3(shuffle_orders=False).eval().half()
@@ -326,11 +328,14 @@ def test_forward_fp16_without_any_library_gemm():
     perms = _draw_perms(78, False)
     sd = {k: v.float() for k, v in model.state_dict().items()}
     x = feat.astype(np.float16).astype(np.float32)
-    ops.LIBRARY_GEMM = False
+    assert ops.LIBRARY_GEMM is False and ops.MLP_ONLY_FUSED_PAYS == ops.MLP_ONLY_FUSED_CHANNELS
+    old = ops.LIBRARY_GEMM, ops.MLP_ONLY_FUSED_PAYS
+    if library:
+        ops.LIBRARY_GEMM, ops.MLP_ONLY_FUSED_PAYS = True, (32, 64, 128)
     try:
         point = _run(model.to(DEV), d, x, torch.float16)
     finally:
-        ops.LIBRARY_GEMM = True
+        ops.LIBRARY_GEMM, ops.MLP_ONLY_FUSED_PAYS = old
     want = ptv3_forward(sd, d["grid_coord"], x, d["offset"], perms=perms)
     assert rel_err(point.feat, want) < 2e-2
 
