@@ -520,6 +520,17 @@ int ptv3_mlp_fused(const void *x, const void *resid, const void *w1, const void 
  * 4 * channels) interleaved chunk by chunk; redo it whenever the parameters change. Same results, bit for bit,
  * as ptv3_mlp_fused. */
 int ptv3_mlp_pack_weights(const void *w1, const void *w2, int dtype, int channels, void *packed, void *stream);
+/* The same packing for several MLPs in one launch (after an optimizer step every copy is stale at once): jobs is a
+ * device array, first_block ascending from 0 with job j owning ptv3_mlp_pack_weights_blocks(channels) blocks,
+ * n_blocks their sum. Both half types move as 16-bit patterns, so a table may mix them. */
+typedef struct {
+    const void *w1, *w2;  /* (4 * channels, channels) and (channels, 4 * channels) */
+    void *packed;         /* 8 * channels^2 elements */
+    int32_t channels, reserved;
+    int64_t first_block;
+} ptv3_mlp_pack_job;
+int64_t ptv3_mlp_pack_weights_blocks(int channels);
+int ptv3_mlp_pack_weights_batch(const ptv3_mlp_pack_job *jobs, int n_jobs, int64_t n_blocks, void *stream);
 int ptv3_mlp_fused_packed(const void *x, const void *resid, const void *packed, const void *b1, const void *b2,
                           int dtype, int64_t n, int channels, void *out, void *stream);
 

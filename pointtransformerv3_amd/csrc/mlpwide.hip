@@ -44,6 +44,24 @@ __global__ __launch_bounds__(256) void mlp_pack_kernel(const T* __restrict__ w1,
     *(u32x4*)(packed + idx * 8) = *(const u32x4*)src;
 }
 
+// the same for several MLPs in one launch: job j owns blocks first_block[j] .. first_block[j + 1]
+__global__ __launch_bounds__(256) void mlp_pack_batch_kernel(const ptv3_mlp_pack_job* __restrict__ jobs, int n_jobs) {
+    int j = 0;
+    for (int i = 1; i < n_jobs; ++i)
+        if (jobs[i].first_block <= (int64_t)blockIdx.x) j = i;   // uniform: a handful of jobs, first_block ascending
+    const ptv3_mlp_pack_job job = jobs[j];
+    const int c = job.channels;
+    const int64_t idx = ((int64_t)blockIdx.x - job.first_block) * 256 + threadIdx.x;
+    if (idx >= (int64_t)c * c) return;
+    const int lane = (int)(idx % 64), jj = (int)(idx / 64 % 2), ub = (int)(idx / 128 % (c / 32));
+    const int u = (int)(idx / 128 / (c / 32)), ku = c / 32;
+    const int chunk = u / (2 * ku), st = (u / ku) & 1, kk = u % ku;
+    const int unit = ub * 32 + lane % 32, k = kk * 32 + (lane / 32) * 16 + jj * 8;
+    const uint16_t *w1 = (const uint16_t*)job.w1, *w2 = (const uint16_t*)job.w2;   // both half types: 16-bit patterns
+    const uint16_t* src = st == 0 ? w1 + (int64_t)(chunk * c + unit) * c + k : w2 + (int64_t)unit * 4 * c + chunk * c + k;
+    *(u32x4*)((uint16_t*)job.packed + idx * 8) = *(const u32x4*)src;
+}
+
 // PACKED: w1 is the packed stream of both matrices and w2 is not read
 template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED>
 __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
@@ -261,6 +279,19 @@ extern "C" int ptv3_mlp_pack_weights(const void* w1, const void* w2, int dtype, 
     // both half types are 16-bit patterns here: one instantiation moves either
     hipLaunchKernelGGL(mlp_pack_kernel<_Float16>, dim3((unsigned)ptv3_ceil_div(pieces, 256)), dim3(256), 0,
                        (hipStream_t)stream_, (const _Float16*)w1, (const _Float16*)w2, channels, (_Float16*)packed);
+    PTV3_RETURN_LAUNCH();
+}
+
+extern "C" int64_t ptv3_mlp_pack_weights_blocks(int channels) {
+    if (channels != 128 && channels != 256 && channels != 512) return 0;
+    return ptv3_ceil_div((int64_t)channels * channels, 256);
+}
+
+extern "C" int ptv3_mlp_pack_weights_batch(const ptv3_mlp_pack_job* jobs, int n_jobs, int64_t n_blocks, void* stream_) {
+    if (n_jobs < 0 || n_blocks < 0 || n_blocks > 0x7fffffffLL) return PTV3_EINVAL;
+    if (n_jobs == 0 || n_blocks == 0) return PTV3_OK;
+    if (!jobs) return PTV3_EINVAL;
+    hipLaunchKernelGGL(mlp_pack_batch_kernel, dim3((unsigned)n_blocks), dim3(256), 0, (hipStream_t)stream_, jobs, n_jobs);
     PTV3_RETURN_LAUNCH();
 }
 

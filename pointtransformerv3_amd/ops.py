@@ -4,6 +4,7 @@ torch is used for device memory and the current stream only; every computation h
 the HIP kernels. All tensors must live on the GPU; CPU tensors are rejected.
 """
 import ctypes
+import weakref
 
 import numpy as np
 import torch
@@ -1355,19 +1356,61 @@ def mlp_fused_packed(x, resid, packed, b1, b2):
     return out
 
 
+_MLP_PACK_JOB = np.dtype([("w1", "<u8"), ("w2", "<u8"), ("packed", "<u8"), ("channels", "<i4"), ("reserved", "<i4"),
+                          ("first_block", "<i8")])
+_MLP_PACK_TABLES = {}
+_MLP_PACK_USERS = weakref.WeakSet()   # the MLPs that have asked for packed weights: one stale copy has all redone
+
+
+def repack_mlp_weights(modules, dtype, device):
+    """Packed weight streams, in dtype, of every MLP in `modules` (fc1: C -> 4C, fc2: 4C -> C, C in
+    MLP_PACKED_CHANNELS) whose copy is missing or older than its parameters (parameter_stamp): one launch for all
+    of them. A module keeps its copies in module._packed_stream[dtype] = ((stamps, device), tensor), redone in place."""
+    lib = _lib.load()
+    jobs, blocks, done = [], 0, []
+    for m in list(modules):
+        w1, w2 = m.fc1.weight, m.fc2.weight
+        c = w2.shape[0]
+        if w1.device != device or c not in MLP_PACKED_CHANNELS or tuple(w1.shape) != (4 * c, c) or tuple(w2.shape) != (c, 4 * c):
+            continue
+        held = m.__dict__.setdefault("_packed_stream", {})
+        now = (parameter_stamp(w1), parameter_stamp(w2), device)
+        entry = held.get(dtype)
+        if entry is not None and entry[0] == now:
+            continue
+        s1, s2 = cast_cached(w1, dtype).detach().contiguous(), cast_cached(w2, dtype).detach().contiguous()
+        packed = entry[1] if entry is not None and entry[1].device == device else torch.empty(
+            8 * c * c, dtype=dtype, device=device)
+        jobs.append((s1.data_ptr(), s2.data_ptr(), packed.data_ptr(), c, 0, blocks))
+        blocks += lib.ptv3_mlp_pack_weights_blocks(c)
+        done.append((held, now, packed, s1, s2))
+    if not jobs:
+        return
+    table = np.array(jobs, dtype=_MLP_PACK_JOB).tobytes()
+    kept = _MLP_PACK_TABLES.get((device, dtype))
+    if kept is None or kept[0] != table:
+        kept = (table, torch.frombuffer(bytearray(table), dtype=torch.uint8).to(device))
+        _MLP_PACK_TABLES[(device, dtype)] = kept
+    with torch.cuda.device(device):
+        _lib.check(lib.ptv3_mlp_pack_weights_batch(kept[1].data_ptr(), len(jobs), blocks, _stream()),
+                   "ptv3_mlp_pack_weights_batch")
+    for held, now, packed, _, _ in done:
+        held[dtype] = (now, packed)
+
+
 def mlp_fused_module(x, resid, mlp):
     """resid + mlp(x) from the fused kernel for a module with fc1 and fc2. At MLP_PACKED_CHANNELS the weights go
     through a packed copy that the module keeps per dtype and that is redone, in place, when a parameter may have
-    changed (parameter_stamp)."""
+    changed (parameter_stamp) -- together with every other MLP's that is stale, in one launch."""
     w1, w2 = mlp.fc1.weight, mlp.fc2.weight
     if x.shape[1] not in MLP_PACKED_CHANNELS:
         return mlp_fused(x, resid, w1, mlp.fc1.bias, w2, mlp.fc2.bias)
-    held = mlp.__dict__.setdefault("_packed_stream", {})
-    key = (parameter_stamp(w1), parameter_stamp(w2), w1.device)
-    entry = held.get(x.dtype)
-    if entry is None or entry[0] != key:
-        packed = mlp_pack_weights(w1, w2, x.dtype, out=None if entry is None or entry[0][2] != w1.device else entry[1])
-        held[x.dtype] = entry = (key, packed)
+    held = mlp.__dict__.get("_packed_stream")
+    entry = held.get(x.dtype) if held else None
+    if entry is None or entry[0] != (parameter_stamp(w1), parameter_stamp(w2), w1.device):
+        _MLP_PACK_USERS.add(mlp)
+        repack_mlp_weights(_MLP_PACK_USERS, x.dtype, w1.device)
+        entry = mlp._packed_stream[x.dtype]
     return mlp_fused_packed(x, resid, entry[1], mlp.fc1.bias, mlp.fc2.bias)
 
 

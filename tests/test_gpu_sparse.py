@@ -287,9 +287,14 @@ def test_mlp_fused_module_repacks_after_a_parameter_write():
     x = torch.randn(500, 128, device=DEV).half()
     r = torch.randn(500, 128, device=DEV).half()
     plain = lambda: o.mlp_fused(x, r, mlp.fc1.weight, mlp.fc1.bias, mlp.fc2.weight, mlp.fc2.bias)
+    other = MLP(256, 1024).half().to(DEV)     # a second stale module rides on the same launch
+    o._MLP_PACK_USERS.add(other)
     first = o.mlp_fused_module(x, r, mlp)
     assert torch.equal(first, plain())
     held = mlp._packed_stream[torch.float16][1]
+    for m in (mlp, other):                    # the batch packs what the single call packs
+        assert torch.equal(m._packed_stream[torch.float16][1],
+                           o.mlp_pack_weights(m.fc1.weight, m.fc2.weight, torch.float16))
     with torch.no_grad():
         mlp.fc2.weight.mul_(0.5)              # bumps the version counter
     second = o.mlp_fused_module(x, r, mlp)
