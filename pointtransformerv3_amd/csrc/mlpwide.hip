@@ -3,7 +3,7 @@
 // As separate kernels this is three passes over an N x 4C tensor (fc1 writes it, GELU rewrites it,
 // fc2 reads it); here a work-group keeps a tile of rows on the CU for the whole chain.
 //
-// A work-group of 8 waves owns R = 64 or 128 rows. The hidden axis is cut into four chunks of C
+// A work-group of 8 waves owns R = 64 ... 192 rows (RT = 2 or 3 groups of 32 rows per wave). The hidden axis is cut into four chunks of C
 // units; per chunk, stage A computes GELU(x W1_chunk^T + b1) for the tile into LDS and stage B adds
 // its product with W2's chunk to the output accumulators, which stay in registers across the
 // chunks. Products are taken transposed with v_mfma_f32_32x32x16 (rows of the A operand = output
@@ -63,13 +63,13 @@ __global__ __launch_bounds__(256) void mlp_pack_batch_kernel(const ptv3_mlp_pack
 }
 
 // PACKED: w1 is the packed stream of both matrices and w2 is not read
-template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED>
+template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RT>
 __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
     const T* __restrict__ x, const T* __restrict__ resid, const T* __restrict__ w1, const T* __restrict__ b1,
     const T* __restrict__ w2, const T* __restrict__ b2, int64_t n, T* __restrict__ out) {
     typedef typename H16<T>::v8 v8;
     static_assert(WM * WN == MW_WAVES && C == 32 * MT * WN, "8 waves cover R x C");
-    constexpr int R = 64 * WM, H = 4 * C, XS = C + MW_PAD;
+    constexpr int R = 32 * RT * WM, H = 4 * C, XS = C + MW_PAD;   // a wave owns RT groups of 32 rows
     constexpr int KU = C / 32;            // 32-wide contraction steps per stage
     constexpr int UNITS = 4 * 2 * KU;     // weight steps per tile: 4 chunks x (stage A, stage B)
     static_assert(KU % DEPTH == 0, "the ring is indexed statically");
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
     const int col = lane & 31, hf = lane >> 5;
     const int wm = wave % WM, wn = wave / WM;
     const int ch0 = wn * 32 * MT;   // first output unit of this wave (hidden unit inside a chunk / channel)
-    const int r0 = wm * 64;         // first row of this wave inside the tile
+    const int r0 = wm * 32 * RT;    // first row of this wave inside the tile
 
     // weight step u: chunk u / (2 KU), stage (u / KU) & 1, 32-wide step u % KU; lane (col, hf) of
     // output tile a takes 2 x 8 consecutive inputs of weight row ch0 + 32 a + col
@@ -109,15 +109,15 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
     for (int j = 0; j < DEPTH; ++j) issue(j, ring[j]);
 
     // one stage: acc[a][rt] += W rows (ring) x tile rows (LDS `src`); u0 = first weight step
-    auto stage = [&](const T* src, f32x16 (&acc)[MT][2], int u0) {
+    auto stage = [&](const T* src, f32x16 (&acc)[MT][RT], int u0) {
         const T* brow = src + (r0 + col) * XS + hf * 16;
         for (int kk0 = 0; kk0 < KU; kk0 += DEPTH) {
 #pragma unroll
             for (int j = 0; j < DEPTH; ++j) {
                 const int kk = kk0 + j;
-                u32x4 bf[2][2];
+                u32x4 bf[RT][2];
 #pragma unroll
-                for (int rt = 0; rt < 2; ++rt) {
+                for (int rt = 0; rt < RT; ++rt) {
                     bf[rt][0] = *(const u32x4*)(brow + rt * 32 * XS + kk * 32);
                     bf[rt][1] = *(const u32x4*)(brow + rt * 32 * XS + kk * 32 + 8);
                 }
@@ -133,7 +133,7 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
 #pragma unroll
                 for (int a = 0; a < MT; ++a)
 #pragma unroll
-                    for (int rt = 0; rt < 2; ++rt) {
+                    for (int rt = 0; rt < RT; ++rt) {
                         acc[a][rt] = H16<T>::mfma(__builtin_bit_cast(v8, af[a][0]), __builtin_bit_cast(v8, bf[rt][0]), acc[a][rt]);
                         acc[a][rt] = H16<T>::mfma(__builtin_bit_cast(v8, af[a][1]), __builtin_bit_cast(v8, bf[rt][1]), acc[a][rt]);
                     }
@@ -155,20 +155,20 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
         }
         __syncthreads();
 
-        f32x16 acc[MT][2];
+        f32x16 acc[MT][RT];
 #pragma unroll
         for (int a = 0; a < MT; ++a)
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt)
+            for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[a][rt][v] = 0.f;
 
         for (int chunk = 0; chunk < 4; ++chunk) {
-            f32x16 hacc[MT][2];
+            f32x16 hacc[MT][RT];
 #pragma unroll
             for (int a = 0; a < MT; ++a)
 #pragma unroll
-                for (int rt = 0; rt < 2; ++rt)
+                for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
                     for (int v = 0; v < 16; ++v) hacc[a][rt][v] = 0.f;
             stage(xt, hacc, chunk * 2 * KU);
@@ -181,7 +181,7 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
                     const u32x2 bb = *(const u32x2*)(b1 + chunk * C + hh);
                     const float bias[4] = {H16<T>::lo(bb[0]), H16<T>::hi(bb[0]), H16<T>::lo(bb[1]), H16<T>::hi(bb[1])};
 #pragma unroll
-                    for (int rt = 0; rt < 2; ++rt) {
+                    for (int rt = 0; rt < RT; ++rt) {
                         float hv[4];
 #pragma unroll
                         for (int q = 0; q < 4; ++q) hv[q] = gelu_erf(H16<T>::round(hacc[a][rt][4 * g + q] + bias[q]));
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
                 const u32x2 bb = *(const u32x2*)(b2 + cc);
                 const float bias[4] = {H16<T>::lo(bb[0]), H16<T>::hi(bb[0]), H16<T>::lo(bb[1]), H16<T>::hi(bb[1])};
 #pragma unroll
-                for (int rt = 0; rt < 2; ++rt)
+                for (int rt = 0; rt < RT; ++rt)
                     *(u32x2*)(ht + (r0 + rt * 32 + col) * XS + cc) =
                         (u32x2){H16<T>::pack2(acc[a][rt][4 * g] + bias[0], acc[a][rt][4 * g + 1] + bias[1]),
                                 H16<T>::pack2(acc[a][rt][4 * g + 2] + bias[2], acc[a][rt][4 * g + 3] + bias[3])};
@@ -227,12 +227,12 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
     }
 }
 
-template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED>
+template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RT = 2>
 int launch_mlp_wide(const void* x, const void* resid, const void* w1, const void* b1, const void* w2, const void* b2,
                     int64_t n, void* out, hipStream_t stream) {
-    constexpr int R = 64 * WM;
+    constexpr int R = 32 * RT * WM;
     const size_t lds = (size_t)2 * R * (C + MW_PAD) * sizeof(T);
-    auto kern = mlp_wide_kernel<T, C, WM, WN, MT, DEPTH, PACKED>;
+    auto kern = mlp_wide_kernel<T, C, WM, WN, MT, DEPTH, PACKED, RT>;
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -251,9 +251,17 @@ int launch_mlp_wide(const void* x, const void* resid, const void* w1, const void
 template <bool PACKED>
 int mlp_wide_any(const void* x, const void* resid, const void* w1, const void* b1, const void* w2, const void* b2,
                  int dtype, int64_t n, int channels, void* out, hipStream_t stream) {
+    // 256 channels: 96-row tiles stream a third less weight per row than 64-row tiles; taken when they also need
+    // fewer rounds of the 256 persistent work-groups per unit of work (a 96-row tile costs about 1.25 of a 64-row one)
+    const int64_t r64 = ptv3_ceil_div(ptv3_ceil_div(n, 64), 256), r96 = ptv3_ceil_div(ptv3_ceil_div(n, 96), 256);
+    const bool three = 5 * r96 < 4 * r64;
+    const int64_t r128 = ptv3_ceil_div(ptv3_ceil_div(n, 128), 256), r192 = ptv3_ceil_div(ptv3_ceil_div(n, 192), 256);
+    const bool three128 = 5 * r192 < 4 * r128;
 #define PTV3_MW(T)                                                                                                          \
     do {                                                                                                                    \
+        if (channels == 128 && three128) return launch_mlp_wide<T, 128, 2, 4, 1, 4, PACKED, 3>(x, resid, w1, b1, w2, b2, n, out, stream); \
         if (channels == 128) return launch_mlp_wide<T, 128, 2, 4, 1, 4, PACKED>(x, resid, w1, b1, w2, b2, n, out, stream);   \
+        if (channels == 256 && three) return launch_mlp_wide<T, 256, 1, 8, 1, 4, PACKED, 3>(x, resid, w1, b1, w2, b2, n, out, stream); \
         if (channels == 256) return launch_mlp_wide<T, 256, 1, 8, 1, 4, PACKED>(x, resid, w1, b1, w2, b2, n, out, stream);   \
         if (channels == 512) return launch_mlp_wide<T, 512, 1, 8, 2, 2, PACKED>(x, resid, w1, b1, w2, b2, n, out, stream);   \
     } while (0)
