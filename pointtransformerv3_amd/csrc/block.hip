@@ -366,9 +366,14 @@ __global__ __launch_bounds__(BLK_THREADS, 2) void block_tail_kernel(
             for (int v = 0; v < 16; ++v) acc[o][v] = 0.f;
 
         for (int ht = 0; ht < H / 32; ++ht) {
+            // the accumulator starts from fc1's bias (the MFMA's C operand) instead of adding it afterwards
             f32x16 d;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) d[v] = 0.f;
+            for (int g = 0; g < 4; ++g) {
+                const f32x4 bb = *(const f32x4*)(b1_lds + ht * 32 + 8 * g + 4 * hf);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) d[4 * g + q] = bb[q];
+            }
             const T* w1row = w1_lds + (ht * 32 + col) * WS + hf * 16;
 #pragma unroll
             for (int o = 0; o < OT; ++o) {
@@ -378,10 +383,9 @@ __global__ __launch_bounds__(BLK_THREADS, 2) void block_tail_kernel(
             uint32_t p[8];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const f32x4 bb = *(const f32x4*)(b1_lds + ht * 32 + 8 * g + 4 * hf);
                 float hv[4];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) hv[q] = gelu_erf(H16<T>::round(d[4 * g + q] + bb[q]));
+                for (int q = 0; q < 4; ++q) hv[q] = gelu_erf(H16<T>::round(d[4 * g + q]));
                 p[2 * g] = H16<T>::pack2(hv[0], hv[1]);
                 p[2 * g + 1] = H16<T>::pack2(hv[2], hv[3]);
             }

@@ -95,22 +95,25 @@ __global__ __launch_bounds__(MLP_THREADS, 2) void mlp_fused_kernel(
 
         for (int ht = 0; ht < H / 32; ++ht) {
             // hidden tile: 32 units x 32 rows
-            f32x16 d;
+            f32x16 d;   // starts from the bias: the MFMAs' C operand
 #pragma unroll
-            for (int v = 0; v < 16; ++v) d[v] = 0.f;
+            for (int g = 0; g < 4; ++g) {
+                const f32x4 bb = *(const f32x4*)(b1_lds + ht * 32 + 8 * g + 4 * hf);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) d[4 * g + q] = bb[q];
+            }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 const v8 wf = __builtin_bit_cast(v8, *(const u32x4*)(w1_lds + (ht * 32 + col) * W1S + ks * 16 + hf * 8));
                 d = H16<T>::mfma(wf, xf[ks], d);
             }
-            // bias, round to storage precision as a separate fc1 would, GELU, round again
+            // round to storage precision as a separate fc1 would, GELU, round again
             uint32_t p[8];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const f32x4 bb = *(const f32x4*)(b1_lds + ht * 32 + 8 * g + 4 * hf);
                 float hv[4];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) hv[q] = gelu_erf(H16<T>::round(d[4 * g + q] + bb[q]));
+                for (int q = 0; q < 4; ++q) hv[q] = gelu_erf(H16<T>::round(d[4 * g + q]));
                 p[2 * g] = H16<T>::pack2(hv[0], hv[1]);
                 p[2 * g + 1] = H16<T>::pack2(hv[2], hv[3]);
             }

@@ -164,13 +164,19 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
                 for (int v = 0; v < 16; ++v) acc[a][rt][v] = 0.f;
 
         for (int chunk = 0; chunk < 4; ++chunk) {
+            // stage A accumulates on top of fc1's bias (the MFMAs' C operand) instead of adding it afterwards
             f32x16 hacc[MT][RT];
 #pragma unroll
             for (int a = 0; a < MT; ++a)
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt)
+                for (int g = 0; g < 4; ++g) {
+                    const u32x2 bb = *(const u32x2*)(b1 + chunk * C + ch0 + a * 32 + 8 * g + 4 * hf);
+                    const float bias[4] = {H16<T>::lo(bb[0]), H16<T>::hi(bb[0]), H16<T>::lo(bb[1]), H16<T>::hi(bb[1])};
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) hacc[a][rt][v] = 0.f;
+                    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) hacc[a][rt][4 * g + q] = bias[q];
+                }
             stage(xt, hacc, chunk * 2 * KU);
             // hacc[a][rt][v]: hidden unit ch0 + 32 a + 8 (v / 4) + 4 hf + v % 4 of row r0 + 32 rt + col
 #pragma unroll
@@ -178,13 +184,11 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     const int hh = ch0 + a * 32 + 8 * g + 4 * hf;
-                    const u32x2 bb = *(const u32x2*)(b1 + chunk * C + hh);
-                    const float bias[4] = {H16<T>::lo(bb[0]), H16<T>::hi(bb[0]), H16<T>::lo(bb[1]), H16<T>::hi(bb[1])};
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt) {
                         float hv[4];
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) hv[q] = gelu_erf(H16<T>::round(hacc[a][rt][4 * g + q] + bias[q]));
+                        for (int q = 0; q < 4; ++q) hv[q] = gelu_erf(H16<T>::round(hacc[a][rt][4 * g + q]));
                         *(u32x2*)(ht + (r0 + rt * 32 + col) * XS + hh) =
                             (u32x2){H16<T>::pack2(hv[0], hv[1]), H16<T>::pack2(hv[2], hv[3])};
                     }
