@@ -107,9 +107,12 @@ int ptv3_attn_slots(const int64_t *order_row, const int64_t *inverse_row, const 
 
 /* model.py:456-484 (flash_attn_varlen_qkvpacked_func call at :476-482 and the torch
  * fallback :460-474): non-causal softmax(q k^T * scale) v inside each sequence, per head.
- * qkv (n_rows, 3*C) with channel layout [3][H][D], D = C/H = 16; rows are fetched through
+ * qkv (n_rows, 3*C) with channel layout [3][H][D], D = C/H; rows are fetched through
  * slot_src and results written to out[slot_dst[i]] (n_rows, C) when slot_dst[i] >= 0.
- * cu_seqlens (n_seq+1,) int32 in padded-slot units; no sequence is longer than max_seqlen. */
+ * cu_seqlens (n_seq+1,) int32 in padded-slot units; no sequence is longer than max_seqlen.
+ * D = 16 in fp16 / bf16 with sequences of up to 2368 keys (every released PTv3 configuration) runs on the MFMA
+ * kernel; fp32, D = 8, 32 or 64, and longer sequences run on a thread-per-query kernel in fp32 arithmetic
+ * (an order of magnitude slower). Other head dims: PTV3_ESHAPE. */
 int ptv3_patch_attn_fwd(const void *qkv, int dtype, int64_t n_rows, int channels, int heads,
                         const int32_t *slot_src, const int32_t *slot_dst,
                         const int32_t *cu_seqlens, int64_t n_seq, int64_t max_seqlen,
@@ -119,14 +122,15 @@ int ptv3_patch_attn_fwd(const void *qkv, int dtype, int64_t n_rows, int channels
  * applies it on its non-fused path, in float): score(query i, key j, head h) +=
  * sum over the axes a of rpe_table[a * R + clamp(g_i[a] - g_j[a], -pos_bnd, pos_bnd) + pos_bnd][h],
  * R = 2 * pos_bnd + 1; grid_coord (n_rows, 3) int32 in point order, rpe_table (3 * R, heads) fp32,
- * pos_bnd <= 128. dropout_p, dropout_seed: attention dropout as in ptv3_patch_attn_fwd_lse (0, 0 for none). */
+ * pos_bnd <= 128; D = C / heads = 8, 16, 32 or 64. dropout_p, dropout_seed: attention dropout as in
+ * ptv3_patch_attn_fwd_lse (0, 0 for none). */
 int ptv3_patch_attn_rpe_fwd(const float *qkv, int64_t n_rows, int channels, int heads,
                             const int32_t *slot_src, const int32_t *slot_dst,
                             const int32_t *cu_seqlens, int64_t n_seq, int64_t max_seqlen, float scale,
                             const int32_t *grid_coord, const float *rpe_table, int pos_bnd, float dropout_p,
                             uint32_t dropout_seed, float *out, void *stream);
 
-/* ptv3_patch_attn_fwd for training. fp16 / bf16: also keeps what the backward pass needs, lse (heads, n_pad)
+/* ptv3_patch_attn_fwd for training (D = 16 only, like the backward entry points). fp16 / bf16: also keeps what the backward pass needs, lse (heads, n_pad)
  * fp32, lse[h][slot] = log2 of the sum over the slot's sequence of 2^(score * log2(e)) for every real slot
  * (filler slots are left unwritten); fp32: lse may be NULL (the backward recomputes it). n_pad =
  * cu_seqlens[n_seq]. dropout_p in [0, 1): attention dropout (model.py:470, :480) -- probability (head, query

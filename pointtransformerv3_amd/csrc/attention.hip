@@ -286,16 +286,23 @@ __global__ __launch_bounds__(ATT_THREADS, 4) void patch_attn_half_kernel(
     }
 }
 
-// ---- fp32: thread per query, 128-key chunks of K and V in LDS.
-constexpr int F32_QB = 256;   // queries per block
-constexpr int F32_KC = 128;   // keys per chunk
+// ---- the general shape: thread per query, fp32 FMA arithmetic, chunks of K and V in LDS (as floats), any
+// sequence length and head dims 8 ... 64. It serves fp32 (parity, the RPE path's sibling), and in half precision
+// every shape the MFMA kernel above does not take: head dims other than 16 and sequences whose K and V do not
+// fit its LDS. An order of magnitude slower than that kernel; there so that such models run at all.
+constexpr int F32_QB = 256;        // queries per block
+constexpr int F32_KV = 2048;       // floats of K (and of V) per chunk: 128 keys at head dim 16
 
-__global__ __launch_bounds__(F32_QB) void patch_attn_f32_kernel(
-    const float* __restrict__ qkv, int channels, int heads, const int32_t* __restrict__ slot_src,
+template <typename T> __device__ __forceinline__ float any_to_float(T v) { return (float)v; }
+
+template <typename T, int D>
+__global__ __launch_bounds__(F32_QB) void patch_attn_any_kernel(
+    const T* __restrict__ qkv, int channels, int heads, const int32_t* __restrict__ slot_src,
     const int32_t* __restrict__ slot_dst, const int32_t* __restrict__ cu_seqlens, int q_blocks,
-    float scale, float* __restrict__ out, Dropout drop) {
-    __shared__ float k_lds[F32_KC][HD];
-    __shared__ float v_lds[F32_KC][HD];
+    float scale, T* __restrict__ out, Dropout drop) {
+    constexpr int KC = F32_KV / D;   // keys per chunk
+    __shared__ float k_lds[KC][D];
+    __shared__ float v_lds[KC][D];
     const int seq = blockIdx.x / (heads * q_blocks);
     const int rem = blockIdx.x % (heads * q_blocks);
     const int head = rem / q_blocks, qb = rem % q_blocks;
@@ -306,57 +313,91 @@ __global__ __launch_bounds__(F32_QB) void patch_attn_f32_kernel(
     const int qi = qb * F32_QB + tid;
     const int64_t row_stride = 3 * (int64_t)channels;
 
-    float q[HD], o[HD];
+    float q[D], o[D];
     int dst = -1;
 #pragma unroll
-    for (int d = 0; d < HD; ++d) { q[d] = 0.f; o[d] = 0.f; }
+    for (int d = 0; d < D; ++d) { q[d] = 0.f; o[d] = 0.f; }
     if (qi < len) {
         dst = slot_dst[s0 + qi];
-        const float* src = qkv + (int64_t)slot_src[s0 + qi] * row_stride + head * HD;
+        const T* src = qkv + (int64_t)slot_src[s0 + qi] * row_stride + head * D;
 #pragma unroll
-        for (int d = 0; d < HD; ++d) q[d] = src[d] * scale;
+        for (int d = 0; d < D; ++d) q[d] = any_to_float(src[d]) * scale;
     }
     const uint32_t hq = drop_hq(drop.seed, (uint32_t)head, (uint32_t)(s0 + qi));
     float m = -INFINITY, l = 0.f;
-    for (int c0 = 0; c0 < len; c0 += F32_KC) {
+    for (int c0 = 0; c0 < len; c0 += KC) {
         __syncthreads();
-        for (int e = tid; e < F32_KC * HD; e += F32_QB) {
-            const int key = e / HD, d = e % HD;
+        for (int e = tid; e < KC * D; e += F32_QB) {
+            const int key = e / D, d = e % D;
             float kv = 0.f, vv = 0.f;
             if (c0 + key < len) {
-                const float* src = qkv + (int64_t)slot_src[s0 + c0 + key] * row_stride + head * HD + d;
-                kv = src[channels];
-                vv = src[2 * channels];
+                const T* src = qkv + (int64_t)slot_src[s0 + c0 + key] * row_stride + head * D + d;
+                kv = any_to_float(src[channels]);
+                vv = any_to_float(src[2 * channels]);
             }
             k_lds[key][d] = kv;
             v_lds[key][d] = vv;
         }
         __syncthreads();
-        const int kn = min(F32_KC, len - c0);
+        const int kn = min(KC, len - c0);
         for (int key = 0; key < kn; ++key) {
             float s = 0.f;
 #pragma unroll
-            for (int d = 0; d < HD; ++d) s = fmaf(q[d], k_lds[key][d], s);
+            for (int d = 0; d < D; ++d) s = fmaf(q[d], k_lds[key][d], s);
             if (s > m) {
                 const float a = __expf(m - s);
                 l *= a;
 #pragma unroll
-                for (int d = 0; d < HD; ++d) o[d] *= a;
+                for (int d = 0; d < D; ++d) o[d] *= a;
                 m = s;
             }
             float p = __expf(s - m);
             l += p;
             if (drop.threshold && !drop_keep(hq, (uint32_t)(s0 + c0 + key), drop.threshold)) p = 0.f;
 #pragma unroll
-            for (int d = 0; d < HD; ++d) o[d] = fmaf(p, v_lds[key][d], o[d]);
+            for (int d = 0; d < D; ++d) o[d] = fmaf(p, v_lds[key][d], o[d]);
         }
     }
     if (dst >= 0) {
         const float inv = drop.inv_keep / l;
-        float* dstp = out + (int64_t)dst * channels + head * HD;
+        T* dstp = out + (int64_t)dst * channels + head * D;
 #pragma unroll
-        for (int d = 0; d < HD; ++d) dstp[d] = o[d] * inv;
+        for (int d = 0; d < D; ++d) dstp[d] = (T)(o[d] * inv);
     }
+}
+
+// the general kernel for (dtype, head dim); PTV3_ESHAPE for a head dim outside 8, 16, 32, 64
+template <typename T>
+int launch_any_t(const void* qkv, int channels, int heads, const int32_t* slot_src, const int32_t* slot_dst,
+                 const int32_t* cu_seqlens, int64_t n_seq, int64_t max_seqlen, float scale, void* out, Dropout drop,
+                 hipStream_t stream) {
+    const int q_blocks = (int)ptv3_ceil_div(max_seqlen, F32_QB);
+    if (n_seq * heads * q_blocks >= (1ll << 31)) return PTV3_EINVAL;
+    const dim3 grid((unsigned)(n_seq * heads * q_blocks));
+#define PTV3_ANY(D)                                                                                              \
+    case D:                                                                                                      \
+        hipLaunchKernelGGL((patch_attn_any_kernel<T, D>), grid, dim3(F32_QB), 0, stream, (const T*)qkv, channels, \
+                           heads, slot_src, slot_dst, cu_seqlens, q_blocks, scale, (T*)out, drop);                \
+        break;
+    switch (channels / heads) {
+        PTV3_ANY(8) PTV3_ANY(16) PTV3_ANY(32) PTV3_ANY(64)
+        default: return PTV3_ESHAPE;
+    }
+#undef PTV3_ANY
+    PTV3_RETURN_LAUNCH();
+}
+
+int launch_any(const void* qkv, int dtype, int channels, int heads, const int32_t* slot_src, const int32_t* slot_dst,
+               const int32_t* cu_seqlens, int64_t n_seq, int64_t max_seqlen, float scale, void* out, Dropout drop,
+               hipStream_t stream) {
+    if (dtype == PTV3_F16)
+        return launch_any_t<_Float16>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq, max_seqlen, scale, out,
+                                      drop, stream);
+    if (dtype == PTV3_BF16)
+        return launch_any_t<__bf16>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq, max_seqlen, scale, out,
+                                    drop, stream);
+    return launch_any_t<float>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq, max_seqlen, scale, out, drop,
+                               stream);
 }
 
 // ---- fp32 with relative position bias (model.py:297-316, :468-469): as above, and every score
@@ -365,14 +406,16 @@ __global__ __launch_bounds__(F32_QB) void patch_attn_f32_kernel(
 // the chunk's key coordinates sit in LDS.
 constexpr int RPE_MAX_BND = 128;
 
+template <int D>
 __global__ __launch_bounds__(F32_QB) void patch_attn_rpe_f32_kernel(
     const float* __restrict__ qkv, int channels, int heads, const int32_t* __restrict__ slot_src,
     const int32_t* __restrict__ slot_dst, const int32_t* __restrict__ cu_seqlens, int q_blocks,
     float scale, const int32_t* __restrict__ grid_coord, const float* __restrict__ rpe_table, int pos_bnd,
     float* __restrict__ out, Dropout drop) {
-    __shared__ float k_lds[F32_KC][HD];
-    __shared__ float v_lds[F32_KC][HD];
-    __shared__ int32_t c_lds[F32_KC][3];
+    constexpr int KC = F32_KV / D;   // keys per chunk
+    __shared__ float k_lds[KC][D];
+    __shared__ float v_lds[KC][D];
+    __shared__ int32_t c_lds[KC][3];
     __shared__ float t_lds[3 * (2 * RPE_MAX_BND + 1)];
     const int seq = blockIdx.x / (heads * q_blocks);
     const int rem = blockIdx.x % (heads * q_blocks);
@@ -386,30 +429,30 @@ __global__ __launch_bounds__(F32_QB) void patch_attn_rpe_f32_kernel(
     const int rnum = 2 * pos_bnd + 1;
     for (int e = tid; e < 3 * rnum; e += F32_QB) t_lds[e] = rpe_table[(int64_t)e * heads + head];
 
-    float q[HD], o[HD];
+    float q[D], o[D];
     int dst = -1, qx = 0, qy = 0, qz = 0;
 #pragma unroll
-    for (int d = 0; d < HD; ++d) { q[d] = 0.f; o[d] = 0.f; }
+    for (int d = 0; d < D; ++d) { q[d] = 0.f; o[d] = 0.f; }
     if (qi < len) {
         dst = slot_dst[s0 + qi];
         const int64_t r = slot_src[s0 + qi];
-        const float* src = qkv + r * row_stride + head * HD;
+        const float* src = qkv + r * row_stride + head * D;
 #pragma unroll
-        for (int d = 0; d < HD; ++d) q[d] = src[d] * scale;
+        for (int d = 0; d < D; ++d) q[d] = src[d] * scale;
         qx = grid_coord[3 * r];
         qy = grid_coord[3 * r + 1];
         qz = grid_coord[3 * r + 2];
     }
     const uint32_t hq = drop_hq(drop.seed, (uint32_t)head, (uint32_t)(s0 + qi));
     float m = -INFINITY, l = 0.f;
-    for (int c0 = 0; c0 < len; c0 += F32_KC) {
+    for (int c0 = 0; c0 < len; c0 += KC) {
         __syncthreads();
-        for (int e = tid; e < F32_KC * HD; e += F32_QB) {
-            const int key = e / HD, d = e % HD;
+        for (int e = tid; e < KC * D; e += F32_QB) {
+            const int key = e / D, d = e % D;
             float kv = 0.f, vv = 0.f;
             if (c0 + key < len) {
                 const int64_t r = slot_src[s0 + c0 + key];
-                const float* src = qkv + r * row_stride + head * HD + d;
+                const float* src = qkv + r * row_stride + head * D + d;
                 kv = src[channels];
                 vv = src[2 * channels];
                 if (d < 3) c_lds[key][d] = grid_coord[3 * r + d];
@@ -418,11 +461,11 @@ __global__ __launch_bounds__(F32_QB) void patch_attn_rpe_f32_kernel(
             v_lds[key][d] = vv;
         }
         __syncthreads();
-        const int kn = min(F32_KC, len - c0);
+        const int kn = min(KC, len - c0);
         for (int key = 0; key < kn; ++key) {
             float s = 0.f;
 #pragma unroll
-            for (int d = 0; d < HD; ++d) s = fmaf(q[d], k_lds[key][d], s);
+            for (int d = 0; d < D; ++d) s = fmaf(q[d], k_lds[key][d], s);
             const int dx = min(max(qx - c_lds[key][0], -pos_bnd), pos_bnd) + pos_bnd;
             const int dy = min(max(qy - c_lds[key][1], -pos_bnd), pos_bnd) + pos_bnd;
             const int dz = min(max(qz - c_lds[key][2], -pos_bnd), pos_bnd) + pos_bnd;
@@ -431,22 +474,33 @@ __global__ __launch_bounds__(F32_QB) void patch_attn_rpe_f32_kernel(
                 const float a = __expf(m - s);
                 l *= a;
 #pragma unroll
-                for (int d = 0; d < HD; ++d) o[d] *= a;
+                for (int d = 0; d < D; ++d) o[d] *= a;
                 m = s;
             }
             float p = __expf(s - m);
             l += p;
             if (drop.threshold && !drop_keep(hq, (uint32_t)(s0 + c0 + key), drop.threshold)) p = 0.f;
 #pragma unroll
-            for (int d = 0; d < HD; ++d) o[d] = fmaf(p, v_lds[key][d], o[d]);
+            for (int d = 0; d < D; ++d) o[d] = fmaf(p, v_lds[key][d], o[d]);
         }
     }
     if (dst >= 0) {
         const float inv = drop.inv_keep / l;
-        float* dstp = out + (int64_t)dst * channels + head * HD;
+        float* dstp = out + (int64_t)dst * channels + head * D;
 #pragma unroll
-        for (int d = 0; d < HD; ++d) dstp[d] = o[d] * inv;
+        for (int d = 0; d < D; ++d) dstp[d] = o[d] * inv;
     }
+}
+
+// LDS of the MFMA kernel for sequences of up to max_seqlen keys: K (+ one prefetch-only step), V^T, per-step key
+// norms (padded to 16 B), ones and zeros. Beyond 160 KB (2368 keys) the sequence does not fit.
+size_t half_lds_bytes(int64_t max_seqlen) {
+    const int64_t lds_keys = (max_seqlen + 63) & ~63ll;
+    return (size_t)(lds_keys + 64) * 32 + (size_t)HD * (lds_keys * 2 + VT_PAD_BYTES) + (size_t)(lds_keys / 64) * sizeof(float) +
+           12 + 192;
+}
+bool half_kernel_takes(int dtype, int channels, int heads, int64_t max_seqlen) {
+    return dtype != PTV3_F32 && channels / heads == HD && half_lds_bytes(max_seqlen) <= 160 * 1024;
 }
 
 template <typename T, bool LSE, bool DROP>
@@ -455,9 +509,7 @@ int launch_half(const void* qkv, int channels, int heads, const int32_t* slot_sr
                 int64_t max_seqlen, float scale, void* out, float* lse, int64_t lse_stride, Dropout drop,
                 hipStream_t stream) {
     const int lds_keys = (int)((max_seqlen + 63) & ~63ll);
-    // K (+ one prefetch-only step), V^T, per-step key norms (padded to 16 B), ones and zeros
-    const size_t lds = (size_t)(lds_keys + 64) * 32 + (size_t)HD * (lds_keys * 2 + VT_PAD_BYTES) +
-                       (size_t)(lds_keys / 64) * sizeof(float) + 12 + 192;
+    const size_t lds = half_lds_bytes(max_seqlen);
     if (lds > 160 * 1024) return PTV3_ESHAPE;
     auto kern = patch_attn_half_kernel<T, LSE, DROP>;
     static size_t lds_allowed = 0;   // per instantiation; raised monotonically
@@ -504,23 +556,21 @@ extern "C" int ptv3_patch_attn_fwd(const void* qkv, int dtype, int64_t n_rows, i
                                    float scale, void* out, void* stream_) {
     if (n_rows < 0 || n_seq < 0 || channels < 1 || heads < 1 || max_seqlen < 1) return PTV3_EINVAL;
     if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
-    if (channels % heads != 0 || channels / heads != HD) return PTV3_ESHAPE;
+    if (channels % heads != 0) return PTV3_ESHAPE;
     if (n_seq * heads >= (1ll << 31)) return PTV3_EINVAL;
     if (n_seq == 0 || n_rows == 0) return PTV3_OK;
     if (!qkv || !slot_src || !slot_dst || !cu_seqlens || !out) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
-    if (dtype == PTV3_F16)
-        return launch_half<_Float16, false, false>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
-                                                   max_seqlen, scale, out, nullptr, 0, Dropout{0u, 0u, 1.f}, stream);
-    if (dtype == PTV3_BF16)
+    if (half_kernel_takes(dtype, channels, heads, max_seqlen)) {
+        if (dtype == PTV3_F16)
+            return launch_half<_Float16, false, false>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
+                                                       max_seqlen, scale, out, nullptr, 0, Dropout{0u, 0u, 1.f}, stream);
         return launch_half<__bf16, false, false>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq,
                                                  max_seqlen, scale, out, nullptr, 0, Dropout{0u, 0u, 1.f}, stream);
-    const int q_blocks = (int)ptv3_ceil_div(max_seqlen, F32_QB);
-    if (n_seq * heads * q_blocks >= (1ll << 31)) return PTV3_EINVAL;
-    hipLaunchKernelGGL(patch_attn_f32_kernel, dim3((unsigned)(n_seq * heads * q_blocks)), dim3(F32_QB),
-                       0, stream, (const float*)qkv, channels, heads, slot_src, slot_dst, cu_seqlens,
-                       q_blocks, scale, (float*)out, Dropout{0u, 0u, 1.f});
-    PTV3_RETURN_LAUNCH();
+    }
+    // fp32, and in half precision other head dims (8, 32, 64) or sequences beyond the MFMA kernel's LDS
+    return launch_any(qkv, dtype, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq, max_seqlen, scale, out,
+                      Dropout{0u, 0u, 1.f}, stream);
 }
 
 extern "C" int ptv3_patch_attn_fwd_lse(const void* qkv, int dtype, int64_t n_rows, int channels, int heads,
@@ -535,14 +585,9 @@ extern "C" int ptv3_patch_attn_fwd_lse(const void* qkv, int dtype, int64_t n_row
     if (!qkv || !slot_src || !slot_dst || !cu_seqlens || !out || (dtype != PTV3_F32 && !lse)) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
     const Dropout drop = {dropout_seed, dropout_p > 0.f ? drop_threshold(dropout_p) : 0u, 1.f / (1.f - dropout_p)};
-    if (dtype == PTV3_F32) {   // the backward recomputes the log-sum-exp rows on this path
-        const int q_blocks = (int)ptv3_ceil_div(max_seqlen, F32_QB);
-        if (n_seq * heads * q_blocks >= (1ll << 31)) return PTV3_EINVAL;
-        hipLaunchKernelGGL(patch_attn_f32_kernel, dim3((unsigned)(n_seq * heads * q_blocks)), dim3(F32_QB), 0, stream,
-                           (const float*)qkv, channels, heads, slot_src, slot_dst, cu_seqlens, q_blocks, scale,
-                           (float*)out, drop);
-        PTV3_RETURN_LAUNCH();
-    }
+    if (dtype == PTV3_F32)   // the backward recomputes the log-sum-exp rows on this path
+        return launch_any(qkv, dtype, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq, max_seqlen, scale, out, drop,
+                          stream);
 #define PTV3_ATT(T, D)                                                                                               \
     return launch_half<T, true, D>(qkv, channels, heads, slot_src, slot_dst, cu_seqlens, n_seq, max_seqlen, scale, out, \
                                    lse, n_pad, drop, stream)
@@ -564,13 +609,22 @@ extern "C" int ptv3_patch_attn_rpe_fwd(const float* qkv, int64_t n_rows, int cha
     const Dropout drop = {dropout_seed, dropout_p > 0.f ? drop_threshold(dropout_p) : 0u, 1.f / (1.f - dropout_p)};
     if (n_rows < 0 || n_seq < 0 || channels < 1 || heads < 1 || max_seqlen < 1) return PTV3_EINVAL;
     if (pos_bnd < 0 || pos_bnd > RPE_MAX_BND) return PTV3_ESHAPE;
-    if (channels % heads != 0 || channels / heads != HD) return PTV3_ESHAPE;
+    if (channels % heads != 0) return PTV3_ESHAPE;
     if (n_seq == 0 || n_rows == 0) return PTV3_OK;
     if (!qkv || !slot_src || !slot_dst || !cu_seqlens || !grid_coord || !rpe_table || !out) return PTV3_EINVAL;
     const int q_blocks = (int)ptv3_ceil_div(max_seqlen, F32_QB);
     if (n_seq * heads * q_blocks >= (1ll << 31)) return PTV3_EINVAL;
-    hipLaunchKernelGGL(patch_attn_rpe_f32_kernel, dim3((unsigned)(n_seq * heads * q_blocks)), dim3(F32_QB), 0,
-                       (hipStream_t)stream_, qkv, channels, heads, slot_src, slot_dst, cu_seqlens, q_blocks, scale,
-                       grid_coord, rpe_table, pos_bnd, out, drop);
+    const dim3 grid((unsigned)(n_seq * heads * q_blocks));
+#define PTV3_RPE(D)                                                                                                  \
+    case D:                                                                                                          \
+        hipLaunchKernelGGL(patch_attn_rpe_f32_kernel<D>, grid, dim3(F32_QB), 0, (hipStream_t)stream_, qkv, channels, \
+                           heads, slot_src, slot_dst, cu_seqlens, q_blocks, scale, grid_coord, rpe_table, pos_bnd, out, \
+                           drop);                                                                                    \
+        break;
+    switch (channels / heads) {
+        PTV3_RPE(8) PTV3_RPE(16) PTV3_RPE(32) PTV3_RPE(64)
+        default: return PTV3_ESHAPE;
+    }
+#undef PTV3_RPE
     PTV3_RETURN_LAUNCH();
 }

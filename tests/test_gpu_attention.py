@@ -18,11 +18,11 @@ def ops():
     return _ops
 
 
-def _case(counts, patch, heads, dtype, seed, scale_in=1.0):
+def _case(counts, patch, heads, dtype, seed, scale_in=1.0, head_dim=16):
     rng = np.random.default_rng(seed)
     g = torch.Generator().manual_seed(seed)
     n = int(sum(counts))
-    C = heads * 16
+    C = heads * head_dim
     offset = np.cumsum(counts).astype(np.int64)
     # a per-scene random permutation plays the role of the serialized order
     order = np.concatenate([s + rng.permutation(c) for s, c in zip(np.concatenate([[0], offset[:-1]]), counts)]).astype(np.int64)
@@ -34,8 +34,29 @@ def _case(counts, patch, heads, dtype, seed, scale_in=1.0):
     o = ops()
     gp, gu, gc = o.pad_index(to_dev(offset), offset.tolist(), patch)
     src, dst = o.attn_slots(to_dev(order), to_dev(inverse), gp, gu)
-    got = o.patch_attention(qkv.to(DEV), heads, src, dst, gc, patch, 16 ** -0.5)
+    got = o.patch_attention(qkv.to(DEV), heads, src, dst, gc, patch, head_dim ** -0.5)
     return got, want
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("head_dim", [8, 32, 64])
+def test_attention_other_head_dims(dtype, head_dim):
+    """Head dims other than 16 (model.py:441-443 allows any channels // num_heads) take the thread-per-query
+    kernel: same bar, ragged last patch and two scenes."""
+    got, want = _case([700, 333], 256, 3, dtype, seed=head_dim, head_dim=head_dim)
+    assert got.dtype == dtype and got.shape == want.shape
+    assert rel_err(got, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_attention_sequences_beyond_the_mfma_kernels_lds(dtype):
+    """Patch 3072: sequences of 3072 keys are more than the MFMA kernel keeps in LDS (2368); the half-precision
+    call then runs on the thread-per-query kernel instead of failing."""
+    got, want = _case([7000, 500], 3072, 2, dtype, seed=21)
+    assert rel_err(got, want) < TOL[dtype]
+    from pointtransformerv3_amd import _lib
+    with pytest.raises(_lib.Ptv3Error):          # a head dim outside 8, 16, 32, 64 is still refused
+        _case([100], 32, 2, dtype, seed=1, head_dim=24)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])

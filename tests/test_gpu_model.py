@@ -296,6 +296,25 @@ def test_forward_other_pooling_strides_fp32():
     assert rel_err(point.feat, want) < 1e-4
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_forward_with_head_dim_32(dtype):
+    """Half as many heads as the default (model.py:441-443: head dim = channels // num_heads = 32 everywhere):
+    the attention then runs on the thread-per-query kernel, fp32 and half precision alike."""
+    from pointtransformerv3_amd import PointTransformerV3
+    kw = dict(enc_depths=(1, 1, 1, 1, 1), dec_depths=(1, 1, 1, 1), enc_num_head=(1, 2, 4, 8, 16), dec_num_head=(2, 2, 4, 8),
+              enc_patch_size=(256,) * 5, dec_patch_size=(256,) * 4)
+    torch.manual_seed(4)
+    model = PointTransformerV3(shuffle_orders=False, enable_flash=dtype != torch.float32, **kw).eval()
+    d, feat = _data(5000, 2, grid=0.02)
+    perms = _draw_perms(41, False)
+    x = feat.astype(np.float16).astype(np.float32)
+    want = ptv3_forward(model.state_dict(), d["grid_coord"], x, d["offset"], enable_flash=dtype != torch.float32,
+                        perms=perms, **kw)
+    point = _run(model.to(DEV).to(dtype), d, x, dtype)
+    assert point.feat.shape == want.shape
+    assert rel_err(point.feat, want) < (1e-4 if dtype == torch.float32 else 2e-2)
+
+
 @pytest.mark.parametrize("sizes", [[50], [1, 3000], [200, 2, 70]])
 def test_forward_tiny_and_ragged_scenes_fp32(sizes):
     """Scenes smaller than a patch, single-point scenes, very unequal scenes in one batch."""
