@@ -35,6 +35,151 @@ template <typename T> struct LwNorm {
     T* out1;
 };
 
+// What the epilogue of a tile needs to know about the lane and its work-group.
+template <typename T> struct LwLane {
+    T* stage;               // the wave's 32 x 64 staging rows
+    const float* b_lds;     // bias [LW_N]
+    const float* p_lds;     // LayerNorm parameters [5][LW_N]
+    float* ex_lds;          // partial sums of the LayerNorms [4][LW_ROWS][4]
+    int c0, row0, col, hf, lane, wave, cout0, nout;
+    int64_t n;
+};
+
+// acc -> out (and ln.out1) for the 64-row tile that starts at row tile_row0; resv: the residual rows of the wave's
+// 32 x 64 block (LN != 0). Contains work-group barriers when LN != 0: every wave calls it the same number of times.
+template <typename T, bool GELU, int LN>
+__device__ __forceinline__ void lw_epilogue(f32x16 (&acc)[2], const u32x4* resv, const LwLane<T>& L, const LwNorm<T>& ln,
+                                            T* out, int64_t tile_row0) {
+    constexpr int NT = 2;
+    T* stage = L.stage;
+    const float *b_lds = L.b_lds, *p_lds = L.p_lds;
+    float* ex_lds = L.ex_lds;
+    const int c0 = L.c0, row0 = L.row0, col = L.col, hf = L.hf, lane = L.lane, wave = L.wave, cout0 = L.cout0, nout = L.nout;
+    const int64_t n = L.n;
+    // acc[b][v]: output channel cout0 + c0 + b*32 + 8*(v/4) + 4*hf + v%4 of row row0 + col of the tile
+    auto store_rows = [&](T* dst) {   // the wave's staged 32 x 64 block as whole row segments
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int orow = it * 8 + (lane >> 3), opc = lane & 7;
+            const u32x4 val = *(const u32x4*)(stage + orow * LW_OSTRIDE + opc * 8);
+            int64_t r = tile_row0 + row0 + orow;
+            r = r < n ? r : n - 1;
+            *(u32x4*)(dst + r * nout + cout0 + c0 + opc * 8) = val;
+        }
+        asm volatile("" ::: "memory");
+    };
+    if constexpr (LN == 0) {
+#pragma unroll
+        for (int b = 0; b < NT; ++b)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const f32x4 bb = *(const f32x4*)(b_lds + c0 + b * 32 + 8 * q + 4 * hf);
+                float r[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    r[i] = acc[b][4 * q + i] + bb[i];
+                    if (GELU) r[i] = gelu_erf(H16<T>::round(r[i]));
+                }
+                *(u32x2*)(stage + col * LW_OSTRIDE + b * 32 + 8 * q + 4 * hf) =
+                    (u32x2){H16<T>::pack2(r[0], r[1]), H16<T>::pack2(r[2], r[3])};
+            }
+        store_rows(out);
+    } else {
+        // ---- the residual block through the staging rows into accumulator order
+#pragma unroll
+        for (int it = 0; it < 4; ++it)
+            *(u32x4*)(stage + (it * 8 + (lane >> 3)) * LW_OSTRIDE + (lane & 7) * 8) = resv[it];
+        asm volatile("" ::: "memory");
+        float val[NT][16];
+#pragma unroll
+        for (int b = 0; b < NT; ++b)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const f32x4 bb = *(const f32x4*)(b_lds + c0 + b * 32 + 8 * q + 4 * hf);
+                const u32x2 rp = *(const u32x2*)(stage + col * LW_OSTRIDE + b * 32 + 8 * q + 4 * hf);
+                const float rr[4] = {H16<T>::lo(rp[0]), H16<T>::hi(rp[0]), H16<T>::lo(rp[1]), H16<T>::hi(rp[1])};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float lin = H16<T>::round(acc[b][4 * q + i] + bb[i]);
+                    // mode 2: the sum is final here; mode 3: the residual waits in the upper half of the pair
+                    val[b][4 * q + i] = LN == 2 ? H16<T>::round(lin + rr[i]) : lin;
+                    if (LN == 3) acc[b][4 * q + i] = rr[i];
+                }
+            }
+        asm volatile("" ::: "memory");
+        // mean and 1 / std of the wave's row over all 256 channels: slot, slot + 1 of the exchange buffer
+        auto row_stats = [&](int slot, float& mean, float& rstd) {
+            float sum = 0.f;
+#pragma unroll
+            for (int b = 0; b < NT; ++b)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) sum += val[b][v];
+            sum += __shfl_xor(sum, 32, PTV3_WAVE);
+            float* mine = ex_lds + (slot * LW_ROWS + row0 + col) * 4;
+            if (hf == 0) mine[wave & 3] = sum;
+            __syncthreads();
+            const f32x4 ps = *(const f32x4*)mine;
+            mean = (ps[0] + ps[1] + ps[2] + ps[3]) * (1.f / LW_N);
+            float dev = 0.f;
+#pragma unroll
+            for (int b = 0; b < NT; ++b)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) dev += (val[b][v] - mean) * (val[b][v] - mean);
+            dev += __shfl_xor(dev, 32, PTV3_WAVE);
+            if (hf == 0) mine[LW_ROWS * 4 + (wave & 3)] = dev;
+            __syncthreads();
+            const f32x4 pd = *(const f32x4*)(mine + LW_ROWS * 4);
+            rstd = rsqrtf((pd[0] + pd[1] + pd[2] + pd[3]) * (1.f / LW_N) + ln.eps);
+        };
+        float mean, rstd;
+        if (LN == 3) {   // s = res + LN(lin), every stage rounded
+            row_stats(0, mean, rstd);
+#pragma unroll
+            for (int b = 0; b < NT; ++b)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int c = c0 + b * 32 + 8 * q + 4 * hf;
+                    const f32x4 ga = *(const f32x4*)(p_lds + c), be = *(const f32x4*)(p_lds + LW_N + c);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float y = (val[b][4 * q + i] - mean) * rstd * ga[i] + be[i];
+                        val[b][4 * q + i] = H16<T>::round(H16<T>::round(y) + acc[b][4 * q + i]);
+                    }
+                }
+        }
+        // ---- out0 = s (+ shift), out1 = LN(s) with the second (mode 3) or only (mode 2) parameters
+#pragma unroll
+        for (int b = 0; b < NT; ++b)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int c = c0 + b * 32 + 8 * q + 4 * hf;
+                f32x4 sh = {0.f, 0.f, 0.f, 0.f};
+                if (LN == 2) sh = *(const f32x4*)(p_lds + 4 * LW_N + c);
+                *(u32x2*)(stage + col * LW_OSTRIDE + b * 32 + 8 * q + 4 * hf) =
+                    (u32x2){H16<T>::pack2(val[b][4 * q] + sh[0], val[b][4 * q + 1] + sh[1]),
+                            H16<T>::pack2(val[b][4 * q + 2] + sh[2], val[b][4 * q + 3] + sh[3])};
+            }
+        store_rows(out);
+        row_stats(2, mean, rstd);
+        const float* ga_l = p_lds + (LN == 3 ? 2 * LW_N : 0);
+        const float* be_l = p_lds + (LN == 3 ? 3 * LW_N : LW_N);
+#pragma unroll
+        for (int b = 0; b < NT; ++b)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int c = c0 + b * 32 + 8 * q + 4 * hf;
+                const f32x4 ga = *(const f32x4*)(ga_l + c), be = *(const f32x4*)(be_l + c);
+                float o[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[i] = (val[b][4 * q + i] - mean) * rstd * ga[i] + be[i];
+                *(u32x2*)(stage + col * LW_OSTRIDE + b * 32 + 8 * q + 4 * hf) =
+                    (u32x2){H16<T>::pack2(o[0], o[1]), H16<T>::pack2(o[2], o[3])};
+            }
+        store_rows(ln.out1);
+    }
+}
+
 // LN = 0: out = act(x W^T + b). LN = 2 / 3 (nout = 256, one tile of output channels, so a work-group holds whole
 // rows): modes 2 / 3 of the Linear + LayerNorm kernel on the accumulators, every intermediate rounded where the
 // separate kernels store it. A row's 256 channels are spread over the four waves of its row half: the sums of a
@@ -168,131 +313,133 @@ __global__ __launch_bounds__(LW_THREADS, 2) void linear_wide_kernel(
                                           __builtin_bit_cast(v8, xf[kc & 1][ks]), acc[b]);
             __builtin_amdgcn_sched_barrier(0);
         }
-        // acc[b][v]: output channel cout0 + c0 + b*32 + 8*(v/4) + 4*hf + v%4 of row row0 + col of the tile
-        auto store_rows = [&](T* dst) {   // the wave's staged 32 x 64 block as whole row segments
-            asm volatile("" ::: "memory");
-#pragma unroll
-            for (int it = 0; it < 4; ++it) {
-                const int orow = it * 8 + (lane >> 3), opc = lane & 7;
-                const u32x4 val = *(const u32x4*)(stage + orow * LW_OSTRIDE + opc * 8);
-                int64_t r = r0 + (int64_t)tile * LW_ROWS + row0 + orow;
-                r = r < n ? r : n - 1;
-                *(u32x4*)(dst + r * nout + cout0 + c0 + opc * 8) = val;
-            }
-            asm volatile("" ::: "memory");
-        };
-        if constexpr (LN == 0) {
-#pragma unroll
-            for (int b = 0; b < NT; ++b)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const f32x4 bb = *(const f32x4*)(b_lds + c0 + b * 32 + 8 * q + 4 * hf);
-                    float r[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        r[i] = acc[b][4 * q + i] + bb[i];
-                        if (GELU) r[i] = gelu_erf(H16<T>::round(r[i]));
-                    }
-                    *(u32x2*)(stage + col * LW_OSTRIDE + b * 32 + 8 * q + 4 * hf) =
-                        (u32x2){H16<T>::pack2(r[0], r[1]), H16<T>::pack2(r[2], r[3])};
-                }
-            store_rows(out);
-        } else {
-            // ---- the residual block through the staging rows into accumulator order
-#pragma unroll
-            for (int it = 0; it < 4; ++it)
-                *(u32x4*)(stage + (it * 8 + (lane >> 3)) * LW_OSTRIDE + (lane & 7) * 8) = resv[it];
-            asm volatile("" ::: "memory");
-            float val[NT][16];
-#pragma unroll
-            for (int b = 0; b < NT; ++b)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const f32x4 bb = *(const f32x4*)(b_lds + c0 + b * 32 + 8 * q + 4 * hf);
-                    const u32x2 rp = *(const u32x2*)(stage + col * LW_OSTRIDE + b * 32 + 8 * q + 4 * hf);
-                    const float rr[4] = {H16<T>::lo(rp[0]), H16<T>::hi(rp[0]), H16<T>::lo(rp[1]), H16<T>::hi(rp[1])};
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const float lin = H16<T>::round(acc[b][4 * q + i] + bb[i]);
-                        // mode 2: the sum is final here; mode 3: the residual waits in the upper half of the pair
-                        val[b][4 * q + i] = LN == 2 ? H16<T>::round(lin + rr[i]) : lin;
-                        if (LN == 3) acc[b][4 * q + i] = rr[i];
-                    }
-                }
-            asm volatile("" ::: "memory");
-            // mean and 1 / std of the wave's row over all 256 channels: slot, slot + 1 of the exchange buffer
-            auto row_stats = [&](int slot, float& mean, float& rstd) {
-                float sum = 0.f;
-#pragma unroll
-                for (int b = 0; b < NT; ++b)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) sum += val[b][v];
-                sum += __shfl_xor(sum, 32, PTV3_WAVE);
-                float* mine = ex_lds + (slot * LW_ROWS + row0 + col) * 4;
-                if (hf == 0) mine[wave & 3] = sum;
-                __syncthreads();
-                const f32x4 ps = *(const f32x4*)mine;
-                mean = (ps[0] + ps[1] + ps[2] + ps[3]) * (1.f / LW_N);
-                float dev = 0.f;
-#pragma unroll
-                for (int b = 0; b < NT; ++b)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) dev += (val[b][v] - mean) * (val[b][v] - mean);
-                dev += __shfl_xor(dev, 32, PTV3_WAVE);
-                if (hf == 0) mine[LW_ROWS * 4 + (wave & 3)] = dev;
-                __syncthreads();
-                const f32x4 pd = *(const f32x4*)(mine + LW_ROWS * 4);
-                rstd = rsqrtf((pd[0] + pd[1] + pd[2] + pd[3]) * (1.f / LW_N) + ln.eps);
-            };
-            float mean, rstd;
-            if (LN == 3) {   // s = res + LN(lin), every stage rounded
-                row_stats(0, mean, rstd);
-#pragma unroll
-                for (int b = 0; b < NT; ++b)
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int c = c0 + b * 32 + 8 * q + 4 * hf;
-                        const f32x4 ga = *(const f32x4*)(p_lds + c), be = *(const f32x4*)(p_lds + LW_N + c);
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const float y = (val[b][4 * q + i] - mean) * rstd * ga[i] + be[i];
-                            val[b][4 * q + i] = H16<T>::round(H16<T>::round(y) + acc[b][4 * q + i]);
-                        }
-                    }
-            }
-            // ---- out0 = s (+ shift), out1 = LN(s) with the second (mode 3) or only (mode 2) parameters
-#pragma unroll
-            for (int b = 0; b < NT; ++b)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int c = c0 + b * 32 + 8 * q + 4 * hf;
-                    f32x4 sh = {0.f, 0.f, 0.f, 0.f};
-                    if (LN == 2) sh = *(const f32x4*)(p_lds + 4 * LW_N + c);
-                    *(u32x2*)(stage + col * LW_OSTRIDE + b * 32 + 8 * q + 4 * hf) =
-                        (u32x2){H16<T>::pack2(val[b][4 * q] + sh[0], val[b][4 * q + 1] + sh[1]),
-                                H16<T>::pack2(val[b][4 * q + 2] + sh[2], val[b][4 * q + 3] + sh[3])};
-                }
-            store_rows(out);
-            row_stats(2, mean, rstd);
-            const float* ga_l = p_lds + (LN == 3 ? 2 * LW_N : 0);
-            const float* be_l = p_lds + (LN == 3 ? 3 * LW_N : LW_N);
-#pragma unroll
-            for (int b = 0; b < NT; ++b)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int c = c0 + b * 32 + 8 * q + 4 * hf;
-                    const f32x4 ga = *(const f32x4*)(ga_l + c), be = *(const f32x4*)(be_l + c);
-                    float o[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) o[i] = (val[b][4 * q + i] - mean) * rstd * ga[i] + be[i];
-                    *(u32x2*)(stage + col * LW_OSTRIDE + b * 32 + 8 * q + 4 * hf) =
-                        (u32x2){H16<T>::pack2(o[0], o[1]), H16<T>::pack2(o[2], o[3])};
-                }
-            store_rows(ln.out1);
-        }
+        const LwLane<T> me = {stage, b_lds, p_lds, ex_lds, c0, row0, col, hf, lane, wave, cout0, nout, n};
+        lw_epilogue<T, GELU, LN>(acc, resv, me, ln, out, r0 + (int64_t)tile * LW_ROWS);
         ptr_cur = ptr_nxt;
         ptr_nxt = ptr_nn;
         ptr_nn = ptr_3;
+    }
+}
+
+// The same layer when a work-group's whole span of rows fits the LDS the weights leave behind (256 outputs and at
+// most 192 rows per work-group: up to 49k rows, the 256-channel level of the default model). With three tiles per
+// work-group the streaming kernel above never gets past its start-up: a tile of rows is all it has in flight, so it
+// runs at the latency of HBM, not its bandwidth. Here every row of the span is asked for before the weights are
+// staged (12 x 16 bytes per thread, 96 KB per CU in flight beside the 128 KB of weights), parked in LDS once the
+// weights are in registers, and the tiles are then computed without another global load or a barrier per step.
+constexpr int RS_TILES = 3;
+constexpr int RS_ROWS = RS_TILES * LW_ROWS;        // 192
+constexpr int RS_XSTRIDE = LW_K + 8;               // halfs per resident row
+constexpr int RS_PIECES = RS_ROWS * (LW_K / 8) / LW_THREADS;   // 16-byte pieces per thread: 12
+
+template <typename T, int LN>
+__global__ __launch_bounds__(LW_THREADS, 2) void linear_wide_resident_kernel(
+    const T* __restrict__ x, const T* __restrict__ weight, const T* __restrict__ bias, int64_t n, T* __restrict__ out,
+    int span_rows, LwNorm<T> ln) {
+    typedef typename H16<T>::v8 v8;
+    constexpr int NT = 2;
+    extern __shared__ __align__(16) unsigned char lw_smem[];
+    T* w_lds = (T*)lw_smem;                                   // [LW_N][LW_WSTRIDE], only while the fragments are taken
+    float* b_lds = (float*)(w_lds + LW_N * LW_WSTRIDE + 2 * LW_ROWS * LW_XSTRIDE);   // [LW_N], where the other kernel has it
+    // after the weights: staging rows of the waves, LayerNorm parameters, partial sums, then the resident rows
+    float* p_lds = (float*)(w_lds + LW_THREADS / PTV3_WAVE * 32 * LW_OSTRIDE);        // [5][LW_N]
+    float* ex_lds = p_lds + 5 * LW_N;                                                 // [4][LW_ROWS][4]
+    T* x_res = (T*)(ex_lds + 4 * LW_ROWS * 4);                                        // [RS_ROWS][RS_XSTRIDE]
+
+    const int64_t r0 = (int64_t)blockIdx.x * span_rows;
+    if (r0 >= n) return;
+    const int64_t r1 = r0 + span_rows < n ? r0 + span_rows : n;
+    const int n_tiles = (int)((r1 - r0 + LW_ROWS - 1) / LW_ROWS);
+    const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
+    const int col = lane & 31, hf = lane >> 5;
+    const int row0 = (wave >> 2) * 32;                 // the wave's first row inside a tile
+    const int c0 = (wave & 3) * (NT * 32);             // its first output channel
+
+    // ---- every row of the span: rows past the end of the matrix repeat its last row
+    u32x4 xr[RS_PIECES];
+#pragma unroll
+    for (int i = 0; i < RS_PIECES; ++i) {
+        const int e = tid + i * LW_THREADS;
+        int64_t r = r0 + e / (LW_K / 8);
+        r = r < n ? r : n - 1;
+        xr[i] = *(const u32x4*)(x + r * LW_K + (e % (LW_K / 8)) * 8);
+    }
+    // ---- the weights: whole rows into LDS, then this wave's fragments into registers
+    {
+        constexpr int PIECES = LW_N * (LW_K / 8) / LW_THREADS;   // 16 per thread, 8 in flight together
+#pragma unroll
+        for (int i0 = 0; i0 < PIECES; i0 += 8) {
+            u32x4 piece[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int e = tid + (i0 + i) * LW_THREADS, co = e / (LW_K / 8), pc = e % (LW_K / 8);
+                piece[i] = *(const u32x4*)(weight + (int64_t)co * LW_K + pc * 8);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int e = tid + (i0 + i) * LW_THREADS, co = e / (LW_K / 8), pc = e % (LW_K / 8);
+                *(u32x4*)(w_lds + co * LW_WSTRIDE + pc * 8) = piece[i];
+            }
+        }
+        if (tid < LW_N) b_lds[tid] = bias ? (float)bias[tid] : 0.f;
+    }
+    __syncthreads();
+    u32x4 wreg[NT][LW_K / 16];
+#pragma unroll
+    for (int b = 0; b < NT; ++b)
+#pragma unroll
+        for (int k = 0; k < LW_K / 16; ++k)
+            wreg[b][k] = *(const u32x4*)(w_lds + (c0 + b * 32 + col) * LW_WSTRIDE + k * 16 + hf * 8);
+    __syncthreads();   // the weight rows are dead: the rows of the span and the parameters take their place
+#pragma unroll
+    for (int i = 0; i < RS_PIECES; ++i) {
+        const int e = tid + i * LW_THREADS;
+        *(u32x4*)(x_res + (e / (LW_K / 8)) * RS_XSTRIDE + (e % (LW_K / 8)) * 8) = xr[i];
+    }
+    if (LN != 0 && tid < LW_N) {
+        p_lds[tid] = (float)ln.gamma[tid];
+        p_lds[LW_N + tid] = (float)ln.beta[tid];
+        p_lds[2 * LW_N + tid] = LN == 3 ? (float)ln.gamma2[tid] : 0.f;
+        p_lds[3 * LW_N + tid] = LN == 3 ? (float)ln.beta2[tid] : 0.f;
+        p_lds[4 * LW_N + tid] = (LN == 2 && ln.shift) ? (float)ln.shift[tid] : 0.f;
+    }
+    T* stage = w_lds + wave * (32 * LW_OSTRIDE);
+    const LwLane<T> me = {stage, b_lds, p_lds, ex_lds, c0, row0, col, hf, lane, wave, 0, LW_N, n};
+    // the residual rows of the first tile (the wave's 32 x 64 block, whole row segments); a tile ahead from there on
+    u32x4 resv[LN != 0 ? 4 : 1], resn[LN != 0 ? 4 : 1];
+    auto fetch_res = [&](int tile, u32x4 (&dst)[LN != 0 ? 4 : 1]) {
+        if (LN != 0) {
+            const int t = tile < n_tiles ? tile : n_tiles - 1;
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                int64_t r = r0 + (int64_t)t * LW_ROWS + row0 + it * 8 + (lane >> 3);
+                r = r < n ? r : n - 1;
+                dst[it] = *(const u32x4*)(ln.res + r * LW_N + c0 + (lane & 7) * 8);
+            }
+        }
+    };
+    fetch_res(0, resv);
+    __syncthreads();
+
+    for (int tile = 0; tile < n_tiles; ++tile) {
+        fetch_res(tile + 1, resn);
+        f32x16 acc[NT];
+#pragma unroll
+        for (int b = 0; b < NT; ++b)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[b][v] = 0.f;
+        const T* xa = x_res + (tile * LW_ROWS + row0 + col) * RS_XSTRIDE + hf * 8;
+#pragma unroll
+        for (int k = 0; k < LW_K / 16; ++k) {
+            const v8 xf = __builtin_bit_cast(v8, *(const u32x4*)(xa + k * 16));
+#pragma unroll
+            for (int b = 0; b < NT; ++b) acc[b] = H16<T>::mfma(__builtin_bit_cast(v8, wreg[b][k]), xf, acc[b]);
+        }
+        lw_epilogue<T, false, LN>(acc, resv, me, ln, out, r0 + (int64_t)tile * LW_ROWS);
+        if (LN != 0) {
+#pragma unroll
+            for (int it = 0; it < 4; ++it) resv[it] = resn[it];
+        }
     }
 }
 
@@ -317,6 +464,24 @@ int launch_linear_wide(const void* x, const void* w, const void* bias, int64_t n
     if (spans < 1) spans = 1;
     int64_t span_rows = ptv3_ceil_div(ptv3_ceil_div(n, spans), LW_ROWS) * LW_ROWS;
     spans = ptv3_ceil_div(n, span_rows);
+    if constexpr (!GELU) {
+        if (col_tiles == 1 && span_rows <= RS_ROWS) {   // the whole span stays in LDS
+            static_assert((8 * 32 * LW_OSTRIDE) * 2 + (5 * LW_N + 4 * LW_ROWS * 4) * 4 + RS_ROWS * RS_XSTRIDE * 2 <=
+                              (LW_N * LW_WSTRIDE + 2 * LW_ROWS * LW_XSTRIDE) * 2,
+                          "staging rows, parameters, partial sums and the resident rows fit the weights' and tiles' LDS");
+            auto rkern = linear_wide_resident_kernel<T, LN>;
+            static bool rallowed = false;
+            if (!rallowed) {
+                hipError_t e = hipFuncSetAttribute((const void*)rkern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+                if (e != hipSuccess) return (int)e;
+                rallowed = true;
+            }
+            hipLaunchKernelGGL(rkern, dim3((unsigned)spans), dim3(LW_THREADS), lds, stream, (const T*)x, (const T*)w,
+                               (const T*)bias, n, (T*)out, (int)span_rows, ln);
+            hipError_t e = hipGetLastError();
+            return e == hipSuccess ? PTV3_OK : (int)e;
+        }
+    }
     hipLaunchKernelGGL(kern, dim3((unsigned)spans, (unsigned)col_tiles), dim3(LW_THREADS), lds, stream, (const T*)x,
                        (const T*)w, (const T*)bias, n, nout, (T*)out, (int)span_rows, ln);
     hipError_t e = hipGetLastError();
