@@ -644,7 +644,8 @@ def test_subm_conv_sparse_parity(dtype, c, n, extent):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("c,n,mode", [(128, 5001, 3), (128, 77, 2), (256, 3000, 3), (256, 40_001, 2), (256, 1, 3), (128, 33, 3),
-                                      (256, 37_681, 3), (256, 60_001, 2), (256, 50_000, 3)])
+                                      (256, 37_681, 3), (256, 60_001, 2), (256, 50_000, 3), (256, 49_152, 2), (256, 49_153, 3),
+                                      (256, 12_289, 2), (256, 191, 3)])
 def test_linear_ln_parity(dtype, c, n, mode):
     """Square Linear + LayerNorm(s) + residual in one kernel (model.py:541-545,587-597) against torch in
     fp32 and against the two kernels it replaces (same rounding points, other summation order)."""
