@@ -366,6 +366,9 @@ __global__ __launch_bounds__(F32_QB) void patch_attn_any_kernel(
     }
 }
 
+// the head dims the thread-per-query kernels are instantiated for
+bool any_head_dim(int d) { return d == 8 || d == 16 || d == 32 || d == 64; }
+
 // the general kernel for (dtype, head dim); PTV3_ESHAPE for a head dim outside 8, 16, 32, 64
 template <typename T>
 int launch_any_t(const void* qkv, int channels, int heads, const int32_t* slot_src, const int32_t* slot_dst,
@@ -556,7 +559,7 @@ extern "C" int ptv3_patch_attn_fwd(const void* qkv, int dtype, int64_t n_rows, i
                                    float scale, void* out, void* stream_) {
     if (n_rows < 0 || n_seq < 0 || channels < 1 || heads < 1 || max_seqlen < 1) return PTV3_EINVAL;
     if (dtype < PTV3_F32 || dtype > PTV3_BF16) return PTV3_EINVAL;
-    if (channels % heads != 0) return PTV3_ESHAPE;
+    if (channels % heads != 0 || !any_head_dim(channels / heads)) return PTV3_ESHAPE;
     if (n_seq * heads >= (1ll << 31)) return PTV3_EINVAL;
     if (n_seq == 0 || n_rows == 0) return PTV3_OK;
     if (!qkv || !slot_src || !slot_dst || !cu_seqlens || !out) return PTV3_EINVAL;
@@ -609,7 +612,7 @@ extern "C" int ptv3_patch_attn_rpe_fwd(const float* qkv, int64_t n_rows, int cha
     const Dropout drop = {dropout_seed, dropout_p > 0.f ? drop_threshold(dropout_p) : 0u, 1.f / (1.f - dropout_p)};
     if (n_rows < 0 || n_seq < 0 || channels < 1 || heads < 1 || max_seqlen < 1) return PTV3_EINVAL;
     if (pos_bnd < 0 || pos_bnd > RPE_MAX_BND) return PTV3_ESHAPE;
-    if (channels % heads != 0) return PTV3_ESHAPE;
+    if (channels % heads != 0 || !any_head_dim(channels / heads)) return PTV3_ESHAPE;
     if (n_seq == 0 || n_rows == 0) return PTV3_OK;
     if (!qkv || !slot_src || !slot_dst || !cu_seqlens || !grid_coord || !rpe_table || !out) return PTV3_EINVAL;
     const int q_blocks = (int)ptv3_ceil_div(max_seqlen, F32_QB);

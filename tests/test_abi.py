@@ -42,7 +42,8 @@ def test_argument_errors_without_a_device():
     assert lib.ptv3_decode(None, 0, 8, 2, None, None, None) == 0
     assert lib.ptv3_argsort(None, 10, 4, 64, None, None, None, 0, None) == -2  # > 63 bits (model.py:103)
     assert lib.ptv3_argsort(None, 0, 4, 30, None, None, None, 0, None) == 0
-    assert lib.ptv3_patch_attn_fwd(None, 1, 10, 64, 2, None, None, None, 1, 1024, 0.25, None, None) == -4
+    assert lib.ptv3_patch_attn_fwd(None, 1, 10, 48, 2, None, None, None, 1, 1024, 0.25, None, None) == -4   # head dim 24
+    assert lib.ptv3_patch_attn_fwd(None, 1, 10, 64, 2, None, None, None, 1, 1024, 0.25, None, None) == -1   # 32: taken; null pointers
     assert lib.ptv3_kmap_build(None, 10, 4, 0, None, None, 0, None) == -4
     assert lib.ptv3_subm_conv_fwd(None, 9, 10, 16, None, 27, 0, None, None, 16, None, None) == -1
     assert b"workspace" in lib.ptv3_strerror(-3)
