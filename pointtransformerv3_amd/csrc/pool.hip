@@ -224,12 +224,24 @@ __global__ __launch_bounds__(256) void segment_reduce_kernel(
     float acc[V];
 #pragma unroll
     for (int k = 0; k < V; ++k) acc[k] = (op == 0) ? -INFINITY : (op == 3 ? INFINITY : 0.f);
-    for (int64_t j = b; j < t; ++j) {
-        const Pack<T, V> p = *(const Pack<T, V>*)(src + indices[j] * c + ch);
+    // four members in flight per thread: their row numbers first, then the rows (a member at a time is two
+    // dependent latencies each); the reduction keeps the order b, b + 1, ...
+    for (int64_t j = b; j < t; j += 4) {
+        int64_t row[4];
 #pragma unroll
-        for (int k = 0; k < V; ++k) {
-            const float v = (float)p.v[k];
-            acc[k] = (op == 0) ? fmaxf(acc[k], v) : (op == 3 ? fminf(acc[k], v) : acc[k] + v);
+        for (int u = 0; u < 4; ++u) row[u] = indices[j + u < t ? j + u : t - 1];
+        Pack<T, V> p[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) p[u] = *(const Pack<T, V>*)(src + row[u] * c + ch);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (j + u < t) {
+#pragma unroll
+                for (int k = 0; k < V; ++k) {
+                    const float v = (float)p[u].v[k];
+                    acc[k] = (op == 0) ? fmaxf(acc[k], v) : (op == 3 ? fminf(acc[k], v) : acc[k] + v);
+                }
+            }
         }
     }
     Pack<T, V> r;
