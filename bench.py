@@ -235,6 +235,48 @@ def conv_case(which, reps):
             "gbs": min_bytes / us / 1e3, "frac_hbm_peak": min_bytes / us / 1e3 / HBM_PEAK_GBS}
 
 
+DENSE_CASES = {   # name: (rows, channels) at the levels of the benchmark batch
+    "tail64": (308_615, 64), "tail32": (403_093, 32), "head64": (308_615, 64), "mlp128": (146_195, 128),
+    "mlp256": (37_681, 256), "linear_ln256": (37_681, 256),
+}
+
+
+def dense_case(which, reps):
+    """One fused dense kernel of a transformer block alone at the rows and width of a level of the benchmark batch,
+    fp16: `tail*` = proj + residual + LayerNorm + MLP + residual (block_tail_kernel), `head64` = cpe Linear +
+    LayerNorm + residual + LayerNorm + qkv Linear, `mlp*` = fc1 + GELU + fc2 + residual (mlp_wide_kernel on packed
+    weights), `linear_ln256` = proj Linear + residual + LayerNorm. The command to put under rocprofv3 --pmc."""
+    from pointtransformerv3_amd import ops
+    from pointtransformerv3_amd.modules import MLP
+    dev = "cuda:0"
+    n, c = DENSE_CASES[which]
+    torch.manual_seed(3)
+    lin = lambda i, o: torch.nn.Linear(i, o).half().to(dev)
+    ln = lambda: torch.nn.LayerNorm(c).half().to(dev)
+    x, res = torch.randn(n, c, device=dev).half(), torch.randn(n, c, device=dev).half()
+    gelus, flops, byts = 0, 0.0, 0.0
+    if which.startswith("tail"):
+        proj, ln2, fc1, fc2 = lin(c, c), ln(), lin(c, 4 * c), lin(4 * c, c)
+        fn = lambda: ops.block_tail_fused(x, res, proj, ln2, fc1, fc2)
+        gelus, flops, byts = 4 * n * c, 2.0 * n * c * c * 9, 3.0 * n * c * 2
+    elif which.startswith("head"):
+        cpe, lnc, ln1, qkv = lin(c, c), ln(), ln(), lin(c, 3 * c)
+        fn = lambda: ops.block_head_fused(x, res, cpe, lnc, ln1, qkv)
+        flops, byts = 2.0 * n * c * c * 4, 6.0 * n * c * 2
+    elif which.startswith("mlp"):
+        mlp = MLP(c, 4 * c).half().to(dev)
+        fn = lambda: ops.mlp_fused_module(x, res, mlp)
+        gelus, flops, byts = 4 * n * c, 2.0 * n * c * c * 8, 3.0 * n * c * 2
+    else:
+        proj, ln2 = lin(c, c), ln()
+        fn = lambda: ops.linear_ln(x, proj, res, ln2, 2)
+        flops, byts = 2.0 * n * c * c, 4.0 * n * c * 2
+    us = _time_us(fn, iters=reps, warmup=3)
+    return {"workload": which, "rows": n, "channels": c, "us": us, "flops": flops, "tflops": flops / us / 1e6,
+            "frac_mfma_peak": flops / us / 1e6 / MFMA_PEAK_TFLOPS, "min_bytes": byts, "gbs": byts / us / 1e3,
+            "frac_hbm_peak": byts / us / 1e3 / HBM_PEAK_GBS, "gelu_evaluations": gelus}
+
+
 def other_configs():
     """The baseline configurations that are not the headline, a few iterations each: config 5 (two LiDAR-like sweeps,
     full forward, fp16), config 2 (patch attention alone, bf16), config 3 (pair lists + 3x3x3 convolution alone, fp16)."""
@@ -515,7 +557,10 @@ def main():
                     help="only run the 3x3x3 submanifold convolution of one workload (baseline config 3, or one encoder "
                          "level of the benchmark batch at its width) --reps times and print its rate: the command to "
                          "put under rocprofv3 --pmc")
-    ap.add_argument("--reps", type=int, default=20, help="timed calls of --conv")
+    ap.add_argument("--dense", metavar="CASE", default=None, choices=sorted(DENSE_CASES),
+                    help="only run one fused dense kernel of a block (block tail / head, fused MLP, Linear + LayerNorm) "
+                         "at the rows and width of a level of the benchmark batch --reps times and print its rate")
+    ap.add_argument("--reps", type=int, default=20, help="timed calls of --conv / --dense")
     ap.add_argument("--train", metavar="DTYPE", default=None, choices=["bfloat16", "float16"],
                     help="instead of the forward benchmark, time a training step (forward, backward, AdamW) of the "
                          "same model and input under autocast to DTYPE and print its own JSON line")
@@ -534,6 +579,9 @@ def main():
         return
     if args.conv:
         print(json.dumps(conv_case(args.conv, args.reps)))
+        return
+    if args.dense:
+        print(json.dumps(dense_case(args.dense, args.reps)))
         return
     if args.train:
         training_step(args)
