@@ -24,6 +24,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16
+HBM_PEAK_GBS = 8000.0
 
 
 class LaunchTimer:
@@ -64,6 +65,35 @@ def conv_min_bytes(work):
     """Rows in and out once, the weights once, one index per pair."""
     n_pairs, n, cin, cout, taps, form = work
     return 2.0 * n * (cin + cout) + 2.0 * taps * cin * cout + 4.0 * n_pairs
+
+
+def encode_bytes(work):
+    """12 B of coordinates + 8 B of scene id read, k codes of 8 B written, per point."""
+    n, k = work
+    return n * (12.0 + 8.0 + 8.0 * k)
+
+
+def argsort_bytes(work):
+    """An 8-bit-digit LSD radix sort that reads and writes (key, index) once per pass, then writes order and
+    inverse: per point and order 24 B per pass + 16 B, passes = ceil(significant bits / 8)."""
+    n, k, bits = work
+    return float(k) * n * (((bits + 7) // 8) * 24.0 + 16.0)
+
+
+def kmap_bytes(work):
+    """16 B of [batch, x, y, z] read and one 4-byte entry per kernel offset written, per voxel and build (the byte
+    model of a stored neighbour map; the pair lists that are written instead are smaller). The count and fill
+    passes of one build are two timed regions: the bytes are booked on the first."""
+    n, ks, part = work
+    return 0.0 if part == "fill" else n * (16.0 + 4.0 * ks ** 3)
+
+
+def hbm_entry(timer, name, bytes_fn, steps, kernels):
+    launches, ms, byts = timer.summary(name, bytes_fn)
+    gbs = byts / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+    return {"kernels": kernels, "bound": "hbm", "launches": launches, "ms_per_step": ms / steps, "achieved": gbs,
+            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+            "bytes_per_step": byts / steps}
 
 
 # per 64 keys x 32 queries a wave has to issue 32 v_exp_f32 (8 cycles each on this part) and 16 packed conversions
@@ -140,9 +170,6 @@ def cpu_baseline_config1(cores):
     return {"value": n / med, "unit": "points/s", "cores": cores, "kind": "port",
             "sample": f"baseline config 1 in full (16,384 points: z + Hilbert serialization at depth 8 and 16, one "
                       f"attention block, fp32), median of 3: {med * 1e3:.0f} ms"}
-
-
-HBM_PEAK_GBS = 8000.0
 
 
 def _time_us(fn, iters=20, warmup=3):
@@ -652,6 +679,12 @@ def main():
                               "hbm_frac": (conv_by / (conv_ms * 1e-3) / 1e9 / HBM_PEAK_GBS) if conv_ms > 0 else 0.0}},
         "cpu_baseline": cpu,
     }
+    # the index kernels of the same timed steps against HBM bandwidth, algorithmic bytes over the time between events
+    result["roofline"]["encode"] = hbm_entry(timer, "encode", encode_bytes, args.steps, "encode_kernel (4 orders in one pass)")
+    result["roofline"]["sort"] = hbm_entry(timer, "argsort", argsort_bytes, args.steps,
+                                           "radix sort passes + order / inverse of the 4 code rows")
+    result["roofline"]["kmap"] = hbm_entry(timer, "kmap", kmap_bytes, args.steps,
+                                           "voxel hash + pair lists of the 5 levels (5x5x5 and 3x3x3 at the first)")
     if not args.no_other_configs:
         del model, data, out
         result["other_configs"] = other_configs()

@@ -277,7 +277,9 @@ int ptv3_subm_conv_pack_weight(const void *weight, int dtype, int channels, int 
 /* ptv3_subm_conv_pack_weight for several weights in one launch (a model repacks all of them when its parameters
  * may have changed). The table lies in device memory; first_block is the running sum of
  * ptv3_subm_conv_pack_weight_blocks(channels, taps) over the jobs before this one, n_blocks the sum over all.
- * Shapes in the table are not checked: a wrong table writes out of bounds. */
+ * The table is trusted: channels must be a multiple of 32 and first_block that running sum. A row with other
+ * channels is skipped by the kernel; a row whose buffers are smaller than (channels, taps, channels) is not
+ * detected and writes out of bounds. */
 typedef struct {
     const void *weight;   /* (channels, taps, channels), f16 or bf16 */
     void *packed;         /* same size and type */
@@ -315,9 +317,11 @@ int ptv3_pool_clusters(const int64_t *code0, const int64_t *order0, int64_t n, i
  * ptv3_pool_clusters, bit for bit, and no workspace argument: the per-block cluster counts live in a fixed
  * 256 KiB array inside the library's device code, one copy per GPU, held until the process ends. Nothing is
  * allocated or freed, here or in a library underneath; the first call on a GPU looks the array's device
- * address up once. n <= ptv3_pool_clusters_static_max_points() = 16,777,216, else PTV3_ESTATIC. The stream
- * must belong to the current device. All calls on one GPU share the array: calls that overlap on one GPU
- * (different streams, or different threads) race on it -- serialise them; calls on one stream are ordered. */
+ * address up once (hipGetSymbolAddress): make that first call outside any graph capture, as a warm-up -- a
+ * call with n = 0 does it and launches nothing. n <= ptv3_pool_clusters_static_max_points() = 16,777,216, else
+ * PTV3_ESTATIC. The stream must belong to the current device. All calls on one GPU share the array: calls that
+ * overlap on one GPU (two streams, or two threads) race on it and give wrong clusters -- serialise them; calls
+ * on one stream are ordered. */
 int64_t ptv3_pool_clusters_static_max_points(void);
 int ptv3_pool_clusters_static(const int64_t *code0, const int64_t *order0, int64_t n, int shift,
                               const int64_t *offset, int n_scenes, int64_t *cluster, int64_t *idx_ptr,
@@ -475,7 +479,7 @@ int ptv3_bn_act(const void *x, const void *running_mean, const void *running_var
 /* nn.Linear of the wide blocks (model.py:541-545 cpe.1, :450 qkv, :487 proj, :510-512 fc1 + GELU):
  * out = act(x w^T + bias), x (n, k), w (nout, k), bias (nout,) or NULL, out (n, nout), act = exact
  * (erf) GELU when gelu != 0. fp16/bf16, k in {32, 64, 128, 256, 512}, nout a multiple of 32 (PTV3_ESHAPE
- * otherwise: use a library GEMM). Tall-and-skinny form: rows held in MFMA operand registers, no loop
+ * otherwise: ptv3_linear_any_fwd takes every shape). Tall-and-skinny form: rows held in MFMA operand registers, no loop
  * over memory along k. */
 int ptv3_linear_fwd(const void *x, const void *w, const void *bias, int dtype, int64_t n, int k, int nout,
                     int gelu, void *out, void *stream);
@@ -491,6 +495,13 @@ int ptv3_linear_wide_fwd(const void *x, const void *w, const void *bias, int dty
  * (PTV3_ESHAPE otherwise). Sums and the residual are added in fp32 and rounded once. */
 int ptv3_linear_gemm_fwd(const void *x, const void *w, const void *bias, const void *resid, int dtype, int64_t n,
                          int k, int nout, void *out, void *stream);
+/* nn.Linear of any shape (every call site above in an fp32 model, the reference's parity path with
+ * enable_flash=False, model.py:458-474; half-precision layers whose widths the kernels above do not take):
+ * out = resid + act(x w^T + bias), act = exact GELU when gelu != 0, resid (n, nout) or NULL (it may be `out`
+ * itself: every element is read before it is written, by the same thread). fp32 / fp16 / bf16, any k and nout;
+ * fp32 FMA arithmetic, one rounding. Not tuned: the MFMA kernels above take the shapes of the released models. */
+int ptv3_linear_any_fwd(const void *x, const void *w, const void *bias, const void *resid, int dtype, int64_t n,
+                        int k, int nout, int gelu, void *out, void *stream);
 /* The same followed by an inference-mode nn.BatchNorm1d and optionally the GELU, the projections of
  * model.py:726-735 (Linear -> BatchNorm1d -> GELU) in one kernel; statistics and affine parameters as
  * for ptv3_bn_act. The Linear's result is rounded to dtype before the normalisation, as when stored. */
@@ -526,7 +537,8 @@ int ptv3_mlp_fused(const void *x, const void *resid, const void *w1, const void 
 int ptv3_mlp_pack_weights(const void *w1, const void *w2, int dtype, int channels, void *packed, void *stream);
 /* The same packing for several MLPs in one launch (after an optimizer step every copy is stale at once): jobs is a
  * device array, first_block ascending from 0 with job j owning ptv3_mlp_pack_weights_blocks(channels) blocks,
- * n_blocks their sum. Both half types move as 16-bit patterns, so a table may mix them. */
+ * n_blocks their sum. Both half types move as 16-bit patterns, so a table may mix them. The table is trusted like
+ * ptv3_pack_job's: channels 128, 256 or 512 (other rows are skipped), buffers of the stated sizes. */
 typedef struct {
     const void *w1, *w2;  /* (4 * channels, channels) and (channels, 4 * channels) */
     void *packed;         /* 8 * channels^2 elements */

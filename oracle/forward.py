@@ -96,7 +96,7 @@ def _block(sd, name, level, heads, patch, order_index):
     level["sparse_feat"] = feat
 
 
-def _pool(sd, name, parent, perm, stride=2):
+def _pool(sd, name, parent, perm, stride=2, argmax=None):
     # model.py:640-651: pooling depth = bit length of (stride - 1), 0 when deeper than the codes
     pooling_depth = (int(np.ceil(stride)) - 1).bit_length()
     if pooling_depth > parent["depth"]:
@@ -105,7 +105,14 @@ def _pool(sd, name, parent, perm, stride=2):
     code, order, inverse = pc["code"], pc["order"], pc["inverse"]
     if perm is not None:
         code, order, inverse = code[perm], order[perm], inverse[perm]
-    feat = OF.segment_csr(_linear(sd, name + ".proj", parent["feat"]), pc["indices"], pc["idx_ptr"], "max")
+    rows = _linear(sd, name + ".proj", parent["feat"])
+    if argmax is None:
+        feat = OF.segment_csr(rows, pc["indices"], pc["idx_ptr"], "max")
+    else:
+        # the member that attains each cluster's maximum is given (row numbers of the parent, one per cluster and
+        # channel): where several members come within rounding of each other a half-precision run may pick another
+        # one than float arithmetic does, and a gradient check against that run has to follow its choice
+        feat = rows.gather(0, torch.as_tensor(argmax, dtype=torch.int64))
     feat = F.gelu(_bn(sd, name + ".norm.0", feat))
     return dict(feat=feat, sparse_feat=feat, grid_coord=pc["grid_coord"], batch=pc["batch"],
                 offset=OI.batch2offset(pc["batch"]), code=code, order=order, inverse=inverse,
@@ -122,13 +129,15 @@ def _unpool(sd, name, child):
     return parent
 
 
-def ptv3_forward(state_dict, grid_coord, feat, offset, perms=None, trace=None, **config):
+def ptv3_forward(state_dict, grid_coord, feat, offset, perms=None, trace=None, pool_argmax=None, **config):
     """Returns the (N, dec_channels[0]) output features in original point order (fp32 torch).
 
     perms: None (no shuffling) or a list of row permutations, one for the initial
     serialization followed by one per pooling stage.
     trace: optional dict; receives the feature tensor after the stem and after every
-    pooling / unpooling / block, keyed by the module's state_dict prefix."""
+    pooling / unpooling / block, keyed by the module's state_dict prefix.
+    pool_argmax: optional list, one (clusters, channels) array of parent row numbers per pooling stage: the
+    members whose projected value is taken as each cluster's maximum (see _pool); None = the true maxima."""
     cfg = dict(DEFAULTS)
     cfg.update(config)
     sd = {k: torch.as_tensor(v).float() for k, v in state_dict.items()}
@@ -162,7 +171,8 @@ def ptv3_forward(state_dict, grid_coord, feat, offset, perms=None, trace=None, *
     n_stage = len(cfg["enc_depths"])
     for s in range(n_stage):
         if s > 0:
-            level = _pool(sd, f"enc.enc{s}.down", level, perms[s], cfg["stride"][s - 1])
+            level = _pool(sd, f"enc.enc{s}.down", level, perms[s], cfg["stride"][s - 1],
+                          None if pool_argmax is None else pool_argmax[s - 1])
             note(f"enc.enc{s}.down", level)
         for i in range(cfg["enc_depths"][s]):
             _block(sd, f"enc.enc{s}.block{i}", level, cfg["enc_num_head"][s], cfg["enc_patch_size"][s], i % k)

@@ -515,12 +515,8 @@ int launch_half(const void* qkv, int channels, int heads, const int32_t* slot_sr
     const size_t lds = half_lds_bytes(max_seqlen);
     if (lds > 160 * 1024) return PTV3_ESHAPE;
     auto kern = patch_attn_half_kernel<T, LSE, DROP>;
-    static size_t lds_allowed = 0;   // per instantiation; raised monotonically
-    if (lds > lds_allowed) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-        lds_allowed = lds;
-    }
+    static LdsGrant grant_lds_allowed;   // per instantiation and device; raised monotonically
+    if (const int rc_ = ptv3_allow_lds((const void*)kern, lds, grant_lds_allowed)) return rc_;
     const float scale_log2e = scale * 1.4426950408889634f;
     // resident work-groups: two per CU (LDS-bound)
     static int slots = 0;

@@ -749,19 +749,10 @@ int launch_half_bwd(const void* qkv, const void* out, const void* dout, int chan
                        : (lse ? attn_bwd_q_kernel<T, true, false> : attn_bwd_q_kernel<T, false, false>);
     float* lse_buf = lse ? lse : ws.lse;
     auto kkv = dropping ? attn_bwd_kv_kernel<T, true> : attn_bwd_kv_kernel<T, false>;
-    static size_t allowed_q[4] = {0, 0, 0, 0}, allowed_kvs[2] = {0, 0};
-    size_t& allowed_kv = allowed_kvs[dropping];
+    static LdsGrant grant_q[4], grant_kv[2];   // per kernel variant and device
     const int qi_ = (lse != nullptr) + 2 * dropping;
-    if (lds_q > allowed_q[qi_]) {
-        hipError_t e = hipFuncSetAttribute((const void*)kq, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_q);
-        if (e != hipSuccess) return (int)e;
-        allowed_q[qi_] = lds_q;
-    }
-    if (lds_kv > allowed_kv) {
-        hipError_t e = hipFuncSetAttribute((const void*)kkv, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_kv);
-        if (e != hipSuccess) return (int)e;
-        allowed_kv = lds_kv;
-    }
+    if (const int rc_ = ptv3_allow_lds((const void*)kq, lds_q, grant_q[qi_])) return rc_;
+    if (const int rc_ = ptv3_allow_lds((const void*)kkv, lds_kv, grant_kv[dropping])) return rc_;
     // one work-group per CU is resident (LDS): the items beyond the last full round are cut into ranges of
     // tiles when that shortens the round (each range stages the sequence again, about 0.15 of an item)
     static int slots = 0;

@@ -438,12 +438,8 @@ int launch_head(const void* conv, const void* shortcut, const void* wc, const vo
     const size_t lds = ((size_t)4 * C * (C + BPAD)) * sizeof(T) + (size_t)(8 * C) * sizeof(float) +
                        (size_t)BLK_WAVES * 32 * (64 + BPAD) * sizeof(T);
     auto kern = block_head_kernel<T, C>;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-        configured = true;
-    }
+    static LdsGrant grant_configured;   // per instantiation and device
+    if (const int rc_ = ptv3_allow_lds((const void*)kern, lds, grant_configured)) return rc_;
     hipLaunchKernelGGL(kern, dim3((unsigned)persistent_blocks(n, lds)), dim3(BLK_THREADS), lds, stream,
                        (const T*)conv, (const T*)shortcut, (const T*)wc, (const T*)bc, (const T*)gc, (const T*)bec,
                        eps_c, (const T*)g1, (const T*)be1, eps_1, (const T*)wq, (const T*)bq, n, (T*)feat, (T*)qkv);
@@ -459,12 +455,8 @@ int launch_tail(const void* attn, const void* shortcut, const void* wp, const vo
     const size_t lds = ((size_t)C * (C + BPAD) + (size_t)H * (C + BPAD) + (size_t)C * (H + BPAD)) * sizeof(T) +
                        (size_t)(4 * C + H) * sizeof(float) + (size_t)BLK_WAVES * 32 * (C + BPAD) * sizeof(T);
     auto kern = block_tail_kernel<T, C>;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-        configured = true;
-    }
+    static LdsGrant grant_configured;   // per instantiation and device
+    if (const int rc_ = ptv3_allow_lds((const void*)kern, lds, grant_configured)) return rc_;
     hipLaunchKernelGGL(kern, dim3((unsigned)persistent_blocks(n, lds)), dim3(BLK_THREADS), lds, stream,
                        (const T*)attn, (const T*)shortcut, (const T*)wp, (const T*)bp, (const T*)g2, (const T*)be2,
                        eps_2, (const T*)w1, (const T*)b1, (const T*)w2, (const T*)b2, n, (T*)out);

@@ -1031,12 +1031,8 @@ int launch_pairs(const void* feat, int cin, int taps, int64_t n_pairs, const int
     const size_t lds = ((size_t)COUT_TILE * (cin + W_PAD) + (size_t)CONV_WAVES * 32 * XS_STRIDE) * sizeof(T);
     if (lds > 160 * 1024) return PTV3_ESHAPE;
     auto kern = subm_conv_pairs_kernel<T, MT, NT, (NT >= 4 ? 32 : 64)>;
-    static size_t lds_allowed = 0;   // per instantiation
-    if (lds > lds_allowed) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-        lds_allowed = lds;
-    }
+    static LdsGrant grant_lds_allowed;   // per instantiation and device; raised monotonically
+    if (const int rc_ = ptv3_allow_lds((const void*)kern, lds, grant_lds_allowed)) return rc_;
     // Rows per work-group: long enough to amortise staging the weights, short enough to give
     // every CU a few work-groups.
     const int64_t col_tiles = ptv3_ceil_div(cout, COUT_TILE);
@@ -1079,12 +1075,8 @@ int launch_pair_wstat(const void* feat, int taps, int64_t n_pairs, const int32_t
     const size_t lds = ((size_t)WS_COUT * (WS_CIN + W_PAD) + 2 * (size_t)WS_ROWS * WS_XSTRIDE) * sizeof(T);
     static_assert(8 * 32 * XS_STRIDE <= WS_COUT * (WS_CIN + W_PAD), "the waves' staging rows fit where the weights were");
     auto kern = pair_wstat_kernel<T>;
-    static bool allowed = false;   // per instantiation
-    if (!allowed) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-        allowed = true;
-    }
+    static LdsGrant grant_allowed;   // per instantiation and device
+    if (const int rc_ = ptv3_allow_lds((const void*)kern, lds, grant_allowed)) return rc_;
     // One work-group per CU (its registers hold the weights). Ranges in whole tiles: one round of work-groups
     // over the machine, long enough to pay for staging one tap's weights.
     const int64_t col_tiles = cout / WS_COUT;

@@ -87,9 +87,10 @@ __global__ __launch_bounds__(CT_THREADS) void pack_weight_batch_kernel(const ptv
         if (jobs[i].first_block <= (int64_t)blockIdx.x) j = i;   // uniform: a handful of jobs, first_block ascending
     const ptv3_pack_job job = jobs[j];
     const int c = job.channels, taps = job.taps;
+    if (c < 32 || c % 32 != 0 || taps < 1) return;   // a row no *_blocks() helper would have sized: touch nothing
     const int64_t total = (int64_t)taps * c * c / 8;
     const int64_t idx = ((int64_t)blockIdx.x - job.first_block) * CT_THREADS + threadIdx.x;
-    if (idx >= total) return;
+    if (idx < 0 || idx >= total) return;
     const int lane = (int)(idx % 64);
     int64_t r = idx / 64;
     const int steps = c / 16, slices = c / 32;
@@ -373,12 +374,8 @@ int launch_tiles(const void* feat, int64_t n, const void* packed_w, const void* 
                  const uint32_t* tile_pair, const uint32_t* vox_taps, void* out, hipStream_t stream) {
     typedef TileShape<C> S;
     auto kern = conv_tile_kernel<T, C>;
-    static bool attr_set = false;   // per instantiation; the attribute is per device function
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS);
-        if (e != hipSuccess) return (int)e;
-        attr_set = true;
-    }
+    static LdsGrant grant_attr_set;   // per instantiation and device
+    if (const int rc_ = ptv3_allow_lds((const void*)kern, S::LDS, grant_attr_set)) return rc_;
     const dim3 grid((unsigned)ptv3_ceil_div(n, CT_TV), (unsigned)(C / S::COUT_WG));
     hipLaunchKernelGGL(kern, grid, dim3(S::THREADS), S::LDS, stream, (const T*)feat, n, (const T*)packed_w,
                        (const T*)bias, tile_tap, tile_pair, vox_taps, (T*)out);

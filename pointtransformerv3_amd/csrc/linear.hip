@@ -222,12 +222,8 @@ int launch_linear_shape(const void* x, const void* w, const void* bias, LinBn bn
     const size_t lds = (size_t)chunk * (K + LIN_PAD) * sizeof(T) + (size_t)chunk * sizeof(float) * (BN ? 4 : 1) +
                        (size_t)LIN_WAVES * 32 * LIN_XSS * sizeof(T);
     auto kern = linear_rows_kernel<T, K, ACT, BN, NW, SW>;
-    static size_t lds_allowed = 0;
-    if (lds > lds_allowed) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-        lds_allowed = lds;
-    }
+    static LdsGrant grant_lds_allowed;   // per instantiation and device; raised monotonically
+    if (const int rc_ = ptv3_allow_lds((const void*)kern, lds, grant_lds_allowed)) return rc_;
     // persistent work-groups: as many as the LDS lets a CU hold, shared out between the chunks
     const int64_t tiles = (n + 31) / 32;
     int64_t per_chunk = ((lds <= 80 * 1024 && NW == 8) ? 512 : 256) / n_chunks;
@@ -280,6 +276,73 @@ int dispatch_linear(const void* x, const void* w, const void* bias, const LinBn*
     return PTV3_ESHAPE;
 }
 
+// The general shape: any number of inputs and outputs, fp32 as well as fp16 / bf16, plain FMA arithmetic in
+// fp32 on 64 x 64 output tiles with 16-input slices of x and w in LDS. It serves the fp32 model (the
+// reference's parity path, model.py:458-474 with enable_flash=False) and half-precision layers whose widths the
+// MFMA kernels above do not take; not tuned.
+constexpr int ANY_TILE = 64, ANY_KC = 16;
+
+template <typename T> __device__ __forceinline__ float any_f(T v) { return (float)v; }
+
+template <typename T>
+__global__ __launch_bounds__(256) void linear_any_kernel(const T* x, const T* w, const T* bias, const T* resid,
+                                                         int64_t n, int k, int nout, int gelu, T* out) {
+    __shared__ float xs[ANY_KC][ANY_TILE + 1];
+    __shared__ float ws[ANY_KC][ANY_TILE + 1];
+    const int tid = threadIdx.x, tr = tid / 16, tc = tid % 16;
+    const int64_t row0 = (int64_t)blockIdx.x * ANY_TILE;
+    const int col0 = blockIdx.y * ANY_TILE;
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int k0 = 0; k0 < k; k0 += ANY_KC) {
+#pragma unroll
+        for (int e = tid; e < ANY_TILE * ANY_KC; e += 256) {
+            const int r = e / ANY_KC, kk = e % ANY_KC;
+            const bool in_k = k0 + kk < k;
+            xs[kk][r] = (in_k && row0 + r < n) ? any_f(x[(row0 + r) * k + k0 + kk]) : 0.f;
+            ws[kk][r] = (in_k && col0 + r < nout) ? any_f(w[(int64_t)(col0 + r) * k + k0 + kk]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < ANY_KC; ++kk) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = xs[kk][tr + 16 * i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = ws[kk][tc + 16 * j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t r = row0 + tr + 16 * i;
+            const int c = col0 + tc + 16 * j;
+            if (r >= n || c >= nout) continue;
+            float v = acc[i][j] + (bias ? any_f(bias[c]) : 0.f);
+            if (gelu) v = 0.5f * v * (1.f + erff(v * 0.70710678118654752f));
+            if (resid) v += any_f(resid[r * nout + c]);
+            out[r * nout + c] = (T)v;
+        }
+}
+
+template <typename T>
+int launch_linear_any(const void* x, const void* w, const void* bias, const void* resid, int64_t n, int k, int nout,
+                      int gelu, void* out, hipStream_t stream) {
+    const dim3 grid((unsigned)ptv3_ceil_div(n, ANY_TILE), (unsigned)ptv3_ceil_div(nout, ANY_TILE));
+    hipLaunchKernelGGL(linear_any_kernel<T>, grid, dim3(256), 0, stream, (const T*)x, (const T*)w, (const T*)bias,
+                       (const T*)resid, n, k, nout, gelu, (T*)out);
+    PTV3_RETURN_LAUNCH();
+}
+
 int check_linear(int dtype, int64_t n, int k, int nout) {
     if (n < 0 || k < 1 || nout < 1) return PTV3_EINVAL;
     if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
@@ -329,4 +392,18 @@ extern "C" int ptv3_linear_bn_act_fwd(const void* x, const void* w, const void* 
     const LinBn bn = {running_mean, running_var, gamma, beta, eps, stats_f32};
     return dispatch_linear(x, w, bias, &bn, dtype, n, k, nout, gelu ? ACT_GELU : ACT_NONE, out, nullptr,
                            (hipStream_t)stream_);
+}
+
+extern "C" int ptv3_linear_any_fwd(const void* x, const void* w, const void* bias, const void* resid, int dtype,
+                                   int64_t n, int k, int nout, int gelu, void* out, void* stream_) {
+    if (n < 0 || k < 1 || nout < 1 || ptv3_ceil_div(n, ANY_TILE) >= (1ll << 31)) return PTV3_EINVAL;
+    if (n == 0) return PTV3_OK;
+    if (!x || !w || !out) return PTV3_EINVAL;
+    hipStream_t stream = (hipStream_t)stream_;
+    switch (dtype) {
+        case PTV3_F32: return launch_linear_any<float>(x, w, bias, resid, n, k, nout, gelu, out, stream);
+        case PTV3_F16: return launch_linear_any<_Float16>(x, w, bias, resid, n, k, nout, gelu, out, stream);
+        case PTV3_BF16: return launch_linear_any<__bf16>(x, w, bias, resid, n, k, nout, gelu, out, stream);
+        default: return PTV3_EINVAL;
+    }
 }

@@ -234,12 +234,8 @@ int launch_linear_ln(const void* x, const void* w, const void* bias, const void*
                      void* out0, void* out1, hipStream_t stream) {
     typedef LlShape<C> S;
     auto kern = linear_ln_kernel<T, C, MODE>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS);
-        if (e != hipSuccess) return (int)e;
-        attr_set = true;
-    }
+    static LdsGrant grant_attr_set;   // per instantiation and device
+    if (const int rc_ = ptv3_allow_lds((const void*)kern, S::LDS, grant_attr_set)) return rc_;
     const int64_t tiles = (n + 31) / 32;
     int64_t grid = 256 * S::OCC;
     const int64_t need = (tiles + S::WAVES - 1) / S::WAVES;

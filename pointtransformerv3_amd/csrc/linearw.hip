@@ -451,12 +451,8 @@ int launch_linear_wide(const void* x, const void* w, const void* bias, int64_t n
     static_assert((8 * 32 * LW_OSTRIDE) * 2 + (5 * LW_N + 4 * LW_ROWS * 4) * 4 <= LW_N * LW_WSTRIDE * 2,
                   "staging rows, LayerNorm parameters and partial sums fit where the weights were");
     auto kern = linear_wide_kernel<T, GELU, LN>;
-    static bool allowed = false;   // per instantiation
-    if (!allowed) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-        allowed = true;
-    }
+    static LdsGrant grant_allowed;   // per instantiation and device
+    if (const int rc_ = ptv3_allow_lds((const void*)kern, lds, grant_allowed)) return rc_;
     // one work-group per CU (its registers hold the weights): the 256 CUs are shared out over the tiles of
     // output channels, and every work-group walks an equal span of rows in whole 64-row tiles
     const int col_tiles = nout / LW_N;
@@ -470,12 +466,8 @@ int launch_linear_wide(const void* x, const void* w, const void* bias, int64_t n
                               (LW_N * LW_WSTRIDE + 2 * LW_ROWS * LW_XSTRIDE) * 2,
                           "staging rows, parameters, partial sums and the resident rows fit the weights' and tiles' LDS");
             auto rkern = linear_wide_resident_kernel<T, LN>;
-            static bool rallowed = false;
-            if (!rallowed) {
-                hipError_t e = hipFuncSetAttribute((const void*)rkern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-                if (e != hipSuccess) return (int)e;
-                rallowed = true;
-            }
+            static LdsGrant grant_rallowed;   // per instantiation and device
+            if (const int rc_ = ptv3_allow_lds((const void*)rkern, lds, grant_rallowed)) return rc_;
             hipLaunchKernelGGL(rkern, dim3((unsigned)spans), dim3(LW_THREADS), lds, stream, (const T*)x, (const T*)w,
                                (const T*)bias, n, (T*)out, (int)span_rows, ln);
             hipError_t e = hipGetLastError();
@@ -498,8 +490,8 @@ int launch_linear_wide(const void* x, const void* w, const void* bias, int64_t n
 // before the single rounding.
 // A 128 x 128 tile moves (128 + 128) x K x 2 bytes out of L2 for 2 x 128 x 128 x K flops, 64 flop per byte: at the
 // ~6.5 TB/s the L2s deliver to 256 CUs that is ~410 TFLOP/s, which is what this kernel measures on all three
-// shapes (43-48 us against 26-29 us for the library GEMM, whose 256 x 160 tiles move 98 flop per byte). The model
-// therefore keeps the library GEMM for these three layers by default and this kernel is the library-free path.
+// shapes (43-48 us; a 256 x 160 tile would move 98 flop per byte). In the default model it takes the two
+// 512 -> 1536 qkv layers; fc2 of the wide blocks runs inside the fused MLP kernel.
 constexpr int GT_THREADS = 256;
 constexpr int GT_N = 128, GT_KC = 64;
 constexpr int GT_STRIDE = GT_KC + 8;         // halfs per staged row
@@ -508,8 +500,8 @@ constexpr int GT_DEPTH = 2;
 
 template <typename T, int MT>
 __global__ __launch_bounds__(GT_THREADS, 2) void linear_gemm_kernel(
-    const T* __restrict__ x, const T* __restrict__ weight, const T* __restrict__ bias, const T* __restrict__ resid,
-    int64_t n, int k, int nout, T* __restrict__ out) {
+    const T* __restrict__ x, const T* __restrict__ weight, const T* __restrict__ bias, const T* resid,
+    int64_t n, int k, int nout, T* out) {   // resid may be out itself (fc2 accumulating onto the stored sum)
     typedef typename H16<T>::v8 v8;
     constexpr int GT_M = MT * 64;
     constexpr int XBUF = GT_M * GT_STRIDE, WBUF = GT_N * GT_STRIDE;
@@ -657,12 +649,8 @@ int launch_linear_gemm_mt(const void* x, const void* w, const void* bias, const 
                           void* out, hipStream_t stream) {
     const size_t lds = 2 * (size_t)(MT * 64 + GT_N) * GT_STRIDE * sizeof(T);
     auto kern = linear_gemm_kernel<T, MT>;
-    static bool allowed = false;   // per instantiation
-    if (!allowed) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-        allowed = true;
-    }
+    static LdsGrant grant_allowed;   // per instantiation and device
+    if (const int rc_ = ptv3_allow_lds((const void*)kern, lds, grant_allowed)) return rc_;
     hipLaunchKernelGGL(kern, dim3((unsigned)ptv3_ceil_div(n, MT * 64), (unsigned)(nout / GT_N)), dim3(GT_THREADS), lds,
                        stream, (const T*)x, (const T*)w, (const T*)bias, (const T*)resid, n, k, nout, (T*)out);
     hipError_t e = hipGetLastError();

@@ -160,12 +160,8 @@ int launch_mlp(const void* x, const void* resid, const void* w1, const void* b1,
     const size_t lds = ((size_t)H * (C + PADH) + (size_t)C * (H + PADH)) * sizeof(T) + (size_t)(H + C) * sizeof(float) +
                        (size_t)MLP_WAVES * 32 * (C + PADH) * sizeof(T);
     auto kern = mlp_fused_kernel<T, C>;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-        configured = true;
-    }
+    static LdsGrant grant_configured;   // per instantiation and device
+    if (const int rc_ = ptv3_allow_lds((const void*)kern, lds, grant_configured)) return rc_;
     // persistent work-groups: weights are staged once per work-group, so no more of them than the
     // machine holds at a time (or than there are row tiles)
     const int64_t tiles = (n + 31) / 32;

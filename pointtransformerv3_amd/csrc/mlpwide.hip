@@ -51,8 +51,9 @@ __global__ __launch_bounds__(256) void mlp_pack_batch_kernel(const ptv3_mlp_pack
         if (jobs[i].first_block <= (int64_t)blockIdx.x) j = i;   // uniform: a handful of jobs, first_block ascending
     const ptv3_mlp_pack_job job = jobs[j];
     const int c = job.channels;
+    if (c != 128 && c != 256 && c != 512) return;   // a width the fused kernel does not take: touch nothing
     const int64_t idx = ((int64_t)blockIdx.x - job.first_block) * 256 + threadIdx.x;
-    if (idx >= (int64_t)c * c) return;
+    if (idx < 0 || idx >= (int64_t)c * c) return;
     const int lane = (int)(idx % 64), jj = (int)(idx / 64 % 2), ub = (int)(idx / 128 % (c / 32));
     const int u = (int)(idx / 128 / (c / 32)), ku = c / 32;
     const int chunk = u / (2 * ku), st = (u / ku) & 1, kk = u % ku;
@@ -237,12 +238,8 @@ int launch_mlp_wide(const void* x, const void* resid, const void* w1, const void
     constexpr int R = 32 * RT * WM;
     const size_t lds = (size_t)2 * R * (C + MW_PAD) * sizeof(T);
     auto kern = mlp_wide_kernel<T, C, WM, WN, MT, DEPTH, PACKED, RT>;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-        configured = true;
-    }
+    static LdsGrant grant_configured;   // per instantiation and device
+    if (const int rc_ = ptv3_allow_lds((const void*)kern, lds, grant_configured)) return rc_;
     // persistent work-groups: as many as the machine holds at a time
     const int64_t tiles = (n + R - 1) / R;
     const int64_t resident = 256;   // one work-group per CU: two waves per SIMD at this register count

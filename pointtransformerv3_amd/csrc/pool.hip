@@ -374,13 +374,14 @@ extern "C" int64_t ptv3_pool_clusters_static_max_points(void) { return STATIC_MA
 extern "C" int ptv3_pool_clusters_static(const int64_t* code0, const int64_t* order0, int64_t n, int shift,
                                          const int64_t* offset, int n_scenes, int64_t* cluster, int64_t* idx_ptr,
                                          int64_t* head, int64_t* n_clusters, void* stream_) {
-    if (n < 1 || shift < 0 || shift > 62 || n_scenes < 0) return PTV3_EINVAL;
+    if (n < 0 || shift < 0 || shift > 62 || n_scenes < 0) return PTV3_EINVAL;
     if (n > STATIC_MAX_POINTS) return PTV3_ESTATIC;
-    if (n_scenes > 0 && !offset) return PTV3_EINVAL;
-    if (!code0 || !order0 || !cluster || !idx_ptr || !head || !n_clusters) return PTV3_EINVAL;
     uint32_t* block_cnt = nullptr;
     const int rc = static_scratch(&block_cnt);
-    if (rc != PTV3_OK) return rc;
+    // n == 0: the warm-up call (outside graph capture) that looks the array's address up and launches nothing
+    if (rc != PTV3_OK || n == 0) return rc;
+    if (n_scenes > 0 && !offset) return PTV3_EINVAL;
+    if (!code0 || !order0 || !cluster || !idx_ptr || !head || !n_clusters) return PTV3_EINVAL;
     return launch_pool_clusters(code0, order0, n, shift, offset, n_scenes, cluster, idx_ptr, head, n_clusters,
                                 block_cnt, (hipStream_t)stream_);
 }

@@ -303,12 +303,8 @@ int run_passes(const int64_t* code, int64_t n, int k, int passes, int64_t* order
 #define PTV3_SCATTER(KI, IN, F, L, U)                                                                       \
     do {                                                                                                    \
         auto kern = scatter_kernel<KI, KO, F, L, U>;                                                        \
-        static bool allowed = false; /* per instantiation: the tile needs more than the default 64 KB */    \
-        if (!allowed) {                                                                                     \
-            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
-            if (e != hipSuccess) return (int)e;                                                             \
-            allowed = true;                                                                                 \
-        }                                                                                                   \
+        static LdsGrant grant; /* per instantiation and device: the tile needs more than the default 64 KB */ \
+        if (const int rc_ = ptv3_allow_lds((const void*)kern, lds, grant)) return rc_;                      \
         hipLaunchKernelGGL(kern, grid, block, lds, stream, IN, iin, n, shift, (const uint32_t*)w.tile_hist, tiles, kout, \
                            iout, order, inverse);                                                           \
     } while (0)

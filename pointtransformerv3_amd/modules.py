@@ -445,11 +445,11 @@ class Block(PointModule):
             feat = ops.mlp_fused_module(normed, feat, mlp)
         elif plain_mlp:
             hidden = ops.linear(normed, mlp.fc1, gelu=True) if exact_gelu else mlp.act(mlp.fc1(normed))
-            if (not ops.LIBRARY_GEMM and ops.linear_gemm_ok(hidden, mlp.fc2.weight) and feat.is_contiguous()
-                    and feat.dtype == hidden.dtype):
+            feat = feat.contiguous()
+            if ops.linear_gemm_ok(hidden, mlp.fc2.weight) and feat.dtype == hidden.dtype:
                 feat = ops.linear_gemm(hidden, mlp.fc2.weight, None, resid=feat)   # onto the stored sum, in place
             else:
-                feat = feat.addmm_(hidden, mlp.fc2.weight.to(hidden.dtype).t())
+                feat = ops.linear_any(hidden, mlp.fc2.weight, None, resid=feat.to(hidden.dtype))
         else:
             feat = feat + mlp(normed)
         point.feat = feat

@@ -28,6 +28,14 @@ def set_launch_timer(timer):
     _LAUNCH_TIMER = timer
 
 
+def _timed(name, work, call):
+    """call(), between two events of the installed launch timer when there is one."""
+    if _LAUNCH_TIMER is not None:
+        _LAUNCH_TIMER.launch(name, work, call)
+    else:
+        call()
+
+
 def _stream():
     return torch.cuda.current_stream().cuda_stream
 
@@ -194,8 +202,8 @@ def encode_orders(grid_coord, batch, depth, orders):
     n, k = g.shape[0], len(orders)
     ids = (ctypes.c_int32 * k)(*[ORDER_IDS[o] for o in orders])
     code = torch.empty((k, n), dtype=torch.int64, device=g.device)
-    _lib.check(lib.ptv3_encode(_ptr(g), _ptr(b), n, int(depth), ids, k, _ptr(code), _stream()),
-               "ptv3_encode")
+    _timed("encode", (n, k), lambda: _lib.check(
+        lib.ptv3_encode(_ptr(g), _ptr(b), n, int(depth), ids, k, _ptr(code), _stream()), "ptv3_encode"))
     return code
 
 
@@ -274,8 +282,9 @@ def argsort_rows(code, key_bits):
     inverse = torch.empty_like(code)
     nbytes = lib.ptv3_argsort_workspace_bytes(n, k)
     ws = _ws(nbytes, code.device)
-    _lib.check(lib.ptv3_argsort(_ptr(code), n, k, int(key_bits), _ptr(order), _ptr(inverse), _ptr(ws),
-                                nbytes, _stream()), "ptv3_argsort")
+    _timed("argsort", (n, k, int(key_bits)), lambda: _lib.check(
+        lib.ptv3_argsort(_ptr(code), n, k, int(key_bits), _ptr(order), _ptr(inverse), _ptr(ws), nbytes, _stream()),
+        "ptv3_argsort"))
     return order, inverse
 
 
@@ -642,16 +651,18 @@ def conv_plan_direct_start(indices, ks):
     if AHEAD_ON_SIDE_STREAM and not Readback.blocking:
         side = _side_stream(dev)
         with torch.cuda.stream(side):
-            _lib.check(lib.ptv3_kmap_plan_count(_ptr(idx), n, int(ks), _ptr(plan.tap_ptr), _ptr(count), _ptr(ws), nbytes,
-                                                _stream()), "ptv3_kmap_plan_count")
+            _timed("kmap", (n, int(ks), "count"), lambda: _lib.check(
+                lib.ptv3_kmap_plan_count(_ptr(idx), n, int(ks), _ptr(plan.tap_ptr), _ptr(count), _ptr(ws), nbytes,
+                                         _stream()), "ptv3_kmap_plan_count"))
             pend.count = Readback(count)
             pend.side_done = torch.cuda.Event()
             pend.side_done.record(side)
         for t in (idx, plan.tap_ptr, count, ws):   # not to be reused before the second stream is through
             t.record_stream(side)
         return pend
-    _lib.check(lib.ptv3_kmap_plan_count(_ptr(idx), n, int(ks), _ptr(plan.tap_ptr), _ptr(count), _ptr(ws), nbytes,
-                                        _stream()), "ptv3_kmap_plan_count")
+    _timed("kmap", (n, int(ks), "count"), lambda: _lib.check(
+        lib.ptv3_kmap_plan_count(_ptr(idx), n, int(ks), _ptr(plan.tap_ptr), _ptr(count), _ptr(ws), nbytes, _stream()),
+        "ptv3_kmap_plan_count"))
     pend.count = Readback(count)
     return pend
 
@@ -666,9 +677,9 @@ def conv_plan_direct_finish(pend):
     plan.row_ptr = torch.empty(n + 1, dtype=torch.int32, device=dev)
     plan.pair_in = torch.empty(max(plan.n_pairs, 1), dtype=torch.int32, device=dev)
     plan.pair_slot = torch.empty(max(plan.n_pairs, 1), dtype=torch.int32, device=dev)
-    _lib.check(lib.ptv3_kmap_plan_fill(_ptr(idx), n, pend.ks, _ptr(plan.tap_ptr), _ptr(plan.row_ptr),
-                                       _ptr(plan.pair_in), _ptr(plan.pair_slot), _ptr(pend.ws), pend.nbytes, _stream()),
-               "ptv3_kmap_plan_fill")
+    _timed("kmap", (n, pend.ks, "fill"), lambda: _lib.check(
+        lib.ptv3_kmap_plan_fill(_ptr(idx), n, pend.ks, _ptr(plan.tap_ptr), _ptr(plan.row_ptr), _ptr(plan.pair_in),
+                                _ptr(plan.pair_slot), _ptr(pend.ws), pend.nbytes, _stream()), "ptv3_kmap_plan_fill"))
     return plan
 
 
@@ -686,19 +697,22 @@ def conv_plan_inner(plan5, pend5):
     row_cnt = torch.empty(n, dtype=torch.int32, device=dev)
     row_ptr = torch.zeros(n + 1, dtype=torch.int32, device=dev)
     count = torch.empty(1, dtype=torch.int64, device=dev)
-    _lib.check(lib.ptv3_kmap_plan_inner_count(_ptr(plan5.tap_ptr), n, _ptr(pend5.ws), pend5.nbytes, _ptr(found3),
-                                              _ptr(row_cnt), _ptr(plan.tap_ptr), _ptr(count), _stream()),
-               "ptv3_kmap_plan_inner_count")
-    plan.n_pairs = Readback(count)
-    torch.cumsum(row_cnt, 0, dtype=torch.int32, out=row_ptr[1:])
-    plan.row_ptr = row_ptr
-    cap = max(plan5.n_pairs, 1)
-    plan.pair_in = torch.empty(cap, dtype=torch.int32, device=dev)
-    plan.pair_slot = torch.empty(cap, dtype=torch.int32, device=dev)
-    _lib.check(lib.ptv3_kmap_plan_inner_fill(_ptr(plan5.tap_ptr), _ptr(plan5.row_ptr), _ptr(plan5.pair_in),
-                                             _ptr(plan5.pair_slot), n, plan5.n_pairs, _ptr(found3), _ptr(plan.tap_ptr),
-                                             _ptr(plan.row_ptr), _ptr(plan.pair_in), _ptr(plan.pair_slot), _stream()),
-               "ptv3_kmap_plan_inner_fill")
+    def build():
+        _lib.check(lib.ptv3_kmap_plan_inner_count(_ptr(plan5.tap_ptr), n, _ptr(pend5.ws), pend5.nbytes, _ptr(found3),
+                                                  _ptr(row_cnt), _ptr(plan.tap_ptr), _ptr(count), _stream()),
+                   "ptv3_kmap_plan_inner_count")
+        plan.n_pairs = Readback(count)
+        torch.cumsum(row_cnt, 0, dtype=torch.int32, out=row_ptr[1:])
+        plan.row_ptr = row_ptr
+        cap = max(plan5.n_pairs, 1)
+        plan.pair_in = torch.empty(cap, dtype=torch.int32, device=dev)
+        plan.pair_slot = torch.empty(cap, dtype=torch.int32, device=dev)
+        _lib.check(lib.ptv3_kmap_plan_inner_fill(_ptr(plan5.tap_ptr), _ptr(plan5.row_ptr), _ptr(plan5.pair_in),
+                                                 _ptr(plan5.pair_slot), n, plan5.n_pairs, _ptr(found3), _ptr(plan.tap_ptr),
+                                                 _ptr(plan.row_ptr), _ptr(plan.pair_in), _ptr(plan.pair_slot), _stream()),
+                   "ptv3_kmap_plan_inner_fill")
+
+    _timed("kmap", (n, 3, "inner"), build)
     return plan
 
 
@@ -1133,8 +1147,8 @@ def linear_rows_ok(x, weight):
 
 
 def linear_rows_pays(x, weight, gelu=False):
-    """Where the tall-and-skinny kernel measured at least as fast as the library GEMM (+ GELU launch) on
-    MI355X: everything up to 256 inputs (3-4x at 32 and 64), all but the 3x-wide qkv at 512."""
+    """Where the tall-and-skinny kernel measured at least as fast as a tiled GEMM (+ GELU launch) on
+    MI355X: everything up to 256 inputs, all but the 3x-wide qkv at 512."""
     if not linear_rows_ok(x, weight):
         return False
     nout, k = weight.shape
@@ -1157,10 +1171,9 @@ def linear(x, mod, gelu=False):
         return torch.nn.functional.gelu(y) if gelu else y
     if linear_rows_pays(x, mod.weight, gelu):
         return linear_rows(x, mod.weight, mod.bias, gelu)
-    if not LIBRARY_GEMM and not gelu and linear_gemm_ok(x, mod.weight):
+    if not gelu and linear_gemm_ok(x, mod.weight):
         return linear_gemm(x, mod.weight, mod.bias)
-    y = torch.nn.functional.linear(x, mod.weight, mod.bias)
-    return torch.nn.functional.gelu(y) if gelu else y
+    return linear_any(x, mod.weight, mod.bias, gelu=gelu)
 
 
 def linear_gelu(x, weight, bias=None):
@@ -1223,12 +1236,26 @@ def linear_gemm(x, weight, bias=None, resid=None):
     return out
 
 
-# The long-contraction layers of the default model are plain GEMMs: fc2 at 256 and 512 channels (inside the fused
-# MLP kernel by default, see MLP_ONLY_FUSED_PAYS) and the 512 -> 1536 qkv, on which the library's 256 x 160 tiles
-# measured 26-29 us against 43-48 us for this package's 128 x 128-tile kernel (both bound by what the L2s deliver
-# per tile, see csrc/linearw.hip). False: no library call anywhere in the forward (the default: every kernel of
-# the path is this package's own; 0.04 ms per forward slower). True: the library GEMM takes them.
-LIBRARY_GEMM = False
+def linear_any(x, weight, bias=None, gelu=False, resid=None):
+    """resid + act(x W^T + b) for any shape and fp32 / fp16 / bf16 (ptv3_linear_any_fwd): the fp32 model and the
+    half-precision widths the MFMA kernels do not take. x may have leading dimensions; with resid the result is
+    written over it."""
+    _dev(x, weight, bias, resid)
+    if x.dtype not in _DTYPE_CODE:
+        raise _lib.Ptv3Error(f"linear: unsupported dtype {x.dtype}")
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, x.shape[-1]).contiguous()
+    n, k = x2.shape
+    w = weight.to(x.dtype).contiguous()
+    b = None if bias is None else bias.to(x.dtype).contiguous()
+    if w.dim() != 2 or w.shape[1] != k:
+        raise _lib.Ptv3Error(f"linear: weight {tuple(w.shape)} does not take {k} inputs")
+    if resid is not None and not (resid.is_contiguous() and resid.dtype == x.dtype and resid.shape == (n, w.shape[0])):
+        raise _lib.Ptv3Error("linear_any: resid must be a contiguous (rows, outputs) tensor of x's dtype")
+    out = resid if resid is not None else torch.empty((n, w.shape[0]), dtype=x.dtype, device=x.device)
+    _lib.check(_lib.load().ptv3_linear_any_fwd(_ptr(x2), _ptr(w), _ptr(b), _ptr(resid), _dtype_code(x2), n, k, w.shape[0],
+                                               int(bool(gelu)), _ptr(out), _stream()), "ptv3_linear_any_fwd")
+    return out if resid is not None else out.reshape(*lead, w.shape[0])
 
 
 def linear_gemm_ok(x, weight):
@@ -1300,8 +1327,8 @@ def linear_bn_act(x, lin, bn, gelu):
 MLP_FUSED_CHANNELS = (32, 64)             # widths of the fused block head / tail kernels
 MLP_ONLY_FUSED_CHANNELS = (32, 64, 128, 256, 512)   # widths the fused MLP kernel supports
 # widths at which the model uses it. At 32 ... 128 it beats fc1 + GELU and fc2 as separate launches by 1.8-2.4x; at
-# 256 and 512 it is on a par with Linear kernel + library GEMM inside the forward (0.02-0.04 ms per forward slower)
-# and keeps the hidden tensor and the library out of the path; (32, 64, 128) restores the separate layers there
+# 256 and 512 it is on a par with fc1 + GELU (linear_wide) and fc2 (tiled GEMM) as separate launches and keeps the
+# 4C-wide hidden tensor out of HBM; (32, 64, 128) restores the separate layers there
 MLP_ONLY_FUSED_PAYS = (32, 64, 128, 256, 512)
 
 

@@ -124,7 +124,8 @@ def test_full_size_forward_properties(lidar):
     of the model is defined on coordinates (curve codes, voxel neighbours, grid clusters), so a
     forward over shuffled rows gives the shuffled result. (b) Scenes of a batch do not interact in
     inference (the scene id tops every code, patches and voxel neighbourhoods stay inside a
-    scene): scene 0 alone gives the rows of scene 0. (c) Two runs agree bit for bit."""
+    scene): scene 0 alone gives the rows of scene 0. (c) Two runs agree bit for bit. (d) The rows of scene 0 in the
+    full batch agree with the CPU oracle run on scene 0 alone, which by (b) is the oracle's answer for the batch."""
     from pointtransformerv3_amd import PointTransformerV3
     torch.manual_seed(4)
     model = PointTransformerV3(in_channels=4 if lidar else 6, shuffle_orders=False).eval().half().to(DEV)
@@ -152,6 +153,11 @@ def test_full_size_forward_properties(lidar):
     d0 = dict(grid_coord=d["grid_coord"][:n0], coord=d["coord"][:n0], offset=d["offset"][:1])
     alone = run(d0, feat[:n0])
     assert float((alone - base[:n0]).abs().max()) / scale < 2e-2
+    # (d) the CPU oracle on that scene alone (seconds at this size), against its rows of the full batch
+    perms = _draw_perms(11, False)
+    sd = {k: v.float() for k, v in model.state_dict().items()}
+    want = ptv3_forward(sd, d0["grid_coord"], feat[:n0], d0["offset"], perms=perms)
+    assert rel_err(base[:n0], want) < 2e-2
 
 
 def test_forward_fp32_with_relative_position_bias():
@@ -335,11 +341,10 @@ def test_forward_tiny_and_ragged_scenes_fp32(sizes):
     assert rel_err(point.feat, want) < 1e-4
 
 
-@pytest.mark.parametrize("library", [False, True])
-def test_forward_fp16_with_and_without_the_library_gemm(library):
-    """The default forward makes no library call (ops.LIBRARY_GEMM = False, the fused MLP at every width). The other
-    setting -- fc1 + GELU and fc2 as separate layers from 256 channels on, fc2 and the 512 -> 1536 qkv on the
-    library's GEMM -- is held to the same bar."""
+@pytest.mark.parametrize("separate", [False, True])
+def test_forward_fp16_fused_and_separate_mlp_layers(separate):
+    """The default forward runs the fused MLP at every width. With fc1 + GELU and fc2 as separate layers from 256
+    channels on (fc2 and the 512 -> 1536 qkv on the package's tiled GEMM) the result is held to the same bar."""
     from pointtransformerv3_amd import PointTransformerV3, ops
     torch.manual_seed(1)
     model = PointTransformerV3(shuffle_orders=False).eval().half()
@@ -347,15 +352,59 @@ def test_forward_fp16_with_and_without_the_library_gemm(library):
     perms = _draw_perms(78, False)
     sd = {k: v.float() for k, v in model.state_dict().items()}
     x = feat.astype(np.float16).astype(np.float32)
-    assert ops.LIBRARY_GEMM is False and ops.MLP_ONLY_FUSED_PAYS == ops.MLP_ONLY_FUSED_CHANNELS
-    old = ops.LIBRARY_GEMM, ops.MLP_ONLY_FUSED_PAYS
-    if library:
-        ops.LIBRARY_GEMM, ops.MLP_ONLY_FUSED_PAYS = True, (32, 64, 128)
+    assert ops.MLP_ONLY_FUSED_PAYS == ops.MLP_ONLY_FUSED_CHANNELS
+    old = ops.MLP_ONLY_FUSED_PAYS
+    if separate:
+        ops.MLP_ONLY_FUSED_PAYS = (32, 64, 128)
     try:
         point = _run(model.to(DEV), d, x, torch.float16)
     finally:
-        ops.LIBRARY_GEMM, ops.MLP_ONLY_FUSED_PAYS = old
+        ops.MLP_ONLY_FUSED_PAYS = old
     want = ptv3_forward(sd, d["grid_coord"], x, d["offset"], perms=perms)
+    assert rel_err(point.feat, want) < 2e-2
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.float16, 2e-3), (torch.bfloat16, 1.6e-2)])
+@pytest.mark.parametrize("n,k,nout", [(1000, 48, 144), (513, 6, 32), (77, 200, 50), (4096, 1024, 256), (1, 1, 1)])
+def test_linear_any_matches_torch(dtype, tol, n, k, nout):
+    """ptv3_linear_any_fwd (every Linear of an fp32 model, odd widths in half precision) against float64 torch:
+    plain, with the exact GELU, and accumulating onto a residual in place."""
+    from pointtransformerv3_amd import ops
+    g = torch.Generator().manual_seed(n + k)
+    x = torch.randn(n, k, generator=g).to(dtype)
+    w = (torch.randn(nout, k, generator=g) / k ** 0.5).to(dtype)
+    b = torch.randn(nout, generator=g).to(dtype)
+    res = torch.randn(n, nout, generator=g).to(dtype)
+    ref = x.double() @ w.double().t() + b.double()
+    got = ops.linear_any(x.to(DEV), w.to(DEV), b.to(DEV))
+    assert got.dtype == dtype and rel_err(got, ref) < tol
+    got = ops.linear_any(x.to(DEV), w.to(DEV), b.to(DEV), gelu=True)
+    assert rel_err(got, torch.nn.functional.gelu(ref)) < tol
+    acc = res.to(DEV).clone()
+    got = ops.linear_any(x.to(DEV), w.to(DEV), None, resid=acc)
+    assert got.data_ptr() == acc.data_ptr()
+    assert rel_err(got, res.double() + x.double() @ w.double().t()) < tol
+    # leading dimensions are kept
+    if n % 2 == 0:
+        got = ops.linear_any(x.to(DEV).reshape(2, n // 2, k), w.to(DEV), b.to(DEV))
+        assert got.shape == (2, n // 2, nout) and rel_err(got.reshape(n, nout), ref) < tol
+
+
+def test_forward_widths_outside_the_mfma_kernels_fp16():
+    """Channel widths the MFMA Linear kernels do not take (48, 96, ...: not 32 * 2^j) run through the general
+    Linear kernel, never through a library, and meet the bar."""
+    from pointtransformerv3_amd import PointTransformerV3
+    kw = dict(enc_depths=(1, 1, 1), enc_channels=(48, 96, 192), enc_num_head=(3, 6, 12), enc_patch_size=(128,) * 3,
+              dec_depths=(1, 1), dec_channels=(48, 96), dec_num_head=(3, 6), dec_patch_size=(128,) * 2,
+              stride=(2, 2), in_channels=6)
+    torch.manual_seed(5)
+    model = PointTransformerV3(shuffle_orders=False, **kw).eval().half()
+    d, feat = _data(3000, 2, grid=0.04)
+    perms = _draw_perms(79, False, n_pool=2)
+    sd = {k: v.float() for k, v in model.state_dict().items()}
+    x = feat.astype(np.float16).astype(np.float32)
+    point = _run(model.to(DEV), d, x, torch.float16)
+    want = ptv3_forward(sd, d["grid_coord"], x, d["offset"], perms=perms, **kw)
     assert rel_err(point.feat, want) < 2e-2
 
 

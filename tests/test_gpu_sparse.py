@@ -326,6 +326,22 @@ def test_gelu_of_the_fused_kernels_over_every_fp16_input():
     assert differ.sum().item() <= 64 and (ulps.numel() == 0 or ulps.max().item() == 1), (differ.sum().item(), ulps.max())
 
 
+def test_gelu_of_the_fused_kernels_at_infinities_and_nan():
+    """Non-finite inputs (a first-layer sum beyond the half-precision range): torch's exact GELU returns NaN for
+    +inf, -inf and NaN alike, and so does the kernels' form (its polynomial meets inf * 0). Each row carries its
+    value in column 0 and the weight copies that column to every output, so no product mixes inf with 0."""
+    o = ops()
+    vals = torch.tensor([float("inf"), float("-inf"), float("nan"), 3.0, -2.0, 65504.0, -65504.0, 0.0])
+    x = torch.zeros(32, 32, dtype=torch.float16)
+    x[:8, 0] = vals.half()
+    w = torch.zeros(32, 32, dtype=torch.float16)
+    w[:, 0] = 1.0
+    got = o.linear_rows(x.to(DEV), w.to(DEV), None, gelu=True).cpu()[:8]
+    want = F.gelu(vals.half())[:, None].expand(8, 32)
+    assert torch.equal(torch.isnan(got), torch.isnan(want)) and int(torch.isnan(got[:, 0]).sum()) == 3
+    assert rel_err(torch.nan_to_num(got), torch.nan_to_num(want)) < 1e-3
+
+
 def _lin(cin, cout, g, dtype, bias=True):
     m = torch.nn.Linear(cin, cout, bias=bias)
     with torch.no_grad():
@@ -432,7 +448,8 @@ def test_subm_conv_config3_full_size_fp16():
     """Baseline config 3 at full size: 200,000 room voxels, 64 -> 64 channels, fp16, Kaiming-uniform
     weights. The pair form from the direct plan is checked (a) against the dense output-stationary form,
     (b) row by row against a float64 evaluation of the definition on 3,000 sampled voxels using the
-    neighbour map, whose symmetry and centre column are checked in passing, and (c) for linearity."""
+    neighbour map, whose symmetry and centre column are checked in passing, (c) for linearity; (d) the form the
+    module's dispatch picks here (sparse tiles) against the same float64 rows."""
     from pointtransformerv3_amd import synthetic
     vox = synthetic.room_voxels(200_000, 3000)["grid_coord"]
     idx = np.concatenate([np.zeros((len(vox), 1), np.int32), vox], 1)
@@ -465,6 +482,26 @@ def test_subm_conv_config3_full_size_fp16():
         want[ok] += ff[src[ok]] @ wf[:, t, :].T
     err = np.abs(got.float().cpu().numpy()[sample] - want).max() / np.abs(want).max()
     assert err < 2e-2, err                                                # (b)
+    # (d) the form the module's dispatch picks at this width and sparsity (the one the benchmark times): the module
+    # call itself, with a spy on the wrapper that confirms which kernel ran, against the same float64 rows
+    from pointtransformerv3_amd import ops as ops_mod, sparse
+    conv = sparse.SubMConv3d(c, c, kernel_size=3, bias=True, indice_key="cfg3").to(DEV).half()
+    with torch.no_grad():
+        conv.weight.copy_(w.reshape(conv.weight.shape))
+        conv.bias.copy_(b)
+    x = sparse.SparseConvTensor(feat.to(DEV), dev_idx, [int(v) + 1 for v in vox.max(0)], 1)
+    calls = []
+    real = ops_mod.subm_conv_sparse
+    ops_mod.subm_conv_sparse = lambda *a, **k: (calls.append(1), real(*a, **k))[1]
+    try:
+        with torch.inference_mode():
+            picked = conv(x).features
+    finally:
+        ops_mod.subm_conv_sparse = real
+    assert calls == [1]                                                   # the sparse tile form
+    err = np.abs(picked.float().cpu().numpy()[sample] - want).max() / np.abs(want).max()
+    assert err < 2e-2, err
+    assert rel_err(picked, dense.float().cpu()) < 2e-2
     twice = o.subm_conv_pairs((feat * 2).to(DEV), plan, w.to(DEV), None)
     once = o.subm_conv_pairs(feat.to(DEV), plan, w.to(DEV), None)
     assert rel_err(twice, 2 * once.float().cpu()) < 2e-3                  # (c)

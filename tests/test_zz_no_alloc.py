@@ -30,7 +30,15 @@ def _both(lib, _lib, n, n_scenes, seed, shift=3):
         args = [code0.data_ptr(), order0.data_ptr(), n, shift, offset.data_ptr(), n_scenes, cluster.data_ptr(),
                 idx_ptr.data_ptr(), head.data_ptr(), count.data_ptr()]
         if static:
+            # the warm-up call (n = 0: looks the buffer's address up, launches nothing), then the real one, which
+            # must leave the amount of free device memory as it found it
+            _lib.check(lib.ptv3_pool_clusters_static(None, None, 0, shift, None, 0, None, None, None, None, stream),
+                       "ptv3_pool_clusters_static warm-up")
+            torch.cuda.synchronize()
+            free_before = torch.cuda.mem_get_info()[0]
             _lib.check(lib.ptv3_pool_clusters_static(*args, stream), "ptv3_pool_clusters_static")
+            torch.cuda.synchronize()
+            assert torch.cuda.mem_get_info()[0] == free_before
         else:
             nbytes = lib.ptv3_pool_clusters_workspace_bytes(n)
             ws = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
