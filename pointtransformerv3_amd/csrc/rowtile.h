@@ -56,6 +56,9 @@ __device__ __forceinline__ int perm32(int kk) { return ((kk >> 2) & 1) * 16 + (k
 // that is 4e-6 relative in erfc, in the tail as well; beyond 5.7 the polynomial keeps falling, the term vanishes
 // and no clamp is needed). Seven FMAs, one v_exp_f32, a max and an FMA: the Abramowitz-Stegun 7.1.26 form it
 // replaces took 13 instructions and two transcendentals, and its 1 - (...) cancels in the negative tail.
+// A non-finite input (a first-layer sum beyond the half-precision range, or NaN) gives NaN: the polynomial meets
+// inf * 0. Clamping |x| would cost an instruction per element and, with min/max returning their non-NaN operand,
+// swallow a NaN; torch's own CPU kernel returns NaN or the limit for +-inf depending on the machine's vector path.
 // Over every finite fp16 input (a test passes them all through a kernel): rounded to fp16 the result differs from the correctly rounded
 // GELU for 47 of 63487 inputs, by one ulp (461 with the 7.1.26 form); rounded to bf16 for 10 inputs with |x| < 8.
 __device__ __forceinline__ float gelu_erf(float x) {

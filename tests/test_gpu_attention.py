@@ -69,6 +69,38 @@ def test_attention_parity(dtype, counts, patch):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("counts,heads", [([700], 2), ([513, 1024, 600], 3), ([1000, 33, 1023], 1), ([40_000], 8),
+                                          ([5000, 3000, 777], 32), ([1024], 1)])
+def test_attention_patch_1024_launch_shapes(dtype, counts, heads):
+    """Patch 1024 in half precision, the shape of every released model: sequences shorter than the patch (ragged
+    last step, a 33-point scene), more items than resident work-groups (a last partial round cut into query
+    ranges), fewer items than work-groups, one item."""
+    got, want = _case(counts, 1024, heads, dtype, seed=sum(counts) + heads)
+    assert got.dtype == dtype and got.shape == want.shape
+    assert torch.isfinite(got.float()).all()
+    assert rel_err(got, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_attention_is_deterministic(dtype):
+    """Two launches over the same input give the same bits."""
+    o = ops()
+    rng = np.random.default_rng(5)
+    counts, heads, patch = [3000, 1500], 4, 1024
+    n, C = sum(counts), heads * 16
+    offset = np.cumsum(counts).astype(np.int64)
+    order = np.concatenate([s + rng.permutation(c) for s, c in zip([0, counts[0]], counts)]).astype(np.int64)
+    inverse = np.empty(n, np.int64)
+    inverse[order] = np.arange(n)
+    qkv = torch.randn(n, 3 * C, generator=torch.Generator().manual_seed(5)).to(dtype).to(DEV)
+    gp, gu, gc = o.pad_index(to_dev(offset), offset.tolist(), patch)
+    src, dst = o.attn_slots(to_dev(order), to_dev(inverse), gp, gu)
+    a = o.patch_attention(qkv, heads, src, dst, gc, patch, 0.25)
+    b = o.patch_attention(qkv, heads, src, dst, gc, patch, 0.25)
+    assert torch.equal(a, b) and torch.isfinite(a.float()).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_attention_large_logits(dtype):
     # |q.k| * scale reaches the tens: the running-max path must keep softmax finite and exact
     got, want = _case([1500], 1024, 2, dtype, seed=9, scale_in=3.0)

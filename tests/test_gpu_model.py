@@ -155,7 +155,7 @@ def test_full_size_forward_properties(lidar):
     assert float((alone - base[:n0]).abs().max()) / scale < 2e-2
     # (d) the CPU oracle on that scene alone (seconds at this size), against its rows of the full batch
     perms = _draw_perms(11, False)
-    sd = {k: v.float() for k, v in model.state_dict().items()}
+    sd = {k: v.float().cpu() for k, v in model.state_dict().items()}
     want = ptv3_forward(sd, d0["grid_coord"], feat[:n0], d0["offset"], perms=perms)
     assert rel_err(base[:n0], want) < 2e-2
 

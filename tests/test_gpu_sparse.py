@@ -327,19 +327,20 @@ def test_gelu_of_the_fused_kernels_over_every_fp16_input():
 
 
 def test_gelu_of_the_fused_kernels_at_infinities_and_nan():
-    """Non-finite inputs (a first-layer sum beyond the half-precision range): torch's exact GELU returns NaN for
-    +inf, -inf and NaN alike, and so does the kernels' form (its polynomial meets inf * 0). Each row carries its
-    value in column 0 and the weight copies that column to every output, so no product mixes inf with 0."""
+    """Non-finite inputs (a first-layer sum beyond the half-precision range): NaN stays NaN and +-inf give NaN too
+    (the polynomial meets inf * 0; torch's CPU kernels return NaN or the limits inf / -0 depending on the machine's
+    vector path) -- a blow-up is never turned into a finite number. Finite neighbours against torch. Each row
+    carries its value in column 0 and the weight copies that column to every output, so no product mixes inf with 0."""
     o = ops()
     vals = torch.tensor([float("inf"), float("-inf"), float("nan"), 3.0, -2.0, 65504.0, -65504.0, 0.0])
     x = torch.zeros(32, 32, dtype=torch.float16)
     x[:8, 0] = vals.half()
     w = torch.zeros(32, 32, dtype=torch.float16)
     w[:, 0] = 1.0
-    got = o.linear_rows(x.to(DEV), w.to(DEV), None, gelu=True).cpu()[:8]
-    want = F.gelu(vals.half())[:, None].expand(8, 32)
-    assert torch.equal(torch.isnan(got), torch.isnan(want)) and int(torch.isnan(got[:, 0]).sum()) == 3
-    assert rel_err(torch.nan_to_num(got), torch.nan_to_num(want)) < 1e-3
+    got = o.linear_rows(x.to(DEV), w.to(DEV), None, gelu=True).cpu()[:8].float()
+    assert bool(torch.isnan(got[:3]).all()) and bool(torch.isfinite(got[3:]).all())
+    want = torch.nn.functional.gelu(vals[3:].double()).float()[:, None].expand(5, 32)
+    assert rel_err(got[3:], want) < 1e-3
 
 
 def _lin(cin, cout, g, dtype, bias=True):
