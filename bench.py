@@ -96,6 +96,42 @@ def hbm_entry(timer, name, bytes_fn, steps, kernels):
             "bytes_per_step": byts / steps}
 
 
+def index_kernels_alone(d):
+    """encode, argsort and the pair-list build called alone, 20 times back to back (so that the queue never runs
+    dry and the time is the kernels', not the host's): at the benchmark batch, and at 16 times its points (64
+    scenes), where these kernels are long enough for bandwidth rather than launch and ramp-up to set the time."""
+    from pointtransformerv3_amd import ops
+    dev = "cuda:0"
+    g = torch.from_numpy(d["grid_coord"]).to(dev)
+    b = torch.from_numpy(d["batch"]).to(dev)
+    orders = ["z", "z-trans", "hilbert", "hilbert-trans"]
+    out = {"encode": {}, "sort": {}, "kmap": {}}
+
+    def entry(us, byts):
+        gbs = byts / us / 1e3
+        return {"us": us, "achieved": gbs, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS}
+
+    for tag, reps in (("alone", 1), ("alone_16x", 16)):
+        gg = g.repeat(reps, 1)
+        bb = (b[None, :] + 4 * torch.arange(reps, device=dev)[:, None]).reshape(-1)
+        n = len(bb)
+        depth = 9
+        bits = 3 * depth + int(4 * reps - 1).bit_length()
+        iters = 20 if reps == 1 else 5
+        us = _time_us(lambda: ops.encode_orders(gg, bb, depth, orders), iters=iters)
+        out["encode"][tag] = dict(entry(us, encode_bytes((n, 4))), points=n)
+        code = ops.encode_orders(gg, bb, depth, orders)
+        us = _time_us(lambda: ops.argsort_rows(code, bits), iters=iters)
+        out["sort"][tag] = dict(entry(us, argsort_bytes((n, 4, bits))), points=n, key_bits=bits)
+        del code
+        idx = torch.cat([bb[:, None].int(), gg.int()], 1).contiguous()
+        for ks in (3, 5):
+            us = _time_us(lambda: ops.conv_plan_direct(idx, ks), iters=iters)
+            out["kmap"][f"{tag}_{ks}x{ks}x{ks}"] = dict(entry(us, kmap_bytes((n, ks, "count"))), voxels=n)
+        del idx, gg, bb
+    return out
+
+
 # per 64 keys x 32 queries a wave has to issue 32 v_exp_f32 (8 cycles each on this part) and 16 packed conversions
 # (4 each) whatever else it does: 320 VALU cycles per 2048 scores and SIMD
 VALU_CYCLES_PER_SCORE = 320.0 / 2048.0
@@ -591,6 +627,10 @@ def main():
     ap.add_argument("--train", metavar="DTYPE", default=None, choices=["bfloat16", "float16"],
                     help="instead of the forward benchmark, time a training step (forward, backward, AdamW) of the "
                          "same model and input under autocast to DTYPE and print its own JSON line")
+    ap.add_argument("--micro", metavar="WHICH", default=None, choices=["issue", "loads"],
+                    help="only run a microbenchmark of the part (libptv3_micro.so): `issue` = issue cycles of the "
+                         "instructions the attention and GELU loops are made of, `loads` = vector-load throughput by "
+                         "access pattern and working set; prints the report as text")
     ap.add_argument("--kernels", metavar="PATH", default=None,
                     help="also measure every kernel alone against its roofline and write the table to PATH")
     args = ap.parse_args()
@@ -598,6 +638,19 @@ def main():
         print("bench.py measures one GPU: this build has no multi-GPU path (scenes would shard across "
               "GPUs with no exchange in inference); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+
+    if args.micro:
+        import ctypes
+        path = os.path.join(ROOT, "pointtransformerv3_amd", "libptv3_micro.so")
+        if not os.path.exists(path):
+            sys.exit(f"{path} not found: build it with `make -C pointtransformerv3_amd/csrc`")
+        lib = ctypes.CDLL(path)
+        lib.ptv3_micro_run.restype = ctypes.c_int
+        lib.ptv3_micro_run.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_size_t]
+        buf = ctypes.create_string_buffer(1 << 16)
+        rc = lib.ptv3_micro_run(args.micro.encode(), buf, len(buf))
+        print(buf.value.decode(), end="")
+        sys.exit(0 if rc == 0 else f"ptv3_micro_run({args.micro}) failed with code {rc}")
 
     from pointtransformerv3_amd import PointTransformerV3, ops
 
@@ -687,6 +740,8 @@ def main():
                                            "voxel hash + pair lists of the 5 levels (5x5x5 and 3x3x3 at the first)")
     if not args.no_other_configs:
         del model, data, out
+        for name, alone in index_kernels_alone(d).items():
+            result["roofline"][name].update(alone)
         result["other_configs"] = other_configs()
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
