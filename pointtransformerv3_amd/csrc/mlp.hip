@@ -111,11 +111,8 @@ __global__ __launch_bounds__(MLP_THREADS, 2) void mlp_fused_kernel(
             uint32_t p[8];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                float hv[4];
-#pragma unroll
-                for (int q = 0; q < 4; ++q) hv[q] = gelu_erf(H16<T>::round(d[4 * g + q]));
-                p[2 * g] = H16<T>::pack2(hv[0], hv[1]);
-                p[2 * g + 1] = H16<T>::pack2(hv[2], hv[3]);
+                p[2 * g] = gelu_round_pack2<T>(d[4 * g], d[4 * g + 1]);
+                p[2 * g + 1] = gelu_round_pack2<T>(d[4 * g + 2], d[4 * g + 3]);
             }
             const v8 pa = __builtin_bit_cast(v8, (u32x4){p[0], p[1], p[2], p[3]});
             const v8 pb = __builtin_bit_cast(v8, (u32x4){p[4], p[5], p[6], p[7]});

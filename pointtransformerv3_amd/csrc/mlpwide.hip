@@ -3,6 +3,8 @@
 // As separate kernels this is three passes over an N x 4C tensor (fc1 writes it, GELU rewrites it,
 // fc2 reads it); here a work-group keeps a tile of rows on the CU for the whole chain.
 //
+// The biases of both layers sit in LDS for the life of the work-group: a vector-memory load of them at the head of a
+// chunk would have to wait for the weight fragments requested before it (loads return in order), draining the ring.
 // A work-group of 8 waves owns R = 64 ... 192 rows (RT = 2 or 3 groups of 32 rows per wave). The hidden axis is cut into four chunks of C
 // units; per chunk, stage A computes GELU(x W1_chunk^T + b1) for the tile into LDS and stage B adds
 // its product with W2's chunk to the output accumulators, which stay in registers across the
@@ -64,21 +66,24 @@ __global__ __launch_bounds__(256) void mlp_pack_batch_kernel(const ptv3_mlp_pack
 }
 
 // PACKED: w1 is the packed stream of both matrices and w2 is not read
-template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RT>
-__global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
+template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RT, int THREADS, int MINW>
+__global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
     const T* __restrict__ x, const T* __restrict__ resid, const T* __restrict__ w1, const T* __restrict__ b1,
     const T* __restrict__ w2, const T* __restrict__ b2, int64_t n, T* __restrict__ out) {
     typedef typename H16<T>::v8 v8;
-    static_assert(WM * WN == MW_WAVES && C == 32 * MT * WN, "8 waves cover R x C");
+    static_assert(WM * WN * PTV3_WAVE == THREADS && C == 32 * MT * WN, "the waves cover R x C");
     constexpr int R = 32 * RT * WM, H = 4 * C, XS = C + MW_PAD;   // a wave owns RT groups of 32 rows
     constexpr int KU = C / 32;            // 32-wide contraction steps per stage
     constexpr int UNITS = 4 * 2 * KU;     // weight steps per tile: 4 chunks x (stage A, stage B)
     static_assert(KU % DEPTH == 0, "the ring is indexed statically");
     constexpr int PPR = C / 8;            // 16-byte pieces per row
-    constexpr int PIECES = R * PPR / MW_THREADS;
+    constexpr int PIECES = R * PPR / THREADS;
     extern __shared__ __align__(16) unsigned char mw_smem[];
     T* xt = (T*)mw_smem;      // [R][XS] input tile
     T* ht = xt + R * XS;      // [R][XS] hidden chunk, then the output tile
+    T* bias_lds = ht + R * XS;   // [4 C] fc1's bias, [C] fc2's: read per chunk without touching the vector-memory queue
+    for (int i = threadIdx.x; i < 5 * C / 8; i += THREADS)
+        *(u32x4*)(bias_lds + i * 8) = *(const u32x4*)((i < 4 * C / 8 ? b1 : b2 - 4 * C) + i * 8);
 
     const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
     const int col = lane & 31, hf = lane >> 5;
@@ -148,7 +153,7 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
         // ---- x tile -> LDS
 #pragma unroll
         for (int i = 0; i < PIECES; ++i) {
-            const int p = tid + i * MW_THREADS;
+            const int p = tid + i * THREADS;
             const int rr = p / PPR, pc = p % PPR;
             u32x4 v = {0, 0, 0, 0};
             if (row0 + rr < n) v = *(const u32x4*)(x + (row0 + rr) * C + pc * 8);
@@ -171,7 +176,7 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
             for (int a = 0; a < MT; ++a)
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const u32x2 bb = *(const u32x2*)(b1 + chunk * C + ch0 + a * 32 + 8 * g + 4 * hf);
+                    const u32x2 bb = *(const u32x2*)(bias_lds + chunk * C + ch0 + a * 32 + 8 * g + 4 * hf);
                     const float bias[4] = {H16<T>::lo(bb[0]), H16<T>::hi(bb[0]), H16<T>::lo(bb[1]), H16<T>::hi(bb[1])};
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt)
@@ -187,11 +192,9 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
                     const int hh = ch0 + a * 32 + 8 * g + 4 * hf;
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt) {
-                        float hv[4];
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) hv[q] = gelu_erf(H16<T>::round(hacc[a][rt][4 * g + q]));
                         *(u32x2*)(ht + (r0 + rt * 32 + col) * XS + hh) =
-                            (u32x2){H16<T>::pack2(hv[0], hv[1]), H16<T>::pack2(hv[2], hv[3])};
+                            (u32x2){gelu_round_pack2<T>(hacc[a][rt][4 * g], hacc[a][rt][4 * g + 1]),
+                                    gelu_round_pack2<T>(hacc[a][rt][4 * g + 2], hacc[a][rt][4 * g + 3])};
                     }
                 }
             __syncthreads();
@@ -205,7 +208,7 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const int cc = ch0 + a * 32 + 8 * g + 4 * hf;
-                const u32x2 bb = *(const u32x2*)(b2 + cc);
+                const u32x2 bb = *(const u32x2*)(bias_lds + 4 * C + cc);
                 const float bias[4] = {H16<T>::lo(bb[0]), H16<T>::hi(bb[0]), H16<T>::lo(bb[1]), H16<T>::hi(bb[1])};
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt)
@@ -216,7 +219,7 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < PIECES; ++i) {
-            const int p = tid + i * MW_THREADS;
+            const int p = tid + i * THREADS;
             const int rr = p / PPR, pc = p % PPR;
             if (row0 + rr < n) {
                 const u32x4 o = *(const u32x4*)(ht + rr * XS + pc * 8);
@@ -232,18 +235,18 @@ __global__ __launch_bounds__(MW_THREADS) void mlp_wide_kernel(
     }
 }
 
-template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RT = 2>
+template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RT = 2, int THREADS = MW_THREADS, int MINW = 2>
 int launch_mlp_wide(const void* x, const void* resid, const void* w1, const void* b1, const void* w2, const void* b2,
                     int64_t n, void* out, hipStream_t stream) {
     constexpr int R = 32 * RT * WM;
-    const size_t lds = (size_t)2 * R * (C + MW_PAD) * sizeof(T);
-    auto kern = mlp_wide_kernel<T, C, WM, WN, MT, DEPTH, PACKED, RT>;
+    const size_t lds = ((size_t)2 * R * (C + MW_PAD) + 5 * C) * sizeof(T);
+    auto kern = mlp_wide_kernel<T, C, WM, WN, MT, DEPTH, PACKED, RT, THREADS, MINW>;
     static LdsGrant grant_configured;   // per instantiation and device
     if (const int rc_ = ptv3_allow_lds((const void*)kern, lds, grant_configured)) return rc_;
     // persistent work-groups: as many as the machine holds at a time
     const int64_t tiles = (n + R - 1) / R;
-    const int64_t resident = 256;   // one work-group per CU: two waves per SIMD at this register count
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles < resident ? tiles : resident)), dim3(MW_THREADS), lds, stream,
+    const int64_t resident = (int64_t)256 * MINW * 256 / THREADS;   // MINW waves per SIMD, THREADS / 256 of them from one work-group
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles < resident ? tiles : resident)), dim3(THREADS), lds, stream,
                        (const T*)x, (const T*)resid, (const T*)w1, (const T*)b1, (const T*)w2, (const T*)b2, n, (T*)out);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? PTV3_OK : (int)e;
