@@ -631,6 +631,12 @@ def main():
                     help="only run a microbenchmark of the part (libptv3_micro.so): `issue` = issue cycles of the "
                          "instructions the attention and GELU loops are made of, `loads` = vector-load throughput by "
                          "access pattern and working set; prints the report as text")
+    ap.add_argument("--summarise", metavar="DIR", default=None,
+                    help="no GPU work: turn the raw files a measurement batch left in DIR (JSON lines of this script, "
+                         "rocprofv3 traces and counter collections) into the text summaries under --out; sections "
+                         "whose raw files are missing say which command writes them")
+    ap.add_argument("--recipe", action="store_true", help="with --summarise DIR: only print the measurement batch as shell lines")
+    ap.add_argument("--out", metavar="DIR", default=os.path.join(ROOT, "profiles"), help="where --summarise writes")
     ap.add_argument("--kernels", metavar="PATH", default=None,
                     help="also measure every kernel alone against its roofline and write the table to PATH")
     args = ap.parse_args()
@@ -638,6 +644,14 @@ def main():
         print("bench.py measures one GPU: this build has no multi-GPU path (scenes would shard across "
               "GPUs with no exchange in inference); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+
+    if args.summarise:
+        import bench_summaries
+        if args.recipe:
+            print("\n".join(bench_summaries.recipe(args.summarise)))
+        else:
+            bench_summaries.summarise(args.summarise, args.out)
+        return
 
     if args.micro:
         import ctypes
