@@ -94,27 +94,53 @@ __global__ __launch_bounds__(NW * PTV3_WAVE, (NW == 8 ? 2 : 1)) void linear_rows
     __syncthreads();
 
     const int64_t n_tiles = (n + 31) / 32;
-    for (int64_t tile = (int64_t)row_group * LIN_WAVES + wave; tile < n_tiles; tile += (int64_t)per_chunk * LIN_WAVES) {
-        const int64_t row0 = tile * 32;
-        // ---- 32 rows -> operand fragments, 64 channels at a time: lane (r, piece) moves 16 bytes
-        v8 xf[KS];
-        constexpr int PART = K < SW ? K : SW;             // channels staged at a time
-        constexpr int PPP = PART / 8;                     // 16-byte pieces per row and part
-        constexpr int ITS = 32 * PPP / PTV3_WAVE;         // pieces per lane and part
+    constexpr int PART = K < SW ? K : SW;             // channels staged at a time
+    constexpr int PPP = PART / 8;                     // 16-byte pieces per row and part
+    constexpr int ITS = 32 * PPP / PTV3_WAVE;         // pieces per lane and part
+    constexpr int PARTS = K / PART;
+    // Up to 128 inputs a wave's 32 rows are 32 registers per lane: the next tile's rows are requested before this
+    // tile's products start, so their way from HBM is covered by a whole tile of work instead of by the other
+    // waves of the SIMD alone: 2-5 % on the plain layers. (At 256 and 512 inputs the operand fragments leave no
+    // room for a second set, and with the BatchNorm / GELU epilogues the extra registers cost a wave per SIMD.)
+    constexpr bool AHEAD = K <= 128 && !BN && ACT == ACT_NONE;
+    auto fetch = [&](int64_t t, u32x4 (&raw)[PARTS][ITS]) {
+        const int64_t r0 = t * 32;
 #pragma unroll
-        for (int part = 0; part < K / PART; ++part) {
-            u32x4 raw[ITS];
+        for (int part = 0; part < PARTS; ++part)
 #pragma unroll
             for (int it = 0; it < ITS; ++it) {
                 const int pidx = it * PTV3_WAVE + lane;    // 32 rows x PPP pieces
-                const int64_t r = row0 + pidx / PPP;
-                raw[it] = (u32x4){0, 0, 0, 0};
-                if (r < n) raw[it] = *(const u32x4*)(x + r * K + part * PART + (pidx % PPP) * 8);
+                const int64_t r = r0 + pidx / PPP;
+                raw[part][it] = (u32x4){0, 0, 0, 0};
+                if (r < n) raw[part][it] = *(const u32x4*)(x + r * K + part * PART + (pidx % PPP) * 8);
             }
+    };
+    const int64_t stride = (int64_t)per_chunk * LIN_WAVES;
+    u32x4 ahead[AHEAD ? PARTS : 1][AHEAD ? ITS : 1];
+    int64_t tile = (int64_t)row_group * LIN_WAVES + wave;
+    if constexpr (AHEAD) {
+        if (tile < n_tiles) fetch(tile, ahead);
+    }
+    for (; tile < n_tiles; tile += stride) {
+        const int64_t row0 = tile * 32;
+        // ---- 32 rows -> operand fragments, 64 channels at a time: lane (r, piece) moves 16 bytes
+        v8 xf[KS];
+        u32x4 raw[PARTS][ITS];
+        if constexpr (AHEAD) {
+#pragma unroll
+            for (int part = 0; part < PARTS; ++part)
+#pragma unroll
+                for (int it = 0; it < ITS; ++it) raw[part][it] = ahead[part][it];
+            if (tile + stride < n_tiles) fetch(tile + stride, ahead);
+        } else {
+            fetch(tile, raw);
+        }
+#pragma unroll
+        for (int part = 0; part < PARTS; ++part) {
 #pragma unroll
             for (int it = 0; it < ITS; ++it) {
                 const int pidx = it * PTV3_WAVE + lane;
-                *(u32x4*)(xs + (pidx / PPP) * LIN_XSS + (pidx % PPP) * 8) = raw[it];
+                *(u32x4*)(xs + (pidx / PPP) * LIN_XSS + (pidx % PPP) * 8) = raw[part][it];
             }
             asm volatile("" ::: "memory");
 #pragma unroll

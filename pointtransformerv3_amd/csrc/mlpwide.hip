@@ -21,6 +21,8 @@
 // contiguous KB costs. ptv3_mlp_pack_weights therefore writes both matrices once in the order of the stream
 // (step, 32-unit block, piece, lane), and the PACKED kernel fetches every fragment as one contiguous KB.
 // Intermediates are rounded to the storage type where the separate layers would have stored them.
+#include <type_traits>
+
 #include "rowtile.h"
 
 namespace {
@@ -65,23 +67,25 @@ __global__ __launch_bounds__(256) void mlp_pack_batch_kernel(const ptv3_mlp_pack
     *(u32x4*)((uint16_t*)job.packed + idx * 8) = *(const u32x4*)src;
 }
 
-// PACKED: w1 is the packed stream of both matrices and w2 is not read
-template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RT, int THREADS, int MINW>
+// PACKED: w1 is the packed stream of both matrices and w2 is not read.
+// A work-group walks its rows in passes of 1 .. RTMAX groups of 32 rows per wave; the host gives every resident
+// work-group the same number of row groups (with tiles of one fixed size the last round of a launch of 37,681 rows at
+// 256 channels ran at half occupancy).
+template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RTMAX, int THREADS, int MINW>
 __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
     const T* __restrict__ x, const T* __restrict__ resid, const T* __restrict__ w1, const T* __restrict__ b1,
-    const T* __restrict__ w2, const T* __restrict__ b2, int64_t n, T* __restrict__ out) {
+    const T* __restrict__ w2, const T* __restrict__ b2, int64_t n, int upw, T* __restrict__ out) {
     typedef typename H16<T>::v8 v8;
     static_assert(WM * WN * PTV3_WAVE == THREADS && C == 32 * MT * WN, "the waves cover R x C");
-    constexpr int R = 32 * RT * WM, H = 4 * C, XS = C + MW_PAD;   // a wave owns RT groups of 32 rows
+    constexpr int RMAX = 32 * RTMAX * WM, H = 4 * C, XS = C + MW_PAD;
     constexpr int KU = C / 32;            // 32-wide contraction steps per stage
-    constexpr int UNITS = 4 * 2 * KU;     // weight steps per tile: 4 chunks x (stage A, stage B)
+    constexpr int UNITS = 4 * 2 * KU;     // weight steps per pass: 4 chunks x (fc1, fc2)
     static_assert(KU % DEPTH == 0, "the ring is indexed statically");
     constexpr int PPR = C / 8;            // 16-byte pieces per row
-    constexpr int PIECES = R * PPR / THREADS;
     extern __shared__ __align__(16) unsigned char mw_smem[];
-    T* xt = (T*)mw_smem;      // [R][XS] input tile
-    T* ht = xt + R * XS;      // [R][XS] hidden chunk, then the output tile
-    T* bias_lds = ht + R * XS;   // [4 C] fc1's bias, [C] fc2's: read per chunk without touching the vector-memory queue
+    T* xt = (T*)mw_smem;                  // [RMAX][XS] input tile
+    T* ht = xt + RMAX * XS;               // [RMAX][XS] hidden chunk, then the output tile
+    T* bias_lds = ht + RMAX * XS;         // [4 C] fc1's bias, [C] fc2's: read per chunk without touching the vector-memory queue
     for (int i = threadIdx.x; i < 5 * C / 8; i += THREADS)
         *(u32x4*)(bias_lds + i * 8) = *(const u32x4*)((i < 4 * C / 8 ? b1 : b2 - 4 * C) + i * 8);
 
@@ -89,12 +93,11 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
     const int col = lane & 31, hf = lane >> 5;
     const int wm = wave % WM, wn = wave / WM;
     const int ch0 = wn * 32 * MT;   // first output unit of this wave (hidden unit inside a chunk / channel)
-    const int r0 = wm * 32 * RT;    // first row of this wave inside the tile
 
-    // weight step u: chunk u / (2 KU), stage (u / KU) & 1, 32-wide step u % KU; lane (col, hf) of
-    // output tile a takes 2 x 8 consecutive inputs of weight row ch0 + 32 a + col
-    auto issue = [&](int u, u32x4 (&r)[MT][2]) {
-        const int chunk = u / (2 * KU), st = (u / KU) & 1, kk = u % KU;
+    // weight step q of a pass: chunk q / (2 KU), layer (q / KU) & 1 (fc1, fc2), 32-wide step kk = q % KU; lane (col, hf)
+    // of output tile a takes 2 x 8 consecutive inputs of weight row ch0 + 32 a + col
+    auto issue = [&](int q, u32x4 (&r)[MT][2]) {
+        const int chunk = q / (2 * KU), st = (q / KU) & 1, kk = q % KU, u = q;
 #pragma unroll
         for (int a = 0; a < MT; ++a) {
             if (PACKED) {
@@ -114,16 +117,21 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
 #pragma unroll
     for (int j = 0; j < DEPTH; ++j) issue(j, ring[j]);
 
-    // one stage: acc[a][rt] += W rows (ring) x tile rows (LDS `src`); u0 = first weight step
-    auto stage = [&](const T* src, f32x16 (&acc)[MT][RT], int u0) {
-        const T* brow = src + (r0 + col) * XS + hf * 16;
-        for (int kk0 = 0; kk0 < KU; kk0 += DEPTH) {
+    // one pass over RT_ row groups per wave, rows [row0, row0 + 32 RT_ WM) of which those below row_end exist
+    auto pass = [&](auto rt_c, int64_t row0, int64_t row_end) {
+        constexpr int RT_ = decltype(rt_c)::value;
+        constexpr int PIECES = 32 * RT_ * WM * PPR / THREADS;
+        const int r0 = wm * 32 * RT_;    // first row of this wave inside the tile
+
+        // one matrix stage: acc[a][rt] += W rows (ring) x tile rows (LDS `src`); q0 = its first weight step
+        auto stage = [&](const T* src, f32x16 (&acc)[MT][RT_], int q0) {
+            const T* brow = src + (r0 + col) * XS + hf * 16;
 #pragma unroll
-            for (int j = 0; j < DEPTH; ++j) {
-                const int kk = kk0 + j;
-                u32x4 bf[RT][2];
+            for (int kk = 0; kk < KU; ++kk) {
+                const int j = kk % DEPTH;
+                u32x4 bf[RT_][2];
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt) {
+                for (int rt = 0; rt < RT_; ++rt) {
                     bf[rt][0] = *(const u32x4*)(brow + rt * 32 * XS + kk * 32);
                     bf[rt][1] = *(const u32x4*)(brow + rt * 32 * XS + kk * 32 + 8);
                 }
@@ -133,45 +141,20 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
                     af[a][0] = ring[j][a][0];
                     af[a][1] = ring[j][a][1];
                 }
-                int un = u0 + kk + DEPTH;
-                if (un >= UNITS) un -= UNITS;   // the stream of the next tile is the same
-                issue(un, ring[j]);
+                int qn = q0 + kk + DEPTH;
+                if (qn >= UNITS) qn -= UNITS;   // the stream of the next pass is the same
+                issue(qn, ring[j]);
 #pragma unroll
                 for (int a = 0; a < MT; ++a)
 #pragma unroll
-                    for (int rt = 0; rt < RT; ++rt) {
+                    for (int rt = 0; rt < RT_; ++rt) {
                         acc[a][rt] = H16<T>::mfma(__builtin_bit_cast(v8, af[a][0]), __builtin_bit_cast(v8, bf[rt][0]), acc[a][rt]);
                         acc[a][rt] = H16<T>::mfma(__builtin_bit_cast(v8, af[a][1]), __builtin_bit_cast(v8, bf[rt][1]), acc[a][rt]);
                     }
             }
-        }
-    };
-
-    const int64_t n_tiles = (n + R - 1) / R;
-    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-        const int64_t row0 = tile * R;
-        // ---- x tile -> LDS
-#pragma unroll
-        for (int i = 0; i < PIECES; ++i) {
-            const int p = tid + i * THREADS;
-            const int rr = p / PPR, pc = p % PPR;
-            u32x4 v = {0, 0, 0, 0};
-            if (row0 + rr < n) v = *(const u32x4*)(x + (row0 + rr) * C + pc * 8);
-            *(u32x4*)(xt + rr * XS + pc * 8) = v;
-        }
-        __syncthreads();
-
-        f32x16 acc[MT][RT];
-#pragma unroll
-        for (int a = 0; a < MT; ++a)
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[a][rt][v] = 0.f;
-
-        for (int chunk = 0; chunk < 4; ++chunk) {
-            // stage A accumulates on top of fc1's bias (the MFMAs' C operand) instead of adding it afterwards
-            f32x16 hacc[MT][RT];
+        };
+        // fc1's sums start from its bias (the MFMAs' C operand) instead of having it added afterwards
+        auto bias_into = [&](f32x16 (&hacc)[MT][RT_], int chunk) {
 #pragma unroll
             for (int a = 0; a < MT; ++a)
 #pragma unroll
@@ -179,11 +162,34 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
                     const u32x2 bb = *(const u32x2*)(bias_lds + chunk * C + ch0 + a * 32 + 8 * g + 4 * hf);
                     const float bias[4] = {H16<T>::lo(bb[0]), H16<T>::hi(bb[0]), H16<T>::lo(bb[1]), H16<T>::hi(bb[1])};
 #pragma unroll
-                    for (int rt = 0; rt < RT; ++rt)
+                    for (int rt = 0; rt < RT_; ++rt)
 #pragma unroll
                         for (int q = 0; q < 4; ++q) hacc[a][rt][4 * g + q] = bias[q];
                 }
-            stage(xt, hacc, chunk * 2 * KU);
+        };
+        // ---- x tile -> LDS
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            const int p = tid + i * THREADS;
+            const int rr = p / PPR, pc = p % PPR;
+            u32x4 v = {0, 0, 0, 0};
+            if (row0 + rr < row_end) v = *(const u32x4*)(x + (row0 + rr) * C + pc * 8);
+            *(u32x4*)(xt + rr * XS + pc * 8) = v;
+        }
+        __syncthreads();
+
+        f32x16 acc[MT][RT_], hacc[MT][RT_];
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int rt = 0; rt < RT_; ++rt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[a][rt][v] = 0.f;
+
+#pragma unroll 1   // unrolled, the chunks' loads are hoisted over each other and spill
+        for (int c = 0; c < 4; ++c) {
+            bias_into(hacc, c);
+            stage(xt, hacc, 2 * c * KU);
             // hacc[a][rt][v]: hidden unit ch0 + 32 a + 8 (v / 4) + 4 hf + v % 4 of row r0 + 32 rt + col
 #pragma unroll
             for (int a = 0; a < MT; ++a)
@@ -191,14 +197,13 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
                 for (int g = 0; g < 4; ++g) {
                     const int hh = ch0 + a * 32 + 8 * g + 4 * hf;
 #pragma unroll
-                    for (int rt = 0; rt < RT; ++rt) {
+                    for (int rt = 0; rt < RT_; ++rt)
                         *(u32x2*)(ht + (r0 + rt * 32 + col) * XS + hh) =
                             (u32x2){gelu_round_pack2<T>(hacc[a][rt][4 * g], hacc[a][rt][4 * g + 1]),
                                     gelu_round_pack2<T>(hacc[a][rt][4 * g + 2], hacc[a][rt][4 * g + 3])};
-                    }
                 }
             __syncthreads();
-            stage(ht, acc, chunk * 2 * KU + KU);
+            stage(ht, acc, (2 * c + 1) * KU);
             __syncthreads();
         }
 
@@ -211,7 +216,7 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
                 const u32x2 bb = *(const u32x2*)(bias_lds + 4 * C + cc);
                 const float bias[4] = {H16<T>::lo(bb[0]), H16<T>::hi(bb[0]), H16<T>::lo(bb[1]), H16<T>::hi(bb[1])};
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt)
+                for (int rt = 0; rt < RT_; ++rt)
                     *(u32x2*)(ht + (r0 + rt * 32 + col) * XS + cc) =
                         (u32x2){H16<T>::pack2(acc[a][rt][4 * g] + bias[0], acc[a][rt][4 * g + 1] + bias[1]),
                                 H16<T>::pack2(acc[a][rt][4 * g + 2] + bias[2], acc[a][rt][4 * g + 3] + bias[3])};
@@ -221,7 +226,7 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
         for (int i = 0; i < PIECES; ++i) {
             const int p = tid + i * THREADS;
             const int rr = p / PPR, pc = p % PPR;
-            if (row0 + rr < n) {
+            if (row0 + rr < row_end) {
                 const u32x4 o = *(const u32x4*)(ht + rr * XS + pc * 8);
                 const u32x4 s = *(const u32x4*)(resid + (row0 + rr) * C + pc * 8);
                 u32x4 r;
@@ -231,23 +236,45 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
                 *(u32x4*)(out + (row0 + rr) * C + pc * 8) = r;
             }
         }
-        // the next tile's first write to ht comes after the barrier that follows its x tile load
+        // the next pass writes the hidden buffers only after the barrier that follows its x tile load
+    };
+
+    // Every work-group does `upw` row groups of 32 WM rows in passes of equal shape: in a round all work-groups take
+    // neighbouring tiles of rt row groups (5 = 3 + 2, 4 = 2 + 2), so the rows in flight at any time are one window
+    // of the matrix and the last round is as full as the first.
+    constexpr int UNIT = 32 * WM;
+    int64_t base = 0;   // first row group of the round
+    for (int left = upw; left > 0;) {
+        const int passes = (left + RTMAX - 1) / RTMAX;
+        const int rt = (left + passes - 1) / passes;
+        const int64_t row0 = (base + (int64_t)blockIdx.x * rt) * UNIT;
+        if (row0 < n) {
+            if (RTMAX >= 3 && rt == 3) pass(std::integral_constant<int, (RTMAX >= 3 ? 3 : 1)>{}, row0, n);
+            else if (RTMAX >= 2 && rt == 2) pass(std::integral_constant<int, (RTMAX >= 2 ? 2 : 1)>{}, row0, n);
+            else pass(std::integral_constant<int, 1>{}, row0, n);
+        }
+        base += (int64_t)gridDim.x * rt;
+        left -= rt;
     }
 }
 
-template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RT = 2, int THREADS = MW_THREADS, int MINW = 2>
+template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RTMAX, int THREADS = MW_THREADS, int MINW = 2>
 int launch_mlp_wide(const void* x, const void* resid, const void* w1, const void* b1, const void* w2, const void* b2,
                     int64_t n, void* out, hipStream_t stream) {
-    constexpr int R = 32 * RT * WM;
-    const size_t lds = ((size_t)2 * R * (C + MW_PAD) + 5 * C) * sizeof(T);
-    auto kern = mlp_wide_kernel<T, C, WM, WN, MT, DEPTH, PACKED, RT, THREADS, MINW>;
+    constexpr int RMAX = 32 * RTMAX * WM, UNIT = 32 * WM;
+    const size_t lds = ((size_t)2 * RMAX * (C + MW_PAD) + 5 * C) * sizeof(T);
+    auto kern = mlp_wide_kernel<T, C, WM, WN, MT, DEPTH, PACKED, RTMAX, THREADS, MINW>;
     static LdsGrant grant_configured;   // per instantiation and device
     if (const int rc_ = ptv3_allow_lds((const void*)kern, lds, grant_configured)) return rc_;
-    // persistent work-groups: as many as the machine holds at a time
-    const int64_t tiles = (n + R - 1) / R;
-    const int64_t resident = (int64_t)256 * MINW * 256 / THREADS;   // MINW waves per SIMD, THREADS / 256 of them from one work-group
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles < resident ? tiles : resident)), dim3(THREADS), lds, stream,
-                       (const T*)x, (const T*)resid, (const T*)w1, (const T*)b1, (const T*)w2, (const T*)b2, n, (T*)out);
+    // as many work-groups as the machine holds at a time (MINW waves per SIMD, THREADS / 256 of them from one
+    // work-group), each with the same number of row groups
+    const int64_t resident = (int64_t)256 * MINW * 256 / THREADS;
+    const int64_t units = (n + UNIT - 1) / UNIT;
+    const int64_t grid = units < resident ? units : resident;
+    const int64_t upw = (units + grid - 1) / grid;
+    if (upw > 0x7fffffffLL) return PTV3_EINVAL;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), lds, stream,
+                       (const T*)x, (const T*)resid, (const T*)w1, (const T*)b1, (const T*)w2, (const T*)b2, n, (int)upw, (T*)out);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? PTV3_OK : (int)e;
 }
@@ -255,19 +282,11 @@ int launch_mlp_wide(const void* x, const void* resid, const void* w1, const void
 template <bool PACKED>
 int mlp_wide_any(const void* x, const void* resid, const void* w1, const void* b1, const void* w2, const void* b2,
                  int dtype, int64_t n, int channels, void* out, hipStream_t stream) {
-    // 256 channels: 96-row tiles stream a third less weight per row than 64-row tiles; taken when they also need
-    // fewer rounds of the 256 persistent work-groups per unit of work (a 96-row tile costs about 1.25 of a 64-row one)
-    const int64_t r64 = ptv3_ceil_div(ptv3_ceil_div(n, 64), 256), r96 = ptv3_ceil_div(ptv3_ceil_div(n, 96), 256);
-    const bool three = 5 * r96 < 4 * r64;
-    const int64_t r128 = ptv3_ceil_div(ptv3_ceil_div(n, 128), 256), r192 = ptv3_ceil_div(ptv3_ceil_div(n, 192), 256);
-    const bool three128 = 5 * r192 < 4 * r128;
-#define PTV3_MW(T)                                                                                                          \
-    do {                                                                                                                    \
-        if (channels == 128 && three128) return launch_mlp_wide<T, 128, 2, 4, 1, 4, PACKED, 3>(x, resid, w1, b1, w2, b2, n, out, stream); \
-        if (channels == 128) return launch_mlp_wide<T, 128, 2, 4, 1, 4, PACKED>(x, resid, w1, b1, w2, b2, n, out, stream);   \
-        if (channels == 256 && three) return launch_mlp_wide<T, 256, 1, 8, 1, 4, PACKED, 3>(x, resid, w1, b1, w2, b2, n, out, stream); \
-        if (channels == 256) return launch_mlp_wide<T, 256, 1, 8, 1, 4, PACKED>(x, resid, w1, b1, w2, b2, n, out, stream);   \
-        if (channels == 512) return launch_mlp_wide<T, 512, 1, 8, 2, 2, PACKED>(x, resid, w1, b1, w2, b2, n, out, stream);   \
+#define PTV3_MW(T)                                                                                                      \
+    do {                                                                                                                \
+        if (channels == 128) return launch_mlp_wide<T, 128, 2, 4, 1, 4, PACKED, 3>(x, resid, w1, b1, w2, b2, n, out, stream); \
+        if (channels == 256) return launch_mlp_wide<T, 256, 1, 8, 1, 4, PACKED, 3>(x, resid, w1, b1, w2, b2, n, out, stream); \
+        if (channels == 512) return launch_mlp_wide<T, 512, 1, 8, 2, 2, PACKED, 2>(x, resid, w1, b1, w2, b2, n, out, stream); \
     } while (0)
     if (dtype == PTV3_F16) PTV3_MW(_Float16);
     if (dtype == PTV3_BF16) PTV3_MW(__bf16);
