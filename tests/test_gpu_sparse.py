@@ -238,7 +238,10 @@ def test_tap_major_layout_is_the_transpose():
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("c,n", [(32, 1), (32, 5000), (64, 33), (64, 70_001), (128, 1), (128, 300), (128, 40_001),
-                                 (256, 63), (256, 64), (256, 20_001), (512, 65), (512, 9000)])
+                                 (256, 63), (256, 64), (256, 20_001), (512, 65), (512, 9000),
+                                 # more row groups than resident work-groups: rounds of 2 + 2, 3 + 2, 3 + 3 + 2 and
+                                 # 2 + 1 groups per wave, the last round partly past the end
+                                 (256, 32_768), (256, 32_773), (128, 114_691), (512, 24_577), (512, 16_385)])
 def test_mlp_fused_parity(dtype, c, n):
     import torch.nn.functional as F
     g = torch.Generator().manual_seed(c + n)
