@@ -258,7 +258,7 @@ def test_mlp_fused_parity(dtype, c, n):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("c,n", [(128, 1), (128, 40_001), (256, 64), (256, 20_001), (512, 9000)])
+@pytest.mark.parametrize("c,n", [(128, 1), (128, 40_001), (256, 64), (256, 20_001), (512, 9000), (256, 32_773), (512, 16_385)])
 def test_mlp_fused_packed_weights_give_the_same_bits(dtype, c, n):
     """The packed weight stream only changes where the kernel finds its operands: against the torch fp32 layers
     within the half-precision bar, and bit for bit what the kernel gives on the layers' own layout."""
