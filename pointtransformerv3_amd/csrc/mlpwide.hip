@@ -28,7 +28,6 @@
 namespace {
 
 constexpr int MW_THREADS = 512;
-constexpr int MW_WAVES = MW_THREADS / PTV3_WAVE;
 constexpr int MW_PAD = 8;   // halfs of padding per LDS row
 
 // weight step u of the stream (UNITS = 8 C / 32 of them): chunk u / (2 KU), stage (u / KU) & 1 (fc1, fc2), 32-wide
