@@ -291,6 +291,15 @@ int ptv3_subm_conv_pack_weight_batch(const ptv3_pack_job *jobs, int n_jobs, int6
 int ptv3_subm_conv_tiles_fwd(const void *feat, int dtype, int64_t n, int channels, int taps,
                              const void *packed_weight, const void *bias, const int32_t *tile_tap,
                              const int32_t *tile_pair, const int32_t *vox_taps, void *out, void *stream);
+/* The same with tiles of tile_voxels outputs: 128 (what the three functions above use), or 96 at 128 channels
+ * (same call site, model.py:546-552). The lists must have been made with the same tile_voxels. A launch runs in
+ * rounds of the work-groups the part holds at a time; the caller picks the size whose last round is fuller. */
+int64_t ptv3_conv_plan_tile_count_sized(int64_t n, int tile_voxels);
+int ptv3_conv_plan_tiles_sized(const int32_t *row_ptr, const int32_t *slot_pair, int64_t n, int taps, int tile_voxels,
+                               int32_t *tile_tap, int32_t *tile_pair, int32_t *vox_taps, void *stream);
+int ptv3_subm_conv_tiles_fwd_sized(const void *feat, int dtype, int64_t n, int channels, int taps, int tile_voxels,
+                                   const void *packed_weight, const void *bias, const int32_t *tile_tap,
+                                   const int32_t *tile_pair, const int32_t *vox_taps, void *out, void *stream);
 
 /* model.py:546-552 (spconv.SubMConv3d, 3x3x3, in == out channels) where a voxel has few neighbours: the same
  * tiles and packed weight as ptv3_subm_conv_tiles_fwd, but the work is in proportion to the pairs (an MFMA row

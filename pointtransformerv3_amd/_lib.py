@@ -56,6 +56,9 @@ SIGNATURES = {
     "ptv3_conv_plan_tiles": (_i32, [_vp, _vp, _i64, _i32, _vp, _vp, _vp, _vp]),
     "ptv3_subm_conv_pack_weight": (_i32, [_vp, _i32, _i32, _i32, _vp, _vp]),
     "ptv3_subm_conv_tiles_fwd": (_i32, [_vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "ptv3_conv_plan_tile_count_sized": (_i64, [_i64, _i32]),
+    "ptv3_conv_plan_tiles_sized": (_i32, [_vp, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _vp]),
+    "ptv3_subm_conv_tiles_fwd_sized": (_i32, [_vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "ptv3_subm_conv_pack_weight_blocks": (_i64, [_i32, _i32]),
     "ptv3_subm_conv_pack_weight_batch": (_i32, [_vp, _i32, _i64, _vp]),
     "ptv3_subm_conv_sparse_fwd": (_i32, [_vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -121,10 +121,10 @@ __global__ __launch_bounds__(CT_THREADS) void plan_slots_kernel(const int32_t* _
     slot_pair[pair_slot[q]] = (int32_t)((uint32_t)lo << 24 | (uint32_t)pair_in[q]);
 }
 
-constexpr int CT_TV = 128;          // output voxels per tile
+constexpr int CT_TV = 128;          // output voxels per tile (the 128-channel tile form also takes tiles of 96)
 constexpr int CT_TILE_WORDS = 32;   // int32 per tile in tile_tap: 28 tap starts (relative), the tile's first pair
 
-// Per tile of CT_TV consecutive voxels: its pairs sorted by tap, inside a tap by output voxel.
+// Per tile of blockDim.x (96 or 128) consecutive voxels: its pairs sorted by tap, inside a tap by output voxel.
 // tile_tap[tile][t] = first pair of tap t relative to the tile's first pair (t = 27: the tile's pair
 // count), [28] = the tile's first pair; tile_pair[.] = voxel inside the tile << 24 | input row, in that
 // order; vox_taps[i] = bit t set when voxel i has a neighbour at tap t.
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(CT_TV) void plan_tiles_kernel(const int32_t* __rest
                                                            uint32_t* __restrict__ vox_taps) {
     __shared__ int32_t wave_cnt[2][32], tstart[32];
     const int tid = threadIdx.x, lane = tid % PTV3_WAVE, wave = tid / PTV3_WAVE;
-    const int64_t v0 = (int64_t)blockIdx.x * CT_TV;
+    const int64_t v0 = (int64_t)blockIdx.x * blockDim.x;
     const bool live = v0 + tid < n;
     int s_lo = 0, s_hi = 0;
     if (live) {
@@ -179,15 +179,18 @@ __global__ __launch_bounds__(CT_TV) void plan_tiles_kernel(const int32_t* __rest
     }
 }
 
-template <int C>
+// TV_ output voxels per tile: 128, or 96 where the four waves split the output channels (128 channels): a launch
+// whose 128-voxel tiles fill 2.2 rounds of the resident work-groups costs three, with 96-voxel tiles 2.97 rounds of
+// tiles that are a quarter cheaper
+template <int C, int TV_ = CT_TV>
 struct TileShape {
-    static constexpr int TV = CT_TV;
+    static constexpr int TV = TV_;
     static constexpr int THREADS = 256;
     static constexpr int COUT_WG = C > 128 ? 128 : C;     // output channels of a work-group
     static constexpr int CW = COUT_WG / 32;               // waves across channels
-    static constexpr int PW = 4 / CW;                     // waves across the four 32-voxel groups of the tile
-    static constexpr int GPW = 4 / PW;                    // groups per wave
-    static constexpr int CH = C >= 128 ? 128 : 64;        // pairs per chunk (128: a tap of a tile is one chunk)
+    static constexpr int PW = 4 / CW;                     // waves across the 32-voxel groups of the tile
+    static constexpr int GPW = TV / 32 / PW;              // groups per wave
+    static constexpr int CH = C >= 128 ? TV : 64;         // pairs per chunk (128 channels: a tap of a tile is one chunk)
     static constexpr int KS = C / 16;                     // MFMA steps along the input channels
     static constexpr int LPR = C / 8;                     // lanes (16 B each) per input row
     static constexpr int RPP = THREADS / LPR;             // rows per gather instruction of the work-group
@@ -198,7 +201,7 @@ struct TileShape {
     static constexpr int DEPTH = 2;                       // chunks in flight
     static constexpr size_t XBUF = (size_t)TV * C * 2;    // bytes of one buffer of input rows (swizzled, no padding)
     static constexpr size_t LDS = 2 * XBUF + (size_t)CAP * 4 + (size_t)C * 2;   // + one row of zeros
-    static_assert(CH % RPP == 0 && NL >= 1 && MAX_CHUNKS <= 128 && LPR >= 8, "tile shape");
+    static_assert(CH % RPP == 0 && NL >= 1 && MAX_CHUNKS <= 128 && LPR >= 8 && GPW * PW * 32 == TV, "tile shape");
 };
 
 // Input rows sit in LDS at the row of their OUTPUT voxel, 16-byte pieces swizzled by the row so that the
@@ -208,12 +211,12 @@ __device__ __forceinline__ int swz(int row, int piece) {
     return row * C + ((piece ^ (row & 7)) * 8);   // in halfs
 }
 
-template <typename T, int C>
-__global__ __launch_bounds__(TileShape<C>::THREADS, TileShape<C>::OCC) void conv_tile_kernel(
+template <typename T, int C, int TV_>
+__global__ __launch_bounds__((TileShape<C, TV_>::THREADS), (TileShape<C, TV_>::OCC)) void conv_tile_kernel(
     const T* __restrict__ feat, int64_t n, const T* __restrict__ packed_w, const T* __restrict__ bias,
     const int32_t* __restrict__ tile_tap, const uint32_t* __restrict__ tile_pair, const uint32_t* __restrict__ vox_taps,
     T* __restrict__ out) {
-    typedef TileShape<C> S;
+    typedef TileShape<C, TV_> S;
     typedef typename TileOps<T>::v8 v8;
     constexpr int TV = S::TV, CW = S::CW, GPW = S::GPW, CH = S::CH, KS = S::KS;
     constexpr int LPR = S::LPR, RPP = S::RPP, NL = S::NL, COUT_WG = S::COUT_WG, DEPTH = S::DEPTH;
@@ -369,26 +372,29 @@ __global__ __launch_bounds__(TileShape<C>::THREADS, TileShape<C>::OCC) void conv
     }
 }
 
-template <typename T, int C>
+template <typename T, int C, int TV_ = CT_TV>
 int launch_tiles(const void* feat, int64_t n, const void* packed_w, const void* bias, const int32_t* tile_tap,
                  const uint32_t* tile_pair, const uint32_t* vox_taps, void* out, hipStream_t stream) {
-    typedef TileShape<C> S;
-    auto kern = conv_tile_kernel<T, C>;
+    typedef TileShape<C, TV_> S;
+    auto kern = conv_tile_kernel<T, C, TV_>;
     static LdsGrant grant_attr_set;   // per instantiation and device
     if (const int rc_ = ptv3_allow_lds((const void*)kern, S::LDS, grant_attr_set)) return rc_;
-    const dim3 grid((unsigned)ptv3_ceil_div(n, CT_TV), (unsigned)(C / S::COUT_WG));
+    const dim3 grid((unsigned)ptv3_ceil_div(n, S::TV), (unsigned)(C / S::COUT_WG));
     hipLaunchKernelGGL(kern, grid, dim3(S::THREADS), S::LDS, stream, (const T*)feat, n, (const T*)packed_w,
                        (const T*)bias, tile_tap, tile_pair, vox_taps, (T*)out);
     PTV3_RETURN_LAUNCH();
 }
 
 template <typename T>
-int dispatch_tiles(const void* feat, int64_t n, int c, const void* packed_w, const void* bias, const int32_t* tile_tap,
-                   const uint32_t* tile_pair, const uint32_t* vox_taps, void* out, hipStream_t stream) {
-    switch (c) {
-        case 64: return launch_tiles<T, 64>(feat, n, packed_w, bias, tile_tap, tile_pair, vox_taps, out, stream);
-        case 128: return launch_tiles<T, 128>(feat, n, packed_w, bias, tile_tap, tile_pair, vox_taps, out, stream);
-    }
+int dispatch_tiles(const void* feat, int64_t n, int c, int tile_voxels, const void* packed_w, const void* bias,
+                   const int32_t* tile_tap, const uint32_t* tile_pair, const uint32_t* vox_taps, void* out,
+                   hipStream_t stream) {
+    if (c == 64 && tile_voxels == 128)
+        return launch_tiles<T, 64>(feat, n, packed_w, bias, tile_tap, tile_pair, vox_taps, out, stream);
+    if (c == 128 && tile_voxels == 128)
+        return launch_tiles<T, 128>(feat, n, packed_w, bias, tile_tap, tile_pair, vox_taps, out, stream);
+    if (c == 128 && tile_voxels == 96)
+        return launch_tiles<T, 128, 96>(feat, n, packed_w, bias, tile_tap, tile_pair, vox_taps, out, stream);
     return PTV3_ESHAPE;
 }
 
@@ -406,15 +412,25 @@ extern "C" int ptv3_conv_plan_slots(const int32_t* tap_ptr, int taps, const int3
 
 extern "C" int64_t ptv3_conv_plan_tile_count(int64_t n) { return n < 0 ? 0 : ptv3_ceil_div(n, CT_TV); }
 
-extern "C" int ptv3_conv_plan_tiles(const int32_t* row_ptr, const int32_t* slot_pair, int64_t n, int taps,
-                                    int32_t* tile_tap, int32_t* tile_pair, int32_t* vox_taps, void* stream_) {
+extern "C" int64_t ptv3_conv_plan_tile_count_sized(int64_t n, int tile_voxels) {
+    return (n < 0 || (tile_voxels != 96 && tile_voxels != 128)) ? 0 : ptv3_ceil_div(n, tile_voxels);
+}
+
+extern "C" int ptv3_conv_plan_tiles_sized(const int32_t* row_ptr, const int32_t* slot_pair, int64_t n, int taps,
+                                          int tile_voxels, int32_t* tile_tap, int32_t* tile_pair, int32_t* vox_taps,
+                                          void* stream_) {
     if (n < 0 || n >= (1ll << 24)) return PTV3_EINVAL;
-    if (taps != CT_TAPS) return PTV3_ESHAPE;
+    if (taps != CT_TAPS || (tile_voxels != 96 && tile_voxels != 128)) return PTV3_ESHAPE;
     if (n == 0) return PTV3_OK;
     if (!row_ptr || !slot_pair || !tile_tap || !tile_pair || !vox_taps) return PTV3_EINVAL;
-    hipLaunchKernelGGL(plan_tiles_kernel, dim3((unsigned)ptv3_ceil_div(n, CT_TV)), dim3(CT_TV), 0,
+    hipLaunchKernelGGL(plan_tiles_kernel, dim3((unsigned)ptv3_ceil_div(n, tile_voxels)), dim3(tile_voxels), 0,
                        (hipStream_t)stream_, row_ptr, slot_pair, n, tile_tap, (uint32_t*)tile_pair, (uint32_t*)vox_taps);
     PTV3_RETURN_LAUNCH();
+}
+
+extern "C" int ptv3_conv_plan_tiles(const int32_t* row_ptr, const int32_t* slot_pair, int64_t n, int taps,
+                                    int32_t* tile_tap, int32_t* tile_pair, int32_t* vox_taps, void* stream_) {
+    return ptv3_conv_plan_tiles_sized(row_ptr, slot_pair, n, taps, CT_TV, tile_tap, tile_pair, vox_taps, stream_);
 }
 
 extern "C" int ptv3_subm_conv_pack_weight(const void* weight, int dtype, int channels, int taps, void* packed,
@@ -447,15 +463,24 @@ extern "C" int ptv3_subm_conv_pack_weight_batch(const ptv3_pack_job* jobs, int n
 extern "C" int ptv3_subm_conv_tiles_fwd(const void* feat, int dtype, int64_t n, int channels, int taps,
                                         const void* packed_weight, const void* bias, const int32_t* tile_tap,
                                         const int32_t* tile_pair, const int32_t* vox_taps, void* out, void* stream_) {
+    return ptv3_subm_conv_tiles_fwd_sized(feat, dtype, n, channels, taps, CT_TV, packed_weight, bias, tile_tap, tile_pair,
+                                          vox_taps, out, stream_);
+}
+
+extern "C" int ptv3_subm_conv_tiles_fwd_sized(const void* feat, int dtype, int64_t n, int channels, int taps,
+                                              int tile_voxels, const void* packed_weight, const void* bias,
+                                              const int32_t* tile_tap, const int32_t* tile_pair, const int32_t* vox_taps,
+                                              void* out, void* stream_) {
     if (n < 0 || n >= (1ll << 24)) return PTV3_EINVAL;
     if (taps != CT_TAPS) return PTV3_ESHAPE;
     if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
     if (channels != 64 && channels != 128) return PTV3_ESHAPE;
+    if (tile_voxels != 128 && !(tile_voxels == 96 && channels == 128)) return PTV3_ESHAPE;
     if (n == 0) return PTV3_OK;
     if (!feat || !packed_weight || !tile_tap || !tile_pair || !vox_taps || !out) return PTV3_EINVAL;
     hipStream_t stream = (hipStream_t)stream_;
     const uint32_t *tp = (const uint32_t*)tile_pair, *vt = (const uint32_t*)vox_taps;
     if (dtype == PTV3_F16)
-        return dispatch_tiles<_Float16>(feat, n, channels, packed_weight, bias, tile_tap, tp, vt, out, stream);
-    return dispatch_tiles<__bf16>(feat, n, channels, packed_weight, bias, tile_tap, tp, vt, out, stream);
+        return dispatch_tiles<_Float16>(feat, n, channels, tile_voxels, packed_weight, bias, tile_tap, tp, vt, out, stream);
+    return dispatch_tiles<__bf16>(feat, n, channels, tile_voxels, packed_weight, bias, tile_tap, tp, vt, out, stream);
 }

@@ -570,19 +570,22 @@ class ConvPlan:
             self._slot_pair = sp
         return self._slot_pair
 
-    def tiles(self):
-        """(tile_tap, tile_pair): every tile's pairs sorted by tap for subm_conv_tiles, made on first use."""
+    def tiles(self, tile_voxels=128):
+        """(tile_tap, tile_pair, vox_taps): every tile's pairs sorted by tap for subm_conv_tiles and subm_conv_sparse,
+        made on first use, per tile size (128 outputs, or 96 for the 128-channel tile form)."""
         if getattr(self, "_tiles", None) is None:
+            self._tiles = {}
+        if tile_voxels not in self._tiles:
             lib = _lib.load()
             dev = self.pair_in.device
-            tile_tap = torch.empty((lib.ptv3_conv_plan_tile_count(self.n), 32), dtype=torch.int32, device=dev)
+            tile_tap = torch.empty((lib.ptv3_conv_plan_tile_count_sized(self.n, tile_voxels), 32), dtype=torch.int32, device=dev)
             tile_pair = torch.empty(max(self.n_pairs, 1), dtype=torch.int32, device=dev)
             vox_taps = torch.empty(max(self.n, 1), dtype=torch.int32, device=dev)
-            _lib.check(lib.ptv3_conv_plan_tiles(_ptr(self.row_ptr), _ptr(self.slot_pair()), self.n, self.taps,
-                                                _ptr(tile_tap), _ptr(tile_pair), _ptr(vox_taps), _stream()),
-                       "ptv3_conv_plan_tiles")
-            self._tiles = (tile_tap, tile_pair, vox_taps)
-        return self._tiles
+            _lib.check(lib.ptv3_conv_plan_tiles_sized(_ptr(self.row_ptr), _ptr(self.slot_pair()), self.n, self.taps,
+                                                      tile_voxels, _ptr(tile_tap), _ptr(tile_pair), _ptr(vox_taps),
+                                                      _stream()), "ptv3_conv_plan_tiles_sized")
+            self._tiles[tile_voxels] = (tile_tap, tile_pair, vox_taps)
+        return self._tiles[tile_voxels]
 
 
 def conv_plan(nbr, tap_major=False):
@@ -770,7 +773,21 @@ def conv_pack_weight(weight, taps, dtype):
     return packed
 
 
-def subm_conv_tiles(feat, plan, packed_weight, bias=None):
+TILE_CONV_RESIDENT = 512   # work-groups of the tile form the part holds at a time (two per CU)
+
+
+def tile_voxels_for(n, channels):
+    """Outputs per tile for the tile form: a launch runs in rounds of TILE_CONV_RESIDENT work-groups and costs whole
+    rounds; a tile's cost is about a quarter fixed (its 27 weight matrices) and the rest in proportion to its
+    outputs. 128 unless tiles of 96 (128 channels only) make the cheaper set of rounds: 146,195 voxels are 2.2
+    rounds of 128-voxel tiles (three rounds paid) or 2.97 rounds of 96-voxel ones."""
+    if channels != 128:
+        return 128
+    cost = {tv: -(-(-(-n // tv)) // TILE_CONV_RESIDENT) * (32 + tv) for tv in (128, 96)}
+    return 96 if cost[96] < cost[128] else 128
+
+
+def subm_conv_tiles(feat, plan, packed_weight, bias=None, tile_voxels=None):
     """3x3x3 submanifold convolution with cin == cout, sums kept on chip per tile of outputs (fp16 / bf16)."""
     _dev(feat, packed_weight, bias)
     lib = _lib.load()
@@ -779,12 +796,14 @@ def subm_conv_tiles(feat, plan, packed_weight, bias=None):
     assert packed_weight.dtype == feat.dtype and packed_weight.numel() == plan.taps * c * c
     b = None if bias is None else bias.to(feat.dtype).contiguous()
     out = torch.empty((n, c), dtype=feat.dtype, device=feat.device)
-    tile_tap, tile_pair, vox_taps = plan.tiles()
+    tv = tile_voxels_for(n, c) if tile_voxels is None else tile_voxels
+    tile_tap, tile_pair, vox_taps = plan.tiles(tv)
 
     def call():
-        _lib.check(lib.ptv3_subm_conv_tiles_fwd(_ptr(feat), _dtype_code(feat), n, c, plan.taps, _ptr(packed_weight),
-                                                _ptr(b), _ptr(tile_tap), _ptr(tile_pair), _ptr(vox_taps), _ptr(out),
-                                                _stream()), "ptv3_subm_conv_tiles_fwd")
+        _lib.check(lib.ptv3_subm_conv_tiles_fwd_sized(_ptr(feat), _dtype_code(feat), n, c, plan.taps, tv,
+                                                      _ptr(packed_weight), _ptr(b), _ptr(tile_tap), _ptr(tile_pair),
+                                                      _ptr(vox_taps), _ptr(out), _stream()),
+                   "ptv3_subm_conv_tiles_fwd_sized")
 
     if _LAUNCH_TIMER is not None:
         _LAUNCH_TIMER.launch("subm_conv", (plan.n_pairs, n, c, c, plan.taps, "tile"), call)

@@ -639,6 +639,25 @@ def test_subm_conv_tiles_parity(dtype, c, n, extent):
     assert torch.equal(got, again)
     nob = o.subm_conv_tiles(feat.to(DEV), plan, packed, None)
     assert rel_err(nob, OF.subm_conv(feat.float(), nbr, w.float(), None)) < TOL[dtype]
+    if c == 128:
+        # tiles of 96 outputs instead of 128: a voxel's sum is taken in tap order either way, so the same bits
+        for tv in (96, 128):
+            assert torch.equal(o.subm_conv_tiles(feat.to(DEV), plan, packed, b.to(DEV), tile_voxels=tv), got)
+        t96, t128 = plan.tiles(96), plan.tiles(128)
+        assert t96[0].shape[0] == -(-len(idx) // 96) and t128[0].shape[0] == -(-len(idx) // 128)
+        assert int(t96[0][:, 27].sum()) == plan.n_pairs == int(t128[0][:, 27].sum())   # every pair in one tile
+        assert torch.equal(t96[2], t128[2])                                              # per-voxel tap sets
+    else:
+        with pytest.raises(Exception):
+            o.subm_conv_tiles(feat.to(DEV), plan, packed, b.to(DEV), tile_voxels=96)     # 96 is for 128 channels
+
+
+def test_tile_size_choice_follows_the_rounds():
+    o = ops()
+    assert o.tile_voxels_for(146_195, 128) == 96      # 2.2 rounds of 128-voxel tiles, 2.97 of 96-voxel ones
+    assert o.tile_voxels_for(60_000, 128) == 128      # one round either way
+    assert o.tile_voxels_for(10_000_000, 128) == 128  # many rounds: the larger tile amortises its weights better
+    assert o.tile_voxels_for(146_195, 64) == 128
 
 
 def test_repack_conv_weights_batch_equals_single_packs():
