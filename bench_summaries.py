@@ -184,8 +184,14 @@ def forward_trace(d, out_dir):
     trace = list(csv.DictReader(open(trace_path)))
     trace.sort(key=lambda r: int(r["Start_Timestamp"]))
     marks = [i for i, r in enumerate(trace) if "offset2batch" in r["Kernel_Name"]]
-    first, per = marks[-steps], len(trace[marks[-2]:marks[-1]])
-    window = trace[first:marks[-1] + per]
+    per = len(trace[marks[-2]:marks[-1]])
+    overlapped = pbench["config"].get("plain_schedule_ms_per_step") is not None
+    if overlapped:
+        # the timed forwards are followed by 2 + steps forwards on the plain schedule; with the index prologue of a
+        # forward running beside the forward before, `steps` marks apart is still `steps` forwards' worth of kernels
+        window = trace[marks[-(2 * steps + 2)]:marks[-(steps + 2)]]
+    else:
+        window = trace[marks[-steps]:marks[-1] + per]
     agg = collections.OrderedDict()
     for r in window:
         dur = int(r["End_Timestamp"]) - int(r["Start_Timestamp"])
@@ -203,7 +209,9 @@ def forward_trace(d, out_dir):
         "command (run from the repository root on the GPU box):",
         "  rocprofv3 --kernel-trace --stats --output-format csv -d DIR/prof_csv -o fwd -- python3 bench.py --no-cpu --no-other-configs --steps %d --warmup %d"
         % (steps, pbench["warmup"]),
-        "source: the kernel trace of that run, the %d timed forwards (a forward = from one offset2batch kernel to the next); times in microseconds\n" % steps,
+        "source: the kernel trace of that run, the %d timed forwards (a forward = from one offset2batch kernel to the next%s); times in microseconds\n"
+        % (steps, "; the index prologue of a forward runs on its own stream beside the forward before, so the window is cut "
+                  "at the prologues and holds every kernel of a forward once" if overlapped else ""),
         "bench.py line of the same run: ms_per_step=%.2f  points/s=%.0f" % (pbench["ms_per_step"], pbench["value"]),
         "  roofline (HIP events inside bench.py): kernel=%s launches=%d avg_launch_us=%.1f flops_per_launch=%.3e achieved=%.1f TFLOP/s frac=%.4f"
         % (rf["kernel"], rf["launches"], rf["avg_launch_us"], rf["flops_per_launch"], rf["achieved"], rf["frac"]),
@@ -218,6 +226,15 @@ def forward_trace(d, out_dir):
                % (tot / steps / 1e3, sum(v[0] for _, v in rows) / steps, span))
     out.append("\nper forward, by group:")
     out += _grouped([(n, v[1], v[0]) for n, v in rows], FORWARD_GROUPS, steps)
+    if overlapped:
+        plain = trace[marks[-steps]:marks[-1] + per]
+        ptot = sum(int(r["End_Timestamp"]) - int(r["Start_Timestamp"]) for r in plain)
+        pspan = (int(plain[-1]["End_Timestamp"]) - int(plain[0]["Start_Timestamp"])) / steps / 1e3
+        out.append("\nthe plain schedule (every forward's index work in front of its own feature kernels), the %d forwards bench.py "
+                   "runs after the timed region: %.1f us of kernels per forward, %.1f us from forward to forward under the profiler; "
+                   "bench.py's own clock: %.2f ms per forward with the profiler, %.2f ms without"
+                   % (steps, ptot / steps / 1e3, pspan, pbench["config"]["plain_schedule_ms_per_step"],
+                      bench["config"]["plain_schedule_ms_per_step"] or float("nan")))
     open(os.path.join(out_dir, "forward_4x100k_fp16_kernel_trace.txt"), "w").write("\n".join(out) + "\n")
     return "forward trace: %.1f us of kernels per forward, ms_per_step %.2f" % (tot / steps / 1e3, bench["ms_per_step"])
 

@@ -50,6 +50,12 @@ class PointTransformerV3(PointModule):
         self.num_stages = len(enc_depths)
         self.order = [order] if isinstance(order, str) else order
         self.cls_mode = cls_mode
+        # Opt-in: the index work of level 0 (no feature is touched) runs on a stream of its own and does not wait
+        # for what the current stream holds, so in a loop of forwards it overlaps the tail of the forward before.
+        # Only for callers whose inputs are complete when forward() is called (nothing that produces them is still
+        # queued on the current stream); evaluation mode only.
+        self.overlap_index_prologue = False
+        self._prologue_state = None
         self.shuffle_orders = shuffle_orders
         n = self.num_stages
         assert n == len(stride) + 1 == len(enc_channels) == len(enc_num_head) == len(enc_patch_size)
@@ -123,6 +129,18 @@ class PointTransformerV3(PointModule):
         # under no_grad) leaves no trace on them: the derived copies (half-precision casts of float masters,
         # the tile convolutions' packed weights) are redone once per forward, in evaluation as well
         ops.invalidate_casts()
+        point = self._index_prologue(data_dict)
+        point = self.embedding(point)
+        point = self.enc(point)
+        if not self.cls_mode:
+            point = self.dec(point)
+        if self._prologue_state is not None:
+            self._prologue_state.forward_queued()
+        return point
+
+    def _level0_index(self, data_dict):
+        """Everything of level 0 that follows from the coordinates alone (model.py:966-970): the Point, its curve
+        codes and orders, the stem's pair lists, the clusters of the first pooling."""
         point = Point(data_dict)
         # the pair lists of the stem and of the first stage's xCPE depend on the coordinates only:
         # their first halves are queued behind the first host read-back and run while the host waits
@@ -131,8 +149,29 @@ class PointTransformerV3(PointModule):
         if self.stride:
             point.pool_ahead(self.stride[0])   # the first pooling's clusters need the codes only
         point.sparsify()
-        point = self.embedding(point)
-        point = self.enc(point)
-        if not self.cls_mode:
-            point = self.dec(point)
+        if self.overlap_index_prologue and not self.training and point.feat.dtype != torch.float32:
+            # with the prologue on a stream of its own, whatever else of level 0 follows from the coordinates goes
+            # there too: the pair and tile lists of the level's convolutions, the attention's padding and slot tables
+            from .sparse import SubMConv3d
+            stage0 = next(iter(self.enc._modules.values()))
+            dec0 = self.dec._modules.get("dec0") if not self.cls_mode else None
+            for m in list(self.embedding.modules()) + list(stage0.modules()):
+                if isinstance(m, SubMConv3d):
+                    m.lists_ahead(point.sparse_conv_feat)
+            blocks = [b for st in (stage0, dec0) if st is not None for b in st._modules.values() if isinstance(b, Block)]
+            if blocks and all(b.attn.enable_flash and b.attn.patch_size == blocks[0].attn.patch_size for b in blocks):
+                for b in blocks:
+                    b.attn._slots(point)
+        return point
+
+    def _index_prologue(self, data_dict):
+        feat = data_dict.get("feat")
+        if (not self.overlap_index_prologue or self.training or torch.is_grad_enabled() or feat is None
+                or not feat.is_cuda or ops.Readback.blocking):
+            self._prologue_state = None
+            return self._level0_index(data_dict)
+        if self._prologue_state is None or self._prologue_state.device != feat.device:
+            self._prologue_state = ops.PrologueOverlap(feat.device)
+        with self._prologue_state.scope():
+            point = self._level0_index(data_dict)
         return point

@@ -3,6 +3,7 @@
 torch is used for device memory and the current stream only; every computation happens in
 the HIP kernels. All tensors must live on the GPU; CPU tensors are rejected.
 """
+import contextlib
 import ctypes
 import weakref
 
@@ -639,6 +640,46 @@ def side_stream(dev, index=0):
 
 def _side_stream(dev):
     return side_stream(dev, 0)
+
+
+class PrologueOverlap:
+    """A stream and two private memory pools for index work that depends on a forward's inputs alone and may
+    therefore run while the forward before it is still computing (PointTransformerV3.overlap_index_prologue).
+
+    scope() runs its body on the prologue stream, which waits for nothing, with every allocation of the body routed
+    to one of the two pools in turn; on leaving it the current stream is made to wait for the body's work.
+    What the body allocates is used by the current stream afterwards without any per-tensor bookkeeping: a pool's
+    memory is handed out again only two forwards later, and forward_queued() (called when the whole forward has been
+    queued) leaves an event on the current stream that the pool's next turn waits for on the host first."""
+
+    def __init__(self, device):
+        self.device = device
+        self.stream = torch.cuda.Stream(device=device)
+        self.pools = [torch.cuda.MemPool(), torch.cuda.MemPool()]
+        self.done = [None, None]   # per pool: the forward that last used it has run to its end on its stream
+        self.turn = 0
+
+    @contextlib.contextmanager
+    def scope(self):
+        self.turn ^= 1
+        if self.done[self.turn] is not None:
+            self.done[self.turn].synchronize()   # two forwards back: over long ago
+        global AHEAD_ON_SIDE_STREAM
+        main = torch.cuda.current_stream(self.device)
+        ahead, AHEAD_ON_SIDE_STREAM = AHEAD_ON_SIDE_STREAM, False   # the shared side stream still holds the last forward's work
+        try:
+            with torch.cuda.stream(self.stream), torch.cuda.use_mem_pool(self.pools[self.turn], self.device):
+                yield
+                ready = torch.cuda.Event()
+                ready.record(self.stream)
+        finally:
+            AHEAD_ON_SIDE_STREAM = ahead
+        main.wait_event(ready)
+
+    def forward_queued(self):
+        ev = torch.cuda.Event()
+        ev.record(torch.cuda.current_stream(self.device))
+        self.done[self.turn] = ev
 
 
 def conv_plan_direct_start(indices, ks):

@@ -116,6 +116,28 @@ class SubMConv3d(nn.Module):
             held = self._packed[dtype]
         return held[1]
 
+    def _tile_form(self, plan, cin, cout):
+        """Which of the two forms that walk the plan's tile lists takes this convolution in half precision:
+        "sparse", "tile" or None (pair or dense form)."""
+        if self.kernel_size != 3 or cin != cout or plan.n >= (1 << 24):
+            return None
+        if cin in ops.CONV_SPARSE_CHANNELS and plan.n_pairs <= self.SPARSE_MODE_MAX_PAIRS_PER_VOXEL * plan.n:
+            return "sparse"
+        if cin in ops.CONV_TILE_CHANNELS and plan.n_pairs >= self.TILE_MODE_MIN_PAIRS_PER_VOXEL * plan.n:
+            return "tile"
+        return None
+
+    def lists_ahead(self, x):
+        """Makes (and caches on x, under this module's indice_key) the index lists the half-precision forward of this
+        module will ask for: the pair lists, and the tile lists where a tile form takes the layer. They follow from
+        the coordinates alone."""
+        plan = x.conv_plan(self.kernel_size, self.indice_key)
+        form = self._tile_form(plan, self.in_channels, self.out_channels)
+        if form == "sparse":
+            plan.tiles(128)
+        elif form == "tile":
+            plan.tiles(ops.tile_voxels_for(plan.n, self.in_channels))
+
     def convolve(self, x, feat, weight, bias, packed=None):
         """The convolution of feat (N, Cin) over x's neighbourhoods with weight (Cout, V, Cin), on whichever
         form fits: dense output-stationary (fp32, or many active taps), pair lists, tiles, or sparse tiles.
@@ -130,14 +152,10 @@ class SubMConv3d(nn.Module):
             feat = nn.functional.pad(feat, (0, pad))
             weight = nn.functional.pad(weight, (0, pad))
         plan = x.conv_plan(self.kernel_size, self.indice_key)
-        if (self.kernel_size == 3 and cin == cout and cin in ops.CONV_SPARSE_CHANNELS and plan.n < (1 << 24)
-                and plan.n_pairs <= self.SPARSE_MODE_MAX_PAIRS_PER_VOXEL * plan.n):
+        form = self._tile_form(plan, cin, cout)
+        if form is not None:
             tiles = packed() if packed is not None else ops.conv_pack_weight(weight, 27, feat.dtype)
-            return ops.subm_conv_sparse(feat, plan, tiles, bias)
-        if (self.kernel_size == 3 and cin == cout and cin in ops.CONV_TILE_CHANNELS
-                and plan.n < (1 << 24) and plan.n_pairs >= self.TILE_MODE_MIN_PAIRS_PER_VOXEL * plan.n):
-            tiles = packed() if packed is not None else ops.conv_pack_weight(weight, 27, feat.dtype)
-            return ops.subm_conv_tiles(feat, plan, tiles, bias)
+            return (ops.subm_conv_sparse if form == "sparse" else ops.subm_conv_tiles)(feat, plan, tiles, bias)
         weight = weight.to(feat.dtype)
         if plan.density() <= self.PAIR_MODE_MAX_DENSITY and cout % 8 == 0:
             return ops.subm_conv_pairs(feat, plan, weight, bias)

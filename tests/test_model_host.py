@@ -103,6 +103,18 @@ def test_forward_on_cpu_tensors_fails_loudly():
         m(data)
 
 
+def test_overlapped_prologue_is_opt_in_and_takes_no_cpu_tensors():
+    from pointtransformerv3_amd import PointTransformerV3
+    from pointtransformerv3_amd._lib import Ptv3Error
+    m = PointTransformerV3(enc_depths=(1, 1, 1, 1, 1), dec_depths=(1, 1, 1, 1)).eval()
+    assert m.overlap_index_prologue is False
+    m.overlap_index_prologue = True
+    data = dict(feat=torch.zeros(10, 6), grid_coord=torch.arange(30).reshape(10, 3).int(), offset=torch.tensor([10]))
+    with torch.inference_mode(), pytest.raises(Ptv3Error):
+        m(data)                       # the plain schedule, and its loud failure, for tensors that are not on the GPU
+    assert m._prologue_state is None
+
+
 def test_cast_of_cpu_parameters_is_computed_not_remembered():
     """Off the GPU a parameter is converted on every call (there is nothing to launch for it): the layouts are
     the ones the GPU kernel writes."""
