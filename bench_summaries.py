@@ -184,14 +184,14 @@ def forward_trace(d, out_dir):
     trace = list(csv.DictReader(open(trace_path)))
     trace.sort(key=lambda r: int(r["Start_Timestamp"]))
     marks = [i for i, r in enumerate(trace) if "offset2batch" in r["Kernel_Name"]]
-    per = len(trace[marks[-2]:marks[-1]])
     overlapped = pbench["config"].get("plain_schedule_ms_per_step") is not None
-    if overlapped:
-        # the timed forwards are followed by 2 + steps forwards on the plain schedule; with the index prologue of a
-        # forward running beside the forward before, `steps` marks apart is still `steps` forwards' worth of kernels
-        window = trace[marks[-(2 * steps + 2)]:marks[-(steps + 2)]]
-    else:
-        window = trace[marks[-steps]:marks[-1] + per]
+    # bench.py's loops, in order: warm-up, the `steps` timed forwards, then (when the timed ones overlapped their index
+    # prologues) 2 + steps forwards on the plain schedule, then 2 + steps with events around every launch. With a
+    # prologue running beside the forward before it, `steps` marks apart is still `steps` forwards' worth of kernels.
+    tail = steps + 2
+    plain = trace[marks[-2 * tail + 2]:marks[-tail]] if overlapped else None
+    t_first = -(2 * tail + steps) if overlapped else -(tail + steps)
+    window = trace[marks[t_first]:marks[t_first + steps]]
     agg = collections.OrderedDict()
     for r in window:
         dur = int(r["End_Timestamp"]) - int(r["Start_Timestamp"])
@@ -227,11 +227,10 @@ def forward_trace(d, out_dir):
     out.append("\nper forward, by group:")
     out += _grouped([(n, v[1], v[0]) for n, v in rows], FORWARD_GROUPS, steps)
     if overlapped:
-        plain = trace[marks[-steps]:marks[-1] + per]
         ptot = sum(int(r["End_Timestamp"]) - int(r["Start_Timestamp"]) for r in plain)
         pspan = (int(plain[-1]["End_Timestamp"]) - int(plain[0]["Start_Timestamp"])) / steps / 1e3
         out.append("\nthe plain schedule (every forward's index work in front of its own feature kernels), the %d forwards bench.py "
-                   "runs after the timed region: %.1f us of kernels per forward, %.1f us from forward to forward under the profiler; "
+                   "times after the timed region: %.1f us of kernels per forward, %.1f us from forward to forward under the profiler; "
                    "bench.py's own clock: %.2f ms per forward with the profiler, %.2f ms without"
                    % (steps, ptot / steps / 1e3, pspan, pbench["config"]["plain_schedule_ms_per_step"],
                       bench["config"]["plain_schedule_ms_per_step"] or float("nan")))
