@@ -549,8 +549,8 @@ int ptv3_mlp_pack_weights(const void *w1, const void *w2, int dtype, int channel
  * n_blocks their sum. Both half types move as 16-bit patterns, so a table may mix them. The table is trusted like
  * ptv3_pack_job's: channels 128, 256 or 512 (other rows are skipped), buffers of the stated sizes. */
 typedef struct {
-    const void *w1, *w2;  /* (4 * channels, channels) and (channels, 4 * channels) */
-    void *packed;         /* 8 * channels^2 elements */
+    const void *w1, *w2;  /* (4 * channels, channels) and (channels, 4 * channels); w2 NULL: w1 is one */
+    void *packed;         /* (channels, channels) matrix. 8 * channels^2 elements (channels^2 without w2) */
     int32_t channels, reserved;
     int64_t first_block;
 } ptv3_mlp_pack_job;
@@ -558,6 +558,20 @@ int64_t ptv3_mlp_pack_weights_blocks(int channels);
 int ptv3_mlp_pack_weights_batch(const ptv3_mlp_pack_job *jobs, int n_jobs, int64_t n_blocks, void *stream);
 int ptv3_mlp_fused_packed(const void *x, const void *resid, const void *packed, const void *b1, const void *b2,
                           int dtype, int64_t n, int channels, void *out, void *stream);
+
+/* Second half of a block at 128 or 256 channels in one kernel, model.py:458-460 (proj), :595-602:
+ *   sum = shortcut + (attn @ w_proj^T + b_proj)
+ *   out = sum + fc2(GELU(fc1(LayerNorm_2(sum))))
+ * attn, shortcut, out: (n, channels) of dtype (PTV3_F16 / PTV3_BF16); biases and LayerNorm parameters (channels) or
+ * (4 * channels) of dtype. mlp_packed as for ptv3_mlp_fused_packed; proj_packed holds channels^2 elements, the
+ * (channels, channels) weight in the same order: written by ptv3_mlp_pack_weights_batch from a job whose w2 is NULL
+ * (w1 = the weight, packed = proj_packed), which owns ptv3_linear_pack_weights_blocks(channels) blocks of the launch.
+ * The projection, the sum and the normalised rows are rounded to dtype where the separate layers would store them
+ * and never leave the CU. PTV3_ESHAPE for other widths or dtypes. */
+int64_t ptv3_linear_pack_weights_blocks(int channels);
+int ptv3_block_tail_wide(const void *attn, const void *shortcut, const void *proj_packed, const void *proj_bias,
+                         const void *ln_weight, const void *ln_bias, float ln_eps, const void *mlp_packed,
+                         const void *b1, const void *b2, int dtype, int64_t n, int channels, void *out, void *stream);
 
 /* Head of a block for thin channels, model.py:541-545, :587-589, :592-593 and :450 in one kernel:
  *   feat = shortcut + LayerNorm_cpe(conv @ w_cpe^T + b_cpe)

@@ -56,7 +56,8 @@ __global__ __launch_bounds__(256) void mlp_pack_batch_kernel(const ptv3_mlp_pack
     const int c = job.channels;
     if (c != 128 && c != 256 && c != 512) return;   // a width the fused kernel does not take: touch nothing
     const int64_t idx = ((int64_t)blockIdx.x - job.first_block) * 256 + threadIdx.x;
-    if (idx < 0 || idx >= (int64_t)c * c) return;
+    // a job without w2 is one C x C matrix (C -> C Linear): the first KU steps of the same layout
+    if (idx < 0 || idx >= (job.w2 ? (int64_t)c * c : (int64_t)c * c / 8)) return;
     const int lane = (int)(idx % 64), jj = (int)(idx / 64 % 2), ub = (int)(idx / 128 % (c / 32));
     const int u = (int)(idx / 128 / (c / 32)), ku = c / 32;
     const int chunk = u / (2 * ku), st = (u / ku) & 1, kk = u % ku;
@@ -67,18 +68,29 @@ __global__ __launch_bounds__(256) void mlp_pack_batch_kernel(const ptv3_mlp_pack
 }
 
 // PACKED: w1 is the packed stream of both matrices and w2 is not read.
+// TAIL (PACKED only): the whole second half of a block. x is the attention's output, resid the block's running sum; a
+// pass first forms sum = resid + (x Wp^T + bp) and LayerNorm(sum) on the CU (wp: Wp packed like fc1's first chunk,
+// the stream then has KU steps more at its head), feeds the normalised rows to the MLP and adds the MLP to the sum,
+// which waits in a third LDS tile: neither the sum nor its normalised copy travels to memory and back.
 // A work-group walks its rows in passes of 1 .. RTMAX groups of 32 rows per wave; the host gives every resident
 // work-group the same number of row groups (with tiles of one fixed size the last round of a launch of 37,681 rows at
 // 256 channels ran at half occupancy).
-template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RTMAX, int THREADS, int MINW>
+struct TailArgs {   // what TAIL adds: the projection (packed), its bias, the LayerNorm's scale, shift and epsilon
+    const void *wp, *bp, *ln_w, *ln_b;
+    float eps;
+};
+
+template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RTMAX, int THREADS, int MINW, bool TAIL>
 __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
     const T* __restrict__ x, const T* __restrict__ resid, const T* __restrict__ w1, const T* __restrict__ b1,
-    const T* __restrict__ w2, const T* __restrict__ b2, int64_t n, int upw, T* __restrict__ out) {
+    const T* __restrict__ w2, const T* __restrict__ b2, int64_t n, int upw, T* __restrict__ out, TailArgs tail) {
+    static_assert(!TAIL || PACKED, "the block tail reads packed weights");
     typedef typename H16<T>::v8 v8;
     static_assert(WM * WN * PTV3_WAVE == THREADS && C == 32 * MT * WN, "the waves cover R x C");
     constexpr int RMAX = 32 * RTMAX * WM, H = 4 * C, XS = C + MW_PAD;
     constexpr int KU = C / 32;            // 32-wide contraction steps per stage
-    constexpr int UNITS = 4 * 2 * KU;     // weight steps per pass: 4 chunks x (fc1, fc2)
+    constexpr int HEAD = TAIL ? KU : 0;   // weight steps of the projection in front of the MLP's
+    constexpr int UNITS = HEAD + 4 * 2 * KU;   // weight steps per pass: (projection,) 4 chunks x (fc1, fc2)
     static_assert(KU % DEPTH == 0, "the ring is indexed statically");
     constexpr int PPR = C / 8;            // 16-byte pieces per row
     extern __shared__ __align__(16) unsigned char mw_smem[];
@@ -87,6 +99,13 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
     T* bias_lds = ht + RMAX * XS;         // [4 C] fc1's bias, [C] fc2's: read per chunk without touching the vector-memory queue
     for (int i = threadIdx.x; i < 5 * C / 8; i += THREADS)
         *(u32x4*)(bias_lds + i * 8) = *(const u32x4*)((i < 4 * C / 8 ? b1 : b2 - 4 * C) + i * 8);
+    T* sum_lds = bias_lds + 8 * C;        // TAIL: [RMAX][XS] the block's running sum; before it the projection's bias
+    if (TAIL)                             // and the LayerNorm's scale and shift, [C] each
+        for (int i = threadIdx.x; i < 3 * C / 8; i += THREADS) {
+            const int which = i / (C / 8), at = i % (C / 8);
+            const T* src = (const T*)(which == 0 ? tail.bp : which == 1 ? tail.ln_w : tail.ln_b);
+            *(u32x4*)(bias_lds + 5 * C + i * 8) = *(const u32x4*)(src + at * 8);
+        }
 
     const int tid = threadIdx.x, wave = tid / PTV3_WAVE, lane = tid % PTV3_WAVE;
     const int col = lane & 31, hf = lane >> 5;
@@ -96,11 +115,12 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
     // weight step q of a pass: chunk q / (2 KU), layer (q / KU) & 1 (fc1, fc2), 32-wide step kk = q % KU; lane (col, hf)
     // of output tile a takes 2 x 8 consecutive inputs of weight row ch0 + 32 a + col
     auto issue = [&](int q, u32x4 (&r)[MT][2]) {
-        const int chunk = q / (2 * KU), st = (q / KU) & 1, kk = q % KU, u = q;
+        const int u = TAIL && q < HEAD ? q : q - HEAD;   // step inside its own packed copy
+        const int chunk = u / (2 * KU), st = (u / KU) & 1, kk = u % KU;
 #pragma unroll
         for (int a = 0; a < MT; ++a) {
             if (PACKED) {
-                const T* p = w1 + ((u * (C / 32) + wn * MT + a) * 2) * 512 + lane * 8;
+                const T* p = (TAIL && q < HEAD ? (const T*)tail.wp : w1) + ((u * (C / 32) + wn * MT + a) * 2) * 512 + lane * 8;
                 r[a][0] = *(const u32x4*)p;
                 r[a][1] = *(const u32x4*)(p + 512);
                 continue;
@@ -171,13 +191,83 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
         for (int i = 0; i < PIECES; ++i) {
             const int p = tid + i * THREADS;
             const int rr = p / PPR, pc = p % PPR;
-            u32x4 v = {0, 0, 0, 0};
-            if (row0 + rr < row_end) v = *(const u32x4*)(x + (row0 + rr) * C + pc * 8);
+            u32x4 v = {0, 0, 0, 0}, sh = {0, 0, 0, 0};
+            if (row0 + rr < row_end) {
+                v = *(const u32x4*)(x + (row0 + rr) * C + pc * 8);
+                if (TAIL) sh = *(const u32x4*)(resid + (row0 + rr) * C + pc * 8);   // waits in LDS for the projection
+            }
             *(u32x4*)(xt + rr * XS + pc * 8) = v;
+            if (TAIL) *(u32x4*)(sum_lds + rr * XS + pc * 8) = sh;
         }
         __syncthreads();
 
         f32x16 acc[MT][RT_], hacc[MT][RT_];
+        if constexpr (TAIL) {
+            // ---- projection of the attention rows (+ bias, from the C operand), rounded, parked in ht
+#pragma unroll
+            for (int a = 0; a < MT; ++a)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const u32x2 bb = *(const u32x2*)(bias_lds + 5 * C + ch0 + a * 32 + 8 * g + 4 * hf);
+                    const float bias[4] = {H16<T>::lo(bb[0]), H16<T>::hi(bb[0]), H16<T>::lo(bb[1]), H16<T>::hi(bb[1])};
+#pragma unroll
+                    for (int rt = 0; rt < RT_; ++rt)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) hacc[a][rt][4 * g + q] = bias[q];
+                }
+            stage(xt, hacc, 0);
+#pragma unroll
+            for (int a = 0; a < MT; ++a)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int cc = ch0 + a * 32 + 8 * g + 4 * hf;
+#pragma unroll
+                    for (int rt = 0; rt < RT_; ++rt)
+                        *(u32x2*)(ht + (r0 + rt * 32 + col) * XS + cc) =
+                            (u32x2){H16<T>::pack2(hacc[a][rt][4 * g], hacc[a][rt][4 * g + 1]),
+                                    H16<T>::pack2(hacc[a][rt][4 * g + 2], hacc[a][rt][4 * g + 3])};
+                }
+            __syncthreads();   // every wave is done reading the attention rows in xt, the projection is in ht
+            // ---- sum = resid + projection (rounded, kept in sum_lds); its LayerNorm (rounded) replaces the x tile.
+            // A row's PPR pieces sit in neighbouring lanes of one wave: the statistics are lane exchanges
+            const int pc = tid % PPR;
+            const u32x4 gq = *(const u32x4*)(bias_lds + 6 * C + pc * 8), bq = *(const u32x4*)(bias_lds + 7 * C + pc * 8);
+#pragma unroll
+            for (int i = 0; i < PIECES; ++i) {
+                const int rr = (tid + i * THREADS) / PPR;
+                const u32x4 o = *(const u32x4*)(ht + rr * XS + pc * 8);
+                const u32x4 sh = *(const u32x4*)(sum_lds + rr * XS + pc * 8);   // written by this thread
+                u32x4 sm;
+                float v[8], tot = 0.f;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    sm[k] = H16<T>::pack2(H16<T>::lo(o[k]) + H16<T>::lo(sh[k]), H16<T>::hi(o[k]) + H16<T>::hi(sh[k]));
+                    v[2 * k] = H16<T>::lo(sm[k]);
+                    v[2 * k + 1] = H16<T>::hi(sm[k]);
+                    tot += v[2 * k] + v[2 * k + 1];
+                }
+                *(u32x4*)(sum_lds + rr * XS + pc * 8) = sm;
+#pragma unroll
+                for (int off = 1; off < PPR; off <<= 1) tot += __shfl_xor(tot, off, PTV3_WAVE);
+                const float mean = tot * (1.f / C);
+                float sq = 0.f;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    v[k] -= mean;
+                    sq += v[k] * v[k];
+                }
+#pragma unroll
+                for (int off = 1; off < PPR; off <<= 1) sq += __shfl_xor(sq, off, PTV3_WAVE);
+                const float rstd = rsqrtf(sq * (1.f / C) + tail.eps);
+                u32x4 nm;
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    nm[k] = H16<T>::pack2(v[2 * k] * rstd * H16<T>::lo(gq[k]) + H16<T>::lo(bq[k]),
+                                          v[2 * k + 1] * rstd * H16<T>::hi(gq[k]) + H16<T>::hi(bq[k]));
+                *(u32x4*)(xt + rr * XS + pc * 8) = nm;
+            }
+            __syncthreads();
+        }
 #pragma unroll
         for (int a = 0; a < MT; ++a)
 #pragma unroll
@@ -188,7 +278,7 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
 #pragma unroll 1   // unrolled, the chunks' loads are hoisted over each other and spill
         for (int c = 0; c < 4; ++c) {
             bias_into(hacc, c);
-            stage(xt, hacc, 2 * c * KU);
+            stage(xt, hacc, HEAD + 2 * c * KU);
             // hacc[a][rt][v]: hidden unit ch0 + 32 a + 8 (v / 4) + 4 hf + v % 4 of row r0 + 32 rt + col
 #pragma unroll
             for (int a = 0; a < MT; ++a)
@@ -202,7 +292,7 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
                                     gelu_round_pack2<T>(hacc[a][rt][4 * g + 2], hacc[a][rt][4 * g + 3])};
                 }
             __syncthreads();
-            stage(ht, acc, (2 * c + 1) * KU);
+            stage(ht, acc, HEAD + (2 * c + 1) * KU);
             __syncthreads();
         }
 
@@ -227,7 +317,8 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
             const int rr = p / PPR, pc = p % PPR;
             if (row0 + rr < row_end) {
                 const u32x4 o = *(const u32x4*)(ht + rr * XS + pc * 8);
-                const u32x4 s = *(const u32x4*)(resid + (row0 + rr) * C + pc * 8);
+                const u32x4 s = TAIL ? *(const u32x4*)(sum_lds + rr * XS + pc * 8)
+                                     : *(const u32x4*)(resid + (row0 + rr) * C + pc * 8);
                 u32x4 r;
 #pragma unroll
                 for (int k = 0; k < 4; ++k)
@@ -257,12 +348,14 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
     }
 }
 
-template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RTMAX, int THREADS = MW_THREADS, int MINW = 2>
+template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RTMAX, bool TAIL = false,
+          int THREADS = MW_THREADS, int MINW = 2>
 int launch_mlp_wide(const void* x, const void* resid, const void* w1, const void* b1, const void* w2, const void* b2,
-                    int64_t n, void* out, hipStream_t stream) {
+                    int64_t n, void* out, hipStream_t stream, TailArgs tail = TailArgs{}) {
     constexpr int RMAX = 32 * RTMAX * WM, UNIT = 32 * WM;
-    const size_t lds = ((size_t)2 * RMAX * (C + MW_PAD) + 5 * C) * sizeof(T);
-    auto kern = mlp_wide_kernel<T, C, WM, WN, MT, DEPTH, PACKED, RTMAX, THREADS, MINW>;
+    const size_t lds = ((size_t)(TAIL ? 3 : 2) * RMAX * (C + MW_PAD) + (TAIL ? 8 : 5) * C) * sizeof(T);
+    static_assert(((size_t)(TAIL ? 3 : 2) * RMAX * (C + MW_PAD) + (TAIL ? 8 : 5) * C) * sizeof(T) <= 160 * 1024, "LDS of a CU");
+    auto kern = mlp_wide_kernel<T, C, WM, WN, MT, DEPTH, PACKED, RTMAX, THREADS, MINW, TAIL>;
     static LdsGrant grant_configured;   // per instantiation and device
     if (const int rc_ = ptv3_allow_lds((const void*)kern, lds, grant_configured)) return rc_;
     // as many work-groups as the machine holds at a time (MINW waves per SIMD, THREADS / 256 of them from one
@@ -273,7 +366,8 @@ int launch_mlp_wide(const void* x, const void* resid, const void* w1, const void
     const int64_t upw = (units + grid - 1) / grid;
     if (upw > 0x7fffffffLL) return PTV3_EINVAL;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), lds, stream,
-                       (const T*)x, (const T*)resid, (const T*)w1, (const T*)b1, (const T*)w2, (const T*)b2, n, (int)upw, (T*)out);
+                       (const T*)x, (const T*)resid, (const T*)w1, (const T*)b1, (const T*)w2, (const T*)b2, n, (int)upw, (T*)out,
+                       tail);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? PTV3_OK : (int)e;
 }
@@ -286,6 +380,21 @@ int mlp_wide_any(const void* x, const void* resid, const void* w1, const void* b
         if (channels == 128) return launch_mlp_wide<T, 128, 2, 4, 1, 4, PACKED, 3>(x, resid, w1, b1, w2, b2, n, out, stream); \
         if (channels == 256) return launch_mlp_wide<T, 256, 1, 8, 1, 4, PACKED, 3>(x, resid, w1, b1, w2, b2, n, out, stream); \
         if (channels == 512) return launch_mlp_wide<T, 512, 1, 8, 2, 2, PACKED, 2>(x, resid, w1, b1, w2, b2, n, out, stream); \
+    } while (0)
+    if (dtype == PTV3_F16) PTV3_MW(_Float16);
+    if (dtype == PTV3_BF16) PTV3_MW(__bf16);
+#undef PTV3_MW
+    return PTV3_ESHAPE;
+}
+
+int block_tail_wide_any(const void* attn, const void* sum, const void* packed, const void* b1, const void* b2, int dtype,
+                        int64_t n, int channels, void* out, hipStream_t stream, TailArgs tail) {
+#define PTV3_MW(T)                                                                                                      \
+    do {                                                                                                                \
+        if (channels == 128)                                                                                            \
+            return launch_mlp_wide<T, 128, 2, 4, 1, 4, true, 3, true>(attn, sum, packed, b1, nullptr, b2, n, out, stream, tail); \
+        if (channels == 256)                                                                                            \
+            return launch_mlp_wide<T, 256, 1, 8, 1, 4, true, 3, true>(attn, sum, packed, b1, nullptr, b2, n, out, stream, tail); \
     } while (0)
     if (dtype == PTV3_F16) PTV3_MW(_Float16);
     if (dtype == PTV3_BF16) PTV3_MW(__bf16);
@@ -333,4 +442,23 @@ extern "C" int ptv3_mlp_fused_packed(const void* x, const void* resid, const voi
     if (n == 0) return PTV3_OK;
     if (!x || !resid || !packed || !b1 || !b2 || !out) return PTV3_EINVAL;
     return mlp_wide_any<true>(x, resid, packed, b1, nullptr, b2, dtype, n, channels, out, (hipStream_t)stream_);
+}
+
+extern "C" int ptv3_block_tail_wide(const void* attn, const void* shortcut, const void* proj_packed, const void* proj_bias,
+                                    const void* ln_weight, const void* ln_bias, float ln_eps, const void* mlp_packed,
+                                    const void* b1, const void* b2, int dtype, int64_t n, int channels, void* out,
+                                    void* stream_) {
+    if (n < 0) return PTV3_EINVAL;
+    if (channels != 128 && channels != 256) return PTV3_ESHAPE;
+    if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
+    if (n == 0) return PTV3_OK;
+    if (!attn || !shortcut || !proj_packed || !proj_bias || !ln_weight || !ln_bias || !mlp_packed || !b1 || !b2 || !out)
+        return PTV3_EINVAL;
+    return block_tail_wide_any(attn, shortcut, mlp_packed, b1, b2, dtype, n, channels, out, (hipStream_t)stream_,
+                               TailArgs{proj_packed, proj_bias, ln_weight, ln_bias, ln_eps});
+}
+
+extern "C" int64_t ptv3_linear_pack_weights_blocks(int channels) {
+    if (channels != 128 && channels != 256 && channels != 512) return 0;
+    return ptv3_ceil_div((int64_t)channels * channels / 8, 256);
 }

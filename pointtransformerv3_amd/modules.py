@@ -434,6 +434,13 @@ class Block(PointModule):
         shift = mlp.fc2.bias if (plain_mlp and not fused_mlp) else None
         point.feat = normed
         attn_out = self.attn.attend(point, ops.linear(normed, self.attn.qkv))
+        if (fused_mlp and self.channels in ops.BLOCK_TAIL_WIDE_CHANNELS and type(self.attn.proj) is nn.Linear
+                and self.attn.proj.bias is not None and not (self.training and self.attn.proj_drop.p > 0)):
+            # proj, the residual, the MLP's pre-norm and the MLP with its residual in one kernel
+            feat = ops.block_tail_wide(attn_out, feat, self.attn.proj, ln2, mlp)
+            point.feat = feat
+            point.sparse_conv_feat = point.sparse_conv_feat.replace_feature(feat)
+            return point
         if ops.linear_ln_ok(attn_out, self.attn.proj) and not (self.training and self.attn.proj_drop.p > 0):
             # proj, the residual and the MLP's pre-norm in one kernel
             feat, normed = ops.linear_ln(attn_out, self.attn.proj, feat, ln2, 2, shift=shift)

@@ -1457,27 +1457,42 @@ _MLP_PACK_TABLES = {}
 _MLP_PACK_USERS = weakref.WeakSet()   # the MLPs that have asked for packed weights: one stale copy has all redone
 
 
+def _pack_stamp(m, device):
+    """What a module's packed copy was made from: an MLP's two weights, or the one weight of a C -> C Linear."""
+    if hasattr(m, "fc1"):
+        return (parameter_stamp(m.fc1.weight), parameter_stamp(m.fc2.weight), device)
+    return (parameter_stamp(m.weight), device)
+
+
 def repack_mlp_weights(modules, dtype, device):
-    """Packed weight streams, in dtype, of every MLP in `modules` (fc1: C -> 4C, fc2: 4C -> C, C in
-    MLP_PACKED_CHANNELS) whose copy is missing or older than its parameters (parameter_stamp): one launch for all
-    of them. A module keeps its copies in module._packed_stream[dtype] = ((stamps, device), tensor), redone in place."""
+    """Packed weight streams, in dtype, of every module in `modules` whose copy is missing or older than its
+    parameters (parameter_stamp), one launch for all of them: MLPs (fc1: C -> 4C, fc2: 4C -> C) and square Linear
+    layers (C -> C, the attention's projection for block_tail_wide), C in MLP_PACKED_CHANNELS. A module keeps its
+    copies in module._packed_stream[dtype] = ((stamps, device), tensor), redone in place."""
     lib = _lib.load()
     jobs, blocks, done = [], 0, []
     for m in list(modules):
-        w1, w2 = m.fc1.weight, m.fc2.weight
-        c = w2.shape[0]
-        if w1.device != device or c not in MLP_PACKED_CHANNELS or tuple(w1.shape) != (4 * c, c) or tuple(w2.shape) != (c, 4 * c):
+        if hasattr(m, "fc1"):
+            w1, w2 = m.fc1.weight, m.fc2.weight
+            c = w2.shape[0]
+            ok = tuple(w1.shape) == (4 * c, c) and tuple(w2.shape) == (c, 4 * c)
+        else:
+            w1, w2 = m.weight, None
+            c = w1.shape[0]
+            ok = tuple(w1.shape) == (c, c)
+        if w1.device != device or c not in MLP_PACKED_CHANNELS or not ok:
             continue
         held = m.__dict__.setdefault("_packed_stream", {})
-        now = (parameter_stamp(w1), parameter_stamp(w2), device)
+        now = _pack_stamp(m, device)
         entry = held.get(dtype)
         if entry is not None and entry[0] == now:
             continue
-        s1, s2 = cast_cached(w1, dtype).detach().contiguous(), cast_cached(w2, dtype).detach().contiguous()
+        s1 = cast_cached(w1, dtype).detach().contiguous()
+        s2 = cast_cached(w2, dtype).detach().contiguous() if w2 is not None else None
         packed = entry[1] if entry is not None and entry[1].device == device else torch.empty(
-            8 * c * c, dtype=dtype, device=device)
-        jobs.append((s1.data_ptr(), s2.data_ptr(), packed.data_ptr(), c, 0, blocks))
-        blocks += lib.ptv3_mlp_pack_weights_blocks(c)
+            (8 if w2 is not None else 1) * c * c, dtype=dtype, device=device)
+        jobs.append((s1.data_ptr(), s2.data_ptr() if s2 is not None else 0, packed.data_ptr(), c, 0, blocks))
+        blocks += lib.ptv3_mlp_pack_weights_blocks(c) if w2 is not None else lib.ptv3_linear_pack_weights_blocks(c)
         done.append((held, now, packed, s1, s2))
     if not jobs:
         return
@@ -1493,20 +1508,49 @@ def repack_mlp_weights(modules, dtype, device):
         held[dtype] = (now, packed)
 
 
+def _packed_stream(m, dtype):
+    """The module's packed copy in dtype, redone first (with every other stale one) when its parameters moved."""
+    held = m.__dict__.get("_packed_stream")
+    entry = held.get(dtype) if held else None
+    device = (m.fc1.weight if hasattr(m, "fc1") else m.weight).device
+    if entry is None or entry[0] != _pack_stamp(m, device):
+        _MLP_PACK_USERS.add(m)
+        repack_mlp_weights(_MLP_PACK_USERS, dtype, device)
+        entry = m._packed_stream[dtype]
+    return entry[1]
+
+
+BLOCK_TAIL_WIDE_CHANNELS = (128, 256)
+
+
+def block_tail_wide(attn, shortcut, proj, ln2, mlp):
+    """sum = shortcut + proj(attn); returns sum + mlp.fc2(GELU(mlp.fc1(ln2(sum)))) from one kernel: the second half
+    of a block (model.py:458-460, :595-602) at BLOCK_TAIL_WIDE_CHANNELS. attn, shortcut (N, C) fp16/bf16; proj a
+    Linear C -> C, ln2 an affine LayerNorm, mlp with fc1: C -> 4C and fc2: 4C -> C (all with biases). The weights go
+    through the modules' packed copies (repack_mlp_weights)."""
+    _dev(attn, shortcut, proj.weight, mlp.fc1.weight, mlp.fc2.weight)
+    lib = _lib.load()
+    attn = attn.contiguous()
+    dt = attn.dtype
+    shortcut = shortcut.to(dt).contiguous()
+    n, c = attn.shape
+    assert c in BLOCK_TAIL_WIDE_CHANNELS and tuple(shortcut.shape) == (n, c)
+    mlp_packed, proj_packed = _packed_stream(mlp, dt), _packed_stream(proj, dt)
+    keep = [cast_cached(t, dt).detach().contiguous() for t in (proj.bias, ln2.weight, ln2.bias, mlp.fc1.bias, mlp.fc2.bias)]
+    out = torch.empty_like(attn)
+    _lib.check(lib.ptv3_block_tail_wide(_ptr(attn), _ptr(shortcut), _ptr(proj_packed), _ptr(keep[0]), _ptr(keep[1]),
+                                        _ptr(keep[2]), float(ln2.eps), _ptr(mlp_packed), _ptr(keep[3]), _ptr(keep[4]),
+                                        _dtype_code(attn), n, c, _ptr(out), _stream()), "ptv3_block_tail_wide")
+    return out
+
+
 def mlp_fused_module(x, resid, mlp):
     """resid + mlp(x) from the fused kernel for a module with fc1 and fc2. At MLP_PACKED_CHANNELS the weights go
     through a packed copy that the module keeps per dtype and that is redone, in place, when a parameter may have
-    changed (parameter_stamp) -- together with every other MLP's that is stale, in one launch."""
-    w1, w2 = mlp.fc1.weight, mlp.fc2.weight
+    changed (parameter_stamp) -- together with every other module's that is stale, in one launch."""
     if x.shape[1] not in MLP_PACKED_CHANNELS:
-        return mlp_fused(x, resid, w1, mlp.fc1.bias, w2, mlp.fc2.bias)
-    held = mlp.__dict__.get("_packed_stream")
-    entry = held.get(x.dtype) if held else None
-    if entry is None or entry[0] != (parameter_stamp(w1), parameter_stamp(w2), w1.device):
-        _MLP_PACK_USERS.add(mlp)
-        repack_mlp_weights(_MLP_PACK_USERS, x.dtype, w1.device)
-        entry = mlp._packed_stream[x.dtype]
-    return mlp_fused_packed(x, resid, entry[1], mlp.fc1.bias, mlp.fc2.bias)
+        return mlp_fused(x, resid, mlp.fc1.weight, mlp.fc1.bias, mlp.fc2.weight, mlp.fc2.bias)
+    return mlp_fused_packed(x, resid, _packed_stream(mlp, x.dtype), mlp.fc1.bias, mlp.fc2.bias)
 
 
 def _opt(t, dt):

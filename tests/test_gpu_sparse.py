@@ -309,6 +309,62 @@ def test_mlp_fused_module_repacks_after_a_parameter_write():
     assert "_packed_stream" not in mlp.state_dict()
 
 
+def _tail_modules(c, dtype, seed):
+    """proj, norm2 and the MLP of a block at width c with weights that are no identity anywhere."""
+    from pointtransformerv3_amd.modules import MLP, LayerNorm
+    torch.manual_seed(seed)
+    proj, ln, mlp = torch.nn.Linear(c, c), LayerNorm(c), MLP(c, 4 * c)
+    with torch.no_grad():
+        ln.weight.uniform_(0.5, 1.5)
+        ln.bias.uniform_(-0.5, 0.5)
+        for lin in (proj, mlp.fc1, mlp.fc2):
+            lin.bias.uniform_(-0.5, 0.5)
+    return [m.to(dtype).to(DEV) for m in (proj, ln, mlp)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("c,n", [(128, 1), (128, 191), (128, 40_001), (128, 114_691), (256, 64), (256, 97), (256, 20_001),
+                                 (256, 32_773)])
+def test_block_tail_wide_parity(dtype, c, n):
+    """The second half of a block in one kernel (projection, residual, LayerNorm, MLP, residual) against the same
+    layers in torch fp32 on the same half-precision inputs and weights, and against the two kernels it replaces."""
+    import torch.nn.functional as F
+    o = ops()
+    proj, ln, mlp = _tail_modules(c, dtype, c + n)
+    g = torch.Generator().manual_seed(7 * c + n)
+    attn = torch.randn(n, c, generator=g).to(dtype).to(DEV)
+    short = (torch.randn(n, c, generator=g) * 2 + 0.75).to(dtype).to(DEV)    # rows with a mean well off zero
+    f = lambda t: t.float()
+    total = f(short) + F.linear(f(attn), f(proj.weight), f(proj.bias))
+    normed = F.layer_norm(total, (c,), f(ln.weight), f(ln.bias), ln.eps)
+    want = total + F.linear(F.gelu(F.linear(normed, f(mlp.fc1.weight), f(mlp.fc1.bias))), f(mlp.fc2.weight), f(mlp.fc2.bias))
+    got = o.block_tail_wide(attn, short, proj, ln, mlp)
+    assert got.dtype == dtype and got.shape == (n, c) and rel_err(got, want.cpu()) < TOL[dtype]
+    feat, nrm = o.linear_ln(attn, proj, short, ln, 2)
+    two = o.mlp_fused_module(nrm, feat, mlp)
+    assert rel_err(got, two.cpu()) < TOL[dtype] / 4      # same layers, roundings at slightly different places
+
+
+def test_block_tail_wide_repacks_after_a_parameter_write():
+    o = ops()
+    proj, ln, mlp = _tail_modules(128, torch.float16, 11)
+    attn = torch.randn(700, 128, device=DEV).half()
+    short = torch.randn(700, 128, device=DEV).half()
+    first = o.block_tail_wide(attn, short, proj, ln, mlp)
+    held = proj._packed_stream[torch.float16][1]
+    assert held.numel() == 128 * 128
+    assert torch.equal(held.view(torch.int16).sort().values, proj.weight.detach().flatten().view(torch.int16).sort().values)
+    kept = proj.weight.detach().clone()
+    with torch.no_grad():
+        proj.weight.mul_(0.5)
+    second = o.block_tail_wide(attn, short, proj, ln, mlp)
+    assert not torch.equal(first, second) and proj._packed_stream[torch.float16][1] is held
+    with torch.no_grad():
+        proj.weight.copy_(kept)
+    assert torch.equal(o.block_tail_wide(attn, short, proj, ln, mlp), first)
+    assert "_packed_stream" not in proj.state_dict()
+
+
 def test_gelu_of_the_fused_kernels_over_every_fp16_input():
     """The GELU the Linear / MLP / block kernels evaluate (one v_exp_f32 and a degree-7 polynomial in its exponent)
     against the correctly rounded erf GELU of nn.GELU, for every finite fp16 input: an identity Linear with the GELU
