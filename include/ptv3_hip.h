@@ -549,9 +549,9 @@ int ptv3_mlp_pack_weights(const void *w1, const void *w2, int dtype, int channel
  * n_blocks their sum. Both half types move as 16-bit patterns, so a table may mix them. The table is trusted like
  * ptv3_pack_job's: channels 128, 256 or 512 (other rows are skipped), buffers of the stated sizes. */
 typedef struct {
-    const void *w1, *w2;  /* (4 * channels, channels) and (channels, 4 * channels); w2 NULL: w1 is one */
-    void *packed;         /* (channels, channels) matrix. 8 * channels^2 elements (channels^2 without w2) */
-    int32_t channels, reserved;
+    const void *w1, *w2;  /* (4 * channels, channels) and (channels, 4 * channels); w2 NULL: w1 is a */
+    void *packed;         /* (k * channels, channels) matrix. 8 * channels^2 elements (k * channels^2 without w2) */
+    int32_t channels, reserved;   /* reserved: k when w2 is NULL (0 counts as 1), else unused */
     int64_t first_block;
 } ptv3_mlp_pack_job;
 int64_t ptv3_mlp_pack_weights_blocks(int channels);
@@ -569,6 +569,21 @@ int ptv3_mlp_fused_packed(const void *x, const void *resid, const void *packed, 
  * The projection, the sum and the normalised rows are rounded to dtype where the separate layers would store them
  * and never leave the CU. PTV3_ESHAPE for other widths or dtypes. */
 int64_t ptv3_linear_pack_weights_blocks(int channels);
+
+/* First half of a block behind its convolution at 128 or 256 channels in one kernel, model.py:541-545 (the xCPE's
+ * Linear and LayerNorm), :587-589, :592-593 (norm1) and :450 (qkv):
+ *   feat = shortcut + LayerNorm_cpe(conv @ w_cpe^T + b_cpe)
+ *   qkv  = LayerNorm_1(feat) @ w_qkv^T + b_qkv
+ * conv, shortcut, feat: (n, channels) of dtype; qkv: (n, 3 * channels). packed holds 4 * channels^2 elements: w_cpe
+ * (channels, channels) and behind it w_qkv (3 * channels, channels), each written by ptv3_mlp_pack_weights_batch from
+ * a job whose w2 is NULL and whose `reserved` is the number of channels-row chunks (1 and 3; packed = the buffer, and
+ * the buffer + channels^2 elements); such a job owns reserved * ptv3_linear_pack_weights_blocks(channels) blocks.
+ * Intermediates are rounded to dtype where the separate layers would store them; the normalised rows never leave
+ * the CU. PTV3_ESHAPE for other widths or dtypes. */
+int ptv3_block_head_wide(const void *conv, const void *shortcut, const void *packed, const void *cpe_bias,
+                         const void *ln_cpe_weight, const void *ln_cpe_bias, float ln_cpe_eps, const void *ln1_weight,
+                         const void *ln1_bias, float ln1_eps, const void *qkv_bias, int dtype, int64_t n, int channels,
+                         void *feat, void *qkv, void *stream);
 int ptv3_block_tail_wide(const void *attn, const void *shortcut, const void *proj_packed, const void *proj_bias,
                          const void *ln_weight, const void *ln_bias, float ln_eps, const void *mlp_packed,
                          const void *b1, const void *b2, int dtype, int64_t n, int channels, void *out, void *stream);

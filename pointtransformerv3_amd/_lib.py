@@ -104,6 +104,7 @@ SIGNATURES = {
     "ptv3_mlp_pack_weights_batch": (_i32, [_vp, _i32, _i64, _vp]),
     "ptv3_mlp_fused_packed": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _vp, _vp]),
     "ptv3_linear_pack_weights_blocks": (_i64, [_i32]),
+    "ptv3_block_head_wide": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _vp, _f32, _vp, _i32, _i64, _i32, _vp, _vp, _vp]),
     "ptv3_block_tail_wide": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _vp, _vp, _i32, _i64, _i32, _vp, _vp]),
     "ptv3_block_head_fused": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _vp, _f32, _vp, _vp, _i32, _i64, _i32,
                                      _vp, _vp, _vp]),

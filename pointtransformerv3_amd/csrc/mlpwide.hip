@@ -56,11 +56,12 @@ __global__ __launch_bounds__(256) void mlp_pack_batch_kernel(const ptv3_mlp_pack
     const int c = job.channels;
     if (c != 128 && c != 256 && c != 512) return;   // a width the fused kernel does not take: touch nothing
     const int64_t idx = ((int64_t)blockIdx.x - job.first_block) * 256 + threadIdx.x;
-    // a job without w2 is one C x C matrix (C -> C Linear): the first KU steps of the same layout
-    if (idx < 0 || idx >= (job.w2 ? (int64_t)c * c : (int64_t)c * c / 8)) return;
+    // a job without w2 is a (k C, C) matrix of k = max(reserved, 1) chunks of C rows, every chunk like a chunk of fc1
+    const int k_chunks = job.reserved > 0 ? job.reserved : 1;
+    if (idx < 0 || idx >= (job.w2 ? (int64_t)c * c : (int64_t)k_chunks * c * c / 8)) return;
     const int lane = (int)(idx % 64), jj = (int)(idx / 64 % 2), ub = (int)(idx / 128 % (c / 32));
     const int u = (int)(idx / 128 / (c / 32)), ku = c / 32;
-    const int chunk = u / (2 * ku), st = (u / ku) & 1, kk = u % ku;
+    const int chunk = job.w2 ? u / (2 * ku) : u / ku, st = job.w2 ? (u / ku) & 1 : 0, kk = u % ku;
     const int unit = ub * 32 + lane % 32, k = kk * 32 + (lane / 32) * 16 + jj * 8;
     const uint16_t *w1 = (const uint16_t*)job.w1, *w2 = (const uint16_t*)job.w2;   // both half types: 16-bit patterns
     const uint16_t* src = st == 0 ? w1 + (int64_t)(chunk * c + unit) * c + k : w2 + (int64_t)unit * 4 * c + chunk * c + k;
@@ -75,31 +76,49 @@ __global__ __launch_bounds__(256) void mlp_pack_batch_kernel(const ptv3_mlp_pack
 // A work-group walks its rows in passes of 1 .. RTMAX groups of 32 rows per wave; the host gives every resident
 // work-group the same number of row groups (with tiles of one fixed size the last round of a launch of 37,681 rows at
 // 256 channels ran at half occupancy).
-struct TailArgs {   // what TAIL adds: the projection (packed), its bias, the LayerNorm's scale, shift and epsilon
-    const void *wp, *bp, *ln_w, *ln_b;
+// HEAD_MODE (PACKED only): the first half of a block behind its convolution. x is the convolution's output, resid the
+// block's input; a pass forms sum = resid + LayerNorm_cpe(x Wc^T + bc), writes it to out, and multiplies
+// LayerNorm_1(sum) by the three C-row chunks of the qkv weight (w1: Wc and Wqkv packed one behind the other, 4 KU
+// steps a pass), writing (N, 3C) rows to extra.qkv: the normalised rows never travel to memory and back.
+struct WideArgs {   // what the block halves add to the MLP's arguments
+    const void *wp, *bp, *ln_w, *ln_b;   // TAIL: packed projection, its bias; LayerNorm_2. HEAD: -, bc; LayerNorm_cpe
     float eps;
+    const void *ln1_w, *ln1_b, *bq;      // HEAD: LayerNorm_1, the qkv bias (3C)
+    float eps1;
+    void* qkv;                           // HEAD: (N, 3C) out
 };
+constexpr int MLP_MODE = 0, TAIL_MODE = 1, HEAD_MODE = 2;
 
-template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RTMAX, int THREADS, int MINW, bool TAIL>
+template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RTMAX, int THREADS, int MINW, int MODE>
 __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
     const T* __restrict__ x, const T* __restrict__ resid, const T* __restrict__ w1, const T* __restrict__ b1,
-    const T* __restrict__ w2, const T* __restrict__ b2, int64_t n, int upw, T* __restrict__ out, TailArgs tail) {
-    static_assert(!TAIL || PACKED, "the block tail reads packed weights");
+    const T* __restrict__ w2, const T* __restrict__ b2, int64_t n, int upw, T* __restrict__ out, WideArgs tail) {
+    constexpr bool TAIL = MODE == TAIL_MODE, HEADM = MODE == HEAD_MODE;
+    static_assert(MODE == MLP_MODE || PACKED, "the block halves read packed weights");
     typedef typename H16<T>::v8 v8;
     static_assert(WM * WN * PTV3_WAVE == THREADS && C == 32 * MT * WN, "the waves cover R x C");
     constexpr int RMAX = 32 * RTMAX * WM, H = 4 * C, XS = C + MW_PAD;
     constexpr int KU = C / 32;            // 32-wide contraction steps per stage
-    constexpr int HEAD = TAIL ? KU : 0;   // weight steps of the projection in front of the MLP's
-    constexpr int UNITS = HEAD + 4 * 2 * KU;   // weight steps per pass: (projection,) 4 chunks x (fc1, fc2)
+    constexpr int FRONT = TAIL ? KU : 0;  // weight steps of the projection in front of the MLP's
+    // weight steps per pass: (projection,) 4 chunks x (fc1, fc2); HEAD: the xCPE's Linear and three chunks of qkv
+    constexpr int UNITS = HEADM ? 4 * KU : FRONT + 4 * 2 * KU;
     static_assert(KU % DEPTH == 0, "the ring is indexed statically");
     constexpr int PPR = C / 8;            // 16-byte pieces per row
     extern __shared__ __align__(16) unsigned char mw_smem[];
     T* xt = (T*)mw_smem;                  // [RMAX][XS] input tile
     T* ht = xt + RMAX * XS;               // [RMAX][XS] hidden chunk, then the output tile
     T* bias_lds = ht + RMAX * XS;         // [4 C] fc1's bias, [C] fc2's: read per chunk without touching the vector-memory queue
-    for (int i = threadIdx.x; i < 5 * C / 8; i += THREADS)
-        *(u32x4*)(bias_lds + i * 8) = *(const u32x4*)((i < 4 * C / 8 ? b1 : b2 - 4 * C) + i * 8);
-    T* sum_lds = bias_lds + 8 * C;        // TAIL: [RMAX][XS] the block's running sum; before it the projection's bias
+    if (!HEADM)
+        for (int i = threadIdx.x; i < 5 * C / 8; i += THREADS)
+            *(u32x4*)(bias_lds + i * 8) = *(const u32x4*)((i < 4 * C / 8 ? b1 : b2 - 4 * C) + i * 8);
+    if (HEADM)   // [C] each: the xCPE Linear's bias, LayerNorm_cpe's scale and shift, LayerNorm_1's; [3 C] the qkv bias
+        for (int i = threadIdx.x; i < 8 * C / 8; i += THREADS) {
+            const int which = i / (C / 8), at = i % (C / 8);
+            const T* src = (const T*)(which == 0 ? tail.bp : which == 1 ? tail.ln_w : which == 2 ? tail.ln_b
+                                      : which == 3 ? tail.ln1_w : which == 4 ? tail.ln1_b : tail.bq);
+            *(u32x4*)(bias_lds + i * 8) = *(const u32x4*)(src + (which >= 5 ? i - 5 * (C / 8) : at) * 8);
+        }
+    T* sum_lds = bias_lds + 8 * C;        // TAIL: [RMAX][XS] the block's running sum (HEAD: a second staging tile); before it the projection's bias
     if (TAIL)                             // and the LayerNorm's scale and shift, [C] each
         for (int i = threadIdx.x; i < 3 * C / 8; i += THREADS) {
             const int which = i / (C / 8), at = i % (C / 8);
@@ -115,12 +134,12 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
     // weight step q of a pass: chunk q / (2 KU), layer (q / KU) & 1 (fc1, fc2), 32-wide step kk = q % KU; lane (col, hf)
     // of output tile a takes 2 x 8 consecutive inputs of weight row ch0 + 32 a + col
     auto issue = [&](int q, u32x4 (&r)[MT][2]) {
-        const int u = TAIL && q < HEAD ? q : q - HEAD;   // step inside its own packed copy
+        const int u = TAIL && q < FRONT ? q : q - FRONT;   // step inside its own packed copy
         const int chunk = u / (2 * KU), st = (u / KU) & 1, kk = u % KU;
 #pragma unroll
         for (int a = 0; a < MT; ++a) {
             if (PACKED) {
-                const T* p = (TAIL && q < HEAD ? (const T*)tail.wp : w1) + ((u * (C / 32) + wn * MT + a) * 2) * 512 + lane * 8;
+                const T* p = (TAIL && q < FRONT ? (const T*)tail.wp : w1) + ((u * (C / 32) + wn * MT + a) * 2) * 512 + lane * 8;
                 r[a][0] = *(const u32x4*)p;
                 r[a][1] = *(const u32x4*)(p + 512);
                 continue;
@@ -202,20 +221,22 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
         __syncthreads();
 
         f32x16 acc[MT][RT_], hacc[MT][RT_];
-        if constexpr (TAIL) {
-            // ---- projection of the attention rows (+ bias, from the C operand), rounded, parked in ht
+        // sums start from a bias vector in LDS (the MFMAs' C operand)
+        auto bias_from = [&](f32x16 (&sums)[MT][RT_], const T* vec) {
 #pragma unroll
             for (int a = 0; a < MT; ++a)
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const u32x2 bb = *(const u32x2*)(bias_lds + 5 * C + ch0 + a * 32 + 8 * g + 4 * hf);
+                    const u32x2 bb = *(const u32x2*)(vec + ch0 + a * 32 + 8 * g + 4 * hf);
                     const float bias[4] = {H16<T>::lo(bb[0]), H16<T>::hi(bb[0]), H16<T>::lo(bb[1]), H16<T>::hi(bb[1])};
 #pragma unroll
                     for (int rt = 0; rt < RT_; ++rt)
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) hacc[a][rt][4 * g + q] = bias[q];
+                        for (int q = 0; q < 4; ++q) sums[a][rt][4 * g + q] = bias[q];
                 }
-            stage(xt, hacc, 0);
+        };
+        // the wave's sums, rounded, into the staging tile
+        auto park = [&](const f32x16 (&sums)[MT][RT_], T* tile) {
 #pragma unroll
             for (int a = 0; a < MT; ++a)
 #pragma unroll
@@ -223,13 +244,43 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
                     const int cc = ch0 + a * 32 + 8 * g + 4 * hf;
 #pragma unroll
                     for (int rt = 0; rt < RT_; ++rt)
-                        *(u32x2*)(ht + (r0 + rt * 32 + col) * XS + cc) =
-                            (u32x2){H16<T>::pack2(hacc[a][rt][4 * g], hacc[a][rt][4 * g + 1]),
-                                    H16<T>::pack2(hacc[a][rt][4 * g + 2], hacc[a][rt][4 * g + 3])};
+                        *(u32x2*)(tile + (r0 + rt * 32 + col) * XS + cc) =
+                            (u32x2){H16<T>::pack2(sums[a][rt][4 * g], sums[a][rt][4 * g + 1]),
+                                    H16<T>::pack2(sums[a][rt][4 * g + 2], sums[a][rt][4 * g + 3])};
                 }
+        };
+        // LayerNorm of a row whose PPR pieces of 8 values sit in neighbouring lanes of one wave (the statistics are
+        // lane exchanges): v (this lane's piece) -> its normalised, scaled and shifted values, rounded and packed
+        auto norm_piece = [&](float (&v)[8], const u32x4 gq, const u32x4 bq, float eps) -> u32x4 {
+            float tot = 0.f;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) tot += v[k];
+#pragma unroll
+            for (int off = 1; off < PPR; off <<= 1) tot += __shfl_xor(tot, off, PTV3_WAVE);
+            const float mean = tot * (1.f / C);
+            float sq = 0.f;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                v[k] -= mean;
+                sq += v[k] * v[k];
+            }
+#pragma unroll
+            for (int off = 1; off < PPR; off <<= 1) sq += __shfl_xor(sq, off, PTV3_WAVE);
+            const float rstd = rsqrtf(sq * (1.f / C) + eps);
+            u32x4 nm;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                nm[k] = H16<T>::pack2(v[2 * k] * rstd * H16<T>::lo(gq[k]) + H16<T>::lo(bq[k]),
+                                      v[2 * k + 1] * rstd * H16<T>::hi(gq[k]) + H16<T>::hi(bq[k]));
+            return nm;
+        };
+        if constexpr (TAIL) {
+            // ---- projection of the attention rows (+ bias), rounded, parked in ht
+            bias_from(hacc, bias_lds + 5 * C);
+            stage(xt, hacc, 0);
+            park(hacc, ht);
             __syncthreads();   // every wave is done reading the attention rows in xt, the projection is in ht
-            // ---- sum = resid + projection (rounded, kept in sum_lds); its LayerNorm (rounded) replaces the x tile.
-            // A row's PPR pieces sit in neighbouring lanes of one wave: the statistics are lane exchanges
+            // ---- sum = resid + projection (rounded, kept in sum_lds); its LayerNorm (rounded) replaces the x tile
             const int pc = tid % PPR;
             const u32x4 gq = *(const u32x4*)(bias_lds + 6 * C + pc * 8), bq = *(const u32x4*)(bias_lds + 7 * C + pc * 8);
 #pragma unroll
@@ -238,35 +289,73 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
                 const u32x4 o = *(const u32x4*)(ht + rr * XS + pc * 8);
                 const u32x4 sh = *(const u32x4*)(sum_lds + rr * XS + pc * 8);   // written by this thread
                 u32x4 sm;
-                float v[8], tot = 0.f;
+                float v[8];
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     sm[k] = H16<T>::pack2(H16<T>::lo(o[k]) + H16<T>::lo(sh[k]), H16<T>::hi(o[k]) + H16<T>::hi(sh[k]));
                     v[2 * k] = H16<T>::lo(sm[k]);
                     v[2 * k + 1] = H16<T>::hi(sm[k]);
-                    tot += v[2 * k] + v[2 * k + 1];
                 }
                 *(u32x4*)(sum_lds + rr * XS + pc * 8) = sm;
-#pragma unroll
-                for (int off = 1; off < PPR; off <<= 1) tot += __shfl_xor(tot, off, PTV3_WAVE);
-                const float mean = tot * (1.f / C);
-                float sq = 0.f;
-#pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    v[k] -= mean;
-                    sq += v[k] * v[k];
-                }
-#pragma unroll
-                for (int off = 1; off < PPR; off <<= 1) sq += __shfl_xor(sq, off, PTV3_WAVE);
-                const float rstd = rsqrtf(sq * (1.f / C) + tail.eps);
-                u32x4 nm;
-#pragma unroll
-                for (int k = 0; k < 4; ++k)
-                    nm[k] = H16<T>::pack2(v[2 * k] * rstd * H16<T>::lo(gq[k]) + H16<T>::lo(bq[k]),
-                                          v[2 * k + 1] * rstd * H16<T>::hi(gq[k]) + H16<T>::hi(bq[k]));
-                *(u32x4*)(xt + rr * XS + pc * 8) = nm;
+                *(u32x4*)(xt + rr * XS + pc * 8) = norm_piece(v, gq, bq, tail.eps);
             }
             __syncthreads();
+        }
+        if constexpr (HEADM) {
+            // ---- the xCPE's Linear on the convolution rows (+ bias), rounded, parked in ht
+            bias_from(hacc, bias_lds);
+            stage(xt, hacc, 0);
+            park(hacc, ht);
+            __syncthreads();
+            // ---- sum = resid + LayerNorm_cpe(that) (both rounded) to memory; LayerNorm_1(sum) replaces the x tile
+            const int pc = tid % PPR;
+            const u32x4 gc = *(const u32x4*)(bias_lds + C + pc * 8), bc = *(const u32x4*)(bias_lds + 2 * C + pc * 8);
+            const u32x4 g1 = *(const u32x4*)(bias_lds + 3 * C + pc * 8), bb1 = *(const u32x4*)(bias_lds + 4 * C + pc * 8);
+#pragma unroll
+            for (int i = 0; i < PIECES; ++i) {
+                const int rr = (tid + i * THREADS) / PPR;
+                const u32x4 o = *(const u32x4*)(ht + rr * XS + pc * 8);
+                const bool live = row0 + rr < row_end;
+                u32x4 sh = {0, 0, 0, 0};
+                if (live) sh = *(const u32x4*)(resid + (row0 + rr) * C + pc * 8);
+                float v[8];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    v[2 * k] = H16<T>::lo(o[k]);
+                    v[2 * k + 1] = H16<T>::hi(o[k]);
+                }
+                const u32x4 z = norm_piece(v, gc, bc, tail.eps);
+                u32x4 sm;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    sm[k] = H16<T>::pack2(H16<T>::lo(z[k]) + H16<T>::lo(sh[k]), H16<T>::hi(z[k]) + H16<T>::hi(sh[k]));
+                    v[2 * k] = H16<T>::lo(sm[k]);
+                    v[2 * k + 1] = H16<T>::hi(sm[k]);
+                }
+                if (live) *(u32x4*)(out + (row0 + rr) * C + pc * 8) = sm;
+                *(u32x4*)(xt + rr * XS + pc * 8) = norm_piece(v, g1, bb1, tail.eps1);
+            }
+            __syncthreads();
+            // ---- qkv in three chunks of C outputs: product (+ bias), rounded, through a staging tile to memory in
+            // 16-byte pieces. Two staging tiles in turn: a chunk is parked while the one before it is still leaving,
+            // and the barrier behind the next park is the one that frees a tile for reuse
+#pragma unroll 1
+            for (int c = 0; c < 3; ++c) {
+                T* tile = (c & 1) ? ht : sum_lds;   // ht was read last by the piece loop above, a barrier ago
+                bias_from(hacc, bias_lds + (5 + c) * C);
+                stage(xt, hacc, (1 + c) * KU);
+                park(hacc, tile);
+                __syncthreads();
+#pragma unroll
+                for (int i = 0; i < PIECES; ++i) {
+                    const int rr = (tid + i * THREADS) / PPR;
+                    if (row0 + rr < row_end)
+                        *(u32x4*)((T*)tail.qkv + (row0 + rr) * (3 * C) + c * C + pc * 8) = *(const u32x4*)(tile + rr * XS + pc * 8);
+                }
+            }
+            // no barrier here: the next pass writes xt (last read before the barrier above), then parks into ht and
+            // the other tile only behind barriers of its own that every wave reaches after these stores
+            return;
         }
 #pragma unroll
         for (int a = 0; a < MT; ++a)
@@ -278,7 +367,7 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
 #pragma unroll 1   // unrolled, the chunks' loads are hoisted over each other and spill
         for (int c = 0; c < 4; ++c) {
             bias_into(hacc, c);
-            stage(xt, hacc, HEAD + 2 * c * KU);
+            stage(xt, hacc, FRONT + 2 * c * KU);
             // hacc[a][rt][v]: hidden unit ch0 + 32 a + 8 (v / 4) + 4 hf + v % 4 of row r0 + 32 rt + col
 #pragma unroll
             for (int a = 0; a < MT; ++a)
@@ -292,7 +381,7 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
                                     gelu_round_pack2<T>(hacc[a][rt][4 * g + 2], hacc[a][rt][4 * g + 3])};
                 }
             __syncthreads();
-            stage(ht, acc, HEAD + (2 * c + 1) * KU);
+            stage(ht, acc, FRONT + (2 * c + 1) * KU);
             __syncthreads();
         }
 
@@ -348,14 +437,15 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
     }
 }
 
-template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RTMAX, bool TAIL = false,
+template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RTMAX, int MODE = MLP_MODE,
           int THREADS = MW_THREADS, int MINW = 2>
 int launch_mlp_wide(const void* x, const void* resid, const void* w1, const void* b1, const void* w2, const void* b2,
-                    int64_t n, void* out, hipStream_t stream, TailArgs tail = TailArgs{}) {
+                    int64_t n, void* out, hipStream_t stream, WideArgs tail = WideArgs{}) {
     constexpr int RMAX = 32 * RTMAX * WM, UNIT = 32 * WM;
-    const size_t lds = ((size_t)(TAIL ? 3 : 2) * RMAX * (C + MW_PAD) + (TAIL ? 8 : 5) * C) * sizeof(T);
-    static_assert(((size_t)(TAIL ? 3 : 2) * RMAX * (C + MW_PAD) + (TAIL ? 8 : 5) * C) * sizeof(T) <= 160 * 1024, "LDS of a CU");
-    auto kern = mlp_wide_kernel<T, C, WM, WN, MT, DEPTH, PACKED, RTMAX, THREADS, MINW, TAIL>;
+    constexpr size_t LDS = ((size_t)(MODE == MLP_MODE ? 2 : 3) * RMAX * (C + MW_PAD) + (MODE == MLP_MODE ? 5 : 8) * C) * sizeof(T);
+    static_assert(LDS <= 160 * 1024, "LDS of a CU");
+    const size_t lds = LDS;
+    auto kern = mlp_wide_kernel<T, C, WM, WN, MT, DEPTH, PACKED, RTMAX, THREADS, MINW, MODE>;
     static LdsGrant grant_configured;   // per instantiation and device
     if (const int rc_ = ptv3_allow_lds((const void*)kern, lds, grant_configured)) return rc_;
     // as many work-groups as the machine holds at a time (MINW waves per SIMD, THREADS / 256 of them from one
@@ -388,13 +478,28 @@ int mlp_wide_any(const void* x, const void* resid, const void* w1, const void* b
 }
 
 int block_tail_wide_any(const void* attn, const void* sum, const void* packed, const void* b1, const void* b2, int dtype,
-                        int64_t n, int channels, void* out, hipStream_t stream, TailArgs tail) {
+                        int64_t n, int channels, void* out, hipStream_t stream, WideArgs tail) {
 #define PTV3_MW(T)                                                                                                      \
     do {                                                                                                                \
         if (channels == 128)                                                                                            \
-            return launch_mlp_wide<T, 128, 2, 4, 1, 4, true, 3, true>(attn, sum, packed, b1, nullptr, b2, n, out, stream, tail); \
+            return launch_mlp_wide<T, 128, 2, 4, 1, 4, true, 3, TAIL_MODE>(attn, sum, packed, b1, nullptr, b2, n, out, stream, tail); \
         if (channels == 256)                                                                                            \
-            return launch_mlp_wide<T, 256, 1, 8, 1, 4, true, 3, true>(attn, sum, packed, b1, nullptr, b2, n, out, stream, tail); \
+            return launch_mlp_wide<T, 256, 1, 8, 1, 4, true, 3, TAIL_MODE>(attn, sum, packed, b1, nullptr, b2, n, out, stream, tail); \
+    } while (0)
+    if (dtype == PTV3_F16) PTV3_MW(_Float16);
+    if (dtype == PTV3_BF16) PTV3_MW(__bf16);
+#undef PTV3_MW
+    return PTV3_ESHAPE;
+}
+
+int block_head_wide_any(const void* conv, const void* shortcut, const void* packed, int dtype, int64_t n, int channels,
+                        void* feat, hipStream_t stream, WideArgs args) {
+#define PTV3_MW(T)                                                                                                      \
+    do {                                                                                                                \
+        if (channels == 128)                                                                                            \
+            return launch_mlp_wide<T, 128, 2, 4, 1, 4, true, 3, HEAD_MODE>(conv, shortcut, packed, nullptr, nullptr, nullptr, n, feat, stream, args); \
+        if (channels == 256)                                                                                            \
+            return launch_mlp_wide<T, 256, 1, 8, 1, 4, true, 3, HEAD_MODE>(conv, shortcut, packed, nullptr, nullptr, nullptr, n, feat, stream, args); \
     } while (0)
     if (dtype == PTV3_F16) PTV3_MW(_Float16);
     if (dtype == PTV3_BF16) PTV3_MW(__bf16);
@@ -455,10 +560,26 @@ extern "C" int ptv3_block_tail_wide(const void* attn, const void* shortcut, cons
     if (!attn || !shortcut || !proj_packed || !proj_bias || !ln_weight || !ln_bias || !mlp_packed || !b1 || !b2 || !out)
         return PTV3_EINVAL;
     return block_tail_wide_any(attn, shortcut, mlp_packed, b1, b2, dtype, n, channels, out, (hipStream_t)stream_,
-                               TailArgs{proj_packed, proj_bias, ln_weight, ln_bias, ln_eps});
+                               WideArgs{proj_packed, proj_bias, ln_weight, ln_bias, ln_eps, nullptr, nullptr, nullptr, 0.f, nullptr});
 }
 
 extern "C" int64_t ptv3_linear_pack_weights_blocks(int channels) {
     if (channels != 128 && channels != 256 && channels != 512) return 0;
     return ptv3_ceil_div((int64_t)channels * channels / 8, 256);
+}
+
+extern "C" int ptv3_block_head_wide(const void* conv, const void* shortcut, const void* packed, const void* cpe_bias,
+                                    const void* ln_cpe_weight, const void* ln_cpe_bias, float ln_cpe_eps,
+                                    const void* ln1_weight, const void* ln1_bias, float ln1_eps, const void* qkv_bias,
+                                    int dtype, int64_t n, int channels, void* feat, void* qkv, void* stream_) {
+    if (n < 0) return PTV3_EINVAL;
+    if (channels != 128 && channels != 256) return PTV3_ESHAPE;
+    if (dtype != PTV3_F16 && dtype != PTV3_BF16) return PTV3_ESHAPE;
+    if (n == 0) return PTV3_OK;
+    if (!conv || !shortcut || !packed || !cpe_bias || !ln_cpe_weight || !ln_cpe_bias || !ln1_weight || !ln1_bias ||
+        !qkv_bias || !feat || !qkv)
+        return PTV3_EINVAL;
+    return block_head_wide_any(conv, shortcut, packed, dtype, n, channels, feat, (hipStream_t)stream_,
+                               WideArgs{nullptr, cpe_bias, ln_cpe_weight, ln_cpe_bias, ln_cpe_eps, ln1_weight, ln1_bias,
+                                        qkv_bias, ln1_eps, qkv});
 }

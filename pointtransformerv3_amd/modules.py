@@ -420,7 +420,13 @@ class Block(PointModule):
             point.sparse_conv_feat = point.sparse_conv_feat.replace_feature(feat)
             return point
         same_eps = ln_cpe.eps == ln1.eps
-        if ops.linear_ln_ok(conv, self.cpe[1]) and same_eps:
+        qkv = None
+        if (fused_mlp and self.channels in ops.BLOCK_HEAD_WIDE_PAYS and type(self.cpe[1]) is nn.Linear
+                and self.cpe[1].bias is not None and type(self.attn.qkv) is nn.Linear and self.attn.qkv.bias is not None
+                and self.attn.enable_flash):
+            # cpe Linear, its LayerNorm, the residual, the attention's pre-norm and qkv in one kernel
+            feat, qkv = ops.block_head_wide(conv, point.feat, self.cpe[1], ln_cpe, ln1, self.attn.qkv)
+        elif ops.linear_ln_ok(conv, self.cpe[1]) and same_eps:
             # cpe Linear, its LayerNorm, the residual and the attention's pre-norm in one kernel
             feat, normed = ops.linear_ln(conv, self.cpe[1], point.feat, ln_cpe, 3, ln2=ln1)
         else:
@@ -432,8 +438,10 @@ class Block(PointModule):
         # When fc2 runs as a separate GEMM it accumulates onto the stored sum (beta = 1), so its
         # bias is added to that sum here: feat + fc2(h) + b2 without a separate add pass
         shift = mlp.fc2.bias if (plain_mlp and not fused_mlp) else None
-        point.feat = normed
-        attn_out = self.attn.attend(point, ops.linear(normed, self.attn.qkv))
+        if qkv is None:
+            point.feat = normed
+            qkv = ops.linear(normed, self.attn.qkv)
+        attn_out = self.attn.attend(point, qkv)
         if (fused_mlp and self.channels in ops.BLOCK_TAIL_WIDE_CHANNELS and type(self.attn.proj) is nn.Linear
                 and self.attn.proj.bias is not None and not (self.training and self.attn.proj_drop.p > 0)):
             # proj, the residual, the MLP's pre-norm and the MLP with its residual in one kernel

@@ -164,6 +164,24 @@ def cast_cached(t, dtype, layout="plain"):
     return entry.out
 
 
+_IDLE_WORK = []        # callables that bring derived parameter copies up to date, see refresh_derived_copies
+_IDLE_EPOCH = [-1]     # the invalidate_casts() count they last ran for
+IDLE_WORK_ALLOWED = True   # off inside PrologueOverlap.scope(): what is allocated there is recycled two forwards on
+
+
+def refresh_derived_copies():
+    """Redo, once per invalidate_casts() epoch, the packed weight copies that the inference kernels will ask for
+    (every convolution's and MLP's that has been used before), at a moment when the host has nothing better to do:
+    Readback.get() calls this when its value is still on the way, the model before it queues an overlapped index
+    prologue. Found stale at their first use instead, the copies cost the host its 0.2 ms of stamp comparisons right
+    where the GPU waits for the launch behind them."""
+    if _IDLE_EPOCH[0] == _CAST_EPOCH[0] or not IDLE_WORK_ALLOWED or torch.is_grad_enabled():
+        return
+    _IDLE_EPOCH[0] = _CAST_EPOCH[0]
+    for fn in _IDLE_WORK:
+        fn()
+
+
 class Readback:
     """Device -> host read of a small tensor that does not drain the stream.
 
@@ -187,6 +205,8 @@ class Readback:
         """The values as a Python list (waits for the copy only)."""
         if Readback.blocking:
             return self.tensor.tolist()
+        if not self.done.query():
+            refresh_derived_copies()
         self.done.synchronize()
         return self.host.tolist()
 
@@ -664,16 +684,18 @@ class PrologueOverlap:
         self.turn ^= 1
         if self.done[self.turn] is not None:
             self.done[self.turn].synchronize()   # two forwards back: over long ago
-        global AHEAD_ON_SIDE_STREAM
+        global AHEAD_ON_SIDE_STREAM, IDLE_WORK_ALLOWED
+        refresh_derived_copies()   # on the current stream, before it: the host is a forward's tail ahead of the GPU here
         main = torch.cuda.current_stream(self.device)
         ahead, AHEAD_ON_SIDE_STREAM = AHEAD_ON_SIDE_STREAM, False   # the shared side stream still holds the last forward's work
+        idle, IDLE_WORK_ALLOWED = IDLE_WORK_ALLOWED, False
         try:
             with torch.cuda.stream(self.stream), torch.cuda.use_mem_pool(self.pools[self.turn], self.device):
                 yield
                 ready = torch.cuda.Event()
                 ready.record(self.stream)
         finally:
-            AHEAD_ON_SIDE_STREAM = ahead
+            AHEAD_ON_SIDE_STREAM, IDLE_WORK_ALLOWED = ahead, idle
         main.wait_event(ready)
 
     def forward_queued(self):
@@ -1457,43 +1479,71 @@ _MLP_PACK_TABLES = {}
 _MLP_PACK_USERS = weakref.WeakSet()   # the MLPs that have asked for packed weights: one stale copy has all redone
 
 
-def _pack_stamp(m, device):
-    """What a module's packed copy was made from: an MLP's two weights, or the one weight of a C -> C Linear."""
+class HeadWeights:
+    """The two Linear layers whose weights block_head_wide streams from one packed copy: the xCPE's C -> C and the
+    attention's C -> 3C. Lives on the qkv module (so that it lasts as long as the layers) and holds the copy."""
+
+    def __init__(self, cpe_linear, qkv_linear):
+        self.parts = (cpe_linear, qkv_linear)
+
+    @staticmethod
+    def of(cpe_linear, qkv_linear):
+        held = qkv_linear.__dict__.get("_head_weights")
+        if held is None or held.parts[0] is not cpe_linear:
+            held = qkv_linear.__dict__["_head_weights"] = HeadWeights(cpe_linear, qkv_linear)
+        return held
+
+
+def _pack_parts(m):
+    """What a module's packed copy is made of: [(weight, rows / C or None for the MLP pair)], and C."""
+    if isinstance(m, HeadWeights):
+        c = m.parts[0].weight.shape[0]
+        ok = tuple(m.parts[0].weight.shape) == (c, c) and tuple(m.parts[1].weight.shape) == (3 * c, c)
+        return [(m.parts[0].weight, 1), (m.parts[1].weight, 3)], c, ok
     if hasattr(m, "fc1"):
-        return (parameter_stamp(m.fc1.weight), parameter_stamp(m.fc2.weight), device)
-    return (parameter_stamp(m.weight), device)
+        c = m.fc2.weight.shape[0]
+        ok = tuple(m.fc1.weight.shape) == (4 * c, c) and tuple(m.fc2.weight.shape) == (c, 4 * c)
+        return [(m.fc1.weight, None), (m.fc2.weight, None)], c, ok
+    c = m.weight.shape[0]
+    return [(m.weight, 1)], c, tuple(m.weight.shape) == (c, c)
+
+
+def _pack_stamp(m, device):
+    """What a module's packed copy was made from: the stamps of its weights."""
+    return tuple(parameter_stamp(w) for w, _ in _pack_parts(m)[0]) + (device,)
 
 
 def repack_mlp_weights(modules, dtype, device):
     """Packed weight streams, in dtype, of every module in `modules` whose copy is missing or older than its
-    parameters (parameter_stamp), one launch for all of them: MLPs (fc1: C -> 4C, fc2: 4C -> C) and square Linear
-    layers (C -> C, the attention's projection for block_tail_wide), C in MLP_PACKED_CHANNELS. A module keeps its
-    copies in module._packed_stream[dtype] = ((stamps, device), tensor), redone in place."""
+    parameters (parameter_stamp), one launch for all of them: MLPs (fc1: C -> 4C, fc2: 4C -> C), square Linear
+    layers (C -> C, the attention's projection for block_tail_wide) and HeadWeights pairs (block_head_wide), C in
+    MLP_PACKED_CHANNELS. A module keeps its copies in module._packed_stream[dtype] = ((stamps, device), tensor),
+    redone in place."""
     lib = _lib.load()
     jobs, blocks, done = [], 0, []
     for m in list(modules):
-        if hasattr(m, "fc1"):
-            w1, w2 = m.fc1.weight, m.fc2.weight
-            c = w2.shape[0]
-            ok = tuple(w1.shape) == (4 * c, c) and tuple(w2.shape) == (c, 4 * c)
-        else:
-            w1, w2 = m.weight, None
-            c = w1.shape[0]
-            ok = tuple(w1.shape) == (c, c)
-        if w1.device != device or c not in MLP_PACKED_CHANNELS or not ok:
+        parts, c, ok = _pack_parts(m)
+        if parts[0][0].device != device or c not in MLP_PACKED_CHANNELS or not ok:
             continue
         held = m.__dict__.setdefault("_packed_stream", {})
         now = _pack_stamp(m, device)
         entry = held.get(dtype)
         if entry is not None and entry[0] == now:
             continue
-        s1 = cast_cached(w1, dtype).detach().contiguous()
-        s2 = cast_cached(w2, dtype).detach().contiguous() if w2 is not None else None
-        packed = entry[1] if entry is not None and entry[1].device == device else torch.empty(
-            (8 if w2 is not None else 1) * c * c, dtype=dtype, device=device)
-        jobs.append((s1.data_ptr(), s2.data_ptr() if s2 is not None else 0, packed.data_ptr(), c, 0, blocks))
-        blocks += lib.ptv3_mlp_pack_weights_blocks(c) if w2 is not None else lib.ptv3_linear_pack_weights_blocks(c)
-        done.append((held, now, packed, s1, s2))
+        srcs = [cast_cached(w, dtype).detach().contiguous() for w, _ in parts]
+        mlp_pair = parts[0][1] is None
+        total = 8 * c * c if mlp_pair else sum(k for _, k in parts) * c * c
+        packed = entry[1] if entry is not None and entry[1].device == device else torch.empty(total, dtype=dtype, device=device)
+        if mlp_pair:
+            jobs.append((srcs[0].data_ptr(), srcs[1].data_ptr(), packed.data_ptr(), c, 0, blocks))
+            blocks += lib.ptv3_mlp_pack_weights_blocks(c)
+        else:
+            at = 0
+            for src, (_, k) in zip(srcs, parts):
+                jobs.append((src.data_ptr(), 0, packed.data_ptr() + at * c * c * packed.element_size(), c, k, blocks))
+                blocks += k * lib.ptv3_linear_pack_weights_blocks(c)
+                at += k
+        done.append((held, now, packed, srcs))
     if not jobs:
         return
     table = np.array(jobs, dtype=_MLP_PACK_JOB).tobytes()
@@ -1504,15 +1554,18 @@ def repack_mlp_weights(modules, dtype, device):
     with torch.cuda.device(device):
         _lib.check(lib.ptv3_mlp_pack_weights_batch(kept[1].data_ptr(), len(jobs), blocks, _stream()),
                    "ptv3_mlp_pack_weights_batch")
-    for held, now, packed, _, _ in done:
+    for held, now, packed, _ in done:
         held[dtype] = (now, packed)
+
+
+_IDLE_WORK.append(lambda: [repack_mlp_weights(_MLP_PACK_USERS, dtype, device) for device, dtype in list(_MLP_PACK_TABLES)])
 
 
 def _packed_stream(m, dtype):
     """The module's packed copy in dtype, redone first (with every other stale one) when its parameters moved."""
     held = m.__dict__.get("_packed_stream")
     entry = held.get(dtype) if held else None
-    device = (m.fc1.weight if hasattr(m, "fc1") else m.weight).device
+    device = _pack_parts(m)[0][0][0].device
     if entry is None or entry[0] != _pack_stamp(m, device):
         _MLP_PACK_USERS.add(m)
         repack_mlp_weights(_MLP_PACK_USERS, dtype, device)
@@ -1521,6 +1574,9 @@ def _packed_stream(m, dtype):
 
 
 BLOCK_TAIL_WIDE_CHANNELS = (128, 256)
+# block_head_wide takes the same widths; where it measured faster than linear_ln + qkv Linear: 74 -> 59 us at
+# 146k x 128, 46.5 -> 46 us at 37.7k x 256 (a pass there is too short for what it costs to start and to leave)
+BLOCK_HEAD_WIDE_PAYS = (128,)
 
 
 def block_tail_wide(attn, shortcut, proj, ln2, mlp):
@@ -1534,7 +1590,7 @@ def block_tail_wide(attn, shortcut, proj, ln2, mlp):
     dt = attn.dtype
     shortcut = shortcut.to(dt).contiguous()
     n, c = attn.shape
-    assert c in BLOCK_TAIL_WIDE_CHANNELS and tuple(shortcut.shape) == (n, c)
+    assert c in (128, 256) and tuple(shortcut.shape) == (n, c)
     mlp_packed, proj_packed = _packed_stream(mlp, dt), _packed_stream(proj, dt)
     keep = [cast_cached(t, dt).detach().contiguous() for t in (proj.bias, ln2.weight, ln2.bias, mlp.fc1.bias, mlp.fc2.bias)]
     out = torch.empty_like(attn)
@@ -1595,6 +1651,30 @@ def block_tail_fused(attn, shortcut, proj, ln2, fc1, fc2):
                                          _ptr(keep[7]), _dtype_code(attn), n, c, keep[4].shape[0], _ptr(out),
                                          _stream()), "ptv3_block_tail_fused")
     return out
+
+
+def block_head_wide(conv, shortcut, cpe_linear, ln_cpe, ln1, qkv_linear):
+    """feat = shortcut + ln_cpe(cpe_linear(conv)); qkv = qkv_linear(ln1(feat)) in one kernel at
+    BLOCK_TAIL_WIDE_CHANNELS (model.py:541-545, :587-593, :450). conv, shortcut (N, C) fp16/bf16; the modules are a
+    Linear C -> C, two affine LayerNorms and a Linear C -> 3C, all with biases. Returns (feat, qkv). The weights go
+    through one packed copy of both matrices (HeadWeights, repack_mlp_weights)."""
+    _dev(conv, shortcut, cpe_linear.weight, qkv_linear.weight)
+    lib = _lib.load()
+    conv = conv.contiguous()
+    dt = conv.dtype
+    shortcut = shortcut.to(dt).contiguous()
+    n, c = conv.shape
+    assert c in (128, 256) and tuple(shortcut.shape) == (n, c)
+    packed = _packed_stream(HeadWeights.of(cpe_linear, qkv_linear), dt)
+    keep = [cast_cached(t, dt).detach().contiguous() for t in (cpe_linear.bias, ln_cpe.weight, ln_cpe.bias, ln1.weight,
+                                                                ln1.bias, qkv_linear.bias)]
+    feat = torch.empty_like(conv)
+    qkv = torch.empty((n, 3 * c), dtype=dt, device=conv.device)
+    _lib.check(lib.ptv3_block_head_wide(_ptr(conv), _ptr(shortcut), _ptr(packed), _ptr(keep[0]), _ptr(keep[1]),
+                                        _ptr(keep[2]), float(ln_cpe.eps), _ptr(keep[3]), _ptr(keep[4]), float(ln1.eps),
+                                        _ptr(keep[5]), _dtype_code(conv), n, c, _ptr(feat), _ptr(qkv), _stream()),
+               "ptv3_block_head_wide")
+    return feat, qkv
 
 
 BATCH_NORM_TRAIN_CHANNELS = (32, 64, 128, 256, 512)

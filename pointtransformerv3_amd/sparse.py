@@ -176,5 +176,8 @@ class SubMConv3d(nn.Module):
 _PACKED_USERS = weakref.WeakSet()
 
 
+ops._IDLE_WORK.append(lambda: [ops.repack_conv_weights(_PACKED_USERS, dtype, device) for device, dtype in list(ops._PACK_TABLES)])
+
+
 def is_spconv_module(module):
     return isinstance(module, SubMConv3d)

@@ -345,6 +345,67 @@ def test_block_tail_wide_parity(dtype, c, n):
     assert rel_err(got, two.cpu()) < TOL[dtype] / 4      # same layers, roundings at slightly different places
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("c,n", [(128, 1), (128, 191), (128, 40_001), (128, 114_691), (256, 64), (256, 97), (256, 20_001),
+                                 (256, 32_773)])
+def test_block_head_wide_parity(dtype, c, n):
+    """The first half of a block behind its convolution in one kernel (Linear, LayerNorm, residual, LayerNorm, qkv)
+    against the same layers in torch fp32 on the same half-precision inputs and weights, and against the two kernels
+    it replaces."""
+    import torch.nn.functional as F
+    from pointtransformerv3_amd.modules import LayerNorm
+    o = ops()
+    torch.manual_seed(c + n)
+    lin, lnc, ln1, qkv = torch.nn.Linear(c, c), LayerNorm(c), LayerNorm(c, eps=1e-4), torch.nn.Linear(c, 3 * c)
+    with torch.no_grad():
+        for ln in (lnc, ln1):
+            ln.weight.uniform_(0.5, 1.5)
+            ln.bias.uniform_(-0.5, 0.5)
+        for m in (lin, qkv):
+            m.bias.uniform_(-0.5, 0.5)
+    lin, lnc, ln1, qkv = [m.to(dtype).to(DEV) for m in (lin, lnc, ln1, qkv)]
+    g = torch.Generator().manual_seed(5 * c + n)
+    conv = (torch.randn(n, c, generator=g) + 0.5).to(dtype).to(DEV)
+    short = (torch.randn(n, c, generator=g) * 2 + 0.75).to(dtype).to(DEV)
+    f = lambda t: t.float()
+    want_feat = f(short) + F.layer_norm(F.linear(f(conv), f(lin.weight), f(lin.bias)), (c,), f(lnc.weight), f(lnc.bias), lnc.eps)
+    want_qkv = F.linear(F.layer_norm(want_feat, (c,), f(ln1.weight), f(ln1.bias), ln1.eps), f(qkv.weight), f(qkv.bias))
+    feat, got = o.block_head_wide(conv, short, lin, lnc, ln1, qkv)
+    assert feat.dtype == dtype and feat.shape == (n, c) and got.dtype == dtype and got.shape == (n, 3 * c)
+    assert rel_err(feat, want_feat.cpu()) < TOL[dtype] and rel_err(got, want_qkv.cpu()) < TOL[dtype]
+    ln1.eps = lnc.eps                      # the two-kernel route takes one epsilon for both norms
+    feat1, got1 = o.block_head_wide(conv, short, lin, lnc, ln1, qkv)
+    feat2, normed = o.linear_ln(conv, lin, short, lnc, 3, ln2=ln1)
+    assert rel_err(feat1, feat2.cpu()) < TOL[dtype] / 4 and rel_err(got1, o.linear(normed, qkv).cpu()) < TOL[dtype] / 4
+
+
+def test_block_head_wide_repacks_after_a_parameter_write():
+    from pointtransformerv3_amd.modules import LayerNorm
+    o = ops()
+    torch.manual_seed(13)
+    lin, lnc, ln1, qkv = [m.half().to(DEV) for m in (torch.nn.Linear(256, 256), LayerNorm(256), LayerNorm(256),
+                                                      torch.nn.Linear(256, 768))]
+    conv = torch.randn(300, 256, device=DEV).half()
+    short = torch.randn(300, 256, device=DEV).half()
+    f0, q0 = o.block_head_wide(conv, short, lin, lnc, ln1, qkv)
+    pack = qkv._head_weights
+    held = pack._packed_stream[torch.float16][1]
+    assert held.numel() == 4 * 256 * 256
+    both = torch.cat([lin.weight.detach().flatten(), qkv.weight.detach().flatten()])
+    assert torch.equal(held.view(torch.int16).sort().values, both.view(torch.int16).sort().values)
+    kept = qkv.weight.detach().clone()
+    with torch.no_grad():
+        qkv.weight.mul_(0.5)
+    f1, q1 = o.block_head_wide(conv, short, lin, lnc, ln1, qkv)
+    assert torch.equal(f0, f1) and not torch.equal(q0, q1) and pack._packed_stream[torch.float16][1] is held
+    with torch.no_grad():
+        qkv.weight.copy_(kept)
+        lin.weight.mul_(0.5)
+    f2, q2 = o.block_head_wide(conv, short, lin, lnc, ln1, qkv)
+    assert not torch.equal(f0, f2) and qkv._head_weights is pack
+    assert "_head_weights" not in qkv.state_dict() and "_packed_stream" not in qkv.state_dict()
+
+
 def test_block_tail_wide_repacks_after_a_parameter_write():
     o = ops()
     proj, ln, mlp = _tail_modules(128, torch.float16, 11)
