@@ -305,14 +305,16 @@ def conv_case(which, reps):
 DENSE_CASES = {   # name: (rows, channels) at the levels of the benchmark batch
     "tail64": (308_615, 64), "tail32": (403_093, 32), "head64": (308_615, 64), "mlp128": (146_195, 128),
     "mlp256": (37_681, 256), "linear_ln256": (37_681, 256),
+    "tail128": (146_195, 128), "tail256": (37_681, 256), "head128": (146_195, 128),
 }
 
 
 def dense_case(which, reps):
     """One fused dense kernel of a transformer block alone at the rows and width of a level of the benchmark batch,
-    fp16: `tail*` = proj + residual + LayerNorm + MLP + residual (block_tail_kernel), `head64` = cpe Linear +
-    LayerNorm + residual + LayerNorm + qkv Linear, `mlp*` = fc1 + GELU + fc2 + residual (mlp_wide_kernel on packed
-    weights), `linear_ln256` = proj Linear + residual + LayerNorm. The command to put under rocprofv3 --pmc."""
+    fp16: `tail*` = proj + residual + LayerNorm + MLP + residual (block_tail_kernel; from 128 channels on the tail mode
+    of mlp_wide_kernel), `head*` = cpe Linear + LayerNorm + residual + LayerNorm + qkv Linear (block_head_kernel, the
+    head mode of mlp_wide_kernel), `mlp*` = fc1 + GELU + fc2 + residual (mlp_wide_kernel on packed weights),
+    `linear_ln256` = proj Linear + residual + LayerNorm. The command to put under rocprofv3 --pmc."""
     from pointtransformerv3_amd import ops
     from pointtransformerv3_amd.modules import MLP
     dev = "cuda:0"
@@ -324,11 +326,17 @@ def dense_case(which, reps):
     gelus, flops, byts = 0, 0.0, 0.0
     if which.startswith("tail"):
         proj, ln2, fc1, fc2 = lin(c, c), ln(), lin(c, 4 * c), lin(4 * c, c)
-        fn = lambda: ops.block_tail_fused(x, res, proj, ln2, fc1, fc2)
+        if c >= 128:      # the TAIL mode of mlp_wide_kernel
+            from pointtransformerv3_amd.modules import LayerNorm
+            mlp, ln2 = MLP(c, 4 * c).half().to(dev), LayerNorm(c).half().to(dev)
+            fn = lambda: ops.block_tail_wide(x, res, proj, ln2, mlp)
+        else:
+            fn = lambda: ops.block_tail_fused(x, res, proj, ln2, fc1, fc2)
         gelus, flops, byts = 4 * n * c, 2.0 * n * c * c * 9, 3.0 * n * c * 2
     elif which.startswith("head"):
         cpe, lnc, ln1, qkv = lin(c, c), ln(), ln(), lin(c, 3 * c)
-        fn = lambda: ops.block_head_fused(x, res, cpe, lnc, ln1, qkv)
+        fn = (lambda: ops.block_head_wide(x, res, cpe, lnc, ln1, qkv)) if c >= 128 else (
+            lambda: ops.block_head_fused(x, res, cpe, lnc, ln1, qkv))
         flops, byts = 2.0 * n * c * c * 4, 6.0 * n * c * 2
     elif which.startswith("mlp"):
         mlp = MLP(c, 4 * c).half().to(dev)
@@ -614,7 +622,7 @@ def main():
     ap.add_argument("--no-overlap", action="store_true",
                     help="time the plain schedule only: by default the model's opt-in overlap_index_prologue is on (the "
                          "inputs are resident and complete before the timed region, which is what it asks for), so the "
-                         "index work of forward k + 1 runs beside the tail of forward k; the plain schedule is timed "
+                         "index work of forward k + 1 runs beside the feature kernels of forward k; the plain schedule is timed "
                          "after the timed region as well and reported beside it")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the short runs of baseline configs 5, 2 and 3 after the timed region")
@@ -761,8 +769,9 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"full PTv3 encoder-decoder forward, default architecture, {args.scenes} room "
                                f"scenes, {n_points} voxelised points, grid 0.02 m, 6-dim input, random-init weights",
-                   "schedule": ("forwards back to back; the index prologue of a forward (curve codes, sort, level-0 pair "
-                                "lists: no feature touched) runs on its own stream beside the tail of the forward before "
+                   "schedule": ("forwards back to back; the index pass of a forward (curve codes, sort, clusters, pooled "
+                                "tables, pair and tile lists, attention tables of every level: no feature touched) runs on "
+                                "its own stream beside the feature kernels of the forward before "
                                 "(PointTransformerV3.overlap_index_prologue, for inputs resident before the call)"
                                 if plain_ms is not None else "forwards back to back, plain schedule"),
                    "plain_schedule_ms_per_step": plain_ms,

@@ -26,9 +26,10 @@ CONV_A = "SQ_INSTS_MFMA SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CYCLES SQ_INSTS_VALU SQ
 DENSE_A = "SQ_INSTS_VALU SQ_INSTS_MFMA SQ_INSTS_VALU_TRANS_F32 SQ_INSTS_VALU_CVT SQ_ACTIVE_INST_VALU SQ_VALU_MFMA_BUSY_CYCLES SQ_WAVE_CYCLES SQ_CYCLES"
 DENSE_B = "SQ_WAIT_INST_ANY SQ_ACTIVE_INST_LDS SQ_LDS_BANK_CONFLICT SQ_INSTS_LDS SQ_BUSY_CYCLES"
 CONV_CASES = ("level0", "level1", "level2", "level3", "level4", "config3")
-DENSE_CASES = ("tail64", "tail32", "head64", "mlp128", "mlp256", "linear_ln256")
+DENSE_CASES = ("tail64", "tail32", "head64", "mlp128", "mlp256", "linear_ln256", "tail128", "tail256", "head128")
 DENSE_KERNEL = {"tail64": "block_tail_kernel", "tail32": "block_tail_kernel", "head64": "block_head_kernel",
-                "mlp128": "mlp_wide_kernel", "mlp256": "mlp_wide_kernel", "linear_ln256": "linear_wide_resident_kernel"}
+                "mlp128": "mlp_wide_kernel", "mlp256": "mlp_wide_kernel", "linear_ln256": "linear_wide_resident_kernel",
+                "tail128": "mlp_wide_kernel", "tail256": "mlp_wide_kernel", "head128": "mlp_wide_kernel"}
 
 
 def recipe(d):

@@ -50,10 +50,11 @@ class PointTransformerV3(PointModule):
         self.num_stages = len(enc_depths)
         self.order = [order] if isinstance(order, str) else order
         self.cls_mode = cls_mode
-        # Opt-in: the index work of level 0 (no feature is touched) runs on a stream of its own and does not wait
-        # for what the current stream holds, so in a loop of forwards it overlaps the tail of the forward before.
-        # Only for callers whose inputs are complete when forward() is called (nothing that produces them is still
-        # queued on the current stream); evaluation mode only.
+        # Opt-in: the index work of every level (curve codes and orders, clusters, pooled tables, pair and tile lists,
+        # attention tables: no feature is touched) runs first, on a stream of its own that does not wait for what
+        # the current stream holds, so in a loop of forwards it runs beside the feature kernels of the forward before
+        # and the feature pass that follows never waits for the host. Only for callers whose inputs are complete when
+        # forward() is called (nothing that produces them is still queued on the current stream); evaluation mode only.
         self.overlap_index_prologue = False
         self._prologue_state = None
         self.shuffle_orders = shuffle_orders
@@ -138,9 +139,12 @@ class PointTransformerV3(PointModule):
             self._prologue_state.forward_queued()
         return point
 
-    def _level0_index(self, data_dict):
+    def _level0_index(self, data_dict, everything=False):
         """Everything of level 0 that follows from the coordinates alone (model.py:966-970): the Point, its curve
-        codes and orders, the stem's pair lists, the clusters of the first pooling."""
+        codes and orders, the stem's pair lists, the clusters of the first pooling. `everything`: also what the
+        modules would otherwise make at their first use, on every level (the caller has put this on a stream of its
+        own): pair and tile lists of the convolutions, padding and slot tables of the attention, and the whole index
+        of the pooled levels (_pooled_index_ahead)."""
         point = Point(data_dict)
         # the pair lists of the stem and of the first stage's xCPE depend on the coordinates only:
         # their first halves are queued behind the first host read-back and run while the host waits
@@ -149,20 +153,49 @@ class PointTransformerV3(PointModule):
         if self.stride:
             point.pool_ahead(self.stride[0])   # the first pooling's clusters need the codes only
         point.sparsify()
-        if self.overlap_index_prologue and not self.training and point.feat.dtype != torch.float32:
-            # with the prologue on a stream of its own, whatever else of level 0 follows from the coordinates goes
-            # there too: the pair and tile lists of the level's convolutions, the attention's padding and slot tables
-            from .sparse import SubMConv3d
+        if everything:
             stage0 = next(iter(self.enc._modules.values()))
             dec0 = self.dec._modules.get("dec0") if not self.cls_mode else None
             for m in list(self.embedding.modules()) + list(stage0.modules()):
                 if isinstance(m, SubMConv3d):
                     m.lists_ahead(point.sparse_conv_feat)
-            blocks = [b for st in (stage0, dec0) if st is not None for b in st._modules.values() if isinstance(b, Block)]
-            if blocks and all(b.attn.enable_flash and b.attn.patch_size == blocks[0].attn.patch_size for b in blocks):
-                for b in blocks:
-                    b.attn._slots(point)
+            self._attention_tables_ahead(point, stage0, dec0)
+            self._pooled_index_ahead(point)
         return point
+
+    @staticmethod
+    def _attention_tables_ahead(point, *stages):
+        blocks = [b for st in stages if st is not None for b in st._modules.values() if isinstance(b, Block)]
+        if blocks and all(b.attn.enable_flash and b.attn.patch_size == blocks[0].attn.patch_size for b in blocks):
+            for b in blocks:
+                b.attn._slots(point)
+
+    def _pooled_index_ahead(self, point):
+        """The index of every pooled level (clusters, pooled codes / coordinates / orders, pair and tile lists,
+        attention tables: model.py:652-679, :165-172, :382-438 read coordinates only), level by level, each left on
+        its parent Point under "_pooled_ahead" for the pooling module to pick up. The pooling stages draw their row
+        shuffles from torch's CPU generator in module order here as they would in the forward: evaluation mode only
+        (stochastic depth and dropout draw from the same generator in between)."""
+        parent = point
+        for s, stage in enumerate(list(self.enc._modules.values())[1:], start=1):
+            down = stage._modules.get("down")
+            if not isinstance(down, SerializedPooling):
+                return
+            pooled = down.pooled_index(parent)
+            if down.next_stride is not None:
+                pooled.pool_ahead(down.next_stride)
+            dec = self.dec._modules.get(f"dec{s}") if not self.cls_mode else None
+            convs = [m for st in (stage, dec) if st is not None for m in st.modules() if isinstance(m, SubMConv3d)]
+            ready = {}
+            for ks, pend in pooled.pop("_pending_plans").items():
+                ready[ks] = ops.conv_plan_direct_finish(pend)
+                for m in convs:
+                    if m.kernel_size == ks:
+                        m.tiles_ahead(ready[ks])
+            pooled["_ready_plans"] = ready
+            self._attention_tables_ahead(pooled, stage, dec)
+            parent["_pooled_ahead"] = pooled
+            parent = pooled
 
     def _index_prologue(self, data_dict):
         feat = data_dict.get("feat")
@@ -173,5 +206,5 @@ class PointTransformerV3(PointModule):
         if self._prologue_state is None or self._prologue_state.device != feat.device:
             self._prologue_state = ops.PrologueOverlap(feat.device)
         with self._prologue_state.scope():
-            point = self._level0_index(data_dict)
+            point = self._level0_index(data_dict, everything=feat.dtype != torch.float32)
         return point

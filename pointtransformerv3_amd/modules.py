@@ -571,7 +571,11 @@ class SerializedPooling(PointModule):
         self.norm = PointSequential(norm_layer(out_channels)) if norm_layer is not None else None
         self.act = PointSequential(act_layer()) if act_layer is not None else None
 
-    def forward(self, point):
+    def pooled_index(self, point, pending=None):
+        """Everything of the pooled level that follows from the parent's coordinates alone (model.py:652-679, :690,
+        :695, :700-703): clusters, the pooled codes / coordinates / scene ids, the pooled orders and inverses, the
+        first halves of the pooled level's pair lists. `pending`: the cluster kernels when the caller has queued
+        them already. One host wait (the cluster count). Returns the pooled Point, without features."""
         pooling_depth = (math.ceil(self.stride) - 1).bit_length()
         if pooling_depth > point.serialized_depth:
             pooling_depth = 0
@@ -582,24 +586,19 @@ class SerializedPooling(PointModule):
 
         # clusters in ascending order of the (shifted) row-0 code
         indices = point.serialized_order[0]
-        ahead = point.pop("_pending_pool", None)   # started when the codes came into being (Point.pool_ahead)
-        pending = ahead[1] if ahead is not None and ahead[0] == shift else \
-            ops.pool_clusters_start(point.serialized_code[0], indices, shift, point.offset)
-        projected = ops.linear(point.feat, self.proj)   # needs no cluster count: runs while the count travels
+        if pending is None:
+            pending = self._clusters_started(point)
         cluster, idx_ptr, head, m, offset, offset_host = ops.pool_clusters_finish(pending)
         # the shuffle of the orders (model.py:675-679) is applied while the pooled tables are written
         perm = torch.randperm(point.serialized_code.shape[0]).tolist() if self.shuffle_orders else None   # CPU generator
         code, grid_coord, batch, indices4 = ops.pool_gather(point.serialized_code, shift, point.grid_coord,
                                                             pooling_depth, point.batch, head, perm)
-        # pooled orders: the distinct clusters met when walking the parent along each curve (same
-        # result as argsort of the pooled codes, model.py:667-674, without sorting)
         # pair lists of the convolutions on the pooled points: first half queued now, finished at first use
         plans = {ks: ops.conv_plan_direct_start(indices4, ks) for ks in self.plan_kernel_sizes}
+        # pooled orders: the distinct clusters met when walking the parent along each curve (same
+        # result as argsort of the pooled codes, model.py:667-674, without sorting)
         order, inverse = ops.pool_orders(point.serialized_order, cluster, m, perm)
-
-        fields = AttrDict(
-            feat=(SegmentReduce.apply(projected, indices, idx_ptr, self.reduce) if ops.wants_grad(projected)
-                  else ops.segment_reduce(projected, indices, idx_ptr, self.reduce)),
+        return Point(AttrDict(
             grid_coord=grid_coord,
             serialized_code=code,
             serialized_order=order,
@@ -611,18 +610,42 @@ class SerializedPooling(PointModule):
             _sparse_indices=indices4,   # [batch, x, y, z] int32, what sparsify() would concatenate
             _pending_plans=plans,
             _pool_members=(indices, idx_ptr),   # the clusters' member lists: the unpooling's backward sums over them
-        )
+            _pooling_inverse=cluster,
+            # max(x >> d) == max(x) >> d: the pooled grid extent needs no reduction and no sync
+            _grid_max_host=[v >> pooling_depth for v in point.grid_max_host()],
+        ))
+
+    def _clusters_started(self, point):
+        """The cluster kernels of this pooling on `point`: those Point.pool_ahead queued, or queued now."""
+        pooling_depth = (math.ceil(self.stride) - 1).bit_length()
+        if pooling_depth > point.serialized_depth:
+            pooling_depth = 0
+        ahead = point.pop("_pending_pool", None)   # started when the codes came into being (Point.pool_ahead)
+        if ahead is not None and ahead[0] == 3 * pooling_depth:
+            return ahead[1]
+        return ops.pool_clusters_start(point.serialized_code[0], point.serialized_order[0], 3 * pooling_depth, point.offset)
+
+    def forward(self, point):
+        pooled = point.pop("_pooled_ahead", None)   # the pooled level's index, when the model built it beforehand
+        built_ahead = pooled is not None
+        if not built_ahead:
+            pending = self._clusters_started(point)
+            projected = ops.linear(point.feat, self.proj)   # needs no cluster count: runs while the count travels
+            pooled = self.pooled_index(point, pending)
+        else:
+            projected = ops.linear(point.feat, self.proj)
+        indices, idx_ptr = pooled["_pool_members"]
+        cluster = pooled.pop("_pooling_inverse")
+        pooled["feat"] = (SegmentReduce.apply(projected, indices, idx_ptr, self.reduce) if ops.wants_grad(projected)
+                          else ops.segment_reduce(projected, indices, idx_ptr, self.reduce))
         if "coord" in point:
-            fields["coord"] = ops.segment_reduce(point.coord.float(), indices, idx_ptr, "mean")
+            pooled["coord"] = ops.segment_reduce(point.coord.float(), indices, idx_ptr, "mean")
         for key in ("condition", "context"):
             if key in point:
-                fields[key] = point[key]
+                pooled[key] = point[key]
         if self.traceable:
-            fields["pooling_inverse"] = cluster
-            fields["pooling_parent"] = point
-        # max(x >> d) == max(x) >> d: the pooled grid extent needs no reduction and no sync
-        fields["_grid_max_host"] = [v >> pooling_depth for v in point.grid_max_host()]
-        pooled = Point(fields)
+            pooled["pooling_inverse"] = cluster
+            pooled["pooling_parent"] = point
         norm = self.norm[0] if self.norm is not None and len(self.norm) == 1 else None
         act = self.act[0] if self.act is not None and len(self.act) == 1 else None
         if norm is not None and _trainable_bn(norm, pooled.feat) and _exact_gelu(act):
@@ -636,7 +659,7 @@ class SerializedPooling(PointModule):
             if self.act is not None:
                 pooled = self.act(pooled)
         pooled.sparsify()
-        if self.next_stride is not None:
+        if not built_ahead and self.next_stride is not None:
             pooled.pool_ahead(self.next_stride)
         return pooled
 

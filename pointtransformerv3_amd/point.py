@@ -200,6 +200,8 @@ class Point(AttrDict):
                                batch_size=len(self.offset_host()))
         for ks, pend in self.pop("_pending_plans", {}).items():
             sct.indice_dict[("pending", ks)] = pend
+        for ks, plan in self.pop("_ready_plans", {}).items():   # finished before the features existed
+            sct.indice_dict[("ready", ks)] = plan
         for ks, src in self.pop("_derived_plans", {}).items():
             sct.indice_dict[("derive", ks)] = src
         self["sparse_conv_feat"] = sct

@@ -131,7 +131,10 @@ class SubMConv3d(nn.Module):
         """Makes (and caches on x, under this module's indice_key) the index lists the half-precision forward of this
         module will ask for: the pair lists, and the tile lists where a tile form takes the layer. They follow from
         the coordinates alone."""
-        plan = x.conv_plan(self.kernel_size, self.indice_key)
+        self.tiles_ahead(x.conv_plan(self.kernel_size, self.indice_key))
+
+    def tiles_ahead(self, plan):
+        """The tile lists of `plan` that this module's half-precision forward will ask for, if it takes a tile form."""
         form = self._tile_form(plan, self.in_channels, self.out_channels)
         if form == "sparse":
             plan.tiles(128)

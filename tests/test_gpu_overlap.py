@@ -1,5 +1,5 @@
-"""PointTransformerV3.overlap_index_prologue: the level-0 index work of a forward on a stream of its own, beside the
-forward before it. The schedule must not change a bit of any output, whatever the sequence of inputs."""
+"""PointTransformerV3.overlap_index_prologue: the index work of every level of a forward first, on a stream of its
+own, beside the forward before it. The schedule must not change a bit of any output, whatever the sequence of inputs."""
 import numpy as np
 import pytest
 import torch
