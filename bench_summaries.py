@@ -203,7 +203,8 @@ def forward_trace(d, out_dir):
         a[3] = max(a[3], dur)
     rows = sorted(agg.items(), key=lambda kv: -kv[1][1])
     tot = sum(v[1] for _, v in rows)
-    span = (int(window[-1]["End_Timestamp"]) - int(window[0]["Start_Timestamp"])) / steps / 1e3
+    # from the first timed forward's first kernel to the last one's, over the forwards in between
+    span = (int(trace[marks[t_first + steps - 1]]["Start_Timestamp"]) - int(window[0]["Start_Timestamp"])) / (steps - 1) / 1e3
     rf, brf = pbench["roofline"], bench["roofline"]
     out = [
         "rocprofv3 kernel-trace summary: full PTv3 forward, 4 room scenes (%d points), fp16, MI355X\n" % POINTS,
@@ -229,7 +230,7 @@ def forward_trace(d, out_dir):
     out += _grouped([(n, v[1], v[0]) for n, v in rows], FORWARD_GROUPS, steps)
     if overlapped:
         ptot = sum(int(r["End_Timestamp"]) - int(r["Start_Timestamp"]) for r in plain)
-        pspan = (int(plain[-1]["End_Timestamp"]) - int(plain[0]["Start_Timestamp"])) / steps / 1e3
+        pspan = (int(trace[marks[-tail - 1]]["Start_Timestamp"]) - int(plain[0]["Start_Timestamp"])) / (steps - 1) / 1e3
         out.append("\nthe plain schedule (every forward's index work in front of its own feature kernels), the %d forwards bench.py "
                    "times after the timed region: %.1f us of kernels per forward, %.1f us from forward to forward under the profiler; "
                    "bench.py's own clock: %.2f ms per forward with the profiler, %.2f ms without"
