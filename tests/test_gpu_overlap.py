@@ -64,3 +64,46 @@ def test_overlap_is_left_alone_in_training_mode_and_under_autograd():
     with torch.inference_mode():
         model(dict(data))
     assert model._prologue_state is not None
+
+
+def test_packed_copies_are_refreshed_while_the_host_waits_and_once_per_epoch():
+    """ops.refresh_derived_copies: the packed weight copies of modules that have been used before are redone when a
+    read-back finds its value still on the way, once per invalidate_casts() epoch, never under autograd and never
+    inside the overlapped prologue's scope (whose allocations are recycled)."""
+    from pointtransformerv3_amd import ops
+    from pointtransformerv3_amd.modules import MLP
+    torch.manual_seed(9)
+    mlp = MLP(128, 512).half().to(DEV)
+    x = torch.randn(300, 128, device=DEV).half()
+    with torch.inference_mode():
+        first = ops.mlp_fused_module(x, x, mlp)                 # registers the module, packs its weights
+        held = mlp._packed_stream[torch.float16]
+        mlp.fc1.weight.data.mul_(2.0)                           # behind autograd's back: only the epoch tells
+        ops.invalidate_casts()
+        calls = []
+        ops._IDLE_WORK.append(lambda: calls.append(1))
+        try:
+            with torch.enable_grad():
+                ops.refresh_derived_copies()
+            assert calls == [] and mlp._packed_stream[torch.float16][0] == held[0]      # not under autograd
+            scope = ops.PrologueOverlap(torch.device(DEV))
+            with scope.scope():
+                assert ops.IDLE_WORK_ALLOWED is False
+                before = len(calls)
+                ops.refresh_derived_copies()
+                assert len(calls) == before                      # not inside the scope (it ran on entering it)
+            assert len(calls) == 1 and ops.IDLE_WORK_ALLOWED is True
+            assert mlp._packed_stream[torch.float16][0] != held[0] and mlp._packed_stream[torch.float16][1] is held[1]
+            ops.refresh_derived_copies()
+            assert len(calls) == 1                               # once per epoch
+            second = ops.mlp_fused_module(x, x, mlp)
+            assert not torch.equal(first, second)
+            assert torch.equal(second, ops.mlp_fused(x, x, mlp.fc1.weight, mlp.fc1.bias, mlp.fc2.weight, mlp.fc2.bias))
+            ops.invalidate_casts()
+            big = torch.randn(1 << 24, device=DEV)
+            for _ in range(20):
+                big = big * 1.0001                               # keeps the stream busy: the read-back has to wait
+            assert ops.Readback(big[:4]).get() is not None
+            assert len(calls) == 2                               # the waiting host did the work
+        finally:
+            ops._IDLE_WORK.pop()
