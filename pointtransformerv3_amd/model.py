@@ -119,9 +119,28 @@ class PointTransformerV3(PointModule):
                 self.dec.add(module=stage, name=f"dec{s}")
 
     def _level0_kernel_sizes(self):
-        from .sparse import SubMConv3d
-        mods = list(self.embedding.modules()) + list(next(iter(self.enc._modules.values())).modules())
-        return tuple(sorted({m.kernel_size for m in mods if isinstance(m, SubMConv3d)}, reverse=True))
+        return self._levels()[0]["kernel_sizes"]
+
+    def _levels(self):
+        """Per level of the encoder, what the index work needs to know of the modules: the pooling module in front
+        of the level, the convolutions that share its pair lists (encoder and decoder stage) and the attention
+        layers whose tables can be made ahead. Walked once: the module structure is taken as fixed from the first
+        forward on."""
+        held = self.__dict__.get("_levels_held")
+        if held is None:
+            held = []
+            for s, stage in enumerate(self.enc._modules.values()):
+                dec = self.dec._modules.get(f"dec{s}") if not self.cls_mode else None
+                enc_side = [self.embedding] * (s == 0) + [stage]
+                both = enc_side + [dec] * (dec is not None)
+                convs = [m for st in both for m in st.modules() if isinstance(m, SubMConv3d)]
+                blocks = [b for st in (stage, dec) if st is not None for b in st._modules.values() if isinstance(b, Block)]
+                same = blocks and all(b.attn.enable_flash and b.attn.patch_size == blocks[0].attn.patch_size for b in blocks)
+                sizes = {m.kernel_size for st in enc_side for m in st.modules() if isinstance(m, SubMConv3d)}
+                held.append(dict(down=stage._modules.get("down"), convs=convs, attention=blocks if same else [],
+                                 kernel_sizes=tuple(sorted(sizes, reverse=True))))
+            object.__setattr__(self, "_levels_held", held)   # not a submodule, not a parameter: stays out of state_dict
+        return held
 
     def forward(self, data_dict):
         """data_dict: feat, grid_coord (or coord + grid_size), offset or batch. Returns the Point
@@ -154,21 +173,13 @@ class PointTransformerV3(PointModule):
             point.pool_ahead(self.stride[0])   # the first pooling's clusters need the codes only
         point.sparsify()
         if everything:
-            stage0 = next(iter(self.enc._modules.values()))
-            dec0 = self.dec._modules.get("dec0") if not self.cls_mode else None
-            for m in list(self.embedding.modules()) + list(stage0.modules()):
-                if isinstance(m, SubMConv3d):
-                    m.lists_ahead(point.sparse_conv_feat)
-            self._attention_tables_ahead(point, stage0, dec0)
+            level0 = self._levels()[0]
+            for m in level0["convs"]:
+                m.lists_ahead(point.sparse_conv_feat)
+            for b in level0["attention"]:
+                b.attn._slots(point)
             self._pooled_index_ahead(point)
         return point
-
-    @staticmethod
-    def _attention_tables_ahead(point, *stages):
-        blocks = [b for st in stages if st is not None for b in st._modules.values() if isinstance(b, Block)]
-        if blocks and all(b.attn.enable_flash and b.attn.patch_size == blocks[0].attn.patch_size for b in blocks):
-            for b in blocks:
-                b.attn._slots(point)
 
     def _pooled_index_ahead(self, point):
         """The index of every pooled level (clusters, pooled codes / coordinates / orders, pair and tile lists,
@@ -177,23 +188,22 @@ class PointTransformerV3(PointModule):
         shuffles from torch's CPU generator in module order here as they would in the forward: evaluation mode only
         (stochastic depth and dropout draw from the same generator in between)."""
         parent = point
-        for s, stage in enumerate(list(self.enc._modules.values())[1:], start=1):
-            down = stage._modules.get("down")
+        for level in self._levels()[1:]:
+            down = level["down"]
             if not isinstance(down, SerializedPooling):
                 return
             pooled = down.pooled_index(parent)
             if down.next_stride is not None:
                 pooled.pool_ahead(down.next_stride)
-            dec = self.dec._modules.get(f"dec{s}") if not self.cls_mode else None
-            convs = [m for st in (stage, dec) if st is not None for m in st.modules() if isinstance(m, SubMConv3d)]
             ready = {}
             for ks, pend in pooled.pop("_pending_plans").items():
                 ready[ks] = ops.conv_plan_direct_finish(pend)
-                for m in convs:
+                for m in level["convs"]:
                     if m.kernel_size == ks:
                         m.tiles_ahead(ready[ks])
             pooled["_ready_plans"] = ready
-            self._attention_tables_ahead(pooled, stage, dec)
+            for b in level["attention"]:
+                b.attn._slots(pooled)
             parent["_pooled_ahead"] = pooled
             parent = pooled
 

@@ -1510,6 +1510,9 @@ def _pack_parts(m):
 
 def _pack_stamp(m, device):
     """What a module's packed copy was made from: the stamps of its weights."""
+    mods = getattr(m, "_modules", None)
+    if mods is not None and "fc1" in mods:   # an MLP, asked for at every use: without the lists of _pack_parts
+        return (parameter_stamp(mods["fc1"]._parameters["weight"]), parameter_stamp(mods["fc2"]._parameters["weight"]), device)
     return tuple(parameter_stamp(w) for w, _ in _pack_parts(m)[0]) + (device,)
 
 
@@ -1565,10 +1568,10 @@ def _packed_stream(m, dtype):
     """The module's packed copy in dtype, redone first (with every other stale one) when its parameters moved."""
     held = m.__dict__.get("_packed_stream")
     entry = held.get(dtype) if held else None
-    device = _pack_parts(m)[0][0][0].device
-    if entry is None or entry[0] != _pack_stamp(m, device):
+    # weights that moved to another device have other addresses: their stamp differs from the one held
+    if entry is None or entry[0] != _pack_stamp(m, entry[0][-1]):
         _MLP_PACK_USERS.add(m)
-        repack_mlp_weights(_MLP_PACK_USERS, dtype, device)
+        repack_mlp_weights(_MLP_PACK_USERS, dtype, _pack_parts(m)[0][0][0].device)
         entry = m._packed_stream[dtype]
     return entry[1]
 
