@@ -598,7 +598,10 @@ class SerializedPooling(PointModule):
         # pooled orders: the distinct clusters met when walking the parent along each curve (same
         # result as argsort of the pooled codes, model.py:667-674, without sorting)
         order, inverse = ops.pool_orders(point.serialized_order, cluster, m, perm)
+        # the clusters' mean coordinates (model.py:687-689) follow from the input coordinates, not from the features
+        extra = {"coord": ops.segment_reduce(point.coord.float(), indices, idx_ptr, "mean")} if "coord" in point else {}
         return Point(AttrDict(
+            **extra,
             grid_coord=grid_coord,
             serialized_code=code,
             serialized_order=order,
@@ -638,8 +641,6 @@ class SerializedPooling(PointModule):
         cluster = pooled.pop("_pooling_inverse")
         pooled["feat"] = (SegmentReduce.apply(projected, indices, idx_ptr, self.reduce) if ops.wants_grad(projected)
                           else ops.segment_reduce(projected, indices, idx_ptr, self.reduce))
-        if "coord" in point:
-            pooled["coord"] = ops.segment_reduce(point.coord.float(), indices, idx_ptr, "mean")
         for key in ("condition", "context"):
             if key in point:
                 pooled[key] = point[key]
