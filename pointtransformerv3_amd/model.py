@@ -155,7 +155,7 @@ class PointTransformerV3(PointModule):
         if not self.cls_mode:
             point = self.dec(point)
         if self._prologue_state is not None:
-            self._prologue_state.forward_queued()
+            self._prologue_state.forward_queued(point)
         return point
 
     def _level0_index(self, data_dict, everything=False):

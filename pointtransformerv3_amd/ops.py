@@ -669,24 +669,32 @@ class PrologueOverlap:
     scope() runs its body on the prologue stream, which waits for nothing, with every allocation of the body routed
     to one of the two pools in turn; on leaving it the current stream is made to wait for the body's work.
     What the body allocates is used by the current stream afterwards without any per-tensor bookkeeping: a pool's
-    memory is handed out again only two forwards later, and forward_queued() (called when the whole forward has been
-    queued) leaves an event on the current stream that the pool's next turn waits for on the host first."""
+    memory is handed out again only two forwards later, after a host wait for an event that the current stream
+    passed when the forward in between was entered -- behind the kernels of the forward that used the pool and behind
+    whatever the caller queued on its results before calling again. The few tensors of a result that a caller may
+    still read after that (PUBLIC_KEYS) are marked for the current stream by forward_queued()."""
+
+    PUBLIC_KEYS = ("batch", "serialized_code", "serialized_order", "serialized_inverse", "pad", "unpad", "cu_seqlens_key")
 
     def __init__(self, device):
         self.device = device
         self.stream = torch.cuda.Stream(device=device)
         self.pools = [torch.cuda.MemPool(), torch.cuda.MemPool()]
-        self.done = [None, None]   # per pool: the forward that last used it has run to its end on its stream
+        self.fence = [None, None]   # per pool: the current stream has passed every use of what it handed out
         self.turn = 0
 
     @contextlib.contextmanager
     def scope(self):
-        self.turn ^= 1
-        if self.done[self.turn] is not None:
-            self.done[self.turn].synchronize()   # two forwards back: over long ago
         global AHEAD_ON_SIDE_STREAM, IDLE_WORK_ALLOWED
-        refresh_derived_copies()   # on the current stream, before it: the host is a forward's tail ahead of the GPU here
         main = torch.cuda.current_stream(self.device)
+        # the pool of the forward before this one: free again once the current stream has come this far
+        entered = torch.cuda.Event()
+        entered.record(main)
+        self.fence[self.turn] = entered
+        self.turn ^= 1
+        if self.fence[self.turn] is not None:
+            self.fence[self.turn].synchronize()   # recorded a forward ago: passed long since
+        refresh_derived_copies()   # on the current stream, before it: the host is a forward's tail ahead of the GPU here
         ahead, AHEAD_ON_SIDE_STREAM = AHEAD_ON_SIDE_STREAM, False   # the shared side stream still holds the last forward's work
         idle, IDLE_WORK_ALLOWED = IDLE_WORK_ALLOWED, False
         try:
@@ -698,10 +706,15 @@ class PrologueOverlap:
             AHEAD_ON_SIDE_STREAM, IDLE_WORK_ALLOWED = ahead, idle
         main.wait_event(ready)
 
-    def forward_queued(self):
-        ev = torch.cuda.Event()
-        ev.record(torch.cuda.current_stream(self.device))
-        self.done[self.turn] = ev
+    def forward_queued(self, point):
+        """The forward that entered scope() last has been queued and returns `point`: its index tensors that a caller
+        may read on the current stream at any later time are marked for that stream (the allocator then holds their
+        memory back until those reads are over); everything else of the index belongs to the forward."""
+        main = torch.cuda.current_stream(self.device)
+        for key in self.PUBLIC_KEYS:
+            t = point.get(key)
+            if isinstance(t, torch.Tensor) and t.is_cuda:
+                t.record_stream(main)
 
 
 def conv_plan_direct_start(indices, ks):
