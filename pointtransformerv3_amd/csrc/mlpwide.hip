@@ -21,6 +21,9 @@
 // contiguous KB costs. ptv3_mlp_pack_weights therefore writes both matrices once in the order of the stream
 // (step, 32-unit block, piece, lane), and the PACKED kernel fetches every fragment as one contiguous KB.
 // Intermediates are rounded to the storage type where the separate layers would have stored them.
+// The same kernel has two more modes at 128 and 256 channels (TAIL_MODE, HEAD_MODE below): the halves of a block in
+// front of and behind its attention, with the projection / the xCPE's Linear and their LayerNorms as further stages
+// of a pass (model.py:541-545, :587-602).
 #include <type_traits>
 
 #include "rowtile.h"
@@ -92,7 +95,7 @@ constexpr int MLP_MODE = 0, TAIL_MODE = 1, HEAD_MODE = 2;
 template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RTMAX, int THREADS, int MINW, int MODE>
 __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
     const T* __restrict__ x, const T* __restrict__ resid, const T* __restrict__ w1, const T* __restrict__ b1,
-    const T* __restrict__ w2, const T* __restrict__ b2, int64_t n, int upw, T* __restrict__ out, WideArgs tail) {
+    const T* __restrict__ w2, const T* __restrict__ b2, int64_t n, int upw, T* __restrict__ out, WideArgs extra) {
     constexpr bool TAIL = MODE == TAIL_MODE, HEADM = MODE == HEAD_MODE;
     static_assert(MODE == MLP_MODE || PACKED, "the block halves read packed weights");
     typedef typename H16<T>::v8 v8;
@@ -114,15 +117,15 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
     if (HEADM)   // [C] each: the xCPE Linear's bias, LayerNorm_cpe's scale and shift, LayerNorm_1's; [3 C] the qkv bias
         for (int i = threadIdx.x; i < 8 * C / 8; i += THREADS) {
             const int which = i / (C / 8), at = i % (C / 8);
-            const T* src = (const T*)(which == 0 ? tail.bp : which == 1 ? tail.ln_w : which == 2 ? tail.ln_b
-                                      : which == 3 ? tail.ln1_w : which == 4 ? tail.ln1_b : tail.bq);
+            const T* src = (const T*)(which == 0 ? extra.bp : which == 1 ? extra.ln_w : which == 2 ? extra.ln_b
+                                      : which == 3 ? extra.ln1_w : which == 4 ? extra.ln1_b : extra.bq);
             *(u32x4*)(bias_lds + i * 8) = *(const u32x4*)(src + (which >= 5 ? i - 5 * (C / 8) : at) * 8);
         }
     T* sum_lds = bias_lds + 8 * C;        // TAIL: [RMAX][XS] the block's running sum (HEAD: a second staging tile); before it the projection's bias
     if (TAIL)                             // and the LayerNorm's scale and shift, [C] each
         for (int i = threadIdx.x; i < 3 * C / 8; i += THREADS) {
             const int which = i / (C / 8), at = i % (C / 8);
-            const T* src = (const T*)(which == 0 ? tail.bp : which == 1 ? tail.ln_w : tail.ln_b);
+            const T* src = (const T*)(which == 0 ? extra.bp : which == 1 ? extra.ln_w : extra.ln_b);
             *(u32x4*)(bias_lds + 5 * C + i * 8) = *(const u32x4*)(src + at * 8);
         }
 
@@ -139,7 +142,7 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
 #pragma unroll
         for (int a = 0; a < MT; ++a) {
             if (PACKED) {
-                const T* p = (TAIL && q < FRONT ? (const T*)tail.wp : w1) + ((u * (C / 32) + wn * MT + a) * 2) * 512 + lane * 8;
+                const T* p = (TAIL && q < FRONT ? (const T*)extra.wp : w1) + ((u * (C / 32) + wn * MT + a) * 2) * 512 + lane * 8;
                 r[a][0] = *(const u32x4*)p;
                 r[a][1] = *(const u32x4*)(p + 512);
                 continue;
@@ -297,7 +300,7 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
                     v[2 * k + 1] = H16<T>::hi(sm[k]);
                 }
                 *(u32x4*)(sum_lds + rr * XS + pc * 8) = sm;
-                *(u32x4*)(xt + rr * XS + pc * 8) = norm_piece(v, gq, bq, tail.eps);
+                *(u32x4*)(xt + rr * XS + pc * 8) = norm_piece(v, gq, bq, extra.eps);
             }
             __syncthreads();
         }
@@ -324,7 +327,7 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
                     v[2 * k] = H16<T>::lo(o[k]);
                     v[2 * k + 1] = H16<T>::hi(o[k]);
                 }
-                const u32x4 z = norm_piece(v, gc, bc, tail.eps);
+                const u32x4 z = norm_piece(v, gc, bc, extra.eps);
                 u32x4 sm;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
@@ -333,7 +336,7 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
                     v[2 * k + 1] = H16<T>::hi(sm[k]);
                 }
                 if (live) *(u32x4*)(out + (row0 + rr) * C + pc * 8) = sm;
-                *(u32x4*)(xt + rr * XS + pc * 8) = norm_piece(v, g1, bb1, tail.eps1);
+                *(u32x4*)(xt + rr * XS + pc * 8) = norm_piece(v, g1, bb1, extra.eps1);
             }
             __syncthreads();
             // ---- qkv in three chunks of C outputs: product (+ bias), rounded, through a staging tile to memory in
@@ -350,7 +353,7 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
                 for (int i = 0; i < PIECES; ++i) {
                     const int rr = (tid + i * THREADS) / PPR;
                     if (row0 + rr < row_end)
-                        *(u32x4*)((T*)tail.qkv + (row0 + rr) * (3 * C) + c * C + pc * 8) = *(const u32x4*)(tile + rr * XS + pc * 8);
+                        *(u32x4*)((T*)extra.qkv + (row0 + rr) * (3 * C) + c * C + pc * 8) = *(const u32x4*)(tile + rr * XS + pc * 8);
                 }
             }
             // no barrier here: the next pass writes xt (last read before the barrier above), then parks into ht and
@@ -440,7 +443,7 @@ __global__ __launch_bounds__(THREADS, MINW) void mlp_wide_kernel(
 template <typename T, int C, int WM, int WN, int MT, int DEPTH, bool PACKED, int RTMAX, int MODE = MLP_MODE,
           int THREADS = MW_THREADS, int MINW = 2>
 int launch_mlp_wide(const void* x, const void* resid, const void* w1, const void* b1, const void* w2, const void* b2,
-                    int64_t n, void* out, hipStream_t stream, WideArgs tail = WideArgs{}) {
+                    int64_t n, void* out, hipStream_t stream, WideArgs extra = WideArgs{}) {
     constexpr int RMAX = 32 * RTMAX * WM, UNIT = 32 * WM;
     constexpr size_t LDS = ((size_t)(MODE == MLP_MODE ? 2 : 3) * RMAX * (C + MW_PAD) + (MODE == MLP_MODE ? 5 : 8) * C) * sizeof(T);
     static_assert(LDS <= 160 * 1024, "LDS of a CU");
@@ -457,7 +460,7 @@ int launch_mlp_wide(const void* x, const void* resid, const void* w1, const void
     if (upw > 0x7fffffffLL) return PTV3_EINVAL;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), lds, stream,
                        (const T*)x, (const T*)resid, (const T*)w1, (const T*)b1, (const T*)w2, (const T*)b2, n, (int)upw, (T*)out,
-                       tail);
+                       extra);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? PTV3_OK : (int)e;
 }
@@ -478,13 +481,13 @@ int mlp_wide_any(const void* x, const void* resid, const void* w1, const void* b
 }
 
 int block_tail_wide_any(const void* attn, const void* sum, const void* packed, const void* b1, const void* b2, int dtype,
-                        int64_t n, int channels, void* out, hipStream_t stream, WideArgs tail) {
+                        int64_t n, int channels, void* out, hipStream_t stream, WideArgs extra) {
 #define PTV3_MW(T)                                                                                                      \
     do {                                                                                                                \
         if (channels == 128)                                                                                            \
-            return launch_mlp_wide<T, 128, 2, 4, 1, 4, true, 3, TAIL_MODE>(attn, sum, packed, b1, nullptr, b2, n, out, stream, tail); \
+            return launch_mlp_wide<T, 128, 2, 4, 1, 4, true, 3, TAIL_MODE>(attn, sum, packed, b1, nullptr, b2, n, out, stream, extra); \
         if (channels == 256)                                                                                            \
-            return launch_mlp_wide<T, 256, 1, 8, 1, 4, true, 3, TAIL_MODE>(attn, sum, packed, b1, nullptr, b2, n, out, stream, tail); \
+            return launch_mlp_wide<T, 256, 1, 8, 1, 4, true, 3, TAIL_MODE>(attn, sum, packed, b1, nullptr, b2, n, out, stream, extra); \
     } while (0)
     if (dtype == PTV3_F16) PTV3_MW(_Float16);
     if (dtype == PTV3_BF16) PTV3_MW(__bf16);
