@@ -187,14 +187,20 @@ class PointTransformerV3(PointModule):
         its parent Point under "_pooled_ahead" for the pooling module to pick up. The pooling stages draw their row
         shuffles from torch's CPU generator in module order here as they would in the forward: evaluation mode only
         (stochastic depth and dropout draw from the same generator in between)."""
-        parent = point
+        parent, made = point, []
         for level in self._levels()[1:]:
             down = level["down"]
             if not isinstance(down, SerializedPooling):
-                return
-            pooled = down.pooled_index(parent)
+                break
+            pooled = down.pooled_index(parent)   # waits for this level's cluster count; its pair counts are queued
             if down.next_stride is not None:
                 pooled.pool_ahead(down.next_stride)
+            parent["_pooled_ahead"] = pooled
+            made.append((level, pooled))
+            parent = pooled
+        # the pair counts of all levels are on their way by now: one wait in effect, instead of one per level between
+        # the levels' cluster kernels
+        for level, pooled in made:
             ready = {}
             for ks, pend in pooled.pop("_pending_plans").items():
                 ready[ks] = ops.conv_plan_direct_finish(pend)
@@ -204,8 +210,6 @@ class PointTransformerV3(PointModule):
             pooled["_ready_plans"] = ready
             for b in level["attention"]:
                 b.attn._slots(pooled)
-            parent["_pooled_ahead"] = pooled
-            parent = pooled
 
     def _index_prologue(self, data_dict):
         feat = data_dict.get("feat")
