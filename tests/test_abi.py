@@ -47,6 +47,16 @@ def test_argument_errors_without_a_device():
     assert lib.ptv3_kmap_build(None, 10, 4, 0, None, None, 0, None) == -4
     assert lib.ptv3_subm_conv_fwd(None, 9, 10, 16, None, 27, 0, None, None, 16, None, None) == -1
     assert b"workspace" in lib.ptv3_strerror(-3)
+    # the block halves at 128 / 256 channels: other widths and dtypes are not theirs, empty input is fine, null pointers
+    tail = lambda dtype, n, c: lib.ptv3_block_tail_wide(None, None, None, None, None, None, 1e-5, None, None, None,
+                                                        dtype, n, c, None, None)
+    head = lambda dtype, n, c: lib.ptv3_block_head_wide(None, None, None, None, None, None, 1e-5, None, None, 1e-5, None,
+                                                        dtype, n, c, None, None, None)
+    for call in (tail, head):
+        assert call(1, 10, 512) == -4 and call(1, 10, 64) == -4 and call(0, 10, 128) == -4   # width, width, fp32
+        assert call(1, 0, 128) == 0 and call(2, 0, 256) == 0
+        assert call(1, 10, 128) == -1 and call(1, -1, 128) == -1
+    assert lib.ptv3_linear_pack_weights_blocks(128) == 8 and lib.ptv3_linear_pack_weights_blocks(96) == 0
 
 
 def test_argument_errors_of_the_training_entry_points():
